@@ -1,0 +1,93 @@
+/*
+ * oxb_hip.h — C ABI of the `native-hip` kernel tier (liboxb_hip.so / liboxb_hip.a).
+ *
+ * This is what a Rust `NativeHipBackend: GpuBackendTrait` binds through
+ * `extern "C"`; each entry point names the reference interface it stands in
+ * for.  Paths are relative to the reference checkout; KG = crates/oxibonsai-kernels/src/gpu_backend.
+ *
+ * Conventions
+ *   - every function returns an oxb_status; 0 is success.  The text of the last
+ *     failure on the calling thread is available from oxb_hip_last_error().
+ *     Codes follow GpuError (KG/mod.rs:317-342) and CudaGraphError::WeightNotFound
+ *     (KG/cuda_graph/types.rs:25-39).  No C++ exception crosses the boundary.
+ *   - pointers without a `d_` prefix are HOST pointers borrowed for the call;
+ *     `d_` pointers are DEVICE pointers.  The library owns all weight memory.
+ *   - calls are serialised by an internal mutex and run on one stream
+ *     (the library's own, or the one given to oxb_hip_set_stream), like the
+ *     reference's Mutex-guarded CudaGraph singleton (KG/cuda_graph/cudagraph_type.rs:18-32).
+ *   - there is no CPU fallback: without a usable GPU every compute entry point
+ *     returns OXB_HIP_NOT_AVAILABLE and the caller decides (the reference's
+ *     dispatcher falls back to its CPU tiers on Err, crates/oxibonsai-kernels/src/dispatch.rs:471-483).
+ */
+#ifndef OXB_HIP_H
+#define OXB_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    OXB_HIP_OK = 0,
+    OXB_HIP_NOT_AVAILABLE = 1,     /* GpuError::NotAvailable      */
+    OXB_HIP_OUT_OF_MEMORY = 2,     /* GpuError::OutOfMemory       */
+    OXB_HIP_KERNEL_LAUNCH = 3,     /* GpuError::KernelLaunch      */
+    OXB_HIP_SYNC_FAILED = 4,       /* GpuError::SyncFailed        */
+    OXB_HIP_INVALID_ARGUMENT = 5,  /* GpuError::InvalidArgument   */
+    OXB_HIP_WEIGHT_NOT_FOUND = 6   /* CudaGraphError::WeightNotFound */
+} oxb_status;
+
+enum { OXB_HIP_FMT_Q1 = 0, OXB_HIP_FMT_TQ2 = 1 };
+
+/* ---- lifecycle: CudaGraph::global() / NativeCudaBackend::new  (KG/cuda_graph/cudagraph_type.rs, KG/mod.rs:1092-1106) */
+int  oxb_hip_init(int device_ordinal);            /* idempotent */
+void oxb_hip_shutdown(void);                      /* frees every weight and workspace */
+/* GpuBackendTrait::name / device_count / memory_info  (KG/mod.rs:360-406) */
+int  oxb_hip_device_count(void);
+int  oxb_hip_device_info(char* name, size_t name_cap, size_t* free_bytes, size_t* total_bytes);
+/* GpuBackendTrait::synchronize (KG/mod.rs:403) */
+int  oxb_hip_synchronize(void);
+/* Run on the caller's HIP stream (hipStream_t passed as void*); NULL restores the library's own stream. */
+int  oxb_hip_set_stream(void* hip_stream);
+const char* oxb_hip_last_error(void);
+
+/* ---- weights: GpuBackendTrait::upload_weights_raw (KG/mod.rs:445) and upload_weights_ternary (:472).
+ * aos = n_rows * (k/128) blocks in the reference's byte order: Q1 18 B [d f16][qs 16], TQ2 34 B [qs 32][d f16].
+ * *id == 0 on entry asks the library to allocate a handle; a non-zero *id is used as given
+ * (the fused paths key weights by caller-chosen ids, crates/oxibonsai-model/src/model/types/forward_cuda/q1.rs:71-72)
+ * and replaces a weight already stored under it. */
+int  oxb_hip_upload_q1(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
+int  oxb_hip_upload_tq2(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
+int  oxb_hip_free_weight(uint64_t id);
+int  oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, size_t* resident_bytes);
+/* Decode the resident copy back to fp32 [n_rows][k]: dequant_1bit_g128 / dequant_tq2_0_g128
+ * (crates/oxibonsai-kernels/src/dequant.rs:15-37, dequant_ternary.rs:42-64) run on the device layout. */
+int  oxb_hip_dequant(uint64_t id, float* out, size_t out_len);
+
+/* ---- GEMV / GEMM on resident weights: gemv_q1_g128_cached (KG/mod.rs:457), gemv_tq2_g128_cached (:484).
+ * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per <= 4 vectors). */
+int  oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch);
+/* Same with device-resident x / y, asynchronous on the current stream. */
+int  oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch);
+
+/* ---- uncached one-shot calls: gemv_q1_g128 (KG/mod.rs:412), gemm_q1_g128 (:425) and their ternary twins.
+ * Validation follows the scalar kernels (crates/oxibonsai-kernels/src/gemv.rs:32-58): k % 128, buffer lengths. */
+int  oxb_hip_gemv_q1_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len,
+                          float* y, size_t y_len, uint32_t n_rows, uint32_t k);
+int  oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len,
+                           float* y, size_t y_len, uint32_t n_rows, uint32_t k);
+
+/* ---- host-only helpers (no GPU needed): the upload-time repack, exposed so it can be checked on any machine.
+ * reformat_q1_aos_to_soa / reformat_tq2_blocks_to_soa (KG/cuda_graph/cudagraph_reformat_*_group.rs). */
+int  oxb_hip_repack_sizes(int fmt, uint32_t n_rows, uint32_t k, size_t* codes_bytes, size_t* scales_bytes);
+int  oxb_hip_repack(int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k,
+                    uint8_t* codes, size_t codes_cap, uint8_t* scales, size_t scales_cap);
+int  oxb_hip_unpack(int fmt, const uint8_t* codes, size_t codes_len, const uint8_t* scales, size_t scales_len,
+                    uint32_t n_rows, uint32_t k, uint8_t* aos, size_t aos_cap);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* OXB_HIP_H */

@@ -1,0 +1,297 @@
+"""ctypes front end of the CPU oracle (``liboxb_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY.  Imported by ``tests/``, by ``__graft_entry__.smoke``
+and by the ``cpu_baseline`` leg of ``bench.py``; the shipped package never
+imports it.  Every function maps 1:1 onto a C function of ``oxb_oracle.h`` /
+``oxb_simd.cpp``, whose comments cite the reference source they restate.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "liboxb_oracle.so")
+_lib = None
+
+OK, NOT_BLOCK_ALIGNED, DIMENSION_MISMATCH, BUFFER_TOO_SMALL = 0, 1, 2, 3
+Q1_BYTES, TQ2_BYTES, QK = 18, 34, 128
+
+
+class OracleError(Exception):
+    def __init__(self, code: int):
+        super().__init__({1: "NotBlockAligned", 2: "DimensionMismatch", 3: "BufferTooSmall"}.get(code, str(code)))
+        self.code = code
+
+
+def build() -> None:
+    subprocess.check_call(["make", "-s", "-C", _HERE])
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        u8p, f32p, sz = C.POINTER(C.c_uint8), C.POINTER(C.c_float), C.c_size_t
+        L.oxb_f16_to_f32.restype = C.c_float
+        L.oxb_f16_to_f32.argtypes = [C.c_uint16]
+        L.oxb_f32_to_f16.restype = C.c_uint16
+        L.oxb_f32_to_f16.argtypes = [C.c_float]
+        for n in ("oxb_dequant_q1", "oxb_dequant_tq2"):
+            getattr(L, n).argtypes = [u8p, sz, f32p, sz]
+        for n in ("oxb_gemv_q1", "oxb_gemv_tq2"):
+            getattr(L, n).argtypes = [u8p, sz, f32p, sz, f32p, sz, sz, sz]
+        for n in ("oxb_gemm_q1", "oxb_gemm_tq2"):
+            getattr(L, n).argtypes = [u8p, sz, f32p, sz, f32p, sz, sz, sz, sz]
+        L.oxb_rms_norm.argtypes = [f32p, f32p, f32p, sz, C.c_float]
+        L.oxb_rms_norm.restype = None
+        L.oxb_silu.argtypes = [C.c_float]
+        L.oxb_silu.restype = C.c_float
+        L.oxb_swiglu.argtypes = [f32p, f32p, f32p, sz]
+        L.oxb_swiglu.restype = None
+        L.oxb_softmax.argtypes = [f32p, sz]
+        L.oxb_softmax.restype = None
+        L.oxb_rope_table.argtypes = [f32p, f32p, sz, sz, C.c_float]
+        L.oxb_rope_table.restype = None
+        L.oxb_rope_apply.argtypes = [f32p, f32p, f32p, f32p, sz]
+        L.oxb_rope_apply.restype = None
+        L.oxb_attention_head.argtypes = [f32p, f32p, f32p, f32p, sz, sz]
+        L.oxb_attention_head.restype = None
+        for n in ("oxb_argmax_last", "oxb_argmax_first"):
+            getattr(L, n).argtypes = [f32p, sz]
+            getattr(L, n).restype = C.c_uint32
+        L.oxb_state_new.restype = C.c_void_p
+        L.oxb_state_new.argtypes = [C.c_void_p]
+        L.oxb_state_free.argtypes = [C.c_void_p]
+        L.oxb_state_free.restype = None
+        L.oxb_forward_ex.argtypes = [C.c_void_p, C.c_void_p, f32p, sz, f32p, f32p]
+        L.oxb_simd_tier.restype = C.c_int
+        L.oxb_simd_threads.restype = C.c_int
+        L.oxb_simd_set_threads.argtypes = [C.c_int]
+        L.oxb_simd_set_threads.restype = None
+        L.oxb_simd_gemv.argtypes = [C.c_int, u8p, sz, f32p, sz, f32p, sz, sz, sz]
+        L.oxb_simd_gemm.argtypes = [C.c_int, u8p, sz, f32p, sz, f32p, sz, sz, sz, sz]
+        _lib = L
+    return _lib
+
+
+def _u8(a):
+    return a.ctypes.data_as(C.POINTER(C.c_uint8))
+
+
+def _f32(a):
+    return a.ctypes.data_as(C.POINTER(C.c_float))
+
+
+def _bytes(a) -> np.ndarray:
+    return np.ascontiguousarray(np.frombuffer(a, dtype=np.uint8) if not isinstance(a, np.ndarray) else a, dtype=np.uint8)
+
+
+def _vec(a) -> np.ndarray:
+    return np.ascontiguousarray(a, dtype=np.float32)
+
+
+def _check(rc: int) -> None:
+    if rc != 0:
+        raise OracleError(rc)
+
+
+def f16_to_f32(h: int) -> float:
+    return float(lib().oxb_f16_to_f32(int(h)))
+
+
+def f32_to_f16(f: float) -> int:
+    return int(lib().oxb_f32_to_f16(float(f)))
+
+
+def dequant(fmt: int, blocks) -> np.ndarray:
+    b = _bytes(blocks)
+    bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
+    n = b.size // bb
+    out = np.empty(n * QK, dtype=np.float32)
+    fn = lib().oxb_dequant_q1 if fmt == 0 else lib().oxb_dequant_tq2
+    _check(fn(_u8(b), n, _f32(out), out.size))
+    return out
+
+
+def gemv(fmt: int, blocks, x, n_rows: int, k: int, y_len: int | None = None) -> np.ndarray:
+    """Scalar reference GEMV.  Buffer lengths are passed as they are, so the
+    reference's validation errors can be provoked."""
+    b, xv = _bytes(blocks), _vec(x)
+    bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
+    y = np.zeros(n_rows if y_len is None else y_len, dtype=np.float32)
+    fn = lib().oxb_gemv_q1 if fmt == 0 else lib().oxb_gemv_tq2
+    _check(fn(_u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, n_rows, k))
+    return y
+
+
+def gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int) -> np.ndarray:
+    b, xv = _bytes(blocks), _vec(x).reshape(-1)
+    bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
+    y = np.zeros(m * n_rows, dtype=np.float32)
+    fn = lib().oxb_gemm_q1 if fmt == 0 else lib().oxb_gemm_tq2
+    _check(fn(_u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, m, n_rows, k))
+    return y.reshape(m, n_rows)
+
+
+def simd_gemv(fmt: int, blocks, x, n_rows: int, k: int, out: np.ndarray | None = None) -> np.ndarray:
+    b, xv = _bytes(blocks), _vec(x)
+    bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
+    y = np.zeros(n_rows, dtype=np.float32) if out is None else out
+    _check(lib().oxb_simd_gemv(fmt, _u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, n_rows, k))
+    return y
+
+
+def simd_gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int) -> np.ndarray:
+    b, xv = _bytes(blocks), _vec(x).reshape(-1)
+    bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
+    y = np.zeros(m * n_rows, dtype=np.float32)
+    _check(lib().oxb_simd_gemm(fmt, _u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, m, n_rows, k))
+    return y.reshape(m, n_rows)
+
+
+def simd_tier() -> str:
+    return {0: "scalar", 1: "avx2+fma", 2: "avx512"}[lib().oxb_simd_tier()]
+
+
+def simd_threads() -> int:
+    return lib().oxb_simd_threads()
+
+
+def rms_norm(x, w, eps: float) -> np.ndarray:
+    xv, wv = _vec(x), _vec(w)
+    out = np.empty_like(xv)
+    lib().oxb_rms_norm(_f32(xv), _f32(wv), _f32(out), xv.size, eps)
+    return out
+
+
+def silu(x: float) -> float:
+    return float(lib().oxb_silu(float(x)))
+
+
+def swiglu(gate, up) -> np.ndarray:
+    g, u = _vec(gate), _vec(up)
+    out = np.empty_like(g)
+    lib().oxb_swiglu(_f32(g), _f32(u), _f32(out), g.size)
+    return out
+
+
+def softmax(v) -> np.ndarray:
+    a = _vec(v).copy()
+    lib().oxb_softmax(_f32(a), a.size)
+    return a
+
+
+def rope_table(head_dim: int, max_seq: int, base: float):
+    half = head_dim // 2
+    c = np.empty((max_seq, half), dtype=np.float32)
+    s = np.empty((max_seq, half), dtype=np.float32)
+    lib().oxb_rope_table(_f32(c), _f32(s), head_dim, max_seq, base)
+    return c, s
+
+
+def rope_apply(v, cos_row, sin_row) -> np.ndarray:
+    a, c, s = _vec(v), _vec(cos_row), _vec(sin_row)
+    out = np.empty_like(a)
+    lib().oxb_rope_apply(_f32(a), _f32(out), _f32(c), _f32(s), a.size // 2)
+    return out
+
+
+def attention_head(q, keys, values, seq_len: int, head_dim: int) -> np.ndarray:
+    qv, kv, vv = _vec(q), _vec(keys).reshape(-1), _vec(values).reshape(-1)
+    out = np.empty(head_dim, dtype=np.float32)
+    lib().oxb_attention_head(_f32(qv), _f32(kv), _f32(vv), _f32(out), seq_len, head_dim)
+    return out
+
+
+def argmax_last(v) -> int:
+    a = _vec(v)
+    return int(lib().oxb_argmax_last(_f32(a), a.size))
+
+
+def argmax_first(v) -> int:
+    a = _vec(v)
+    return int(lib().oxb_argmax_first(_f32(a), a.size))
+
+
+# ---------------------------------------------------------------------------
+# Whole-model decode (oxb_forward_ex).  The ctypes structs mirror oxb_oracle.h.
+# ---------------------------------------------------------------------------
+class _Linear(C.Structure):
+    _fields_ = [("blocks", C.POINTER(C.c_uint8)), ("n_rows", C.c_size_t), ("k", C.c_size_t)]
+
+
+class _Layer(C.Structure):
+    _fields_ = [("attn_norm", C.POINTER(C.c_float)), ("q_norm", C.POINTER(C.c_float)),
+                ("k_norm", C.POINTER(C.c_float)), ("ffn_norm", C.POINTER(C.c_float)),
+                ("q", _Linear), ("k", _Linear), ("v", _Linear), ("o", _Linear),
+                ("gate", _Linear), ("up", _Linear), ("down", _Linear)]
+
+
+class _Model(C.Structure):
+    _fields_ = [("fmt", C.c_int)] + [(n, C.c_size_t) for n in
+                                      ("n_layers", "h", "inter", "nq", "nkv", "hd", "vocab", "max_seq")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float), ("layers", C.POINTER(_Layer)),
+                ("final_norm", C.POINTER(C.c_float)), ("lm_head", _Linear), ("kv_f16", C.c_int)]
+
+
+class OracleModel:
+    """CPU decode of a synthetic Qwen3-shaped model held as reference AoS blocks.
+
+    ``weights`` is the dict produced by ``oxibonsai_amd.synth.make_model``:
+    per layer ``attn_norm, q_norm, k_norm, ffn_norm`` (f32 arrays) and
+    ``q, k, v, o, gate, up, down`` (uint8 AoS block arrays), plus
+    ``final_norm`` and ``lm_head``.
+    """
+
+    def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False):
+        self.cfg = cfg
+        self._keep = []
+        fmt = cfg["fmt"]
+        h, inter, nq, nkv, hd = cfg["h"], cfg["inter"], cfg["nq"], cfg["nkv"], cfg["hd"]
+
+        def lin(arr, n_rows, k):
+            a = _bytes(arr)
+            self._keep.append(a)
+            return _Linear(_u8(a), n_rows, k)
+
+        def vec(arr):
+            a = _vec(arr)
+            self._keep.append(a)
+            return _f32(a)
+
+        layers = (_Layer * cfg["n_layers"])()
+        for i, lw in enumerate(weights["layers"]):
+            layers[i] = _Layer(vec(lw["attn_norm"]), vec(lw["q_norm"]), vec(lw["k_norm"]), vec(lw["ffn_norm"]),
+                               lin(lw["q"], nq * hd, h), lin(lw["k"], nkv * hd, h), lin(lw["v"], nkv * hd, h),
+                               lin(lw["o"], h, nq * hd), lin(lw["gate"], inter, h), lin(lw["up"], inter, h),
+                               lin(lw["down"], h, inter))
+        self._layers = layers
+        self._model = _Model(fmt, cfg["n_layers"], h, inter, nq, nkv, hd, cfg["vocab"], cfg["max_seq"],
+                             cfg["eps"], cfg["rope_theta"], layers, vec(weights["final_norm"]),
+                             lin(weights["lm_head"], cfg["vocab"], h), 1 if kv_f16 else 0)
+        self._state = lib().oxb_state_new(C.byref(self._model))
+
+    def forward(self, hidden, pos: int, want_normed: bool = False):
+        hv = _vec(hidden)
+        logits = np.empty(self.cfg["vocab"], dtype=np.float32)
+        normed = np.empty(self.cfg["h"], dtype=np.float32)
+        _check(lib().oxb_forward_ex(C.byref(self._model), self._state, _f32(hv), pos, _f32(logits), _f32(normed)))
+        return (logits, normed) if want_normed else logits
+
+    def reset(self):
+        lib().oxb_state_free(self._state)
+        self._state = lib().oxb_state_new(C.byref(self._model))
+
+    def __del__(self):
+        try:
+            if self._state:
+                lib().oxb_state_free(self._state)
+                self._state = None
+        except Exception:
+            pass

@@ -1,0 +1,406 @@
+/*
+ * oxb_oracle.c — scalar CPU restatement of the reference's sub-2-bit path.
+ * TEST INFRASTRUCTURE ONLY (see oxb_oracle.h).  Build: -O2 -ffp-contract=off.
+ */
+#include "oxb_oracle.h"
+
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* ------------------------------------------------------------------------- */
+/* binary16 <-> binary32.  The reference uses half::f16::{to_f32,from_f32}     */
+/* (half 2.7.1; call sites kernels/src/gemv.rs:65, gemv_ternary.rs:87,        */
+/* core/src/tensor.rs:70): IEEE-754 widening is exact, narrowing is RNE.      */
+/* ------------------------------------------------------------------------- */
+float oxb_f16_to_f32(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: normalise */
+            int e = -1;
+            do { man <<= 1; e++; } while (!(man & 0x400u));
+            man &= 0x3FFu;
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | (man << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 127 - 15) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+uint16_t oxb_f32_to_f16(float f) {
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t abs = x & 0x7FFFFFFFu;
+    if (abs >= 0x7F800000u) { /* inf / nan */
+        return (uint16_t)(sign | 0x7C00u | (abs > 0x7F800000u ? (0x200u | ((abs >> 13) & 0x3FFu)) : 0));
+    }
+    if (abs >= 0x477FF000u) { /* rounds to >= 65520 -> inf */
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (abs < 0x33000001u) { /* < 2^-25 (or == 2^-25 tie -> even 0) */
+        return sign;
+    }
+    int32_t e = (int32_t)(abs >> 23) - 127;
+    uint32_t man = (abs & 0x7FFFFFu) | 0x800000u;
+    uint32_t shift, half_man;
+    if (e < -14) { /* subnormal result */
+        shift = (uint32_t)(13 + (-14 - e));
+        half_man = man >> shift;
+        uint32_t rem = man & ((1u << shift) - 1u);
+        uint32_t halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (half_man & 1u))) half_man++;
+        return (uint16_t)(sign | half_man);
+    }
+    shift = 13;
+    half_man = man >> shift; /* includes the implicit bit at 0x400 */
+    uint32_t rem = man & 0x1FFFu;
+    uint32_t out = ((uint32_t)(e + 15) << 10) + (half_man - 0x400u);
+    if (rem > 0x1000u || (rem == 0x1000u && (out & 1u))) out++;
+    return (uint16_t)(sign | out);
+}
+
+static inline float q1_scale(const uint8_t* b) { /* [d LE][qs16]: core/src/tensor.rs:25-32 */
+    return oxb_f16_to_f32((uint16_t)(b[0] | (b[1] << 8)));
+}
+static inline float tq2_scale(const uint8_t* b) { /* [qs32][d LE]: core/src/quant_ternary.rs:64-71 */
+    return oxb_f16_to_f32((uint16_t)(b[32] | (b[33] << 8)));
+}
+/* core/src/quant_ternary.rs:191-200, kernels/src/gemv_ternary.rs:19-27 */
+static inline float tq2_code(uint8_t byte, unsigned lane) {
+    switch ((byte >> (lane * 2)) & 3u) {
+        case 0: return -1.0f;
+        case 1: return 0.0f;
+        case 2: return 1.0f;
+        default: return 0.0f;
+    }
+}
+
+/* kernels/src/dequant.rs:15-37 */
+int oxb_dequant_q1(const uint8_t* blocks, size_t n_blocks, float* out, size_t out_len) {
+    if (out_len < n_blocks * OXB_QK) return OXB_ERR_BUFFER_TOO_SMALL;
+    for (size_t i = 0; i < n_blocks; i++) {
+        const uint8_t* b = blocks + i * OXB_Q1_BYTES;
+        float d = q1_scale(b);
+        for (size_t j = 0; j < OXB_QK; j++) {
+            unsigned bit = (b[2 + j / 8] >> (j % 8)) & 1u;
+            out[i * OXB_QK + j] = bit ? d : -d;
+        }
+    }
+    return OXB_OK;
+}
+
+/* kernels/src/dequant_ternary.rs:42-64 */
+int oxb_dequant_tq2(const uint8_t* blocks, size_t n_blocks, float* out, size_t out_len) {
+    if (out_len < n_blocks * OXB_QK) return OXB_ERR_BUFFER_TOO_SMALL;
+    for (size_t i = 0; i < n_blocks; i++) {
+        const uint8_t* b = blocks + i * OXB_TQ2_BYTES;
+        float d = tq2_scale(b);
+        for (size_t byte = 0; byte < 32; byte++)
+            for (unsigned lane = 0; lane < 4; lane++)
+                out[i * OXB_QK + byte * 4 + lane] = d * tq2_code(b[byte], lane);
+    }
+    return OXB_OK;
+}
+
+/* kernels/src/gemv.rs:60-84 — inner loop of one row. */
+static float q1_row_dot(const uint8_t* row_blocks, size_t blocks_per_row, const float* x) {
+    float sum = 0.0f;
+    for (size_t bi = 0; bi < blocks_per_row; bi++) {
+        const uint8_t* b = row_blocks + bi * OXB_Q1_BYTES;
+        float d = q1_scale(b);
+        const float* xb = x + bi * OXB_QK;
+        float block_sum = 0.0f;
+        for (size_t j = 0; j < OXB_QK; j++) {
+            float sign = ((b[2 + j / 8] >> (j % 8)) & 1u) ? 1.0f : -1.0f;
+            block_sum += sign * xb[j];
+        }
+        sum += d * block_sum;
+    }
+    return sum;
+}
+
+/* kernels/src/gemv_ternary.rs:83-102 — inner loop of one row. */
+static float tq2_row_dot(const uint8_t* row_blocks, size_t blocks_per_row, const float* x) {
+    float sum = 0.0f;
+    for (size_t bi = 0; bi < blocks_per_row; bi++) {
+        const uint8_t* b = row_blocks + bi * OXB_TQ2_BYTES;
+        float d = tq2_scale(b);
+        const float* xb = x + bi * OXB_QK;
+        float block_sum = 0.0f;
+        for (size_t byte = 0; byte < 32; byte++)
+            for (unsigned lane = 0; lane < 4; lane++)
+                block_sum += tq2_code(b[byte], lane) * xb[byte * 4 + lane];
+        sum += d * block_sum;
+    }
+    return sum;
+}
+
+/* kernels/src/gemv.rs:25-87 (validation order :32-58) */
+int oxb_gemv_q1(const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                float* y, size_t y_len, size_t n_rows, size_t k) {
+    if (k % OXB_QK != 0) return OXB_ERR_NOT_BLOCK_ALIGNED;
+    if (x_len < k) return OXB_ERR_DIMENSION_MISMATCH;
+    if (y_len < n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
+    size_t bpr = k / OXB_QK;
+    if (n_blocks < n_rows * bpr) return OXB_ERR_BUFFER_TOO_SMALL;
+    for (size_t r = 0; r < n_rows; r++)
+        y[r] = q1_row_dot(blocks + r * bpr * OXB_Q1_BYTES, bpr, x);
+    return OXB_OK;
+}
+
+/* kernels/src/gemv_ternary.rs:48-105 (short block slice is DimensionMismatch, :76-81) */
+int oxb_gemv_tq2(const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                 float* y, size_t y_len, size_t n_rows, size_t k) {
+    if (k % OXB_QK != 0) return OXB_ERR_NOT_BLOCK_ALIGNED;
+    if (x_len < k) return OXB_ERR_DIMENSION_MISMATCH;
+    if (y_len < n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
+    size_t bpr = k / OXB_QK;
+    if (n_blocks < n_rows * bpr) return OXB_ERR_DIMENSION_MISMATCH;
+    for (size_t r = 0; r < n_rows; r++)
+        y[r] = tq2_row_dot(blocks + r * bpr * OXB_TQ2_BYTES, bpr, x);
+    return OXB_OK;
+}
+
+/* kernels/src/gemm.rs:19-87: Y[mi][ni] = dot(W[ni,:], X[mi,:]) */
+int oxb_gemm_q1(const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                float* y, size_t y_len, size_t m, size_t n_rows, size_t k) {
+    if (k % OXB_QK != 0) return OXB_ERR_NOT_BLOCK_ALIGNED;
+    if (x_len < m * k) return OXB_ERR_DIMENSION_MISMATCH;
+    if (y_len < m * n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
+    size_t bpr = k / OXB_QK;
+    if (n_blocks < n_rows * bpr) return OXB_ERR_BUFFER_TOO_SMALL;
+    for (size_t mi = 0; mi < m; mi++)
+        for (size_t ni = 0; ni < n_rows; ni++)
+            y[mi * n_rows + ni] = q1_row_dot(blocks + ni * bpr * OXB_Q1_BYTES, bpr, x + mi * k);
+    return OXB_OK;
+}
+
+/* kernels/src/gemm_ternary.rs:35-69: a GEMV per batch row. */
+int oxb_gemm_tq2(const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                 float* y, size_t y_len, size_t m, size_t n_rows, size_t k) {
+    if (k % OXB_QK != 0) return OXB_ERR_NOT_BLOCK_ALIGNED;
+    if (x_len < m * k) return OXB_ERR_DIMENSION_MISMATCH;
+    if (y_len < m * n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
+    for (size_t mi = 0; mi < m; mi++) {
+        int rc = oxb_gemv_tq2(blocks, n_blocks, x + mi * k, k, y + mi * n_rows, n_rows, n_rows, k);
+        if (rc) return rc;
+    }
+    return OXB_OK;
+}
+
+/* kernels/src/simd_float_ops.rs:204-215 */
+void oxb_rms_norm(const float* in, const float* w, float* out, size_t n, float eps) {
+    float sum_sq = 0.0f;
+    for (size_t i = 0; i < n; i++) sum_sq += in[i] * in[i];
+    float rms = sqrtf(sum_sq / (float)n + eps);
+    float inv_rms = 1.0f / rms;
+    for (size_t i = 0; i < n; i++) out[i] = w[i] * in[i] * inv_rms;
+}
+
+/* kernels/src/simd_float_ops.rs:217-220; model/src/layers/swiglu.rs:9-12 */
+float oxb_silu(float x) { return x / (1.0f + expf(-x)); }
+
+/* kernels/src/simd_float_ops.rs:232-236 */
+void oxb_swiglu(const float* gate, const float* up, float* out, size_t n) {
+    for (size_t i = 0; i < n; i++) out[i] = oxb_silu(gate[i]) * up[i];
+}
+
+/* kernels/src/simd_float_ops.rs:187-201 */
+void oxb_softmax(float* v, size_t n) {
+    float mx = -INFINITY;
+    for (size_t i = 0; i < n; i++) mx = fmaxf(mx, v[i]);
+    float sum = 0.0f;
+    for (size_t i = 0; i < n; i++) { v[i] = expf(v[i] - mx); sum += v[i]; }
+    if (sum > 0.0f) {
+        float inv = 1.0f / sum;
+        for (size_t i = 0; i < n; i++) v[i] *= inv;
+    }
+}
+
+/* model/src/layers/rope.rs:27-48: all arithmetic in f32 (powf, cos, sin). */
+void oxb_rope_table(float* cos_t, float* sin_t, size_t head_dim, size_t max_seq, float freq_base) {
+    size_t half = head_dim / 2;
+    for (size_t pos = 0; pos < max_seq; pos++)
+        for (size_t i = 0; i < half; i++) {
+            float freq = 1.0f / powf(freq_base, 2.0f * (float)i / (float)head_dim);
+            float angle = (float)pos * freq;
+            cos_t[pos * half + i] = cosf(angle);
+            sin_t[pos * half + i] = sinf(angle);
+        }
+}
+
+/* kernels/src/simd_float_ops.rs:240-253: half-split pairs (i, i + half). */
+void oxb_rope_apply(const float* in, float* out, const float* c, const float* s, size_t half) {
+    for (size_t i = 0; i < half; i++) {
+        float x0 = in[i], x1 = in[half + i];
+        out[i] = x0 * c[i] - x1 * s[i];
+        out[half + i] = x0 * s[i] + x1 * c[i];
+    }
+}
+
+/* model/src/layers/attention_fused.rs:166-226 (online softmax state) and :329-400
+ * (contiguous K/V walk).  The reference's dot product is AVX dual-accumulator on
+ * x86 (:139-164); the plain index-order sum is used here, the difference being a
+ * summation order the tolerances cover. */
+void oxb_attention_head(const float* q, const float* keys, const float* values, float* out,
+                        size_t seq_len, size_t hd) {
+    for (size_t d = 0; d < hd; d++) out[d] = 0.0f;
+    if (seq_len == 0) return;
+    float scale = 1.0f / sqrtf((float)hd);
+    float max_val = -INFINITY, sum_exp = 0.0f;
+    for (size_t t = 0; t < seq_len; t++) {
+        const float* kt = keys + t * hd;
+        float dot = 0.0f;
+        for (size_t d = 0; d < hd; d++) dot += q[d] * kt[d];
+        float score = dot * scale;
+        if (score > max_val) {
+            float rescale = (max_val == -INFINITY) ? 0.0f : expf(max_val - score);
+            sum_exp *= rescale;
+            for (size_t d = 0; d < hd; d++) out[d] *= rescale;
+            max_val = score;
+        }
+        float e = expf(score - max_val);
+        sum_exp += e;
+        const float* vt = values + t * hd;
+        for (size_t d = 0; d < hd; d++) out[d] += e * vt[d];
+    }
+    if (sum_exp > 0.0f) {
+        float inv = 1.0f / sum_exp;
+        for (size_t d = 0; d < hd; d++) out[d] *= inv;
+    }
+}
+
+/* runtime/src/sampling.rs:84-91,182-189: Iterator::max_by keeps the LAST maximum. */
+uint32_t oxb_argmax_last(const float* v, size_t n) {
+    size_t best = 0;
+    for (size_t i = 1; i < n; i++) if (v[i] >= v[best]) best = i;
+    return (uint32_t)best;
+}
+/* kernels/src/gpu_backend/cuda_kernels.rs:407-436: strict '>' keeps the FIRST maximum. */
+uint32_t oxb_argmax_first(const float* v, size_t n) {
+    size_t best = 0;
+    for (size_t i = 1; i < n; i++) if (v[i] > v[best]) best = i;
+    return (uint32_t)best;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Whole-model decode step: model/src/model/types/mod.rs:633-934 (embedding   */
+/* row -> blocks -> output_norm -> LM head) around                            */
+/* model/src/block/types/forward.rs:92-408 (one transformer block).           */
+/* KV layout: model/src/kv_cache.rs:118-120  [layer][kv_head][pos][d].        */
+/* ------------------------------------------------------------------------- */
+struct oxb_state {
+    float *k_cache, *v_cache;     /* [L][nkv][max_seq][hd] */
+    float *cos_t, *sin_t;         /* [max_seq][hd/2] */
+    float *hidden, *normed, *q, *k, *v, *qn, *kn, *qr, *kr, *attn, *proj, *gate, *up, *act, *down;
+};
+
+static int linear_fwd(int fmt, const oxb_linear* l, const float* x, float* y) {
+    size_t nb = l->n_rows * (l->k / OXB_QK);
+    return fmt == 0 ? oxb_gemv_q1(l->blocks, nb, x, l->k, y, l->n_rows, l->n_rows, l->k)
+                    : oxb_gemv_tq2(l->blocks, nb, x, l->k, y, l->n_rows, l->n_rows, l->k);
+}
+
+oxb_state* oxb_state_new(const oxb_model* m) {
+    oxb_state* s = (oxb_state*)calloc(1, sizeof(*s));
+    if (!s) return NULL;
+    size_t kv = m->n_layers * m->nkv * m->max_seq * m->hd;
+    size_t qd = m->nq * m->hd, kd = m->nkv * m->hd;
+    s->k_cache = (float*)calloc(kv, 4);
+    s->v_cache = (float*)calloc(kv, 4);
+    s->cos_t = (float*)malloc(m->max_seq * (m->hd / 2) * 4);
+    s->sin_t = (float*)malloc(m->max_seq * (m->hd / 2) * 4);
+    oxb_rope_table(s->cos_t, s->sin_t, m->hd, m->max_seq, m->rope_theta);
+    s->hidden = (float*)malloc(m->h * 4);
+    s->normed = (float*)malloc(m->h * 4);
+    s->q = (float*)malloc(qd * 4);  s->qn = (float*)malloc(qd * 4);  s->qr = (float*)malloc(qd * 4);
+    s->k = (float*)malloc(kd * 4);  s->kn = (float*)malloc(kd * 4);  s->kr = (float*)malloc(kd * 4);
+    s->v = (float*)malloc(kd * 4);
+    s->attn = (float*)malloc(qd * 4);
+    s->proj = (float*)malloc(m->h * 4);
+    s->gate = (float*)malloc(m->inter * 4);
+    s->up = (float*)malloc(m->inter * 4);
+    s->act = (float*)malloc(m->inter * 4);
+    s->down = (float*)malloc(m->h * 4);
+    return s;
+}
+
+void oxb_state_free(oxb_state* s) {
+    if (!s) return;
+    free(s->k_cache); free(s->v_cache); free(s->cos_t); free(s->sin_t);
+    free(s->hidden); free(s->normed); free(s->q); free(s->qn); free(s->qr);
+    free(s->k); free(s->kn); free(s->kr); free(s->v); free(s->attn); free(s->proj);
+    free(s->gate); free(s->up); free(s->act); free(s->down);
+    free(s);
+}
+
+int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos,
+                   float* logits, float* normed_out) {
+    if (pos >= m->max_seq) return OXB_ERR_DIMENSION_MISMATCH;
+    const size_t h = m->h, hd = m->hd, half = hd / 2, nq = m->nq, nkv = m->nkv;
+    const size_t group = nq / nkv;
+    memcpy(s->hidden, hidden_in, h * 4);
+    const float* c = s->cos_t + pos * half;
+    const float* sn = s->sin_t + pos * half;
+    for (size_t L = 0; L < m->n_layers; L++) {
+        const oxb_layer* ly = &m->layers[L];
+        int rc;
+        oxb_rms_norm(s->hidden, ly->attn_norm, s->normed, h, m->eps);            /* forward.rs:94 */
+        if ((rc = linear_fwd(m->fmt, &ly->q, s->normed, s->q))) return rc;       /* :172-174 */
+        if ((rc = linear_fwd(m->fmt, &ly->k, s->normed, s->k))) return rc;
+        if ((rc = linear_fwd(m->fmt, &ly->v, s->normed, s->v))) return rc;
+        for (size_t hh = 0; hh < nq; hh++) {                                      /* :179-206 */
+            oxb_rms_norm(s->q + hh * hd, ly->q_norm, s->qn + hh * hd, hd, m->eps);
+            oxb_rope_apply(s->qn + hh * hd, s->qr + hh * hd, c, sn, half);
+        }
+        for (size_t hh = 0; hh < nkv; hh++) {
+            oxb_rms_norm(s->k + hh * hd, ly->k_norm, s->kn + hh * hd, hd, m->eps);
+            oxb_rope_apply(s->kn + hh * hd, s->kr + hh * hd, c, sn, half);
+        }
+        for (size_t hh = 0; hh < nkv; hh++) {                                     /* :209-213 */
+            size_t off = ((L * nkv + hh) * m->max_seq + pos) * hd;
+            for (size_t d = 0; d < hd; d++) {
+                float kv = s->kr[hh * hd + d], vv = s->v[hh * hd + d];
+                if (m->kv_f16) { /* cuda_attn_kernels.rs:228-251 rounds to f16 on store */
+                    kv = oxb_f16_to_f32(oxb_f32_to_f16(kv));
+                    vv = oxb_f16_to_f32(oxb_f32_to_f16(vv));
+                }
+                s->k_cache[off + d] = kv;
+                s->v_cache[off + d] = vv;
+            }
+        }
+        for (size_t qh = 0; qh < nq; qh++) {                                      /* block/functions.rs:78-127 */
+            size_t kvh = qh / group;
+            size_t base = (L * nkv + kvh) * m->max_seq * hd;
+            oxb_attention_head(s->qr + qh * hd, s->k_cache + base, s->v_cache + base,
+                               s->attn + qh * hd, pos + 1, hd);
+        }
+        if ((rc = linear_fwd(m->fmt, &ly->o, s->attn, s->proj))) return rc;      /* :389-392 */
+        for (size_t i = 0; i < h; i++) s->hidden[i] += s->proj[i];
+        oxb_rms_norm(s->hidden, ly->ffn_norm, s->normed, h, m->eps);             /* :393 */
+        if ((rc = linear_fwd(m->fmt, &ly->gate, s->normed, s->gate))) return rc; /* :394-403 */
+        if ((rc = linear_fwd(m->fmt, &ly->up, s->normed, s->up))) return rc;
+        oxb_swiglu(s->gate, s->up, s->act, m->inter);                            /* :404 */
+        if ((rc = linear_fwd(m->fmt, &ly->down, s->act, s->down))) return rc;    /* :405-408 */
+        for (size_t i = 0; i < h; i++) s->hidden[i] += s->down[i];
+    }
+    oxb_rms_norm(s->hidden, m->final_norm, s->normed, h, m->eps);                /* mod.rs:869-870 */
+    if (normed_out) memcpy(normed_out, s->normed, h * 4);
+    if (logits) return linear_fwd(m->fmt, &m->lm_head, s->normed, logits);       /* mod.rs:874-880 */
+    return OXB_OK;
+}
+
+int oxb_forward(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos, float* logits) {
+    return oxb_forward_ex(m, s, hidden_in, pos, logits, NULL);
+}

@@ -1,0 +1,401 @@
+// runtime.hip — the C ABI of the native-hip tier: device/stream ownership, the
+// weight handle table, workspaces, validation and error reporting.
+//
+// Host-side counterpart of the reference's CudaGraph singleton and
+// NativeCudaBackend (crates/oxibonsai-kernels/src/gpu_backend/cuda_graph/
+// cudagraph_type.rs:18-32, nativecudabackend_traits.rs:29-188): one device, one
+// stream, a process-wide map u64 -> resident weight, every call under a mutex.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/oxb_hip.h"
+#include "gemv_kernels.h"
+#include "layout.h"
+#include "repack.h"
+#include "runtime_internal.h"
+
+namespace oxb {
+
+thread_local std::string t_last_error;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    t_last_error = buf;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+    int code = (e == hipErrorOutOfMemory) ? OXB_HIP_OUT_OF_MEMORY : OXB_HIP_KERNEL_LAUNCH;
+    return fail(code, "%s: %s", what, hipGetErrorString(e));
+}
+
+Runtime g_rt;
+std::recursive_mutex g_mu;
+
+int DevBuf::ensure(size_t bytes) {
+    if (bytes <= cap) return OXB_HIP_OK;
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    cap = 0;
+    size_t want = bytes + (bytes >> 2);
+    want = (want + 255) & ~(size_t)255;
+    hipError_t e = hipMalloc(&ptr, want);
+    if (e != hipSuccess) {
+        ptr = nullptr;
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", want, g_rt.device);
+    }
+    cap = want;
+    return OXB_HIP_OK;
+}
+
+void DevBuf::release() {
+    if (ptr) (void)hipFree(ptr);
+    ptr = nullptr;
+    cap = 0;
+}
+
+int ensure_init() {
+    if (g_rt.ready) return OXB_HIP_OK;
+    return oxb_hip_init(g_rt.device < 0 ? 0 : g_rt.device);
+}
+
+Weight* find_weight(uint64_t id) {
+    auto it = g_rt.weights.find(id);
+    return it == g_rt.weights.end() ? nullptr : &it->second;
+}
+
+static void free_weight_mem(Weight& w) {
+    if (w.d_base) (void)hipFree(w.d_base);
+    w.d_base = nullptr;
+}
+
+int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
+    if (!id) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: id pointer is null");
+    if (k == 0 || k % OXB_QK != 0)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
+    if (n_rows == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: n_rows is 0");
+    const size_t bb = fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES;
+    const size_t need = (size_t)n_rows * (k / OXB_QK) * bb;
+    if (!aos || n_bytes < need)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer holds %zu bytes, %zu needed", n_bytes, need);
+    int rc = ensure_init();
+    if (rc) return rc;
+
+    Weight w;
+    w.L = oxb_make_layout((uint32_t)fmt, n_rows, k);
+    const size_t total = w.L.codes_bytes + w.L.scales_bytes;
+    std::vector<uint8_t> host(total);
+    oxb_repack_aos_to_tiled(w.L, aos, reinterpret_cast<uint32_t*>(host.data()),
+                            reinterpret_cast<uint16_t*>(host.data() + w.L.codes_bytes));
+    hipError_t e = hipMalloc(&w.d_base, total);
+    if (e != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", total, g_rt.device);
+    e = hipMemcpy(w.d_base, host.data(), total, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(w.d_base);
+        return hip_fail(e, "weight upload");
+    }
+    w.d_codes = reinterpret_cast<uint32_t*>(w.d_base);
+    w.d_scales = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(w.d_base) + w.L.codes_bytes);
+    if (*id == 0) *id = g_rt.next_id++;
+    if (Weight* old = find_weight(*id)) free_weight_mem(*old);
+    g_rt.weights[*id] = w;
+    return OXB_HIP_OK;
+}
+
+// x (device, [batch][k]) -> y (device, [batch][ldy]) through quantiser + GEMV, <= 4 vectors per pass.
+int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
+                const float* d_residual) {
+    const uint32_t k = w.L.k;
+    for (uint32_t b0 = 0; b0 < batch; b0 += 4) {
+        const uint32_t nb = (batch - b0) < 4 ? (batch - b0) : 4;
+        int rc;
+        if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, 4)))) return rc;
+        if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, 4)))) return rc;
+        if ((rc = g_rt.ws_xexp.ensure(16 * sizeof(int32_t)))) return rc;
+        hipError_t e = oxb_launch_quant_x((int)w.L.fmt, d_x + (size_t)b0 * k, k, nb, (uint32_t*)g_rt.ws_xq.ptr,
+                                          (int32_t*)g_rt.ws_cneg.ptr, (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
+        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: quant_x");
+        OxbGemvParams p;
+        memset(&p, 0, sizeof p);
+        p.codes = w.d_codes;
+        p.scales = w.d_scales;
+        p.xq = (const uint32_t*)g_rt.ws_xq.ptr;
+        p.cneg = (const int32_t*)g_rt.ws_cneg.ptr;
+        p.xexp = (const int32_t*)g_rt.ws_xexp.ptr;
+        p.y = d_y + (size_t)b0 * ldy;
+        p.residual = d_residual ? d_residual + (size_t)b0 * ldy : nullptr;
+        p.n_rows = w.L.n_rows;
+        p.n_tiles = w.L.n_tiles;
+        p.n_sb = w.L.n_sb;
+        p.NC = 4 * nb;
+        p.ldy = ldy;
+        for (uint32_t sb = 0; sb < w.L.n_sb; sb += 32) {
+            p.sb_begin = sb;
+            p.sb_count = (w.L.n_sb - sb) < 32 ? (w.L.n_sb - sb) : 32;
+            p.mode = sb == 0 ? mode : OXB_GEMV_ACCUM;
+            e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
+            if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
+        }
+    }
+    return OXB_HIP_OK;
+}
+
+static int check_shape(const Weight& w, uint32_t n_rows, uint32_t k) {
+    if (k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
+    if (w.L.n_rows != n_rows || w.L.k != k)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight is %ux%u, call asks for %ux%u", w.L.n_rows,
+                    w.L.k, n_rows, k);
+    return OXB_HIP_OK;
+}
+
+static int sync_stream(const char* what) {
+    hipError_t e = hipStreamSynchronize(g_rt.stream);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: %s: %s", what, hipGetErrorString(e));
+    return OXB_HIP_OK;
+}
+
+static int oneshot_gemv(int fmt, const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len, float* y,
+                        size_t y_len, uint32_t n_rows, uint32_t k) {
+    // Validation order of the scalar kernels (gemv.rs:32-58 / gemv_ternary.rs:55-81).
+    if (k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
+    if (x_len < k) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: input holds %zu values, %u needed", x_len, k);
+    if (y_len < n_rows) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: output holds %zu values, %u needed", y_len, n_rows);
+    if (n_rows == 0) return OXB_HIP_OK;
+    uint64_t id = 0;
+    int rc = upload_weight(&id, fmt, aos, n_bytes, n_rows, k);
+    if (rc) return rc;
+    rc = oxb_hip_gemv(id, x, y, n_rows, k, 1);
+    int rc2 = oxb_hip_free_weight(id);
+    return rc ? rc : rc2;
+}
+
+}  // namespace oxb
+
+using namespace oxb;
+
+extern "C" {
+
+const char* oxb_hip_last_error(void) { return t_last_error.c_str(); }
+
+int oxb_hip_device_count(void) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess) return 0;
+    return n;
+}
+
+int oxb_hip_init(int device_ordinal) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (g_rt.ready) {
+        if (device_ordinal != g_rt.device)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: already initialised on device %d", g_rt.device);
+        return OXB_HIP_OK;
+    }
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0) return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: no HIP device");
+    if (device_ordinal < 0 || device_ordinal >= n)
+        return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: device %d of %d", device_ordinal, n);
+    if ((e = hipSetDevice(device_ordinal)) != hipSuccess) return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: %s", hipGetErrorString(e));
+    hipDeviceProp_t prop;
+    if ((e = hipGetDeviceProperties(&prop, device_ordinal)) != hipSuccess)
+        return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: %s", hipGetErrorString(e));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: kernels are built for gfx950, device is %s", prop.gcnArchName);
+    if ((e = hipStreamCreateWithFlags(&g_rt.own_stream, hipStreamNonBlocking)) != hipSuccess)
+        return hip_fail(e, "stream creation");
+    g_rt.stream = g_rt.own_stream;
+    g_rt.device = device_ordinal;
+    g_rt.n_cus = (uint32_t)prop.multiProcessorCount;
+    snprintf(g_rt.name, sizeof g_rt.name, "%s (%s)", prop.name, prop.gcnArchName);
+    g_rt.ready = true;
+    return OXB_HIP_OK;
+}
+
+void oxb_hip_shutdown(void) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!g_rt.ready) return;
+    (void)hipStreamSynchronize(g_rt.stream);
+    shutdown_models();
+    for (auto& kv : g_rt.weights) free_weight_mem(kv.second);
+    g_rt.weights.clear();
+    g_rt.ws_x.release();
+    g_rt.ws_y.release();
+    g_rt.ws_xq.release();
+    g_rt.ws_cneg.release();
+    g_rt.ws_xexp.release();
+    (void)hipStreamDestroy(g_rt.own_stream);
+    g_rt.own_stream = nullptr;
+    g_rt.stream = nullptr;
+    g_rt.ready = false;
+}
+
+int oxb_hip_device_info(char* name, size_t name_cap, size_t* free_bytes, size_t* total_bytes) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    int rc = ensure_init();
+    if (rc) return rc;
+    if (name && name_cap) snprintf(name, name_cap, "%s", g_rt.name);
+    size_t f = 0, t = 0;
+    hipError_t e = hipMemGetInfo(&f, &t);
+    if (e != hipSuccess) return hip_fail(e, "memory info");
+    if (free_bytes) *free_bytes = f;
+    if (total_bytes) *total_bytes = t;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_synchronize(void) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    int rc = ensure_init();
+    if (rc) return rc;
+    return sync_stream("synchronize");
+}
+
+int oxb_hip_set_stream(void* hip_stream) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    int rc = ensure_init();
+    if (rc) return rc;
+    g_rt.stream = hip_stream ? (hipStream_t)hip_stream : g_rt.own_stream;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_upload_q1(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return upload_weight(id, OXB_FMT_Q1, aos, n_bytes, n_rows, k);
+}
+
+int oxb_hip_upload_tq2(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return upload_weight(id, OXB_FMT_TQ2, aos, n_bytes, n_rows, k);
+}
+
+int oxb_hip_free_weight(uint64_t id) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    if (g_rt.ready) (void)hipStreamSynchronize(g_rt.stream);
+    free_weight_mem(*w);
+    g_rt.weights.erase(id);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, size_t* resident_bytes) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    if (fmt) *fmt = (int)w->L.fmt;
+    if (n_rows) *n_rows = w->L.n_rows;
+    if (k) *k = w->L.k;
+    if (resident_bytes) *resident_bytes = w->L.codes_bytes + w->L.scales_bytes;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_dequant(uint64_t id, float* out, size_t out_len) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    const size_t n = (size_t)w->L.n_rows * w->L.k;
+    if (!out || out_len < n) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: output holds %zu values, %zu needed", out_len, n);
+    int rc = g_rt.ws_y.ensure(n * sizeof(float));
+    if (rc) return rc;
+    hipError_t e = oxb_launch_dequant(w->L, w->d_codes, w->d_scales, (float*)g_rt.ws_y.ptr, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "kernel launch failed: dequant");
+    e = hipMemcpyAsync(out, g_rt.ws_y.ptr, n * sizeof(float), hipMemcpyDeviceToHost, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "dequant download");
+    return sync_stream("dequant");
+}
+
+int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!d_x || !d_y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
+    return gemv_device(*w, d_x, d_y, batch, n_rows, OXB_GEMV_STORE, nullptr);
+}
+
+int oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!x || !y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
+    const size_t xb = (size_t)batch * k * sizeof(float), yb = (size_t)batch * n_rows * sizeof(float);
+    if ((rc = g_rt.ws_x.ensure(xb))) return rc;
+    if ((rc = g_rt.ws_y.ensure(yb))) return rc;
+    hipError_t e = hipMemcpyAsync(g_rt.ws_x.ptr, x, xb, hipMemcpyHostToDevice, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "input upload");
+    rc = gemv_device(*w, (const float*)g_rt.ws_x.ptr, (float*)g_rt.ws_y.ptr, batch, n_rows, OXB_GEMV_STORE, nullptr);
+    if (rc) return rc;
+    e = hipMemcpyAsync(y, g_rt.ws_y.ptr, yb, hipMemcpyDeviceToHost, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "output download");
+    return sync_stream("gemv");
+}
+
+int oxb_hip_gemv_q1_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len, float* y, size_t y_len,
+                         uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return oneshot_gemv(OXB_FMT_Q1, aos, n_bytes, x, x_len, y, y_len, n_rows, k);
+}
+
+int oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len, float* y, size_t y_len,
+                          uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return oneshot_gemv(OXB_FMT_TQ2, aos, n_bytes, x, x_len, y, y_len, n_rows, k);
+}
+
+// ---- host-only repack helpers -------------------------------------------------
+static int repack_args(int fmt, uint32_t n_rows, uint32_t k) {
+    if (fmt != OXB_FMT_Q1 && fmt != OXB_FMT_TQ2) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown format %d", fmt);
+    if (k == 0 || k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
+    if (n_rows == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: n_rows is 0");
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_repack_sizes(int fmt, uint32_t n_rows, uint32_t k, size_t* codes_bytes, size_t* scales_bytes) {
+    int rc = repack_args(fmt, n_rows, k);
+    if (rc) return rc;
+    OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
+    if (codes_bytes) *codes_bytes = L.codes_bytes;
+    if (scales_bytes) *scales_bytes = L.scales_bytes;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_repack(int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k, uint8_t* codes,
+                   size_t codes_cap, uint8_t* scales, size_t scales_cap) {
+    int rc = repack_args(fmt, n_rows, k);
+    if (rc) return rc;
+    OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
+    const size_t need = (size_t)n_rows * (k / OXB_QK) * (fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES);
+    if (!aos || n_bytes < need) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer holds %zu bytes, %zu needed", n_bytes, need);
+    if (!codes || !scales || codes_cap < L.codes_bytes || scales_cap < L.scales_bytes)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: output sections too small");
+    oxb_repack_aos_to_tiled(L, aos, reinterpret_cast<uint32_t*>(codes), reinterpret_cast<uint16_t*>(scales));
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_unpack(int fmt, const uint8_t* codes, size_t codes_len, const uint8_t* scales, size_t scales_len,
+                   uint32_t n_rows, uint32_t k, uint8_t* aos, size_t aos_cap) {
+    int rc = repack_args(fmt, n_rows, k);
+    if (rc) return rc;
+    OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
+    const size_t need = (size_t)n_rows * (k / OXB_QK) * (fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES);
+    if (!codes || !scales || codes_len < L.codes_bytes || scales_len < L.scales_bytes || !aos || aos_cap < need)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: buffer sizes do not match the layout");
+    oxb_repack_tiled_to_aos(L, reinterpret_cast<const uint32_t*>(codes), reinterpret_cast<const uint16_t*>(scales), aos);
+    return OXB_HIP_OK;
+}
+
+}  // extern "C"

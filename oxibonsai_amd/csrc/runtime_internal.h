@@ -1,0 +1,50 @@
+// runtime_internal.h — state shared by the translation units of the library.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+#include <string>
+#include <unordered_map>
+
+#include "layout.h"
+
+namespace oxb {
+
+struct DevBuf {  // grow-only device scratch
+    void* ptr = nullptr;
+    size_t cap = 0;
+    int ensure(size_t bytes);
+    void release();
+};
+
+struct Weight {  // one resident matrix: [codes section][scales section]
+    OxbLayout L;
+    void* d_base = nullptr;
+    uint32_t* d_codes = nullptr;
+    uint16_t* d_scales = nullptr;
+};
+
+struct Runtime {
+    bool ready = false;
+    int device = -1;
+    uint32_t n_cus = 0;
+    char name[256] = {0};
+    hipStream_t own_stream = nullptr, stream = nullptr;
+    std::unordered_map<uint64_t, Weight> weights;
+    uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
+    DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
+};
+
+extern Runtime g_rt;
+extern std::recursive_mutex g_mu;
+
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char* what);
+int ensure_init();
+Weight* find_weight(uint64_t id);
+int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
+int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
+                const float* d_residual);
+void shutdown_models();
+
+}  // namespace oxb

@@ -1,0 +1,214 @@
+"""GPU parity of the native-hip GEMV path against the CPU oracle, through the C ABI.
+
+Tolerances: decode bit-exact; GEMV within 1e-3 relative under the reference's own gate
+(abs_err < 1e-3 || |a-b| / max(|a|, |b|, 1e-3) < 1e-3), tightened here by a bound of
+1e-5 of the output scale and by a comparison with the float64 product."""
+import numpy as np
+import pytest
+
+import oxibonsai_amd as ox
+from helpers import (Q1, TQ2, block, cross_tier_q1, dense_f64, metal_tq2, parity_violations, q1_block, rel_err,
+                     simd_parity_tq2, tq2_block)
+from oracle import oracle
+from oxibonsai_amd import synth
+
+pytestmark = pytest.mark.gpu
+GEMV_REL_TOL = 1e-3
+
+
+def _upload(be, fmt, a, n, k):
+    return be.upload_weights_raw(a, n, k) if fmt == Q1 else be.upload_weights_ternary(a, n, k)
+
+
+def _gemv(be, fmt, h, x, n, k):
+    return be.gemv_q1_g128_cached(h, x, n, k) if fmt == Q1 else be.gemv_tq2_g128_cached(h, x, n, k)
+
+
+def test_backend_identity(backend):
+    assert backend.name() == "native-hip" and backend.is_accelerated()
+    assert backend.device_count() >= 1
+    assert "gfx950" in backend.device_name()
+    free, total = backend.memory_info()
+    assert 0 < free <= total and total > 200 * 2**30
+    backend.synchronize()
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+@pytest.mark.parametrize("shape", [(1, 128), (16, 512), (17, 640), (100, 2048), (250, 1152)])
+def test_dequant_bit_exact(backend, fmt, shape):
+    n, k = shape
+    a = synth.make_blocks(fmt, 300 + n, n, k)
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        got = backend.dequant(h)
+    finally:
+        backend.free_weights(h)
+    want = oracle.dequant(fmt, a).reshape(n, k)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_bit_exact_special_codes_and_scales(backend):
+    # all 256 code bytes (incl. the reserved 0b11 lanes) and awkward scales (subnormal, max, negative)
+    qs = np.arange(256, dtype=np.uint8).reshape(8, 32)
+    scales = [1.0, 6e-8, 65504.0, -0.375, 0.0, 3.1e-5, 0.1, 7.0]
+    a = np.concatenate([tq2_block(s, qs[i]) for i, s in enumerate(scales)])
+    h = backend.upload_weights_ternary(a, 2, 512)
+    got = backend.dequant(h)
+    backend.free_weights(h)
+    assert np.array_equal(got.view(np.uint32), oracle.dequant(TQ2, a).reshape(2, 512).view(np.uint32))
+    a = np.concatenate([q1_block(s, qs[i][:16]) for i, s in enumerate(scales)])
+    h = backend.upload_weights_raw(a, 4, 256)
+    got = backend.dequant(h)
+    backend.free_weights(h)
+    assert np.array_equal(got.view(np.uint32), oracle.dequant(Q1, a).reshape(4, 256).view(np.uint32))
+
+
+def test_reference_kats_through_the_abi(backend):
+    ones = np.ones(128, np.float32)
+    # crates/oxibonsai-kernels/src/gemv.rs:101-150, gpu_backend/mod.rs:1353-1398
+    assert abs(backend.gemv_q1_g128(q1_block(1.0, 0xFF), np.arange(128, dtype=np.float32), 1, 128)[0] - 8128.0) < 1.0
+    assert abs(backend.gemv_q1_g128(q1_block(2.0, 0x00), ones, 1, 128)[0] + 256.0) < 1.0
+    two = np.concatenate([q1_block(1.0, 0xFF), q1_block(1.0, 0x00)])
+    y = backend.gemv_q1_g128(two, ones, 2, 128)
+    assert abs(y[0] - 128.0) < 1.0 and abs(y[1] + 128.0) < 1.0
+    # two blocks per row (tests/gpu_backend_tests.rs:282-376)
+    row = np.concatenate([q1_block(0.5, 0xFF), q1_block(0.25, 0x00)])
+    assert abs(backend.gemv_q1_g128(row, np.ones(256, np.float32), 1, 256)[0] - (64.0 - 32.0)) < 1e-3
+    # crates/oxibonsai-kernels/src/gemv_ternary.rs:212-324
+    y = backend.gemv_tq2_g128(np.concatenate([tq2_block(1.0, 0xAA)] * 2), ones, 2, 128)
+    assert abs(y[0] - 128.0) < 0.5 and abs(y[1] - 128.0) < 0.5
+    y = backend.gemv_tq2_g128(np.concatenate([tq2_block(1.0, 0x00)] * 2), ones, 2, 128)
+    assert abs(y[0] + 128.0) < 0.5 and abs(y[1] + 128.0) < 0.5
+    assert abs(backend.gemv_tq2_g128(tq2_block(1.0, 0x46), ones, 1, 128)[0]) < 1e-4
+    assert abs(backend.gemv_tq2_g128(tq2_block(1.0, 0xFF), ones, 1, 128)[0]) < 1e-4
+    y = backend.gemv_tq2_g128(np.concatenate([tq2_block(1.0, 0xAA)] * 8), np.ones(256, np.float32), 4, 256)
+    assert np.all(np.abs(y - 256.0) < 1.0)
+
+
+def test_reference_generators(backend):
+    n, k = 128, 1024
+    a = cross_tier_q1(n, k)
+    x = np.array([(i % 17) * 0.25 - 2.0 for i in range(k)], dtype=np.float32)
+    got = backend.gemv_q1_g128(a, x, n, k)
+    assert np.max(np.abs(got - oracle.gemv(Q1, a, x, n, k))) < 1.0              # cross_tier.rs tolerance
+    assert np.max(rel_err(got, dense_f64(Q1, a, n, k) @ x.astype(np.float64))) < GEMV_REL_TOL
+    a, x = simd_parity_tq2(64, 128)
+    assert np.mean((backend.gemv_tq2_g128(a, x, 64, 128) - oracle.gemv(TQ2, a, x, 64, 128)) ** 2) < 1e-6
+    a = metal_tq2(64, 512)
+    x = np.array([((i * 7 + 3) % 19) * 0.1 - 0.9 for i in range(512)], dtype=np.float32)
+    assert np.max(np.abs(backend.gemv_tq2_g128(a, x, 64, 512) - oracle.gemv(TQ2, a, x, 64, 512))) < 1e-3
+
+
+# BASELINE configs 0 and 1 at full size, plus ragged / tiny / very wide shapes.
+SHAPES = [
+    (TQ2, 12288, 2048), (Q1, 6144, 4096), (Q1, 24576, 4096), (Q1, 4096, 12288),
+    (TQ2, 6144, 4096), (TQ2, 4096, 12288),
+    (Q1, 1, 128), (TQ2, 1, 128), (Q1, 37, 640), (TQ2, 250, 1152), (Q1, 1000, 2560), (TQ2, 333, 9728),
+    (Q1, 48, 12800), (Q1, 40, 20480), (TQ2, 24, 17408),
+]
+
+
+@pytest.mark.parametrize("fmt,n,k", SHAPES)
+def test_gemv_matches_oracle(backend, fmt, n, k):
+    a = synth.make_blocks(fmt, 1000 + n + k, n, k)
+    x = synth.normal_f32(77 + k, k)
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        got = _gemv(backend, fmt, h, x, n, k)
+    finally:
+        backend.free_weights(h)
+    want = oracle.gemv(fmt, a, x, n, k)
+    assert parity_violations(got, want, GEMV_REL_TOL) == 0
+    scale = np.max(np.abs(want))
+    assert np.max(np.abs(got - want)) < 1e-5 * scale                      # far below the gate
+    if n * k <= 2**25:                                                     # float64 truth where it is cheap
+        truth = dense_f64(fmt, a, n, k) @ x.astype(np.float64)
+        assert np.max(np.abs(got - truth)) <= 2 * np.max(np.abs(want - truth)) + 1e-7 * scale
+
+
+@pytest.mark.parametrize("fmt,n,k", [(Q1, 6144, 4096), (Q1, 4096, 12288), (TQ2, 12288, 2048), (Q1, 50, 384)])
+@pytest.mark.parametrize("batch", [2, 5, 8])
+def test_gemv_batched_matches_oracle(backend, fmt, n, k, batch):
+    a = synth.make_blocks(fmt, 2000 + n, n, k)
+    xs = synth.normal_f32(5, batch * k).reshape(batch, k)
+    xs[1] *= 1e-3                       # vectors of very different magnitude share a launch
+    if batch > 4:
+        xs[4] *= 250.0
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        got = backend.gemv_cached_batch(h, xs, n, k)
+    finally:
+        backend.free_weights(h)
+    want = oracle.gemm(fmt, a, xs, batch, n, k)
+    for b in range(batch):
+        scale = max(np.max(np.abs(want[b])), 1e-30)
+        assert np.max(np.abs(got[b] - want[b])) < 1e-5 * scale + 1e-6, b
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+def test_gemv_properties(backend, fmt):
+    n, k = 777, 3072
+    a = synth.make_blocks(fmt, 31, n, k)
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        x1, x2 = synth.normal_f32(1, k), synth.normal_f32(2, k)
+        y1, y2 = _gemv(backend, fmt, h, x1, n, k), _gemv(backend, fmt, h, x2, n, k)
+        y12 = _gemv(backend, fmt, h, x1 + x2, n, k)
+        assert np.max(np.abs(y12 - (y1 + y2))) < 1e-4                              # linearity
+        assert np.array_equal(_gemv(backend, fmt, h, x1, n, k), y1)                # deterministic
+        assert np.all(_gemv(backend, fmt, h, np.zeros(k, np.float32), n, k) == 0.0)  # zero input
+        assert np.max(np.abs(_gemv(backend, fmt, h, 1e-30 * x1, n, k) - 1e-30 * y1.astype(np.float64))) < 1e-35
+        assert np.max(rel_err(_gemv(backend, fmt, h, 1e20 * x1, n, k), 1e20 * y1.astype(np.float64))) < 1e-4
+        xbad = x1.copy()
+        xbad[5] = np.nan
+        assert np.all(np.isnan(_gemv(backend, fmt, h, xbad, n, k)))                 # NaN in -> NaN out
+        xo = x1.copy()
+        xo[100] = 5000.0                                                            # one massive outlier
+        want = dense_f64(fmt, a, n, k) @ xo.astype(np.float64)
+        assert np.max(np.abs(_gemv(backend, fmt, h, xo, n, k) - want)) < 1e-6 * np.max(np.abs(want))
+        assert np.array_equal(backend.gemv_cached_batch(h, np.stack([x1, x2]), n, k)[1], y2)  # gemm row = gemv
+    finally:
+        backend.free_weights(h)
+    zero = a.copy().reshape(-1, 18 if fmt == Q1 else 34)
+    zero[:, (0 if fmt == Q1 else 32):(2 if fmt == Q1 else 34)] = 0
+    h = _upload(backend, fmt, zero.reshape(-1), n, k)
+    assert np.all(_gemv(backend, fmt, h, x1, n, k) == 0.0)                          # zero scale -> 0
+    backend.free_weights(h)
+
+
+def test_error_paths(backend):
+    b = q1_block(1.0, 0xFF)
+    ones = np.ones(128, np.float32)
+    for call in (lambda: backend.gemv_q1_g128(b, np.ones(100, np.float32), 1, 100),   # k % 128
+                 lambda: backend.gemv_q1_g128(b, np.ones(64, np.float32), 1, 128),    # short input
+                 lambda: backend.gemv_q1_g128(b, ones, 2, 128),                        # short weights
+                 lambda: backend.gemv_tq2_g128(tq2_block(1.0, 0xAA), ones, 2, 128),
+                 lambda: backend.upload_weights_raw(b, 1, 100)):
+        with pytest.raises(ox.GpuError) as e:
+            call()
+        assert e.value.kind == "InvalidArgument"
+    with pytest.raises(ox.GpuError) as e:
+        backend.gemv_q1_g128_cached(0xDEAD, ones, 1, 128)
+    assert e.value.kind == "WeightNotFound"
+    h = backend.upload_weights_raw(b, 1, 128)
+    with pytest.raises(ox.GpuError) as e:
+        backend.gemv_q1_g128_cached(h, np.ones(256, np.float32), 1, 256)              # shape differs from upload
+    assert e.value.kind == "InvalidArgument"
+    assert abs(backend.gemv_q1_g128_cached(h, ones, 1, 128)[0] - 128.0) < 1e-3        # still usable afterwards
+    backend.free_weights(h)
+    with pytest.raises(ox.GpuError) as e:
+        backend.free_weights(h)
+    assert e.value.kind == "WeightNotFound"
+
+
+def test_caller_chosen_handle_ids_and_replacement(backend):
+    a1, a2 = synth.make_blocks(Q1, 1, 32, 256), synth.make_blocks(Q1, 2, 32, 256)
+    x = synth.normal_f32(3, 256)
+    h = backend.upload_weights_raw(a1, 32, 256, handle_id=4_000_000)
+    assert h == 4_000_000
+    y1 = backend.gemv_q1_g128_cached(h, x, 32, 256)
+    assert backend.upload_weights_raw(a2, 32, 256, handle_id=4_000_000) == 4_000_000   # replaces
+    y2 = backend.gemv_q1_g128_cached(h, x, 32, 256)
+    assert np.max(np.abs(y1 - oracle.gemv(Q1, a1, x, 32, 256))) < 1e-5
+    assert np.max(np.abs(y2 - oracle.gemv(Q1, a2, x, 32, 256))) < 1e-5
+    backend.free_weights(h)

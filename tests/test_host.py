@@ -1,0 +1,137 @@
+"""Host-side logic of the native-hip library that runs without a GPU: the C ABI surface,
+the AoS -> resident repack, argument validation, and the arithmetic model of the device GEMV."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+
+import kernel_model
+import oxibonsai_amd as ox
+from helpers import Q1, TQ2, block, cross_tier_q1, dense_f64, metal_tq2, simd_parity_tq2
+from oracle import oracle
+from oxibonsai_amd import _lib, synth
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "oxb_hip.h")).read()
+    declared = set(re.findall(r"\b(oxb_hip_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 15
+    L = C.CDLL(_lib.LIB_PATH)
+    missing = [s for s in sorted(declared) if not hasattr(L, s)]
+    assert not missing, missing
+    assert declared == set(_lib._SIGNATURES), declared ^ set(_lib._SIGNATURES)
+
+
+def test_static_library_is_built():
+    assert os.path.exists(os.path.join(os.path.dirname(_lib.LIB_PATH), "liboxb_hip.a"))
+
+
+def test_no_gpu_means_not_available_not_a_fallback():
+    L = _lib.lib()
+    if L.oxb_hip_device_count() > 0:
+        pytest.skip("a GPU is present")
+    with pytest.raises(ox.GpuError) as e:
+        ox.NativeHipBackend(0)
+    assert e.value.kind == "NotAvailable"
+    b = block(Q1, 1.0, 0xFF)
+    x, y = np.ones(128, np.float32), np.zeros(1, np.float32)
+    rc = L.oxb_hip_gemv_q1_g128(b.ctypes.data_as(_lib.u8p), b.size, x.ctypes.data_as(_lib.f32p), 128,
+                                y.ctypes.data_as(_lib.f32p), 1, 1, 128)
+    assert rc == 1 and "not available" in _lib.last_error().lower()
+    assert y[0] == 0.0
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+@pytest.mark.parametrize("shape", [(1, 128), (16, 512), (17, 640), (40, 1152), (100, 2048)])
+def test_repack_round_trip(fmt, shape):
+    n, k = shape
+    a = synth.make_blocks(fmt, 100 + n, n, k)
+    codes, scales = ox.repack(fmt, a, n, k)
+    assert codes.size % 1024 == 0 and scales.size % 128 == 0      # 1 KiB code units, 16-byte aligned sections
+    assert np.array_equal(ox.unpack(fmt, codes, scales, n, k), a)
+
+
+def test_repack_reserved_ternary_code_decodes_to_zero():
+    a = block(TQ2, 0.5, 0xFF)  # all 0b11
+    codes, scales = ox.repack(TQ2, a, 1, 128)
+    back = ox.unpack(TQ2, codes, scales, 1, 128)
+    assert np.all(oracle.dequant(TQ2, back) == 0.0) and np.all(oracle.dequant(TQ2, a) == 0.0)
+    mixed = block(TQ2, 0.5, 0x9C)
+    back = ox.unpack(TQ2, *ox.repack(TQ2, mixed, 1, 128), 1, 128)
+    assert np.array_equal(oracle.dequant(TQ2, back), oracle.dequant(TQ2, mixed))
+
+
+def test_repack_padding_is_zero():
+    n, k = 5, 128  # 11 padded rows, 3 padded blocks
+    a = synth.make_blocks(Q1, 9, n, k)
+    codes, scales = ox.repack(Q1, a, n, k)
+    s16 = scales.view(np.uint16).reshape(4, 4, 4)  # [rg][q][v]
+    assert np.all(s16[:, 1:, :] == 0)              # blocks 1..3 of the superblock do not exist
+    assert np.all(s16[2:, :, :] == 0) and s16[1, 0, 1] == 0
+    w = codes.view(np.uint32).reshape(64, 4)
+    assert np.all(w[:, 1:] == 0)
+
+
+def test_repack_argument_validation():
+    a = synth.make_blocks(Q1, 1, 4, 256)
+    with pytest.raises(ox.GpuError) as e:
+        ox.repack(Q1, a, 4, 200)
+    assert e.value.kind == "InvalidArgument"
+    with pytest.raises(ox.GpuError):
+        ox.repack(Q1, a[:-1], 4, 256)
+    with pytest.raises(ox.GpuError):
+        ox.repack(Q1, a, 0, 256)
+    with pytest.raises(ox.GpuError):
+        ox.repack(7, a, 4, 256)
+
+
+# ---- arithmetic model of the device GEMV against the oracle -------------------------------------
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+@pytest.mark.parametrize("shape", [(16, 128), (40, 640), (33, 1024)])
+def test_device_arithmetic_model_matches_oracle(fmt, shape):
+    n, k = shape
+    a = synth.make_blocks(fmt, 11 + fmt, n, k)
+    x = synth.normal_f32(5, k)
+    y = kernel_model.gemv(fmt, *ox.repack(fmt, a, n, k), n, k, x)
+    want = dense_f64(fmt, a, n, k) @ x.astype(np.float64)
+    yo = oracle.gemv(fmt, a, x, n, k)
+    assert np.max(np.abs(y - want)) <= max(np.max(np.abs(yo - want)) * 2, 1e-6)   # no worse than fp32 order effects
+    assert np.max(np.abs(y - yo)) < 1e-5
+
+
+def test_device_arithmetic_model_reference_kats():
+    for fmt, pat, x, want in [
+        (Q1, 0xFF, np.arange(128, dtype=np.float32), 8128.0),
+        (Q1, 0x00, np.ones(128, np.float32), -128.0),
+        (TQ2, 0xAA, np.ones(128, np.float32), 128.0),
+        (TQ2, 0x00, np.ones(128, np.float32), -128.0),
+        (TQ2, 0x46, np.ones(128, np.float32), 0.0),
+        (TQ2, 0xFF, np.ones(128, np.float32), 0.0),
+    ]:
+        a = block(fmt, 1.0, pat)
+        y = kernel_model.gemv(fmt, *ox.repack(fmt, a, 1, 128), 1, 128, x)
+        assert abs(y[0] - want) < 1e-3, (fmt, hex(pat), y[0])
+
+
+def test_device_arithmetic_model_reference_generators_and_outliers():
+    a = cross_tier_q1(32, 512)
+    x = np.array([(i % 17) * 0.25 - 2.0 for i in range(512)], dtype=np.float32)
+    y = kernel_model.gemv(Q1, *ox.repack(Q1, a, 32, 512), 32, 512, x)
+    assert np.max(np.abs(y - oracle.gemv(Q1, a, x, 32, 512))) < 1e-2     # outputs are O(1000)
+    a, x = simd_parity_tq2(16, 128)
+    y = kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 128), 16, 128, x)
+    assert np.mean((y - oracle.gemv(TQ2, a, x, 16, 128)) ** 2) < 1e-6
+    a = metal_tq2(16, 256)
+    # one activation 1000x larger than the rest: the per-vector exponent must not wash out the others
+    x = synth.normal_f32(3, 256)
+    x[17] = 3000.0
+    y = kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 256), 16, 256, x)
+    want = dense_f64(TQ2, a, 16, 256) @ x.astype(np.float64)
+    assert np.max(np.abs(y - want)) < 1e-3 * 1e-3 * np.max(np.abs(want)) + 1e-4
+    assert np.all(kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 256), 16, 256, np.zeros(256, np.float32)) == 0)
+    x[3] = np.inf
+    assert np.all(np.isnan(kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 256), 16, 256, x)))
