@@ -67,10 +67,17 @@ int  oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, s
 int  oxb_hip_dequant(uint64_t id, float* out, size_t out_len);
 
 /* ---- GEMV / GEMM on resident weights: gemv_q1_g128_cached (KG/mod.rs:457), gemv_tq2_g128_cached (:484).
- * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per <= 4 vectors). */
+ * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per two vectors). */
 int  oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch);
 /* Same with device-resident x / y, asynchronous on the current stream. */
 int  oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch);
+
+/* Measurement aid (the reference's counterpart is its CUDA_PROFILE / OXIBONSAI_PROFILE_GPU instrumentation,
+ * KG/cuda_full_layer/mod.rs:339-344, KG/metal_full_layer/functions.rs:17-35): quantise d_x once, then launch the
+ * GEMV kernel alone `iters` times, launch i on weight ids[i % n_ids] (same shape and format), bracketed by HIP
+ * events on the stream the kernel runs on.  *avg_us = mean time per launch in microseconds. */
+int  oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y,
+                          uint32_t n_rows, uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us);
 
 /* ---- uncached one-shot calls: gemv_q1_g128 (KG/mod.rs:412), gemm_q1_g128 (:425) and their ternary twins.
  * Validation follows the scalar kernels (crates/oxibonsai-kernels/src/gemv.rs:32-58): k % 128, buffer lengths. */

@@ -32,6 +32,8 @@ _SIGNATURES = {
     "oxb_hip_dequant": ([C.c_uint64, f32p, C.c_size_t], C.c_int),
     "oxb_hip_gemv": ([C.c_uint64, f32p, f32p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_gemv_dev": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
+    "oxb_hip_profile_gemv": ([u64p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
+                              C.c_uint32, f32p], C.c_int),
     "oxb_hip_gemv_q1_g128": ([u8p, C.c_size_t, f32p, C.c_size_t, f32p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_gemv_tq2_g128": ([u8p, C.c_size_t, f32p, C.c_size_t, f32p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_repack_sizes": ([C.c_int, C.c_uint32, C.c_uint32, szp, szp], C.c_int),

@@ -103,7 +103,7 @@ class NativeHipBackend:
 
     def gemm_q1_g128(self, block_bytes, input, m: int, n_rows: int, k: int) -> np.ndarray:
         """[m x k] inputs -> [m x n_rows]; the trait's default loops GEMV per row (mod.rs:425-440),
-        here the weights are uploaded once and streamed once per four input rows."""
+        here the weights are uploaded once and streamed once per two input rows."""
         return self._oneshot_gemm(Q1, block_bytes, input, m, n_rows, k)
 
     def gemm_tq2_g128(self, block_bytes, input, m: int, n_rows: int, k: int) -> np.ndarray:

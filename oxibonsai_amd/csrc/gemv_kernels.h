@@ -5,6 +5,8 @@
 
 #include "layout.h"
 
+#define OXB_GEMV_MAX_BATCH 2  // activation vectors per pass over the weights
+#define OXB_GEMV_MAX_SB 24    // superblocks (512 weights of K) one launch covers: 8 waves x 3
 enum { OXB_GEMV_STORE = 0, OXB_GEMV_ACCUM = 1, OXB_GEMV_RESIDUAL = 2 };
 
 struct OxbGemvParams {
@@ -17,7 +19,7 @@ struct OxbGemvParams {
     const float* residual;   // [batch][ldy], mode RESIDUAL only
     uint32_t n_rows, n_tiles, n_sb;
     uint32_t sb_begin, sb_count;  // K range handled by this launch, in superblocks
-    uint32_t NC;                  // 4 * batch, batch <= 4
+    uint32_t NC;                  // 8 * batch, batch <= 2 (eight digit columns per vector)
     uint32_t ldy;
     uint32_t slots;               // filled by the launcher
     int mode;

@@ -10,10 +10,11 @@
 // 1/4 VALU op: one AND with 0x01010101 << j (Q1) or 0x03030303 << 2jj (TQ2)
 // turns a code dword into four int8 MFMA operands worth 2^j (4^jj) each, and the
 // activation vector is pre-divided by the same power of two when it is
-// quantised.  The fp32 activation is carried exactly enough: each x is scaled by
-// a per-vector power of two to a 30-bit integer and split into four balanced
-// int8 digits which occupy four MFMA columns, so one 16x16x64 MFMA multiplies
-// 16 rows x 64 weights by all four digits (and up to four batch columns).
+// quantised.  The fp32 activation is carried exactly: each x is scaled by a
+// per-vector power of two to a 54-bit integer (every element within 2^22 of the
+// largest one keeps all 24 mantissa bits) and split into eight balanced int8
+// digits which occupy eight MFMA columns, so one 16x16x64 MFMA multiplies 16
+// rows x 64 weights by all eight digits of up to two activation vectors.
 // Block sums are exact integers; the per-block f16 scale is applied in fp32.
 //
 // Kernels:
@@ -29,28 +30,97 @@
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
-#define OXB_XQ_P 29  // |x * 2^(P-E)| < 2^29, doubled values stay below 2^30
+#define OXB_XQ_P 53  // |x * 2^(P-E)| < 2^53, doubled values stay below 2^54
+#define OXB_XQ_DIGITS 8
 
 // ---------------------------------------------------------------------------
 // Activation quantiser.
 //
-// Output, for vector n of the batch (NC = 4*batch columns, column c = 4n+digit):
+// Output, for vector n of the batch (NC = 8*batch columns, column c = 8n+digit):
 //   xq  [((blk*2+m)*4+g)*NC + c][jj]  one dword = 4 int8 (bb = 0..3), the MFMA
 //        B operand of lane (c,g), register jj, of MFMA m of block blk;
-//        Q1 : element bb is digit(c%4) of  s_j * 2*r(k),  k = 128blk+32g+8bb+j, j = 4m+jj,
+//        Q1 : element bb is digit(c%8) of  s_j * 2*r(k),  k = 128blk+32g+8bb+j, j = 4m+jj,
 //             r(k) = rint(x[k] * 2^(P-E-j)),  s_j = -1 for j = 7 (0x80 is -128 as int8)
-//        TQ2: element bb is digit(c%4) of  r(k) = rint(x[k] * 2^(P-E-2jj)), k = 128blk+32g+16m+4bb+jj
+//        TQ2: element bb is digit(c%8) of  r(k) = rint(x[k] * 2^(P-E-2jj)), k = 128blk+32g+16m+4bb+jj
 //   cneg[blk][c][0..3]  four copies of -C, C = the part of the block sum that the
 //        biased encodings add (Q1: sum_k 2^j digit(r); TQ2: sum_{jj<3} 4^jj digit(r)),
 //        used as the MFMA accumulator's start value;
 //   xexp[n]  E - P, or INT_MIN when the vector holds a NaN or an infinity.
 // ---------------------------------------------------------------------------
+#define OXB_QUANT_THREADS 512
+
+// rint(v * 2^shift) as a 64-bit integer, using fp32 operations only.  Scaling by a power of
+// two is exact, rintf is exact, and the split at 2^27 leaves two parts that fit an int32.
+__device__ __forceinline__ long long scaled_rint_i64(float v, int shift) {
+    const float r = rintf(ldexpf(v, shift));              // |r| < 2^54, an integer
+    const float hi = truncf(r * 7.450580596923828e-09f);  // r / 2^27
+    const float lo = r - hi * 134217728.0f;               // exact: |lo| < 2^27
+    return ((long long)(int)hi << 27) + (long long)(int)lo;
+}
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+// Quantise the 16 activations that one lane group (blk, m, g) of the MFMA B operand holds and
+// store their eight digit planes; returns nothing, accumulates the block's correction sums.
 template <int FMT>
-__global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ x, uint32_t k, uint32_t nblk_pad,
-                                                       uint32_t NC, uint32_t* __restrict__ xq,
-                                                       int32_t* __restrict__ cneg, int32_t* __restrict__ xexp) {
-    extern __shared__ int32_t csum[];  // [nblk_pad][4]
-    __shared__ float red[256];
+__device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_t blk, uint32_t m, uint32_t g,
+                                           int base_shift, bool live, uint32_t NC, uint32_t n,
+                                           uint32_t* __restrict__ xq, int cs[8]) {
+    uint32_t out[8][4];
+#pragma unroll
+    for (int d = 0; d < 8; d++) {
+        cs[d] = 0;
+        out[d][0] = out[d][1] = out[d][2] = out[d][3] = 0;
+    }
+    if (live) {
+        const float* xb = xn + blk * 128 + 32 * g;
+#pragma unroll
+        for (uint32_t bb = 0; bb < 4; bb++) {
+            // Q1: k = 8bb + 4m + jj;  TQ2: k = 16m + 4bb + jj   (jj = 0..3 contiguous)
+            const float4 v4 = *reinterpret_cast<const float4*>(xb + (FMT == OXB_FMT_Q1 ? 8 * bb + 4 * m : 16 * m + 4 * bb));
+            const float vv[4] = {v4.x, v4.y, v4.z, v4.w};
+#pragma unroll
+            for (uint32_t jj = 0; jj < 4; jj++) {
+                long long xi, cr;
+                int cmul;
+                if (FMT == OXB_FMT_Q1) {
+                    const uint32_t j = 4 * m + jj;
+                    const long long r = scaled_rint_i64(vv[jj], base_shift - (int)j);
+                    xi = (j == 7) ? -2 * r : 2 * r;
+                    cr = r;
+                    cmul = 1 << j;
+                } else {
+                    xi = scaled_rint_i64(vv[jj], base_shift - 2 * (int)jj);
+                    cr = xi;
+                    cmul = (jj < 3) ? (1 << (2 * jj)) : 0;
+                }
+                // balanced base-256 digits: byte d of t is the signed digit d
+                const unsigned long long bias = 0x0080808080808080ull;
+                const unsigned long long t = ((unsigned long long)xi + bias) ^ bias;
+                const unsigned long long tc = ((unsigned long long)cr + bias) ^ bias;
+#pragma unroll
+                for (int d = 0; d < 8; d++) {
+                    out[d][jj] |= (uint32_t)((t >> (8 * d)) & 0xFFu) << (8 * bb);
+                    cs[d] += (int)(int8_t)(tc >> (8 * d)) * cmul;
+                }
+            }
+        }
+    }
+    uint4* dst = reinterpret_cast<uint4*>(xq) + (size_t)((blk * 2 + m) * 4 + g) * NC + 8 * n;
+#pragma unroll
+    for (int d = 0; d < 8; d++) dst[d] = make_uint4(out[d][0], out[d][1], out[d][2], out[d][3]);
+}
+
+template <int FMT>
+__global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float* __restrict__ x, uint32_t k,
+                                                                     uint32_t nblk_pad, uint32_t NC,
+                                                                     uint32_t* __restrict__ xq,
+                                                                     int32_t* __restrict__ cneg,
+                                                                     int32_t* __restrict__ xexp) {
+    __shared__ float red[OXB_QUANT_THREADS / 64];
     __shared__ int bad_flag;
     const uint32_t n = blockIdx.x, tid = threadIdx.x;
     const float* xn = x + (size_t)n * k;
@@ -58,75 +128,47 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
     if (tid == 0) bad_flag = 0;
     float mx = 0.0f;
     int bad = 0;
-    for (uint32_t i = tid; i < k; i += 256) {
-        float v = xn[i];
-        bad |= !(fabsf(v) <= 3.402823466e38f);
-        mx = fmaxf(mx, fabsf(v));
+    for (uint32_t i = tid * 4; i < k; i += OXB_QUANT_THREADS * 4) {
+        const float4 v = *reinterpret_cast<const float4*>(xn + i);
+        const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        bad |= !(fabsf(v.x) <= 3.402823466e38f) | !(fabsf(v.y) <= 3.402823466e38f) |
+               !(fabsf(v.z) <= 3.402823466e38f) | !(fabsf(v.w) <= 3.402823466e38f);
+        mx = fmaxf(mx, a);
     }
-    red[tid] = mx;
-    for (uint32_t i = tid; i < nblk_pad * 4; i += 256) csum[i] = 0;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    if ((tid & 63u) == 0) red[tid >> 6] = mx;
     __syncthreads();
     if (bad) bad_flag = 1;
-    for (uint32_t s = 128; s > 0; s >>= 1) {
-        if (tid < s) red[tid] = fmaxf(red[tid], red[tid + s]);
-        __syncthreads();
-    }
     mx = red[0];
+#pragma unroll
+    for (int i = 1; i < OXB_QUANT_THREADS / 64; i++) mx = fmaxf(mx, red[i]);
+    __syncthreads();
     int E = 0;
     if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
     const int base_shift = OXB_XQ_P - E;
     const uint32_t nblk = k / OXB_QK;
+    const bool ok = mx > 0.0f && !bad_flag;
 
-    for (uint32_t u = tid; u < nblk_pad * 32; u += 256) {
-        const uint32_t blk = u >> 5, m = (u >> 4) & 1u, g = (u >> 2) & 3u, jj = u & 3u;
-        uint32_t out[4] = {0, 0, 0, 0};
-        if (blk < nblk && mx > 0.0f && !bad_flag) {
-            int c0 = 0, c1 = 0, c2 = 0, c3 = 0;
+    // unit u = (blk, m, g): eight consecutive lanes cover one block
+    for (uint32_t u = tid; u < nblk_pad * 8; u += OXB_QUANT_THREADS) {
+        const uint32_t blk = u >> 3, m = (u >> 2) & 1u, g = u & 3u;
+        int cs[8];
+        quant_unit<FMT>(xn, blk, m, g, base_shift, ok && blk < nblk, NC, n, xq, cs);
+        // sum the correction over the block's eight lanes: i <-> 7-i, then within quads
 #pragma unroll
-            for (uint32_t bb = 0; bb < 4; bb++) {
-                int xi, cr, cmul;
-                if (FMT == OXB_FMT_Q1) {
-                    const uint32_t j = 4 * m + jj;
-                    const float v = xn[blk * 128 + 32 * g + 8 * bb + j];
-                    const int r = (int)rintf(ldexpf(v, base_shift - (int)j));
-                    xi = (j == 7) ? -2 * r : 2 * r;
-                    cr = r;
-                    cmul = 1 << j;
-                } else {
-                    const float v = xn[blk * 128 + 32 * g + 16 * m + 4 * bb + jj];
-                    xi = (int)rintf(ldexpf(v, base_shift - 2 * (int)jj));
-                    cr = xi;
-                    cmul = (jj < 3) ? (1 << (2 * jj)) : 0;
-                }
-                // balanced base-256 digits: byte d of t is the signed digit d
-                const uint32_t t = ((uint32_t)xi + 0x00808080u) ^ 0x00808080u;
-                out[0] |= ((t >> 0) & 0xFFu) << (8 * bb);
-                out[1] |= ((t >> 8) & 0xFFu) << (8 * bb);
-                out[2] |= ((t >> 16) & 0xFFu) << (8 * bb);
-                out[3] |= ((t >> 24) & 0xFFu) << (8 * bb);
-                const uint32_t tc = ((uint32_t)cr + 0x00808080u) ^ 0x00808080u;
-                c0 += (int)(int8_t)(tc >> 0) * cmul;
-                c1 += (int)(int8_t)(tc >> 8) * cmul;
-                c2 += (int)(int8_t)(tc >> 16) * cmul;
-                c3 += (int)(int8_t)(tc >> 24) * cmul;
-            }
-            atomicAdd(&csum[blk * 4 + 0], c0);
-            atomicAdd(&csum[blk * 4 + 1], c1);
-            atomicAdd(&csum[blk * 4 + 2], c2);
-            atomicAdd(&csum[blk * 4 + 3], c3);
+        for (int d = 0; d < 8; d++) {
+            int v = cs[d];
+            v += dpp_i32<0x141>(v);   // row_half_mirror
+            v += dpp_i32<0xB1>(v);    // quad_perm [1,0,3,2]
+            v += dpp_i32<0x4E>(v);    // quad_perm [2,3,0,1]
+            cs[d] = v;
         }
-        const size_t base = ((size_t)((blk * 2 + m) * 4 + g) * NC + 4 * n) * 4 + jj;
-        xq[base + 0] = out[0];
-        xq[base + 4] = out[1];
-        xq[base + 8] = out[2];
-        xq[base + 12] = out[3];
-    }
-    __syncthreads();
-    for (uint32_t i = tid; i < nblk_pad * 4; i += 256) {
-        const uint32_t blk = i >> 2, dgt = i & 3u;
-        const int c = -csum[i];
-        int4 v = make_int4(c, c, c, c);
-        *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 4 * n + dgt) * 4) = v;
+        // lane j of the eight writes digit j (four copies: the MFMA takes it as a 4-register operand)
+        int mine = cs[0];
+#pragma unroll
+        for (int d = 1; d < 8; d++) mine = ((u & 7u) == (uint32_t)d) ? cs[d] : mine;
+        *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + (u & 7u)) * 4) = make_int4(-mine, -mine, -mine, -mine);
     }
     if (tid == 0) xexp[n] = bad_flag ? INT32_MIN : (mx > 0.0f ? E - OXB_XQ_P : 0);
 }
@@ -137,24 +179,99 @@ __global__ __launch_bounds__(256) void quant_x_kernel(const float* __restrict__ 
 // the matching slice of the digit planes in registers for the whole kernel, so
 // the inner loop is: one coalesced 1 KiB code load per superblock, 4 ANDs + 1
 // MFMA per 64 weights of 16 rows, 4 cvt + 4 fma per block for the scale.
-// Partial row sums of the S waves meet in LDS; the last step recombines the
-// four digit columns and applies the epilogue (store / += / SwiGLU).
+// The eight digit columns are weighed and added across lanes (DPP), the partial
+// row sums of the S waves meet in LDS and the last step applies the epilogue (store / +=).
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
 }
 
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {  // DPP move, out-of-range lanes read 0
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+#define OXB_DPP_ROW_SHR(n) (0x110 + (n))
+#define OXB_DPP_ROW_NEWBCAST(n) (0x150 + (n))  // lane n of each 16-lane row to the whole row
+
+// Codes and scales of one row tile, restricted to this wave's K slice, as they wait in registers.
+template <int FMT, int NSBW>
+struct TileRegs {
+    static constexpr int UNITS = (FMT == OXB_FMT_Q1) ? 1 : 2;  // 1 KiB code units per superblock
+    v4i w[NSBW][UNITS];
+    uint32_t sc[NSBW];  // lane (c, rg): f16 pair (c & 7) of row group rg, pair 2q+p = scales of block q, rows 2p, 2p+1
+};
+
+template <int FMT, int NSBW>
+__device__ __forceinline__ void load_tile(TileRegs<FMT, NSBW>& t, const v4i* __restrict__ codes,
+                                          const uint32_t* __restrict__ scales, uint32_t tile, uint32_t n_sb, int sb0,
+                                          int nsb_w, uint32_t lane) {
+    constexpr int UNITS = TileRegs<FMT, NSBW>::UNITS;
+#pragma unroll
+    for (int i = 0; i < NSBW; i++) {
+        if (i < nsb_w) {
+            const size_t unit = (size_t)tile * n_sb + (uint32_t)(sb0 + i);
+#pragma unroll
+            for (int u = 0; u < UNITS; u++) t.w[i][u] = codes[(unit * UNITS + u) * 64 + lane];
+            t.sc[i] = scales[unit * 32 + (lane >> 4) * 8 + (lane & 7u)];
+        }
+    }
+}
+
+// One block: two MFMAs over its 128 weights, then the f16 scale in fp32.
+template <int FMT, int Q>
+__device__ __forceinline__ void block_mac(v4f& accf, uint32_t d0, uint32_t d1, const v4i& b0, const v4i& b1,
+                                          const v4i& c4, uint32_t scdw) {
+    v4i a0, a1;
+    if (FMT == OXB_FMT_Q1) {  // d0 == d1: 32 sign bits
+        a0 = (v4i){(int)(d0 & 0x01010101u), (int)(d0 & 0x02020202u), (int)(d0 & 0x04040404u), (int)(d0 & 0x08080808u)};
+        a1 = (v4i){(int)(d0 & 0x10101010u), (int)(d0 & 0x20202020u), (int)(d0 & 0x40404040u), (int)(d0 & 0x80808080u)};
+    } else {  // 16 two-bit fields each
+        a0 = (v4i){(int)(d0 & 0x03030303u), (int)(d0 & 0x0C0C0C0Cu), (int)(d0 & 0x30303030u), (int)(d0 & 0xC0C0C0C0u)};
+        a1 = (v4i){(int)(d1 & 0x03030303u), (int)(d1 & 0x0C0C0C0Cu), (int)(d1 & 0x30303030u), (int)(d1 & 0xC0C0C0C0u)};
+    }
+    v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, c4, 0, 0, 0);
+    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, acc, 0, 0, 0);
+    const uint32_t p0 = dpp_u32<OXB_DPP_ROW_NEWBCAST(2 * Q)>(scdw);      // scales of rows 4g+0, 4g+1
+    const uint32_t p1 = dpp_u32<OXB_DPP_ROW_NEWBCAST(2 * Q + 1)>(scdw);  // rows 4g+2, 4g+3
+    accf[0] = fmaf((float)acc[0], f16_bits_to_f32(p0 & 0xFFFFu), accf[0]);
+    accf[1] = fmaf((float)acc[1], f16_bits_to_f32(p0 >> 16), accf[1]);
+    accf[2] = fmaf((float)acc[2], f16_bits_to_f32(p1 & 0xFFFFu), accf[2]);
+    accf[3] = fmaf((float)acc[3], f16_bits_to_f32(p1 >> 16), accf[3]);
+}
+
 template <int FMT, int NSBW, int SMAX>
-__global__ __launch_bounds__(SMAX * 64) void gemv_mfma_kernel(const OxbGemvParams p) {
-    extern __shared__ float part[];  // [slot][S][NC][16]
+__global__ __launch_bounds__(SMAX * 64, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(const OxbGemvParams p) {
+    extern __shared__ float part[];  // [slot][S][batch][16]
+    constexpr int UNITS = TileRegs<FMT, NSBW>::UNITS;
+    constexpr int TG = (8 / (NSBW * UNITS)) > 0 ? (8 / (NSBW * UNITS)) : 1;  // row tiles in flight per wave
     const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
     const uint32_t c = lane & 15u, g = lane >> 4;  // B operand: column c, k-group g; D: column c, rows 4g..4g+3
-    const uint32_t NC = p.NC;
+    const uint32_t NC = p.NC, batch = NC >> 3;
     const bool col_on = c < NC;
 
     const int sb0 = (int)(p.sb_begin + s * NSBW);
     int nsb_w = (int)(p.sb_begin + p.sb_count) - sb0;
     nsb_w = nsb_w < 0 ? 0 : (nsb_w > NSBW ? NSBW : nsb_w);
+
+    // Contiguous range of row tiles for this workgroup.
+    const uint32_t G = gridDim.x, wg = blockIdx.x;
+    const uint32_t base_cnt = p.n_tiles / G, rem = p.n_tiles % G;
+    const uint32_t t_begin = wg * base_cnt + (wg < rem ? wg : rem);
+    const uint32_t t_count = base_cnt + (wg < rem ? 1u : 0u);
+
+    const v4i* codes = reinterpret_cast<const v4i*>(p.codes);
+    const uint32_t* scales = reinterpret_cast<const uint32_t*>(p.scales);
+
+    // Start the weight stream first: the HBM latency of the first TG tiles overlaps the
+    // (L2-resident) digit-plane loads below.
+    TileRegs<FMT, NSBW> ring[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++)
+        if ((uint32_t)t < t_count) load_tile<FMT, NSBW>(ring[t], codes, scales, t_begin + t, p.n_sb, sb0, nsb_w, lane);
 
     // Digit planes and accumulator start values of this wave's K slice.
     v4i B[NSBW][4][2];
@@ -172,87 +289,71 @@ __global__ __launch_bounds__(SMAX * 64) void gemv_mfma_kernel(const OxbGemvParam
                 C4[i][q] = reinterpret_cast<const v4i*>(p.cneg)[(size_t)blk * NC + c];
             }
         }
+    // Column c carries digit (c & 7) of vector (c >> 3): its partial sums weigh 2^(8 digit + E - P).
+    const int xe = col_on ? p.xexp[c >> 3] : 0;
+    const int my_exp = (xe == INT32_MIN ? 0 : xe) + 8 * (int)(c & 7u);
 
-    // Contiguous range of row tiles for this workgroup.
-    const uint32_t G = gridDim.x, wg = blockIdx.x;
-    const uint32_t base_cnt = p.n_tiles / G, rem = p.n_tiles % G;
-    const uint32_t t_begin = wg * base_cnt + (wg < rem ? wg : rem);
-    const uint32_t t_count = base_cnt + (wg < rem ? 1u : 0u);
-    const uint32_t max_count = base_cnt + (rem ? 1u : 0u);  // uniform barrier count across the grid is not needed,
-                                                            // but it must be uniform inside the workgroup: it is.
-    (void)max_count;
-
-    const v4i* codes = reinterpret_cast<const v4i*>(p.codes);
-    const v4i* scales = reinterpret_cast<const v4i*>(p.scales);
-    constexpr int UNITS = (FMT == OXB_FMT_Q1) ? 1 : 2;  // 1 KiB code units per superblock
-
-    for (uint32_t chunk0 = 0; chunk0 < t_count; chunk0 += p.slots) {
-        const uint32_t chunk_n = (t_count - chunk0) < p.slots ? (t_count - chunk0) : p.slots;
-        for (uint32_t sl = 0; sl < chunk_n; sl++) {
-            const uint32_t tile = t_begin + chunk0 + sl;
-            v4f accf = {0.f, 0.f, 0.f, 0.f};
+    uint32_t sl = 0, chunk0 = 0;  // slots filled in the LDS chunk, first tile of the chunk
+    for (uint32_t lt0 = 0; lt0 < t_count; lt0 += TG) {
 #pragma unroll
-            for (int i = 0; i < NSBW; i++) {
-                if (i < nsb_w) {
-                    const size_t unit = (size_t)tile * p.n_sb + (uint32_t)(sb0 + i);
-                    v4i w[UNITS];
+        for (int t = 0; t < TG; t++) {
+            const uint32_t lt = lt0 + t;
+            if (lt < t_count) {  // uniform over the workgroup
+                v4f accf = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                    for (int u = 0; u < UNITS; u++) w[u] = codes[(unit * UNITS + u) * 64 + lane];
-                    const v4i sc0 = scales[(unit * 4 + g) * 2 + 0];  // f16 [q=0,1][v]
-                    const v4i sc1 = scales[(unit * 4 + g) * 2 + 1];  // f16 [q=2,3][v]
-#pragma unroll
-                    for (int q = 0; q < 4; q++) {
-                        v4i a0, a1;
+                for (int i = 0; i < NSBW; i++) {
+                    if (i < nsb_w) {
+                        const TileRegs<FMT, NSBW>& r = ring[t];
                         if (FMT == OXB_FMT_Q1) {
-                            const uint32_t wq = (uint32_t)w[0][q];
-                            a0 = (v4i){(int)(wq & 0x01010101u), (int)(wq & 0x02020202u), (int)(wq & 0x04040404u),
-                                       (int)(wq & 0x08080808u)};
-                            a1 = (v4i){(int)(wq & 0x10101010u), (int)(wq & 0x20202020u), (int)(wq & 0x40404040u),
-                                       (int)(wq & 0x80808080u)};
+                            block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][0], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
+                            block_mac<FMT, 1>(accf, r.w[i][0][1], r.w[i][0][1], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
+                            block_mac<FMT, 2>(accf, r.w[i][0][2], r.w[i][0][2], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
+                            block_mac<FMT, 3>(accf, r.w[i][0][3], r.w[i][0][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
                         } else {
-                            const uint32_t d0 = (uint32_t)w[q >> 1][(q & 1) * 2 + 0];
-                            const uint32_t d1 = (uint32_t)w[q >> 1][(q & 1) * 2 + 1];
-                            a0 = (v4i){(int)(d0 & 0x03030303u), (int)(d0 & 0x0C0C0C0Cu), (int)(d0 & 0x30303030u),
-                                       (int)(d0 & 0xC0C0C0C0u)};
-                            a1 = (v4i){(int)(d1 & 0x03030303u), (int)(d1 & 0x0C0C0C0Cu), (int)(d1 & 0x30303030u),
-                                       (int)(d1 & 0xC0C0C0C0u)};
+                            block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][1], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
+                            block_mac<FMT, 1>(accf, r.w[i][0][2], r.w[i][0][3], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
+                            block_mac<FMT, 2>(accf, r.w[i][UNITS - 1][0], r.w[i][UNITS - 1][1], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
+                            block_mac<FMT, 3>(accf, r.w[i][UNITS - 1][2], r.w[i][UNITS - 1][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
                         }
-                        v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, B[i][q][0], C4[i][q], 0, 0, 0);
-                        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, B[i][q][1], acc, 0, 0, 0);
-                        const v4i sc = (q < 2) ? sc0 : sc1;
-                        const uint32_t lo = (uint32_t)sc[(q & 1) * 2 + 0], hi = (uint32_t)sc[(q & 1) * 2 + 1];
-                        accf[0] = fmaf((float)acc[0], f16_bits_to_f32(lo & 0xFFFFu), accf[0]);
-                        accf[1] = fmaf((float)acc[1], f16_bits_to_f32(lo >> 16), accf[1]);
-                        accf[2] = fmaf((float)acc[2], f16_bits_to_f32(hi & 0xFFFFu), accf[2]);
-                        accf[3] = fmaf((float)acc[3], f16_bits_to_f32(hi >> 16), accf[3]);
                     }
                 }
-            }
-            if (col_on) *reinterpret_cast<v4f*>(&part[(((size_t)sl * S + s) * NC + c) * 16 + g * 4]) = accf;
-        }
-        __syncthreads();
-        // Recombine: thread -> (slot, batch column n, row); fixed summation order over waves.
-        const uint32_t batch = NC >> 2;
-        for (uint32_t idx = threadIdx.x; idx < chunk_n * batch * 16; idx += blockDim.x) {
-            const uint32_t r = idx & 15u, n = (idx >> 4) % batch, sl = idx / (16 * batch);
-            const uint32_t row = (t_begin + chunk0 + sl) * 16 + r;
-            if (row >= p.n_rows) continue;
-            float f[4];
+                // refill this ring slot with the tile TG ahead
+                if (lt + TG < t_count)
+                    load_tile<FMT, NSBW>(ring[t], codes, scales, t_begin + lt + TG, p.n_sb, sb0, nsb_w, lane);
+                // weigh the digit, then add the eight digit columns of each vector (lanes c-7..c of the row)
 #pragma unroll
-            for (int dgt = 0; dgt < 4; dgt++) {
-                float a = 0.f;
-                for (uint32_t w = 0; w < S; w++) a += part[(((size_t)sl * S + w) * NC + 4 * n + dgt) * 16 + r];
-                f[dgt] = a;
+                for (int v = 0; v < 4; v++) {
+                    float a = ldexpf(accf[v], my_exp);
+                    a += dpp_f32<OXB_DPP_ROW_SHR(1)>(a);
+                    a += dpp_f32<OXB_DPP_ROW_SHR(2)>(a);
+                    a += dpp_f32<OXB_DPP_ROW_SHR(4)>(a);
+                    accf[v] = a;
+                }
+                if (col_on && (c & 7u) == 7u)
+                    *reinterpret_cast<v4f*>(&part[(((size_t)(sl + t) * S + s) * batch + (c >> 3)) * 16 + g * 4]) = accf;
             }
-            float v = fmaf(fmaf(fmaf(f[3], 256.f, f[2]), 256.f, f[1]), 256.f, f[0]);
-            const int e = p.xexp[n];
-            v = (e == INT32_MIN) ? __int_as_float(0x7FC00000) : ldexpf(v, e);
-            const size_t o = (size_t)n * p.ldy + row;
-            if (p.mode == OXB_GEMV_ACCUM) v += p.y[o];
-            else if (p.mode == OXB_GEMV_RESIDUAL) v += p.residual[o];
-            p.y[o] = v;
         }
-        __syncthreads();
+        const uint32_t done = (t_count - lt0) < (uint32_t)TG ? (t_count - lt0) : (uint32_t)TG;
+        sl += done;
+        if (sl + TG > p.slots || lt0 + TG >= t_count) {
+            __syncthreads();
+            // thread -> (slot, vector n, row): sum the S partial results in a fixed order.
+            for (uint32_t idx = threadIdx.x; idx < sl * batch * 16; idx += blockDim.x) {
+                const uint32_t r = idx & 15u, n = (idx >> 4) % batch, slot = idx / (16 * batch);
+                const uint32_t row = (t_begin + chunk0 + slot) * 16 + r;
+                if (row >= p.n_rows) continue;
+                float v = 0.f;
+                for (uint32_t w = 0; w < S; w++) v += part[(((size_t)slot * S + w) * batch + n) * 16 + r];
+                if (p.xexp[n] == INT32_MIN) v = __int_as_float(0x7FC00000);
+                const size_t o = (size_t)n * p.ldy + row;
+                if (p.mode == OXB_GEMV_ACCUM) v += p.y[o];
+                else if (p.mode == OXB_GEMV_RESIDUAL) v += p.residual[o];
+                p.y[o] = v;
+            }
+            __syncthreads();
+            chunk0 += sl;
+            sl = 0;
+        }
     }
 }
 
@@ -286,61 +387,66 @@ __global__ __launch_bounds__(256) void dequant_kernel(OxbLayout L, const uint32_
 // Host-side launchers.
 // ---------------------------------------------------------------------------
 size_t oxb_xq_bytes(uint32_t k, uint32_t batch) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = 4 * batch;
+    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
     return (size_t)nblk_pad * 8 * NC * 16;
 }
 size_t oxb_cneg_bytes(uint32_t k, uint32_t batch) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = 4 * batch;
+    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
     return (size_t)nblk_pad * NC * 16;
 }
 
 hipError_t oxb_launch_quant_x(int fmt, const float* d_x, uint32_t k, uint32_t batch, uint32_t* d_xq, int32_t* d_cneg,
                               int32_t* d_xexp, hipStream_t st) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = 4 * batch;
-    const size_t shm = (size_t)nblk_pad * 4 * sizeof(int32_t);
+    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
+    const size_t shm = 0;
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, dim3(batch), dim3(256), shm, st, d_x, k, nblk_pad, NC, d_xq,
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, dim3(batch), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
                            d_cneg, d_xexp);
     else
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, dim3(batch), dim3(256), shm, st, d_x, k, nblk_pad, NC, d_xq,
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, dim3(batch), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
                            d_cneg, d_xexp);
     return hipGetLastError();
 }
 
 template <int FMT, int NSBW, int SMAX>
-static hipError_t launch_gemv_t(const OxbGemvParams& p, uint32_t S, uint32_t grid, size_t shm, hipStream_t st) {
-    hipLaunchKernelGGL((gemv_mfma_kernel<FMT, NSBW, SMAX>), dim3(grid), dim3(S * 64), shm, st, p);
+static hipError_t launch_gemv_t(OxbGemvParams p, uint32_t S, uint32_t n_cus, hipStream_t st) {
+    // Grid = what is resident at once, so every workgroup starts immediately and streams its
+    // share of row tiles; partial sums of at most `slots` tiles wait in LDS for the recombination.
+    constexpr uint32_t UNITS = (FMT == OXB_FMT_Q1) ? 1 : 2;
+    constexpr uint32_t TG = (8 / (NSBW * UNITS)) > 0 ? (8 / (NSBW * UNITS)) : 1;  // as in the kernel
+    const size_t per_slot = (size_t)S * (p.NC / 8) * 64u;
+    uint32_t slots = 4 * TG;
+    static int occ_cache[17] = {0};
+    int occ = occ_cache[S];
+    if (occ == 0) {
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, gemv_mfma_kernel<FMT, NSBW, SMAX>, (int)(S * 64),
+                                                         slots * per_slot) != hipSuccess || occ < 1)
+            occ = 1;
+        if (occ > 4) occ = 4;
+        occ_cache[S] = occ;
+    }
+    uint32_t grid = n_cus * (uint32_t)occ;
+    if (grid > p.n_tiles) grid = p.n_tiles;
+    p.slots = slots;  // the kernel recombines whenever fewer than TG slots are left
+    hipLaunchKernelGGL((gemv_mfma_kernel<FMT, NSBW, SMAX>), dim3(grid), dim3(S * 64), slots * per_slot, st, p);
     return hipGetLastError();
 }
 
 hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {
-    // K slice per wave: NSBW superblocks; S waves per workgroup.
+    // K slice per wave: NSBW superblocks; S <= 8 waves per workgroup.
     uint32_t nsbw = (p.sb_count + 7u) / 8u;
     if (nsbw < 1) nsbw = 1;
-    if (nsbw > 4) return hipErrorInvalidValue;  // caller splits K into chunks of <= 32 superblocks
+    if (nsbw > 3) return hipErrorInvalidValue;  // caller splits K into chunks of OXB_GEMV_MAX_SB superblocks
     const uint32_t S = (p.sb_count + nsbw - 1) / nsbw;
-    // Aim at 16 waves per CU.
-    uint32_t wg_per_cu = 16u / S;
-    if (wg_per_cu < 1) wg_per_cu = 1;
-    uint32_t grid = n_cus * wg_per_cu;
-    if (grid > p.n_tiles) grid = p.n_tiles;
-    if (grid == 0) return hipSuccess;
-    const uint32_t max_tiles = (p.n_tiles + grid - 1) / grid;
-    uint32_t slots = (64u * 1024u) / (S * p.NC * 64u);
-    if (slots > max_tiles) slots = max_tiles;
-    if (slots < 1) slots = 1;
-    p.slots = slots;
-    const size_t shm = (size_t)slots * S * p.NC * 64u;
-#define OXB_CASE(F, N, SM)                                                 \
-    if (fmt == F && nsbw == N) return launch_gemv_t<F, N, SM>(p, S, grid, shm, st);
-    OXB_CASE(OXB_FMT_Q1, 1, 8)
-    OXB_CASE(OXB_FMT_Q1, 2, 8)
-    OXB_CASE(OXB_FMT_Q1, 3, 8)
-    OXB_CASE(OXB_FMT_Q1, 4, 8)
-    OXB_CASE(OXB_FMT_TQ2, 1, 8)
-    OXB_CASE(OXB_FMT_TQ2, 2, 8)
-    OXB_CASE(OXB_FMT_TQ2, 3, 8)
-    OXB_CASE(OXB_FMT_TQ2, 4, 8)
+    if (p.n_tiles == 0) return hipSuccess;
+#define OXB_CASE(F, N)                                                   \
+    if (fmt == F && nsbw == N) return launch_gemv_t<F, N, 8>(p, S, n_cus, st);
+    OXB_CASE(OXB_FMT_Q1, 1)
+    OXB_CASE(OXB_FMT_Q1, 2)
+    OXB_CASE(OXB_FMT_Q1, 3)
+    OXB_CASE(OXB_FMT_TQ2, 1)
+    OXB_CASE(OXB_FMT_TQ2, 2)
+    OXB_CASE(OXB_FMT_TQ2, 3)
 #undef OXB_CASE
     return hipErrorInvalidValue;
 }

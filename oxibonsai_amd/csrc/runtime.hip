@@ -114,15 +114,15 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
     return OXB_HIP_OK;
 }
 
-// x (device, [batch][k]) -> y (device, [batch][ldy]) through quantiser + GEMV, <= 4 vectors per pass.
+// x (device, [batch][k]) -> y (device, [batch][ldy]) through quantiser + GEMV, OXB_GEMV_MAX_BATCH vectors per pass.
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual) {
     const uint32_t k = w.L.k;
-    for (uint32_t b0 = 0; b0 < batch; b0 += 4) {
-        const uint32_t nb = (batch - b0) < 4 ? (batch - b0) : 4;
+    for (uint32_t b0 = 0; b0 < batch; b0 += OXB_GEMV_MAX_BATCH) {
+        const uint32_t nb = (batch - b0) < OXB_GEMV_MAX_BATCH ? (batch - b0) : OXB_GEMV_MAX_BATCH;
         int rc;
-        if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, 4)))) return rc;
-        if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, 4)))) return rc;
+        if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
+        if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
         if ((rc = g_rt.ws_xexp.ensure(16 * sizeof(int32_t)))) return rc;
         hipError_t e = oxb_launch_quant_x((int)w.L.fmt, d_x + (size_t)b0 * k, k, nb, (uint32_t*)g_rt.ws_xq.ptr,
                                           (int32_t*)g_rt.ws_cneg.ptr, (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
@@ -139,11 +139,11 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
         p.n_rows = w.L.n_rows;
         p.n_tiles = w.L.n_tiles;
         p.n_sb = w.L.n_sb;
-        p.NC = 4 * nb;
+        p.NC = 8 * nb;
         p.ldy = ldy;
-        for (uint32_t sb = 0; sb < w.L.n_sb; sb += 32) {
+        for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
             p.sb_begin = sb;
-            p.sb_count = (w.L.n_sb - sb) < 32 ? (w.L.n_sb - sb) : 32;
+            p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
             p.mode = sb == 0 ? mode : OXB_GEMV_ACCUM;
             e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
             if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
@@ -323,6 +323,71 @@ int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows,
     if (rc) return rc;
     if (!d_x || !d_y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
     return gemv_device(*w, d_x, d_y, batch, n_rows, OXB_GEMV_STORE, nullptr);
+}
+
+int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,
+                         uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!ids || n_ids == 0 || !d_x || !d_y || !avg_us || iters == 0)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
+    std::vector<const Weight*> ws;
+    for (uint32_t i = 0; i < n_ids; i++) {
+        Weight* w = find_weight(ids[i]);
+        if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)ids[i]);
+        int rc = check_shape(*w, n_rows, k);
+        if (rc) return rc;
+        if (!ws.empty() && w->L.fmt != ws[0]->L.fmt)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weights differ in format");
+        ws.push_back(w);
+    }
+    if (ws[0]->L.n_sb > OXB_GEMV_MAX_SB) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k too large for a single launch");
+    int rc;
+    if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
+    if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
+    if ((rc = g_rt.ws_xexp.ensure(16 * sizeof(int32_t)))) return rc;
+    const int fmt = (int)ws[0]->L.fmt;
+    hipError_t e = oxb_launch_quant_x(fmt, d_x, k, 1, (uint32_t*)g_rt.ws_xq.ptr, (int32_t*)g_rt.ws_cneg.ptr,
+                                      (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "kernel launch failed: quant_x");
+    OxbGemvParams p;
+    memset(&p, 0, sizeof p);
+    p.xq = (const uint32_t*)g_rt.ws_xq.ptr;
+    p.cneg = (const int32_t*)g_rt.ws_cneg.ptr;
+    p.xexp = (const int32_t*)g_rt.ws_xexp.ptr;
+    p.y = d_y;
+    p.n_rows = n_rows;
+    p.n_tiles = ws[0]->L.n_tiles;
+    p.n_sb = ws[0]->L.n_sb;
+    p.sb_begin = 0;
+    p.sb_count = p.n_sb;
+    p.NC = 8;
+    p.ldy = n_rows;
+    p.mode = OXB_GEMV_STORE;
+    hipEvent_t ev0, ev1;
+    if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");
+    if ((e = hipEventCreate(&ev1)) != hipSuccess) { (void)hipEventDestroy(ev0); return hip_fail(e, "event creation"); }
+    rc = OXB_HIP_OK;
+    for (uint32_t i = 0; i < warmup + iters && rc == OXB_HIP_OK; i++) {
+        if (i == warmup) (void)hipEventRecord(ev0, g_rt.stream);
+        const Weight* w = ws[i % n_ids];
+        p.codes = w->d_codes;
+        p.scales = w->d_scales;
+        e = oxb_launch_gemv(fmt, p, g_rt.n_cus, g_rt.stream);
+        if (e != hipSuccess) rc = hip_fail(e, "kernel launch failed: gemv");
+    }
+    (void)hipEventRecord(ev1, g_rt.stream);
+    if (rc == OXB_HIP_OK) {
+        e = hipEventSynchronize(ev1);
+        if (e != hipSuccess) rc = fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: %s", hipGetErrorString(e));
+    }
+    if (rc == OXB_HIP_OK) {
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, ev0, ev1);
+        *avg_us = ms * 1000.0f / (float)iters;
+    }
+    (void)hipEventDestroy(ev0);
+    (void)hipEventDestroy(ev1);
+    return rc;
 }
 
 int oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch) {
