@@ -21,7 +21,8 @@ struct OxbGemvParams {
     uint32_t sb_begin, sb_count;  // K range handled by this launch, in superblocks
     uint32_t NC;                  // 8 * batch, batch <= 2 (eight digit columns per vector)
     uint32_t ldy;
-    uint32_t slots;               // filled by the launcher
+    uint32_t groups;              // filled by the launcher: groups of in-flight tiles per workgroup
+    uint32_t codes_bytes, scales_bytes, xq_bytes, cneg_bytes;  // buffer extents (loads beyond them read 0)
     int mode;
 };
 

@@ -179,8 +179,8 @@ __global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float*
 // the matching slice of the digit planes in registers for the whole kernel, so
 // the inner loop is: one coalesced 1 KiB code load per superblock, 4 ANDs + 1
 // MFMA per 64 weights of 16 rows, 4 cvt + 4 fma per block for the scale.
-// The eight digit columns are weighed and added across lanes (DPP), the partial
-// row sums of the S waves meet in LDS and the last step applies the epilogue (store / +=).
+// Partial row sums of the S waves meet in LDS; the last step weighs and adds the eight digit
+// columns (DPP) and applies the epilogue (store / +=).
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
@@ -197,6 +197,25 @@ __device__ __forceinline__ float dpp_f32(float v) {
 #define OXB_DPP_ROW_SHR(n) (0x110 + (n))
 #define OXB_DPP_ROW_NEWBCAST(n) (0x150 + (n))  // lane n of each 16-lane row to the whole row
 
+// Buffer resources: a load whose byte offset lies outside the buffer returns 0 and moves no
+// data, which replaces every "is this tile / superblock / column in range" branch below.
+typedef unsigned v4u __attribute__((ext_vector_type(4)));
+#define OXB_OOB 0xFFFFFFF0u
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
+}
+// voff is per lane and is what the range check sees; soff is wave-uniform (an SGPR) and is not checked.
+__device__ __forceinline__ v4i buf_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+    return (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
+}
+__device__ __forceinline__ uint32_t buf_load_b32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
+    return __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
+}
+// Workgroup barrier that orders LDS traffic only: global loads already in flight (the
+// prefetched weight tiles) stay in flight across it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Codes and scales of one row tile, restricted to this wave's K slice, as they wait in registers.
 template <int FMT, int NSBW>
 struct TileRegs {
@@ -205,19 +224,20 @@ struct TileRegs {
     uint32_t sc[NSBW];  // lane (c, rg): f16 pair (c & 7) of row group rg, pair 2q+p = scales of block q, rows 2p, 2p+1
 };
 
+// `valid`, `tile` and the unit index are wave-uniform: they travel in scalar registers, the lane
+// part of the address (lane_c, lane_s) is fixed for the whole kernel.
 template <int FMT, int NSBW>
-__device__ __forceinline__ void load_tile(TileRegs<FMT, NSBW>& t, const v4i* __restrict__ codes,
-                                          const uint32_t* __restrict__ scales, uint32_t tile, uint32_t n_sb, int sb0,
-                                          int nsb_w, uint32_t lane) {
+__device__ __forceinline__ void load_tile(TileRegs<FMT, NSBW>& t, __amdgpu_buffer_rsrc_t codes,
+                                          __amdgpu_buffer_rsrc_t scales, uint32_t tile, bool valid, uint32_t n_sb,
+                                          uint32_t sb0, int sb_lim, uint32_t lane_c, uint32_t lane_s) {
     constexpr int UNITS = TileRegs<FMT, NSBW>::UNITS;
 #pragma unroll
     for (int i = 0; i < NSBW; i++) {
-        if (i < nsb_w) {
-            const size_t unit = (size_t)tile * n_sb + (uint32_t)(sb0 + i);
+        const bool ok = valid && i < sb_lim;
+        const uint32_t unit = __builtin_amdgcn_readfirstlane(tile * n_sb + sb0 + (uint32_t)i);
 #pragma unroll
-            for (int u = 0; u < UNITS; u++) t.w[i][u] = codes[(unit * UNITS + u) * 64 + lane];
-            t.sc[i] = scales[unit * 32 + (lane >> 4) * 8 + (lane & 7u)];
-        }
+        for (int u = 0; u < UNITS; u++) t.w[i][u] = buf_load_b128(codes, ok ? lane_c : OXB_OOB, (unit * UNITS + u) * 1024u);
+        t.sc[i] = buf_load_b32(scales, ok ? lane_s : OXB_OOB, unit * 128u);
     }
 }
 
@@ -243,117 +263,103 @@ __device__ __forceinline__ void block_mac(v4f& accf, uint32_t d0, uint32_t d1, c
     accf[3] = fmaf((float)acc[3], f16_bits_to_f32(p1 >> 16), accf[3]);
 }
 
-template <int FMT, int NSBW, int SMAX>
-__global__ __launch_bounds__(SMAX * 64, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(const OxbGemvParams p) {
-    extern __shared__ float part[];  // [slot][S][batch][16]
+// Workgroup wg handles row tiles [wg * groups * TG, +groups * TG); TG tiles are in flight per
+// wave at any time and are recombined together.  All control flow is uniform and branch-free
+// inside a group, so the compiler can wait for exactly the tile it is about to use.
+template <int FMT, int NSBW, int TG>
+__global__ __launch_bounds__(512, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(const OxbGemvParams p) {
+    extern __shared__ float part[];  // [2][TG][S][NC][16]
     constexpr int UNITS = TileRegs<FMT, NSBW>::UNITS;
-    constexpr int TG = (8 / (NSBW * UNITS)) > 0 ? (8 / (NSBW * UNITS)) : 1;  // row tiles in flight per wave
     const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
     const uint32_t c = lane & 15u, g = lane >> 4;  // B operand: column c, k-group g; D: column c, rows 4g..4g+3
-    const uint32_t NC = p.NC, batch = NC >> 3;
+    const uint32_t NC = p.NC;
     const bool col_on = c < NC;
 
-    const int sb0 = (int)(p.sb_begin + s * NSBW);
-    int nsb_w = (int)(p.sb_begin + p.sb_count) - sb0;
-    nsb_w = nsb_w < 0 ? 0 : (nsb_w > NSBW ? NSBW : nsb_w);
+    const uint32_t lane_c = lane * 16u, lane_s = ((lane >> 4) * 8u + (lane & 7u)) * 4u;
+    const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
+    const int sb_lim = (int)(p.sb_begin + p.sb_count) - (int)sb0;  // superblocks of this wave's slice that exist
 
-    // Contiguous range of row tiles for this workgroup.
-    const uint32_t G = gridDim.x, wg = blockIdx.x;
-    const uint32_t base_cnt = p.n_tiles / G, rem = p.n_tiles % G;
-    const uint32_t t_begin = wg * base_cnt + (wg < rem ? wg : rem);
-    const uint32_t t_count = base_cnt + (wg < rem ? 1u : 0u);
+    const __amdgpu_buffer_rsrc_t r_codes = make_rsrc(p.codes, p.codes_bytes);
+    const __amdgpu_buffer_rsrc_t r_scales = make_rsrc(p.scales, p.scales_bytes);
+    const __amdgpu_buffer_rsrc_t r_xq = make_rsrc(p.xq, p.xq_bytes);
+    const __amdgpu_buffer_rsrc_t r_cneg = make_rsrc(p.cneg, p.cneg_bytes);
 
-    const v4i* codes = reinterpret_cast<const v4i*>(p.codes);
-    const uint32_t* scales = reinterpret_cast<const uint32_t*>(p.scales);
-
-    // Start the weight stream first: the HBM latency of the first TG tiles overlaps the
-    // (L2-resident) digit-plane loads below.
-    TileRegs<FMT, NSBW> ring[TG];
-#pragma unroll
-    for (int t = 0; t < TG; t++)
-        if ((uint32_t)t < t_count) load_tile<FMT, NSBW>(ring[t], codes, scales, t_begin + t, p.n_sb, sb0, nsb_w, lane);
-
-    // Digit planes and accumulator start values of this wave's K slice.
+    // Digit planes and accumulator start values of this wave's K slice (L2-resident), issued
+    // first so that the weight stream behind them can be consumed tile by tile as it arrives.
     v4i B[NSBW][4][2];
     v4i C4[NSBW][4];
 #pragma unroll
     for (int i = 0; i < NSBW; i++)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            B[i][q][0] = B[i][q][1] = C4[i][q] = (v4i){0, 0, 0, 0};
-            if (i < nsb_w && col_on) {
-                const uint32_t blk = (uint32_t)(sb0 + i) * 4 + q;
-                const v4i* xq4 = reinterpret_cast<const v4i*>(p.xq);
-                B[i][q][0] = xq4[(size_t)((blk * 2 + 0) * 4 + g) * NC + c];
-                B[i][q][1] = xq4[(size_t)((blk * 2 + 1) * 4 + g) * NC + c];
-                C4[i][q] = reinterpret_cast<const v4i*>(p.cneg)[(size_t)blk * NC + c];
-            }
+            const bool ok = col_on && i < sb_lim;
+            const uint32_t blk = (sb0 + (uint32_t)i) * 4 + q;
+            B[i][q][0] = buf_load_b128(r_xq, ok ? (((blk * 2 + 0) * 4 + g) * NC + c) * 16u : OXB_OOB);
+            B[i][q][1] = buf_load_b128(r_xq, ok ? (((blk * 2 + 1) * 4 + g) * NC + c) * 16u : OXB_OOB);
+            C4[i][q] = buf_load_b128(r_cneg, ok ? (blk * NC + c) * 16u : OXB_OOB);
         }
-    // Column c carries digit (c & 7) of vector (c >> 3): its partial sums weigh 2^(8 digit + E - P).
-    const int xe = col_on ? p.xexp[c >> 3] : 0;
-    const int my_exp = (xe == INT32_MIN ? 0 : xe) + 8 * (int)(c & 7u);
+    // In the recombination, thread t handles column (t % NC): digit (t % 8) of vector (t % NC) / 8.
+    const int xe = p.xexp[(threadIdx.x % NC) >> 3];
 
-    uint32_t sl = 0, chunk0 = 0;  // slots filled in the LDS chunk, first tile of the chunk
-    for (uint32_t lt0 = 0; lt0 < t_count; lt0 += TG) {
+    const uint32_t tpw = p.groups * TG, t_begin = blockIdx.x * tpw;
+    const uint32_t t_end = (t_begin + tpw) < p.n_tiles ? (t_begin + tpw) : p.n_tiles;
+
+    // The scheduling barriers pin the issue order of the loads: memory returns in issue order, so
+    // "tile t has arrived" is a wait for all but the loads issued after it.
+    __builtin_amdgcn_sched_barrier(0);
+    TileRegs<FMT, NSBW> ring[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++) {
+        load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, t_begin + t, t_begin + t < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+
+    for (uint32_t grp = 0; grp < p.groups; grp++) {
+        float* buf = part + (size_t)(grp & 1u) * TG * S * NC * 16;
 #pragma unroll
         for (int t = 0; t < TG; t++) {
-            const uint32_t lt = lt0 + t;
-            if (lt < t_count) {  // uniform over the workgroup
-                v4f accf = {0.f, 0.f, 0.f, 0.f};
+            const uint32_t tile = t_begin + grp * TG + t;
+            v4f accf = {0.f, 0.f, 0.f, 0.f};
+            const TileRegs<FMT, NSBW>& r = ring[t];
 #pragma unroll
-                for (int i = 0; i < NSBW; i++) {
-                    if (i < nsb_w) {
-                        const TileRegs<FMT, NSBW>& r = ring[t];
-                        if (FMT == OXB_FMT_Q1) {
-                            block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][0], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
-                            block_mac<FMT, 1>(accf, r.w[i][0][1], r.w[i][0][1], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
-                            block_mac<FMT, 2>(accf, r.w[i][0][2], r.w[i][0][2], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
-                            block_mac<FMT, 3>(accf, r.w[i][0][3], r.w[i][0][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
-                        } else {
-                            block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][1], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
-                            block_mac<FMT, 1>(accf, r.w[i][0][2], r.w[i][0][3], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
-                            block_mac<FMT, 2>(accf, r.w[i][UNITS - 1][0], r.w[i][UNITS - 1][1], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
-                            block_mac<FMT, 3>(accf, r.w[i][UNITS - 1][2], r.w[i][UNITS - 1][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
-                        }
-                    }
+            for (int i = 0; i < NSBW; i++) {
+                if (FMT == OXB_FMT_Q1) {
+                    block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][0], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
+                    block_mac<FMT, 1>(accf, r.w[i][0][1], r.w[i][0][1], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
+                    block_mac<FMT, 2>(accf, r.w[i][0][2], r.w[i][0][2], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
+                    block_mac<FMT, 3>(accf, r.w[i][0][3], r.w[i][0][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
+                } else {
+                    block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][1], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
+                    block_mac<FMT, 1>(accf, r.w[i][0][2], r.w[i][0][3], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
+                    block_mac<FMT, 2>(accf, r.w[i][UNITS - 1][0], r.w[i][UNITS - 1][1], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
+                    block_mac<FMT, 3>(accf, r.w[i][UNITS - 1][2], r.w[i][UNITS - 1][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
                 }
-                // refill this ring slot with the tile TG ahead
-                if (lt + TG < t_count)
-                    load_tile<FMT, NSBW>(ring[t], codes, scales, t_begin + lt + TG, p.n_sb, sb0, nsb_w, lane);
-                // weigh the digit, then add the eight digit columns of each vector (lanes c-7..c of the row)
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    float a = ldexpf(accf[v], my_exp);
-                    a += dpp_f32<OXB_DPP_ROW_SHR(1)>(a);
-                    a += dpp_f32<OXB_DPP_ROW_SHR(2)>(a);
-                    a += dpp_f32<OXB_DPP_ROW_SHR(4)>(a);
-                    accf[v] = a;
-                }
-                if (col_on && (c & 7u) == 7u)
-                    *reinterpret_cast<v4f*>(&part[(((size_t)(sl + t) * S + s) * batch + (c >> 3)) * 16 + g * 4]) = accf;
             }
+            // refill this ring slot with the tile TG ahead (reads nothing past the workgroup's range)
+            load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile + TG, tile + TG < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+            __builtin_amdgcn_sched_barrier(0);
+            if (col_on) *reinterpret_cast<v4f*>(&buf[(((size_t)t * S + s) * NC + c) * 16 + g * 4]) = accf;
         }
-        const uint32_t done = (t_count - lt0) < (uint32_t)TG ? (t_count - lt0) : (uint32_t)TG;
-        sl += done;
-        if (sl + TG > p.slots || lt0 + TG >= t_count) {
-            __syncthreads();
-            // thread -> (slot, vector n, row): sum the S partial results in a fixed order.
-            for (uint32_t idx = threadIdx.x; idx < sl * batch * 16; idx += blockDim.x) {
-                const uint32_t r = idx & 15u, n = (idx >> 4) % batch, slot = idx / (16 * batch);
-                const uint32_t row = (t_begin + chunk0 + slot) * 16 + r;
-                if (row >= p.n_rows) continue;
-                float v = 0.f;
-                for (uint32_t w = 0; w < S; w++) v += part[(((size_t)slot * S + w) * batch + n) * 16 + r];
-                if (p.xexp[n] == INT32_MIN) v = __int_as_float(0x7FC00000);
-                const size_t o = (size_t)n * p.ldy + row;
+        lds_barrier();
+        // thread -> (slot, row, column): add the S partial sums in a fixed order, weigh the digit
+        // by 2^(8 digit + E - P), then add the eight digit columns of a vector across lanes.
+        for (uint32_t idx = threadIdx.x; idx < (uint32_t)TG * 16 * NC; idx += blockDim.x) {
+            const uint32_t cc = idx % NC, rr = (idx / NC) & 15u, slot = idx / (16 * NC);
+            float v = 0.f;
+            for (uint32_t w = 0; w < S; w++) v += buf[(((size_t)slot * S + w) * NC + cc) * 16 + rr];
+            v = (xe == INT32_MIN) ? __int_as_float(0x7FC00000) : ldexpf(v, xe + 8 * (int)(cc & 7u));
+            v += dpp_f32<OXB_DPP_ROW_SHR(1)>(v);
+            v += dpp_f32<OXB_DPP_ROW_SHR(2)>(v);
+            v += dpp_f32<OXB_DPP_ROW_SHR(4)>(v);
+            const uint32_t tile = t_begin + grp * TG + slot, row = tile * 16 + rr;
+            if ((cc & 7u) == 7u && tile < t_end && row < p.n_rows) {
+                const size_t o = (size_t)(cc >> 3) * p.ldy + row;
                 if (p.mode == OXB_GEMV_ACCUM) v += p.y[o];
                 else if (p.mode == OXB_GEMV_RESIDUAL) v += p.residual[o];
                 p.y[o] = v;
             }
-            __syncthreads();
-            chunk0 += sl;
-            sl = 0;
         }
+        // no second barrier: the next group writes the other half of `part`
     }
 }
 
@@ -408,27 +414,10 @@ hipError_t oxb_launch_quant_x(int fmt, const float* d_x, uint32_t k, uint32_t ba
     return hipGetLastError();
 }
 
-template <int FMT, int NSBW, int SMAX>
-static hipError_t launch_gemv_t(OxbGemvParams p, uint32_t S, uint32_t n_cus, hipStream_t st) {
-    // Grid = what is resident at once, so every workgroup starts immediately and streams its
-    // share of row tiles; partial sums of at most `slots` tiles wait in LDS for the recombination.
-    constexpr uint32_t UNITS = (FMT == OXB_FMT_Q1) ? 1 : 2;
-    constexpr uint32_t TG = (8 / (NSBW * UNITS)) > 0 ? (8 / (NSBW * UNITS)) : 1;  // as in the kernel
-    const size_t per_slot = (size_t)S * (p.NC / 8) * 64u;
-    uint32_t slots = 4 * TG;
-    static int occ_cache[17] = {0};
-    int occ = occ_cache[S];
-    if (occ == 0) {
-        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&occ, gemv_mfma_kernel<FMT, NSBW, SMAX>, (int)(S * 64),
-                                                         slots * per_slot) != hipSuccess || occ < 1)
-            occ = 1;
-        if (occ > 4) occ = 4;
-        occ_cache[S] = occ;
-    }
-    uint32_t grid = n_cus * (uint32_t)occ;
-    if (grid > p.n_tiles) grid = p.n_tiles;
-    p.slots = slots;  // the kernel recombines whenever fewer than TG slots are left
-    hipLaunchKernelGGL((gemv_mfma_kernel<FMT, NSBW, SMAX>), dim3(grid), dim3(S * 64), slots * per_slot, st, p);
+template <int FMT, int NSBW, int TG>
+static hipError_t launch_gemv_t(OxbGemvParams p, uint32_t S, uint32_t grid, hipStream_t st) {
+    const size_t shm = 2 * (size_t)TG * S * p.NC * 64u;
+    hipLaunchKernelGGL((gemv_mfma_kernel<FMT, NSBW, TG>), dim3(grid), dim3(S * 64), shm, st, p);
     return hipGetLastError();
 }
 
@@ -439,14 +428,36 @@ hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t
     if (nsbw > 3) return hipErrorInvalidValue;  // caller splits K into chunks of OXB_GEMV_MAX_SB superblocks
     const uint32_t S = (p.sb_count + nsbw - 1) / nsbw;
     if (p.n_tiles == 0) return hipSuccess;
-#define OXB_CASE(F, N)                                                   \
-    if (fmt == F && nsbw == N) return launch_gemv_t<F, N, 8>(p, S, n_cus, st);
-    OXB_CASE(OXB_FMT_Q1, 1)
-    OXB_CASE(OXB_FMT_Q1, 2)
-    OXB_CASE(OXB_FMT_Q1, 3)
-    OXB_CASE(OXB_FMT_TQ2, 1)
-    OXB_CASE(OXB_FMT_TQ2, 2)
-    OXB_CASE(OXB_FMT_TQ2, 3)
+    if (p.codes_bytes >= 0x7FFFFFFFull || p.xq_bytes >= 0x7FFFFFFFull) return hipErrorInvalidValue;
+    // Choose workgroups per CU (j), tiles in flight per wave (TG) and groups of TG tiles per
+    // workgroup so that the busiest CU computes the fewest tile slots; prefer more waves, then
+    // a deeper ring.  The partial-sum buffers 2 x TG x S x NC x 64 B stay <= 64 KiB.
+    const uint32_t units = fmt == OXB_FMT_Q1 ? 1u : 2u;
+    const uint32_t occ = nsbw == 1 ? 2u : 1u;  // what the register budget of the variant allows
+    uint32_t tg_max = nsbw == 1 ? 4u : (nsbw == 2 ? 4u / units : 1u);
+    while (tg_max > 1 && 2u * tg_max * S * p.NC * 64u > 64u * 1024u) tg_max--;
+    uint32_t best_cost = 0xFFFFFFFFu, tg = 1, grid = 1;
+    for (uint32_t j = occ; j >= 1; j--)
+        for (uint32_t t = tg_max; t >= 1; t--) {
+            const uint32_t tpw0 = (p.n_tiles + n_cus * j - 1) / (n_cus * j);
+            const uint32_t groups = (tpw0 + t - 1) / t, tpw = groups * t;
+            const uint32_t g = (p.n_tiles + tpw - 1) / tpw;
+            const uint32_t cost = ((g + n_cus - 1) / n_cus) * tpw;
+            if (cost < best_cost || (cost == best_cost && g > grid)) {  // ties: more workgroups in flight
+                best_cost = cost;
+                tg = t;
+                grid = g;
+                p.groups = groups;
+            }
+        }
+#define OXB_CASE(F, N, T)                                                \
+    if (fmt == F && nsbw == N && tg == T) return launch_gemv_t<F, N, T>(p, S, grid, st);
+    OXB_CASE(OXB_FMT_Q1, 1, 1) OXB_CASE(OXB_FMT_Q1, 1, 2) OXB_CASE(OXB_FMT_Q1, 1, 3) OXB_CASE(OXB_FMT_Q1, 1, 4)
+    OXB_CASE(OXB_FMT_Q1, 2, 1) OXB_CASE(OXB_FMT_Q1, 2, 2) OXB_CASE(OXB_FMT_Q1, 2, 3) OXB_CASE(OXB_FMT_Q1, 2, 4)
+    OXB_CASE(OXB_FMT_Q1, 3, 1)
+    OXB_CASE(OXB_FMT_TQ2, 1, 1) OXB_CASE(OXB_FMT_TQ2, 1, 2) OXB_CASE(OXB_FMT_TQ2, 1, 3) OXB_CASE(OXB_FMT_TQ2, 1, 4)
+    OXB_CASE(OXB_FMT_TQ2, 2, 1) OXB_CASE(OXB_FMT_TQ2, 2, 2)
+    OXB_CASE(OXB_FMT_TQ2, 3, 1)
 #undef OXB_CASE
     return hipErrorInvalidValue;
 }

@@ -141,6 +141,10 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
         p.n_sb = w.L.n_sb;
         p.NC = 8 * nb;
         p.ldy = ldy;
+        p.codes_bytes = (uint32_t)w.L.codes_bytes;
+        p.scales_bytes = (uint32_t)w.L.scales_bytes;
+        p.xq_bytes = (uint32_t)oxb_xq_bytes(k, nb);
+        p.cneg_bytes = (uint32_t)oxb_cneg_bytes(k, nb);
         for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
             p.sb_begin = sb;
             p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
@@ -362,6 +366,8 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
     p.sb_count = p.n_sb;
     p.NC = 8;
     p.ldy = n_rows;
+    p.xq_bytes = (uint32_t)oxb_xq_bytes(k, 1);
+    p.cneg_bytes = (uint32_t)oxb_cneg_bytes(k, 1);
     p.mode = OXB_GEMV_STORE;
     hipEvent_t ev0, ev1;
     if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");
@@ -372,6 +378,8 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
         const Weight* w = ws[i % n_ids];
         p.codes = w->d_codes;
         p.scales = w->d_scales;
+        p.codes_bytes = (uint32_t)w->L.codes_bytes;
+        p.scales_bytes = (uint32_t)w->L.scales_bytes;
         e = oxb_launch_gemv(fmt, p, g_rt.n_cus, g_rt.stream);
         if (e != hipSuccess) rc = hip_fail(e, "kernel launch failed: gemv");
     }
