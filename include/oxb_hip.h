@@ -86,6 +86,39 @@ int  oxb_hip_gemv_q1_g128(const uint8_t* aos, size_t n_bytes, const float* x, si
 int  oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len,
                            float* y, size_t y_len, uint32_t n_rows, uint32_t k);
 
+/* ---- batch_ffn_phase (KG/mod.rs:519; CUDA: KG/cuda_graph/nativecudabackend_traits.rs:122-188 -> encode_ffn_phase,
+ * KG/cuda_graph/cudagraph_encoding.rs:72-160): hidden += O * attn_out; normed = RMSNorm(hidden); hidden += down * SwiGLU(gate||up * normed),
+ * in place on the host vector `hidden[h]`.  fmt selects Q1 / TQ2 weights; gate_up holds the gate rows, then the up rows. */
+int  oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float* norm_w, float eps,
+                       uint64_t o_id, uint64_t gate_up_id, uint64_t down_id, uint32_t h, uint32_t inter, uint32_t attn_k);
+
+/* ---- fused whole-model decode: try_cuda_full_forward[_ternary]_with_gpu_lm_head
+ * (KG/cuda_full_layer/encode_q1.rs:881-900, encode_ternary.rs:755-774) with per-layer parameters as in
+ * CudaFullForwardLayerParams (KG/cuda_full_layer/mod.rs:250-268): norm vectors and weight matrices are named by
+ * handle.  Norm vectors are uploaded with oxb_hip_upload_f32; `qkv` is the Q|K|V row concatenation
+ * ((nq + 2 nkv) * hd rows), `gate_up` the gate|up concatenation (2 * inter rows), as the reference builds them
+ * (crates/oxibonsai-model/src/block/types/upload.rs:21-39). */
+int  oxb_hip_upload_f32(uint64_t* id, const float* w, size_t n);
+int  oxb_hip_free_f32(uint64_t id);
+typedef struct { uint64_t attn_norm, qkv, q_norm, k_norm, o, ffn_norm, gate_up, down; } oxb_layer_ids;
+typedef struct {
+    int fmt;                       /* OXB_HIP_FMT_Q1 / OXB_HIP_FMT_TQ2 for every matrix */
+    uint32_t n_layers, h, inter, nq, nkv, hd, vocab, max_seq, batch;
+    float eps, rope_theta;
+    const oxb_layer_ids* layers;   /* [n_layers], read during the call only */
+    uint64_t final_norm, lm_head;
+} oxb_model_desc;
+/* Allocates the FP16 KV cache [batch][layer][kv_head][max_seq][hd] (CudaKvCache, KG/cuda_full_layer/mod.rs:112-139),
+ * the activation buffers (mod.rs:149-181) and the RoPE table (crates/oxibonsai-model/src/layers/rope.rs:27-48). */
+int  oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model);
+int  oxb_hip_model_reset(uint64_t model);
+int  oxb_hip_model_destroy(uint64_t model);
+/* One token for each of the `batch` sequences: hidden[batch][h] are the embedding rows, pos[batch] the positions.
+ * Runs all layers, the final norm, the LM head and a first-maximum argmax on the device (a HIP graph after the first
+ * call).  logits_or_null: [batch][vocab]; token_out: [batch] greedy ids (either may be NULL). */
+int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out);
+int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is replayed from a captured graph */
+
 /* ---- host-only helpers (no GPU needed): the upload-time repack, exposed so it can be checked on any machine.
  * reformat_q1_aos_to_soa / reformat_tq2_blocks_to_soa (KG/cuda_graph/cudagraph_reformat_*_group.rs). */
 int  oxb_hip_repack_sizes(int fmt, uint32_t n_rows, uint32_t k, size_t* codes_bytes, size_t* scales_bytes);

@@ -277,11 +277,12 @@ class OracleModel:
                              lin(weights["lm_head"], cfg["vocab"], h), 1 if kv_f16 else 0)
         self._state = lib().oxb_state_new(C.byref(self._model))
 
-    def forward(self, hidden, pos: int, want_normed: bool = False):
+    def forward(self, hidden, pos: int, want_normed: bool = False, want_logits: bool = True):
         hv = _vec(hidden)
-        logits = np.empty(self.cfg["vocab"], dtype=np.float32)
+        logits = np.empty(self.cfg["vocab"], dtype=np.float32) if want_logits else None
         normed = np.empty(self.cfg["h"], dtype=np.float32)
-        _check(lib().oxb_forward_ex(C.byref(self._model), self._state, _f32(hv), pos, _f32(logits), _f32(normed)))
+        _check(lib().oxb_forward_ex(C.byref(self._model), self._state, _f32(hv), pos,
+                                    _f32(logits) if want_logits else None, _f32(normed)))
         return (logits, normed) if want_normed else logits
 
     def reset(self):

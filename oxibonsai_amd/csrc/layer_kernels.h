@@ -1,0 +1,36 @@
+// layer_kernels.h — launch interface of the layer glue kernels (see layer_kernels.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+struct OxbQkParams {
+    const float* qkv;      // [batch][qkv_stride]: q heads | k heads | v heads
+    uint32_t qkv_stride;
+    const float *q_norm, *k_norm;  // [hd]
+    const float *cos_t, *sin_t;    // [max_seq][hd/2]
+    const uint32_t* pos;           // [batch], device
+    float* q_rope;                 // [batch][nq][hd]
+    __half *k_cache, *v_cache;     // [batch][n_layers][nkv][max_seq][hd]
+    uint32_t nq, nkv, hd, max_seq, n_layers, layer;
+    float eps;
+};
+
+struct OxbAttnParams {
+    const float* q;                      // [batch][nq][hd]
+    const __half *k_cache, *v_cache;
+    float* part;                         // [batch][nq][n_splits][hd + 2]
+    const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
+    uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
+    float scale;                         // 1 / sqrt(hd)
+};
+
+hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t nb,
+                                    uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed_or_null,
+                                    hipStream_t st);
+hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
+                                   int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
+hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);
+size_t oxb_attn_smem_bytes(uint32_t nq, uint32_t nkv, uint32_t hd, uint32_t chunk);
+hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
+hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, hipStream_t st);

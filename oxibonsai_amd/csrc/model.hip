@@ -1,6 +1,476 @@
-// model.hip — fused whole-model decode / prefill entry points (placeholder until the pipeline lands).
+// model.hip — fused whole-model decode behind the C ABI.
+//
+// Stands in for the reference's fused GPU forward
+//   try_cuda_full_forward[_ternary]_with_gpu_lm_head   gpu_backend/cuda_full_layer/encode_q1.rs:881, encode_ternary.rs:755
+//   encode_layer_device / encode_layer_into_ternary     encode_q1.rs:297-463, encode_ternary.rs:116-291
+//   CudaKvCache (FP16, [layer][kv_head][max_seq][hd])   gpu_backend/cuda_full_layer/mod.rs:112-139
+//   graph capture / replay of the whole token            encode_q1.rs:569-797
+// and for GpuBackendTrait::batch_ffn_phase (gpu_backend/mod.rs:519).
+// One decode step is a fixed kernel sequence that reads the token position from device memory,
+// so it is captured once into a hipGraph and replayed for every following token.  Logits stay on
+// the device; the greedy token id comes from an on-device argmax (the reference's Metal tier does
+// the same, metal_full_layer/functions_3.rs:676-720).
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <cmath>
+#include <cstdlib>
+#include <cstring>
+#include <memory>
+#include <vector>
+
+#include "../../include/oxb_hip.h"
+#include "gemv_kernels.h"
+#include "layer_kernels.h"
 #include "runtime_internal.h"
 
 namespace oxb {
-void shutdown_models() {}
+
+struct XqBuf {  // quantised activation of one GEMV pass (<= OXB_GEMV_MAX_BATCH vectors)
+    uint32_t* xq = nullptr;
+    int32_t* cneg = nullptr;
+    int32_t* xexp = nullptr;
+};
+
+struct Model {
+    oxb_model_desc d;
+    std::vector<oxb_layer_ids> layers;
+    // activations
+    float *hidden = nullptr, *qkv = nullptr, *q_rope = nullptr, *attn_part = nullptr, *attn_out = nullptr,
+          *gu = nullptr, *logits = nullptr;
+    uint32_t *tokens = nullptr, *pos = nullptr;
+    __half *k_cache = nullptr, *v_cache = nullptr;
+    float *cos_t = nullptr, *sin_t = nullptr;
+    void* xq_mem = nullptr;
+    XqBuf xq;
+    uint32_t chunk = 0, n_splits = 0;
+    // graph
+    hipGraphExec_t graph_exec = nullptr;
+    bool graph_failed = false;
+    bool want_logits_in_graph = true;
+    std::vector<void*> allocs;
+};
+
+static std::unordered_map<uint64_t, std::unique_ptr<Model>> g_models;
+static uint64_t g_next_model = 1;
+
+static int dev_alloc(Model& m, void** p, size_t bytes) {
+    hipError_t e = hipMalloc(p, bytes ? bytes : 16);
+    if (e != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", bytes, g_rt.device);
+    m.allocs.push_back(*p);
+    return OXB_HIP_OK;
+}
+
+static void free_model(Model& m) {
+    if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
+    m.graph_exec = nullptr;
+    for (void* p : m.allocs) (void)hipFree(p);
+    m.allocs.clear();
+}
+
+void shutdown_models() {
+    for (auto& kv : g_models) free_model(*kv.second);
+    g_models.clear();
+}
+
+static const float* vec_ptr(uint64_t id, uint32_t n, const char* what, int* rc) {
+    auto it = g_rt.vectors.find(id);
+    if (it == g_rt.vectors.end()) {
+        *rc = fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (%s) not found", (unsigned long long)id, what);
+        return nullptr;
+    }
+    if (it->second.n != n) {
+        *rc = fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %s holds %zu values, %u expected", what, it->second.n, n);
+        return nullptr;
+    }
+    return it->second.d;
+}
+
+static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, const char* what, int* rc) {
+    const Weight* w = find_weight(id);
+    if (!w) {
+        *rc = fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (%s) not found", (unsigned long long)id, what);
+        return nullptr;
+    }
+    if ((int)w->L.fmt != fmt || w->L.n_rows != n_rows || w->L.k != k) {
+        *rc = fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %s is fmt %u %ux%u, model needs fmt %d %ux%u", what,
+                   w->L.fmt, w->L.n_rows, w->L.k, fmt, n_rows, k);
+        return nullptr;
+    }
+    return w;
+}
+
+// GEMV on an already quantised input.
+static int gemv_xq(const Weight& w, const XqBuf& xb, uint32_t nb, float* d_y, uint32_t ldy, int mode,
+                   const float* d_res) {
+    OxbGemvParams p;
+    memset(&p, 0, sizeof p);
+    p.codes = w.d_codes;
+    p.scales = w.d_scales;
+    p.xq = xb.xq;
+    p.cneg = xb.cneg;
+    p.xexp = xb.xexp;
+    p.y = d_y;
+    p.residual = d_res;
+    p.n_rows = w.L.n_rows;
+    p.n_tiles = w.L.n_tiles;
+    p.n_sb = w.L.n_sb;
+    p.NC = 8 * nb;
+    p.ldy = ldy;
+    p.codes_bytes = (uint32_t)w.L.codes_bytes;
+    p.scales_bytes = (uint32_t)w.L.scales_bytes;
+    p.xq_bytes = (uint32_t)oxb_xq_bytes(w.L.k, nb);
+    p.cneg_bytes = (uint32_t)oxb_cneg_bytes(w.L.k, nb);
+    for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
+        p.sb_begin = sb;
+        p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
+        p.mode = sb == 0 ? mode : OXB_GEMV_ACCUM;
+        hipError_t e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
+        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
+    }
+    return OXB_HIP_OK;
+}
+
+#define OXB_TRY_HIP(expr, what)                               \
+    do {                                                      \
+        hipError_t e_ = (expr);                               \
+        if (e_ != hipSuccess) return hip_fail(e_, what);      \
+    } while (0)
+#define OXB_TRY(expr)            \
+    do {                         \
+        int rc_ = (expr);        \
+        if (rc_) return rc_;     \
+    } while (0)
+
+// The FFN half of a layer on vectors [b0, b0+nb): O-proj + residual, RMSNorm, gate||up, SwiGLU, down + residual.
+static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn_out, const float* ffn_norm, float eps,
+                      const Weight& o, const Weight& gate_up, const Weight& down, float* gu, uint32_t h,
+                      uint32_t inter, uint32_t attn_k, uint32_t nb) {
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(oxb_launch_quant_x(fmt, attn_out, attn_k, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: quant_x");
+    OXB_TRY(gemv_xq(o, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
+    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(fmt, hidden, ffn_norm, eps, h, nb, xb.xq, xb.cneg, xb.xexp, nullptr, st),
+                "kernel launch failed: rmsnorm_quant");
+    OXB_TRY(gemv_xq(gate_up, xb, nb, gu, 2 * inter, OXB_GEMV_STORE, nullptr));
+    OXB_TRY_HIP(oxb_launch_swiglu_quant(fmt, gu, inter, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: swiglu_quant");
+    OXB_TRY(gemv_xq(down, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
+    return OXB_HIP_OK;
+}
+
+// Every kernel of one decode step, for all sequences of the batch (no host synchronisation).
+static int encode_decode_step(Model& m, bool with_lm_head) {
+    const oxb_model_desc& d = m.d;
+    hipStream_t st = g_rt.stream;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < d.n_layers; L++) {
+        const oxb_layer_ids& ly = m.layers[L];
+        const float* attn_norm = vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
+        const float* q_norm = vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
+        const float* k_norm = vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
+        const float* ffn_norm = vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
+        const Weight* wqkv = mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
+        const Weight* wo = mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
+        const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
+        const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
+        if (rc) return rc;
+        // attention input: RMSNorm -> QKV, two sequences per pass over the weights
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
+            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
+            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, attn_norm, d.eps, d.h, nb, m.xq.xq,
+                                                 m.xq.cneg, m.xq.xexp, nullptr, st),
+                        "kernel launch failed: rmsnorm_quant");
+            OXB_TRY(gemv_xq(*wqkv, m.xq, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows, OXB_GEMV_STORE, nullptr));
+        }
+        OxbQkParams qp;
+        qp.qkv = m.qkv;
+        qp.qkv_stride = qkv_rows;
+        qp.q_norm = q_norm;
+        qp.k_norm = k_norm;
+        qp.cos_t = m.cos_t;
+        qp.sin_t = m.sin_t;
+        qp.pos = m.pos;
+        qp.q_rope = m.q_rope;
+        qp.k_cache = m.k_cache;
+        qp.v_cache = m.v_cache;
+        qp.nq = d.nq;
+        qp.nkv = d.nkv;
+        qp.hd = d.hd;
+        qp.max_seq = d.max_seq;
+        qp.n_layers = d.n_layers;
+        qp.layer = L;
+        qp.eps = d.eps;
+        OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, d.batch, st), "kernel launch failed: qk_norm_rope_store");
+        OxbAttnParams ap;
+        ap.q = m.q_rope;
+        ap.k_cache = m.k_cache;
+        ap.v_cache = m.v_cache;
+        ap.part = m.attn_part;
+        ap.pos = m.pos;
+        ap.nq = d.nq;
+        ap.nkv = d.nkv;
+        ap.hd = d.hd;
+        ap.max_seq = d.max_seq;
+        ap.n_layers = d.n_layers;
+        ap.layer = L;
+        ap.chunk = m.chunk;
+        ap.n_splits = m.n_splits;
+        ap.scale = 1.0f / sqrtf((float)d.hd);
+        OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, m.attn_out, st), "kernel launch failed: attention");
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
+            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
+            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo,
+                               *wgu, *wdn, m.gu + (size_t)b0 * 2 * d.inter, d.h, d.inter, qd, nb));
+        }
+    }
+    if (with_lm_head) {
+        const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
+        const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+        if (rc) return rc;
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
+            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
+            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, final_norm, d.eps, d.h, nb, m.xq.xq,
+                                                 m.xq.cneg, m.xq.xexp, nullptr, st),
+                        "kernel launch failed: rmsnorm_quant");
+            OXB_TRY(gemv_xq(*lm, m.xq, nb, m.logits + (size_t)b0 * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
+        }
+        OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, st), "kernel launch failed: argmax");
+    }
+    return OXB_HIP_OK;
+}
+
+static Model* find_model(uint64_t id) {
+    auto it = g_models.find(id);
+    return it == g_models.end() ? nullptr : it->second.get();
+}
+
 }  // namespace oxb
+
+using namespace oxb;
+
+extern "C" {
+
+int oxb_hip_upload_f32(uint64_t* id, const float* w, size_t n) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!id || !w || n == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or empty vector");
+    OXB_TRY(ensure_init());
+    Vector v;
+    v.n = n;
+    if (hipMalloc((void**)&v.d, n * sizeof(float)) != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", n * sizeof(float), g_rt.device);
+    hipError_t e = hipMemcpy(v.d, w, n * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(v.d);
+        return hip_fail(e, "vector upload");
+    }
+    if (*id == 0) *id = g_rt.next_id++;
+    auto it = g_rt.vectors.find(*id);
+    if (it != g_rt.vectors.end()) (void)hipFree(it->second.d);
+    g_rt.vectors[*id] = v;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_free_f32(uint64_t id) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    auto it = g_rt.vectors.find(id);
+    if (it == g_rt.vectors.end()) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    if (g_rt.ready) (void)hipStreamSynchronize(g_rt.stream);
+    (void)hipFree(it->second.d);
+    g_rt.vectors.erase(it);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!desc || !model || !desc->layers) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
+    OXB_TRY(ensure_init());
+    const oxb_model_desc& d = *desc;
+    if (d.fmt != OXB_FMT_Q1 && d.fmt != OXB_FMT_TQ2) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown format %d", d.fmt);
+    if (!d.n_layers || !d.h || !d.inter || !d.nq || !d.nkv || !d.vocab || !d.max_seq || !d.batch)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: a model dimension is 0");
+    if (d.hd != 32 && d.hd != 64 && d.hd != 128 && d.hd != 256)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: head_dim %u (supported: 32, 64, 128, 256)", d.hd);
+    if (d.nq % d.nkv != 0 || d.nq / d.nkv > 8)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u query heads per %u kv heads (need a whole ratio <= 8)", d.nq, d.nkv);
+    if (d.h % 128 || d.inter % 128 || (d.nq * d.hd) % 128)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden, intermediate and nq*hd must be multiples of 128");
+    auto mp = std::make_unique<Model>();
+    Model& m = *mp;
+    m.d = d;
+    m.layers.assign(d.layers, d.layers + d.n_layers);
+    m.d.layers = nullptr;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    // check every handle now, so that a decode step cannot fail half way
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < d.n_layers && !rc; L++) {
+        const oxb_layer_ids& ly = m.layers[L];
+        vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
+        vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
+        vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
+        vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
+        mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
+        mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
+        mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
+        mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
+    }
+    if (!rc) vec_ptr(d.final_norm, d.h, "final_norm", &rc);
+    if (!rc) mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+    if (rc) return rc;
+
+    m.chunk = 1024;
+    while (m.chunk > 64 && m.chunk / 2 >= d.max_seq) m.chunk /= 2;
+    m.n_splits = (d.max_seq + m.chunk - 1) / m.chunk;
+    const size_t B = d.batch;
+    const size_t kv_elems = B * d.n_layers * d.nkv * (size_t)d.max_seq * d.hd;
+    uint32_t kmax = d.h > d.inter ? d.h : d.inter;
+    if (qd > kmax) kmax = qd;
+    const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
+    if ((rc = dev_alloc(m, (void**)&m.hidden, B * d.h * 4)) || (rc = dev_alloc(m, (void**)&m.qkv, B * qkv_rows * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.q_rope, B * qd * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + 2) * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, (void**)&m.k_cache, kv_elems * 2)) ||
+        (rc = dev_alloc(m, (void**)&m.v_cache, kv_elems * 2)) ||
+        (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
+        (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + 256))) {
+        free_model(m);
+        return rc;
+    }
+    m.xq.xq = (uint32_t*)m.xq_mem;
+    m.xq.cneg = (int32_t*)((uint8_t*)m.xq_mem + xq_b);
+    m.xq.xexp = (int32_t*)((uint8_t*)m.xq_mem + xq_b + cn_b);
+    // RoPE table, computed as RopeTable::new does (crates/oxibonsai-model/src/layers/rope.rs:27-48): all in f32.
+    {
+        const size_t half = d.hd / 2;
+        std::vector<float> c((size_t)d.max_seq * half), s((size_t)d.max_seq * half);
+        for (size_t pos = 0; pos < d.max_seq; pos++)
+            for (size_t i = 0; i < half; i++) {
+                const float freq = 1.0f / powf(d.rope_theta, 2.0f * (float)i / (float)d.hd);
+                const float angle = (float)pos * freq;
+                c[pos * half + i] = cosf(angle);
+                s[pos * half + i] = sinf(angle);
+            }
+        hipError_t e = hipMemcpy(m.cos_t, c.data(), c.size() * 4, hipMemcpyHostToDevice);
+        if (e == hipSuccess) e = hipMemcpy(m.sin_t, s.data(), s.size() * 4, hipMemcpyHostToDevice);
+        if (e != hipSuccess) {
+            free_model(m);
+            return hip_fail(e, "rope table upload");
+        }
+    }
+    const char* no_graph = getenv("OXB_HIP_DISABLE_GRAPH");
+    m.graph_failed = no_graph && no_graph[0] == '1';
+    *model = g_next_model++;
+    g_models[*model] = std::move(mp);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_destroy(uint64_t model) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    (void)hipStreamSynchronize(g_rt.stream);
+    free_model(*m);
+    g_models.erase(model);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_reset(uint64_t model) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    // positions are supplied per call and attention reads only 0..pos, so nothing has to be cleared
+    (void)hipStreamSynchronize(g_rt.stream);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (!hidden || !pos) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden or pos");
+    for (uint32_t b = 0; b < d.batch; b++)
+        if (pos[b] >= d.max_seq)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    if (m.graph_exec) {
+        OXB_TRY_HIP(hipGraphLaunch(m.graph_exec, st), "graph launch");
+    } else if (!m.graph_failed && st == g_rt.own_stream) {
+        // capture the whole token once; on any capture problem fall back to plain launches for good
+        hipGraph_t graph = nullptr;
+        hipError_t e = hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal);
+        int rc = OXB_HIP_OK;
+        if (e == hipSuccess) {
+            rc = encode_decode_step(m, true);
+            hipError_t e2 = hipStreamEndCapture(st, &graph);
+            if (rc == OXB_HIP_OK && e2 == hipSuccess && graph) e = hipGraphInstantiate(&m.graph_exec, graph, nullptr, nullptr, 0);
+            else e = e2 == hipSuccess ? hipErrorUnknown : e2;
+            if (graph) (void)hipGraphDestroy(graph);
+        }
+        if (rc) return rc;
+        if (e != hipSuccess || !m.graph_exec) {
+            (void)hipGetLastError();
+            m.graph_exec = nullptr;
+            m.graph_failed = true;
+            OXB_TRY(encode_decode_step(m, true));
+        } else {
+            OXB_TRY_HIP(hipGraphLaunch(m.graph_exec, st), "graph launch");
+        }
+    } else {
+        OXB_TRY(encode_decode_step(m, true));
+    }
+    if (token_out) OXB_TRY_HIP(hipMemcpyAsync(token_out, m.tokens, (size_t)d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
+    if (logits_or_null)
+        OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits, (size_t)d.batch * d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_uses_graph(uint64_t model) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    return m && m->graph_exec ? 1 : 0;
+}
+
+int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float* norm_w, float eps, uint64_t o_id,
+                      uint64_t gate_up_id, uint64_t down_id, uint32_t h, uint32_t inter, uint32_t attn_k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!hidden || !attn_out || !norm_w) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
+    if (h % 128 || inter % 128 || attn_k % 128) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: dimensions must be multiples of 128");
+    int rc = OXB_HIP_OK;
+    const Weight* wo = mat_ptr(o_id, fmt, h, attn_k, "attn_proj", &rc);
+    const Weight* wgu = mat_ptr(gate_up_id, fmt, 2 * inter, h, "gate_up", &rc);
+    const Weight* wdn = mat_ptr(down_id, fmt, h, inter, "down", &rc);
+    if (rc) return rc;
+    uint32_t kmax = h > inter ? h : inter;
+    if (attn_k > kmax) kmax = attn_k;
+    const size_t xq_b = oxb_xq_bytes(kmax, 1), cn_b = oxb_cneg_bytes(kmax, 1);
+    OXB_TRY(g_rt.ws_xq.ensure(xq_b + cn_b + 256));
+    OXB_TRY(g_rt.ws_x.ensure(((size_t)h * 2 + attn_k) * 4));
+    OXB_TRY(g_rt.ws_y.ensure((size_t)2 * inter * 4));
+    XqBuf xb;
+    xb.xq = (uint32_t*)g_rt.ws_xq.ptr;
+    xb.cneg = (int32_t*)((uint8_t*)g_rt.ws_xq.ptr + xq_b);
+    xb.xexp = (int32_t*)((uint8_t*)g_rt.ws_xq.ptr + xq_b + cn_b);
+    float* d_hidden = (float*)g_rt.ws_x.ptr;
+    float* d_norm = d_hidden + h;
+    float* d_attn = d_norm + h;
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(d_hidden, hidden, (size_t)h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(d_norm, norm_w, (size_t)h * 4, hipMemcpyHostToDevice, st), "norm upload");
+    OXB_TRY_HIP(hipMemcpyAsync(d_attn, attn_out, (size_t)attn_k * 4, hipMemcpyHostToDevice, st), "attn_out upload");
+    OXB_TRY(encode_ffn(fmt, xb, d_hidden, d_attn, d_norm, eps, *wo, *wgu, *wdn, (float*)g_rt.ws_y.ptr, h, inter, attn_k, 1));
+    OXB_TRY_HIP(hipMemcpyAsync(hidden, d_hidden, (size_t)h * 4, hipMemcpyDeviceToHost, st), "hidden download");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+}
+
+}  // extern "C"

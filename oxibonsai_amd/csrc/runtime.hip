@@ -234,6 +234,8 @@ void oxb_hip_shutdown(void) {
     shutdown_models();
     for (auto& kv : g_rt.weights) free_weight_mem(kv.second);
     g_rt.weights.clear();
+    for (auto& kv : g_rt.vectors) (void)hipFree(kv.second.d);
+    g_rt.vectors.clear();
     g_rt.ws_x.release();
     g_rt.ws_y.release();
     g_rt.ws_xq.release();

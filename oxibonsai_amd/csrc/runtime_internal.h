@@ -24,6 +24,11 @@ struct Weight {  // one resident matrix: [codes section][scales section]
     uint16_t* d_scales = nullptr;
 };
 
+struct Vector {  // a resident fp32 vector (norm weights)
+    float* d = nullptr;
+    size_t n = 0;
+};
+
 struct Runtime {
     bool ready = false;
     int device = -1;
@@ -31,6 +36,7 @@ struct Runtime {
     char name[256] = {0};
     hipStream_t own_stream = nullptr, stream = nullptr;
     std::unordered_map<uint64_t, Weight> weights;
+    std::unordered_map<uint64_t, Vector> vectors;
     uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
 };

@@ -1,0 +1,108 @@
+"""Host-side mirror of the reference's fused whole-model GPU forward.
+
+``HipModel`` plays the part of ``BonsaiModel``'s GPU branch
+(crates/oxibonsai-model/src/model/types/forward_cuda/{q1,ternary}.rs): it uploads every
+layer's blocks once (fused Q|K|V and gate|up concatenations are made on the AoS bytes, as
+crates/oxibonsai-model/src/block/types/upload.rs:21-39 does), then each ``forward`` is one
+call of ``oxb_hip_decode`` = ``try_cuda_full_forward_with_gpu_lm_head``."""
+from __future__ import annotations
+
+import ctypes as C
+
+import numpy as np
+
+from . import _lib
+from .backend import GpuError, NativeHipBackend, _check
+from .synth import Q1
+
+
+class _LayerIds(C.Structure):
+    _fields_ = [(n, C.c_uint64) for n in ("attn_norm", "qkv", "q_norm", "k_norm", "o", "ffn_norm", "gate_up", "down")]
+
+
+class _ModelDesc(C.Structure):
+    _fields_ = [("fmt", C.c_int)] + [(n, C.c_uint32) for n in
+                                      ("n_layers", "h", "inter", "nq", "nkv", "hd", "vocab", "max_seq", "batch")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float), ("layers", C.POINTER(_LayerIds)),
+                ("final_norm", C.c_uint64), ("lm_head", C.c_uint64)]
+
+
+class HipModel:
+    """cfg: fmt, n_layers, h, inter, nq, nkv, hd, vocab, max_seq, eps, rope_theta.
+    weights: dict of oxibonsai_amd.synth.make_model (reference AoS blocks + f32 norm vectors)."""
+
+    def __init__(self, backend: NativeHipBackend, cfg: dict, weights: dict, batch: int = 1):
+        self.be, self.cfg, self.batch = backend, cfg, batch
+        self._lib = _lib.lib()
+        self._mats, self._vecs = [], []
+        fmt, h, inter, hd = cfg["fmt"], cfg["h"], cfg["inter"], cfg["hd"]
+        qd, kd = cfg["nq"] * hd, cfg["nkv"] * hd
+        ids = (_LayerIds * cfg["n_layers"])()
+        for i, lw in enumerate(weights["layers"]):
+            qkv = np.concatenate([lw["q"], lw["k"], lw["v"]])
+            gate_up = np.concatenate([lw["gate"], lw["up"]])
+            ids[i] = _LayerIds(self._vec(lw["attn_norm"]), self._mat(qkv, qd + 2 * kd, h), self._vec(lw["q_norm"]),
+                               self._vec(lw["k_norm"]), self._mat(lw["o"], h, qd), self._vec(lw["ffn_norm"]),
+                               self._mat(gate_up, 2 * inter, h), self._mat(lw["down"], h, inter))
+        self._ids = ids
+        desc = _ModelDesc(fmt, cfg["n_layers"], h, inter, cfg["nq"], cfg["nkv"], hd, cfg["vocab"], cfg["max_seq"], batch,
+                          cfg["eps"], cfg["rope_theta"], ids, self._vec(weights["final_norm"]),
+                          self._mat(weights["lm_head"], cfg["vocab"], h))
+        mid = C.c_uint64(0)
+        _check(self._lib.oxb_hip_model_create(C.byref(desc), C.byref(mid)))
+        self.id = mid.value
+
+    def _mat(self, blocks, n_rows, k):
+        fmt = self.cfg["fmt"]
+        h = self.be.upload_weights_raw(blocks, n_rows, k) if fmt == Q1 else self.be.upload_weights_ternary(blocks, n_rows, k)
+        self._mats.append(h)
+        return int(h)
+
+    def _vec(self, v):
+        a = np.ascontiguousarray(v, dtype=np.float32)
+        hid = C.c_uint64(0)
+        _check(self._lib.oxb_hip_upload_f32(C.byref(hid), a.ctypes.data_as(_lib.f32p), a.size))
+        self._vecs.append(hid.value)
+        return hid.value
+
+    def forward(self, hidden, pos, want_logits: bool = True):
+        """hidden: [batch, h] embedding rows; pos: [batch] positions -> (logits [batch, vocab] or None, tokens [batch])."""
+        hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(self.batch, self.cfg["h"])
+        pv = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, dtype=np.uint32), (self.batch,)))
+        logits = np.empty((self.batch, self.cfg["vocab"]), dtype=np.float32) if want_logits else None
+        tokens = np.empty(self.batch, dtype=np.uint32)
+        _check(self._lib.oxb_hip_decode(self.id, hv.ctypes.data_as(_lib.f32p), pv.ctypes.data_as(_lib.u32p),
+                                        logits.ctypes.data_as(_lib.f32p) if want_logits else None,
+                                        tokens.ctypes.data_as(_lib.u32p)))
+        return logits, tokens
+
+    def uses_graph(self) -> bool:
+        return bool(self._lib.oxb_hip_model_uses_graph(self.id))
+
+    def reset(self):
+        _check(self._lib.oxb_hip_model_reset(self.id))
+
+    def close(self):
+        if self.id:
+            _check(self._lib.oxb_hip_model_destroy(self.id))
+            self.id = 0
+            for h in self._mats:
+                self.be.free_weights(h)
+            for v in self._vecs:
+                _check(self._lib.oxb_hip_free_f32(v))
+            self._mats, self._vecs = [], []
+
+
+def batch_ffn_phase(backend: NativeHipBackend, fmt: int, hidden, attn_out, norm_weight, norm_eps: float,
+                    attn_proj_handle: int, gate_up_handle: int, down_handle: int, h: int, intermediate: int,
+                    attn_proj_k: int) -> np.ndarray:
+    """GpuBackendTrait::batch_ffn_phase (gpu_backend/mod.rs:519): returns the updated hidden vector."""
+    hv = np.array(hidden, dtype=np.float32, copy=True)
+    av = np.ascontiguousarray(attn_out, dtype=np.float32)
+    nv = np.ascontiguousarray(norm_weight, dtype=np.float32)
+    if hv.size < h or av.size < attn_proj_k or nv.size < h:
+        raise GpuError(5, "invalid argument: buffer shorter than its dimension")
+    _check(_lib.lib().oxb_hip_ffn_phase(fmt, hv.ctypes.data_as(_lib.f32p), av.ctypes.data_as(_lib.f32p),
+                                        nv.ctypes.data_as(_lib.f32p), norm_eps, int(attn_proj_handle),
+                                        int(gate_up_handle), int(down_handle), h, intermediate, attn_proj_k))
+    return hv

@@ -80,3 +80,69 @@ def test_argmax_tie_rules():
     v = np.array([1.0, 5.0, 3.0, 5.0, 2.0], dtype=np.float32)
     assert oracle.argmax_last(v) == 3      # runtime/src/sampling.rs:182-189 (max_by keeps the last)
     assert oracle.argmax_first(v) == 1     # gpu_backend/cuda_kernels.rs:407-436 (strict >)
+
+
+# ---- whole-model decode against an independent float64 numpy forward -------------------------------
+def _f64_forward(cfg, w, hiddens):
+    """Textbook Qwen3 decode in float64 from the dequantised matrices (no oracle code involved except dequant,
+    which test_oracle.py pins bit for bit)."""
+    from helpers import dense_f64
+    fmt, h, hd, nq, nkv = cfg["fmt"], cfg["h"], cfg["hd"], cfg["nq"], cfg["nkv"]
+    inter, half = cfg["inter"], cfg["hd"] // 2
+
+    def rms(x, wt):
+        return wt * x / np.sqrt(np.mean(x * x) + cfg["eps"])
+
+    def rope(v, pos):
+        i = np.arange(half, dtype=np.float64)
+        ang = pos * cfg["rope_theta"] ** (-2.0 * i / hd)
+        c, s = np.cos(ang), np.sin(ang)
+        return np.concatenate([v[:half] * c - v[half:] * s, v[:half] * s + v[half:] * c])
+
+    mats = [{k: dense_f64(fmt, lw[k], *shape) for k, shape in
+             (("q", (nq * hd, h)), ("k", (nkv * hd, h)), ("v", (nkv * hd, h)), ("o", (h, nq * hd)),
+              ("gate", (inter, h)), ("up", (inter, h)), ("down", (h, inter)))} for lw in w["layers"]]
+    lm = dense_f64(fmt, w["lm_head"], cfg["vocab"], h)
+    K = [[[] for _ in range(nkv)] for _ in w["layers"]]
+    V = [[[] for _ in range(nkv)] for _ in w["layers"]]
+    outs = []
+    for pos, hid in enumerate(hiddens):
+        x = hid.astype(np.float64)
+        for L, lw in enumerate(w["layers"]):
+            n = rms(x, lw["attn_norm"].astype(np.float64))
+            q, k, v = mats[L]["q"] @ n, mats[L]["k"] @ n, mats[L]["v"] @ n
+            for kh in range(nkv):
+                K[L][kh].append(rope(rms(k[kh * hd:(kh + 1) * hd], lw["k_norm"].astype(np.float64)), pos))
+                V[L][kh].append(v[kh * hd:(kh + 1) * hd])
+            att = np.zeros(nq * hd)
+            for qh in range(nq):
+                qv = rope(rms(q[qh * hd:(qh + 1) * hd], lw["q_norm"].astype(np.float64)), pos)
+                kh = qh // (nq // nkv)
+                sc = np.array(K[L][kh]) @ qv / np.sqrt(hd)
+                p = np.exp(sc - sc.max())
+                att[qh * hd:(qh + 1) * hd] = (p / p.sum()) @ np.array(V[L][kh])
+            x = x + mats[L]["o"] @ att
+            n = rms(x, lw["ffn_norm"].astype(np.float64))
+            g, u = mats[L]["gate"] @ n, mats[L]["up"] @ n
+            x = x + mats[L]["down"] @ (g / (1 + np.exp(-g)) * u)
+        outs.append(lm @ rms(x, w["final_norm"].astype(np.float64)))
+    return outs
+
+
+def test_model_forward_matches_float64_numpy():
+    import pytest
+    from oxibonsai_amd import synth
+    base = dict(n_layers=2, h=128, inter=256, nq=4, nkv=2, hd=32, vocab=32, max_seq=16, eps=1e-6, rope_theta=1e6)
+    for fmt in (0, 1):
+        cfg = dict(base, fmt=fmt)
+        w = synth.make_model(cfg, 7 + fmt)
+        hiddens = [synth.embedding_rows(3, [t], cfg["h"])[0] * 50.0 for t in (5, 9, 2, 30, 11, 4)]
+        want = _f64_forward(cfg, w, hiddens)
+        m = oracle.OracleModel(cfg, w, kv_f16=False)
+        for pos, hid in enumerate(hiddens):
+            got = m.forward(hid, pos)
+            assert np.max(np.abs(got - want[pos])) < 2e-4 * max(1.0, np.max(np.abs(want[pos]))), (fmt, pos)
+        # with the f16 KV rounding of the reference's GPU cache the logits move, but only slightly
+        m16 = oracle.OracleModel(cfg, w, kv_f16=True)
+        d = max(np.max(np.abs(m16.forward(hid, pos) - want[pos])) for pos, hid in enumerate(hiddens))
+        assert 0 < d < 2e-2
