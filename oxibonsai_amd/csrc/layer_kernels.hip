@@ -146,7 +146,7 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
 //  CPU: block/functions.rs:78-127 -> layers/attention_fused.rs:329-400).
 // Grid (n_splits, nkv, batch), 256 threads.  A workgroup serves all q heads of one kv head for one
 // chunk of positions, so K and V are read once per group: scores with one position per thread,
-// then the weighted sum with one head dimension per thread.  It writes the un-normalised partial
+// then the weighted sum with eight head dimensions and a slice of the positions per thread.  It writes the un-normalised partial
 // output, the chunk maximum and the chunk sum; attn_combine_kernel merges the chunks.
 // ---------------------------------------------------------------------------
 #define OXB_ATTN_THREADS 256
@@ -248,20 +248,39 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
         if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = lsum[h];
     }
     __syncthreads();  // also publishes the exponentials
-    // weighted sum of V: thread -> (dimension d, slice of positions)
-    const uint32_t n_slices = OXB_ATTN_THREADS / hd, d = tid % hd, slice = tid / hd;
-    float acc[OXB_ATTN_MAXG];
+    // weighted sum of V: thread -> (group of 8 dimensions, slice of positions); one 16-byte load per position
+    const uint32_t n_grp = hd / 8, n_slices = OXB_ATTN_THREADS / n_grp, grp = tid % n_grp, slice = tid / n_grp;
+    float acc[OXB_ATTN_MAXG][8];
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++) acc[h] = 0.f;
+    for (int h = 0; h < OXB_ATTN_MAXG; h++)
+#pragma unroll
+        for (int i = 0; i < 8; i++) acc[h][i] = 0.f;
+#pragma unroll 4
     for (uint32_t t = s0 + slice; t < s1; t += n_slices) {
-        const float v = __half2float(V[(size_t)t * hd + d]);
+        const uint4 vv = *reinterpret_cast<const uint4*>(V + (size_t)t * hd + grp * 8);
+        const __half2* v2 = reinterpret_cast<const __half2*>(&vv);
+        float vf[8];
 #pragma unroll
-        for (int h = 0; h < OXB_ATTN_MAXG; h++)
-            if ((uint32_t)h < G) acc[h] = fmaf(sc[h * chunk + (t - s0)], v, acc[h]);
+        for (int i = 0; i < 4; i++) {
+            const float2 f = __half22float2(v2[i]);
+            vf[2 * i] = f.x;
+            vf[2 * i + 1] = f.y;
+        }
+#pragma unroll
+        for (int h = 0; h < OXB_ATTN_MAXG; h++) {
+            if ((uint32_t)h < G) {
+                const float pr = sc[h * chunk + (t - s0)];
+#pragma unroll
+                for (int i = 0; i < 8; i++) acc[h][i] = fmaf(pr, vf[i], acc[h][i]);
+            }
+        }
     }
 #pragma unroll
     for (int h = 0; h < OXB_ATTN_MAXG; h++)
-        if ((uint32_t)h < G) accs[(slice * G + h) * hd + d] = acc[h];
+        if ((uint32_t)h < G) {
+#pragma unroll
+            for (int i = 0; i < 8; i++) accs[(slice * G + h) * hd + grp * 8 + i] = acc[h][i];
+        }
     __syncthreads();
     for (uint32_t i = tid; i < G * hd; i += OXB_ATTN_THREADS) {
         float v = 0.f;
@@ -355,7 +374,7 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 }
 
 size_t oxb_attn_smem_bytes(uint32_t nq, uint32_t nkv, uint32_t hd, uint32_t chunk) {
-    const uint32_t G = nq / nkv, slices = OXB_ATTN_THREADS / hd;
+    const uint32_t G = nq / nkv, slices = OXB_ATTN_THREADS / (hd / 8);
     return ((size_t)G * hd + (size_t)G * chunk + OXB_ATTN_MAXG * 4 + (size_t)slices * G * hd) * sizeof(float);
 }
 
