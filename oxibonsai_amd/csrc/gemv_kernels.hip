@@ -32,7 +32,7 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 // The activation quantiser (quant_device.h) produces the MFMA B operands ("digit planes").
-#define OXB_QUANT_THREADS 512
+#define OXB_QUANT_THREADS 256
 
 template <int FMT>
 __global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float* __restrict__ x, uint32_t k,
@@ -54,7 +54,7 @@ __global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float*
     }
     bool any_bad;
     mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);
-    quantise_vector<FMT>(xn, k, nblk_pad, NC, n, mx, any_bad, xq, cneg, xexp);
+    quantise_vector<FMT>(xn, k, nblk_pad, NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
 }
 
 // ---------------------------------------------------------------------------
@@ -290,10 +290,10 @@ hipError_t oxb_launch_quant_x(int fmt, const float* d_x, uint32_t k, uint32_t ba
     const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
     const size_t shm = 0;
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, dim3(batch), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, dim3(batch, oxb_quant_parts(k)), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
                            d_cneg, d_xexp);
     else
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, dim3(batch), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, dim3(batch, oxb_quant_parts(k)), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
                            d_cneg, d_xexp);
     return hipGetLastError();
 }

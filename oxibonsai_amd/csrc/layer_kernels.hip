@@ -13,7 +13,7 @@
 #include "layer_kernels.h"
 #include "quant_device.h"
 
-#define OXB_LAYER_THREADS 512
+#define OXB_LAYER_THREADS 256
 
 __device__ __forceinline__ float block_sum(float v, float* red) {  // two barriers; red: blockDim.x / 64 floats
 #pragma unroll
@@ -30,7 +30,8 @@ __device__ __forceinline__ float block_sum(float v, float* red) {  // two barrie
 // RMSNorm fused with the activation quantiser (rms_norm: crates/oxibonsai-kernels/src/
 // simd_float_ops.rs:204-215; GPU twin rmsnorm_weighted_v2, gpu_backend/cuda_kernels.rs:335-374).
 // out[i] = w[i] * x[i] * (1 / sqrt(mean(x^2) + eps)); the normalised vector lives only in LDS.
-// Grid: one workgroup per vector of the pass.
+// Grid (vectors of the pass, parts): every part repeats the two reductions (the vector is a few KB in L2) and
+// quantises its share of the blocks.
 // ---------------------------------------------------------------------------
 template <int FMT>
 __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const float* __restrict__ x,
@@ -58,13 +59,13 @@ __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const 
     for (uint32_t i = tid; i < h; i += OXB_LAYER_THREADS) {
         const float v = w[i] * lds_x[i] * inv_rms;
         lds_x[i] = v;
-        if (normed_out) normed_out[(size_t)n * h + i] = v;
+        if (normed_out && blockIdx.y == 0) normed_out[(size_t)n * h + i] = v;
         bad |= oxb_not_finite(v);
         mx = fmaxf(mx, fabsf(v));
     }
     bool any_bad;
     mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);  // its barriers also publish lds_x
-    quantise_vector<FMT>(lds_x, h, oxb_nblk_pad(h), NC, n, mx, any_bad, xq, cneg, xexp);
+    quantise_vector<FMT>(lds_x, h, oxb_nblk_pad(h), NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
 }
 
 // ---------------------------------------------------------------------------
@@ -94,7 +95,7 @@ __global__ __launch_bounds__(OXB_LAYER_THREADS) void swiglu_quant_kernel(const f
     }
     bool any_bad;
     mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);
-    quantise_vector<FMT>(lds_x, inter, oxb_nblk_pad(inter), NC, n, mx, any_bad, xq, cneg, xexp);
+    quantise_vector<FMT>(lds_x, inter, oxb_nblk_pad(inter), NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
 }
 
 // ---------------------------------------------------------------------------
@@ -150,146 +151,157 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
 // output, the chunk maximum and the chunk sum; attn_combine_kernel merges the chunks.
 // ---------------------------------------------------------------------------
 #define OXB_ATTN_THREADS 256
-#define OXB_ATTN_MAXG 8  // q heads per kv head supported
+#define OXB_ATTN_CHUNK 256  // positions per workgroup = threads: one position per thread in the score phase
 
+__device__ __forceinline__ void unpack8(const uint4& u, float f[8]) {
+    const __half2* h2 = reinterpret_cast<const __half2*>(&u);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float2 t = __half22float2(h2[i]);
+        f[2 * i] = t.x;
+        f[2 * i + 1] = t.y;
+    }
+}
+
+// HD = head dimension, GM = q heads per kv head rounded up to a power of two (loops over heads are
+// unrolled to GM and predicated on the real count G).
+template <int HD, int GM>
 __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnParams p) {
-    extern __shared__ float smem[];  // q[G][hd] | sc[G][chunk] | red[G][4] | accs[slices][G][hd]
-    const uint32_t split = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z, tid = threadIdx.x;
-    const uint32_t hd = p.hd, G = p.nq / p.nkv, chunk = p.chunk;
+    constexpr int NG = HD / 8;                       // 16-byte groups per row
+    constexpr int NSL = OXB_ATTN_THREADS / NG;       // position slices in the weighted-sum phase
+    constexpr int PPS = OXB_ATTN_CHUNK / NSL;        // positions per slice
+    __shared__ float q_s[GM * HD];
+    __shared__ float sc[GM * OXB_ATTN_CHUNK];
+    __shared__ float red[GM * 4];
+    __shared__ float accs[NSL * GM * HD];
+    // blockIdx.y = kv head * nsub + sub: with more than GM q heads per kv head the group is served
+    // by nsub workgroups of up to GM heads each
+    const uint32_t nsub = gridDim.y / p.nkv, kvh = blockIdx.y / nsub, sub = blockIdx.y % nsub;
+    const uint32_t split = blockIdx.x, b = blockIdx.z, tid = threadIdx.x;
+    const uint32_t Gall = p.nq / p.nkv, h0 = kvh * Gall + sub * GM;  // first q head served here
+    const uint32_t G = (Gall - sub * GM) < (uint32_t)GM ? (Gall - sub * GM) : (uint32_t)GM;
     const uint32_t seq_len = p.pos[b] + 1;
-    const uint32_t s0 = split * chunk;
-    const uint32_t s1 = (s0 + chunk) < seq_len ? (s0 + chunk) : seq_len;
-    float* part = p.part + (((size_t)b * p.nq + (size_t)kvh * G) * p.n_splits + split) * (hd + 2);
-    const size_t part_head = (size_t)p.n_splits * (hd + 2);
+    const uint32_t s0 = split * OXB_ATTN_CHUNK;
+    const uint32_t s1 = (s0 + OXB_ATTN_CHUNK) < seq_len ? (s0 + OXB_ATTN_CHUNK) : seq_len;
+    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + split) * (HD + 2);
+    const size_t part_head = (size_t)p.n_splits * (HD + 2);
     if (s0 >= seq_len) {  // nothing in this chunk: mark it empty for every head of the group
         if (tid < G) {
-            part[tid * part_head + hd] = -INFINITY;
-            part[tid * part_head + hd + 1] = 0.f;
+            part[tid * part_head + HD] = -INFINITY;
+            part[tid * part_head + HD + 1] = 0.f;
         }
         return;
     }
-    float* q_s = smem;
-    float* sc = q_s + G * hd;
-    float* red = sc + G * chunk;
-    float* accs = red + OXB_ATTN_MAXG * 4;
-    for (uint32_t i = tid; i < G * hd; i += OXB_ATTN_THREADS) q_s[i] = p.q[((size_t)b * p.nq + (size_t)kvh * G) * hd + i];
-    __syncthreads();
-    const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * hd;
+    const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * HD;
     const __half* K = p.k_cache + base;
     const __half* V = p.v_cache + base;
+    const uint32_t t = s0 + tid;
+    const bool live = t < s1;
 
-    // scores: one position per thread
-    float lmax[OXB_ATTN_MAXG];
+    // this thread's K row, all of it in flight at once
+    uint4 kreg[NG];
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++) lmax[h] = -INFINITY;
-    for (uint32_t t = s0 + tid; t < s1; t += OXB_ATTN_THREADS) {
-        float dot[OXB_ATTN_MAXG];
+    for (int i = 0; i < NG; i++)
+        kreg[i] = live ? reinterpret_cast<const uint4*>(K + (size_t)t * HD)[i] : make_uint4(0, 0, 0, 0);
+    for (uint32_t i = tid; i < G * HD; i += OXB_ATTN_THREADS) q_s[i] = p.q[((size_t)b * p.nq + h0) * HD + i];
+    __syncthreads();
+
+    // scores
+    float dot[GM];
 #pragma unroll
-        for (int h = 0; h < OXB_ATTN_MAXG; h++) dot[h] = 0.f;
-        const uint4* kr = reinterpret_cast<const uint4*>(K + (size_t)t * hd);
-        for (uint32_t d8 = 0; d8 < hd / 8; d8++) {
-            const uint4 kk = kr[d8];
-            const __half2* k2 = reinterpret_cast<const __half2*>(&kk);
-            float kf[8];
+    for (int h = 0; h < GM; h++) dot[h] = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const float2 f = __half22float2(k2[i]);
-                kf[2 * i] = f.x;
-                kf[2 * i + 1] = f.y;
-            }
+    for (int i = 0; i < NG; i++) {
+        float kf[8];
+        unpack8(kreg[i], kf);
 #pragma unroll
-            for (int h = 0; h < OXB_ATTN_MAXG; h++) {
-                if ((uint32_t)h < G) {
-                    const float* qh = q_s + h * hd + d8 * 8;
-#pragma unroll
-                    for (int i = 0; i < 8; i++) dot[h] = fmaf(qh[i], kf[i], dot[h]);
-                }
-            }
-        }
-#pragma unroll
-        for (int h = 0; h < OXB_ATTN_MAXG; h++) {
+        for (int h = 0; h < GM; h++) {
             if ((uint32_t)h < G) {
-                const float s = dot[h] * p.scale;
-                sc[h * chunk + (t - s0)] = s;
-                lmax[h] = fmaxf(lmax[h], s);
+                const float4 qa = *reinterpret_cast<const float4*>(&q_s[h * HD + i * 8]);
+                const float4 qb = *reinterpret_cast<const float4*>(&q_s[h * HD + i * 8 + 4]);
+                dot[h] = fmaf(qa.x, kf[0], dot[h]);
+                dot[h] = fmaf(qa.y, kf[1], dot[h]);
+                dot[h] = fmaf(qa.z, kf[2], dot[h]);
+                dot[h] = fmaf(qa.w, kf[3], dot[h]);
+                dot[h] = fmaf(qb.x, kf[4], dot[h]);
+                dot[h] = fmaf(qb.y, kf[5], dot[h]);
+                dot[h] = fmaf(qb.z, kf[6], dot[h]);
+                dot[h] = fmaf(qb.w, kf[7], dot[h]);
             }
         }
+    }
+    // start the V loads of the weighted-sum phase now; they land while the softmax statistics are made
+    const uint32_t grp = tid % NG, slice = tid / NG;
+    uint4 vreg[PPS];
+#pragma unroll
+    for (int i = 0; i < PPS; i++) {
+        const uint32_t tv = s0 + slice + (uint32_t)i * NSL;
+        vreg[i] = tv < s1 ? *reinterpret_cast<const uint4*>(V + (size_t)tv * HD + grp * 8) : make_uint4(0, 0, 0, 0);
     }
     // chunk maximum per head
+    float m[GM];
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++) {
+    for (int h = 0; h < GM; h++) {
+        float s = live ? dot[h] * p.scale : -INFINITY;
+        dot[h] = s;
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) lmax[h] = fmaxf(lmax[h], __shfl_xor(lmax[h], o, 64));
-        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = lmax[h];
+        for (int o = 32; o > 0; o >>= 1) s = fmaxf(s, __shfl_xor(s, o, 64));
+        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = s;
     }
     __syncthreads();
-    float m[OXB_ATTN_MAXG], lsum[OXB_ATTN_MAXG];
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++) {
-        m[h] = fmaxf(fmaxf(red[h * 4], red[h * 4 + 1]), fmaxf(red[h * 4 + 2], red[h * 4 + 3]));
-        lsum[h] = 0.f;
-    }
+    for (int h = 0; h < GM; h++) m[h] = fmaxf(fmaxf(red[h * 4], red[h * 4 + 1]), fmaxf(red[h * 4 + 2], red[h * 4 + 3]));
     __syncthreads();
     // exponentials and their sum
-    for (uint32_t t = s0 + tid; t < s1; t += OXB_ATTN_THREADS) {
 #pragma unroll
-        for (int h = 0; h < OXB_ATTN_MAXG; h++) {
-            if ((uint32_t)h < G) {
-                const float e = expf(sc[h * chunk + (t - s0)] - m[h]);
-                sc[h * chunk + (t - s0)] = e;
-                lsum[h] += e;
-            }
-        }
+    for (int h = 0; h < GM; h++) {
+        float e = ((uint32_t)h < G && live) ? expf(dot[h] - m[h]) : 0.f;
+        if ((uint32_t)h < G) sc[h * OXB_ATTN_CHUNK + tid] = e;
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, 64);
+        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = e;
     }
+    __syncthreads();  // publishes the exponentials and the per-wave sums
+    // weighted sum of V: thread -> (group of 8 dimensions, slice of positions)
+    float acc[GM][8];
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) lsum[h] += __shfl_xor(lsum[h], o, 64);
-        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = lsum[h];
-    }
-    __syncthreads();  // also publishes the exponentials
-    // weighted sum of V: thread -> (group of 8 dimensions, slice of positions); one 16-byte load per position
-    const uint32_t n_grp = hd / 8, n_slices = OXB_ATTN_THREADS / n_grp, grp = tid % n_grp, slice = tid / n_grp;
-    float acc[OXB_ATTN_MAXG][8];
-#pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++)
+    for (int h = 0; h < GM; h++)
 #pragma unroll
         for (int i = 0; i < 8; i++) acc[h][i] = 0.f;
-#pragma unroll 4
-    for (uint32_t t = s0 + slice; t < s1; t += n_slices) {
-        const uint4 vv = *reinterpret_cast<const uint4*>(V + (size_t)t * hd + grp * 8);
-        const __half2* v2 = reinterpret_cast<const __half2*>(&vv);
+#pragma unroll
+    for (int i = 0; i < PPS; i++) {
         float vf[8];
+        unpack8(vreg[i], vf);
+        const uint32_t lt = slice + (uint32_t)i * NSL;  // position within the chunk; exponentials past s1 are 0
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
-            const float2 f = __half22float2(v2[i]);
-            vf[2 * i] = f.x;
-            vf[2 * i + 1] = f.y;
-        }
-#pragma unroll
-        for (int h = 0; h < OXB_ATTN_MAXG; h++) {
+        for (int h = 0; h < GM; h++) {
             if ((uint32_t)h < G) {
-                const float pr = sc[h * chunk + (t - s0)];
+                const float pr = sc[h * OXB_ATTN_CHUNK + lt];
 #pragma unroll
-                for (int i = 0; i < 8; i++) acc[h][i] = fmaf(pr, vf[i], acc[h][i]);
+                for (int j = 0; j < 8; j++) acc[h][j] = fmaf(pr, vf[j], acc[h][j]);
             }
         }
     }
 #pragma unroll
-    for (int h = 0; h < OXB_ATTN_MAXG; h++)
+    for (int h = 0; h < GM; h++)
         if ((uint32_t)h < G) {
-#pragma unroll
-            for (int i = 0; i < 8; i++) accs[(slice * G + h) * hd + grp * 8 + i] = acc[h][i];
+            *reinterpret_cast<float4*>(&accs[(slice * GM + h) * HD + grp * 8]) = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
+            *reinterpret_cast<float4*>(&accs[(slice * GM + h) * HD + grp * 8 + 4]) = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
         }
     __syncthreads();
-    for (uint32_t i = tid; i < G * hd; i += OXB_ATTN_THREADS) {
+    for (uint32_t i = tid; i < G * HD; i += OXB_ATTN_THREADS) {
+        const uint32_t h = i / HD, d = i % HD;
         float v = 0.f;
-        for (uint32_t s = 0; s < n_slices; s++) v += accs[s * G * hd + i];
-        part[(i / hd) * part_head + (i % hd)] = v;
+#pragma unroll
+        for (int s = 0; s < NSL; s++) v += accs[(s * GM + h) * HD + d];
+        part[h * part_head + d] = v;
     }
     if (tid < G) {
-        part[tid * part_head + hd] = m[tid];
-        part[tid * part_head + hd + 1] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
+        float mm = m[0];
+#pragma unroll
+        for (int h = 1; h < GM; h++) mm = (tid == (uint32_t)h) ? m[h] : mm;
+        part[tid * part_head + HD] = mm;
+        part[tid * part_head + HD + 1] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
     }
 }
 
@@ -348,10 +360,10 @@ hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w,
                                     hipStream_t st) {
     const size_t shm = (size_t)h * sizeof(float);
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_Q1>, dim3(nb), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w, eps,
+        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_Q1>, dim3(nb, oxb_quant_parts(h)), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w, eps,
                            h, 8 * nb, d_xq, d_cneg, d_xexp, d_normed_or_null);
     else
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_TQ2>, dim3(nb), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w,
+        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_TQ2>, dim3(nb, oxb_quant_parts(h)), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w,
                            eps, h, 8 * nb, d_xq, d_cneg, d_xexp, d_normed_or_null);
     return hipGetLastError();
 }
@@ -360,10 +372,10 @@ hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, u
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st) {
     const size_t shm = (size_t)inter * sizeof(float);
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, dim3(nb), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
+        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, dim3(nb, oxb_quant_parts(inter)), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
                            8 * nb, d_xq, d_cneg, d_xexp);
     else
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_TQ2>, dim3(nb), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
+        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_TQ2>, dim3(nb, oxb_quant_parts(inter)), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
                            8 * nb, d_xq, d_cneg, d_xexp);
     return hipGetLastError();
 }
@@ -373,15 +385,26 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
     return hipGetLastError();
 }
 
-size_t oxb_attn_smem_bytes(uint32_t nq, uint32_t nkv, uint32_t hd, uint32_t chunk) {
-    const uint32_t G = nq / nkv, slices = OXB_ATTN_THREADS / (hd / 8);
-    return ((size_t)G * hd + (size_t)G * chunk + OXB_ATTN_MAXG * 4 + (size_t)slices * G * hd) * sizeof(float);
+template <int HD>
+static hipError_t launch_attn_hd(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
+    const uint32_t G = p.nq / p.nkv;
+    const dim3 block(OXB_ATTN_THREADS);
+    if (G == 1) hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), dim3(p.n_splits, p.nkv, batch), block, 0, st, p);
+    else if (G == 2) hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), dim3(p.n_splits, p.nkv, batch), block, 0, st, p);
+    else hipLaunchKernelGGL((attn_decode_kernel<HD, 4>), dim3(p.n_splits, p.nkv * ((G + 3) / 4), batch), block, 0, st, p);
+    return hipGetLastError();
 }
 
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st) {
-    hipLaunchKernelGGL(attn_decode_kernel, dim3(p.n_splits, p.nkv, batch), dim3(OXB_ATTN_THREADS),
-                       oxb_attn_smem_bytes(p.nq, p.nkv, p.hd, p.chunk), st, p);
-    hipError_t e = hipGetLastError();
+    if (p.chunk != OXB_ATTN_CHUNK) return hipErrorInvalidValue;
+    hipError_t e;
+    switch (p.hd) {
+        case 32: e = launch_attn_hd<32>(p, batch, st); break;
+        case 64: e = launch_attn_hd<64>(p, batch, st); break;
+        case 128: e = launch_attn_hd<128>(p, batch, st); break;
+        case 256: e = launch_attn_hd<256>(p, batch, st); break;
+        default: return hipErrorInvalidValue;
+    }
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(attn_combine_kernel, dim3(p.nq, batch), dim3(p.hd), 0, st, p, d_out);
     return hipGetLastError();

@@ -318,8 +318,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     if (!rc) mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
     if (rc) return rc;
 
-    m.chunk = 256;  // positions per attention workgroup: one per thread in the score phase
-    while (m.chunk > 64 && m.chunk / 2 >= d.max_seq) m.chunk /= 2;
+    m.chunk = OXB_ATTN_CHUNK_POSITIONS;
     m.n_splits = (d.max_seq + m.chunk - 1) / m.chunk;
     const size_t B = d.batch;
     const size_t kv_elems = B * d.n_layers * d.nkv * (size_t)d.max_seq * d.hd;

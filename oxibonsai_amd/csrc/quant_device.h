@@ -108,19 +108,23 @@ __device__ __forceinline__ float block_absmax(float mx, int bad, float* red, int
 }
 
 // Quantise vector n (values at xn[0..k), any address space) given its absolute maximum.
-// All threads of the workgroup call it; blockDim.x must be a multiple of 64.
+// All threads of the workgroup call it; blockDim.x must be a multiple of 64.  Workgroup
+// (part of parts) takes an equal share of the 64-unit groups, so several workgroups can split
+// one vector after each has found the same maximum.
 template <int FMT>
 __device__ __forceinline__ void quantise_vector(const float* __restrict__ xn, uint32_t k, uint32_t nblk_pad,
                                                 uint32_t NC, uint32_t n, float mx, bool any_bad,
                                                 uint32_t* __restrict__ xq, int32_t* __restrict__ cneg,
-                                                int32_t* __restrict__ xexp) {
+                                                int32_t* __restrict__ xexp, uint32_t part = 0, uint32_t parts = 1) {
     int E = 0;
     if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
     const int base_shift = OXB_XQ_P - E;
     const uint32_t nblk = k / OXB_QK;
     const bool ok = mx > 0.0f && !any_bad;
     // unit u = (blk, m, g): eight consecutive lanes cover one block
-    for (uint32_t u = threadIdx.x; u < nblk_pad * 8; u += blockDim.x) {
+    const uint32_t n_units = nblk_pad * 8, per = (((n_units + 63) / 64 + parts - 1) / parts) * 64;  // n_units % 32 == 0
+    const uint32_t u_end = (part + 1) * per < n_units ? (part + 1) * per : n_units;
+    for (uint32_t u = part * per + threadIdx.x; u < u_end; u += blockDim.x) {
         const uint32_t blk = u >> 3, m = (u >> 2) & 1u, g = u & 3u;
         int cs[8];
         quant_unit<FMT>(xn, blk, m, g, base_shift, ok && blk < nblk, NC, n, xq, cs);
@@ -139,7 +143,13 @@ __device__ __forceinline__ void quantise_vector(const float* __restrict__ xn, ui
         for (int d = 1; d < 8; d++) mine = ((u & 7u) == (uint32_t)d) ? cs[d] : mine;
         *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + (u & 7u)) * 4) = make_int4(-mine, -mine, -mine, -mine);
     }
-    if (threadIdx.x == 0) xexp[n] = any_bad ? INT32_MIN : (mx > 0.0f ? E - OXB_XQ_P : 0);
+    if (threadIdx.x == 0 && part == 0) xexp[n] = any_bad ? INT32_MIN : (mx > 0.0f ? E - OXB_XQ_P : 0);
+}
+
+// Workgroups that share one vector: one per 64 units (1024 activations), at most 16.
+__host__ __device__ inline uint32_t oxb_quant_parts(uint32_t k) {
+    const uint32_t p = (((k + 511u) / 512u) * 32u + 63u) / 64u;
+    return p < 1 ? 1 : (p > 16 ? 16 : p);
 }
 
 __host__ __device__ inline uint32_t oxb_nblk_pad(uint32_t k) { return ((k + 511u) / 512u) * 4u; }

@@ -151,3 +151,25 @@ def test_batch_ffn_phase_matches_oracle(backend, fmt):
     want = hid + oracle.gemv(fmt, down, act, h, inter)
     assert parity_violations(got, want) == 0
     assert np.max(np.abs(got - want)) < 1e-4 * np.max(np.abs(want))
+
+
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 1, 32), (6, 2, 64), (5, 1, 128), (2, 2, 64)])
+def test_gqa_group_shapes(backend, nq, nkv, hd):
+    # 8, 3, 5 and 1 query heads per kv head: groups above four are split over several attention workgroups
+    h = nq * hd if (nq * hd) % 128 == 0 else 128 * ((nq * hd + 127) // 128)
+    cfg = dict(n_layers=2, h=256, inter=384, nq=nq, nkv=nkv, hd=hd, vocab=64, max_seq=320, eps=1e-6, rope_theta=1e4, fmt=TQ2)
+    if (nq * hd) % 128:
+        pytest.skip("nq*hd must be a multiple of 128")
+    w = synth.make_model(cfg, 77 + nq)
+    cpu = oracle.OracleModel(cfg, w, kv_f16=True)
+    gpu = HipModel(backend, cfg, w)
+    try:
+        for pos in range(300):
+            hidden = synth.embedding_rows(5, [pos % 50], cfg["h"])[0] * 50.0
+            check = pos < 4 or pos in (255, 256, 257, 299)
+            want = cpu.forward(hidden, pos, want_logits=check)
+            got, _ = gpu.forward(hidden, pos, want_logits=check)
+            if check:
+                assert parity_violations(got[0], want) == 0, pos
+    finally:
+        gpu.close()
