@@ -28,8 +28,6 @@
 #include "layout.h"
 #include "quant_device.h"
 
-typedef int v4i __attribute__((ext_vector_type(4)));
-typedef float v4f __attribute__((ext_vector_type(4)));
 
 // The activation quantiser (quant_device.h) produces the MFMA B operands ("digit planes").
 #define OXB_QUANT_THREADS 256
@@ -69,36 +67,6 @@ __global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float*
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
 }
-
-template <int CTRL>
-__device__ __forceinline__ uint32_t dpp_u32(uint32_t v) {  // DPP move, out-of-range lanes read 0
-    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
-}
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
-}
-#define OXB_DPP_ROW_SHR(n) (0x110 + (n))
-#define OXB_DPP_ROW_NEWBCAST(n) (0x150 + (n))  // lane n of each 16-lane row to the whole row
-
-// Buffer resources: a load whose byte offset lies outside the buffer returns 0 and moves no
-// data, which replaces every "is this tile / superblock / column in range" branch below.
-typedef unsigned v4u __attribute__((ext_vector_type(4)));
-#define OXB_OOB 0xFFFFFFF0u
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);
-}
-// voff is per lane and is what the range check sees; soff is wave-uniform (an SGPR) and is not checked.
-__device__ __forceinline__ v4i buf_load_b128(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
-    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
-    return (v4i){(int)v.x, (int)v.y, (int)v.z, (int)v.w};
-}
-__device__ __forceinline__ uint32_t buf_load_b32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff = 0) {
-    return __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, 0);
-}
-// Workgroup barrier that orders LDS traffic only: global loads already in flight (the
-// prefetched weight tiles) stay in flight across it.
-__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
 // Codes and scales of one row tile, restricted to this wave's K slice, as they wait in registers.
 template <int FMT, int NSBW>

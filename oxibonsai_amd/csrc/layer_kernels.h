@@ -25,9 +25,10 @@ struct OxbAttnParams {
     float scale;                         // 1 / sqrt(hd)
 };
 
-hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t nb,
-                                    uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed_or_null,
-                                    hipStream_t st);
+// w_absmax = max |w[i]|, known when the norm weights are uploaded.
+hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
+                                    uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp,
+                                    float* d_normed_or_null, hipStream_t st);
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);

@@ -30,68 +30,82 @@ __device__ __forceinline__ float block_sum(float v, float* red) {  // two barrie
 // RMSNorm fused with the activation quantiser (rms_norm: crates/oxibonsai-kernels/src/
 // simd_float_ops.rs:204-215; GPU twin rmsnorm_weighted_v2, gpu_backend/cuda_kernels.rs:335-374).
 // out[i] = w[i] * x[i] * (1 / sqrt(mean(x^2) + eps)); the normalised vector lives only in LDS.
-// Grid (vectors of the pass, parts): every part repeats the two reductions (the vector is a few KB in L2) and
-// quantises its share of the blocks.
+// Grid (vectors of the pass, parts): every part repeats the reduction (the vector is a few KB in
+// L2) and quantises its share of the blocks.  x and w are fetched together, EPT elements per thread.
+// The quantiser's exponent does not need the exact maximum, only a bound: |out[i]| <= max|w| * sqrt(h)
+// because |x[i]| / rms <= sqrt(h).  With 54-bit fixed point the slack of sqrt(h) costs no mantissa bit
+// of any element within 2^22 / sqrt(h) of the largest one.
 // ---------------------------------------------------------------------------
-template <int FMT>
+template <int FMT, int EPT>
 __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const float* __restrict__ x,
                                                                            const float* __restrict__ w, float eps,
-                                                                           uint32_t h, uint32_t NC,
+                                                                           float w_absmax, uint32_t h, uint32_t NC,
                                                                            uint32_t* __restrict__ xq,
                                                                            int32_t* __restrict__ cneg,
                                                                            int32_t* __restrict__ xexp,
                                                                            float* __restrict__ normed_out) {
     extern __shared__ float lds_x[];  // [h]
     __shared__ float red[OXB_LAYER_THREADS / 64];
-    __shared__ int bad_flag;
     const uint32_t n = blockIdx.x, tid = threadIdx.x;
     const float* xn = x + (size_t)n * h;
-    float ss = 0.f;
-    for (uint32_t i = tid; i < h; i += OXB_LAYER_THREADS) {
-        const float v = xn[i];
-        lds_x[i] = v;
-        ss += v * v;
+    float xv[EPT], wv[EPT];
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+        const uint32_t i = tid + (uint32_t)e * OXB_LAYER_THREADS;
+        xv[e] = i < h ? xn[i] : 0.f;
+        wv[e] = i < h ? w[i] : 0.f;
     }
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; e++) ss = fmaf(xv[e], xv[e], ss);
     ss = block_sum(ss, red);
     const float inv_rms = 1.0f / sqrtf(ss / (float)h + eps);
-    float mx = 0.f;
-    int bad = 0;
-    for (uint32_t i = tid; i < h; i += OXB_LAYER_THREADS) {
-        const float v = w[i] * lds_x[i] * inv_rms;
-        lds_x[i] = v;
-        if (normed_out && blockIdx.y == 0) normed_out[(size_t)n * h + i] = v;
-        bad |= oxb_not_finite(v);
-        mx = fmaxf(mx, fabsf(v));
+#pragma unroll
+    for (int e = 0; e < EPT; e++) {
+        const uint32_t i = tid + (uint32_t)e * OXB_LAYER_THREADS;
+        const float v = wv[e] * xv[e] * inv_rms;
+        if (i < h) {
+            lds_x[i] = v;
+            if (normed_out && blockIdx.y == 0) normed_out[(size_t)n * h + i] = v;
+        }
     }
-    bool any_bad;
-    mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);  // its barriers also publish lds_x
-    quantise_vector<FMT>(lds_x, h, oxb_nblk_pad(h), NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
+    __syncthreads();
+    // a NaN or infinity anywhere in x or w shows up in the sum of squares or in the bound
+    const float bound = w_absmax * sqrtf((float)h);
+    const bool any_bad = oxb_not_finite(ss) || oxb_not_finite(bound);
+    quantise_vector<FMT>(lds_x, h, oxb_nblk_pad(h), NC, n, ss > 0.f ? bound : 0.f, any_bad, xq, cneg, xexp, blockIdx.y,
+                         gridDim.y);
 }
 
 // ---------------------------------------------------------------------------
 // SwiGLU fused with the quantiser: act[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
 // (crates/oxibonsai-kernels/src/simd_float_ops.rs:217-236; GPU twin swiglu_fused, cuda_kernels.rs:394-401).
-// gu = [gate: inter | up: inter] per vector.
+// gu = [gate: inter | up: inter] per vector.  Grid (vectors, parts), 1024 threads.
 // ---------------------------------------------------------------------------
+#define OXB_SWIGLU_THREADS 1024
 template <int FMT>
-__global__ __launch_bounds__(OXB_LAYER_THREADS) void swiglu_quant_kernel(const float* __restrict__ gu, uint32_t inter,
-                                                                          uint32_t NC, uint32_t* __restrict__ xq,
-                                                                          int32_t* __restrict__ cneg,
-                                                                          int32_t* __restrict__ xexp) {
+__global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const float* __restrict__ gu, uint32_t inter,
+                                                                           uint32_t NC, uint32_t* __restrict__ xq,
+                                                                           int32_t* __restrict__ cneg,
+                                                                           int32_t* __restrict__ xexp) {
     extern __shared__ float lds_x[];  // [inter]
-    __shared__ float red[OXB_LAYER_THREADS / 64];
+    __shared__ float red[OXB_SWIGLU_THREADS / 64];
     __shared__ int bad_flag;
     const uint32_t n = blockIdx.x, tid = threadIdx.x;
     const float* g = gu + (size_t)n * 2 * inter;
     const float* u = g + inter;
     float mx = 0.f;
     int bad = 0;
-    for (uint32_t i = tid; i < inter; i += OXB_LAYER_THREADS) {
-        const float gv = g[i];
-        const float v = (gv / (1.0f + expf(-gv))) * u[i];
-        lds_x[i] = v;
-        bad |= oxb_not_finite(v);
-        mx = fmaxf(mx, fabsf(v));
+    for (uint32_t i = tid * 4; i < inter; i += OXB_SWIGLU_THREADS * 4) {  // inter % 128 == 0
+        const float4 g4 = *reinterpret_cast<const float4*>(g + i), u4 = *reinterpret_cast<const float4*>(u + i);
+        float4 a;
+        a.x = (g4.x / (1.0f + expf(-g4.x))) * u4.x;
+        a.y = (g4.y / (1.0f + expf(-g4.y))) * u4.y;
+        a.z = (g4.z / (1.0f + expf(-g4.z))) * u4.z;
+        a.w = (g4.w / (1.0f + expf(-g4.w))) * u4.w;
+        *reinterpret_cast<float4*>(lds_x + i) = a;
+        bad |= oxb_not_finite(a.x) | oxb_not_finite(a.y) | oxb_not_finite(a.z) | oxb_not_finite(a.w);
+        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
     }
     bool any_bad;
     mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);
@@ -153,7 +167,7 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
 #define OXB_ATTN_THREADS 256
 #define OXB_ATTN_CHUNK 256  // positions per workgroup = threads: one position per thread in the score phase
 
-__device__ __forceinline__ void unpack8(const uint4& u, float f[8]) {
+__device__ __forceinline__ void unpack8(const v4i& u, float f[8]) {
     const __half2* h2 = reinterpret_cast<const __half2*>(&u);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
@@ -170,7 +184,6 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     constexpr int NG = HD / 8;                       // 16-byte groups per row
     constexpr int NSL = OXB_ATTN_THREADS / NG;       // position slices in the weighted-sum phase
     constexpr int PPS = OXB_ATTN_CHUNK / NSL;        // positions per slice
-    __shared__ float q_s[GM * HD];
     __shared__ float sc[GM * OXB_ATTN_CHUNK];
     __shared__ float red[GM * 4];
     __shared__ float accs[NSL * GM * HD];
@@ -198,65 +211,86 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     const uint32_t t = s0 + tid;
     const bool live = t < s1;
 
-    // this thread's K row, all of it in flight at once
-    uint4 kreg[NG];
+    // scores: lanes walk the K rows 16 bytes at a time, so one wave load covers whole rows back to
+    // back (fully coalesced); every pass handles RPP rows of the chunk, all passes are in flight at once
+    constexpr int RPP = OXB_ATTN_THREADS / NG, NPASS = OXB_ATTN_CHUNK / RPP;
+    const uint32_t ch = tid % NG, rr = tid / NG;
+    float qf[GM][8];  // this lane's 8 dimensions of every q head
 #pragma unroll
-    for (int i = 0; i < NG; i++)
-        kreg[i] = live ? reinterpret_cast<const uint4*>(K + (size_t)t * HD)[i] : make_uint4(0, 0, 0, 0);
-    for (uint32_t i = tid; i < G * HD; i += OXB_ATTN_THREADS) q_s[i] = p.q[((size_t)b * p.nq + h0) * HD + i];
-    __syncthreads();
-
-    // scores
-    float dot[GM];
+    for (int h = 0; h < GM; h++) {
+        if ((uint32_t)h < G) {
+            const float* qp = p.q + ((size_t)b * p.nq + h0 + h) * HD + ch * 8;
+            const float4 qa = *reinterpret_cast<const float4*>(qp), qb = *reinterpret_cast<const float4*>(qp + 4);
+            qf[h][0] = qa.x; qf[h][1] = qa.y; qf[h][2] = qa.z; qf[h][3] = qa.w;
+            qf[h][4] = qb.x; qf[h][5] = qb.y; qf[h][6] = qb.z; qf[h][7] = qb.w;
+        } else {
 #pragma unroll
-    for (int h = 0; h < GM; h++) dot[h] = 0.f;
-#pragma unroll
-    for (int i = 0; i < NG; i++) {
-        float kf[8];
-        unpack8(kreg[i], kf);
-#pragma unroll
-        for (int h = 0; h < GM; h++) {
-            if ((uint32_t)h < G) {
-                const float4 qa = *reinterpret_cast<const float4*>(&q_s[h * HD + i * 8]);
-                const float4 qb = *reinterpret_cast<const float4*>(&q_s[h * HD + i * 8 + 4]);
-                dot[h] = fmaf(qa.x, kf[0], dot[h]);
-                dot[h] = fmaf(qa.y, kf[1], dot[h]);
-                dot[h] = fmaf(qa.z, kf[2], dot[h]);
-                dot[h] = fmaf(qa.w, kf[3], dot[h]);
-                dot[h] = fmaf(qb.x, kf[4], dot[h]);
-                dot[h] = fmaf(qb.y, kf[5], dot[h]);
-                dot[h] = fmaf(qb.z, kf[6], dot[h]);
-                dot[h] = fmaf(qb.w, kf[7], dot[h]);
-            }
+            for (int j = 0; j < 8; j++) qf[h][j] = 0.f;
         }
     }
-    // start the V loads of the weighted-sum phase now; they land while the softmax statistics are made
+    // K rows of the score phase and V rows of the weighted-sum phase, all requested now: both depend
+    // only on pos.  Buffer loads return 0 past s1 without a branch or a select after the load.
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(K, p.max_seq * HD * 2u), rv = make_rsrc(V, p.max_seq * HD * 2u);
+    v4i kreg[NPASS];
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+        const uint32_t tk = s0 + (uint32_t)i * RPP + rr;
+        kreg[i] = buf_load_b128(rk, tk < s1 ? (tk * HD + ch * 8u) * 2u : OXB_OOB);
+    }
     const uint32_t grp = tid % NG, slice = tid / NG;
-    uint4 vreg[PPS];
+    v4i vreg[PPS];
 #pragma unroll
     for (int i = 0; i < PPS; i++) {
         const uint32_t tv = s0 + slice + (uint32_t)i * NSL;
-        vreg[i] = tv < s1 ? *reinterpret_cast<const uint4*>(V + (size_t)tv * HD + grp * 8) : make_uint4(0, 0, 0, 0);
+        vreg[i] = buf_load_b128(rv, tv < s1 ? (tv * HD + grp * 8u) * 2u : OXB_OOB);
+    }
+    float lmax[GM];
+#pragma unroll
+    for (int h = 0; h < GM; h++) lmax[h] = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < NPASS; i++) {
+        float kf[8];
+        unpack8(kreg[i], kf);
+        const uint32_t lt = (uint32_t)i * RPP + rr;  // position within the chunk
+#pragma unroll
+        for (int h = 0; h < GM; h++) {
+            float d = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; j++) d = fmaf(qf[h][j], kf[j], d);
+            // add the NG partial sums of the row: they sit in consecutive lanes
+            d += dpp_f32<0x111>(d);                    // row_shr:1
+            if (NG > 2) d += dpp_f32<0x112>(d);        // row_shr:2
+            if (NG > 4) d += dpp_f32<0x114>(d);        // row_shr:4
+            if (NG > 8) d += dpp_f32<0x118>(d);        // row_shr:8
+            if (NG > 16) d += __shfl_up(d, 16, 64);    // head_dim 256: two 16-lane rows per K row
+            if (ch == NG - 1 && (uint32_t)h < G) {
+                const float sv = (s0 + lt < s1) ? d * p.scale : -INFINITY;
+                sc[h * OXB_ATTN_CHUNK + lt] = sv;
+                lmax[h] = fmaxf(lmax[h], sv);
+            }
+        }
     }
     // chunk maximum per head
     float m[GM];
 #pragma unroll
     for (int h = 0; h < GM; h++) {
-        float s = live ? dot[h] * p.scale : -INFINITY;
-        dot[h] = s;
+        float sv = lmax[h];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) s = fmaxf(s, __shfl_xor(s, o, 64));
-        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = s;
+        for (int o = 32; o > 0; o >>= 1) sv = fmaxf(sv, __shfl_xor(sv, o, 64));
+        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = sv;
     }
-    __syncthreads();
+    __syncthreads();  // also publishes the scores
 #pragma unroll
     for (int h = 0; h < GM; h++) m[h] = fmaxf(fmaxf(red[h * 4], red[h * 4 + 1]), fmaxf(red[h * 4 + 2], red[h * 4 + 3]));
     __syncthreads();
-    // exponentials and their sum
+    // exponentials and their sum: one position per thread
 #pragma unroll
     for (int h = 0; h < GM; h++) {
-        float e = ((uint32_t)h < G && live) ? expf(dot[h] - m[h]) : 0.f;
-        if ((uint32_t)h < G) sc[h * OXB_ATTN_CHUNK + tid] = e;
+        float e = 0.f;
+        if ((uint32_t)h < G) {
+            e = live ? expf(sc[h * OXB_ATTN_CHUNK + tid] - m[h]) : 0.f;
+            sc[h * OXB_ATTN_CHUNK + tid] = e;
+        }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, 64);
         if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = e;
@@ -355,28 +389,40 @@ __global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ 
 // ---------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------
-hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t nb,
-                                    uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed_or_null,
-                                    hipStream_t st) {
+template <int FMT>
+static hipError_t launch_rmsnorm_fmt(const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
+                                     uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed,
+                                     hipStream_t st) {
     const size_t shm = (size_t)h * sizeof(float);
-    if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_Q1>, dim3(nb, oxb_quant_parts(h)), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w, eps,
-                           h, 8 * nb, d_xq, d_cneg, d_xexp, d_normed_or_null);
-    else
-        hipLaunchKernelGGL(rmsnorm_quant_kernel<OXB_FMT_TQ2>, dim3(nb, oxb_quant_parts(h)), dim3(OXB_LAYER_THREADS), shm, st, d_x, d_w,
-                           eps, h, 8 * nb, d_xq, d_cneg, d_xexp, d_normed_or_null);
-    return hipGetLastError();
+    const dim3 grid(nb, oxb_quant_parts(h)), block(OXB_LAYER_THREADS);
+    const uint32_t ept = (h + OXB_LAYER_THREADS - 1) / OXB_LAYER_THREADS;
+#define OXB_RMS_CASE(E)                                                                                              \
+    if (ept <= E) {                                                                                                  \
+        hipLaunchKernelGGL((rmsnorm_quant_kernel<FMT, E>), grid, block, shm, st, d_x, d_w, eps, w_absmax, h, 8 * nb, \
+                           d_xq, d_cneg, d_xexp, d_normed);                                                          \
+        return hipGetLastError();                                                                                    \
+    }
+    OXB_RMS_CASE(4) OXB_RMS_CASE(8) OXB_RMS_CASE(16) OXB_RMS_CASE(32) OXB_RMS_CASE(64)
+#undef OXB_RMS_CASE
+    return hipErrorInvalidValue;  // h > 16384
+}
+
+hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
+                                    uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp,
+                                    float* d_normed_or_null, hipStream_t st) {
+    return fmt == OXB_FMT_Q1
+               ? launch_rmsnorm_fmt<OXB_FMT_Q1>(d_x, d_w, eps, w_absmax, h, nb, d_xq, d_cneg, d_xexp, d_normed_or_null, st)
+               : launch_rmsnorm_fmt<OXB_FMT_TQ2>(d_x, d_w, eps, w_absmax, h, nb, d_xq, d_cneg, d_xexp, d_normed_or_null, st);
 }
 
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st) {
     const size_t shm = (size_t)inter * sizeof(float);
+    const dim3 grid(nb, oxb_quant_parts(inter)), block(OXB_SWIGLU_THREADS);
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, dim3(nb, oxb_quant_parts(inter)), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
-                           8 * nb, d_xq, d_cneg, d_xexp);
+        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, grid, block, shm, st, d_gu, inter, 8 * nb, d_xq, d_cneg, d_xexp);
     else
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_TQ2>, dim3(nb, oxb_quant_parts(inter)), dim3(OXB_LAYER_THREADS), shm, st, d_gu, inter,
-                           8 * nb, d_xq, d_cneg, d_xexp);
+        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_TQ2>, grid, block, shm, st, d_gu, inter, 8 * nb, d_xq, d_cneg, d_xexp);
     return hipGetLastError();
 }
 

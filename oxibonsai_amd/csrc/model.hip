@@ -87,6 +87,11 @@ static const float* vec_ptr(uint64_t id, uint32_t n, const char* what, int* rc) 
     return it->second.d;
 }
 
+static float vec_absmax(uint64_t id) {
+    auto it = g_rt.vectors.find(id);
+    return it == g_rt.vectors.end() ? 0.f : it->second.absmax;
+}
+
 static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, const char* what, int* rc) {
     const Weight* w = find_weight(id);
     if (!w) {
@@ -144,13 +149,14 @@ static int gemv_xq(const Weight& w, const XqBuf& xb, uint32_t nb, float* d_y, ui
     } while (0)
 
 // The FFN half of a layer on vectors [b0, b0+nb): O-proj + residual, RMSNorm, gate||up, SwiGLU, down + residual.
-static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn_out, const float* ffn_norm, float eps,
+static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn_out, const float* ffn_norm,
+                      float ffn_norm_absmax, float eps,
                       const Weight& o, const Weight& gate_up, const Weight& down, float* gu, uint32_t h,
                       uint32_t inter, uint32_t attn_k, uint32_t nb) {
     hipStream_t st = g_rt.stream;
     OXB_TRY_HIP(oxb_launch_quant_x(fmt, attn_out, attn_k, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: quant_x");
     OXB_TRY(gemv_xq(o, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
-    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(fmt, hidden, ffn_norm, eps, h, nb, xb.xq, xb.cneg, xb.xexp, nullptr, st),
+    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(fmt, hidden, ffn_norm, eps, ffn_norm_absmax, h, nb, xb.xq, xb.cneg, xb.xexp, nullptr, st),
                 "kernel launch failed: rmsnorm_quant");
     OXB_TRY(gemv_xq(gate_up, xb, nb, gu, 2 * inter, OXB_GEMV_STORE, nullptr));
     OXB_TRY_HIP(oxb_launch_swiglu_quant(fmt, gu, inter, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: swiglu_quant");
@@ -178,7 +184,7 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         // attention input: RMSNorm -> QKV, two sequences per pass over the weights
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, attn_norm, d.eps, d.h, nb, m.xq.xq,
+            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, attn_norm, d.eps, vec_absmax(ly.attn_norm), d.h, nb, m.xq.xq,
                                                  m.xq.cneg, m.xq.xexp, nullptr, st),
                         "kernel launch failed: rmsnorm_quant");
             OXB_TRY(gemv_xq(*wqkv, m.xq, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows, OXB_GEMV_STORE, nullptr));
@@ -220,7 +226,8 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, m.attn_out, st), "kernel launch failed: attention");
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo,
+            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm,
+                               vec_absmax(ly.ffn_norm), d.eps, *wo,
                                *wgu, *wdn, m.gu + (size_t)b0 * 2 * d.inter, d.h, d.inter, qd, nb));
         }
     }
@@ -230,7 +237,7 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         if (rc) return rc;
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, final_norm, d.eps, d.h, nb, m.xq.xq,
+            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, final_norm, d.eps, vec_absmax(d.final_norm), d.h, nb, m.xq.xq,
                                                  m.xq.cneg, m.xq.xexp, nullptr, st),
                         "kernel launch failed: rmsnorm_quant");
             OXB_TRY(gemv_xq(*lm, m.xq, nb, m.logits + (size_t)b0 * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
@@ -257,6 +264,10 @@ int oxb_hip_upload_f32(uint64_t* id, const float* w, size_t n) {
     OXB_TRY(ensure_init());
     Vector v;
     v.n = n;
+    for (size_t i = 0; i < n; i++) {
+        const float a = fabsf(w[i]);
+        if (a > v.absmax || a != a) v.absmax = a;  // a NaN sticks
+    }
     if (hipMalloc((void**)&v.d, n * sizeof(float)) != hipSuccess)
         return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", n * sizeof(float), g_rt.device);
     hipError_t e = hipMemcpy(v.d, w, n * sizeof(float), hipMemcpyHostToDevice);
@@ -465,7 +476,11 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     OXB_TRY_HIP(hipMemcpyAsync(d_hidden, hidden, (size_t)h * 4, hipMemcpyHostToDevice, st), "hidden upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_norm, norm_w, (size_t)h * 4, hipMemcpyHostToDevice, st), "norm upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_attn, attn_out, (size_t)attn_k * 4, hipMemcpyHostToDevice, st), "attn_out upload");
-    OXB_TRY(encode_ffn(fmt, xb, d_hidden, d_attn, d_norm, eps, *wo, *wgu, *wdn, (float*)g_rt.ws_y.ptr, h, inter, attn_k, 1));
+    float nw_absmax = 0.f;
+    for (uint32_t i = 0; i < h; i++) nw_absmax = fmaxf(nw_absmax, fabsf(norm_w[i]));  // NaN-free maximum; a NaN weight yields NaN outputs
+    for (uint32_t i = 0; i < h; i++)
+        if (norm_w[i] != norm_w[i]) nw_absmax = norm_w[i];
+    OXB_TRY(encode_ffn(fmt, xb, d_hidden, d_attn, d_norm, nw_absmax, eps, *wo, *wgu, *wdn, (float*)g_rt.ws_y.ptr, h, inter, attn_k, 1));
     OXB_TRY_HIP(hipMemcpyAsync(hidden, d_hidden, (size_t)h * 4, hipMemcpyDeviceToHost, st), "hidden download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));

@@ -17,6 +17,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "device_utils.h"
 #include "layout.h"
 
 #define OXB_XQ_P 53  // |x * 2^(P-E)| < 2^53, doubled values stay below 2^54
@@ -33,13 +34,34 @@ __device__ __forceinline__ long long scaled_rint_i64(float v, int shift) {
     return ((long long)(int)hi << 27) + (long long)(int)lo;
 }
 
-template <int CTRL>
-__device__ __forceinline__ int dpp_i32(int v) {
-    return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+// Transpose a 4 x 4 byte matrix held in four dwords: o[d] = { t[0].byte d, t[1].byte d, t[2].byte d, t[3].byte d }.
+__device__ __forceinline__ void transpose_bytes4(const uint32_t t[4], uint32_t o[4]) {
+    const uint32_t p01l = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u), p01h = __builtin_amdgcn_perm(t[1], t[0], 0x07030602u);
+    const uint32_t p23l = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u), p23h = __builtin_amdgcn_perm(t[3], t[2], 0x07030602u);
+    o[0] = __builtin_amdgcn_perm(p23l, p01l, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(p23l, p01l, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(p23h, p01h, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(p23h, p01h, 0x07060302u);
+}
+
+// Balanced base-256 digits of four 64-bit integers, digit-major: dig[d] = one dword holding digit d of
+// v[0..3] as int8.  Adding 0x80 to every byte below the top one and flipping that bit back turns
+// the two's-complement bytes into signed digits in [-128, 127] with the carries propagated.
+__device__ __forceinline__ void digits_of4(const long long v[4], uint32_t dig[8]) {
+    const unsigned long long bias = 0x0080808080808080ull;
+    uint32_t lo[4], hi[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const unsigned long long t = ((unsigned long long)v[i] + bias) ^ bias;
+        lo[i] = (uint32_t)t;
+        hi[i] = (uint32_t)(t >> 32);
+    }
+    transpose_bytes4(lo, dig);
+    transpose_bytes4(hi, dig + 4);
 }
 
 // Quantise the 16 activations that one lane group (blk, m, g) of the MFMA B operand holds and
-// store their eight digit planes; returns nothing, accumulates the block's correction sums.
+// store their eight digit planes; cs[d] returns this group's share of the block's correction sums.
 template <int FMT>
 __device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_t blk, uint32_t m, uint32_t g,
                                            int base_shift, bool live, uint32_t NC, uint32_t n,
@@ -52,43 +74,48 @@ __device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_
     }
     if (live) {
         const float* xb = xn + blk * 128 + 32 * g;
+        float vv[4][4];  // [bb][jj]
 #pragma unroll
         for (uint32_t bb = 0; bb < 4; bb++) {
             // Q1: k = 8bb + 4m + jj;  TQ2: k = 16m + 4bb + jj   (jj = 0..3 contiguous)
             const float4 v4 = *reinterpret_cast<const float4*>(xb + (FMT == OXB_FMT_Q1 ? 8 * bb + 4 * m : 16 * m + 4 * bb));
-            const float vv[4] = {v4.x, v4.y, v4.z, v4.w};
+            vv[bb][0] = v4.x;
+            vv[bb][1] = v4.y;
+            vv[bb][2] = v4.z;
+            vv[bb][3] = v4.w;
+        }
 #pragma unroll
-            for (uint32_t jj = 0; jj < 4; jj++) {
-                long long xi, cr;
-                int cmul;
-                if (FMT == OXB_FMT_Q1) {
-                    const uint32_t j = 4 * m + jj;
-                    const long long r = scaled_rint_i64(vv[jj], base_shift - (int)j);
-                    xi = (j == 7) ? -2 * r : 2 * r;
-                    cr = r;
-                    cmul = 1 << j;
-                } else {
-                    xi = scaled_rint_i64(vv[jj], base_shift - 2 * (int)jj);
-                    cr = xi;
-                    cmul = (jj < 3) ? (1 << (2 * jj)) : 0;
+        for (uint32_t jj = 0; jj < 4; jj++) {
+            long long xi[4], cr[4];
+            uint32_t dig[8], cdig[8];
+            if (FMT == OXB_FMT_Q1) {
+                const uint32_t j = 4 * m + jj;
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) {
+                    cr[bb] = scaled_rint_i64(vv[bb][jj], base_shift - (int)j);
+                    xi[bb] = (j == 7) ? -2 * cr[bb] : 2 * cr[bb];
                 }
-                // balanced base-256 digits: byte d of t is the signed digit d
-                const unsigned long long bias = 0x0080808080808080ull;
-                const unsigned long long t = ((unsigned long long)xi + bias) ^ bias;
-                const unsigned long long tc = ((unsigned long long)cr + bias) ^ bias;
+                digits_of4(xi, dig);
+                digits_of4(cr, cdig);
 #pragma unroll
-                for (int d = 0; d < 8; d++) {
-                    out[d][jj] |= (uint32_t)((t >> (8 * d)) & 0xFFu) << (8 * bb);
-                    cs[d] += (int)(int8_t)(tc >> (8 * d)) * cmul;
+                for (int d = 0; d < 8; d++) cs[d] += __builtin_amdgcn_sdot4((int)cdig[d], 0x01010101, 0, false) << j;
+            } else {
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) xi[bb] = scaled_rint_i64(vv[bb][jj], base_shift - 2 * (int)jj);
+                digits_of4(xi, dig);
+                if (jj < 3) {
+#pragma unroll
+                    for (int d = 0; d < 8; d++) cs[d] += __builtin_amdgcn_sdot4((int)dig[d], 0x01010101, 0, false) << (2 * jj);
                 }
             }
+#pragma unroll
+            for (int d = 0; d < 8; d++) out[d][jj] = dig[d];
         }
     }
     uint4* dst = reinterpret_cast<uint4*>(xq) + (size_t)((blk * 2 + m) * 4 + g) * NC + 8 * n;
 #pragma unroll
     for (int d = 0; d < 8; d++) dst[d] = make_uint4(out[d][0], out[d][1], out[d][2], out[d][3]);
 }
-
 
 // Workgroup-wide maximum of |x| and a "not finite" flag; `red` holds blockDim.x / 64 floats.
 // Every thread gets the results.  Contains two barriers.

@@ -27,6 +27,7 @@ struct Weight {  // one resident matrix: [codes section][scales section]
 struct Vector {  // a resident fp32 vector (norm weights)
     float* d = nullptr;
     size_t n = 0;
+    float absmax = 0.f;  // max |value|, the RMSNorm kernel's bound for its output range
 };
 
 struct Runtime {
