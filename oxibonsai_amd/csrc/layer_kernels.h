@@ -32,6 +32,6 @@ hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w,
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);
-#define OXB_ATTN_CHUNK_POSITIONS 256  // KV positions one attention workgroup covers
+#define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
 hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, hipStream_t st);

@@ -165,7 +165,7 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
 // output, the chunk maximum and the chunk sum; attn_combine_kernel merges the chunks.
 // ---------------------------------------------------------------------------
 #define OXB_ATTN_THREADS 256
-#define OXB_ATTN_CHUNK 256  // positions per workgroup = threads: one position per thread in the score phase
+#define OXB_ATTN_CHUNK 128  // KV positions per workgroup
 
 __device__ __forceinline__ void unpack8(const v4i& u, float f[8]) {
     const __half2* h2 = reinterpret_cast<const __half2*>(&u);
@@ -209,7 +209,7 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     const __half* K = p.k_cache + base;
     const __half* V = p.v_cache + base;
     const uint32_t t = s0 + tid;
-    const bool live = t < s1;
+    const bool live = tid < OXB_ATTN_CHUNK && t < s1;  // the threads that own one position in the softmax phase
 
     // scores: lanes walk the K rows 16 bytes at a time, so one wave load covers whole rows back to
     // back (fully coalesced); every pass handles RPP rows of the chunk, all passes are in flight at once
@@ -288,8 +288,10 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     for (int h = 0; h < GM; h++) {
         float e = 0.f;
         if ((uint32_t)h < G) {
-            e = live ? expf(sc[h * OXB_ATTN_CHUNK + tid] - m[h]) : 0.f;
-            sc[h * OXB_ATTN_CHUNK + tid] = e;
+            if (tid < OXB_ATTN_CHUNK) {
+                e = live ? expf(sc[h * OXB_ATTN_CHUNK + tid] - m[h]) : 0.f;
+                sc[h * OXB_ATTN_CHUNK + tid] = e;
+            }
         }
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, 64);
