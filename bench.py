@@ -29,6 +29,9 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+# HBM bytes one gate||up GEMV launch moves: rocprofv3 FETCH_SIZE (x 2.000, calibrated on a 256 MiB copy) + WRITE_SIZE
+# (x 1.000), see profiles/gemv_q1_qwen3_8b_set_hbm_traffic.txt.  The algorithmic figure is 14 270 464.
+GATE_UP_HBM_TRAFFIC_BYTES = 14_617_600
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
 
@@ -66,6 +69,73 @@ def cpu_baseline(blocks: dict, xs: dict, budget_s: float = 12.0) -> dict:
             "sample": f"{reps} passes over the same 3-GEMV set (median), {sum(times):.1f} s of CPU time"}
 
 
+DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd=128, vocab=151936,
+                  max_seq=32768, eps=1e-6, rope_theta=1e6)   # BASELINE.json configs[4]: Qwen3-8B shape, Q1_0_g128
+
+
+def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool) -> dict:
+    """Greedy batch-1 decode of the random-init 8B-shape Q1 model: fill the context with `prompt_len`
+    sequential decode steps (what the reference does for short prompts, model/types/mod.rs:315-321), then time
+    `n_tokens` greedy steps.  The time is what the caller of the fused entry point sees per token:
+    embedding row H2D, the replayed HIP graph (36 layers, final norm, LM head, argmax), token id D2H."""
+    from oxibonsai_amd import synth
+    from oxibonsai_amd.model import HipModel
+    cfg = DECODE_CFG
+    w = synth.make_model(cfg, 0xB0A5A104)
+    m = HipModel(be, cfg, w, batch=1)
+    weight_bytes = sum(len(lw[k]) for lw in w["layers"] for k in ("q", "k", "v", "o", "gate", "up", "down")) + len(w["lm_head"])
+    ids = (synth.splitmix64(0xB0A5A1040F, prompt_len) % np.uint64(cfg["vocab"])).astype(np.int64)
+    table = {}
+
+    def emb(t):
+        if t not in table:
+            table[t] = synth.embedding_rows(0xE3B, [t], cfg["h"])[0] * 50.0
+        return table[t]
+
+    tok = 0
+    for pos in range(prompt_len):
+        _, out = m.forward(emb(int(ids[pos])), pos, want_logits=False)
+        tok = int(out[0])
+    tokens, spent = [], 0.0
+    for i in range(n_tokens):
+        hidden = emb(tok)
+        t0 = time.perf_counter()
+        _, out = m.forward(hidden, prompt_len + i, want_logits=False)
+        spent += time.perf_counter() - t0
+        tok = int(out[0])
+        tokens.append(tok)
+    res = {"model": "random-init Qwen3-8B shape, Q1_0_g128 (36 layers, h 4096, 32/8 heads, inter 12288, vocab 151936)",
+           "batch": 1, "context_before": prompt_len, "tokens": n_tokens, "tok_per_s": round(n_tokens / spent, 2),
+           "ms_per_token": round(spent / n_tokens * 1e3, 4), "hip_graph": m.uses_graph(),
+           "weight_bytes_per_token": weight_bytes,
+           "kv_bytes_per_token_at_end": 2 * cfg["n_layers"] * cfg["nkv"] * cfg["hd"] * 2 * (prompt_len + n_tokens),
+           "weight_stream_GBps": round(weight_bytes / (spent / n_tokens) / 1e9, 1),
+           "distinct_tokens": len(set(tokens))}
+    m.close()
+    if with_cpu:
+        # CPU SIMD tier on the same matrices: linear layers only (one layer x 36 + LM head), an upper bound on its tok/s
+        from oracle import oracle
+        lw = w["layers"][0]
+        x_h, x_q, x_i = synth.normal_f32(1, cfg["h"]), synth.normal_f32(2, cfg["nq"] * cfg["hd"]), synth.normal_f32(3, cfg["inter"])
+        mats = [(np.concatenate([lw["q"], lw["k"], lw["v"]]), x_h, 6144, 4096), (lw["o"], x_q, 4096, 4096),
+                (np.concatenate([lw["gate"], lw["up"]]), x_h, 24576, 4096), (lw["down"], x_i, 4096, 12288)]
+        def layer():
+            for b, x, n, k in mats:
+                oracle.simd_gemv(FMT_Q1, b, x, n, k)
+        layer()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            layer()
+        t_layer = (time.perf_counter() - t0) / 5
+        oracle.simd_gemv(FMT_Q1, w["lm_head"], x_h, cfg["vocab"], cfg["h"])
+        t0 = time.perf_counter()
+        oracle.simd_gemv(FMT_Q1, w["lm_head"], x_h, cfg["vocab"], cfg["h"])
+        t_lm = time.perf_counter() - t0
+        res["cpu_linear_layers_only_tok_per_s"] = round(1.0 / (36 * t_layer + t_lm), 2)
+        res["cpu_cores"] = oracle.simd_threads()
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -73,6 +143,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--copies", type=int, default=24, help="distinct resident copies of the weight set")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-decode", action="store_true", help="skip the 8B-shape decode leg")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run a plain 256 MiB device copy, the known-size kernel that hardware-counter runs are scaled by")
+    ap.add_argument("--decode-context", type=int, default=2048)
+    ap.add_argument("--decode-tokens", type=int, default=128)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (multi-GPU sharding is design-only)",
@@ -184,17 +259,26 @@ def main() -> int:
                    "resident_weight_bytes": resident, "pct_of_hbm_peak": round(100 * value / HBM_PEAK_GBPS, 2),
                    "host_wall_ms_per_step": round(wall_ms / args.steps, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                      "kernel": "gemv_mfma_kernel<Q1> gate||up 24576x4096", "bytes_per_launch": kbytes,
                      "avg_launch_us": round(avg_us.value, 3), "per_kernel": per_kernel},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(blocks, xs)
-    print(json.dumps(out), flush=True)
     for name, _, _ in SHAPES:
         for h in ids[name]:
             be.free_weights(h)
     L.oxb_hip_set_stream(None)
+    torch.cuda.synchronize()
+    if args.calibrate:
+        src = torch.ones(64 * 2**20, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    if not args.no_decode:
+        out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu)
+    print(json.dumps(out), flush=True)
     return 0
 
 
