@@ -86,6 +86,17 @@ int  oxb_hip_gemv_q1_g128(const uint8_t* aos, size_t n_bytes, const float* x, si
 int  oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len,
                            float* y, size_t y_len, uint32_t n_rows, uint32_t k);
 
+/* ---- prefill GEMM: GpuBackendTrait::gemm_q1_g128 (KG/mod.rs:425-441; scalar semantics K/gemm.rs:19-87,
+ * K/gemm_ternary.rs:35-69; CUDA tier: gemm_q1_g128_v7 / gemm_tq2_g128_v7, KG/cuda_prefill_kernels.rs:74-140, 457-551).
+ * y[m][n_rows] = x[m][k] * W^T on the fp16 matrix cores with fp32 accumulation: weights and products are exact,
+ * activations are rounded to fp16 after a per-row power-of-two scaling (relative 2^-11 per element).  Use
+ * oxb_hip_gemv with batch = m where fp32-exact products are required.  _dev takes device pointers and does not
+ * synchronize; profile_gemm packs x once, then times `iters` GEMM launches with events on the library's stream. */
+int  oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_rows, uint32_t k);
+int  oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k);
+int  oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
+                          uint32_t warmup, uint32_t iters, float* avg_us);
+
 /* ---- batch_ffn_phase (KG/mod.rs:519; CUDA: KG/cuda_graph/nativecudabackend_traits.rs:122-188 -> encode_ffn_phase,
  * KG/cuda_graph/cudagraph_encoding.rs:72-160): hidden += O * attn_out; normed = RMSNorm(hidden); hidden += down * SwiGLU(gate||up * normed),
  * in place on the host vector `hidden[h]`.  fmt selects Q1 / TQ2 weights; gate_up holds the gate rows, then the up rows. */

@@ -101,15 +101,16 @@ class NativeHipBackend:
         _check(fn(_u8(b), b.size, _f32(x), x.size, _f32(y), y.size, n_rows, k))
         return y
 
-    def gemm_q1_g128(self, block_bytes, input, m: int, n_rows: int, k: int) -> np.ndarray:
-        """[m x k] inputs -> [m x n_rows]; the trait's default loops GEMV per row (mod.rs:425-440),
-        here the weights are uploaded once and streamed once per two input rows."""
-        return self._oneshot_gemm(Q1, block_bytes, input, m, n_rows, k)
+    def gemm_q1_g128(self, block_bytes, input, m: int, n_rows: int, k: int, exact: bool | None = None) -> np.ndarray:
+        """[m x k] inputs -> [m x n_rows] (mod.rs:425-440).  m > 16 runs the fp16 matrix-core prefill GEMM
+        (activations rounded to fp16); m <= 16 or ``exact=True`` streams the weights once per two input rows
+        through the GEMV kernel with fp32-exact products, like the reference's per-row loop."""
+        return self._oneshot_gemm(Q1, block_bytes, input, m, n_rows, k, exact)
 
-    def gemm_tq2_g128(self, block_bytes, input, m: int, n_rows: int, k: int) -> np.ndarray:
-        return self._oneshot_gemm(TQ2, block_bytes, input, m, n_rows, k)
+    def gemm_tq2_g128(self, block_bytes, input, m: int, n_rows: int, k: int, exact: bool | None = None) -> np.ndarray:
+        return self._oneshot_gemm(TQ2, block_bytes, input, m, n_rows, k, exact)
 
-    def _oneshot_gemm(self, fmt, block_bytes, input, m, n_rows, k):
+    def _oneshot_gemm(self, fmt, block_bytes, input, m, n_rows, k, exact=None):
         x = np.ascontiguousarray(input, dtype=np.float32).reshape(-1)
         if k % QK != 0:
             raise GpuError(5, f"invalid argument: k={k} is not a multiple of 128")
@@ -117,9 +118,22 @@ class NativeHipBackend:
             raise GpuError(5, f"invalid argument: input holds {x.size} values, {m * k} needed")
         h = self._upload(fmt, block_bytes, n_rows, k)
         try:
-            return self._gemv_cached(h, x[:m * k], n_rows, k, m)
+            if exact is None:
+                exact = m <= 16
+            if exact:
+                return self._gemv_cached(h, x[:m * k], n_rows, k, m)
+            return self.gemm_cached(h, x[:m * k], m, n_rows, k)
         finally:
             self.free_weights(h)
+
+    def gemm_cached(self, handle: int, input, m: int, n_rows: int, k: int) -> np.ndarray:
+        """Prefill GEMM on a resident weight: fp16 matrix cores, fp32 accumulation."""
+        x = np.ascontiguousarray(input, dtype=np.float32).reshape(-1)
+        if x.size != m * k:
+            raise GpuError(5, f"invalid argument: input holds {x.size} values, {m * k} needed")
+        y = np.empty((m, n_rows), dtype=np.float32)
+        _check(self._lib.oxb_hip_gemm(int(handle), _f32(x), _f32(y), m, n_rows, k))
+        return y
 
     # -- resident weights -------------------------------------------------------
     def upload_weights_raw(self, block_bytes, n_rows: int | None = None, k: int | None = None,

@@ -1,0 +1,33 @@
+// gemm_kernels.h — launch interface of the prefill GEMM (fp16 MFMA) and its activation packer.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "layout.h"
+
+enum { OXB_GEMM_STORE = 0, OXB_GEMM_RESIDUAL = 2 };
+
+struct OxbGemmParams {
+    const uint32_t* codes;   // resident codes section
+    const uint16_t* scales;  // resident scales section
+    const uint32_t* xh;      // packed fp16 activations (oxb_launch_xh_pack)
+    const int32_t* xsh;      // [M] exponent that undoes the row scaling, INT32_MIN for a non-finite row
+    float* y;                // [M][ldy]
+    const float* residual;   // [M][ldy], mode RESIDUAL only
+    uint32_t n_rows, n_tiles, n_sb;
+    uint32_t M, M_pad;       // token rows, and that count rounded up to 16
+    uint32_t ldy;
+    uint32_t tpw;            // row tiles per workgroup   (filled by the launcher)
+    uint32_t n_mt;           // token tiles of the launch (filled by the launcher)
+    uint32_t codes_bytes, scales_bytes, xh_bytes;  // buffer extents (loads beyond them read 0)
+    int mode;
+};
+
+// Bytes of the packed activation buffer for M token rows of length k.
+size_t oxb_xh_bytes(uint32_t k, uint32_t M);
+
+// x[M][ldx] fp32 (the first k of every row) -> fp16 in MFMA B-operand order, each row scaled by a power of two
+// so that its largest element lies in [2^14, 2^15).
+hipError_t oxb_launch_xh_pack(int fmt, const float* d_x, uint32_t ldx, uint32_t k, uint32_t M, uint32_t* d_xh,
+                              int32_t* d_xsh, hipStream_t st);
+hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st);

@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "../../include/oxb_hip.h"
+#include "gemm_kernels.h"
 #include "gemv_kernels.h"
 #include "layout.h"
 #include "repack.h"
@@ -156,6 +157,39 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
     return OXB_HIP_OK;
 }
 
+int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
+                const float* d_residual) {
+    const uint32_t k = w.L.k;
+    if ((uint64_t)m * k >= (1ull << 31))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u rows of %u activations exceed one GEMM call", m, k);
+    int rc;
+    if ((rc = g_rt.ws_xh.ensure(oxb_xh_bytes(k, m)))) return rc;
+    if ((rc = g_rt.ws_xsh.ensure(((size_t)m + 16) * sizeof(int32_t)))) return rc;
+    hipError_t e = oxb_launch_xh_pack((int)w.L.fmt, d_x, ldx, k, m, (uint32_t*)g_rt.ws_xh.ptr, (int32_t*)g_rt.ws_xsh.ptr,
+                                      g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "kernel launch failed: xh_pack");
+    OxbGemmParams p;
+    memset(&p, 0, sizeof p);
+    p.codes = w.d_codes;
+    p.scales = w.d_scales;
+    p.xh = (const uint32_t*)g_rt.ws_xh.ptr;
+    p.xsh = (const int32_t*)g_rt.ws_xsh.ptr;
+    p.y = d_y;
+    p.residual = d_residual;
+    p.n_rows = w.L.n_rows;
+    p.n_tiles = w.L.n_tiles;
+    p.n_sb = w.L.n_sb;
+    p.M = m;
+    p.ldy = ldy;
+    p.codes_bytes = (uint32_t)w.L.codes_bytes;
+    p.scales_bytes = (uint32_t)w.L.scales_bytes;
+    p.xh_bytes = (uint32_t)oxb_xh_bytes(k, m);
+    p.mode = mode;
+    e = oxb_launch_gemm((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemm");
+    return OXB_HIP_OK;
+}
+
 static int check_shape(const Weight& w, uint32_t n_rows, uint32_t k) {
     if (k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
     if (w.L.n_rows != n_rows || w.L.k != k)
@@ -241,6 +275,8 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_xq.release();
     g_rt.ws_cneg.release();
     g_rt.ws_xexp.release();
+    g_rt.ws_xh.release();
+    g_rt.ws_xsh.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.own_stream = nullptr;
     g_rt.stream = nullptr;
@@ -384,6 +420,85 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
         p.scales_bytes = (uint32_t)w->L.scales_bytes;
         e = oxb_launch_gemv(fmt, p, g_rt.n_cus, g_rt.stream);
         if (e != hipSuccess) rc = hip_fail(e, "kernel launch failed: gemv");
+    }
+    (void)hipEventRecord(ev1, g_rt.stream);
+    if (rc == OXB_HIP_OK) {
+        e = hipEventSynchronize(ev1);
+        if (e != hipSuccess) rc = fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: %s", hipGetErrorString(e));
+    }
+    if (rc == OXB_HIP_OK) {
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, ev0, ev1);
+        *avg_us = ms * 1000.0f / (float)iters;
+    }
+    (void)hipEventDestroy(ev0);
+    (void)hipEventDestroy(ev1);
+    return rc;
+}
+
+int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
+    return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr);
+}
+
+int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_rows, uint32_t k) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!x || !y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
+    const size_t xb = (size_t)m * k * sizeof(float), yb = (size_t)m * n_rows * sizeof(float);
+    if ((rc = g_rt.ws_x.ensure(xb))) return rc;
+    if ((rc = g_rt.ws_y.ensure(yb))) return rc;
+    hipError_t e = hipMemcpyAsync(g_rt.ws_x.ptr, x, xb, hipMemcpyHostToDevice, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "input upload");
+    rc = gemm_device(*w, (const float*)g_rt.ws_x.ptr, k, (float*)g_rt.ws_y.ptr, m, n_rows, OXB_GEMM_STORE, nullptr);
+    if (rc) return rc;
+    e = hipMemcpyAsync(y, g_rt.ws_y.ptr, yb, hipMemcpyDeviceToHost, g_rt.stream);
+    if (e != hipSuccess) return hip_fail(e, "output download");
+    return sync_stream("gemm");
+}
+
+int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
+                         uint32_t warmup, uint32_t iters, float* avg_us) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!d_x || !d_y || !avg_us || m == 0 || iters == 0)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
+    if ((rc = gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr))) return rc;  // packs x, warms up
+    OxbGemmParams p;
+    memset(&p, 0, sizeof p);
+    p.codes = w->d_codes;
+    p.scales = w->d_scales;
+    p.xh = (const uint32_t*)g_rt.ws_xh.ptr;
+    p.xsh = (const int32_t*)g_rt.ws_xsh.ptr;
+    p.y = d_y;
+    p.n_rows = n_rows;
+    p.n_tiles = w->L.n_tiles;
+    p.n_sb = w->L.n_sb;
+    p.M = m;
+    p.ldy = n_rows;
+    p.codes_bytes = (uint32_t)w->L.codes_bytes;
+    p.scales_bytes = (uint32_t)w->L.scales_bytes;
+    p.xh_bytes = (uint32_t)oxb_xh_bytes(k, m);
+    p.mode = OXB_GEMM_STORE;
+    hipEvent_t ev0, ev1;
+    hipError_t e;
+    if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");
+    if ((e = hipEventCreate(&ev1)) != hipSuccess) { (void)hipEventDestroy(ev0); return hip_fail(e, "event creation"); }
+    for (uint32_t i = 0; i < warmup + iters && rc == OXB_HIP_OK; i++) {
+        if (i == warmup) (void)hipEventRecord(ev0, g_rt.stream);
+        e = oxb_launch_gemm((int)w->L.fmt, p, g_rt.n_cus, g_rt.stream);
+        if (e != hipSuccess) rc = hip_fail(e, "kernel launch failed: gemm");
     }
     (void)hipEventRecord(ev1, g_rt.stream);
     if (rc == OXB_HIP_OK) {
