@@ -26,6 +26,7 @@ __device__ __forceinline__ float dpp_f32(float v) {
 // Buffer resources: a load whose byte offset lies outside the buffer returns 0 and moves no
 // data, which replaces every "is this tile / superblock / column in range" branch below.
 typedef unsigned v4u __attribute__((ext_vector_type(4)));
+typedef unsigned v2u __attribute__((ext_vector_type(2)));
 #define OXB_OOB 0xFFFFFFF0u
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)bytes, 0x00020000);

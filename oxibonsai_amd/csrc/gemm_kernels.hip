@@ -95,53 +95,55 @@ __global__ __launch_bounds__(256) void xh_pack_kernel(const float* __restrict__ 
 // ---------------------------------------------------------------------------
 // GEMM.
 // ---------------------------------------------------------------------------
-template <int FMT, int RT>
-struct WeightRegs {
-    v4i c[RT][FMT == OXB_FMT_Q1 ? 1 : 2];  // one superblock of codes per row tile
-    uint32_t d[RT][4];                     // fp16 scale bits of this lane's row, blocks 0..3 of the superblock
+// Codes and scales of one row tile for half a superblock (two 128-weight blocks), as loaded: the unit of the
+// in-place register ring (half 0 is reloaded for the next superblock while half 1 is still being consumed).
+template <int FMT>
+struct HalfRegs {
+    uint32_t c[FMT == OXB_FMT_Q1 ? 2 : 4];  // Q1: dword e = sign bits of block e; TQ2: dwords 2e, 2e+1 = fields of block e
+    uint32_t d[2];                          // fp16 scale bits of blocks 0, 1 of the half (this lane's row)
 };
 
-template <int FMT, int RT>
-__device__ __forceinline__ void load_weights(WeightRegs<FMT, RT>& W, __amdgpu_buffer_rsrc_t rc, __amdgpu_buffer_rsrc_t rs,
-                                             uint32_t t0, uint32_t n_valid, uint32_t n_sb, uint32_t sb, uint32_t lane) {
-    constexpr uint32_t UNIT = FMT == OXB_FMT_Q1 ? 1024u : 2048u;
+template <int FMT>
+__device__ __forceinline__ void load_half(HalfRegs<FMT>& H, __amdgpu_buffer_rsrc_t rc, __amdgpu_buffer_rsrc_t rs,
+                                          uint32_t tile, bool ok, uint32_t n_sb, uint32_t sb, int half, uint32_t lane) {
     const uint32_t r = lane & 15u;
-#pragma unroll
-    for (int rt = 0; rt < RT; rt++) {
-        const bool ok = (uint32_t)rt < n_valid && sb < n_sb;
-        const uint32_t unit = (t0 + rt) * n_sb + sb;
-        const uint32_t cv = ok ? lane * 16u : OXB_OOB;
-        W.c[rt][0] = buf_load_b128(rc, cv, unit * UNIT);
-        if (FMT != OXB_FMT_Q1) W.c[rt][FMT == OXB_FMT_Q1 ? 0 : 1] = buf_load_b128(rc, ok ? lane * 16u + 1024u : OXB_OOB, unit * UNIT);
-        const uint32_t sv = ok ? ((r >> 2) * 16u + (r & 3u)) * 2u : OXB_OOB;
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-            W.d[rt][q] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)(ok ? sv + q * 8u : OXB_OOB), (int)(unit * 128u), 0);
+    const uint32_t unit = tile * n_sb + sb;  // wave-uniform
+    ok = ok && sb < n_sb;
+    if (FMT == OXB_FMT_Q1) {
+        const v2u v = __builtin_amdgcn_raw_buffer_load_b64(rc, (int)(ok ? lane * 16u + half * 8u : OXB_OOB), (int)(unit * 1024u), 0);
+        H.c[0] = v.x, H.c[1] = v.y;
+    } else {
+        const v4i v = buf_load_b128(rc, ok ? lane * 16u + half * 1024u : OXB_OOB, unit * 2048u);
+        H.c[0] = (uint32_t)v.x, H.c[1] = (uint32_t)v.y, H.c[FMT == OXB_FMT_Q1 ? 0 : 2] = (uint32_t)v.z,
+        H.c[FMT == OXB_FMT_Q1 ? 1 : 3] = (uint32_t)v.w;
     }
+    const uint32_t sv = ((r >> 2) * 16u + (r & 3u)) * 2u + half * 16u;  // scale of block 2*half, then +8 bytes
+#pragma unroll
+    for (int e = 0; e < 2; e++)
+        H.d[e] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)(ok ? sv + e * 8u : OXB_OOB), (int)(unit * 128u), 0);
 }
 
 // Per (row tile, block) state prepared once and used by the four MFMA steps of the block.
-template <int FMT>
 struct BlockDec {
-    uint32_t w0, w1;  // Q1: w0 = inverted sign bits (xor the scale's sign); TQ2: fields of halves m = 0, 1 as value+1
-    uint32_t d2;      // Q1: |d| in both halves; TQ2: d in both halves
+    uint32_t w0, w1;  // Q1: w0 = inverted sign bits (xor the scale's sign); TQ2: fields of the 16-weight halves as value+1
+    uint32_t d2;      // Q1: |d| in both halves of the dword; TQ2: d in both halves
 };
 
 template <int FMT>
-__device__ __forceinline__ BlockDec<FMT> prepare_block(const v4i (&c)[FMT == OXB_FMT_Q1 ? 1 : 2], uint32_t dbits, int q) {
-    BlockDec<FMT> B;
+__device__ __forceinline__ BlockDec prepare_block(const HalfRegs<FMT>& H, int e) {
+    BlockDec B;
+    const uint32_t dbits = H.d[e];
     const uint32_t dd = (dbits & 0xFFFFu) * 0x00010001u;
     if (FMT == OXB_FMT_Q1) {
         // weight = bit ? d : -d  ->  sign bit = ~bit ^ sign(d)
         const uint32_t flip = (uint32_t)((int32_t)(dbits << 16) >> 31);
-        B.w0 = ~(uint32_t)c[0][q] ^ flip;
+        B.w0 = ~H.c[e] ^ flip;
         B.w1 = 0;
         B.d2 = dd & 0x7FFF7FFFu;
     } else {
         // fields at in-byte position 3 are 2-bit two's complement (3, 0, 1 for -1, 0, +1): adding 1 modulo 4
         // turns them into value+1 like the others
-        const int half = q >> 1, e = q & 1;
-        const uint32_t a = (uint32_t)c[half][2 * e], b = (uint32_t)c[half][2 * e + 1];
+        const uint32_t a = H.c[FMT == OXB_FMT_Q1 ? 0 : 2 * e], b = H.c[FMT == OXB_FMT_Q1 ? 0 : 2 * e + 1];
         B.w0 = (a & 0x3F3F3F3Fu) | (((a & 0xC0C0C0C0u) + 0x40404040u) & 0xC0C0C0C0u);
         B.w1 = (b & 0x3F3F3F3Fu) | (((b & 0xC0C0C0C0u) + 0x40404040u) & 0xC0C0C0C0u);
         B.d2 = dd;
@@ -151,7 +153,7 @@ __device__ __forceinline__ BlockDec<FMT> prepare_block(const v4i (&c)[FMT == OXB
 
 // The A operand of MFMA step s (0..3) of the block.
 template <int FMT>
-__device__ __forceinline__ v8h decode_step(const BlockDec<FMT>& B, int s) {
+__device__ __forceinline__ v8h decode_step(const BlockDec& B, int s) {
     uint32_t o[4];
     if (FMT == OXB_FMT_Q1) {
 #pragma unroll
@@ -172,11 +174,52 @@ __device__ __forceinline__ v8h decode_step(const BlockDec<FMT>& B, int s) {
     return __builtin_bit_cast(v8h, u);
 }
 
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+// One 128-weight block of the K loop: 4 MFMA steps over the staged token tile `xsb`.  The A operands of the
+// step after the current one are expanded while the current step's MFMAs run (for the last step: the first
+// step of the next block, from `bdn`), and each B operand is reloaded for the next step right after its last use.
+template <int FMT, int RT, int CT>
+__device__ __forceinline__ void block_steps(const v8h* __restrict__ xsb, v8h (&A)[RT], const BlockDec (&bd)[RT],
+                                            const BlockDec (&bdn)[RT], v4f (&acc)[RT][CT], uint32_t boff) {
+    constexpr int BM = 16 * CT;
+    v8h B[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ct++) B[ct] = xsb[boff + ct * 16];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        v8h An[RT];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) An[rt] = s < 3 ? decode_step<FMT>(bd[rt], s + 1) : decode_step<FMT>(bdn[rt], 0);
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++)  // row tiles past the range hold zero weights
+                acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[rt], B[ct], acc[rt][ct], 0, 0, 0);
+            if (s < 3) B[ct] = xsb[boff + (s + 1) * BM + ct * 16];
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) A[rt] = An[rt];
+        // issue order: one MFMA, then the VALU work that expands the next A operand, a B reload per token tile
+#pragma unroll
+        for (int i = 0; i < RT * CT; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, FMT == OXB_FMT_Q1 ? 1 : 2, 0);
+            if (s < 3 && i % RT == RT - 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);  // one scheduling region per step keeps compile time bounded
+    }
+}
+
 template <int FMT, int RT, int CT>
 __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGemmParams p) {
     constexpr int BM = 16 * CT;
-    __shared__ __attribute__((aligned(16))) uint4 xs[2][16 * BM];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, r = lane & 15u, g = lane >> 4;
+    // two stages of the token tile: [chunk 4g+s][token] x 16 bytes.  Separate arrays, so that loads in flight
+    // into one stage do not make reads of the other wait.
+    __shared__ __attribute__((aligned(16))) uint4 xs0[16 * BM];
+    __shared__ __attribute__((aligned(16))) uint4 xs1[16 * BM];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, g = lane >> 4;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));  // keeps unit offsets in SGPRs
     const uint32_t m_t = blockIdx.x % p.n_mt, n_g = blockIdx.x / p.n_mt;
     const uint32_t m0 = m_t * BM;
     // row tiles: the workgroup's [wg_t0, wg_t1), split evenly over the four waves
@@ -195,7 +238,8 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) acc[rt][ct] = (v4f){0.f, 0.f, 0.f, 0.f};
 
-    // this thread's share of an X stage: CT items of 16 bytes; item id = it*256 + tid -> chunk id / BM, token id % BM
+    // this thread's share of an X stage: CT items of 16 bytes; item id = it*256 + tid -> chunk id / BM, token id % BM.
+    // The loads write LDS directly: lane l of a wave fills bytes [16 l, 16 l + 16) after the wave's base.
     uint32_t xoff[CT];
 #pragma unroll
     for (int it = 0; it < CT; it++) {
@@ -204,51 +248,74 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     }
     const uint32_t blk_stride = 16u * p.M_pad * 16u;  // bytes of xh per block
     const uint32_t nblk = p.n_sb * 4u;
+    auto stage_x = [&](uint32_t blk, uint4* xs) {
+        const uint32_t soff = (blk < nblk ? blk : nblk - 1) * blk_stride;  // past the end: restage the last block
+#pragma unroll
+        for (int it = 0; it < CT; it++)
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, (lds_ptr_t)(xs + it * OXB_GEMM_THREADS + wave * 64), 16,
+                                                     (int)xoff[it], (int)soff, 0, 0);
+    };
+    auto publish = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
-    v4i xr[CT];
+    HalfRegs<FMT> H[RT][2];
+    stage_x(0, xs0);
 #pragma unroll
-    for (int it = 0; it < CT; it++) xr[it] = buf_load_b128(rx, xoff[it], 0);
-    WeightRegs<FMT, RT> Wn;
-    load_weights<FMT, RT>(Wn, rc, rs, t0, n_valid, p.n_sb, 0, lane);
+    for (int rt = 0; rt < RT; rt++) {
+        load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, 0, 0, lane);
+        load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, 0, 1, lane);
+    }
+    publish();
+    BlockDec bd[RT], bdn[RT];
+    v8h A[RT];
 #pragma unroll
-    for (int it = 0; it < CT; it++) reinterpret_cast<v4i*>(xs[0])[it * OXB_GEMM_THREADS + tid] = xr[it];
-    lds_barrier();
+    for (int rt = 0; rt < RT; rt++) {
+        bd[rt] = prepare_block<FMT>(H[rt][0], 0);
+        A[rt] = decode_step<FMT>(bd[rt], 0);
+    }
+    const uint32_t boff = g * 4 * BM + r;  // this lane's B operand of step s, token tile ct: xs[boff + s*BM + 16 ct]
+    const v8h* x0 = reinterpret_cast<const v8h*>(xs0);
+    const v8h* x1 = reinterpret_cast<const v8h*>(xs1);
 
     for (uint32_t sb = 0; sb < p.n_sb; sb++) {
-        WeightRegs<FMT, RT> W = Wn;
-        load_weights<FMT, RT>(Wn, rc, rs, t0, n_valid, p.n_sb, sb + 1, lane);
+        // block 0 of the superblock
+        stage_x(sb * 4 + 1, xs1);
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const uint32_t blk = sb * 4 + q;
-            const int buf = q & 1;
-            const bool more = blk + 1 < nblk;
-            if (more) {
+        for (int rt = 0; rt < RT; rt++) bdn[rt] = prepare_block<FMT>(H[rt][0], 1);
+        block_steps<FMT, RT, CT>(x0, A, bd, bdn, acc, boff);
+        publish();
+        // block 1: half 0 is consumed; reload it for the next superblock
+        stage_x(sb * 4 + 2, xs0);
 #pragma unroll
-                for (int it = 0; it < CT; it++) xr[it] = buf_load_b128(rx, xoff[it], (blk + 1) * blk_stride);
-            }
-            BlockDec<FMT> bd[RT];
-#pragma unroll
-            for (int rt = 0; rt < RT; rt++) bd[rt] = prepare_block<FMT>(W.c[rt], W.d[rt][q], q);
-            const v8h* xsb = reinterpret_cast<const v8h*>(xs[buf]);
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                v8h A[RT];
-#pragma unroll
-                for (int rt = 0; rt < RT; rt++) A[rt] = decode_step<FMT>(bd[rt], s);
-#pragma unroll
-                for (int ct = 0; ct < CT; ct++) {
-                    const v8h B = xsb[(g * 4 + s) * BM + ct * 16 + r];
-#pragma unroll
-                    for (int rt = 0; rt < RT; rt++)  // row tiles past the range hold zero weights
-                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[rt], B, acc[rt][ct], 0, 0, 0);
-                }
-            }
-            if (more) {
-#pragma unroll
-                for (int it = 0; it < CT; it++) reinterpret_cast<v4i*>(xs[buf ^ 1])[it * OXB_GEMM_THREADS + tid] = xr[it];
-            }
-            lds_barrier();
+        for (int rt = 0; rt < RT; rt++) {
+            bd[rt] = bdn[rt];
+            bdn[rt] = prepare_block<FMT>(H[rt][1], 0);
         }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
+        block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
+        publish();
+        // block 2
+        stage_x(sb * 4 + 3, xs1);
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            bd[rt] = bdn[rt];
+            bdn[rt] = prepare_block<FMT>(H[rt][1], 1);
+        }
+        block_steps<FMT, RT, CT>(x0, A, bd, bdn, acc, boff);
+        publish();
+        // block 3: half 1 is consumed; the next block is block 0 of the next superblock (half 0, already reloaded)
+        stage_x(sb * 4 + 4, xs0);
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            bd[rt] = bdn[rt];
+            bdn[rt] = prepare_block<FMT>(H[rt][0], 0);
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
+        block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
+        publish();
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) bd[rt] = bdn[rt];
     }
 
     // epilogue: lane holds rows 4g..4g+3 of the row tile for token 16ct + r
@@ -318,15 +385,17 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     constexpr uint32_t CT = 8, BM = 16 * CT;
     p.M_pad = (p.M + 15u) / 16u * 16u;
     p.n_mt = (p.M + BM - 1) / BM;
-    // Row tiles per workgroup: minimise (rounds of workgroups over the CUs) x (row tiles per wave).
-    static const uint32_t rts[] = {1, 2, 3, 4, 5};
+    // Row tiles per workgroup: minimise (rounds of workgroups over the CUs) x (time of one workgroup), where a
+    // workgroup costs its row tiles per wave plus about one more for staging, barriers and operand latency.
+    // Ties go to the larger tile (less re-reading of X).
+    static const uint32_t rts[] = {5, 4, 3, 2, 1};
     uint32_t best_rt = 0, best_tpw = 0;
     uint64_t best_cost = ~0ull;
     for (uint32_t rt : rts) {
         for (uint32_t tpw = 4 * rt; tpw > 4 * rt - 4; tpw--) {
             const uint32_t groups = (p.n_tiles + tpw - 1) / tpw;
             const uint64_t wgs = (uint64_t)groups * p.n_mt;
-            const uint64_t cost = ((wgs + n_cus - 1) / n_cus) * rt * 64 + rt;  // ties: fewer tiles per wave
+            const uint64_t cost = ((wgs + n_cus - 1) / n_cus) * (rt + 1);
             if (cost < best_cost) best_cost = cost, best_rt = rt, best_tpw = tpw;
         }
     }
