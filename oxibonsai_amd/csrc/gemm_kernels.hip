@@ -151,27 +151,51 @@ __device__ __forceinline__ BlockDec prepare_block(const HalfRegs<FMT>& H, int e)
     return B;
 }
 
-// The A operand of MFMA step s (0..3) of the block.
-template <int FMT>
-__device__ __forceinline__ v8h decode_step(const BlockDec& B, int s) {
-    uint32_t o[4];
+// The A operands of MFMA step s (0..3) of the block for all row tiles.  Written operation by operation across
+// the RT x 4 independent dwords, so that consecutive VALU instructions do not depend on each other.
+template <int FMT, int RT>
+__device__ __forceinline__ void decode_step(const BlockDec (&B)[RT], int s, v8h (&A)[RT]) {
+    uint32_t o[RT][4];
+    // The masks live in registers (VOP3 encodings take no literal), opaque to the compiler so that
+    // (x & mask) | y stays one v_and_or_b32.
+    uint32_t kmask, kmagic;
     if (FMT == OXB_FMT_Q1) {
+        asm volatile("s_mov_b32 %0, 0x80008000" : "=s"(kmask));
 #pragma unroll
-        for (int p = 0; p < 4; p++) o[p] = ((B.w0 << (15 - (4 * s + p))) & 0x80008000u) | B.d2;
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) o[rt][p] = B[rt].w0 << (15 - (4 * s + p));
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) o[rt][p] = (o[rt][p] & kmask) | B[rt].d2;
     } else {
-        const uint32_t w = (s >> 1) ? B.w1 : B.w0;
-        const v2h dd = __builtin_bit_cast(v2h, B.d2);
+        asm volatile("s_mov_b32 %0, 0x00030003" : "=s"(kmask));
+        asm volatile("v_mov_b32 %0, 0x64006400" : "=v"(kmagic));
         const v2h bias = {(_Float16)1025.0f, (_Float16)1025.0f};
+        v2h v[RT][4];
 #pragma unroll
-        for (int p = 0; p < 4; p++) {
-            // 0x6400 | field is the fp16 number 1024 + field; both steps below are exact
-            const uint32_t t = ((w >> (2 * (4 * (s & 1) + p))) & 0x00030003u) | 0x64006400u;
-            const v2h v = (__builtin_bit_cast(v2h, t) - bias) * dd;
-            o[p] = __builtin_bit_cast(uint32_t, v);
-        }
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) o[rt][p] = ((s >> 1) ? B[rt].w1 : B[rt].w0) >> (2 * (4 * (s & 1) + p));
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) o[rt][p] = (o[rt][p] & kmask) | kmagic;  // fp16 1024 + field
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) v[rt][p] = __builtin_bit_cast(v2h, o[rt][p]) - bias;  // exact: field - 1
+#pragma unroll
+        for (int p = 0; p < 4; p++)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) o[rt][p] = __builtin_bit_cast(uint32_t, v[rt][p] * __builtin_bit_cast(v2h, B[rt].d2));
     }
-    const v4u u = {o[0], o[1], o[2], o[3]};
-    return __builtin_bit_cast(v8h, u);
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++) {
+        const v4u u = {o[rt][0], o[rt][1], o[rt][2], o[rt][3]};
+        A[rt] = __builtin_bit_cast(v8h, u);
+    }
 }
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -183,14 +207,19 @@ template <int FMT, int RT, int CT>
 __device__ __forceinline__ void block_steps(const v8h* __restrict__ xsb, v8h (&A)[RT], const BlockDec (&bd)[RT],
                                             const BlockDec (&bdn)[RT], v4f (&acc)[RT][CT], uint32_t boff) {
     constexpr int BM = 16 * CT;
+    constexpr int NV = FMT == OXB_FMT_Q1 ? 1 : 2;  // VALU instructions issued after each MFMA
     v8h B[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ct++) B[ct] = xsb[boff + ct * 16];
+    // all B operands of the first step are requested at once, so their LDS latency is paid once per block
+    __builtin_amdgcn_sched_group_barrier(0x100, CT, 0);
 #pragma unroll
     for (int s = 0; s < 4; s++) {
         v8h An[RT];
-#pragma unroll
-        for (int rt = 0; rt < RT; rt++) An[rt] = s < 3 ? decode_step<FMT>(bd[rt], s + 1) : decode_step<FMT>(bdn[rt], 0);
+        if (s < 3)
+            decode_step<FMT, RT>(bd, s + 1, An);
+        else
+            decode_step<FMT, RT>(bdn, 0, An);
 #pragma unroll
         for (int ct = 0; ct < CT; ct++) {
 #pragma unroll
@@ -204,7 +233,11 @@ __device__ __forceinline__ void block_steps(const v8h* __restrict__ xsb, v8h (&A
 #pragma unroll
         for (int i = 0; i < RT * CT; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, FMT == OXB_FMT_Q1 ? 1 : 2, 0);
+            // (the first step also absorbs the per-block preparation of the next block's codes)
+            if (s == 0)
+                __builtin_amdgcn_sched_group_barrier(0x002, NV + 1, 0);
+            else
+                __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
             if (s < 3 && i % RT == RT - 1) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
         __builtin_amdgcn_sched_barrier(0);  // one scheduling region per step keeps compile time bounded
@@ -268,10 +301,8 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     BlockDec bd[RT], bdn[RT];
     v8h A[RT];
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++) {
-        bd[rt] = prepare_block<FMT>(H[rt][0], 0);
-        A[rt] = decode_step<FMT>(bd[rt], 0);
-    }
+    for (int rt = 0; rt < RT; rt++) bd[rt] = prepare_block<FMT>(H[rt][0], 0);
+    decode_step<FMT, RT>(bd, 0, A);
     const uint32_t boff = g * 4 * BM + r;  // this lane's B operand of step s, token tile ct: xs[boff + s*BM + 16 ct]
     const v8h* x0 = reinterpret_cast<const v8h*>(xs0);
     const v8h* x1 = reinterpret_cast<const v8h*>(xs1);
