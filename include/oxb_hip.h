@@ -128,6 +128,14 @@ int  oxb_hip_model_destroy(uint64_t model);
  * Runs all layers, the final norm, the LM head and a first-maximum argmax on the device (a HIP graph after the first
  * call).  logits_or_null: [batch][vocab]; token_out: [batch] greedy ids (either may be NULL). */
 int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out);
+/* Batched prefill: try_cuda_prefill / try_cuda_prefill_ternary (KG/cuda_prefill/try_apis.rs:42, 318; per layer
+ * encode_prefill_layer[_ternary], KG/cuda_prefill/encode_q1.rs:123, encode_ternary.rs:114).  hidden = [n_tokens][h]
+ * embedding rows of sequence `seq` (0 .. batch-1) for positions pos_start .. pos_start + n_tokens - 1; keys and
+ * values of those positions are written to the sequence's cache, so decode (or another prefill chunk) continues
+ * at pos_start + n_tokens.  Projections run as prefill GEMMs (oxb_hip_gemm), attention as one causal launch per
+ * layer; logits [vocab] and the greedy token are those of the last token (either pointer may be null). */
+int  oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t n_tokens, uint32_t pos_start,
+                     float* logits_or_null, uint32_t* token_out_or_null);
 int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is replayed from a captured graph */
 
 /* ---- host-only helpers (no GPU needed): the upload-time repack, exposed so it can be checked on any machine.

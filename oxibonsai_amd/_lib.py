@@ -48,6 +48,7 @@ _SIGNATURES = {
     "oxb_hip_model_reset": ([C.c_uint64], C.c_int),
     "oxb_hip_model_destroy": ([C.c_uint64], C.c_int),
     "oxb_hip_decode": ([C.c_uint64, f32p, u32p, f32p, u32p], C.c_int),
+    "oxb_hip_prefill": ([C.c_uint64, C.c_uint32, f32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_model_uses_graph": ([C.c_uint64], C.c_int),
     "oxb_hip_repack_sizes": ([C.c_int, C.c_uint32, C.c_uint32, szp, szp], C.c_int),
     "oxb_hip_repack": ([C.c_int, u8p, C.c_size_t, C.c_uint32, C.c_uint32, u8p, C.c_size_t, u8p, C.c_size_t], C.c_int),

@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "lib")
-SOURCES = ["runtime.hip", "gemv_kernels.hip", "gemm_kernels.hip", "layer_kernels.hip", "model.hip", "repack.cpp"]
+SOURCES = ["runtime.hip", "gemv_kernels.hip", "gemm_kernels.hip", "layer_kernels.hip", "prefill_kernels.hip", "model.hip", "repack.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # packed-FP32 VALU forms are kept out of every kernel
@@ -46,7 +46,7 @@ def build(verbose: bool = False) -> str:
             print(msgs, flush=True)
         return obj
 
-    with ThreadPoolExecutor(max_workers=5) as ex:
+    with ThreadPoolExecutor(max_workers=6) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     so = lib_path()
     subprocess.check_call([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", so, *objs])

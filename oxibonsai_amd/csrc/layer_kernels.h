@@ -9,7 +9,8 @@ struct OxbQkParams {
     uint32_t qkv_stride;
     const float *q_norm, *k_norm;  // [hd]
     const float *cos_t, *sin_t;    // [max_seq][hd/2]
-    const uint32_t* pos;           // [batch], device
+    const uint32_t* pos;           // [batch], device; null: row b is token pos_base + b of sequence `seq` (prefill)
+    uint32_t pos_base, seq;
     float* q_rope;                 // [batch][nq][hd]
     __half *k_cache, *v_cache;     // [batch][n_layers][nkv][max_seq][hd]
     uint32_t nq, nkv, hd, max_seq, n_layers, layer;

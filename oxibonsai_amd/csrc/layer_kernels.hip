@@ -127,14 +127,15 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
     const uint32_t hh = is_q ? head : head - p.nq;
     const float* in = p.qkv + (size_t)b * p.qkv_stride + (is_q ? (size_t)hh * hd : (size_t)(p.nq + hh) * hd);
     const float* w = is_q ? p.q_norm : p.k_norm;
-    const uint32_t pos = p.pos[b];
+    const uint32_t pos = p.pos ? p.pos[b] : p.pos_base + b;
+    const uint32_t seq = p.pos ? b : p.seq;
     float ss = 0.f;
     for (uint32_t d = tid; d < hd; d += 128) ss += in[d] * in[d];
     ss = block_sum(ss, red);
     const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
     const float* cs = p.cos_t + (size_t)pos * half;
     const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t cache_off = ((((size_t)b * p.n_layers + p.layer) * p.nkv + hh) * p.max_seq + pos) * hd;
+    const size_t cache_off = ((((size_t)seq * p.n_layers + p.layer) * p.nkv + hh) * p.max_seq + pos) * hd;
     for (uint32_t d = tid; d < half; d += 128) {
         const float lo = w[d] * in[d] * inv_rms, hi = w[d + half] * in[d + half] * inv_rms;
         const float c = cs[d], s = sn[d];

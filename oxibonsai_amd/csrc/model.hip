@@ -20,8 +20,10 @@
 #include <vector>
 
 #include "../../include/oxb_hip.h"
+#include "gemm_kernels.h"
 #include "gemv_kernels.h"
 #include "layer_kernels.h"
+#include "prefill_kernels.h"
 #include "runtime_internal.h"
 
 namespace oxb {
@@ -49,6 +51,11 @@ struct Model {
     bool graph_failed = false;
     bool want_logits_in_graph = true;
     std::vector<void*> allocs;
+    // prefill activations for up to pf_cap token rows (allocated on first use)
+    uint32_t pf_cap = 0;
+    float *pf_hidden = nullptr, *pf_normed = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr,
+          *pf_gu = nullptr, *pf_act = nullptr;
+    std::vector<void*> pf_allocs;
 };
 
 static std::unordered_map<uint64_t, std::unique_ptr<Model>> g_models;
@@ -67,6 +74,9 @@ static void free_model(Model& m) {
     m.graph_exec = nullptr;
     for (void* p : m.allocs) (void)hipFree(p);
     m.allocs.clear();
+    for (void* p : m.pf_allocs) (void)hipFree(p);
+    m.pf_allocs.clear();
+    m.pf_cap = 0;
 }
 
 void shutdown_models() {
@@ -197,6 +207,8 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         qp.cos_t = m.cos_t;
         qp.sin_t = m.sin_t;
         qp.pos = m.pos;
+        qp.pos_base = 0;
+        qp.seq = 0;
         qp.q_rope = m.q_rope;
         qp.k_cache = m.k_cache;
         qp.v_cache = m.v_cache;
@@ -244,6 +256,106 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         }
         OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, st), "kernel launch failed: argmax");
     }
+    return OXB_HIP_OK;
+}
+
+// Prefill buffers for `rows` token rows.
+static int ensure_prefill_buffers(Model& m, uint32_t rows) {
+    if (rows <= m.pf_cap) return OXB_HIP_OK;
+    (void)hipStreamSynchronize(g_rt.stream);
+    for (void* p : m.pf_allocs) (void)hipFree(p);
+    m.pf_allocs.clear();
+    m.pf_cap = 0;
+    const oxb_model_desc& d = m.d;
+    const size_t R = (rows + 127u) / 128u * 128u, qd = (size_t)d.nq * d.hd, qkv_rows = qd + 2 * (size_t)d.nkv * d.hd;
+    struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_normed, R * d.h}, {&m.pf_qkv, R * qkv_rows},
+                                             {&m.pf_q, R * qd},       {&m.pf_attn, R * qd},    {&m.pf_gu, R * 2 * d.inter},
+                                             {&m.pf_act, R * d.inter}};
+    for (auto& b : bufs) {
+        if (hipMalloc((void**)b.p, b.n * sizeof(float)) != hipSuccess) {
+            for (void* p : m.pf_allocs) (void)hipFree(p);
+            m.pf_allocs.clear();
+            return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", b.n * sizeof(float), g_rt.device);
+        }
+        m.pf_allocs.push_back(*b.p);
+    }
+    m.pf_cap = (uint32_t)R;
+    return OXB_HIP_OK;
+}
+
+// All layers for M token rows of sequence `seq` at positions pos_start .. pos_start + M - 1: batched
+// projections on the matrix cores, one causal attention launch per layer, KV written to the cache; then the
+// LM head and the greedy token for the last row.
+static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start) {
+    const oxb_model_desc& d = m.d;
+    hipStream_t st = g_rt.stream;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < d.n_layers; L++) {
+        const oxb_layer_ids& ly = m.layers[L];
+        const float* attn_norm = vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
+        const float* q_norm = vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
+        const float* k_norm = vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
+        const float* ffn_norm = vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
+        const Weight* wqkv = mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
+        const Weight* wo = mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
+        const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
+        const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
+        if (rc) return rc;
+        OXB_TRY_HIP(oxb_launch_rmsnorm_rows(m.pf_hidden, attn_norm, d.eps, d.h, M, m.pf_normed, st), "kernel launch failed: rmsnorm_rows");
+        OXB_TRY(gemm_device(*wqkv, m.pf_normed, d.h, m.pf_qkv, M, qkv_rows, OXB_GEMM_STORE, nullptr));
+        OxbQkParams qp;
+        qp.qkv = m.pf_qkv;
+        qp.qkv_stride = qkv_rows;
+        qp.q_norm = q_norm;
+        qp.k_norm = k_norm;
+        qp.cos_t = m.cos_t;
+        qp.sin_t = m.sin_t;
+        qp.pos = nullptr;
+        qp.pos_base = pos_start;
+        qp.seq = seq;
+        qp.q_rope = m.pf_q;
+        qp.k_cache = m.k_cache;
+        qp.v_cache = m.v_cache;
+        qp.nq = d.nq;
+        qp.nkv = d.nkv;
+        qp.hd = d.hd;
+        qp.max_seq = d.max_seq;
+        qp.n_layers = d.n_layers;
+        qp.layer = L;
+        qp.eps = d.eps;
+        OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, M, st), "kernel launch failed: qk_norm_rope_store");
+        OxbPrefillAttnParams ap;
+        const size_t layer_off = (((size_t)seq * d.n_layers + L) * d.nkv) * (size_t)d.max_seq * d.hd;
+        ap.q = m.pf_q;
+        ap.k_cache = m.k_cache + layer_off;
+        ap.v_cache = m.v_cache + layer_off;
+        ap.out = m.pf_attn;
+        ap.M = M;
+        ap.pos_start = pos_start;
+        ap.nq = d.nq;
+        ap.nkv = d.nkv;
+        ap.hd = d.hd;
+        ap.max_seq = d.max_seq;
+        ap.scale = 1.0f / sqrtf((float)d.hd);
+        OXB_TRY_HIP(oxb_launch_attn_prefill(ap, st), "kernel launch failed: attn_prefill");
+        OXB_TRY(gemm_device(*wo, m.pf_attn, qd, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden));
+        OXB_TRY_HIP(oxb_launch_rmsnorm_rows(m.pf_hidden, ffn_norm, d.eps, d.h, M, m.pf_normed, st), "kernel launch failed: rmsnorm_rows");
+        OXB_TRY(gemm_device(*wgu, m.pf_normed, d.h, m.pf_gu, M, 2 * d.inter, OXB_GEMM_STORE, nullptr));
+        OXB_TRY_HIP(oxb_launch_swiglu_rows(m.pf_gu, d.inter, M, m.pf_act, st), "kernel launch failed: swiglu_rows");
+        OXB_TRY(gemm_device(*wdn, m.pf_act, d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden));
+    }
+    // last token: final norm, LM head, greedy token (fp32-exact products, as in a decode step)
+    const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
+    const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+    if (rc) return rc;
+    float* last = m.hidden + (size_t)seq * d.h;
+    OXB_TRY_HIP(hipMemcpyAsync(last, m.pf_hidden + (size_t)(M - 1) * d.h, (size_t)d.h * 4, hipMemcpyDeviceToDevice, st), "last row copy");
+    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, last, final_norm, d.eps, vec_absmax(d.final_norm), d.h, 1, m.xq.xq, m.xq.cneg, m.xq.xexp,
+                                         nullptr, st),
+                "kernel launch failed: rmsnorm_quant");
+    OXB_TRY(gemv_xq(*lm, m.xq, 1, m.logits + (size_t)seq * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
+    OXB_TRY_HIP(oxb_launch_argmax(m.logits + (size_t)seq * d.vocab, d.vocab, 1, m.tokens + seq, st), "kernel launch failed: argmax");
     return OXB_HIP_OK;
 }
 
@@ -440,6 +552,30 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
         OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits, (size_t)d.batch * d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t n_tokens, uint32_t pos_start,
+                    float* logits_or_null, uint32_t* token_out_or_null) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (!hidden || n_tokens == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden or no tokens");
+    if (seq >= d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, d.batch);
+    if ((uint64_t)pos_start + n_tokens > d.max_seq)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
+                    (unsigned long long)pos_start + n_tokens - 1, d.max_seq);
+    OXB_TRY(ensure_prefill_buffers(m, n_tokens));
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(m.pf_hidden, hidden, (size_t)n_tokens * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY(encode_prefill(m, seq, n_tokens, pos_start));
+    if (token_out_or_null) OXB_TRY_HIP(hipMemcpyAsync(token_out_or_null, m.tokens + seq, 4, hipMemcpyDeviceToHost, st), "token download");
+    if (logits_or_null)
+        OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits + (size_t)seq * d.vocab, (size_t)d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: prefill: %s", hipGetErrorString(e));
     return OXB_HIP_OK;
 }
 

@@ -1,0 +1,19 @@
+// prefill_kernels.h — launch interface of the token-batched prefill glue (see prefill_kernels.hip).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+struct OxbPrefillAttnParams {
+    const float* q;                   // [M][nq][hd], after QK-norm and RoPE
+    const __half *k_cache, *v_cache;  // this sequence's, this layer's cache: [nkv][max_seq][hd]
+    float* out;                       // [M][nq * hd]
+    uint32_t M, pos_start;            // query t sits at position pos_start + t and sees keys 0 .. pos_start + t
+    uint32_t nq, nkv, hd, max_seq;
+    float scale;                      // 1 / sqrt(hd)
+};
+
+hipError_t oxb_launch_rmsnorm_rows(const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t M, float* d_out,
+                                   hipStream_t st);
+hipError_t oxb_launch_swiglu_rows(const float* d_gu, uint32_t inter, uint32_t M, float* d_act, hipStream_t st);
+hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st);

@@ -76,6 +76,18 @@ class HipModel:
                                         tokens.ctypes.data_as(_lib.u32p)))
         return logits, tokens
 
+    def prefill(self, hidden, pos_start: int = 0, seq: int = 0, want_logits: bool = True):
+        """Batched prefill of one sequence (try_cuda_prefill, gpu_backend/cuda_prefill/try_apis.rs:42, 318).
+        hidden: [n_tokens, h] embedding rows for positions pos_start.. -> (last-token logits [vocab] or None,
+        greedy token of the last position).  Decode continues at pos_start + n_tokens."""
+        hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(-1, self.cfg["h"])
+        logits = np.empty(self.cfg["vocab"], dtype=np.float32) if want_logits else None
+        token = np.empty(1, dtype=np.uint32)
+        _check(self._lib.oxb_hip_prefill(self.id, seq, hv.ctypes.data_as(_lib.f32p), hv.shape[0], pos_start,
+                                         logits.ctypes.data_as(_lib.f32p) if want_logits else None,
+                                         token.ctypes.data_as(_lib.u32p)))
+        return logits, int(token[0])
+
     def uses_graph(self) -> bool:
         return bool(self._lib.oxb_hip_model_uses_graph(self.id))
 
