@@ -20,7 +20,7 @@ struct OxbQkParams {
 struct OxbAttnParams {
     const float* q;                      // [batch][nq][hd]
     const __half *k_cache, *v_cache;
-    float* part;                         // [batch][nq][n_splits][hd + 2]
+    float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
     float scale;                         // 1 / sqrt(hd)
@@ -33,6 +33,14 @@ hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w,
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);
-#define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers
-hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
-hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, hipStream_t st);
+#define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers at a time
+#define OXB_ATTN_MAX_SPLITS 64        // slots the KV sequence is split over; slot s walks chunks s, s + n_splits, ...
+#define OXB_ATTN_PART_PAD 4           // floats after the hd outputs of a slot: maximum, sum, 2 unused (16-byte rows)
+// Split-KV attention into p.part, then the merge of the slots fused with the quantiser of the O projection's
+// input for sequences b0 .. b0 + nb - 1 (nb <= 2); d_out_or_null also receives the fp32 attention output [batch][nq*hd].
+hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
+hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
+                                         int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st);
+// d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.
+#define OXB_ARGMAX_MAX_PARTS 256u
+hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st);

@@ -195,20 +195,24 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     const uint32_t Gall = p.nq / p.nkv, h0 = kvh * Gall + sub * GM;  // first q head served here
     const uint32_t G = (Gall - sub * GM) < (uint32_t)GM ? (Gall - sub * GM) : (uint32_t)GM;
     const uint32_t seq_len = p.pos[b] + 1;
-    const uint32_t s0 = split * OXB_ATTN_CHUNK;
-    const uint32_t s1 = (s0 + OXB_ATTN_CHUNK) < seq_len ? (s0 + OXB_ATTN_CHUNK) : seq_len;
-    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + split) * (HD + 2);
-    const size_t part_head = (size_t)p.n_splits * (HD + 2);
-    if (s0 >= seq_len) {  // nothing in this chunk: mark it empty for every head of the group
-        if (tid < G) {
-            part[tid * part_head + HD] = -INFINITY;
-            part[tid * part_head + HD + 1] = 0.f;
-        }
-        return;
-    }
+    const uint32_t n_chunks = (seq_len + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK;
+    // slot `split` takes chunks split, split + n_splits, ...; slots past the last chunk are never read
+    if (split >= n_chunks) return;
+    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + split) * (HD + OXB_ATTN_PART_PAD);
+    const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
     const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * HD;
     const __half* K = p.k_cache + base;
     const __half* V = p.v_cache + base;
+    const __amdgpu_buffer_rsrc_t rk = make_rsrc(K, p.max_seq * HD * 2u), rv = make_rsrc(V, p.max_seq * HD * 2u);
+    // running result over this slot's chunks: thread -> outputs i = tid, tid + 256, ... of the G * HD
+    constexpr int OPT = (GM * HD + OXB_ATTN_THREADS - 1) / OXB_ATTN_THREADS;
+    float run_o[OPT], run_m[OPT], run_l[OPT];
+#pragma unroll
+    for (int j = 0; j < OPT; j++) run_o[j] = 0.f, run_m[j] = -INFINITY, run_l[j] = 0.f;
+
+    for (uint32_t chunk = split; chunk < n_chunks; chunk += p.n_splits) {
+    const uint32_t s0 = chunk * OXB_ATTN_CHUNK;
+    const uint32_t s1 = (s0 + OXB_ATTN_CHUNK) < seq_len ? (s0 + OXB_ATTN_CHUNK) : seq_len;
     const uint32_t t = s0 + tid;
     const bool live = tid < OXB_ATTN_CHUNK && t < s1;  // the threads that own one position in the softmax phase
 
@@ -231,7 +235,6 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     }
     // K rows of the score phase and V rows of the weighted-sum phase, all requested now: both depend
     // only on pos.  Buffer loads return 0 past s1 without a branch or a select after the load.
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(K, p.max_seq * HD * 2u), rv = make_rsrc(V, p.max_seq * HD * 2u);
     v4i kreg[NPASS];
 #pragma unroll
     for (int i = 0; i < NPASS; i++) {
@@ -326,67 +329,150 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
             *reinterpret_cast<float4*>(&accs[(slice * GM + h) * HD + grp * 8 + 4]) = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
         }
     __syncthreads();
-    for (uint32_t i = tid; i < G * HD; i += OXB_ATTN_THREADS) {
-        const uint32_t h = i / HD, d = i % HD;
-        float v = 0.f;
+    // merge the chunk into the running result (online softmax across chunks)
 #pragma unroll
-        for (int s = 0; s < NSL; s++) v += accs[(s * GM + h) * HD + d];
-        part[h * part_head + d] = v;
+    for (int j = 0; j < OPT; j++) {
+        const uint32_t i = tid + (uint32_t)j * OXB_ATTN_THREADS;
+        if (i < G * HD) {
+            const uint32_t h = i / HD, d = i % HD;
+            float v = 0.f;
+#pragma unroll
+            for (int s = 0; s < NSL; s++) v += accs[(s * GM + h) * HD + d];
+            const float mc = m[0], lc = red[h * 4] + red[h * 4 + 1] + red[h * 4 + 2] + red[h * 4 + 3];
+            float mh = mc;
+#pragma unroll
+            for (int hh = 1; hh < GM; hh++) mh = (h == (uint32_t)hh) ? m[hh] : mh;
+            const float mn = fmaxf(run_m[j], mh);
+            const float a = expf(run_m[j] - mn), bw = expf(mh - mn);   // a = 0 for the first chunk
+            run_o[j] = run_o[j] * a + v * bw;
+            run_l[j] = run_l[j] * a + lc * bw;
+            run_m[j] = mn;
+        }
     }
-    if (tid < G) {
-        float mm = m[0];
+    __syncthreads();  // the next chunk reuses sc, red and accs
+    }
 #pragma unroll
-        for (int h = 1; h < GM; h++) mm = (tid == (uint32_t)h) ? m[h] : mm;
-        part[tid * part_head + HD] = mm;
-        part[tid * part_head + HD + 1] = red[tid * 4] + red[tid * 4 + 1] + red[tid * 4 + 2] + red[tid * 4 + 3];
+    for (int j = 0; j < OPT; j++) {
+        const uint32_t i = tid + (uint32_t)j * OXB_ATTN_THREADS;
+        if (i < G * HD) {
+            const uint32_t h = i / HD, d = i % HD;
+            part[h * part_head + d] = run_o[j];
+            if (d == 0) {
+                part[h * part_head + HD] = run_m[j];
+                part[h * part_head + HD + 1] = run_l[j];
+            }
+        }
     }
 }
 
-// Merge the chunk results of one q head: grid (nq, batch), hd threads.
-__global__ __launch_bounds__(256) void attn_combine_kernel(OxbAttnParams p, float* __restrict__ out) {
-    const uint32_t qh = blockIdx.x, b = blockIdx.y, d = threadIdx.x, hd = p.hd;
-    const float* part = p.part + ((size_t)b * p.nq + qh) * p.n_splits * (hd + 2);
-    const uint32_t used = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
-    float M = -INFINITY;
-    for (uint32_t s = 0; s < used; s++) M = fmaxf(M, part[(size_t)s * (hd + 2) + hd]);
-    float L = 0.f, acc = 0.f;
-    for (uint32_t s = 0; s < used; s++) {
-        const float* ps = part + (size_t)s * (hd + 2);
-        const float wgt = expf(ps[hd] - M);
-        L = fmaf(ps[hd + 1], wgt, L);
-        acc = fmaf(ps[d], wgt, acc);
+// Merge the slot results of every q head of one sequence and quantise the attention output for the
+// O projection, in one workgroup (1024 threads): softmax weights of the slots per head (one wave per
+// head, one slot per lane), the weighted sum with four outputs per thread, then the activation quantiser.
+// Grid (vectors of the pass); sequence b0 + blockIdx.x becomes vector blockIdx.x of the quantised pass.
+template <int FMT>
+__global__ __launch_bounds__(1024) void attn_combine_quant_kernel(OxbAttnParams p, uint32_t b0, uint32_t NC,
+                                                                   uint32_t nblk_pad, uint32_t* __restrict__ xq,
+                                                                   int32_t* __restrict__ cneg, int32_t* __restrict__ xexp,
+                                                                   float* __restrict__ out_or_null) {
+    extern __shared__ float sm[];  // [qd] outputs | [nq][64] slot weights | [nq] 1 / sum
+    __shared__ float red[16];
+    __shared__ int bad_flag;
+    const uint32_t n = blockIdx.x, b = b0 + n, tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
+    const uint32_t stride = hd + OXB_ATTN_PART_PAD;
+    float* o = sm;
+    float* wts = sm + qd;
+    float* inv_l = wts + p.nq * 64;
+    const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
+    const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
+    const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
+    for (uint32_t h = tid >> 6; h < p.nq; h += 16) {
+        const float* ph = part + ((size_t)h * p.n_splits + lane) * stride + hd;
+        const float mv = lane < used ? ph[0] : -INFINITY, lv = lane < used ? ph[1] : 0.f;
+        float M = mv;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+        const float w = lane < used ? expf(mv - M) : 0.f;
+        float L = w * lv;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+        wts[h * 64 + lane] = w;
+        if (lane == 0) inv_l[h] = L > 0.f ? 1.0f / L : 0.f;
     }
-    out[((size_t)b * p.nq + qh) * hd + d] = L > 0.f ? acc / L : 0.f;
+    __syncthreads();
+    float mx = 0.f;
+    int bad = 0;
+    for (uint32_t e = tid * 4; e < qd; e += 4096) {
+        const uint32_t h = e / hd, d = e % hd;
+        const float* ph = part + (size_t)h * p.n_splits * stride + d;
+        float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+        uint32_t s = 0;
+        for (; s + 4 <= used; s += 4) {
+            float4 v[4];
+#pragma unroll
+            for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(ph + (size_t)(s + u) * stride);
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const float w = wts[h * 64 + s + u];
+                acc.x = fmaf(v[u].x, w, acc.x), acc.y = fmaf(v[u].y, w, acc.y), acc.z = fmaf(v[u].z, w, acc.z), acc.w = fmaf(v[u].w, w, acc.w);
+            }
+        }
+        for (; s < used; s++) {
+            const float4 v = *reinterpret_cast<const float4*>(ph + (size_t)s * stride);
+            const float w = wts[h * 64 + s];
+            acc.x = fmaf(v.x, w, acc.x), acc.y = fmaf(v.y, w, acc.y), acc.z = fmaf(v.z, w, acc.z), acc.w = fmaf(v.w, w, acc.w);
+        }
+        const float il = inv_l[h];
+        acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
+        *reinterpret_cast<float4*>(o + e) = acc;
+        if (out_or_null) *reinterpret_cast<float4*>(out_or_null + (size_t)b * qd + e) = acc;
+        bad |= oxb_not_finite(acc.x) | oxb_not_finite(acc.y) | oxb_not_finite(acc.z) | oxb_not_finite(acc.w);
+        mx = fmaxf(fmaxf(mx, fmaxf(fabsf(acc.x), fabsf(acc.y))), fmaxf(fabsf(acc.z), fabsf(acc.w)));
+    }
+    bool any_bad;
+    mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);  // its barriers also publish the outputs
+    quantise_vector<FMT>(o, qd, nblk_pad, NC, n, mx, any_bad, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
 // Greedy selection: index of the first maximum (strict '>', as argmax_f32, cuda_kernels.rs:407-436).
-// One workgroup per vector.
+// Two stages: grid (parts, vectors) workgroups each reduce a contiguous span to (value, index), then one
+// wave per vector merges the parts; ties go to the lower index at every step.
 // ---------------------------------------------------------------------------
-__global__ __launch_bounds__(1024) void argmax_kernel(const float* __restrict__ logits, uint32_t n,
-                                                       uint32_t* __restrict__ out) {
-    __shared__ float sv[16];
-    __shared__ uint32_t si[16];
-    const float* v = logits + (size_t)blockIdx.x * n;
+__device__ __forceinline__ void argmax_merge(float& best, uint32_t& idx, float ob, uint32_t oi) {
+    if (oi != 0xFFFFFFFFu && (idx == 0xFFFFFFFFu || ob > best || (ob == best && oi < idx))) { best = ob; idx = oi; }
+}
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits, uint32_t n, uint32_t span,
+                                                              float* __restrict__ pv, uint32_t* __restrict__ pi) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    const float* v = logits + (size_t)blockIdx.y * n;
+    const uint32_t i0 = blockIdx.x * span, i1 = min(i0 + span, n);
     float best = -INFINITY;
     uint32_t idx = 0xFFFFFFFFu;
-    for (uint32_t i = threadIdx.x; i < n; i += 1024) {
+    for (uint32_t i = i0 + threadIdx.x; i < i1; i += 256) {
         const float x = v[i];
         if (idx == 0xFFFFFFFFu || x > best) { best = x; idx = i; }
     }
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        const float ob = __shfl_xor(best, o, 64);
-        const uint32_t oi = __shfl_xor(idx, o, 64);
-        if (ob > best || (ob == best && oi < idx)) { best = ob; idx = oi; }
-    }
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(best, idx, __shfl_xor(best, o, 64), __shfl_xor(idx, o, 64));
     if ((threadIdx.x & 63u) == 0) { sv[threadIdx.x >> 6] = best; si[threadIdx.x >> 6] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 16; w++)
-            if (sv[w] > best || (sv[w] == best && si[w] < idx)) { best = sv[w]; idx = si[w]; }
-        out[blockIdx.x] = idx == 0xFFFFFFFFu ? 0u : idx;
+        for (int w = 1; w < 4; w++) argmax_merge(best, idx, sv[w], si[w]);
+        pv[blockIdx.y * gridDim.x + blockIdx.x] = best;
+        pi[blockIdx.y * gridDim.x + blockIdx.x] = idx;
     }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
+                                                           uint32_t parts, uint32_t* __restrict__ out) {
+    float best = -INFINITY;
+    uint32_t idx = 0xFFFFFFFFu;
+    for (uint32_t i = threadIdx.x; i < parts; i += 64) argmax_merge(best, idx, pv[blockIdx.x * parts + i], pi[blockIdx.x * parts + i]);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(best, idx, __shfl_xor(best, o, 64), __shfl_xor(idx, o, 64));
+    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0xFFFFFFFFu ? 0u : idx;
 }
 
 // ---------------------------------------------------------------------------
@@ -444,22 +530,44 @@ static hipError_t launch_attn_hd(const OxbAttnParams& p, uint32_t batch, hipStre
     return hipGetLastError();
 }
 
-hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st) {
-    if (p.chunk != OXB_ATTN_CHUNK) return hipErrorInvalidValue;
-    hipError_t e;
+hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
+    if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
     switch (p.hd) {
-        case 32: e = launch_attn_hd<32>(p, batch, st); break;
-        case 64: e = launch_attn_hd<64>(p, batch, st); break;
-        case 128: e = launch_attn_hd<128>(p, batch, st); break;
-        case 256: e = launch_attn_hd<256>(p, batch, st); break;
+        case 32: return launch_attn_hd<32>(p, batch, st);
+        case 64: return launch_attn_hd<64>(p, batch, st);
+        case 128: return launch_attn_hd<128>(p, batch, st);
+        case 256: return launch_attn_hd<256>(p, batch, st);
         default: return hipErrorInvalidValue;
     }
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(p.nq, batch), dim3(p.hd), 0, st, p, d_out);
+}
+
+hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
+                                         int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st) {
+    const uint32_t qd = p.nq * p.hd;
+    if (nb == 0 || nb > 2 || (qd % OXB_QK) != 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
+    const size_t shm = ((size_t)qd + p.nq * 64 + p.nq) * sizeof(float);
+    if (shm > 60 * 1024) return hipErrorInvalidValue;
+    const uint32_t NC = OXB_XQ_DIGITS * nb, nblk_pad = oxb_nblk_pad(qd);
+    if (fmt == OXB_FMT_Q1)
+        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_Q1>, dim3(nb), dim3(1024), shm, st, p, b0, NC, nblk_pad, d_xq, d_cneg,
+                           d_xexp, d_out_or_null);
+    else
+        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_TQ2>, dim3(nb), dim3(1024), shm, st, p, b0, NC, nblk_pad, d_xq, d_cneg,
+                           d_xexp, d_out_or_null);
     return hipGetLastError();
 }
 
-hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, hipStream_t st) {
-    hipLaunchKernelGGL(argmax_kernel, dim3(batch), dim3(1024), 0, st, d_logits, n, d_out);
+uint32_t oxb_argmax_parts(uint32_t n) {
+    const uint32_t p = (n + 2047u) / 2048u;
+    return p < 1 ? 1 : (p > OXB_ARGMAX_MAX_PARTS ? OXB_ARGMAX_MAX_PARTS : p);
+}
+
+hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st) {
+    if (n == 0 || batch == 0 || !d_ws) return hipErrorInvalidValue;
+    const uint32_t parts = oxb_argmax_parts(n), span = (n + parts - 1) / parts;
+    float* pv = reinterpret_cast<float*>(d_ws);
+    uint32_t* pi = reinterpret_cast<uint32_t*>(d_ws) + (size_t)batch * parts;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, span, pv, pi);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(batch), dim3(64), 0, st, pv, pi, parts, d_out);
     return hipGetLastError();
 }

@@ -41,6 +41,7 @@ struct Model {
     float *hidden = nullptr, *qkv = nullptr, *q_rope = nullptr, *attn_part = nullptr, *attn_out = nullptr,
           *gu = nullptr, *logits = nullptr;
     uint32_t *tokens = nullptr, *pos = nullptr;
+    void* argmax_ws = nullptr;
     __half *k_cache = nullptr, *v_cache = nullptr;
     float *cos_t = nullptr, *sin_t = nullptr;
     void* xq_mem = nullptr;
@@ -164,7 +165,8 @@ static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn
                       const Weight& o, const Weight& gate_up, const Weight& down, float* gu, uint32_t h,
                       uint32_t inter, uint32_t attn_k, uint32_t nb) {
     hipStream_t st = g_rt.stream;
-    OXB_TRY_HIP(oxb_launch_quant_x(fmt, attn_out, attn_k, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: quant_x");
+    if (attn_out)  // null: xb already holds the quantised attention output
+        OXB_TRY_HIP(oxb_launch_quant_x(fmt, attn_out, attn_k, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: quant_x");
     OXB_TRY(gemv_xq(o, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
     OXB_TRY_HIP(oxb_launch_rmsnorm_quant(fmt, hidden, ffn_norm, eps, ffn_norm_absmax, h, nb, xb.xq, xb.cneg, xb.xexp, nullptr, st),
                 "kernel launch failed: rmsnorm_quant");
@@ -235,10 +237,12 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         ap.chunk = m.chunk;
         ap.n_splits = m.n_splits;
         ap.scale = 1.0f / sqrtf((float)d.hd);
-        OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, m.attn_out, st), "kernel launch failed: attention");
+        OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, st), "kernel launch failed: attention");
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm,
+            OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, b0, nb, m.xq.xq, m.xq.cneg, m.xq.xexp, nullptr, st),
+                        "kernel launch failed: attn_combine_quant");
+            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, nullptr, ffn_norm,
                                vec_absmax(ly.ffn_norm), d.eps, *wo,
                                *wgu, *wdn, m.gu + (size_t)b0 * 2 * d.inter, d.h, d.inter, qd, nb));
         }
@@ -254,7 +258,7 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
                         "kernel launch failed: rmsnorm_quant");
             OXB_TRY(gemv_xq(*lm, m.xq, nb, m.logits + (size_t)b0 * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
         }
-        OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, st), "kernel launch failed: argmax");
+        OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, m.argmax_ws, st), "kernel launch failed: argmax");
     }
     return OXB_HIP_OK;
 }
@@ -355,7 +359,7 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
                                          nullptr, st),
                 "kernel launch failed: rmsnorm_quant");
     OXB_TRY(gemv_xq(*lm, m.xq, 1, m.logits + (size_t)seq * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
-    OXB_TRY_HIP(oxb_launch_argmax(m.logits + (size_t)seq * d.vocab, d.vocab, 1, m.tokens + seq, st), "kernel launch failed: argmax");
+    OXB_TRY_HIP(oxb_launch_argmax(m.logits + (size_t)seq * d.vocab, d.vocab, 1, m.tokens + seq, m.argmax_ws, st), "kernel launch failed: argmax");
     return OXB_HIP_OK;
 }
 
@@ -418,6 +422,8 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u query heads per %u kv heads (need a whole ratio <= 8)", d.nq, d.nkv);
     if (d.h % 128 || d.inter % 128 || (d.nq * d.hd) % 128)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden, intermediate and nq*hd must be multiples of 128");
+    if (((size_t)d.nq * d.hd + (size_t)d.nq * 65) * sizeof(float) > 60 * 1024)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: nq*hd = %u exceeds what the attention merge holds in LDS", d.nq * d.hd);
     auto mp = std::make_unique<Model>();
     Model& m = *mp;
     m.d = d;
@@ -443,6 +449,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
 
     m.chunk = OXB_ATTN_CHUNK_POSITIONS;
     m.n_splits = (d.max_seq + m.chunk - 1) / m.chunk;
+    if (m.n_splits > OXB_ATTN_MAX_SPLITS) m.n_splits = OXB_ATTN_MAX_SPLITS;
     const size_t B = d.batch;
     const size_t kv_elems = B * d.n_layers * d.nkv * (size_t)d.max_seq * d.hd;
     uint32_t kmax = d.h > d.inter ? d.h : d.inter;
@@ -450,10 +457,10 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
     if ((rc = dev_alloc(m, (void**)&m.hidden, B * d.h * 4)) || (rc = dev_alloc(m, (void**)&m.qkv, B * qkv_rows * 4)) ||
         (rc = dev_alloc(m, (void**)&m.q_rope, B * qd * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + 2) * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, (void**)&m.k_cache, kv_elems * 2)) ||
+        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = dev_alloc(m, (void**)&m.k_cache, kv_elems * 2)) ||
         (rc = dev_alloc(m, (void**)&m.v_cache, kv_elems * 2)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
