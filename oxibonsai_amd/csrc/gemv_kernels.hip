@@ -32,27 +32,22 @@
 // The activation quantiser (quant_device.h) produces the MFMA B operands ("digit planes").
 #define OXB_QUANT_THREADS 256
 
+// Grid (vectors, parts): each workgroup takes whole exponent groups of one vector, finds their maxima and
+// quantises them; no workgroup needs anything from another.
 template <int FMT>
-__global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float* __restrict__ x, uint32_t k,
-                                                                     uint32_t nblk_pad, uint32_t NC,
+__global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float* __restrict__ x, uint32_t k, uint32_t NC,
+                                                                     uint32_t gsb, uint32_t n_groups,
                                                                      uint32_t* __restrict__ xq,
                                                                      int32_t* __restrict__ cneg,
                                                                      int32_t* __restrict__ xexp) {
-    __shared__ float red[OXB_QUANT_THREADS / 64];
-    __shared__ int bad_flag;
-    const uint32_t n = blockIdx.x, tid = threadIdx.x;
+    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
+    const uint32_t n = blockIdx.x;
+    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
+    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
+    if (g0 >= g1) return;
     const float* xn = x + (size_t)n * k;
-    float mx = 0.0f;
-    int bad = 0;
-    for (uint32_t i = tid * 4; i < k; i += OXB_QUANT_THREADS * 4) {
-        const float4 v = *reinterpret_cast<const float4*>(xn + i);
-        const float a = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
-        bad |= oxb_not_finite(v.x) | oxb_not_finite(v.y) | oxb_not_finite(v.z) | oxb_not_finite(v.w);
-        mx = fmaxf(mx, a);
-    }
-    bool any_bad;
-    mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);
-    quantise_vector<FMT>(xn, k, nblk_pad, NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
+    gstat_scan(xn, k, gsb, g0, g1, gstat);
+    quantise_groups<FMT>(xn, k, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
@@ -150,8 +145,14 @@ __global__ __launch_bounds__(512, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(con
             B[i][q][1] = buf_load_b128(r_xq, ok ? (((blk * 2 + 1) * 4 + g) * NC + c) * 16u : OXB_OOB);
             C4[i][q] = buf_load_b128(r_cneg, ok ? (blk * NC + c) * 16u : OXB_OOB);
         }
-    // In the recombination, thread t handles column (t % NC): digit (t % 8) of vector (t % NC) / 8.
-    const int xe = p.xexp[(threadIdx.x % NC) >> 3];
+    // In the recombination, thread t handles column (t % NC): digit (t % 8) of vector (t % NC) / 8, and needs
+    // the exponent of every wave's K slice (= exponent group) of that vector.
+    __shared__ int xes[2 * 8];  // [vector][wave]; published by the first barrier of the tile loop
+    if (threadIdx.x < 16) {
+        const uint32_t vec = threadIdx.x >> 3, w = threadIdx.x & 7u;
+        xes[threadIdx.x] = (vec * 8 < NC && w < S) ? p.xexp[vec * p.n_groups + p.sb_begin / NSBW + w] : 0;
+    }
+    const uint32_t my_vec = (threadIdx.x % NC) >> 3;
 
     const uint32_t tpw = p.groups * TG, t_begin = blockIdx.x * tpw;
     const uint32_t t_end = (t_begin + tpw) < p.n_tiles ? (t_begin + tpw) : p.n_tiles;
@@ -198,8 +199,15 @@ __global__ __launch_bounds__(512, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(con
         for (uint32_t idx = threadIdx.x; idx < (uint32_t)TG * 16 * NC; idx += blockDim.x) {
             const uint32_t cc = idx % NC, rr = (idx / NC) & 15u, slot = idx / (16 * NC);
             float v = 0.f;
-            for (uint32_t w = 0; w < S; w++) v += buf[(((size_t)slot * S + w) * NC + cc) * 16 + rr];
-            v = (xe == INT32_MIN) ? __int_as_float(0x7FC00000) : ldexpf(v, xe + 8 * (int)(cc & 7u));
+            bool nan = false;
+#pragma unroll
+            for (int w = 0; w < 8; w++)
+                if ((uint32_t)w < S) {
+                    const int xe = xes[my_vec * 8 + w];
+                    nan |= xe == INT32_MIN;
+                    v += ldexpf(buf[(((size_t)slot * S + w) * NC + cc) * 16 + rr], xe + 8 * (int)(cc & 7u));
+                }
+            if (nan) v = __int_as_float(0x7FC00000);
             v += dpp_f32<OXB_DPP_ROW_SHR(1)>(v);
             v += dpp_f32<OXB_DPP_ROW_SHR(2)>(v);
             v += dpp_f32<OXB_DPP_ROW_SHR(4)>(v);
@@ -255,14 +263,16 @@ size_t oxb_cneg_bytes(uint32_t k, uint32_t batch) {
 
 hipError_t oxb_launch_quant_x(int fmt, const float* d_x, uint32_t k, uint32_t batch, uint32_t* d_xq, int32_t* d_cneg,
                               int32_t* d_xexp, hipStream_t st) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
-    const size_t shm = 0;
+    const uint32_t n_sb = (k + 511u) / 512u, NC = OXB_XQ_DIGITS * batch;
+    const uint32_t gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
+    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
+    const dim3 grid(batch, n_groups < 16 ? n_groups : 16);
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, dim3(batch, oxb_quant_parts(k)), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
-                           d_cneg, d_xexp);
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, grid, dim3(OXB_QUANT_THREADS), 0, st, d_x, k, NC, gsb, n_groups, d_xq, d_cneg,
+                           d_xexp);
     else
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, dim3(batch, oxb_quant_parts(k)), dim3(OXB_QUANT_THREADS), shm, st, d_x, k, nblk_pad, NC, d_xq,
-                           d_cneg, d_xexp);
+        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, grid, dim3(OXB_QUANT_THREADS), 0, st, d_x, k, NC, gsb, n_groups, d_xq, d_cneg,
+                           d_xexp);
     return hipGetLastError();
 }
 
@@ -274,10 +284,10 @@ static hipError_t launch_gemv_t(OxbGemvParams p, uint32_t S, uint32_t grid, hipS
 }
 
 hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {
-    // K slice per wave: NSBW superblocks; S <= 8 waves per workgroup.
-    uint32_t nsbw = (p.sb_count + 7u) / 8u;
-    if (nsbw < 1) nsbw = 1;
-    if (nsbw > 3) return hipErrorInvalidValue;  // caller splits K into chunks of OXB_GEMV_MAX_SB superblocks
+    // K slice per wave = one exponent group of the quantised input: NSBW superblocks; S <= 8 waves per workgroup.
+    const uint32_t nsbw = oxb_xq_gsb(p.n_sb);
+    p.n_groups = oxb_xq_groups(p.n_sb);
+    if (p.sb_count > 8 * nsbw || p.sb_begin % nsbw) return hipErrorInvalidValue;  // caller splits K into chunks of OXB_GEMV_MAX_SB superblocks
     const uint32_t S = (p.sb_count + nsbw - 1) / nsbw;
     if (p.n_tiles == 0) return hipSuccess;
     if (p.codes_bytes >= 0x7FFFFFFFull || p.xq_bytes >= 0x7FFFFFFFull) return hipErrorInvalidValue;

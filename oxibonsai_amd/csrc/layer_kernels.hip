@@ -46,6 +46,7 @@ __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const 
                                                                            float* __restrict__ normed_out) {
     extern __shared__ float lds_x[];  // [h]
     __shared__ float red[OXB_LAYER_THREADS / 64];
+    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
     const uint32_t n = blockIdx.x, tid = threadIdx.x;
     const float* xn = x + (size_t)n * h;
     float xv[EPT], wv[EPT];
@@ -69,12 +70,13 @@ __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const 
             if (normed_out && blockIdx.y == 0) normed_out[(size_t)n * h + i] = v;
         }
     }
-    __syncthreads();
-    // a NaN or infinity anywhere in x or w shows up in the sum of squares or in the bound
-    const float bound = w_absmax * sqrtf((float)h);
-    const bool any_bad = oxb_not_finite(ss) || oxb_not_finite(bound);
-    quantise_vector<FMT>(lds_x, h, oxb_nblk_pad(h), NC, n, ss > 0.f ? bound : 0.f, any_bad, xq, cneg, xexp, blockIdx.y,
-                         gridDim.y);
+    // this workgroup's exponent groups (a NaN or infinity anywhere in x shows up in every group through inv_rms)
+    const uint32_t n_sb = (h + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
+    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
+    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
+    if (g0 >= g1) return;
+    gstat_scan(lds_x, h, gsb, g0, g1, gstat);  // its first barrier publishes lds_x
+    quantise_groups<FMT>(lds_x, h, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
@@ -82,21 +84,23 @@ __global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const 
 // (crates/oxibonsai-kernels/src/simd_float_ops.rs:217-236; GPU twin swiglu_fused, cuda_kernels.rs:394-401).
 // gu = [gate: inter | up: inter] per vector.  Grid (vectors, parts), 1024 threads.
 // ---------------------------------------------------------------------------
-#define OXB_SWIGLU_THREADS 1024
+#define OXB_SWIGLU_THREADS 256
 template <int FMT>
 __global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const float* __restrict__ gu, uint32_t inter,
                                                                            uint32_t NC, uint32_t* __restrict__ xq,
                                                                            int32_t* __restrict__ cneg,
                                                                            int32_t* __restrict__ xexp) {
-    extern __shared__ float lds_x[];  // [inter]
-    __shared__ float red[OXB_SWIGLU_THREADS / 64];
-    __shared__ int bad_flag;
+    extern __shared__ float lds_x[];  // [inter]; a workgroup fills only the span of its exponent groups
+    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
     const uint32_t n = blockIdx.x, tid = threadIdx.x;
+    const uint32_t n_sb = (inter + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
+    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
+    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
+    if (g0 >= g1) return;
+    const uint32_t e0 = g0 * gsb * 512u, e1 = g1 * gsb * 512u < inter ? g1 * gsb * 512u : inter;
     const float* g = gu + (size_t)n * 2 * inter;
     const float* u = g + inter;
-    float mx = 0.f;
-    int bad = 0;
-    for (uint32_t i = tid * 4; i < inter; i += OXB_SWIGLU_THREADS * 4) {  // inter % 128 == 0
+    for (uint32_t i = e0 + tid * 4; i < e1; i += OXB_SWIGLU_THREADS * 4) {  // inter % 128 == 0
         const float4 g4 = *reinterpret_cast<const float4*>(g + i), u4 = *reinterpret_cast<const float4*>(u + i);
         float4 a;
         a.x = (g4.x / (1.0f + expf(-g4.x))) * u4.x;
@@ -104,12 +108,9 @@ __global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const 
         a.z = (g4.z / (1.0f + expf(-g4.z))) * u4.z;
         a.w = (g4.w / (1.0f + expf(-g4.w))) * u4.w;
         *reinterpret_cast<float4*>(lds_x + i) = a;
-        bad |= oxb_not_finite(a.x) | oxb_not_finite(a.y) | oxb_not_finite(a.z) | oxb_not_finite(a.w);
-        mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
     }
-    bool any_bad;
-    mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);
-    quantise_vector<FMT>(lds_x, inter, oxb_nblk_pad(inter), NC, n, mx, any_bad, xq, cneg, xexp, blockIdx.y, gridDim.y);
+    gstat_scan(lds_x, inter, gsb, g0, g1, gstat);  // its first barrier publishes lds_x
+    quantise_groups<FMT>(lds_x, inter, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
@@ -365,28 +366,35 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     }
 }
 
-// Merge the slot results of every q head of one sequence and quantise the attention output for the
-// O projection, in one workgroup (1024 threads): softmax weights of the slots per head (one wave per
-// head, one slot per lane), the weighted sum with four outputs per thread, then the activation quantiser.
-// Grid (vectors of the pass); sequence b0 + blockIdx.x becomes vector blockIdx.x of the quantised pass.
+// Merge the slot results of the q heads and quantise the attention output for the O projection.  Grid
+// (vectors of the pass, parts), 256 threads: a workgroup takes whole exponent groups of the output vector
+// (nq * hd values), i.e. a run of dimensions that it merges (softmax weights of the slots per head: one wave
+// per head, one slot per lane; then the weighted sum, four outputs per thread) and quantises on its own.
+// Sequence b0 + blockIdx.x becomes vector blockIdx.x of the quantised pass.
 template <int FMT>
-__global__ __launch_bounds__(1024) void attn_combine_quant_kernel(OxbAttnParams p, uint32_t b0, uint32_t NC,
-                                                                   uint32_t nblk_pad, uint32_t* __restrict__ xq,
-                                                                   int32_t* __restrict__ cneg, int32_t* __restrict__ xexp,
-                                                                   float* __restrict__ out_or_null) {
-    extern __shared__ float sm[];  // [qd] outputs | [nq][64] slot weights | [nq] 1 / sum
-    __shared__ float red[16];
-    __shared__ int bad_flag;
+__global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p, uint32_t b0, uint32_t NC,
+                                                                  uint32_t* __restrict__ xq, int32_t* __restrict__ cneg,
+                                                                  int32_t* __restrict__ xexp,
+                                                                  float* __restrict__ out_or_null) {
+    extern __shared__ float sm[];  // [span] outputs of this workgroup | [heads here][64] slot weights | [heads here] 1 / sum
+    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
     const uint32_t n = blockIdx.x, b = b0 + n, tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
+    const uint32_t n_sb = (qd + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
+    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
+    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
+    if (g0 >= g1) return;
+    const uint32_t e0 = g0 * gsb * 512u, e1 = g1 * gsb * 512u < qd ? g1 * gsb * 512u : qd;
+    const uint32_t h_first = e0 / hd, h_last = (e1 - 1) / hd, nh = h_last - h_first + 1;  // heads touched by the span
     const uint32_t stride = hd + OXB_ATTN_PART_PAD;
-    float* o = sm;
-    float* wts = sm + qd;
-    float* inv_l = wts + p.nq * 64;
+    const uint32_t span_pad = gsb * 512u * per;
+    float* o = sm;  // o[e - e0]
+    float* wts = sm + span_pad;
+    float* inv_l = wts + nh * 64;
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
     const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
-    for (uint32_t h = tid >> 6; h < p.nq; h += 16) {
-        const float* ph = part + ((size_t)h * p.n_splits + lane) * stride + hd;
+    for (uint32_t hh = tid >> 6; hh < nh; hh += 4) {
+        const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
         const float mv = lane < used ? ph[0] : -INFINITY, lv = lane < used ? ph[1] : 0.f;
         float M = mv;
 #pragma unroll
@@ -395,14 +403,12 @@ __global__ __launch_bounds__(1024) void attn_combine_quant_kernel(OxbAttnParams 
         float L = w * lv;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
-        wts[h * 64 + lane] = w;
-        if (lane == 0) inv_l[h] = L > 0.f ? 1.0f / L : 0.f;
+        wts[hh * 64 + lane] = w;
+        if (lane == 0) inv_l[hh] = L > 0.f ? 1.0f / L : 0.f;
     }
     __syncthreads();
-    float mx = 0.f;
-    int bad = 0;
-    for (uint32_t e = tid * 4; e < qd; e += 4096) {
-        const uint32_t h = e / hd, d = e % hd;
+    for (uint32_t e = e0 + tid * 4; e < e1; e += 1024) {
+        const uint32_t h = e / hd, d = e % hd, hh = h - h_first;
         const float* ph = part + (size_t)h * p.n_splits * stride + d;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
         uint32_t s = 0;
@@ -412,25 +418,23 @@ __global__ __launch_bounds__(1024) void attn_combine_quant_kernel(OxbAttnParams 
             for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(ph + (size_t)(s + u) * stride);
 #pragma unroll
             for (int u = 0; u < 4; u++) {
-                const float w = wts[h * 64 + s + u];
+                const float w = wts[hh * 64 + s + u];
                 acc.x = fmaf(v[u].x, w, acc.x), acc.y = fmaf(v[u].y, w, acc.y), acc.z = fmaf(v[u].z, w, acc.z), acc.w = fmaf(v[u].w, w, acc.w);
             }
         }
         for (; s < used; s++) {
             const float4 v = *reinterpret_cast<const float4*>(ph + (size_t)s * stride);
-            const float w = wts[h * 64 + s];
+            const float w = wts[hh * 64 + s];
             acc.x = fmaf(v.x, w, acc.x), acc.y = fmaf(v.y, w, acc.y), acc.z = fmaf(v.z, w, acc.z), acc.w = fmaf(v.w, w, acc.w);
         }
-        const float il = inv_l[h];
+        const float il = inv_l[hh];
         acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
-        *reinterpret_cast<float4*>(o + e) = acc;
+        *reinterpret_cast<float4*>(o + (e - e0)) = acc;
         if (out_or_null) *reinterpret_cast<float4*>(out_or_null + (size_t)b * qd + e) = acc;
-        bad |= oxb_not_finite(acc.x) | oxb_not_finite(acc.y) | oxb_not_finite(acc.z) | oxb_not_finite(acc.w);
-        mx = fmaxf(fmaxf(mx, fmaxf(fabsf(acc.x), fabsf(acc.y))), fmaxf(fabsf(acc.z), fabsf(acc.w)));
     }
-    bool any_bad;
-    mx = block_absmax(mx, bad, red, &bad_flag, &any_bad);  // its barriers also publish the outputs
-    quantise_vector<FMT>(o, qd, nblk_pad, NC, n, mx, any_bad, xq, cneg, xexp);
+    // the quantiser indexes the vector from its start: hand it the span shifted back by e0
+    gstat_scan(o - e0, qd, gsb, g0, g1, gstat);  // its first barrier publishes the outputs
+    quantise_groups<FMT>(o - e0, qd, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
@@ -483,7 +487,9 @@ static hipError_t launch_rmsnorm_fmt(const float* d_x, const float* d_w, float e
                                      uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed,
                                      hipStream_t st) {
     const size_t shm = (size_t)h * sizeof(float);
-    const dim3 grid(nb, oxb_quant_parts(h)), block(OXB_LAYER_THREADS);
+    const uint32_t n_groups = oxb_xq_groups((h + 511u) / 512u);
+    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
+    const dim3 grid(nb, n_groups < 8 ? n_groups : 8), block(OXB_LAYER_THREADS);
     const uint32_t ept = (h + OXB_LAYER_THREADS - 1) / OXB_LAYER_THREADS;
 #define OXB_RMS_CASE(E)                                                                                              \
     if (ept <= E) {                                                                                                  \
@@ -507,7 +513,9 @@ hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w,
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st) {
     const size_t shm = (size_t)inter * sizeof(float);
-    const dim3 grid(nb, oxb_quant_parts(inter)), block(OXB_SWIGLU_THREADS);
+    const uint32_t n_groups = oxb_xq_groups((inter + 511u) / 512u);
+    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
+    const dim3 grid(nb, n_groups < 16 ? n_groups : 16), block(OXB_SWIGLU_THREADS);
     if (fmt == OXB_FMT_Q1)
         hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, grid, block, shm, st, d_gu, inter, 8 * nb, d_xq, d_cneg, d_xexp);
     else
@@ -545,15 +553,19 @@ hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32
                                          int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st) {
     const uint32_t qd = p.nq * p.hd;
     if (nb == 0 || nb > 2 || (qd % OXB_QK) != 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
-    const size_t shm = ((size_t)qd + p.nq * 64 + p.nq) * sizeof(float);
+    const uint32_t n_sb = (qd + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
+    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
+    const uint32_t parts = n_groups < 16 ? n_groups : 16, per = (n_groups + parts - 1) / parts;
+    const uint32_t span = gsb * 512u * per, heads = span / p.hd + 2;
+    const size_t shm = ((size_t)span + heads * 65) * sizeof(float);
     if (shm > 60 * 1024) return hipErrorInvalidValue;
-    const uint32_t NC = OXB_XQ_DIGITS * nb, nblk_pad = oxb_nblk_pad(qd);
+    const uint32_t NC = OXB_XQ_DIGITS * nb;
     if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_Q1>, dim3(nb), dim3(1024), shm, st, p, b0, NC, nblk_pad, d_xq, d_cneg,
-                           d_xexp, d_out_or_null);
+        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_Q1>, dim3(nb, parts), dim3(256), shm, st, p, b0, NC, d_xq, d_cneg, d_xexp,
+                           d_out_or_null);
     else
-        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_TQ2>, dim3(nb), dim3(1024), shm, st, p, b0, NC, nblk_pad, d_xq, d_cneg,
-                           d_xexp, d_out_or_null);
+        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_TQ2>, dim3(nb, parts), dim3(256), shm, st, p, b0, NC, d_xq, d_cneg, d_xexp,
+                           d_out_or_null);
     return hipGetLastError();
 }
 

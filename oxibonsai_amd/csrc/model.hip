@@ -464,7 +464,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         (rc = dev_alloc(m, (void**)&m.v_cache, kv_elems * 2)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
-        (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + 256))) {
+        (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + OXB_XEXP_BYTES))) {
         free_model(m);
         return rc;
     }
@@ -605,7 +605,7 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     uint32_t kmax = h > inter ? h : inter;
     if (attn_k > kmax) kmax = attn_k;
     const size_t xq_b = oxb_xq_bytes(kmax, 1), cn_b = oxb_cneg_bytes(kmax, 1);
-    OXB_TRY(g_rt.ws_xq.ensure(xq_b + cn_b + 256));
+    OXB_TRY(g_rt.ws_xq.ensure(xq_b + cn_b + OXB_XEXP_BYTES));
     OXB_TRY(g_rt.ws_x.ensure(((size_t)h * 2 + attn_k) * 4));
     OXB_TRY(g_rt.ws_y.ensure((size_t)2 * inter * 4));
     XqBuf xb;

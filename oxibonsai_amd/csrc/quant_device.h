@@ -10,9 +10,12 @@
 //   cneg[blk][c][0..3]  four copies of -C, C = the part of the block sum that the biased
 //        encodings add (Q1: sum_k 2^j digit(r); TQ2: sum_{jj<3} 4^jj digit(r)), used as the
 //        MFMA accumulator's start value;
-//   xexp[n]  E - P, or INT_MIN when the vector holds a NaN or an infinity,
-// where 2^E > max|x| >= 2^(E-1) and P = 53: every element within 2^22 of the largest keeps all
-// 24 mantissa bits, so the integer block sums are exact for practical inputs.
+//   xexp[n][group]  E - P of the exponent group, or INT_MIN when the group holds a NaN or an infinity,
+// where 2^E > max|x| >= 2^(E-1) over the group and P = 53: every element within 2^22 of the group's
+// largest keeps all 24 mantissa bits, so the integer block sums are exact for practical inputs.
+// An exponent group is the K slice one GEMV wave owns (oxb_xq_gsb superblocks of 512 activations): its
+// exponent needs no information from the rest of the vector, so a producer of activations can quantise the
+// slice it has just computed, and the GEMV applies the exponent when it adds the waves' partial sums.
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -22,6 +25,8 @@
 
 #define OXB_XQ_P 53  // |x * 2^(P-E)| < 2^53, doubled values stay below 2^54
 #define OXB_XQ_DIGITS 8
+
+__host__ __device__ inline uint32_t oxb_nblk_pad(uint32_t k) { return ((k + 511u) / 512u) * 4u; }
 
 __device__ __forceinline__ int oxb_not_finite(float v) { return !(fabsf(v) <= 3.402823466e38f); }
 
@@ -117,6 +122,18 @@ __device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_
     for (int d = 0; d < 8; d++) dst[d] = make_uint4(out[d][0], out[d][1], out[d][2], out[d][3]);
 }
 
+// Superblocks per exponent group and groups per vector of n_sb superblocks: the K slice of one GEMV wave
+// (eight waves share up to 24 superblocks; longer vectors take several launches of 3-superblock slices).
+__host__ __device__ inline uint32_t oxb_xq_gsb(uint32_t n_sb) {
+    const uint32_t g = (n_sb + 7u) / 8u;
+    return g < 1 ? 1 : (g > 3 ? 3 : g);
+}
+__host__ __device__ inline uint32_t oxb_xq_groups(uint32_t n_sb) {
+    const uint32_t gsb = oxb_xq_gsb(n_sb);
+    return n_sb ? (n_sb + gsb - 1) / gsb : 1;
+}
+#define OXB_XQ_MAX_GROUPS 64  // vectors up to 64 * 3 * 512 = 98304 activations
+
 // Workgroup-wide maximum of |x| and a "not finite" flag; `red` holds blockDim.x / 64 floats.
 // Every thread gets the results.  Contains two barriers.
 __device__ __forceinline__ float block_absmax(float mx, int bad, float* red, int* bad_flag, bool* any_bad) {
@@ -134,27 +151,65 @@ __device__ __forceinline__ float block_absmax(float mx, int bad, float* red, int
     return mx;
 }
 
-// Quantise vector n (values at xn[0..k), any address space) given its absolute maximum.
-// All threads of the workgroup call it; blockDim.x must be a multiple of 64.  Workgroup
-// (part of parts) takes an equal share of the 64-unit groups, so several workgroups can split
-// one vector after each has found the same maximum.
+// Group statistics kept in LDS by a quantising workgroup: gstat[2 * i] = bit pattern of the largest |x| of
+// its i-th group (non-negative floats order like their bit patterns), gstat[2 * i + 1] = "not finite" flag.
+__device__ __forceinline__ void gstat_clear(uint32_t* gstat, uint32_t n_groups_here) {
+    for (uint32_t i = threadIdx.x; i < 2 * n_groups_here; i += blockDim.x) gstat[i] = 0;
+}
+// Every lane of a wave passes values of the same group (a wave covers 256 consecutive activations at a
+// 256-aligned index, and groups are multiples of 512).
+__device__ __forceinline__ void gstat_update_wave(uint32_t* gstat, uint32_t local_group, float mx, int bad) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        bad |= __shfl_xor(bad, o, 64);
+    }
+    if ((threadIdx.x & 63u) == 0) {
+        atomicMax(&gstat[2 * local_group], __float_as_uint(mx));
+        if (bad) atomicOr(&gstat[2 * local_group + 1], 1u);
+    }
+}
+
+// Maxima of groups [g_begin, g_end) of the values xn[0..k) (any address space) into gstat.  All threads of
+// the workgroup call it; blockDim.x is a multiple of 64.  Ends with a barrier.
+__device__ __forceinline__ void gstat_scan(const float* __restrict__ xn, uint32_t k, uint32_t gsb, uint32_t g_begin,
+                                           uint32_t g_end, uint32_t* gstat) {
+    gstat_clear(gstat, g_end - g_begin);
+    __syncthreads();
+    const uint32_t gel = gsb * 512u, e0 = g_begin * gel, e1 = g_end * gel < k ? g_end * gel : k;
+    for (uint32_t base = e0 + (threadIdx.x >> 6) * 256u; base < e1; base += (blockDim.x >> 6) * 256u) {
+        const uint32_t i = base + (threadIdx.x & 63u) * 4u;
+        float mx = 0.f;
+        int bad = 0;
+        if (i < e1) {  // k is a multiple of 128
+            const float4 v = *reinterpret_cast<const float4*>(xn + i);
+            bad = oxb_not_finite(v.x) | oxb_not_finite(v.y) | oxb_not_finite(v.z) | oxb_not_finite(v.w);
+            mx = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fabsf(v.z), fabsf(v.w)));
+        }
+        gstat_update_wave(gstat, base / gel - g_begin, mx, bad);
+    }
+    __syncthreads();
+}
+
+// Quantise groups [g_begin, g_end) of vector n (values at xn[0..k), any address space) given their statistics
+// in gstat (published by a barrier).  All threads of the workgroup call it.
 template <int FMT>
-__device__ __forceinline__ void quantise_vector(const float* __restrict__ xn, uint32_t k, uint32_t nblk_pad,
-                                                uint32_t NC, uint32_t n, float mx, bool any_bad,
-                                                uint32_t* __restrict__ xq, int32_t* __restrict__ cneg,
-                                                int32_t* __restrict__ xexp, uint32_t part = 0, uint32_t parts = 1) {
-    int E = 0;
-    if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
-    const int base_shift = OXB_XQ_P - E;
-    const uint32_t nblk = k / OXB_QK;
-    const bool ok = mx > 0.0f && !any_bad;
-    // unit u = (blk, m, g): eight consecutive lanes cover one block
-    const uint32_t n_units = nblk_pad * 8, per = (((n_units + 63) / 64 + parts - 1) / parts) * 64;  // n_units % 32 == 0
-    const uint32_t u_end = (part + 1) * per < n_units ? (part + 1) * per : n_units;
-    for (uint32_t u = part * per + threadIdx.x; u < u_end; u += blockDim.x) {
-        const uint32_t blk = u >> 3, m = (u >> 2) & 1u, g = u & 3u;
+__device__ __forceinline__ void quantise_groups(const float* __restrict__ xn, uint32_t k, uint32_t NC, uint32_t n,
+                                                uint32_t gsb, uint32_t n_groups, uint32_t g_begin, uint32_t g_end,
+                                                const uint32_t* gstat, uint32_t* __restrict__ xq,
+                                                int32_t* __restrict__ cneg, int32_t* __restrict__ xexp) {
+    const uint32_t nblk = k / OXB_QK, nblk_pad = oxb_nblk_pad(k);
+    // unit u = (blk, m, g): eight consecutive lanes cover one block; a group holds gsb * 32 units
+    const uint32_t upg = gsb * 32u, u0 = g_begin * upg;
+    const uint32_t u1 = g_end * upg < nblk_pad * 8u ? g_end * upg : nblk_pad * 8u;
+    for (uint32_t u = u0 + threadIdx.x; u < u1; u += blockDim.x) {
+        const uint32_t blk = u >> 3, m = (u >> 2) & 1u, g = u & 3u, lg = u / upg - g_begin;
+        const float mx = __uint_as_float(gstat[2 * lg]);
+        const bool ok = mx > 0.0f && gstat[2 * lg + 1] == 0;
+        int E = 0;
+        if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
         int cs[8];
-        quant_unit<FMT>(xn, blk, m, g, base_shift, ok && blk < nblk, NC, n, xq, cs);
+        quant_unit<FMT>(xn, blk, m, g, OXB_XQ_P - E, ok && blk < nblk, NC, n, xq, cs);
         // sum the correction over the block's eight lanes: i <-> 7-i, then within quads
 #pragma unroll
         for (int d = 0; d < 8; d++) {
@@ -170,13 +225,11 @@ __device__ __forceinline__ void quantise_vector(const float* __restrict__ xn, ui
         for (int d = 1; d < 8; d++) mine = ((u & 7u) == (uint32_t)d) ? cs[d] : mine;
         *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + (u & 7u)) * 4) = make_int4(-mine, -mine, -mine, -mine);
     }
-    if (threadIdx.x == 0 && part == 0) xexp[n] = any_bad ? INT32_MIN : (mx > 0.0f ? E - OXB_XQ_P : 0);
+    for (uint32_t gi = g_begin + threadIdx.x; gi < g_end; gi += blockDim.x) {
+        const float mx = __uint_as_float(gstat[2 * (gi - g_begin)]);
+        int E = 0;
+        if (mx > 0.0f) (void)frexpf(mx, &E);
+        xexp[n * n_groups + gi] = gstat[2 * (gi - g_begin) + 1] ? INT32_MIN : (mx > 0.0f ? E - OXB_XQ_P : 0);
+    }
 }
 
-// Workgroups that share one vector: one per 64 units (1024 activations), at most 16.
-__host__ __device__ inline uint32_t oxb_quant_parts(uint32_t k) {
-    const uint32_t p = (((k + 511u) / 512u) * 32u + 63u) / 64u;
-    return p < 1 ? 1 : (p > 16 ? 16 : p);
-}
-
-__host__ __device__ inline uint32_t oxb_nblk_pad(uint32_t k) { return ((k + 511u) / 512u) * 4u; }

@@ -124,7 +124,7 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
         int rc;
         if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
         if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-        if ((rc = g_rt.ws_xexp.ensure(16 * sizeof(int32_t)))) return rc;
+        if ((rc = g_rt.ws_xexp.ensure(OXB_XEXP_BYTES))) return rc;
         hipError_t e = oxb_launch_quant_x((int)w.L.fmt, d_x + (size_t)b0 * k, k, nb, (uint32_t*)g_rt.ws_xq.ptr,
                                           (int32_t*)g_rt.ws_cneg.ptr, (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
         if (e != hipSuccess) return hip_fail(e, "kernel launch failed: quant_x");
@@ -386,7 +386,7 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
     int rc;
     if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
     if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-    if ((rc = g_rt.ws_xexp.ensure(16 * sizeof(int32_t)))) return rc;
+    if ((rc = g_rt.ws_xexp.ensure(OXB_XEXP_BYTES))) return rc;
     const int fmt = (int)ws[0]->L.fmt;
     hipError_t e = oxb_launch_quant_x(fmt, d_x, k, 1, (uint32_t*)g_rt.ws_xq.ptr, (int32_t*)g_rt.ws_cneg.ptr,
                                       (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
