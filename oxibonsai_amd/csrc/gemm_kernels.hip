@@ -32,61 +32,101 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 #define OXB_GEMM_THREADS 256
 
 // ---------------------------------------------------------------------------
-// Activation packer.  One workgroup = 16 token rows; grid.y workgroups share the blocks of those rows.
+// Activation packer, fused with the row-wise producer of the activations:
+//   OXB_PACK_IDENT   a[m][k] = x[m][k]
+//   OXB_PACK_RMSNORM a[m][k] = w[k] * x[m][k] / sqrt(mean_k x[m][k]^2 + eps)      (simd_float_ops.rs:204-215)
+//   OXB_PACK_SWIGLU  a[m][k] = silu(x[m][k]) * x[m][k + K],  x = [gate | up]        (simd_float_ops.rs:217-236)
+// Two kernels: row_stats (one workgroup per token row) finds the row's multiplier - the producer's scalar
+// times the power of two that puts the row's largest |a| into [2^14, 2^15) - and the exponent that undoes the
+// power of two; xh_pack (one workgroup = 16 token rows x a share of the blocks) recomputes a from x and writes
+// fp16 in MFMA B-operand order.  The fp32 activations never go to memory.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     const v2h h = {(_Float16)a, (_Float16)b};
     return __builtin_bit_cast(uint32_t, h);
 }
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 
-template <int FMT>
-__global__ __launch_bounds__(256) void xh_pack_kernel(const float* __restrict__ x, uint32_t ldx, uint32_t k, uint32_t M,
-                                                       uint32_t M_pad, uint32_t nblk_pad, uint4* __restrict__ xh,
-                                                       int32_t* __restrict__ xsh) {
-    __shared__ int sh_shift[16];
-    const uint32_t tid = threadIdx.x, m0 = blockIdx.x * 16;
-    {  // row maxima: 16 lanes per row
-        const uint32_t j = tid >> 4, i = tid & 15u, m = m0 + j;
-        float mx = 0.0f;
-        int bad = 0;
-        if (m < M) {
-            const float* xr = x + (size_t)m * ldx;
-            for (uint32_t kk = i * 4; kk < k; kk += 64) {
-                const float4 v = *reinterpret_cast<const float4*>(xr + kk);
-                bad |= !(fabsf(v.x) <= 3.402823466e38f) | !(fabsf(v.y) <= 3.402823466e38f) |
-                       !(fabsf(v.z) <= 3.402823466e38f) | !(fabsf(v.w) <= 3.402823466e38f);
-                mx = fmaxf(fmaxf(mx, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
-            }
+template <int OP>
+__global__ __launch_bounds__(256) void row_stats_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                         uint32_t ldx, uint32_t k, float eps, float* __restrict__ rowmul,
+                                                         int32_t* __restrict__ xsh) {
+    __shared__ float red_s[4], red_m[4];
+    __shared__ int red_b[4];
+    const uint32_t m = blockIdx.x, tid = threadIdx.x;
+    const float* xr = x + (size_t)m * ldx;
+    float ss = 0.f, mx = 0.f;
+    int bad = 0;
+    for (uint32_t i = tid * 4; i < k; i += 1024) {
+        const float4 v = *reinterpret_cast<const float4*>(xr + i);
+        float4 a = v;
+        if (OP == OXB_PACK_RMSNORM) {
+            const float4 g = *reinterpret_cast<const float4*>(w + i);
+            ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
+            a = make_float4(g.x * v.x, g.y * v.y, g.z * v.z, g.w * v.w);
+        } else if (OP == OXB_PACK_SWIGLU) {
+            const float4 u = *reinterpret_cast<const float4*>(xr + k + i);
+            a = make_float4(silu_mul(v.x, u.x), silu_mul(v.y, u.y), silu_mul(v.z, u.z), silu_mul(v.w, u.w));
         }
-#pragma unroll
-        for (int o = 8; o > 0; o >>= 1) {
-            mx = fmaxf(mx, __shfl_xor(mx, o, 16));
-            bad |= __shfl_xor(bad, o, 16);
-        }
-        if (i == 0) {
-            int E = 0;
-            if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
-            const int shift = mx > 0.0f ? 15 - E : 0;
-            sh_shift[j] = bad ? INT32_MIN : shift;
-            if (blockIdx.y == 0 && m < M) xsh[m] = bad ? INT32_MIN : -shift;
-        }
+        bad |= !(fabsf(a.x) <= 3.402823466e38f) | !(fabsf(a.y) <= 3.402823466e38f) | !(fabsf(a.z) <= 3.402823466e38f) |
+               !(fabsf(a.w) <= 3.402823466e38f);
+        mx = fmaxf(fmaxf(mx, fmaxf(fabsf(a.x), fabsf(a.y))), fmaxf(fabsf(a.z), fabsf(a.w)));
     }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        ss += __shfl_xor(ss, o, 64);
+        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+        bad |= __shfl_xor(bad, o, 64);
+    }
+    if ((tid & 63u) == 0) red_s[tid >> 6] = ss, red_m[tid >> 6] = mx, red_b[tid >> 6] = bad;
     __syncthreads();
+    if (tid == 0) {
+        ss = red_s[0] + red_s[1] + red_s[2] + red_s[3];
+        mx = fmaxf(fmaxf(red_m[0], red_m[1]), fmaxf(red_m[2], red_m[3]));
+        bad = red_b[0] | red_b[1] | red_b[2] | red_b[3];
+        float scalar = 1.0f;
+        if (OP == OXB_PACK_RMSNORM) {
+            scalar = 1.0f / sqrtf(ss / (float)k + eps);
+            mx *= scalar;
+            bad |= !(fabsf(scalar) <= 3.402823466e38f) | !(fabsf(mx) <= 3.402823466e38f);
+        }
+        int E = 0;
+        if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
+        const int shift = mx > 0.0f ? 15 - E : 0;
+        rowmul[m] = bad ? 0.0f : ldexpf(scalar, shift);
+        xsh[m] = bad ? INT32_MIN : -shift;
+    }
+}
+
+template <int FMT, int OP>
+__global__ __launch_bounds__(256) void xh_pack_kernel(const float* __restrict__ x, const float* __restrict__ w, uint32_t ldx,
+                                                       uint32_t k, uint32_t M, uint32_t M_pad, uint32_t nblk_pad,
+                                                       const float* __restrict__ rowmul, uint4* __restrict__ xh) {
+    const uint32_t tid = threadIdx.x, m0 = blockIdx.x * 16;
     const uint32_t j = tid & 15u, c = tid >> 4, g = c >> 2, s = c & 3u, m = m0 + j;
-    const int shift = sh_shift[j];
-    const bool live = m < M && shift != INT32_MIN;
+    const bool live = m < M;
+    const float mul = live ? rowmul[m] : 0.0f;
     const uint32_t k0 = FMT == OXB_FMT_Q1 ? 32 * g + 4 * s : 32 * g + 16 * (s >> 1) + 4 * (s & 1u);
     const uint32_t k1 = k0 + (FMT == OXB_FMT_Q1 ? 16 : 8);
     for (uint32_t blk = blockIdx.y; blk < nblk_pad; blk += gridDim.y) {
         uint4 o = make_uint4(0, 0, 0, 0);
         if (live && blk * 128 < k) {
             const float* xb = x + (size_t)m * ldx + blk * 128;
-            const float4 a = *reinterpret_cast<const float4*>(xb + k0);
-            const float4 b = *reinterpret_cast<const float4*>(xb + k1);
-            o.x = pack_h2(ldexpf(a.x, shift), ldexpf(b.x, shift));
-            o.y = pack_h2(ldexpf(a.y, shift), ldexpf(b.y, shift));
-            o.z = pack_h2(ldexpf(a.z, shift), ldexpf(b.z, shift));
-            o.w = pack_h2(ldexpf(a.w, shift), ldexpf(b.w, shift));
+            float4 a = *reinterpret_cast<const float4*>(xb + k0);
+            float4 b = *reinterpret_cast<const float4*>(xb + k1);
+            if (OP == OXB_PACK_RMSNORM) {
+                const float4 wa = *reinterpret_cast<const float4*>(w + blk * 128 + k0), wb = *reinterpret_cast<const float4*>(w + blk * 128 + k1);
+                a = make_float4(wa.x * a.x, wa.y * a.y, wa.z * a.z, wa.w * a.w);
+                b = make_float4(wb.x * b.x, wb.y * b.y, wb.z * b.z, wb.w * b.w);
+            } else if (OP == OXB_PACK_SWIGLU) {
+                const float4 ua = *reinterpret_cast<const float4*>(xb + k + k0), ub = *reinterpret_cast<const float4*>(xb + k + k1);
+                a = make_float4(silu_mul(a.x, ua.x), silu_mul(a.y, ua.y), silu_mul(a.z, ua.z), silu_mul(a.w, ua.w));
+                b = make_float4(silu_mul(b.x, ub.x), silu_mul(b.y, ub.y), silu_mul(b.z, ub.z), silu_mul(b.w, ub.w));
+            }
+            o.x = pack_h2(a.x * mul, b.x * mul);
+            o.y = pack_h2(a.y * mul, b.y * mul);
+            o.z = pack_h2(a.z * mul, b.z * mul);
+            o.w = pack_h2(a.w * mul, b.w * mul);
         }
         xh[(size_t)(blk * 16 + c) * M_pad + m] = o;
     }
@@ -388,19 +428,31 @@ size_t oxb_xh_bytes(uint32_t k, uint32_t M) {
     return nblk_pad * 16 * M_pad * 16;
 }
 
-hipError_t oxb_launch_xh_pack(int fmt, const float* d_x, uint32_t ldx, uint32_t k, uint32_t M, uint32_t* d_xh,
-                              int32_t* d_xsh, hipStream_t st) {
+template <int OP>
+static void launch_pack_op(int fmt, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, uint32_t M, uint32_t M_pad,
+                           uint32_t nblk_pad, float eps, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st) {
+    hipLaunchKernelGGL(row_stats_kernel<OP>, dim3(M), dim3(256), 0, st, d_x, d_w, ldx, k, eps, d_rowmul, d_xsh);
+    const dim3 grid(M_pad / 16, nblk_pad < 16 ? nblk_pad : 16);
+    if (fmt == OXB_FMT_Q1)
+        hipLaunchKernelGGL((xh_pack_kernel<OXB_FMT_Q1, OP>), grid, dim3(256), 0, st, d_x, d_w, ldx, k, M, M_pad, nblk_pad, d_rowmul,
+                           reinterpret_cast<uint4*>(d_xh));
+    else
+        hipLaunchKernelGGL((xh_pack_kernel<OXB_FMT_TQ2, OP>), grid, dim3(256), 0, st, d_x, d_w, ldx, k, M, M_pad, nblk_pad, d_rowmul,
+                           reinterpret_cast<uint4*>(d_xh));
+}
+
+hipError_t oxb_launch_xh_pack(int fmt, int op, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, float eps,
+                              uint32_t M, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st) {
     if (M == 0 || k == 0 || (k % OXB_QK) != 0 || (ldx & 3u) != 0) return hipErrorInvalidValue;
+    if (op == OXB_PACK_RMSNORM && !d_w) return hipErrorInvalidValue;
     const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, M_pad = (M + 15u) / 16u * 16u;
     if (oxb_xh_bytes(k, M) >= 0xFFFFFFF0ull) return hipErrorInvalidValue;
-    uint32_t split = nblk_pad < 16 ? nblk_pad : 16;
-    const dim3 grid(M_pad / 16, split);
-    if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(xh_pack_kernel<OXB_FMT_Q1>, grid, dim3(256), 0, st, d_x, ldx, k, M, M_pad, nblk_pad,
-                           reinterpret_cast<uint4*>(d_xh), d_xsh);
-    else
-        hipLaunchKernelGGL(xh_pack_kernel<OXB_FMT_TQ2>, grid, dim3(256), 0, st, d_x, ldx, k, M, M_pad, nblk_pad,
-                           reinterpret_cast<uint4*>(d_xh), d_xsh);
+    switch (op) {
+        case OXB_PACK_IDENT: launch_pack_op<OXB_PACK_IDENT>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
+        case OXB_PACK_RMSNORM: launch_pack_op<OXB_PACK_RMSNORM>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
+        case OXB_PACK_SWIGLU: launch_pack_op<OXB_PACK_SWIGLU>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
+        default: return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

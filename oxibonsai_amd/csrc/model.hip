@@ -54,8 +54,7 @@ struct Model {
     std::vector<void*> allocs;
     // prefill activations for up to pf_cap token rows (allocated on first use)
     uint32_t pf_cap = 0;
-    float *pf_hidden = nullptr, *pf_normed = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr,
-          *pf_gu = nullptr, *pf_act = nullptr;
+    float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
     std::vector<void*> pf_allocs;
 };
 
@@ -272,9 +271,8 @@ static int ensure_prefill_buffers(Model& m, uint32_t rows) {
     m.pf_cap = 0;
     const oxb_model_desc& d = m.d;
     const size_t R = (rows + 127u) / 128u * 128u, qd = (size_t)d.nq * d.hd, qkv_rows = qd + 2 * (size_t)d.nkv * d.hd;
-    struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_normed, R * d.h}, {&m.pf_qkv, R * qkv_rows},
-                                             {&m.pf_q, R * qd},       {&m.pf_attn, R * qd},    {&m.pf_gu, R * 2 * d.inter},
-                                             {&m.pf_act, R * d.inter}};
+    struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_qkv, R * qkv_rows}, {&m.pf_q, R * qd},
+                                             {&m.pf_attn, R * qd},    {&m.pf_gu, R * 2 * d.inter}};
     for (auto& b : bufs) {
         if (hipMalloc((void**)b.p, b.n * sizeof(float)) != hipSuccess) {
             for (void* p : m.pf_allocs) (void)hipFree(p);
@@ -288,7 +286,7 @@ static int ensure_prefill_buffers(Model& m, uint32_t rows) {
 }
 
 // All layers for M token rows of sequence `seq` at positions pos_start .. pos_start + M - 1: batched
-// projections on the matrix cores, one causal attention launch per layer, KV written to the cache; then the
+// projections on the matrix cores (RMSNorm and SwiGLU fused into the fp16 packer of the GEMM that consumes them), one causal attention launch per layer, KV written to the cache; then the
 // LM head and the greedy token for the last row.
 static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start) {
     const oxb_model_desc& d = m.d;
@@ -306,8 +304,7 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
         const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
         if (rc) return rc;
-        OXB_TRY_HIP(oxb_launch_rmsnorm_rows(m.pf_hidden, attn_norm, d.eps, d.h, M, m.pf_normed, st), "kernel launch failed: rmsnorm_rows");
-        OXB_TRY(gemm_device(*wqkv, m.pf_normed, d.h, m.pf_qkv, M, qkv_rows, OXB_GEMM_STORE, nullptr));
+        OXB_TRY(gemm_device(*wqkv, m.pf_hidden, d.h, m.pf_qkv, M, qkv_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, attn_norm, d.eps));
         OxbQkParams qp;
         qp.qkv = m.pf_qkv;
         qp.qkv_stride = qkv_rows;
@@ -343,11 +340,9 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         ap.max_seq = d.max_seq;
         ap.scale = 1.0f / sqrtf((float)d.hd);
         OXB_TRY_HIP(oxb_launch_attn_prefill(ap, st), "kernel launch failed: attn_prefill");
-        OXB_TRY(gemm_device(*wo, m.pf_attn, qd, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden));
-        OXB_TRY_HIP(oxb_launch_rmsnorm_rows(m.pf_hidden, ffn_norm, d.eps, d.h, M, m.pf_normed, st), "kernel launch failed: rmsnorm_rows");
-        OXB_TRY(gemm_device(*wgu, m.pf_normed, d.h, m.pf_gu, M, 2 * d.inter, OXB_GEMM_STORE, nullptr));
-        OXB_TRY_HIP(oxb_launch_swiglu_rows(m.pf_gu, d.inter, M, m.pf_act, st), "kernel launch failed: swiglu_rows");
-        OXB_TRY(gemm_device(*wdn, m.pf_act, d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden));
+        OXB_TRY(gemm_device(*wo, m.pf_attn, qd, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_IDENT, nullptr, 0.f));
+        OXB_TRY(gemm_device(*wgu, m.pf_hidden, d.h, m.pf_gu, M, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps));
+        OXB_TRY(gemm_device(*wdn, m.pf_gu, 2 * d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_SWIGLU, nullptr, 0.f));
     }
     // last token: final norm, LM head, greedy token (fp32-exact products, as in a decode step)
     const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);

@@ -1,4 +1,4 @@
-// prefill_kernels.h — launch interface of the token-batched prefill glue (see prefill_kernels.hip).
+// prefill_kernels.h — launch interface of the prefill attention (see prefill_kernels.hip).
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
@@ -13,7 +13,4 @@ struct OxbPrefillAttnParams {
     float scale;                      // 1 / sqrt(hd)
 };
 
-hipError_t oxb_launch_rmsnorm_rows(const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t M, float* d_out,
-                                   hipStream_t st);
-hipError_t oxb_launch_swiglu_rows(const float* d_gu, uint32_t inter, uint32_t M, float* d_act, hipStream_t st);
 hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st);

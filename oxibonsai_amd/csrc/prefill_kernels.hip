@@ -1,5 +1,5 @@
-// prefill_kernels.hip — the token-batched glue of the prefill pipeline: row-wise RMSNorm and SwiGLU over
-// M token rows and a causal attention over the FP16 KV cache on the matrix cores.
+// prefill_kernels.hip — causal attention of the prefill pipeline over the FP16 KV cache on the matrix cores
+// (the row-wise RMSNorm and SwiGLU of the pipeline live in the GEMM's activation packer, gemm_kernels.hip).
 //
 // The reference's prefill (gpu_backend/cuda_prefill/encode_q1.rs:123-300, encode_ternary.rs:114-314) batches
 // the projections but walks the tokens one by one through its decode attention kernels
@@ -12,54 +12,6 @@
 #include "prefill_kernels.h"
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-
-__device__ __forceinline__ float block_sum_256(float v, float* red) {  // two barriers; red: 4 floats
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    const float s = red[0] + red[1] + red[2] + red[3];
-    __syncthreads();
-    return s;
-}
-
-// out[m][i] = w[i] * x[m][i] / sqrt(mean_i(x[m][i]^2) + eps)
-// (rms_norm: crates/oxibonsai-kernels/src/simd_float_ops.rs:204-215; GPU twin batched_rmsnorm_v2,
-//  gpu_backend/cuda_prefill_kernels.rs:373-424).  One workgroup per token row.
-__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                            float eps, uint32_t h, float* __restrict__ out) {
-    __shared__ float red[4];
-    const float* xr = x + (size_t)blockIdx.x * h;
-    float* orow = out + (size_t)blockIdx.x * h;
-    float ss = 0.f;
-    for (uint32_t i = threadIdx.x * 4; i < h; i += 1024) {
-        const float4 v = *reinterpret_cast<const float4*>(xr + i);
-        ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
-    }
-    ss = block_sum_256(ss, red);
-    const float inv_rms = 1.0f / sqrtf(ss / (float)h + eps);
-    for (uint32_t i = threadIdx.x * 4; i < h; i += 1024) {
-        const float4 v = *reinterpret_cast<const float4*>(xr + i);
-        const float4 g = *reinterpret_cast<const float4*>(w + i);
-        *reinterpret_cast<float4*>(orow + i) = make_float4(g.x * v.x * inv_rms, g.y * v.y * inv_rms, g.z * v.z * inv_rms, g.w * v.w * inv_rms);
-    }
-}
-
-// act[m][i] = silu(gate[m][i]) * up[m][i], gu[m] = [gate: inter | up: inter]
-// (simd_float_ops.rs:217-236; GPU twin batched_swiglu, cuda_prefill_kernels.rs:341-354).
-__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float* __restrict__ gu, uint32_t inter,
-                                                           float* __restrict__ act) {
-    const uint32_t i = (blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= inter) return;
-    const float* g = gu + (size_t)blockIdx.y * 2 * inter;
-    const float4 g4 = *reinterpret_cast<const float4*>(g + i), u4 = *reinterpret_cast<const float4*>(g + inter + i);
-    float4 a;
-    a.x = (g4.x / (1.0f + expf(-g4.x))) * u4.x;
-    a.y = (g4.y / (1.0f + expf(-g4.y))) * u4.y;
-    a.z = (g4.z / (1.0f + expf(-g4.z))) * u4.z;
-    a.w = (g4.w / (1.0f + expf(-g4.w))) * u4.w;
-    *reinterpret_cast<float4*>(act + (size_t)blockIdx.y * inter + i) = a;
-}
 
 // ---------------------------------------------------------------------------
 // Causal attention of M query tokens (positions pos_start .. pos_start + M - 1) over keys 0 .. own position
@@ -174,19 +126,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         for (int sl = 0; sl < NS; sl++)
             *reinterpret_cast<float4*>(o + 16 * sl) = make_float4(O[sl][0] * inv, O[sl][1] * inv, O[sl][2] * inv, O[sl][3] * inv);
     }
-}
-
-hipError_t oxb_launch_rmsnorm_rows(const float* d_x, const float* d_w, float eps, uint32_t h, uint32_t M, float* d_out,
-                                   hipStream_t st) {
-    if (M == 0 || (h & 3u)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(rmsnorm_rows_kernel, dim3(M), dim3(256), 0, st, d_x, d_w, eps, h, d_out);
-    return hipGetLastError();
-}
-
-hipError_t oxb_launch_swiglu_rows(const float* d_gu, uint32_t inter, uint32_t M, float* d_act, hipStream_t st) {
-    if (M == 0 || (inter & 3u)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(swiglu_rows_kernel, dim3((inter + 1023) / 1024, M), dim3(256), 0, st, d_gu, inter, d_act);
-    return hipGetLastError();
 }
 
 hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st) {

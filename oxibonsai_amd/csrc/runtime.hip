@@ -158,15 +158,16 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
 }
 
 int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
-                const float* d_residual) {
+                const float* d_residual, int pack_op, const float* d_pack_w, float eps) {
     const uint32_t k = w.L.k;
     if ((uint64_t)m * k >= (1ull << 31))
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u rows of %u activations exceed one GEMM call", m, k);
     int rc;
     if ((rc = g_rt.ws_xh.ensure(oxb_xh_bytes(k, m)))) return rc;
     if ((rc = g_rt.ws_xsh.ensure(((size_t)m + 16) * sizeof(int32_t)))) return rc;
-    hipError_t e = oxb_launch_xh_pack((int)w.L.fmt, d_x, ldx, k, m, (uint32_t*)g_rt.ws_xh.ptr, (int32_t*)g_rt.ws_xsh.ptr,
-                                      g_rt.stream);
+    if ((rc = g_rt.ws_rowmul.ensure(((size_t)m + 16) * sizeof(float)))) return rc;
+    hipError_t e = oxb_launch_xh_pack((int)w.L.fmt, pack_op, d_x, d_pack_w, ldx, k, eps, m, (float*)g_rt.ws_rowmul.ptr,
+                                      (uint32_t*)g_rt.ws_xh.ptr, (int32_t*)g_rt.ws_xsh.ptr, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch failed: xh_pack");
     OxbGemmParams p;
     memset(&p, 0, sizeof p);
@@ -277,6 +278,7 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_xexp.release();
     g_rt.ws_xh.release();
     g_rt.ws_xsh.release();
+    g_rt.ws_rowmul.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.own_stream = nullptr;
     g_rt.stream = nullptr;
@@ -443,7 +445,7 @@ int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint
     int rc = check_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
-    return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr);
+    return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f);
 }
 
 int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_rows, uint32_t k) {
@@ -458,7 +460,7 @@ int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_r
     if ((rc = g_rt.ws_y.ensure(yb))) return rc;
     hipError_t e = hipMemcpyAsync(g_rt.ws_x.ptr, x, xb, hipMemcpyHostToDevice, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "input upload");
-    rc = gemm_device(*w, (const float*)g_rt.ws_x.ptr, k, (float*)g_rt.ws_y.ptr, m, n_rows, OXB_GEMM_STORE, nullptr);
+    rc = gemm_device(*w, (const float*)g_rt.ws_x.ptr, k, (float*)g_rt.ws_y.ptr, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f);
     if (rc) return rc;
     e = hipMemcpyAsync(y, g_rt.ws_y.ptr, yb, hipMemcpyDeviceToHost, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "output download");
@@ -474,7 +476,7 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     if (rc) return rc;
     if (!d_x || !d_y || !avg_us || m == 0 || iters == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
-    if ((rc = gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr))) return rc;  // packs x, warms up
+    if ((rc = gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f))) return rc;  // packs x, warms up
     OxbGemmParams p;
     memset(&p, 0, sizeof p);
     p.codes = w->d_codes;

@@ -40,7 +40,7 @@ struct Runtime {
     std::unordered_map<uint64_t, Vector> vectors;
     uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
-    DevBuf ws_xh, ws_xsh;  // prefill GEMM: packed fp16 activations and per-row exponents
+    DevBuf ws_xh, ws_xsh, ws_rowmul;  // prefill GEMM: packed fp16 activations, per-row exponents and multipliers
 };
 
 extern Runtime g_rt;
@@ -53,9 +53,10 @@ Weight* find_weight(uint64_t id);
 int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual);
-// x (device, [m][ldx]) -> y (device, [m][ldy]) through the fp16 packer + MFMA GEMM.
+// x (device, [m][ldx]) -> y (device, [m][ldy]) through the fp16 packer + MFMA GEMM.  pack_op (OXB_PACK_*) names the
+// row-wise producer fused into the packer: RMSNorm with weights d_pack_w and eps, or SwiGLU of x = [gate | up].
 int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
-                const float* d_residual);
+                const float* d_residual, int pack_op, const float* d_pack_w, float eps);
 void shutdown_models();
 
 }  // namespace oxb
