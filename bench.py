@@ -34,6 +34,7 @@ HBM_PEAK_GBPS = 8000.0
 GATE_UP_HBM_TRAFFIC_BYTES = 14_617_600
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
+FMT_TQ2 = 1
 
 
 def algorithmic_bytes(n_rows: int, k: int, batch: int = 1, block_bytes: int = 18) -> int:
@@ -143,6 +144,38 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool) -> dict:
     return res
 
 
+PREFILL_SHAPES = [("qkv", 5120, 2560), ("gate_up", 19456, 2560), ("down", 2560, 9728)]   # BASELINE.json configs[2]
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def prefill_gemm_leg(be, L, torch, m_tokens: int = 512) -> dict:
+    """TQ2_0_g128 prefill GEMM at Qwen3-4B shapes, M = 512 tokens: the GEMM kernel alone (activations already
+    packed to fp16), timed with HIP events on the library's stream; 2 * M * N * K flops per launch."""
+    from oxibonsai_amd import _lib, synth
+    res = {"workload": f"TQ2_0_g128 prefill GEMM, Qwen3-4B shapes, M = {m_tokens}", "dtype": "fp16 MFMA, fp32 accumulate",
+           "peak_TFLOPs": MFMA_F16_PEAK_TFLOPS, "per_kernel": {}}
+    total_flop = total_us = 0.0
+    for i, (name, n, k) in enumerate(PREFILL_SHAPES):
+        a = synth.make_blocks(FMT_TQ2, 0xB0A5A10200 + i, n, k)
+        h = be.upload_weights_ternary(a, n, k)
+        x = torch.randn(m_tokens, k, device="cuda", dtype=torch.float32)
+        y = torch.empty(m_tokens, n, device="cuda", dtype=torch.float32)
+        torch.cuda.synchronize()
+        us = C.c_float(0.0)
+        rc = L.oxb_hip_profile_gemm(int(h), x.data_ptr(), y.data_ptr(), m_tokens, n, k, 5, 50, C.byref(us))
+        be.free_weights(h)
+        if rc:
+            raise RuntimeError(_lib.last_error())
+        flop = 2.0 * m_tokens * n * k
+        total_flop += flop
+        total_us += us.value
+        res["per_kernel"][name] = {"us": round(us.value, 2), "TFLOPs": round(flop / us.value * 1e-6, 1),
+                                   "frac_of_mfma_peak": round(flop / us.value * 1e-6 / MFMA_F16_PEAK_TFLOPS, 4)}
+    res["TFLOPs"] = round(total_flop / total_us * 1e-6, 1)
+    res["frac_of_mfma_peak"] = round(total_flop / total_us * 1e-6 / MFMA_F16_PEAK_TFLOPS, 4)
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -151,6 +184,7 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=24, help="distinct resident copies of the weight set")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the 8B-shape decode leg")
+    ap.add_argument("--no-prefill-gemm", action="store_true", help="skip the prefill GEMM leg")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel that hardware-counter runs are scaled by")
     ap.add_argument("--decode-context", type=int, default=2048)
@@ -283,6 +317,8 @@ def main() -> int:
         for _ in range(3):
             dst.copy_(src)
         torch.cuda.synchronize()
+    if not args.no_prefill_gemm:
+        out["prefill_gemm"] = prefill_gemm_leg(be, L, torch)
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu)
     print(json.dumps(out), flush=True)
