@@ -16,7 +16,8 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // ---------------------------------------------------------------------------
 // Causal attention of M query tokens (positions pos_start .. pos_start + M - 1) over keys 0 .. own position
 // of one sequence, GQA, online softmax (semantics: block/functions.rs:78-127 -> layers/attention_fused.rs:329-400
-// applied per token).  One wave = 16 queries of one q head; no LDS, no barriers.
+// applied per token).  One wave = 16 queries of one q head, working on its own: no barriers; the wave stages
+// each 32-key V block in its private slice of LDS, from where the transposed operand is gathered.
 //
 // Both products run on v_mfma_f32_16x16x32_f16 in transposed form, so the score tile comes out with the
 // query in the lane (column) and needs no transposition before the second product:
@@ -29,10 +30,14 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // ---------------------------------------------------------------------------
 template <int HD>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams p) {
-    constexpr int KS = HD / 32;   // MFMA k-steps over the head dimension
-    constexpr int NS = HD / 16;   // 16-wide slices of the output
+    constexpr int KS = HD / 32;        // MFMA k-steps over the head dimension
+    constexpr int NS = HD / 16;        // 16-wide slices of the output
+    constexpr int VL = HD / 16;        // 16-byte pieces of a 32-key V block per lane
+    constexpr int VSTR = HD + 8;       // LDS row stride in fp16: 16 bytes of padding keep the gathers conflict-free
+    __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];  // one V block per wave
     const uint32_t lane = threadIdx.x & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    _Float16* vs = vs_all[wave];
     const uint32_t n_qt = (p.M + 15u) / 16u;
     const uint32_t task = blockIdx.x * 4 + wave;
     if (task >= n_qt * p.nq) return;
@@ -66,18 +71,44 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    for (uint32_t key0 = 0; key0 < kv_len; key0 += 32) {
-        // scores of keys key0 .. key0+31 for the 16 queries
+    // K rows of the two 16-key tiles (A operands) and this lane's pieces of the 32-key V block, one block ahead.
+    // Rows past the last key repeat it; their scores are masked.
+    v8h k0r[KS], k1r[KS];
+    v4i vr[VL];
+    auto load_k = [&](uint32_t key0) {
         const uint32_t kr0 = min(key0 + qi, kv_len - 1), kr1 = min(key0 + 16 + qi, kv_len - 1);
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            k0r[s] = *reinterpret_cast<const v8h*>(K + (size_t)kr0 * HD + 32 * s + 8 * g);
+            k1r[s] = *reinterpret_cast<const v8h*>(K + (size_t)kr1 * HD + 32 * s + 8 * g);
+        }
+    };
+    auto load_v = [&](uint32_t key0) {  // piece i of the lane: row (i * 64 + lane) / (HD / 8), 16-byte column (..) % (HD / 8)
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const uint32_t id = i * 64 + lane, row = min(key0 + id / (HD / 8), kv_len - 1), col = id % (HD / 8);
+            vr[i] = *reinterpret_cast<const v4i*>(V + (size_t)row * HD + col * 8);
+        }
+    };
+    load_k(0);
+    load_v(0);
+
+    for (uint32_t key0 = 0; key0 < kv_len; key0 += 32) {
+        // stage the V block (the previous block's reads were issued before this point: LDS runs in order)
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const uint32_t id = i * 64 + lane;
+            *reinterpret_cast<v4i*>(vs + (id / (HD / 8)) * VSTR + (id % (HD / 8)) * 8) = vr[i];
+        }
+        load_v(key0 + 32);
+        // scores of keys key0 .. key0+31 for the 16 queries
         v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-            const v8h a0 = *reinterpret_cast<const v8h*>(K + (size_t)kr0 * HD + 32 * s + 8 * g);
-            const v8h a1 = *reinterpret_cast<const v8h*>(K + (size_t)kr1 * HD + 32 * s + 8 * g);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qh[s], s0, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ql[s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qh[s], s1, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ql[s], s1, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], qh[s], s0, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], ql[s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], qh[s], s1, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], ql[s], s1, 0, 0, 0);
         }
         // this lane: query qi, keys key0 + 4g + v and key0 + 16 + 4g + v
         float sv[8];
@@ -88,6 +119,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
             sv[4 + v] = key0 + 16 + 4 * g + v <= qpos ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
         }
+        load_k(key0 + 32);
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);       // finite from the first block on: key 0 is visible to every query
@@ -104,15 +136,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         sum += __shfl_xor(sum, 32, 64);
         l_run = l_run * alpha + sum;
         m_run = m_new;
-        // O^T += V^T P^T; A operand: V[key(g, e)][16 slice + qi]
-        uint32_t vrow[8];
-#pragma unroll
-        for (int e = 0; e < 8; e++) vrow[e] = min(key0 + (e < 4 ? 4 * g + e : 16 + 4 * g + e - 4), kv_len - 1);
+        // O^T += V^T P^T; A operand: V[key(g, e)][16 slice + qi] gathered from the staged block
+        // (rows past the last key hold a repeated row; their probabilities are 0)
 #pragma unroll
         for (int sl = 0; sl < NS; sl++) {
             v8h a;
 #pragma unroll
-            for (int e = 0; e < 8; e++) a[e] = V[(size_t)vrow[e] * HD + 16 * sl + qi];
+            for (int e = 0; e < 8; e++) a[e] = vs[(e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) * VSTR + 16 * sl + qi];
 #pragma unroll
             for (int v = 0; v < 4; v++) O[sl][v] *= alpha;
             O[sl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, O[sl], 0, 0, 0);
