@@ -19,6 +19,9 @@ struct OxbGemmParams {
     uint32_t ldy;
     uint32_t tpw;            // row tiles per workgroup   (filled by the launcher)
     uint32_t n_mt;           // token tiles of the launch (filled by the launcher)
+    uint32_t n_ng;           // row groups of the launch  (filled by the launcher)
+    uint32_t ksplit, sb_per_split;  // K slices and superblocks per slice (filled by the launcher)
+    float* part;             // [ksplit][M][ldy] partial sums, needed when oxb_gemm_ksplit(...) > 1
     uint32_t codes_bytes, scales_bytes, xh_bytes;  // buffer extents (loads beyond them read 0)
     int mode;
 };
@@ -33,4 +36,6 @@ size_t oxb_xh_bytes(uint32_t k, uint32_t M);
 enum { OXB_PACK_IDENT = 0, OXB_PACK_RMSNORM = 1, OXB_PACK_SWIGLU = 2 };
 hipError_t oxb_launch_xh_pack(int fmt, int op, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, float eps,
                               uint32_t M, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st);
+// Number of K slices the launcher will use for this shape (1: no workspace needed).
+uint32_t oxb_gemm_ksplit(const OxbGemmParams& p, uint32_t n_cus);
 hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st);

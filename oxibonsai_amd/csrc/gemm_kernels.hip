@@ -293,8 +293,10 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     __shared__ __attribute__((aligned(16))) uint4 xs1[16 * BM];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));  // keeps unit offsets in SGPRs
-    const uint32_t m_t = blockIdx.x % p.n_mt, n_g = blockIdx.x / p.n_mt;
+    const uint32_t m_t = blockIdx.x % p.n_mt, n_g = (blockIdx.x / p.n_mt) % p.n_ng, ks = blockIdx.x / (p.n_mt * p.n_ng);
     const uint32_t m0 = m_t * BM;
+    // K slice of this workgroup, in superblocks
+    const uint32_t sb0 = ks * p.sb_per_split, sb1 = min(sb0 + p.sb_per_split, p.n_sb);
     // row tiles: the workgroup's [wg_t0, wg_t1), split evenly over the four waves
     const uint32_t wg_t0 = n_g * p.tpw, wg_t1 = min(wg_t0 + p.tpw, p.n_tiles);
     const uint32_t per = (p.tpw + 3u) / 4u;  // <= RT
@@ -331,11 +333,11 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     auto publish = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
 
     HalfRegs<FMT> H[RT][2];
-    stage_x(0, xs0);
+    stage_x(sb0 * 4, xs0);
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, 0, 0, lane);
-        load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, 0, 1, lane);
+        load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
+        load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
     }
     publish();
     BlockDec bd[RT], bdn[RT];
@@ -347,7 +349,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     const v8h* x0 = reinterpret_cast<const v8h*>(xs0);
     const v8h* x1 = reinterpret_cast<const v8h*>(xs1);
 
-    for (uint32_t sb = 0; sb < p.n_sb; sb++) {
+    for (uint32_t sb = sb0; sb < sb1; sb++) {
         // block 0 of the superblock
         stage_x(sb * 4 + 1, xs1);
 #pragma unroll
@@ -396,8 +398,9 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
         const uint32_t m = m0 + ct * 16 + r;
         if (m >= p.M) continue;
         const int e = p.xsh[m];
-        float* yr = p.y + (size_t)m * p.ldy;
-        const float* rr = p.mode == OXB_GEMM_RESIDUAL ? p.residual + (size_t)m * p.ldy : nullptr;
+        // with K split over workgroups, slice ks writes its partial sums to plane ks of the workspace
+        float* yr = p.ksplit > 1 ? p.part + ((size_t)ks * p.M + m) * p.ldy : p.y + (size_t)m * p.ldy;
+        const float* rr = (p.mode == OXB_GEMM_RESIDUAL && p.ksplit == 1) ? p.residual + (size_t)m * p.ldy : nullptr;
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             if ((uint32_t)rt >= n_valid) continue;
@@ -418,6 +421,24 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             }
         }
     }
+}
+
+// y = (residual +) the K slices' partial sums, added in slice order (deterministic).
+__global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, uint32_t ksplit, size_t plane,
+                                                                  const float* __restrict__ residual, float* __restrict__ y,
+                                                                  size_t n4) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4) return;
+    float4 a = reinterpret_cast<const float4*>(part)[i];
+    for (uint32_t s = 1; s < ksplit; s++) {
+        const float4 b = reinterpret_cast<const float4*>(part + s * plane)[i];
+        a.x += b.x, a.y += b.y, a.z += b.z, a.w += b.w;
+    }
+    if (residual) {
+        const float4 r = reinterpret_cast<const float4*>(residual)[i];
+        a.x += r.x, a.y += r.y, a.z += r.z, a.w += r.w;
+    }
+    reinterpret_cast<float4*>(y)[i] = a;
 }
 
 // ---------------------------------------------------------------------------
@@ -462,30 +483,57 @@ static hipError_t launch_gemm_case(const OxbGemmParams& p, uint32_t grid, hipStr
     return hipGetLastError();
 }
 
+struct GemmPlan { uint32_t rt, tpw, ksplit, sb_per_split; };
+
+// Row tiles per workgroup and K slices: minimise (rounds of workgroups over the CUs) x (time of one workgroup),
+// where a workgroup costs, per superblock of its K slice, its row tiles per wave plus about one more for staging,
+// barriers and operand latency, plus a fixed part for its start and epilogue.  Splitting K adds a pass over the
+// output per slice (the partial sums are written, then added in slice order).  Ties go to the larger tile.
+static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
+    constexpr uint32_t BM = 128;
+    const uint32_t n_mt = (p.M + BM - 1) / BM;
+    static const uint32_t rts[] = {5, 4, 3, 2, 1};
+    GemmPlan best = {1, 4, 1, p.n_sb};
+    uint64_t best_cost = ~0ull;
+    const bool can_split = (p.ldy & 3u) == 0;
+    for (uint32_t ks = 1; ks <= (can_split ? 8u : 1u) && ks <= p.n_sb; ks++) {
+        const uint32_t spk = (p.n_sb + ks - 1) / ks;
+        if (ks > 1 && (p.n_sb + spk - 1) / spk != ks) continue;  // same slices as a smaller count
+        for (uint32_t rt : rts) {
+            for (uint32_t tpw = 4 * rt; tpw > 4 * rt - 4; tpw--) {
+                const uint32_t groups = (p.n_tiles + tpw - 1) / tpw;
+                const uint64_t wgs = (uint64_t)groups * n_mt * ks;
+                uint64_t cost = ((wgs + n_cus - 1) / n_cus) * ((uint64_t)spk * (rt + 1) + 2 * rt + 2);
+                if (ks > 1) cost += (uint64_t)ks * 2 + 4;  // the reduction pass
+                if (cost < best_cost) best_cost = cost, best = {rt, tpw, ks, spk};
+            }
+        }
+    }
+    return best;
+}
+
+uint32_t oxb_gemm_ksplit(const OxbGemmParams& p, uint32_t n_cus) {
+    if (p.M == 0 || p.n_rows == 0 || p.n_sb == 0) return 1;
+    return plan_gemm(p, n_cus).ksplit;
+}
+
 hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
     if (p.M == 0 || p.n_rows == 0) return hipSuccess;
     if (p.n_sb == 0 || (uint64_t)p.n_tiles * p.n_sb * 2048ull >= 0xFFFFFFF0ull) return hipErrorInvalidValue;
     constexpr uint32_t CT = 8, BM = 16 * CT;
     p.M_pad = (p.M + 15u) / 16u * 16u;
     p.n_mt = (p.M + BM - 1) / BM;
-    // Row tiles per workgroup: minimise (rounds of workgroups over the CUs) x (time of one workgroup), where a
-    // workgroup costs its row tiles per wave plus about one more for staging, barriers and operand latency.
-    // Ties go to the larger tile (less re-reading of X).
-    static const uint32_t rts[] = {5, 4, 3, 2, 1};
-    uint32_t best_rt = 0, best_tpw = 0;
-    uint64_t best_cost = ~0ull;
-    for (uint32_t rt : rts) {
-        for (uint32_t tpw = 4 * rt; tpw > 4 * rt - 4; tpw--) {
-            const uint32_t groups = (p.n_tiles + tpw - 1) / tpw;
-            const uint64_t wgs = (uint64_t)groups * p.n_mt;
-            const uint64_t cost = ((wgs + n_cus - 1) / n_cus) * (rt + 1);
-            if (cost < best_cost) best_cost = cost, best_rt = rt, best_tpw = tpw;
-        }
-    }
+    const GemmPlan plan = plan_gemm(p, n_cus);
+    const uint32_t best_rt = plan.rt, best_tpw = plan.tpw;
+    p.ksplit = plan.ksplit;
+    p.sb_per_split = plan.sb_per_split;
+    if (p.ksplit > 1 && !p.part) return hipErrorInvalidValue;
     p.tpw = best_tpw;
-    const uint32_t grid = ((p.n_tiles + p.tpw - 1) / p.tpw) * p.n_mt;
+    p.n_ng = (p.n_tiles + p.tpw - 1) / p.tpw;
+    const uint32_t grid = p.n_ng * p.n_mt * p.ksplit;
+    hipError_t err = hipErrorInvalidValue;
 #define OXB_GEMM_CASE(F, R) \
-    if (fmt == F && best_rt == R) return launch_gemm_case<F, R, CT>(p, grid, st);
+    if (fmt == F && best_rt == R) err = launch_gemm_case<F, R, CT>(p, grid, st);
     OXB_GEMM_CASE(OXB_FMT_Q1, 1)
     OXB_GEMM_CASE(OXB_FMT_Q1, 2)
     OXB_GEMM_CASE(OXB_FMT_Q1, 3)
@@ -497,5 +545,9 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     OXB_GEMM_CASE(OXB_FMT_TQ2, 4)
     OXB_GEMM_CASE(OXB_FMT_TQ2, 5)
 #undef OXB_GEMM_CASE
-    return hipErrorInvalidValue;
+    if (err != hipSuccess || p.ksplit == 1) return err;
+    const size_t plane = (size_t)p.M * p.ldy, n4 = plane / 4;
+    hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, st, p.part, p.ksplit, plane,
+                       p.mode == OXB_GEMM_RESIDUAL ? p.residual : nullptr, p.y, n4);
+    return hipGetLastError();
 }

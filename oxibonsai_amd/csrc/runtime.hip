@@ -186,6 +186,11 @@ int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uin
     p.scales_bytes = (uint32_t)w.L.scales_bytes;
     p.xh_bytes = (uint32_t)oxb_xh_bytes(k, m);
     p.mode = mode;
+    const uint32_t ksplit = oxb_gemm_ksplit(p, g_rt.n_cus);
+    if (ksplit > 1) {
+        if ((rc = g_rt.ws_part.ensure((size_t)ksplit * m * ldy * sizeof(float)))) return rc;
+        p.part = (float*)g_rt.ws_part.ptr;
+    }
     e = oxb_launch_gemm((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemm");
     return OXB_HIP_OK;
@@ -279,6 +284,7 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_xh.release();
     g_rt.ws_xsh.release();
     g_rt.ws_rowmul.release();
+    g_rt.ws_part.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.own_stream = nullptr;
     g_rt.stream = nullptr;
@@ -493,6 +499,7 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     p.scales_bytes = (uint32_t)w->L.scales_bytes;
     p.xh_bytes = (uint32_t)oxb_xh_bytes(k, m);
     p.mode = OXB_GEMM_STORE;
+    p.part = (float*)g_rt.ws_part.ptr;  // sized by the gemm_device call above
     hipEvent_t ev0, ev1;
     hipError_t e;
     if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");

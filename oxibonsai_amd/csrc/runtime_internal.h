@@ -41,6 +41,7 @@ struct Runtime {
     uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
     DevBuf ws_xh, ws_xsh, ws_rowmul;  // prefill GEMM: packed fp16 activations, per-row exponents and multipliers
+    DevBuf ws_part;                   // prefill GEMM: partial sums of the K slices when K is split over workgroups
 };
 
 extern Runtime g_rt;
