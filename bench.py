@@ -31,7 +31,7 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one gate||up GEMV launch moves: rocprofv3 FETCH_SIZE (x 2.000, calibrated on a 256 MiB copy) + WRITE_SIZE
 # (x 1.000), see profiles/gemv_q1_qwen3_8b_set_hbm_traffic.txt.  The algorithmic figure is 14 270 464.
-GATE_UP_HBM_TRAFFIC_BYTES = 14_617_600
+GATE_UP_HBM_TRAFFIC_BYTES = 14_642_176
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
 FMT_TQ2 = 1
@@ -57,7 +57,7 @@ def cpu_baseline(blocks: dict, xs: dict, budget_s: float = 12.0) -> dict:
     t0 = time.perf_counter()
     one_pass()
     per = max(time.perf_counter() - t0, 1e-6)
-    reps = int(max(5, min(2000, budget_s / per)))
+    reps = int(max(5, min(20000, budget_s / per)))
     times = []
     for _ in range(reps):
         t0 = time.perf_counter()
@@ -289,6 +289,18 @@ def main() -> int:
         us = C.c_float(0.0)
         L.oxb_hip_profile_gemv(arr, args.copies, d_x[nm].data_ptr(), d_y[nm].data_ptr(), r, kk, 20, 200, C.byref(us))
         per_kernel[nm] = {"us": round(us.value, 3), "GB/s": round(algorithmic_bytes(r, kk) / (us.value * 1e-6) / 1e9, 1)}
+    # the same kernel on a matrix large enough to amortise the launch: the LM head 151936x4096 (3 rotating copies, 262 MB)
+    lm_rows, lm_k = 151936, 4096
+    lm_blocks = synth.make_q1_blocks(0xB0A5A101F0, lm_rows * (lm_k // 128), 0.01, 0.1)
+    lm_ids = [be.upload_weights_raw(lm_blocks, lm_rows, lm_k) for _ in range(3)]
+    lm_y = torch.zeros(lm_rows, dtype=torch.float32, device="cuda")
+    arr = (C.c_uint64 * 3)(*[int(h) for h in lm_ids])
+    us = C.c_float(0.0)
+    L.oxb_hip_profile_gemv(arr, 3, d_x["qkv"].data_ptr(), lm_y.data_ptr(), lm_rows, lm_k, 6, 60, C.byref(us))
+    per_kernel["lm_head_151936x4096"] = {"us": round(us.value, 3),
+                                         "GB/s": round(algorithmic_bytes(lm_rows, lm_k) / (us.value * 1e-6) / 1e9, 1)}
+    for h in lm_ids:
+        be.free_weights(h)
 
     out = {
         "metric": "quant GEMV HBM GB/s", "value": round(value, 2), "unit": "GB/s",
