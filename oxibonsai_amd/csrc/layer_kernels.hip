@@ -441,6 +441,7 @@ __global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p
         *reinterpret_cast<float4*>(o + (e - e0)) = acc;
         if (out_or_null) *reinterpret_cast<float4*>(out_or_null + (size_t)b * qd + e) = acc;
     }
+    if (!xq) return;  // merge only: the caller consumes the fp32 output
     // the quantiser indexes the vector from its start: hand it the span shifted back by e0
     gstat_scan(o - e0, qd, gsb, g0, g1, gstat);  // its first barrier publishes the outputs
     quantise_groups<FMT>(o - e0, qd, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
@@ -561,7 +562,9 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
 hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
                                          int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st) {
     const uint32_t qd = p.nq * p.hd;
-    if (nb == 0 || nb > 2 || (qd % OXB_QK) != 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
+    // with d_xq == nullptr the kernel only merges (any nb) and d_out_or_null must be given
+    if (nb == 0 || (d_xq && nb > 2) || (!d_xq && !d_out_or_null) || (qd % OXB_QK) != 0 || p.n_splits > OXB_ATTN_MAX_SPLITS)
+        return hipErrorInvalidValue;
     const uint32_t n_sb = (qd + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
     if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
     const uint32_t parts = n_groups < 16 ? n_groups : 16, per = (n_groups + parts - 1) / parts;

@@ -56,6 +56,7 @@ struct Model {
     uint32_t pf_cap = 0;
     float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
     std::vector<void*> pf_allocs;
+    GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
 };
 
 static std::unordered_map<uint64_t, std::unique_ptr<Model>> g_models;
@@ -77,6 +78,7 @@ static void free_model(Model& m) {
     for (void* p : m.pf_allocs) (void)hipFree(p);
     m.pf_allocs.clear();
     m.pf_cap = 0;
+    m.gws.release();
 }
 
 void shutdown_models() {
@@ -175,8 +177,82 @@ static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn
     return OXB_HIP_OK;
 }
 
+// Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
+// matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
+// the weights once per two sequences.
+#define OXB_DECODE_GEMM_MIN_BATCH 8
+
+static int encode_decode_step_gemm(Model& m) {
+    const oxb_model_desc& d = m.d;
+    hipStream_t st = g_rt.stream;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd, B = d.batch;
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < d.n_layers; L++) {
+        const oxb_layer_ids& ly = m.layers[L];
+        const float* attn_norm = vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
+        const float* q_norm = vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
+        const float* k_norm = vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
+        const float* ffn_norm = vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
+        const Weight* wqkv = mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
+        const Weight* wo = mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
+        const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
+        const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
+        if (rc) return rc;
+        OXB_TRY(gemm_device(*wqkv, m.hidden, d.h, m.qkv, B, qkv_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, attn_norm, d.eps, &m.gws));
+        OxbQkParams qp;
+        qp.qkv = m.qkv;
+        qp.qkv_stride = qkv_rows;
+        qp.q_norm = q_norm;
+        qp.k_norm = k_norm;
+        qp.cos_t = m.cos_t;
+        qp.sin_t = m.sin_t;
+        qp.pos = m.pos;
+        qp.pos_base = 0;
+        qp.seq = 0;
+        qp.q_rope = m.q_rope;
+        qp.k_cache = m.k_cache;
+        qp.v_cache = m.v_cache;
+        qp.nq = d.nq;
+        qp.nkv = d.nkv;
+        qp.hd = d.hd;
+        qp.max_seq = d.max_seq;
+        qp.n_layers = d.n_layers;
+        qp.layer = L;
+        qp.eps = d.eps;
+        OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, B, st), "kernel launch failed: qk_norm_rope_store");
+        OxbAttnParams ap;
+        ap.q = m.q_rope;
+        ap.k_cache = m.k_cache;
+        ap.v_cache = m.v_cache;
+        ap.part = m.attn_part;
+        ap.pos = m.pos;
+        ap.nq = d.nq;
+        ap.nkv = d.nkv;
+        ap.hd = d.hd;
+        ap.max_seq = d.max_seq;
+        ap.n_layers = d.n_layers;
+        ap.layer = L;
+        ap.chunk = m.chunk;
+        ap.n_splits = m.n_splits;
+        ap.scale = 1.0f / sqrtf((float)d.hd);
+        OXB_TRY_HIP(oxb_launch_attn_decode(ap, B, st), "kernel launch failed: attention");
+        OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
+                    "kernel launch failed: attn_combine");
+        OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
+        OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
+        OXB_TRY(gemm_device(*wdn, m.gu, 2 * d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_SWIGLU, nullptr, 0.f, &m.gws));
+    }
+    const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
+    const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+    if (rc) return rc;
+    OXB_TRY(gemm_device(*lm, m.hidden, d.h, m.logits, B, d.vocab, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, final_norm, d.eps, &m.gws));
+    OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, B, m.tokens, m.argmax_ws, st), "kernel launch failed: argmax");
+    return OXB_HIP_OK;
+}
+
 // Every kernel of one decode step, for all sequences of the batch (no host synchronisation).
 static int encode_decode_step(Model& m, bool with_lm_head) {
+    if (m.d.batch >= OXB_DECODE_GEMM_MIN_BATCH && with_lm_head) return encode_decode_step_gemm(m);
     const oxb_model_desc& d = m.d;
     hipStream_t st = g_rt.stream;
     const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
@@ -482,6 +558,32 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         if (e != hipSuccess) {
             free_model(m);
             return hip_fail(e, "rope table upload");
+        }
+    }
+    if (d.batch >= OXB_DECODE_GEMM_MIN_BATCH) {
+        // the GEMM-based decode step is captured into a graph: size the library's GEMM workspaces now
+        uint32_t kx = d.h > d.inter ? d.h : d.inter;
+        if (qd > kx) kx = qd;
+        size_t part_bytes = 0;
+        const struct { uint64_t id; uint32_t n, k; } shapes[] = {{m.layers[0].qkv, qkv_rows, d.h}, {m.layers[0].o, d.h, qd},
+                                                                 {m.layers[0].gate_up, 2 * d.inter, d.h},
+                                                                 {m.layers[0].down, d.h, d.inter}, {d.lm_head, d.vocab, d.h}};
+        for (const auto& sh : shapes) {
+            const Weight* w = find_weight(sh.id);
+            OxbGemmParams gp;
+            memset(&gp, 0, sizeof gp);
+            gp.n_rows = sh.n;
+            gp.n_tiles = w->L.n_tiles;
+            gp.n_sb = w->L.n_sb;
+            gp.M = d.batch;
+            gp.ldy = sh.n;
+            const size_t b = (size_t)oxb_gemm_ksplit(gp, g_rt.n_cus) * d.batch * sh.n * sizeof(float);
+            if (oxb_gemm_ksplit(gp, g_rt.n_cus) > 1 && b > part_bytes) part_bytes = b;
+        }
+        if ((rc = m.gws.xh.ensure(oxb_xh_bytes(kx, d.batch))) || (rc = m.gws.xsh.ensure(((size_t)d.batch + 16) * 4)) ||
+            (rc = m.gws.rowmul.ensure(((size_t)d.batch + 16) * 4)) || (part_bytes && (rc = m.gws.part.ensure(part_bytes)))) {
+            free_model(m);
+            return rc;
         }
     }
     const char* no_graph = getenv("OXB_HIP_DISABLE_GRAPH");

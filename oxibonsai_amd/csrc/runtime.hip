@@ -158,23 +158,24 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
 }
 
 int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
-                const float* d_residual, int pack_op, const float* d_pack_w, float eps) {
+                const float* d_residual, int pack_op, const float* d_pack_w, float eps, GemmWorkspace* ws) {
+    if (!ws) ws = &g_rt.gemm_ws;
     const uint32_t k = w.L.k;
     if ((uint64_t)m * k >= (1ull << 31))
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u rows of %u activations exceed one GEMM call", m, k);
     int rc;
-    if ((rc = g_rt.ws_xh.ensure(oxb_xh_bytes(k, m)))) return rc;
-    if ((rc = g_rt.ws_xsh.ensure(((size_t)m + 16) * sizeof(int32_t)))) return rc;
-    if ((rc = g_rt.ws_rowmul.ensure(((size_t)m + 16) * sizeof(float)))) return rc;
-    hipError_t e = oxb_launch_xh_pack((int)w.L.fmt, pack_op, d_x, d_pack_w, ldx, k, eps, m, (float*)g_rt.ws_rowmul.ptr,
-                                      (uint32_t*)g_rt.ws_xh.ptr, (int32_t*)g_rt.ws_xsh.ptr, g_rt.stream);
+    if ((rc = ws->xh.ensure(oxb_xh_bytes(k, m)))) return rc;
+    if ((rc = ws->xsh.ensure(((size_t)m + 16) * sizeof(int32_t)))) return rc;
+    if ((rc = ws->rowmul.ensure(((size_t)m + 16) * sizeof(float)))) return rc;
+    hipError_t e = oxb_launch_xh_pack((int)w.L.fmt, pack_op, d_x, d_pack_w, ldx, k, eps, m, (float*)ws->rowmul.ptr,
+                                      (uint32_t*)ws->xh.ptr, (int32_t*)ws->xsh.ptr, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch failed: xh_pack");
     OxbGemmParams p;
     memset(&p, 0, sizeof p);
     p.codes = w.d_codes;
     p.scales = w.d_scales;
-    p.xh = (const uint32_t*)g_rt.ws_xh.ptr;
-    p.xsh = (const int32_t*)g_rt.ws_xsh.ptr;
+    p.xh = (const uint32_t*)ws->xh.ptr;
+    p.xsh = (const int32_t*)ws->xsh.ptr;
     p.y = d_y;
     p.residual = d_residual;
     p.n_rows = w.L.n_rows;
@@ -188,8 +189,8 @@ int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uin
     p.mode = mode;
     const uint32_t ksplit = oxb_gemm_ksplit(p, g_rt.n_cus);
     if (ksplit > 1) {
-        if ((rc = g_rt.ws_part.ensure((size_t)ksplit * m * ldy * sizeof(float)))) return rc;
-        p.part = (float*)g_rt.ws_part.ptr;
+        if ((rc = ws->part.ensure((size_t)ksplit * m * ldy * sizeof(float)))) return rc;
+        p.part = (float*)ws->part.ptr;
     }
     e = oxb_launch_gemm((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemm");
@@ -281,10 +282,7 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_xq.release();
     g_rt.ws_cneg.release();
     g_rt.ws_xexp.release();
-    g_rt.ws_xh.release();
-    g_rt.ws_xsh.release();
-    g_rt.ws_rowmul.release();
-    g_rt.ws_part.release();
+    g_rt.gemm_ws.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.own_stream = nullptr;
     g_rt.stream = nullptr;
@@ -487,8 +485,8 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     memset(&p, 0, sizeof p);
     p.codes = w->d_codes;
     p.scales = w->d_scales;
-    p.xh = (const uint32_t*)g_rt.ws_xh.ptr;
-    p.xsh = (const int32_t*)g_rt.ws_xsh.ptr;
+    p.xh = (const uint32_t*)g_rt.gemm_ws.xh.ptr;
+    p.xsh = (const int32_t*)g_rt.gemm_ws.xsh.ptr;
     p.y = d_y;
     p.n_rows = n_rows;
     p.n_tiles = w->L.n_tiles;
@@ -499,7 +497,7 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     p.scales_bytes = (uint32_t)w->L.scales_bytes;
     p.xh_bytes = (uint32_t)oxb_xh_bytes(k, m);
     p.mode = OXB_GEMM_STORE;
-    p.part = (float*)g_rt.ws_part.ptr;  // sized by the gemm_device call above
+    p.part = (float*)g_rt.gemm_ws.part.ptr;  // sized by the gemm_device call above
     hipEvent_t ev0, ev1;
     hipError_t e;
     if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");

@@ -17,6 +17,14 @@ struct DevBuf {  // grow-only device scratch
     void release();
 };
 
+// Scratch of one GEMM call: packed fp16 activations, per-row exponents and multipliers, and the partial sums of
+// the K slices when K is split over workgroups.  A sequence of calls captured into a graph needs buffers of its
+// own that never move.
+struct GemmWorkspace {
+    DevBuf xh, xsh, rowmul, part;
+    void release() { xh.release(); xsh.release(); rowmul.release(); part.release(); }
+};
+
 struct Weight {  // one resident matrix: [codes section][scales section]
     OxbLayout L;
     void* d_base = nullptr;
@@ -40,8 +48,7 @@ struct Runtime {
     std::unordered_map<uint64_t, Vector> vectors;
     uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
-    DevBuf ws_xh, ws_xsh, ws_rowmul;  // prefill GEMM: packed fp16 activations, per-row exponents and multipliers
-    DevBuf ws_part;                   // prefill GEMM: partial sums of the K slices when K is split over workgroups
+    GemmWorkspace gemm_ws;  // shared by every GEMM call that does not bring its own
 };
 
 extern Runtime g_rt;
@@ -56,8 +63,9 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
                 const float* d_residual);
 // x (device, [m][ldx]) -> y (device, [m][ldy]) through the fp16 packer + MFMA GEMM.  pack_op (OXB_PACK_*) names the
 // row-wise producer fused into the packer: RMSNorm with weights d_pack_w and eps, or SwiGLU of x = [gate | up].
+// ws = nullptr uses (and may grow) the runtime's shared workspace.
 int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
-                const float* d_residual, int pack_op, const float* d_pack_w, float eps);
+                const float* d_residual, int pack_op, const float* d_pack_w, float eps, GemmWorkspace* ws = nullptr);
 void shutdown_models();
 
 }  // namespace oxb

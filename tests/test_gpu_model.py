@@ -173,3 +173,26 @@ def test_gqa_group_shapes(backend, nq, nkv, hd):
                 assert parity_violations(got[0], want) == 0, pos
     finally:
         gpu.close()
+
+
+@pytest.mark.parametrize("fmt", [TQ2, Q1])
+def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt):
+    """From 8 sequences on, a decode step sends its projections through the prefill GEMM (fp16 activations):
+    logits are held to the prefill tolerance 1e-2 under the reference's gate form; the step is still replayed
+    from a captured graph and sequences stay independent."""
+    cfg = dict(SMALL, fmt=fmt)
+    w = synth.make_model(cfg, 61 + fmt)
+    B = 9
+    gpu = HipModel(backend, cfg, w, batch=B)
+    cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
+    try:
+        for step in range(6):
+            hidden = np.stack([synth.embedding_rows(70 + b, [3 * step + b], cfg["h"])[0] * 50.0 for b in range(B)])
+            got, toks = gpu.forward(hidden, np.full(B, step, dtype=np.uint32))
+            for b in range(B):
+                want = cpus[b].forward(hidden[b], step)
+                assert parity_violations(got[b], want, 1e-2) == 0, (step, b, float(np.max(np.abs(got[b] - want))))
+                assert toks[b] == int(np.argmax(got[b]))
+        assert gpu.uses_graph()
+    finally:
+        gpu.close()
