@@ -65,30 +65,24 @@ __device__ __forceinline__ void digits_of4(const long long v[4], uint32_t dig[8]
     transpose_bytes4(hi, dig + 4);
 }
 
-// Quantise the 16 activations that one lane group (blk, m, g) of the MFMA B operand holds and
-// store their eight digit planes; cs[d] returns this group's share of the block's correction sums.
+// Offset (in floats, from the start of the block's 32-weight group g) of the four consecutive activations
+// jj = 0..3 that byte position bb of MFMA m pairs with:  Q1: k = 8bb + 4m + jj;  TQ2: k = 16m + 4bb + jj.
 template <int FMT>
-__device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_t blk, uint32_t m, uint32_t g,
-                                           int base_shift, bool live, uint32_t NC, uint32_t n,
-                                           uint32_t* __restrict__ xq, int cs[8]) {
-    uint32_t out[8][4];
+__device__ __forceinline__ uint32_t unit_val_offset(uint32_t m, uint32_t bb) {
+    return FMT == OXB_FMT_Q1 ? 8 * bb + 4 * m : 16 * m + 4 * bb;
+}
+
+// Digits of the 16 activations vv[bb][jj] that one lane group (blk, m, g) of the MFMA B operand holds:
+// out[d][jj] = one dword of digit plane d, cs[d] = this group's share of the block's correction sums.
+template <int FMT>
+__device__ __forceinline__ void quant_unit_digits(const float (&vv)[4][4], uint32_t m, int base_shift, bool live,
+                                                  uint32_t (&out)[8][4], int (&cs)[8]) {
 #pragma unroll
     for (int d = 0; d < 8; d++) {
         cs[d] = 0;
         out[d][0] = out[d][1] = out[d][2] = out[d][3] = 0;
     }
     if (live) {
-        const float* xb = xn + blk * 128 + 32 * g;
-        float vv[4][4];  // [bb][jj]
-#pragma unroll
-        for (uint32_t bb = 0; bb < 4; bb++) {
-            // Q1: k = 8bb + 4m + jj;  TQ2: k = 16m + 4bb + jj   (jj = 0..3 contiguous)
-            const float4 v4 = *reinterpret_cast<const float4*>(xb + (FMT == OXB_FMT_Q1 ? 8 * bb + 4 * m : 16 * m + 4 * bb));
-            vv[bb][0] = v4.x;
-            vv[bb][1] = v4.y;
-            vv[bb][2] = v4.z;
-            vv[bb][3] = v4.w;
-        }
 #pragma unroll
         for (uint32_t jj = 0; jj < 4; jj++) {
             long long xi[4], cr[4];
@@ -117,6 +111,40 @@ __device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_
             for (int d = 0; d < 8; d++) out[d][jj] = dig[d];
         }
     }
+}
+
+// Sum the correction shares over the eight lanes (m, g) of a block - consecutive lanes starting at a multiple
+// of eight - and return, in lane j of the eight, the sum of digit j.
+__device__ __forceinline__ int block_correction(int (&cs)[8], uint32_t lane_in_block) {
+#pragma unroll
+    for (int d = 0; d < 8; d++) {
+        int v = cs[d];
+        v += dpp_i32<0x141>(v);  // row_half_mirror: i <-> 7 - i
+        v += dpp_i32<0xB1>(v);   // quad_perm [1,0,3,2]
+        v += dpp_i32<0x4E>(v);   // quad_perm [2,3,0,1]
+        cs[d] = v;
+    }
+    int mine = cs[0];
+#pragma unroll
+    for (int d = 1; d < 8; d++) mine = (lane_in_block == (uint32_t)d) ? cs[d] : mine;
+    return mine;
+}
+
+// Quantise the 16 activations that one lane group (blk, m, g) of the MFMA B operand holds and
+// store their eight digit planes; cs[d] returns this group's share of the block's correction sums.
+template <int FMT>
+__device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_t blk, uint32_t m, uint32_t g,
+                                           int base_shift, bool live, uint32_t NC, uint32_t n,
+                                           uint32_t* __restrict__ xq, int (&cs)[8]) {
+    uint32_t out[8][4];
+    float vv[4][4];  // [bb][jj]
+#pragma unroll
+    for (uint32_t bb = 0; bb < 4; bb++) {
+        float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (live) v4 = *reinterpret_cast<const float4*>(xn + blk * 128 + 32 * g + unit_val_offset<FMT>(m, bb));
+        vv[bb][0] = v4.x, vv[bb][1] = v4.y, vv[bb][2] = v4.z, vv[bb][3] = v4.w;
+    }
+    quant_unit_digits<FMT>(vv, m, base_shift, live, out, cs);
     uint4* dst = reinterpret_cast<uint4*>(xq) + (size_t)((blk * 2 + m) * 4 + g) * NC + 8 * n;
 #pragma unroll
     for (int d = 0; d < 8; d++) dst[d] = make_uint4(out[d][0], out[d][1], out[d][2], out[d][3]);
@@ -210,19 +238,8 @@ __device__ __forceinline__ void quantise_groups(const float* __restrict__ xn, ui
         if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
         int cs[8];
         quant_unit<FMT>(xn, blk, m, g, OXB_XQ_P - E, ok && blk < nblk, NC, n, xq, cs);
-        // sum the correction over the block's eight lanes: i <-> 7-i, then within quads
-#pragma unroll
-        for (int d = 0; d < 8; d++) {
-            int v = cs[d];
-            v += dpp_i32<0x141>(v);  // row_half_mirror
-            v += dpp_i32<0xB1>(v);   // quad_perm [1,0,3,2]
-            v += dpp_i32<0x4E>(v);   // quad_perm [2,3,0,1]
-            cs[d] = v;
-        }
-        // lane j of the eight writes digit j (four copies: the MFMA takes it as a 4-register operand)
-        int mine = cs[0];
-#pragma unroll
-        for (int d = 1; d < 8; d++) mine = ((u & 7u) == (uint32_t)d) ? cs[d] : mine;
+        // lane j of the block's eight writes digit j (four copies: the MFMA takes it as a 4-register operand)
+        const int mine = block_correction(cs, u & 7u);
         *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + (u & 7u)) * 4) = make_int4(-mine, -mine, -mine, -mine);
     }
     for (uint32_t gi = g_begin + threadIdx.x; gi < g_end; gi += blockDim.x) {
