@@ -18,8 +18,14 @@ struct OxbQkParams {
 };
 
 struct OxbAttnParams {
-    const float* q;                      // [batch][nq][hd]
-    const __half *k_cache, *v_cache;
+    const float* q;                      // [batch][nq][hd] after QK-norm and RoPE (attn_decode_kernel only)
+    // attn_decode_fused_kernel reads the raw projections instead and does QK-norm, RoPE and the KV store itself
+    const float* qkv;                    // [batch][qkv_stride]: q heads | k heads | v heads
+    uint32_t qkv_stride;
+    const float *q_norm, *k_norm;        // [hd]
+    const float *cos_t, *sin_t;          // [max_seq][hd/2]
+    float eps;
+    __half *k_cache, *v_cache;           // [batch][n_layers][nkv][max_seq][hd]
     float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
@@ -39,6 +45,9 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 // Split-KV attention into p.part, then the merge of the slots fused with the quantiser of the O projection's
 // input for sequences b0 .. b0 + nb - 1 (nb <= 2); d_out_or_null also receives the fp32 attention output [batch][nq*hd].
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
+// The same attention on the matrix cores, fused with QK-norm, RoPE and the KV store of the new position
+// (qkv, q_norm, k_norm, cos_t, sin_t, eps set; q unused).  Writes the same p.part layout.
+hipError_t oxb_launch_attn_decode_fused(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
 hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
                                          int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.

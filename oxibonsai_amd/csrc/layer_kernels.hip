@@ -375,6 +375,194 @@ __global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnPa
     }
 }
 
+// ---------------------------------------------------------------------------
+// Decode attention on the matrix cores, fused with what precedes it in the layer: per-head QK-RMSNorm, RoPE and
+// the FP16 store of the new position's K and V (fused_qk_norm_rope + fused_kv_store + batched attention,
+// gpu_backend/cuda_attn_kernels.rs:160-438).  Grid (n_splits, nkv, batch), 256 threads = 4 waves.
+// A workgroup serves all q heads of one kv head (<= 16, the columns of the MFMA tiles) for one slot of the KV
+// sequence: slot s walks chunks s, s + n_splits, ... of 128 positions, wave w takes keys [32w, 32w + 32) of each.
+//   S^T[key][head] = sum_d K[key][d] Q[head][d]     A = K rows straight from the cache, B = Q * scale as fp16 hi + lo
+//   O^T[d][head]  += sum_key V[key][d] P[head][key]  A = V gathered from the wave's LDS copy of the block,
+//                                                    B = the lane's own probabilities as fp16 hi + lo
+// so scores and weighted sums keep fp32-level accuracy.  Every wave runs its own online softmax; the four results
+// meet in LDS.  The workgroup whose slot holds the new position computes K (norm + RoPE) and V of that position,
+// stores them to the cache and, after a barrier, reads them back like any other row.
+// ---------------------------------------------------------------------------
+typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+
+template <int HD>
+__global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p) {
+    constexpr int KS = HD / 32, NS = HD / 16, VL = HD / 16, VSTR = HD + 8;
+    __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];  // V block per wave; later the merge buffers
+    __shared__ float qs[16 * HD];                                           // Q * scale of the group's heads
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t slot = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
+    const uint32_t G = p.nq / p.nkv, h0 = kvh * G, half = HD / 2;
+    const uint32_t pos = p.pos[b], seq_len = pos + 1;
+    const uint32_t n_chunks = (seq_len + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK;
+    if (slot >= n_chunks) return;  // never read by the merge
+    const float* qkv = p.qkv + (size_t)b * p.qkv_stride;
+    const float* cs = p.cos_t + (size_t)pos * half;
+    const float* sn = p.sin_t + (size_t)pos * half;
+    const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * HD;
+    _Float16* Kc = reinterpret_cast<_Float16*>(p.k_cache) + base;
+    _Float16* Vc = reinterpret_cast<_Float16*>(p.v_cache) + base;
+
+    // --- Q of the group's heads: RMSNorm over the head, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd) ---
+    for (uint32_t h = wave; h < G; h += 4) {
+        const float* in = qkv + (size_t)(h0 + h) * HD;
+        float ss = 0.f;
+        for (uint32_t d = lane; d < HD; d += 64) ss = fmaf(in[d], in[d], ss);
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
+        for (uint32_t d = lane; d < half; d += 64) {
+            const float lo = p.q_norm[d] * in[d] * inv, hi = p.q_norm[d + half] * in[d + half] * inv;
+            qs[h * HD + d] = (lo * cs[d] - hi * sn[d]) * p.scale;
+            qs[h * HD + d + half] = (lo * sn[d] + hi * cs[d]) * p.scale;
+        }
+    }
+    // --- K and V of the new position, by the workgroup whose slot walks its chunk (wave 0 and wave 1) ---
+    if ((pos / OXB_ATTN_CHUNK) % p.n_splits == slot) {
+        if (wave == 0) {
+            const float* in = qkv + (size_t)(p.nq + kvh) * HD;
+            float ss = 0.f;
+            for (uint32_t d = lane; d < HD; d += 64) ss = fmaf(in[d], in[d], ss);
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
+            for (uint32_t d = lane; d < half; d += 64) {
+                const float lo = p.k_norm[d] * in[d] * inv, hi = p.k_norm[d + half] * in[d + half] * inv;
+                Kc[(size_t)pos * HD + d] = (_Float16)(lo * cs[d] - hi * sn[d]);
+                Kc[(size_t)pos * HD + d + half] = (_Float16)(lo * sn[d] + hi * cs[d]);
+            }
+        } else if (wave == 1) {
+            const float* in = qkv + (size_t)(p.nq + p.nkv + kvh) * HD;
+            for (uint32_t d = lane; d < HD; d += 64) Vc[(size_t)pos * HD + d] = (_Float16)in[d];
+        }
+    }
+    __syncthreads();  // publishes qs and, within this workgroup, the new cache rows
+
+    // B operands: lane (head = qi, g) holds Q[head][32 s + 8 g .. + 7] as hi + lo
+    v8h_t qh[KS], ql[KS];
+#pragma unroll
+    for (int s = 0; s < KS; s++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float x = qi < G ? qs[qi * HD + 32 * s + 8 * g + e] : 0.f;
+            const _Float16 hi = (_Float16)x;
+            qh[s][e] = hi;
+            ql[s][e] = (_Float16)(x - (float)hi);
+        }
+    v4f O[NS];
+#pragma unroll
+    for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    _Float16* vs = vs_all[wave];
+
+    for (uint32_t chunk = slot; chunk < n_chunks; chunk += p.n_splits) {
+        const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
+        if (key0 >= seq_len) continue;  // this wave's quarter of the last chunk is empty
+        const uint32_t kr0 = min(key0 + qi, seq_len - 1), kr1 = min(key0 + 16 + qi, seq_len - 1);
+        v8h_t k0r[KS], k1r[KS];
+        v4i vr[VL];
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
+            k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
+        }
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const uint32_t id = i * 64 + lane, row = min(key0 + id / (HD / 8), seq_len - 1), col = id % (HD / 8);
+            vr[i] = *reinterpret_cast<const v4i*>(Vc + (size_t)row * HD + col * 8);
+        }
+        v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], qh[s], s0, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], ql[s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], qh[s], s1, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], ql[s], s1, 0, 0, 0);
+        }
+        // this lane: head qi, keys key0 + 4g + v and key0 + 16 + 4g + v
+        float sv[8];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            sv[v] = key0 + 4 * g + v < seq_len ? s0[v] : -INFINITY;
+            sv[4 + v] = key0 + 16 + 4 * g + v < seq_len ? s1[v] : -INFINITY;
+            mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);      // finite: key0 < seq_len
+        const float alpha = expf(m_run - m_new);   // 0 for the wave's first block
+        float sum = 0.f;
+        v8h_t ph, pl;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const float pe = expf(sv[e] - m_new);
+            sum += pe;
+            const _Float16 hi = (_Float16)pe;
+            ph[e] = hi;
+            pl[e] = (_Float16)(pe - (float)hi);
+        }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+        // stage the V block in the wave's LDS slice, then gather the transposed operand
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const uint32_t id = i * 64 + lane;
+            *reinterpret_cast<v4i*>(vs + (id / (HD / 8)) * VSTR + (id % (HD / 8)) * 8) = vr[i];
+        }
+#pragma unroll
+        for (int sl = 0; sl < NS; sl++) {
+            v8h_t a;
+#pragma unroll
+            for (int e = 0; e < 8; e++) a[e] = vs[(e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) * VSTR + 16 * sl + qi];
+#pragma unroll
+            for (int v = 0; v < 4; v++) O[sl][v] *= alpha;
+            O[sl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ph, O[sl], 0, 0, 0);
+            O[sl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pl, O[sl], 0, 0, 0);
+        }
+    }
+    // --- merge the four waves: lane (head = qi, g) holds O[head][16 sl + 4 g + v], m_run, l_run ---
+    __syncthreads();  // the V slices are dead: reuse them
+    static_assert(sizeof(vs_all) >= (4 * 16 * HD + 2 * 4 * 16) * sizeof(float), "merge buffers must fit in the V slices");
+    float* mo = reinterpret_cast<float*>(&vs_all[0][0]);  // [wave][head 16][HD], then [wave][head 16] m, [wave][head 16] l
+    float* mm = mo + 4 * 16 * HD;
+    float* ml = mm + 4 * 16;
+#pragma unroll
+    for (int sl = 0; sl < NS; sl++)
+        *reinterpret_cast<float4*>(&mo[(wave * 16 + qi) * HD + 16 * sl + 4 * g]) = make_float4(O[sl][0], O[sl][1], O[sl][2], O[sl][3]);
+    if (g == 0) {
+        mm[wave * 16 + qi] = m_run;
+        ml[wave * 16 + qi] = l_run;
+    }
+    __syncthreads();
+    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + slot) * (HD + OXB_ATTN_PART_PAD);
+    const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
+    for (uint32_t i = tid; i < G * HD; i += 256) {
+        const uint32_t h = i / HD, d = i % HD;
+        const float M = fmaxf(fmaxf(mm[h], mm[16 + h]), fmaxf(mm[32 + h], mm[48 + h]));
+        float o = 0.f, l = 0.f;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const float wgt = expf(mm[w * 16 + h] - M);  // 0 for a wave that saw no key
+            o = fmaf(mo[(w * 16 + h) * HD + d], wgt, o);
+            l = fmaf(ml[w * 16 + h], wgt, l);
+        }
+        part[h * part_head + d] = o;
+        if (d == 0) {
+            part[h * part_head + HD] = M;
+            part[h * part_head + HD + 1] = l;
+        }
+    }
+}
+
 // Merge the slot results of the q heads and quantise the attention output for the O projection.  Grid
 // (vectors of the pass, parts), 256 threads: a workgroup takes whole exponent groups of the output vector
 // (nq * hd values), i.e. a run of dimensions that it merges (softmax weights of the slots per head: one wave
@@ -557,6 +745,21 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
         case 256: return launch_attn_hd<256>(p, batch, st);
         default: return hipErrorInvalidValue;
     }
+}
+
+hipError_t oxb_launch_attn_decode_fused(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
+    if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
+        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t)
+        return hipErrorInvalidValue;
+    const dim3 grid(p.n_splits, p.nkv, batch), block(256);
+    switch (p.hd) {
+        case 32: hipLaunchKernelGGL(attn_decode_fused_kernel<32>, grid, block, 0, st, p); break;
+        case 64: hipLaunchKernelGGL(attn_decode_fused_kernel<64>, grid, block, 0, st, p); break;
+        case 128: hipLaunchKernelGGL(attn_decode_fused_kernel<128>, grid, block, 0, st, p); break;
+        case 256: hipLaunchKernelGGL(attn_decode_fused_kernel<256>, grid, block, 0, st, p); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
 }
 
 hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,

@@ -177,6 +177,65 @@ static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn
     return OXB_HIP_OK;
 }
 
+// QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch; leaves the slot
+// results in m.attn_part and the parameters the merge needs in *ap.  Up to 16 q heads per kv head run in one
+// fused launch on the matrix cores; wider groups take the two-kernel route.
+static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out) {
+    const oxb_model_desc& d = m.d;
+    hipStream_t st = g_rt.stream;
+    const uint32_t qkv_rows = (d.nq + 2 * d.nkv) * d.hd;
+    OxbAttnParams ap;
+    ap.q = m.q_rope;
+    ap.qkv = m.qkv;
+    ap.qkv_stride = qkv_rows;
+    ap.q_norm = q_norm;
+    ap.k_norm = k_norm;
+    ap.cos_t = m.cos_t;
+    ap.sin_t = m.sin_t;
+    ap.eps = d.eps;
+    ap.k_cache = m.k_cache;
+    ap.v_cache = m.v_cache;
+    ap.part = m.attn_part;
+    ap.pos = m.pos;
+    ap.nq = d.nq;
+    ap.nkv = d.nkv;
+    ap.hd = d.hd;
+    ap.max_seq = d.max_seq;
+    ap.n_layers = d.n_layers;
+    ap.layer = L;
+    ap.chunk = m.chunk;
+    ap.n_splits = m.n_splits;
+    ap.scale = 1.0f / sqrtf((float)d.hd);
+    *out = ap;
+    if (d.nq / d.nkv <= 16) {
+        OXB_TRY_HIP(oxb_launch_attn_decode_fused(ap, d.batch, st), "kernel launch failed: attention");
+        return OXB_HIP_OK;
+    }
+    OxbQkParams qp;
+    qp.qkv = m.qkv;
+    qp.qkv_stride = qkv_rows;
+    qp.q_norm = q_norm;
+    qp.k_norm = k_norm;
+    qp.cos_t = m.cos_t;
+    qp.sin_t = m.sin_t;
+    qp.pos = m.pos;
+    qp.pos_base = 0;
+    qp.seq = 0;
+    qp.q_rope = m.q_rope;
+    qp.k_cache = m.k_cache;
+    qp.v_cache = m.v_cache;
+    qp.nq = d.nq;
+    qp.nkv = d.nkv;
+    qp.hd = d.hd;
+    qp.max_seq = d.max_seq;
+    qp.n_layers = d.n_layers;
+    qp.layer = L;
+    qp.eps = d.eps;
+    OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, d.batch, st), "kernel launch failed: qk_norm_rope_store");
+    OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, st), "kernel launch failed: attention");
+    return OXB_HIP_OK;
+}
+
 // Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
 // matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
 // the weights once per two sequences.
@@ -199,43 +258,8 @@ static int encode_decode_step_gemm(Model& m) {
         const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
         if (rc) return rc;
         OXB_TRY(gemm_device(*wqkv, m.hidden, d.h, m.qkv, B, qkv_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, attn_norm, d.eps, &m.gws));
-        OxbQkParams qp;
-        qp.qkv = m.qkv;
-        qp.qkv_stride = qkv_rows;
-        qp.q_norm = q_norm;
-        qp.k_norm = k_norm;
-        qp.cos_t = m.cos_t;
-        qp.sin_t = m.sin_t;
-        qp.pos = m.pos;
-        qp.pos_base = 0;
-        qp.seq = 0;
-        qp.q_rope = m.q_rope;
-        qp.k_cache = m.k_cache;
-        qp.v_cache = m.v_cache;
-        qp.nq = d.nq;
-        qp.nkv = d.nkv;
-        qp.hd = d.hd;
-        qp.max_seq = d.max_seq;
-        qp.n_layers = d.n_layers;
-        qp.layer = L;
-        qp.eps = d.eps;
-        OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, B, st), "kernel launch failed: qk_norm_rope_store");
         OxbAttnParams ap;
-        ap.q = m.q_rope;
-        ap.k_cache = m.k_cache;
-        ap.v_cache = m.v_cache;
-        ap.part = m.attn_part;
-        ap.pos = m.pos;
-        ap.nq = d.nq;
-        ap.nkv = d.nkv;
-        ap.hd = d.hd;
-        ap.max_seq = d.max_seq;
-        ap.n_layers = d.n_layers;
-        ap.layer = L;
-        ap.chunk = m.chunk;
-        ap.n_splits = m.n_splits;
-        ap.scale = 1.0f / sqrtf((float)d.hd);
-        OXB_TRY_HIP(oxb_launch_attn_decode(ap, B, st), "kernel launch failed: attention");
+        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
         OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
                     "kernel launch failed: attn_combine");
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
@@ -276,43 +300,8 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
                         "kernel launch failed: rmsnorm_quant");
             OXB_TRY(gemv_xq(*wqkv, m.xq, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows, OXB_GEMV_STORE, nullptr));
         }
-        OxbQkParams qp;
-        qp.qkv = m.qkv;
-        qp.qkv_stride = qkv_rows;
-        qp.q_norm = q_norm;
-        qp.k_norm = k_norm;
-        qp.cos_t = m.cos_t;
-        qp.sin_t = m.sin_t;
-        qp.pos = m.pos;
-        qp.pos_base = 0;
-        qp.seq = 0;
-        qp.q_rope = m.q_rope;
-        qp.k_cache = m.k_cache;
-        qp.v_cache = m.v_cache;
-        qp.nq = d.nq;
-        qp.nkv = d.nkv;
-        qp.hd = d.hd;
-        qp.max_seq = d.max_seq;
-        qp.n_layers = d.n_layers;
-        qp.layer = L;
-        qp.eps = d.eps;
-        OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, d.batch, st), "kernel launch failed: qk_norm_rope_store");
         OxbAttnParams ap;
-        ap.q = m.q_rope;
-        ap.k_cache = m.k_cache;
-        ap.v_cache = m.v_cache;
-        ap.part = m.attn_part;
-        ap.pos = m.pos;
-        ap.nq = d.nq;
-        ap.nkv = d.nkv;
-        ap.hd = d.hd;
-        ap.max_seq = d.max_seq;
-        ap.n_layers = d.n_layers;
-        ap.layer = L;
-        ap.chunk = m.chunk;
-        ap.n_splits = m.n_splits;
-        ap.scale = 1.0f / sqrtf((float)d.hd);
-        OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, st), "kernel launch failed: attention");
+        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
             OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, b0, nb, m.xq.xq, m.xq.cneg, m.xq.xexp, nullptr, st),
