@@ -72,82 +72,49 @@ __device__ __forceinline__ uint32_t unit_val_offset(uint32_t m, uint32_t bb) {
     return FMT == OXB_FMT_Q1 ? 8 * bb + 4 * m : 16 * m + 4 * bb;
 }
 
-// Digits of the 16 activations vv[bb][jj] that one lane group (blk, m, g) of the MFMA B operand holds:
-// out[d][jj] = one dword of digit plane d, cs[d] = this group's share of the block's correction sums.
+// One lane's share of the quantiser: the four activations v[bb] that register jj of lane group (blk, m, g) of the
+// MFMA B operand packs into one dword.  dig[d] = that dword of digit plane d; cs[d] = this lane's share of the
+// block's correction sums.  Zeros in give zeros out.
 template <int FMT>
-__device__ __forceinline__ void quant_unit_digits(const float (&vv)[4][4], uint32_t m, int base_shift, bool live,
-                                                  uint32_t (&out)[8][4], int (&cs)[8]) {
+__device__ __forceinline__ void quant_quarter(const float (&v)[4], uint32_t m, uint32_t jj, int base_shift,
+                                              uint32_t (&dig)[8], int (&cs)[8]) {
+    long long xi[4];
+    if (FMT == OXB_FMT_Q1) {
+        const uint32_t j = 4 * m + jj;
+        long long cr[4];
+        uint32_t cdig[8];
 #pragma unroll
-    for (int d = 0; d < 8; d++) {
-        cs[d] = 0;
-        out[d][0] = out[d][1] = out[d][2] = out[d][3] = 0;
-    }
-    if (live) {
-#pragma unroll
-        for (uint32_t jj = 0; jj < 4; jj++) {
-            long long xi[4], cr[4];
-            uint32_t dig[8], cdig[8];
-            if (FMT == OXB_FMT_Q1) {
-                const uint32_t j = 4 * m + jj;
-#pragma unroll
-                for (int bb = 0; bb < 4; bb++) {
-                    cr[bb] = scaled_rint_i64(vv[bb][jj], base_shift - (int)j);
-                    xi[bb] = (j == 7) ? -2 * cr[bb] : 2 * cr[bb];
-                }
-                digits_of4(xi, dig);
-                digits_of4(cr, cdig);
-#pragma unroll
-                for (int d = 0; d < 8; d++) cs[d] += __builtin_amdgcn_sdot4((int)cdig[d], 0x01010101, 0, false) << j;
-            } else {
-#pragma unroll
-                for (int bb = 0; bb < 4; bb++) xi[bb] = scaled_rint_i64(vv[bb][jj], base_shift - 2 * (int)jj);
-                digits_of4(xi, dig);
-                if (jj < 3) {
-#pragma unroll
-                    for (int d = 0; d < 8; d++) cs[d] += __builtin_amdgcn_sdot4((int)dig[d], 0x01010101, 0, false) << (2 * jj);
-                }
-            }
-#pragma unroll
-            for (int d = 0; d < 8; d++) out[d][jj] = dig[d];
+        for (int bb = 0; bb < 4; bb++) {
+            cr[bb] = scaled_rint_i64(v[bb], base_shift - (int)j);
+            xi[bb] = (j == 7) ? -2 * cr[bb] : 2 * cr[bb];
         }
+        digits_of4(xi, dig);
+        digits_of4(cr, cdig);
+#pragma unroll
+        for (int d = 0; d < 8; d++) cs[d] = __builtin_amdgcn_sdot4((int)cdig[d], 0x01010101, 0, false) << j;
+    } else {
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) xi[bb] = scaled_rint_i64(v[bb], base_shift - 2 * (int)jj);
+        digits_of4(xi, dig);
+#pragma unroll
+        for (int d = 0; d < 8; d++) cs[d] = jj < 3 ? __builtin_amdgcn_sdot4((int)dig[d], 0x01010101, 0, false) << (2 * jj) : 0;
     }
 }
 
-// Sum the correction shares over the eight lanes (m, g) of a block - consecutive lanes starting at a multiple
-// of eight - and return, in lane j of the eight, the sum of digit j.
-__device__ __forceinline__ int block_correction(int (&cs)[8], uint32_t lane_in_block) {
+// Sum the correction shares over the 32 lanes of a block (consecutive lanes starting at a multiple of 32) with a
+// halving exchange: every step a lane keeps half of its digits and receives the partner's share of those.
+// Returns, in every lane, the block's sum of digit 4 * bit0 + 2 * bit1 + bit2 of the lane index.
+__device__ __forceinline__ int block_correction32(const int (&cs)[8], uint32_t lane_in_block) {
+    const bool b0 = lane_in_block & 1u, b1 = lane_in_block & 2u, b2 = lane_in_block & 4u;
+    int r[4], s[2];
 #pragma unroll
-    for (int d = 0; d < 8; d++) {
-        int v = cs[d];
-        v += dpp_i32<0x141>(v);  // row_half_mirror: i <-> 7 - i
-        v += dpp_i32<0xB1>(v);   // quad_perm [1,0,3,2]
-        v += dpp_i32<0x4E>(v);   // quad_perm [2,3,0,1]
-        cs[d] = v;
-    }
-    int mine = cs[0];
+    for (int d = 0; d < 4; d++) r[d] = (b0 ? cs[d + 4] : cs[d]) + dpp_i32<0xB1>(b0 ? cs[d] : cs[d + 4]);  // quad_perm [1,0,3,2]
 #pragma unroll
-    for (int d = 1; d < 8; d++) mine = (lane_in_block == (uint32_t)d) ? cs[d] : mine;
-    return mine;
-}
-
-// Quantise the 16 activations that one lane group (blk, m, g) of the MFMA B operand holds and
-// store their eight digit planes; cs[d] returns this group's share of the block's correction sums.
-template <int FMT>
-__device__ __forceinline__ void quant_unit(const float* __restrict__ xn, uint32_t blk, uint32_t m, uint32_t g,
-                                           int base_shift, bool live, uint32_t NC, uint32_t n,
-                                           uint32_t* __restrict__ xq, int (&cs)[8]) {
-    uint32_t out[8][4];
-    float vv[4][4];  // [bb][jj]
-#pragma unroll
-    for (uint32_t bb = 0; bb < 4; bb++) {
-        float4 v4 = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (live) v4 = *reinterpret_cast<const float4*>(xn + blk * 128 + 32 * g + unit_val_offset<FMT>(m, bb));
-        vv[bb][0] = v4.x, vv[bb][1] = v4.y, vv[bb][2] = v4.z, vv[bb][3] = v4.w;
-    }
-    quant_unit_digits<FMT>(vv, m, base_shift, live, out, cs);
-    uint4* dst = reinterpret_cast<uint4*>(xq) + (size_t)((blk * 2 + m) * 4 + g) * NC + 8 * n;
-#pragma unroll
-    for (int d = 0; d < 8; d++) dst[d] = make_uint4(out[d][0], out[d][1], out[d][2], out[d][3]);
+    for (int d = 0; d < 2; d++) s[d] = (b1 ? r[d + 2] : r[d]) + dpp_i32<0x4E>(b1 ? r[d] : r[d + 2]);      // quad_perm [2,3,0,1]
+    int t = (b2 ? s[1] : s[0]) + __shfl_xor(b2 ? s[0] : s[1], 4, 64);
+    t += __shfl_xor(t, 8, 64);
+    t += __shfl_xor(t, 16, 64);
+    return t;
 }
 
 // Superblocks per exponent group and groups per vector of n_sb superblocks: the K slice of one GEMV wave
@@ -227,20 +194,33 @@ __device__ __forceinline__ void quantise_groups(const float* __restrict__ xn, ui
                                                 const uint32_t* gstat, uint32_t* __restrict__ xq,
                                                 int32_t* __restrict__ cneg, int32_t* __restrict__ xexp) {
     const uint32_t nblk = k / OXB_QK, nblk_pad = oxb_nblk_pad(k);
-    // unit u = (blk, m, g): eight consecutive lanes cover one block; a group holds gsb * 32 units
+    // Lane q = (unit u = (blk, m, g), register jj): 32 consecutive lanes cover one block; a group holds gsb * 32
+    // units.  Group and padding boundaries are multiples of 32 lanes, so the lanes of a block leave the loop together.
     const uint32_t upg = gsb * 32u, u0 = g_begin * upg;
     const uint32_t u1 = g_end * upg < nblk_pad * 8u ? g_end * upg : nblk_pad * 8u;
-    for (uint32_t u = u0 + threadIdx.x; u < u1; u += blockDim.x) {
+    for (uint32_t q = u0 * 4u + threadIdx.x; q < u1 * 4u; q += blockDim.x) {
+        const uint32_t u = q >> 2, jj = q & 3u;
         const uint32_t blk = u >> 3, m = (u >> 2) & 1u, g = u & 3u, lg = u / upg - g_begin;
         const float mx = __uint_as_float(gstat[2 * lg]);
-        const bool ok = mx > 0.0f && gstat[2 * lg + 1] == 0;
+        const bool live = mx > 0.0f && gstat[2 * lg + 1] == 0 && blk < nblk;
         int E = 0;
         if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
+        float v[4];
+#pragma unroll
+        for (uint32_t bb = 0; bb < 4; bb++) v[bb] = live ? xn[blk * 128 + 32 * g + unit_val_offset<FMT>(m, bb) + jj] : 0.f;
+        uint32_t dig[8];
         int cs[8];
-        quant_unit<FMT>(xn, blk, m, g, OXB_XQ_P - E, ok && blk < nblk, NC, n, xq, cs);
-        // lane j of the block's eight writes digit j (four copies: the MFMA takes it as a 4-register operand)
-        const int mine = block_correction(cs, u & 7u);
-        *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + (u & 7u)) * 4) = make_int4(-mine, -mine, -mine, -mine);
+        quant_quarter<FMT>(v, m, jj, OXB_XQ_P - E, dig, cs);
+        uint32_t* dst = xq + ((size_t)((blk * 2 + m) * 4 + g) * NC + 8 * n) * 4 + jj;
+#pragma unroll
+        for (int d = 0; d < 8; d++) dst[4 * d] = dig[d];
+        // the first eight lanes of the block write one digit's correction each (four copies: the MFMA takes it
+        // as a 4-register operand)
+        const int mine = block_correction32(cs, q & 31u);
+        if ((q & 24u) == 0) {
+            const uint32_t d = ((q & 1u) << 2) | (q & 2u) | ((q >> 2) & 1u);
+            *reinterpret_cast<int4*>(cneg + ((size_t)blk * NC + 8 * n + d) * 4) = make_int4(-mine, -mine, -mine, -mine);
+        }
     }
     for (uint32_t gi = g_begin + threadIdx.x; gi < g_end; gi += blockDim.x) {
         const float mx = __uint_as_float(gstat[2 * (gi - g_begin)]);
