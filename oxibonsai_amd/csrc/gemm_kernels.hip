@@ -39,7 +39,8 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 // Two kernels: row_stats (one workgroup per token row) finds the row's multiplier - the producer's scalar
 // times the power of two that puts the row's largest |a| into [2^14, 2^15) - and the exponent that undoes the
 // power of two; xh_pack (one workgroup = 16 token rows x a share of the blocks) recomputes a from x and writes
-// fp16 in MFMA B-operand order.  The fp32 activations never go to memory.
+// fp16 in MFMA B-operand order.  The fp32 activations never go to memory.  A few token rows (decode batches)
+// take both steps in one launch, xh_pack_rows, one workgroup per row.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
     const v2h h = {(_Float16)a, (_Float16)b};
@@ -47,14 +48,11 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 }
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 
+// Multiplier and exponent of one token row; all 256 threads of the workgroup call it, thread 0 gets the result.
 template <int OP>
-__global__ __launch_bounds__(256) void row_stats_kernel(const float* __restrict__ x, const float* __restrict__ w,
-                                                         uint32_t ldx, uint32_t k, float eps, float* __restrict__ rowmul,
-                                                         int32_t* __restrict__ xsh) {
-    __shared__ float red_s[4], red_m[4];
-    __shared__ int red_b[4];
-    const uint32_t m = blockIdx.x, tid = threadIdx.x;
-    const float* xr = x + (size_t)m * ldx;
+__device__ __forceinline__ void row_stats(const float* __restrict__ xr, const float* __restrict__ w, uint32_t k, float eps,
+                                          float* red_s, float* red_m, int* red_b, float* mul_out, int32_t* xsh_out) {
+    const uint32_t tid = threadIdx.x;
     float ss = 0.f, mx = 0.f;
     int bad = 0;
     for (uint32_t i = tid * 4; i < k; i += 1024) {
@@ -93,8 +91,71 @@ __global__ __launch_bounds__(256) void row_stats_kernel(const float* __restrict_
         int E = 0;
         if (mx > 0.0f) (void)frexpf(mx, &E);  // mx = f * 2^E, f in [0.5, 1)
         const int shift = mx > 0.0f ? 15 - E : 0;
-        rowmul[m] = bad ? 0.0f : ldexpf(scalar, shift);
-        xsh[m] = bad ? INT32_MIN : -shift;
+        *mul_out = bad ? 0.0f : ldexpf(scalar, shift);
+        *xsh_out = bad ? INT32_MIN : -shift;
+    }
+}
+
+template <int OP>
+__global__ __launch_bounds__(256) void row_stats_kernel(const float* __restrict__ x, const float* __restrict__ w,
+                                                         uint32_t ldx, uint32_t k, float eps, float* __restrict__ rowmul,
+                                                         int32_t* __restrict__ xsh) {
+    __shared__ float red_s[4], red_m[4];
+    __shared__ int red_b[4];
+    const uint32_t m = blockIdx.x;
+    float mul = 0.f;
+    int32_t e = 0;
+    row_stats<OP>(x + (size_t)m * ldx, w, k, eps, red_s, red_m, red_b, &mul, &e);
+    if (threadIdx.x == 0) rowmul[m] = mul, xsh[m] = e;
+}
+
+// The eight activations of token row xr that chunk c = 4g + s of block blk holds, scaled by mul, as four fp16 pairs.
+template <int FMT, int OP>
+__device__ __forceinline__ uint4 pack_item(const float* __restrict__ xr, const float* __restrict__ w, uint32_t k, uint32_t blk,
+                                           uint32_t c, float mul) {
+    const uint32_t g = c >> 2, s = c & 3u;
+    const uint32_t k0 = FMT == OXB_FMT_Q1 ? 32 * g + 4 * s : 32 * g + 16 * (s >> 1) + 4 * (s & 1u);
+    const uint32_t k1 = k0 + (FMT == OXB_FMT_Q1 ? 16 : 8);
+    const float* xb = xr + blk * 128;
+    float4 a = *reinterpret_cast<const float4*>(xb + k0);
+    float4 b = *reinterpret_cast<const float4*>(xb + k1);
+    if (OP == OXB_PACK_RMSNORM) {
+        const float4 wa = *reinterpret_cast<const float4*>(w + blk * 128 + k0), wb = *reinterpret_cast<const float4*>(w + blk * 128 + k1);
+        a = make_float4(wa.x * a.x, wa.y * a.y, wa.z * a.z, wa.w * a.w);
+        b = make_float4(wb.x * b.x, wb.y * b.y, wb.z * b.z, wb.w * b.w);
+    } else if (OP == OXB_PACK_SWIGLU) {
+        const float4 ua = *reinterpret_cast<const float4*>(xb + k + k0), ub = *reinterpret_cast<const float4*>(xb + k + k1);
+        a = make_float4(silu_mul(a.x, ua.x), silu_mul(a.y, ua.y), silu_mul(a.z, ua.z), silu_mul(a.w, ua.w));
+        b = make_float4(silu_mul(b.x, ub.x), silu_mul(b.y, ub.y), silu_mul(b.z, ub.z), silu_mul(b.w, ub.w));
+    }
+    return make_uint4(pack_h2(a.x * mul, b.x * mul), pack_h2(a.y * mul, b.y * mul), pack_h2(a.z * mul, b.z * mul),
+                      pack_h2(a.w * mul, b.w * mul));
+}
+
+// Both steps in one launch for a few token rows (decode batches): one workgroup per token row finds the row's
+// multiplier and then packs the row; rows M .. M_pad - 1 are zero-filled.  Same arithmetic as the two-kernel route.
+template <int FMT, int OP>
+__global__ __launch_bounds__(256) void xh_pack_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, uint32_t ldx,
+                                                            uint32_t k, float eps, uint32_t M, uint32_t M_pad, uint32_t nblk_pad,
+                                                            int32_t* __restrict__ xsh, uint4* __restrict__ xh) {
+    __shared__ float red_s[4], red_m[4];
+    __shared__ int red_b[4];
+    __shared__ float mul_s;
+    const uint32_t m = blockIdx.x, tid = threadIdx.x;
+    const float* xr = x + (size_t)m * ldx;
+    float mul = 0.f;
+    if (m < M) {  // uniform over the workgroup
+        int32_t e = 0;
+        row_stats<OP>(xr, w, k, eps, red_s, red_m, red_b, &mul, &e);
+        if (tid == 0) mul_s = mul, xsh[m] = e;
+        __syncthreads();
+        mul = mul_s;
+    }
+    for (uint32_t id = tid; id < nblk_pad * 16; id += 256) {
+        const uint32_t blk = id >> 4, c = id & 15u;
+        uint4 o = make_uint4(0, 0, 0, 0);
+        if (m < M && blk * 128 < k) o = pack_item<FMT, OP>(xr, w, k, blk, c, mul);
+        xh[(size_t)id * M_pad + m] = o;
     }
 }
 
@@ -103,31 +164,12 @@ __global__ __launch_bounds__(256) void xh_pack_kernel(const float* __restrict__ 
                                                        uint32_t k, uint32_t M, uint32_t M_pad, uint32_t nblk_pad,
                                                        const float* __restrict__ rowmul, uint4* __restrict__ xh) {
     const uint32_t tid = threadIdx.x, m0 = blockIdx.x * 16;
-    const uint32_t j = tid & 15u, c = tid >> 4, g = c >> 2, s = c & 3u, m = m0 + j;
+    const uint32_t j = tid & 15u, c = tid >> 4, m = m0 + j;
     const bool live = m < M;
     const float mul = live ? rowmul[m] : 0.0f;
-    const uint32_t k0 = FMT == OXB_FMT_Q1 ? 32 * g + 4 * s : 32 * g + 16 * (s >> 1) + 4 * (s & 1u);
-    const uint32_t k1 = k0 + (FMT == OXB_FMT_Q1 ? 16 : 8);
     for (uint32_t blk = blockIdx.y; blk < nblk_pad; blk += gridDim.y) {
         uint4 o = make_uint4(0, 0, 0, 0);
-        if (live && blk * 128 < k) {
-            const float* xb = x + (size_t)m * ldx + blk * 128;
-            float4 a = *reinterpret_cast<const float4*>(xb + k0);
-            float4 b = *reinterpret_cast<const float4*>(xb + k1);
-            if (OP == OXB_PACK_RMSNORM) {
-                const float4 wa = *reinterpret_cast<const float4*>(w + blk * 128 + k0), wb = *reinterpret_cast<const float4*>(w + blk * 128 + k1);
-                a = make_float4(wa.x * a.x, wa.y * a.y, wa.z * a.z, wa.w * a.w);
-                b = make_float4(wb.x * b.x, wb.y * b.y, wb.z * b.z, wb.w * b.w);
-            } else if (OP == OXB_PACK_SWIGLU) {
-                const float4 ua = *reinterpret_cast<const float4*>(xb + k + k0), ub = *reinterpret_cast<const float4*>(xb + k + k1);
-                a = make_float4(silu_mul(a.x, ua.x), silu_mul(a.y, ua.y), silu_mul(a.z, ua.z), silu_mul(a.w, ua.w));
-                b = make_float4(silu_mul(b.x, ub.x), silu_mul(b.y, ub.y), silu_mul(b.z, ub.z), silu_mul(b.w, ub.w));
-            }
-            o.x = pack_h2(a.x * mul, b.x * mul);
-            o.y = pack_h2(a.y * mul, b.y * mul);
-            o.z = pack_h2(a.z * mul, b.z * mul);
-            o.w = pack_h2(a.w * mul, b.w * mul);
-        }
+        if (live && blk * 128 < k) o = pack_item<FMT, OP>(x + (size_t)m * ldx, w, k, blk, c, mul);
         xh[(size_t)(blk * 16 + c) * M_pad + m] = o;
     }
 }
@@ -423,6 +465,121 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     }
 }
 
+// ---------------------------------------------------------------------------
+// GEMM for a few token rows (M <= 32: decode batches).  The wide kernel above would spend its time on barriers
+// and on MFMAs over padding; here the weights stream once at GEMV-like rates.  A workgroup = 8 waves owns RT row
+// tiles; the waves split K (contiguous runs of superblocks), each expands its weights and multiplies them with
+// B operands read straight from the packed activations (they stay in L2, no LDS stage, no barrier in the loop),
+// prefetched one block ahead; the eight partial sums meet in LDS and are added in wave order.
+// ---------------------------------------------------------------------------
+#define OXB_GEMM_NARROW_THREADS 512
+
+template <int FMT, int RT, int CT>
+__global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(const OxbGemmParams p) {
+    __shared__ float red[8][RT * CT * 4][64];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, g = lane >> 4;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t t0 = blockIdx.x * RT;
+    const uint32_t n_valid = p.n_tiles - t0 < (uint32_t)RT ? p.n_tiles - t0 : (uint32_t)RT;
+    const uint32_t per = (p.n_sb + 7u) / 8u, sb0 = wave * per, sb1 = min(sb0 + per, p.n_sb);
+    const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.codes, p.codes_bytes), rs = make_rsrc(p.scales, p.scales_bytes);
+    const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.xh, p.xh_bytes);
+
+    v4f acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) acc[rt][ct] = (v4f){0.f, 0.f, 0.f, 0.f};
+
+    if (sb0 < sb1) {
+        const uint32_t blk_stride = 16u * p.M_pad * 16u;  // bytes of xh per block
+        const uint32_t blk_end = sb1 * 4u;
+        // B operand of step s, token tile ct of a block: chunk 4g + s, token 16 ct + r
+        v8h B[2][4][CT];
+        auto load_b = [&](uint32_t blk, v8h (&dst)[4][CT]) {
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+#pragma unroll
+                for (int ct = 0; ct < CT; ct++) {
+                    const uint32_t off = ((4u * g + s) * p.M_pad + ct * 16u + r) * 16u;
+                    dst[s][ct] = __builtin_bit_cast(v8h, buf_load_b128(rx, blk < blk_end ? off : OXB_OOB, blk * blk_stride));
+                }
+        };
+        HalfRegs<FMT> H[RT][2], Hn[RT][2];
+#pragma unroll
+        for (int rt = 0; rt < RT; rt++) {
+            load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
+            load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
+        }
+        load_b(sb0 * 4u, B[0]);
+        for (uint32_t sb = sb0; sb < sb1; sb++) {
+            // next superblock's weights (all zero past the slice: never used)
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                load_half<FMT>(Hn[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid && sb + 1 < sb1, p.n_sb, sb + 1, 0, lane);
+                load_half<FMT>(Hn[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid && sb + 1 < sb1, p.n_sb, sb + 1, 1, lane);
+            }
+#pragma unroll
+            for (int bi = 0; bi < 4; bi++) {
+                load_b(sb * 4u + bi + 1, B[(bi + 1) & 1]);
+                BlockDec bd[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) bd[rt] = prepare_block<FMT>(H[rt][bi >> 1], bi & 1);
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    v8h A[RT];
+                    decode_step<FMT, RT>(bd, s, A);
+#pragma unroll
+                    for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+                        for (int rt = 0; rt < RT; rt++)  // row tiles past the range hold zero weights
+                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[rt], B[bi & 1][s][ct], acc[rt][ct], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) H[rt][0] = Hn[rt][0], H[rt][1] = Hn[rt][1];
+        }
+    }
+#pragma unroll
+    for (int rt = 0; rt < RT; rt++)
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) red[wave][(rt * CT + ct) * 4 + v][lane] = acc[rt][ct][v];
+    __syncthreads();
+    // wave w finishes the accumulator tiles w, w + 8, ...: lane holds rows 4g..4g+3 of row tile rt for token 16ct + r
+    const bool vec_ok = (p.ldy & 3u) == 0;
+    for (uint32_t idx = wave; idx < (uint32_t)(RT * CT); idx += 8) {
+        const uint32_t rt = idx / CT, ct = idx % CT, m = ct * 16 + r;
+        if (rt >= n_valid || m >= p.M) continue;
+        float o[4];
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            float a = red[0][idx * 4 + v][lane];
+#pragma unroll
+            for (int w = 1; w < 8; w++) a += red[w][idx * 4 + v][lane];
+            o[v] = a;
+        }
+        const int e = p.xsh[m];
+#pragma unroll
+        for (int v = 0; v < 4; v++) o[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(o[v], e);
+        float* yr = p.y + (size_t)m * p.ldy;
+        const float* rr = p.mode == OXB_GEMM_RESIDUAL ? p.residual + (size_t)m * p.ldy : nullptr;
+        const uint32_t n = (t0 + rt) * 16 + 4 * g;
+        if (vec_ok && n + 3 < p.n_rows) {
+            if (rr) {
+                const float4 q4 = *reinterpret_cast<const float4*>(rr + n);
+                o[0] += q4.x, o[1] += q4.y, o[2] += q4.z, o[3] += q4.w;
+            }
+            *reinterpret_cast<float4*>(yr + n) = make_float4(o[0], o[1], o[2], o[3]);
+        } else {
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                if (n + v < p.n_rows) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
+        }
+    }
+}
+
 // y = (residual +) the K slices' partial sums, added in slice order (deterministic).
 __global__ __launch_bounds__(256) void gemm_splitk_reduce_kernel(const float* __restrict__ part, uint32_t ksplit, size_t plane,
                                                                   const float* __restrict__ residual, float* __restrict__ y,
@@ -449,9 +606,20 @@ size_t oxb_xh_bytes(uint32_t k, uint32_t M) {
     return nblk_pad * 16 * M_pad * 16;
 }
 
+#define OXB_PACK_ROWS_MAX 64  // up to this many token rows the one-launch packer is used
+
 template <int OP>
 static void launch_pack_op(int fmt, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, uint32_t M, uint32_t M_pad,
                            uint32_t nblk_pad, float eps, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st) {
+    if (M <= OXB_PACK_ROWS_MAX) {
+        if (fmt == OXB_FMT_Q1)
+            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_Q1, OP>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, M_pad,
+                               nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));
+        else
+            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_TQ2, OP>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, M_pad,
+                               nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));
+        return;
+    }
     hipLaunchKernelGGL(row_stats_kernel<OP>, dim3(M), dim3(256), 0, st, d_x, d_w, ldx, k, eps, d_rowmul, d_xsh);
     const dim3 grid(M_pad / 16, nblk_pad < 16 ? nblk_pad : 16);
     if (fmt == OXB_FMT_Q1)
@@ -512,16 +680,42 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
     return best;
 }
 
+template <int FMT, int RT, int CT>
+static hipError_t launch_narrow_case(const OxbGemmParams& p, hipStream_t st) {
+    hipLaunchKernelGGL((gemm_narrow_kernel<FMT, RT, CT>), dim3((p.n_tiles + RT - 1) / RT), dim3(OXB_GEMM_NARROW_THREADS), 0, st, p);
+    return hipGetLastError();
+}
+
+// Row tiles per workgroup: as many as still leave about one workgroup per CU (every workgroup reads all of the
+// packed activations, so fewer, fatter workgroups mean less traffic out of L2).
+static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
+    p.ksplit = 1;
+    p.sb_per_split = p.n_sb;
+    const uint32_t rt = p.n_tiles >= 4 * n_cus ? 4 : (p.n_tiles >= 2 * n_cus ? 2 : 1);
+    const uint32_t ct = p.M_pad / 16;
+#define OXB_NARROW_CASE(F, R, C) \
+    if (fmt == F && rt == R && ct == C) return launch_narrow_case<F, R, C>(p, st);
+    OXB_NARROW_CASE(OXB_FMT_Q1, 1, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 2, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 4, 1)
+    OXB_NARROW_CASE(OXB_FMT_Q1, 1, 2) OXB_NARROW_CASE(OXB_FMT_Q1, 2, 2) OXB_NARROW_CASE(OXB_FMT_Q1, 4, 2)
+    OXB_NARROW_CASE(OXB_FMT_TQ2, 1, 1) OXB_NARROW_CASE(OXB_FMT_TQ2, 2, 1) OXB_NARROW_CASE(OXB_FMT_TQ2, 4, 1)
+    OXB_NARROW_CASE(OXB_FMT_TQ2, 1, 2) OXB_NARROW_CASE(OXB_FMT_TQ2, 2, 2) OXB_NARROW_CASE(OXB_FMT_TQ2, 4, 2)
+#undef OXB_NARROW_CASE
+    return hipErrorInvalidValue;
+}
+
+#define OXB_GEMM_NARROW_MAX_M 32  // up to this many token rows the narrow kernel is used
+
 uint32_t oxb_gemm_ksplit(const OxbGemmParams& p, uint32_t n_cus) {
-    if (p.M == 0 || p.n_rows == 0 || p.n_sb == 0) return 1;
+    if (p.M == 0 || p.n_rows == 0 || p.n_sb == 0 || p.M <= OXB_GEMM_NARROW_MAX_M) return 1;
     return plan_gemm(p, n_cus).ksplit;
 }
 
 hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
     if (p.M == 0 || p.n_rows == 0) return hipSuccess;
     if (p.n_sb == 0 || (uint64_t)p.n_tiles * p.n_sb * 2048ull >= 0xFFFFFFF0ull) return hipErrorInvalidValue;
-    constexpr uint32_t CT = 8, BM = 16 * CT;
     p.M_pad = (p.M + 15u) / 16u * 16u;
+    if (p.M <= OXB_GEMM_NARROW_MAX_M) return launch_gemm_narrow(fmt, p, n_cus, st);
+    constexpr uint32_t CT = 8, BM = 16 * CT;
     p.n_mt = (p.M + BM - 1) / BM;
     const GemmPlan plan = plan_gemm(p, n_cus);
     const uint32_t best_rt = plan.rt, best_tpw = plan.tpw;

@@ -409,6 +409,28 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     _Float16* Kc = reinterpret_cast<_Float16*>(p.k_cache) + base;
     _Float16* Vc = reinterpret_cast<_Float16*>(p.v_cache) + base;
 
+    // K rows of the two 16-key tiles (A operands) and this lane's pieces of the 32-key V block of a chunk.
+    // Rows past the last key repeat it; their scores are masked.
+    v8h_t k0r[KS], k1r[KS];
+    v4i vr[VL];
+    auto load_k = [&](uint32_t chunk) {
+        const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
+        const uint32_t kr0 = min(key0 + qi, seq_len - 1), kr1 = min(key0 + 16 + qi, seq_len - 1);
+#pragma unroll
+        for (int s = 0; s < KS; s++) {
+            k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
+            k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
+        }
+    };
+    auto load_v = [&](uint32_t chunk) {
+        const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
+#pragma unroll
+        for (int i = 0; i < VL; i++) {
+            const uint32_t id = i * 64 + lane, row = min(key0 + id / (HD / 8), seq_len - 1), col = id % (HD / 8);
+            vr[i] = *reinterpret_cast<const v4i*>(Vc + (size_t)row * HD + col * 8);
+        }
+    };
+
     // --- Q of the group's heads: RMSNorm over the head, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd) ---
     for (uint32_t h = wave; h < G; h += 4) {
         const float* in = qkv + (size_t)(h0 + h) * HD;
@@ -443,6 +465,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     }
     __syncthreads();  // publishes qs and, within this workgroup, the new cache rows
+    load_k(slot);
+    load_v(slot);
 
     // B operands: lane (head = qi, g) holds Q[head][32 s + 8 g .. + 7] as hi + lo
     v8h_t qh[KS], ql[KS];
@@ -463,20 +487,15 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
 
     for (uint32_t chunk = slot; chunk < n_chunks; chunk += p.n_splits) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
-        if (key0 >= seq_len) continue;  // this wave's quarter of the last chunk is empty
-        const uint32_t kr0 = min(key0 + qi, seq_len - 1), kr1 = min(key0 + 16 + qi, seq_len - 1);
-        v8h_t k0r[KS], k1r[KS];
-        v4i vr[VL];
-#pragma unroll
-        for (int s = 0; s < KS; s++) {
-            k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
-            k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
-        }
+        const bool more = chunk + p.n_splits < n_chunks;
+        // stage the V block in the wave's LDS slice (the previous block's gathers were issued before: LDS runs in
+        // order) and request the next chunk's
 #pragma unroll
         for (int i = 0; i < VL; i++) {
-            const uint32_t id = i * 64 + lane, row = min(key0 + id / (HD / 8), seq_len - 1), col = id % (HD / 8);
-            vr[i] = *reinterpret_cast<const v4i*>(Vc + (size_t)row * HD + col * 8);
+            const uint32_t id = i * 64 + lane;
+            *reinterpret_cast<v4i*>(vs + (id / (HD / 8)) * VSTR + (id % (HD / 8)) * 8) = vr[i];
         }
+        if (more) load_v(chunk + p.n_splits);
         v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; s++) {
@@ -485,6 +504,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], qh[s], s1, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], ql[s], s1, 0, 0, 0);
         }
+        if (more) load_k(chunk + p.n_splits);
+        if (key0 >= seq_len) continue;  // this wave's quarter of the last chunk is empty
         // this lane: head qi, keys key0 + 4g + v and key0 + 16 + 4g + v
         float sv[8];
         float mx = -INFINITY;
@@ -512,12 +533,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         sum += __shfl_xor(sum, 32, 64);
         l_run = l_run * alpha + sum;
         m_run = m_new;
-        // stage the V block in the wave's LDS slice, then gather the transposed operand
-#pragma unroll
-        for (int i = 0; i < VL; i++) {
-            const uint32_t id = i * 64 + lane;
-            *reinterpret_cast<v4i*>(vs + (id / (HD / 8)) * VSTR + (id % (HD / 8)) * 8) = vr[i];
-        }
+        // O^T += V^T P^T; A operand gathered from the staged block
 #pragma unroll
         for (int sl = 0; sl < NS; sl++) {
             v8h_t a;

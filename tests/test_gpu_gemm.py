@@ -41,7 +41,10 @@ def _check_against_truth(got, w64, x, extra=0.0):
 
 @pytest.mark.parametrize("fmt", [Q1, TQ2])
 @pytest.mark.parametrize("shape", [(1, 16, 128), (17, 40, 256), (33, 100, 640), (128, 256, 1024), (130, 250, 1152),
-                                   (300, 70, 2048), (16, 1, 512), (15, 17, 384), (129, 333, 128)])
+                                   (300, 70, 2048), (16, 1, 512), (15, 17, 384), (129, 333, 128),
+                                   # few token rows (decode batches): 1, 2 and 4 row tiles per workgroup, K runs
+                                   # that do not divide by the eight waves, one and two token tiles
+                                   (8, 8200, 256), (32, 16400, 128), (20, 4100, 1152), (5, 48, 12288), (31, 9000, 1536)])
 def test_gemm_matches_oracle(backend, fmt, shape):
     m, n, k = shape
     a = synth.make_blocks(fmt, 900 + m + n, n, k)
@@ -54,10 +57,11 @@ def test_gemm_matches_oracle(backend, fmt, shape):
 
 
 @pytest.mark.parametrize("fmt", [Q1, TQ2])
-def test_gemm_is_bit_exact_on_fp16_representable_inputs(backend, fmt):
+@pytest.mark.parametrize("m,n", [(48, 64), (24, 64), (9, 8208)])
+def test_gemm_is_bit_exact_on_fp16_representable_inputs(backend, fmt, m, n):
     # integer activations below 2048 and power-of-two scales: every product and every partial sum is an exact
     # fp32 number, so any disagreement in the k order of the two MFMA operands shows as a wrong integer
-    m, n, k = 48, 64, 640
+    k = 640
     rng = np.random.default_rng(5)
     bpr = k // 128
     blocks = []
