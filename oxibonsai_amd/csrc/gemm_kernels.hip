@@ -479,8 +479,14 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
     __shared__ float red[8][RT * CT * 4][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
-    const uint32_t t0 = blockIdx.x * RT;
-    const uint32_t n_valid = p.n_tiles - t0 < (uint32_t)RT ? p.n_tiles - t0 : (uint32_t)RT;
+    // Row tiles of this workgroup.  Plain modes: RT consecutive tiles.  SWIGLU mode (the matrix is gate || up,
+    // RT even): RT/2 consecutive gate tiles and the up tiles of the same rows, so the epilogue holds both factors.
+    const bool sw = p.mode == OXB_GEMM_SWIGLU;
+    constexpr uint32_t HP = RT > 1 ? RT / 2 : 1;
+    const uint32_t t0 = sw ? blockIdx.x * HP : blockIdx.x * RT;
+    const uint32_t t_lim = sw ? p.n_tiles / 2 : p.n_tiles;
+    auto tile_of = [&](int rt) -> uint32_t { return sw ? ((uint32_t)rt < HP ? t0 + rt : p.n_tiles / 2 + t0 + rt - HP) : t0 + rt; };
+    auto valid = [&](int rt) -> bool { return sw ? t0 + ((uint32_t)rt % HP) < t_lim : t0 + rt < t_lim; };
     const uint32_t per = (p.n_sb + 7u) / 8u, sb0 = wave * per, sb1 = min(sb0 + per, p.n_sb);
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.codes, p.codes_bytes), rs = make_rsrc(p.scales, p.scales_bytes);
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.xh, p.xh_bytes);
@@ -508,16 +514,16 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
         HalfRegs<FMT> H[RT][2], Hn[RT][2];
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
-            load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
-            load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
+            load_half<FMT>(H[rt][0], rc, rs, tile_of(rt), valid(rt), p.n_sb, sb0, 0, lane);
+            load_half<FMT>(H[rt][1], rc, rs, tile_of(rt), valid(rt), p.n_sb, sb0, 1, lane);
         }
         load_b(sb0 * 4u, B[0]);
         for (uint32_t sb = sb0; sb < sb1; sb++) {
             // next superblock's weights (all zero past the slice: never used)
 #pragma unroll
             for (int rt = 0; rt < RT; rt++) {
-                load_half<FMT>(Hn[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid && sb + 1 < sb1, p.n_sb, sb + 1, 0, lane);
-                load_half<FMT>(Hn[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid && sb + 1 < sb1, p.n_sb, sb + 1, 1, lane);
+                load_half<FMT>(Hn[rt][0], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 0, lane);
+                load_half<FMT>(Hn[rt][1], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 1, lane);
             }
 #pragma unroll
             for (int bi = 0; bi < 4; bi++) {
@@ -549,24 +555,32 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
     __syncthreads();
     // wave w finishes the accumulator tiles w, w + 8, ...: lane holds rows 4g..4g+3 of row tile rt for token 16ct + r
     const bool vec_ok = (p.ldy & 3u) == 0;
-    for (uint32_t idx = wave; idx < (uint32_t)(RT * CT); idx += 8) {
-        const uint32_t rt = idx / CT, ct = idx % CT, m = ct * 16 + r;
-        if (rt >= n_valid || m >= p.M) continue;
-        float o[4];
+    auto total = [&](uint32_t idx, float (&o)[4], int e) {
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             float a = red[0][idx * 4 + v][lane];
 #pragma unroll
             for (int w = 1; w < 8; w++) a += red[w][idx * 4 + v][lane];
-            o[v] = a;
+            o[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(a, e);
         }
+    };
+    const uint32_t n_out = sw ? HP * CT : RT * CT;
+    for (uint32_t idx = wave; idx < n_out; idx += 8) {
+        const uint32_t rt = idx / CT, ct = idx % CT, m = ct * 16 + r;
+        if (!valid((int)rt) || m >= p.M) continue;
         const int e = p.xsh[m];
+        float o[4];
+        total(idx, o, e);
+        if (sw) {  // y[m][row] = silu(gate) * up, rows counted within the gate half
+            float u[4];
+            total((rt + HP) * CT + ct, u, e);
 #pragma unroll
-        for (int v = 0; v < 4; v++) o[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(o[v], e);
+            for (int v = 0; v < 4; v++) o[v] = silu_mul(o[v], u[v]);
+        }
         float* yr = p.y + (size_t)m * p.ldy;
         const float* rr = p.mode == OXB_GEMM_RESIDUAL ? p.residual + (size_t)m * p.ldy : nullptr;
-        const uint32_t n = (t0 + rt) * 16 + 4 * g;
-        if (vec_ok && n + 3 < p.n_rows) {
+        const uint32_t n = (t0 + rt) * 16 + 4 * g, n_lim = sw ? p.n_rows / 2 : p.n_rows;
+        if (vec_ok && n + 3 < n_lim) {
             if (rr) {
                 const float4 q4 = *reinterpret_cast<const float4*>(rr + n);
                 o[0] += q4.x, o[1] += q4.y, o[2] += q4.z, o[3] += q4.w;
@@ -575,7 +589,7 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
         } else {
 #pragma unroll
             for (int v = 0; v < 4; v++)
-                if (n + v < p.n_rows) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
+                if (n + v < n_lim) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
         }
     }
 }
@@ -682,7 +696,8 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
 
 template <int FMT, int RT, int CT>
 static hipError_t launch_narrow_case(const OxbGemmParams& p, hipStream_t st) {
-    hipLaunchKernelGGL((gemm_narrow_kernel<FMT, RT, CT>), dim3((p.n_tiles + RT - 1) / RT), dim3(OXB_GEMM_NARROW_THREADS), 0, st, p);
+    const uint32_t grid = p.mode == OXB_GEMM_SWIGLU ? (p.n_tiles / 2 + RT / 2 - 1) / (RT > 1 ? RT / 2 : 1) : (p.n_tiles + RT - 1) / RT;
+    hipLaunchKernelGGL((gemm_narrow_kernel<FMT, RT, CT>), dim3(grid), dim3(OXB_GEMM_NARROW_THREADS), 0, st, p);
     return hipGetLastError();
 }
 
@@ -691,7 +706,11 @@ static hipError_t launch_narrow_case(const OxbGemmParams& p, hipStream_t st) {
 static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
     p.ksplit = 1;
     p.sb_per_split = p.n_sb;
-    const uint32_t rt = p.n_tiles >= 4 * n_cus ? 4 : (p.n_tiles >= 2 * n_cus ? 2 : 1);
+    uint32_t rt = p.n_tiles >= 4 * n_cus ? 4 : (p.n_tiles >= 2 * n_cus ? 2 : 1);
+    if (p.mode == OXB_GEMM_SWIGLU) {
+        if ((p.n_rows & 31u) != 0) return hipErrorInvalidValue;  // gate and up halves of whole row tiles
+        if (rt < 2) rt = 2;
+    }
     const uint32_t ct = p.M_pad / 16;
 #define OXB_NARROW_CASE(F, R, C) \
     if (fmt == F && rt == R && ct == C) return launch_narrow_case<F, R, C>(p, st);
@@ -703,7 +722,6 @@ static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, h
     return hipErrorInvalidValue;
 }
 
-#define OXB_GEMM_NARROW_MAX_M 32  // up to this many token rows the narrow kernel is used
 
 uint32_t oxb_gemm_ksplit(const OxbGemmParams& p, uint32_t n_cus) {
     if (p.M == 0 || p.n_rows == 0 || p.n_sb == 0 || p.M <= OXB_GEMM_NARROW_MAX_M) return 1;
@@ -715,6 +733,7 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     if (p.n_sb == 0 || (uint64_t)p.n_tiles * p.n_sb * 2048ull >= 0xFFFFFFF0ull) return hipErrorInvalidValue;
     p.M_pad = (p.M + 15u) / 16u * 16u;
     if (p.M <= OXB_GEMM_NARROW_MAX_M) return launch_gemm_narrow(fmt, p, n_cus, st);
+    if (p.mode == OXB_GEMM_SWIGLU) return hipErrorInvalidValue;  // only the narrow kernel has that epilogue
     constexpr uint32_t CT = 8, BM = 16 * CT;
     p.n_mt = (p.M + BM - 1) / BM;
     const GemmPlan plan = plan_gemm(p, n_cus);

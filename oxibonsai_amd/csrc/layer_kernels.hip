@@ -393,8 +393,10 @@ typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 template <int HD>
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p) {
     constexpr int KS = HD / 32, NS = HD / 16, VL = HD / 16, VSTR = HD + 8;
-    __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];  // V block per wave; later the merge buffers
-    __shared__ float qs[16 * HD];                                           // Q * scale of the group's heads
+    // V block per wave; before the loop its start holds Q * scale of the group's heads, after it the merge buffers
+    __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];
+    static_assert(sizeof(vs_all) >= 16 * HD * sizeof(float), "Q must fit in the V slices");
+    float* qs = reinterpret_cast<float*>(&vs_all[0][0]);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t slot = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
@@ -479,6 +481,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             qh[s][e] = hi;
             ql[s][e] = (_Float16)(x - (float)hi);
         }
+    __syncthreads();  // Q is in registers everywhere: its LDS copy may be overwritten
     v4f O[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};

@@ -263,8 +263,13 @@ static int encode_decode_step_gemm(Model& m) {
         OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
                     "kernel launch failed: attn_combine");
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
-        OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
-        OXB_TRY(gemm_device(*wdn, m.gu, 2 * d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_SWIGLU, nullptr, 0.f, &m.gws));
+        if (B <= OXB_GEMM_NARROW_MAX_M) {  // SwiGLU in the epilogue of the gate || up product
+            OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
+            OXB_TRY(gemm_device(*wdn, m.gu, d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
+        } else {
+            OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
+            OXB_TRY(gemm_device(*wdn, m.gu, 2 * d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_SWIGLU, nullptr, 0.f, &m.gws));
+        }
     }
     const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
     const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);

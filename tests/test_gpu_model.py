@@ -153,9 +153,10 @@ def test_batch_ffn_phase_matches_oracle(backend, fmt):
     assert np.max(np.abs(got - want)) < 1e-4 * np.max(np.abs(want))
 
 
-@pytest.mark.parametrize("nq,nkv,hd", [(8, 1, 32), (6, 2, 64), (5, 1, 128), (2, 2, 64)])
+@pytest.mark.parametrize("nq,nkv,hd", [(8, 1, 32), (6, 2, 64), (5, 1, 128), (2, 2, 64), (20, 1, 32)])
 def test_gqa_group_shapes(backend, nq, nkv, hd):
-    # 8, 3, 5 and 1 query heads per kv head: groups above four are split over several attention workgroups
+    # 8, 3, 5 and 1 query heads per kv head share one attention workgroup (up to 16 do); 20 take the route with
+    # separate QK-norm / RoPE / KV-store and attention kernels
     h = nq * hd if (nq * hd) % 128 == 0 else 128 * ((nq * hd + 127) // 128)
     cfg = dict(n_layers=2, h=256, inter=384, nq=nq, nkv=nkv, hd=hd, vocab=64, max_seq=320, eps=1e-6, rope_theta=1e4, fmt=TQ2)
     if (nq * hd) % 128:
@@ -176,17 +177,17 @@ def test_gqa_group_shapes(backend, nq, nkv, hd):
 
 
 @pytest.mark.parametrize("fmt", [TQ2, Q1])
-def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt):
+@pytest.mark.parametrize("B", [9, 20, 40])   # one and two token tiles of the narrow GEMM, then the wide one
+def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt, B):
     """From 8 sequences on, a decode step sends its projections through the prefill GEMM (fp16 activations):
     logits are held to the prefill tolerance 1e-2 under the reference's gate form; the step is still replayed
     from a captured graph and sequences stay independent."""
     cfg = dict(SMALL, fmt=fmt)
     w = synth.make_model(cfg, 61 + fmt)
-    B = 9
     gpu = HipModel(backend, cfg, w, batch=B)
     cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
     try:
-        for step in range(6):
+        for step in range(4):
             hidden = np.stack([synth.embedding_rows(70 + b, [3 * step + b], cfg["h"])[0] * 50.0 for b in range(B)])
             got, toks = gpu.forward(hidden, np.full(B, step, dtype=np.uint32))
             for b in range(B):
