@@ -18,8 +18,7 @@ struct OxbQkParams {
 };
 
 struct OxbAttnParams {
-    const float* q;                      // [batch][nq][hd] after QK-norm and RoPE (attn_decode_kernel only)
-    // attn_decode_fused_kernel reads the raw projections instead and does QK-norm, RoPE and the KV store itself
+    // the attention kernel reads the raw projections and does QK-norm, RoPE and the KV store itself
     const float* qkv;                    // [batch][qkv_stride]: q heads | k heads | v heads
     uint32_t qkv_stride;
     const float *q_norm, *k_norm;        // [hd]
@@ -42,12 +41,10 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 #define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers at a time
 #define OXB_ATTN_MAX_SPLITS 64        // slots the KV sequence is split over; slot s walks chunks s, s + n_splits, ...
 #define OXB_ATTN_PART_PAD 4           // floats after the hd outputs of a slot: maximum, sum, 2 unused (16-byte rows)
-// Split-KV attention into p.part, then the merge of the slots fused with the quantiser of the O projection's
-// input for sequences b0 .. b0 + nb - 1 (nb <= 2); d_out_or_null also receives the fp32 attention output [batch][nq*hd].
+// QK-norm, RoPE, KV store of the new position and split-KV attention (at most 16 q heads per kv head) into
+// p.part, then the merge of the slots fused with the quantiser of the O projection's input for sequences
+// b0 .. b0 + nb - 1 (nb <= 2); d_out_or_null also receives the fp32 attention output [batch][nq*hd].
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
-// The same attention on the matrix cores, fused with QK-norm, RoPE and the KV store of the new position
-// (qkv, q_norm, k_norm, cos_t, sin_t, eps set; q unused).  Writes the same p.part layout.
-hipError_t oxb_launch_attn_decode_fused(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
 hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
                                          int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.

@@ -165,220 +165,17 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
     }
 }
 
+#define OXB_ATTN_CHUNK 128  // KV positions per chunk of the split-KV decode attention
+
 // ---------------------------------------------------------------------------
-// Decode attention, split over the KV sequence (flash-decode).  softmax(q K^T / sqrt(hd)) V with
-// GQA (kv_head = q_head / (nq / nkv)) over positions 0..pos[b]
+// Decode attention, split over the KV sequence (flash-decode), on the matrix cores: softmax(q K^T / sqrt(hd)) V
+// with GQA (kv_head = q_head / (nq / nkv)) over positions 0..pos[b]
 // (batched_attn_scores_v2 / batched_softmax / batched_attn_weighted_sum, cuda_attn_kernels.rs:264-438;
-//  CPU: block/functions.rs:78-127 -> layers/attention_fused.rs:329-400).
-// Grid (n_splits, nkv, batch), 256 threads.  A workgroup serves all q heads of one kv head for one
-// chunk of positions, so K and V are read once per group: scores with one position per thread,
-// then the weighted sum with eight head dimensions and a slice of the positions per thread.  It writes the un-normalised partial
-// output, the chunk maximum and the chunk sum; attn_combine_kernel merges the chunks.
-// ---------------------------------------------------------------------------
-#define OXB_ATTN_THREADS 256
-#define OXB_ATTN_CHUNK 128  // KV positions per workgroup
-
-__device__ __forceinline__ void unpack8(const v4i& u, float f[8]) {
-    const __half2* h2 = reinterpret_cast<const __half2*>(&u);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const float2 t = __half22float2(h2[i]);
-        f[2 * i] = t.x;
-        f[2 * i + 1] = t.y;
-    }
-}
-
-// HD = head dimension, GM = q heads per kv head rounded up to a power of two (loops over heads are
-// unrolled to GM and predicated on the real count G).
-template <int HD, int GM>
-__global__ __launch_bounds__(OXB_ATTN_THREADS) void attn_decode_kernel(OxbAttnParams p) {
-    constexpr int NG = HD / 8;                       // 16-byte groups per row
-    constexpr int NSL = OXB_ATTN_THREADS / NG;       // position slices in the weighted-sum phase
-    constexpr int PPS = OXB_ATTN_CHUNK / NSL;        // positions per slice
-    __shared__ float sc[GM * OXB_ATTN_CHUNK];
-    __shared__ float red[GM * 4];
-    __shared__ float accs[NSL * GM * HD];
-    // blockIdx.y = kv head * nsub + sub: with more than GM q heads per kv head the group is served
-    // by nsub workgroups of up to GM heads each
-    const uint32_t nsub = gridDim.y / p.nkv, kvh = blockIdx.y / nsub, sub = blockIdx.y % nsub;
-    const uint32_t split = blockIdx.x, b = blockIdx.z, tid = threadIdx.x;
-    const uint32_t Gall = p.nq / p.nkv, h0 = kvh * Gall + sub * GM;  // first q head served here
-    const uint32_t G = (Gall - sub * GM) < (uint32_t)GM ? (Gall - sub * GM) : (uint32_t)GM;
-    const uint32_t seq_len = p.pos[b] + 1;
-    const uint32_t n_chunks = (seq_len + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK;
-    // slot `split` takes chunks split, split + n_splits, ...; slots past the last chunk are never read
-    if (split >= n_chunks) return;
-    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + split) * (HD + OXB_ATTN_PART_PAD);
-    const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
-    const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * HD;
-    const __half* K = p.k_cache + base;
-    const __half* V = p.v_cache + base;
-    const __amdgpu_buffer_rsrc_t rk = make_rsrc(K, p.max_seq * HD * 2u), rv = make_rsrc(V, p.max_seq * HD * 2u);
-    // running result over this slot's chunks: thread -> outputs i = tid, tid + 256, ... of the G * HD
-    constexpr int OPT = (GM * HD + OXB_ATTN_THREADS - 1) / OXB_ATTN_THREADS;
-    float run_o[OPT], run_m[OPT], run_l[OPT];
-#pragma unroll
-    for (int j = 0; j < OPT; j++) run_o[j] = 0.f, run_m[j] = -INFINITY, run_l[j] = 0.f;
-
-    for (uint32_t chunk = split; chunk < n_chunks; chunk += p.n_splits) {
-    const uint32_t s0 = chunk * OXB_ATTN_CHUNK;
-    const uint32_t s1 = (s0 + OXB_ATTN_CHUNK) < seq_len ? (s0 + OXB_ATTN_CHUNK) : seq_len;
-    const uint32_t t = s0 + tid;
-    const bool live = tid < OXB_ATTN_CHUNK && t < s1;  // the threads that own one position in the softmax phase
-
-    // scores: lanes walk the K rows 16 bytes at a time, so one wave load covers whole rows back to
-    // back (fully coalesced); every pass handles RPP rows of the chunk, all passes are in flight at once
-    constexpr int RPP = OXB_ATTN_THREADS / NG, NPASS = OXB_ATTN_CHUNK / RPP;
-    const uint32_t ch = tid % NG, rr = tid / NG;
-    float qf[GM][8];  // this lane's 8 dimensions of every q head
-#pragma unroll
-    for (int h = 0; h < GM; h++) {
-        if ((uint32_t)h < G) {
-            const float* qp = p.q + ((size_t)b * p.nq + h0 + h) * HD + ch * 8;
-            const float4 qa = *reinterpret_cast<const float4*>(qp), qb = *reinterpret_cast<const float4*>(qp + 4);
-            qf[h][0] = qa.x; qf[h][1] = qa.y; qf[h][2] = qa.z; qf[h][3] = qa.w;
-            qf[h][4] = qb.x; qf[h][5] = qb.y; qf[h][6] = qb.z; qf[h][7] = qb.w;
-        } else {
-#pragma unroll
-            for (int j = 0; j < 8; j++) qf[h][j] = 0.f;
-        }
-    }
-    // K rows of the score phase and V rows of the weighted-sum phase, all requested now: both depend
-    // only on pos.  Buffer loads return 0 past s1 without a branch or a select after the load.
-    v4i kreg[NPASS];
-#pragma unroll
-    for (int i = 0; i < NPASS; i++) {
-        const uint32_t tk = s0 + (uint32_t)i * RPP + rr;
-        kreg[i] = buf_load_b128(rk, tk < s1 ? (tk * HD + ch * 8u) * 2u : OXB_OOB);
-    }
-    const uint32_t grp = tid % NG, slice = tid / NG;
-    v4i vreg[PPS];
-#pragma unroll
-    for (int i = 0; i < PPS; i++) {
-        const uint32_t tv = s0 + slice + (uint32_t)i * NSL;
-        vreg[i] = buf_load_b128(rv, tv < s1 ? (tv * HD + grp * 8u) * 2u : OXB_OOB);
-    }
-    float lmax[GM];
-#pragma unroll
-    for (int h = 0; h < GM; h++) lmax[h] = -INFINITY;
-#pragma unroll
-    for (int i = 0; i < NPASS; i++) {
-        float kf[8];
-        unpack8(kreg[i], kf);
-        const uint32_t lt = (uint32_t)i * RPP + rr;  // position within the chunk
-#pragma unroll
-        for (int h = 0; h < GM; h++) {
-            float d = 0.f;
-#pragma unroll
-            for (int j = 0; j < 8; j++) d = fmaf(qf[h][j], kf[j], d);
-            // add the NG partial sums of the row: they sit in consecutive lanes
-            d += dpp_f32<0x111>(d);                    // row_shr:1
-            if (NG > 2) d += dpp_f32<0x112>(d);        // row_shr:2
-            if (NG > 4) d += dpp_f32<0x114>(d);        // row_shr:4
-            if (NG > 8) d += dpp_f32<0x118>(d);        // row_shr:8
-            if (NG > 16) d += __shfl_up(d, 16, 64);    // head_dim 256: two 16-lane rows per K row
-            if (ch == NG - 1 && (uint32_t)h < G) {
-                const float sv = (s0 + lt < s1) ? d * p.scale : -INFINITY;
-                sc[h * OXB_ATTN_CHUNK + lt] = sv;
-                lmax[h] = fmaxf(lmax[h], sv);
-            }
-        }
-    }
-    // chunk maximum per head
-    float m[GM];
-#pragma unroll
-    for (int h = 0; h < GM; h++) {
-        float sv = lmax[h];
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) sv = fmaxf(sv, __shfl_xor(sv, o, 64));
-        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = sv;
-    }
-    __syncthreads();  // also publishes the scores
-#pragma unroll
-    for (int h = 0; h < GM; h++) m[h] = fmaxf(fmaxf(red[h * 4], red[h * 4 + 1]), fmaxf(red[h * 4 + 2], red[h * 4 + 3]));
-    __syncthreads();
-    // exponentials and their sum: one position per thread
-#pragma unroll
-    for (int h = 0; h < GM; h++) {
-        float e = 0.f;
-        if ((uint32_t)h < G) {
-            if (tid < OXB_ATTN_CHUNK) {
-                e = live ? expf(sc[h * OXB_ATTN_CHUNK + tid] - m[h]) : 0.f;
-                sc[h * OXB_ATTN_CHUNK + tid] = e;
-            }
-        }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) e += __shfl_xor(e, o, 64);
-        if ((tid & 63u) == 0) red[h * 4 + (tid >> 6)] = e;
-    }
-    __syncthreads();  // publishes the exponentials and the per-wave sums
-    // weighted sum of V: thread -> (group of 8 dimensions, slice of positions)
-    float acc[GM][8];
-#pragma unroll
-    for (int h = 0; h < GM; h++)
-#pragma unroll
-        for (int i = 0; i < 8; i++) acc[h][i] = 0.f;
-#pragma unroll
-    for (int i = 0; i < PPS; i++) {
-        float vf[8];
-        unpack8(vreg[i], vf);
-        const uint32_t lt = slice + (uint32_t)i * NSL;  // position within the chunk; exponentials past s1 are 0
-#pragma unroll
-        for (int h = 0; h < GM; h++) {
-            if ((uint32_t)h < G) {
-                const float pr = sc[h * OXB_ATTN_CHUNK + lt];
-#pragma unroll
-                for (int j = 0; j < 8; j++) acc[h][j] = fmaf(pr, vf[j], acc[h][j]);
-            }
-        }
-    }
-#pragma unroll
-    for (int h = 0; h < GM; h++)
-        if ((uint32_t)h < G) {
-            *reinterpret_cast<float4*>(&accs[(slice * GM + h) * HD + grp * 8]) = make_float4(acc[h][0], acc[h][1], acc[h][2], acc[h][3]);
-            *reinterpret_cast<float4*>(&accs[(slice * GM + h) * HD + grp * 8 + 4]) = make_float4(acc[h][4], acc[h][5], acc[h][6], acc[h][7]);
-        }
-    __syncthreads();
-    // merge the chunk into the running result (online softmax across chunks)
-#pragma unroll
-    for (int j = 0; j < OPT; j++) {
-        const uint32_t i = tid + (uint32_t)j * OXB_ATTN_THREADS;
-        if (i < G * HD) {
-            const uint32_t h = i / HD, d = i % HD;
-            float v = 0.f;
-#pragma unroll
-            for (int s = 0; s < NSL; s++) v += accs[(s * GM + h) * HD + d];
-            const float mc = m[0], lc = red[h * 4] + red[h * 4 + 1] + red[h * 4 + 2] + red[h * 4 + 3];
-            float mh = mc;
-#pragma unroll
-            for (int hh = 1; hh < GM; hh++) mh = (h == (uint32_t)hh) ? m[hh] : mh;
-            const float mn = fmaxf(run_m[j], mh);
-            const float a = expf(run_m[j] - mn), bw = expf(mh - mn);   // a = 0 for the first chunk
-            run_o[j] = run_o[j] * a + v * bw;
-            run_l[j] = run_l[j] * a + lc * bw;
-            run_m[j] = mn;
-        }
-    }
-    __syncthreads();  // the next chunk reuses sc, red and accs
-    }
-#pragma unroll
-    for (int j = 0; j < OPT; j++) {
-        const uint32_t i = tid + (uint32_t)j * OXB_ATTN_THREADS;
-        if (i < G * HD) {
-            const uint32_t h = i / HD, d = i % HD;
-            part[h * part_head + d] = run_o[j];
-            if (d == 0) {
-                part[h * part_head + HD] = run_m[j];
-                part[h * part_head + HD + 1] = run_l[j];
-            }
-        }
-    }
-}
-
-// ---------------------------------------------------------------------------
-// Decode attention on the matrix cores, fused with what precedes it in the layer: per-head QK-RMSNorm, RoPE and
-// the FP16 store of the new position's K and V (fused_qk_norm_rope + fused_kv_store + batched attention,
-// gpu_backend/cuda_attn_kernels.rs:160-438).  Grid (n_splits, nkv, batch), 256 threads = 4 waves.
+//  CPU: block/functions.rs:78-127 -> layers/attention_fused.rs:329-400), fused with what precedes it in the layer:
+// per-head QK-RMSNorm, RoPE and the FP16 store of the new position's K and V (fused_qk_norm_rope + fused_kv_store,
+// cuda_attn_kernels.rs:160-251).  Grid (n_splits, nkv, batch), 256 threads = 4 waves.  It writes, per q head and
+// slot, the un-normalised partial output, the running maximum and the running sum; attn_combine_quant_kernel
+// merges the slots.
 // A workgroup serves all q heads of one kv head (<= 16, the columns of the MFMA tiles) for one slot of the KV
 // sequence: slot s walks chunks s, s + n_splits, ... of 128 positions, wave w takes keys [32w, 32w + 32) of each.
 //   S^T[key][head] = sum_d K[key][d] Q[head][d]     A = K rows straight from the cache, B = Q * scale as fp16 hi + lo
@@ -745,28 +542,7 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
     return hipGetLastError();
 }
 
-template <int HD>
-static hipError_t launch_attn_hd(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
-    const uint32_t G = p.nq / p.nkv;
-    const dim3 block(OXB_ATTN_THREADS);
-    if (G == 1) hipLaunchKernelGGL((attn_decode_kernel<HD, 1>), dim3(p.n_splits, p.nkv, batch), block, 0, st, p);
-    else if (G == 2) hipLaunchKernelGGL((attn_decode_kernel<HD, 2>), dim3(p.n_splits, p.nkv, batch), block, 0, st, p);
-    else hipLaunchKernelGGL((attn_decode_kernel<HD, 4>), dim3(p.n_splits, p.nkv * ((G + 3) / 4), batch), block, 0, st, p);
-    return hipGetLastError();
-}
-
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
-    if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
-    switch (p.hd) {
-        case 32: return launch_attn_hd<32>(p, batch, st);
-        case 64: return launch_attn_hd<64>(p, batch, st);
-        case 128: return launch_attn_hd<128>(p, batch, st);
-        case 256: return launch_attn_hd<256>(p, batch, st);
-        default: return hipErrorInvalidValue;
-    }
-}
-
-hipError_t oxb_launch_attn_decode_fused(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
     if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
         !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t)
         return hipErrorInvalidValue;

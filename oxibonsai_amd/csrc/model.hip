@@ -38,7 +38,7 @@ struct Model {
     oxb_model_desc d;
     std::vector<oxb_layer_ids> layers;
     // activations
-    float *hidden = nullptr, *qkv = nullptr, *q_rope = nullptr, *attn_part = nullptr, *attn_out = nullptr,
+    float *hidden = nullptr, *qkv = nullptr, *attn_part = nullptr, *attn_out = nullptr,
           *gu = nullptr, *logits = nullptr;
     uint32_t *tokens = nullptr, *pos = nullptr;
     void* argmax_ws = nullptr;
@@ -177,17 +177,13 @@ static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn
     return OXB_HIP_OK;
 }
 
-// QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch; leaves the slot
-// results in m.attn_part and the parameters the merge needs in *ap.  Up to 16 q heads per kv head run in one
-// fused launch on the matrix cores; wider groups take the two-kernel route.
+// QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch, one launch; leaves the
+// slot results in m.attn_part and the parameters the merge needs in *ap.
 static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out) {
     const oxb_model_desc& d = m.d;
-    hipStream_t st = g_rt.stream;
-    const uint32_t qkv_rows = (d.nq + 2 * d.nkv) * d.hd;
     OxbAttnParams ap;
-    ap.q = m.q_rope;
     ap.qkv = m.qkv;
-    ap.qkv_stride = qkv_rows;
+    ap.qkv_stride = (d.nq + 2 * d.nkv) * d.hd;
     ap.q_norm = q_norm;
     ap.k_norm = k_norm;
     ap.cos_t = m.cos_t;
@@ -207,32 +203,7 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.n_splits = m.n_splits;
     ap.scale = 1.0f / sqrtf((float)d.hd);
     *out = ap;
-    if (d.nq / d.nkv <= 16) {
-        OXB_TRY_HIP(oxb_launch_attn_decode_fused(ap, d.batch, st), "kernel launch failed: attention");
-        return OXB_HIP_OK;
-    }
-    OxbQkParams qp;
-    qp.qkv = m.qkv;
-    qp.qkv_stride = qkv_rows;
-    qp.q_norm = q_norm;
-    qp.k_norm = k_norm;
-    qp.cos_t = m.cos_t;
-    qp.sin_t = m.sin_t;
-    qp.pos = m.pos;
-    qp.pos_base = 0;
-    qp.seq = 0;
-    qp.q_rope = m.q_rope;
-    qp.k_cache = m.k_cache;
-    qp.v_cache = m.v_cache;
-    qp.nq = d.nq;
-    qp.nkv = d.nkv;
-    qp.hd = d.hd;
-    qp.max_seq = d.max_seq;
-    qp.n_layers = d.n_layers;
-    qp.layer = L;
-    qp.eps = d.eps;
-    OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, d.batch, st), "kernel launch failed: qk_norm_rope_store");
-    OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, st), "kernel launch failed: attention");
+    OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, g_rt.stream), "kernel launch failed: attention");
     return OXB_HIP_OK;
 }
 
@@ -483,8 +454,8 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: a model dimension is 0");
     if (d.hd != 32 && d.hd != 64 && d.hd != 128 && d.hd != 256)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: head_dim %u (supported: 32, 64, 128, 256)", d.hd);
-    if (d.nq % d.nkv != 0 || d.nq / d.nkv > 8)
-        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u query heads per %u kv heads (need a whole ratio <= 8)", d.nq, d.nkv);
+    if (d.nq % d.nkv != 0 || d.nq / d.nkv > 16)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u query heads per %u kv heads (need a whole ratio <= 16)", d.nq, d.nkv);
     if (d.h % 128 || d.inter % 128 || (d.nq * d.hd) % 128)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden, intermediate and nq*hd must be multiples of 128");
     if (((size_t)d.nq * d.hd + (size_t)d.nq * 65) * sizeof(float) > 60 * 1024)
@@ -525,7 +496,6 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     if (qd > kmax) kmax = qd;
     const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
     if ((rc = dev_alloc(m, (void**)&m.hidden, B * d.h * 4)) || (rc = dev_alloc(m, (void**)&m.qkv, B * qkv_rows * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.q_rope, B * qd * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
