@@ -74,7 +74,7 @@ DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd
                   max_seq=32768, eps=1e-6, rope_theta=1e6)   # BASELINE.json configs[4]: Qwen3-8B shape, Q1_0_g128
 
 
-def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool) -> dict:
+def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32)) -> dict:
     """Greedy batch-1 decode of the random-init 8B-shape Q1 model: one batched prefill of `prompt_len` random
     token ids fills the context (timed on its own), then `n_tokens` greedy steps are timed.  The per-token time
     is what the caller of the fused entry point sees: embedding row H2D, the replayed HIP graph (36 layers,
@@ -120,6 +120,27 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool) -> dict:
            "weight_stream_GBps": round(weight_bytes / (spent / n_tokens) / 1e9, 1),
            "distinct_tokens": len(set(tokens))}
     m.close()
+    # the same model decoding several sequences at once (weights stream once per step for the whole batch); each
+    # sequence gets its own prefilled context of `prompt_len` positions
+    res["batched"] = []
+    for B in batches:
+        cfg_b = dict(cfg, max_seq=prompt_len + 64)
+        mb = HipModel(be, cfg_b, w, batch=B)
+        for sq in range(B):
+            mb.prefill(np.roll(rows, sq, axis=0), seq=sq, want_logits=False)
+        toks = [int(ids[sq]) for sq in range(B)]
+        steps_b, spent = 32, 0.0
+        for i in range(steps_b + 2):
+            hidden = np.stack([emb(t) for t in toks])
+            t0 = time.perf_counter()
+            _, out = mb.forward(hidden, np.full(B, prompt_len + i, dtype=np.uint32), want_logits=False)
+            if i >= 2:      # the first step records the graph, the second replays it for the first time
+                spent += time.perf_counter() - t0
+            toks = [int(t) for t in out]
+        res["batched"].append({"batch": B, "context_before": prompt_len, "steps": steps_b,
+                               "ms_per_step": round(spent / steps_b * 1e3, 4),
+                               "tok_per_s": round(B * steps_b / spent, 1), "hip_graph": mb.uses_graph()})
+        mb.close()
     if with_cpu:
         # CPU SIMD tier on the same matrices: linear layers only (one layer x 36 + LM head), an upper bound on its tok/s
         from oracle import oracle
@@ -189,6 +210,7 @@ def main() -> int:
                     help="also run a plain 256 MiB device copy, the known-size kernel that hardware-counter runs are scaled by")
     ap.add_argument("--decode-context", type=int, default=2048)
     ap.add_argument("--decode-tokens", type=int, default=128)
+    ap.add_argument("--decode-batches", type=str, default="8,32", help="batch sizes of the batched decode runs ('' = none)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (multi-GPU sharding is design-only)",
@@ -332,7 +354,8 @@ def main() -> int:
     if not args.no_prefill_gemm:
         out["prefill_gemm"] = prefill_gemm_leg(be, L, torch)
     if not args.no_decode:
-        out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu)
+        out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
+                                   tuple(int(b) for b in args.decode_batches.split(",") if b))
     print(json.dumps(out), flush=True)
     return 0
 

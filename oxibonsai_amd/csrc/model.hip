@@ -210,7 +210,7 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
 // Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
 // matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
 // the weights once per two sequences.
-#define OXB_DECODE_GEMM_MIN_BATCH 8
+#define OXB_DECODE_GEMM_MIN_BATCH 3
 
 static int encode_decode_step_gemm(Model& m) {
     const oxb_model_desc& d = m.d;

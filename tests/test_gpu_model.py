@@ -79,20 +79,22 @@ def test_mid_model_long_context_crosses_attention_chunks(backend):
         gpu.close()
 
 
-def test_batched_sequences_are_independent(backend):
+@pytest.mark.parametrize("B,tol", [(2, 1e-3), (3, 1e-2)])
+def test_batched_sequences_are_independent(backend, B, tol):
+    # two sequences share one pass of the fp32-exact GEMV; from three on the projections take the fp16 matrix-core
+    # route and are held to its tolerance
     cfg = dict(SMALL, fmt=TQ2)
     w = synth.make_model(cfg, 31)
-    B = 3
     gpu = HipModel(backend, cfg, w, batch=B)
     cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
     try:
         for step in range(10):
             hidden = np.stack([synth.embedding_rows(40 + b, [step + b], cfg["h"])[0] * 50.0 for b in range(B)])
-            pos = np.array([step, step, step], dtype=np.uint32)
+            pos = np.full(B, step, dtype=np.uint32)
             got, toks = gpu.forward(hidden, pos)
             for b in range(B):
                 want = cpus[b].forward(hidden[b], step)
-                assert parity_violations(got[b], want) == 0, (step, b)
+                assert parity_violations(got[b], want, tol) == 0, (step, b)
     finally:
         gpu.close()
 
@@ -179,7 +181,7 @@ def test_gqa_group_shapes(backend, nq, nkv, hd):
 @pytest.mark.parametrize("fmt", [TQ2, Q1])
 @pytest.mark.parametrize("B", [9, 20, 40])   # one and two token tiles of the narrow GEMM, then the wide one
 def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt, B):
-    """From 8 sequences on, a decode step sends its projections through the prefill GEMM (fp16 activations):
+    """From 3 sequences on, a decode step sends its projections through the matrix-core GEMM (fp16 activations):
     logits are held to the prefill tolerance 1e-2 under the reference's gate form; the step is still replayed
     from a captured graph and sequences stay independent."""
     cfg = dict(SMALL, fmt=fmt)
