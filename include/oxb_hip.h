@@ -126,7 +126,9 @@ int  oxb_hip_model_reset(uint64_t model);
 int  oxb_hip_model_destroy(uint64_t model);
 /* One token for each of the `batch` sequences: hidden[batch][h] are the embedding rows, pos[batch] the positions.
  * Runs all layers, the final norm, the LM head and a first-maximum argmax on the device (a HIP graph after the first
- * call).  logits_or_null: [batch][vocab]; token_out: [batch] greedy ids (either may be NULL). */
+ * call).  logits_or_null: [batch][vocab]; token_out: [batch] greedy ids (either may be NULL).
+ * Batches of 1 and 2 use the fp32-exact GEMV; from 3 sequences on the projections run as fp16 matrix-core GEMMs
+ * (the arithmetic of oxb_hip_gemm / oxb_hip_prefill). */
 int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out);
 /* Batched prefill: try_cuda_prefill / try_cuda_prefill_ternary (KG/cuda_prefill/try_apis.rs:42, 318; per layer
  * encode_prefill_layer[_ternary], KG/cuda_prefill/encode_q1.rs:123, encode_ternary.rs:114).  hidden = [n_tokens][h]
