@@ -140,6 +140,44 @@ int  oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t
                      float* logits_or_null, uint32_t* token_out_or_null);
 int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is replayed from a captured graph */
 
+/* ---- the steps either side of the fused forward: checkpoint file -> device, token ids in, token ids out.
+ * oxb_hip_gguf_info (no GPU needed) and oxb_hip_load_gguf read a GGUF file the way GgufFile::parse does
+ * (crates/oxibonsai-core/src/gguf/reader.rs:11-80, header.rs, metadata.rs, tensor_info.rs) and assemble the model
+ * the way BonsaiModel::from_gguf does (crates/oxibonsai-model/src/model/types/mod.rs:71-160; tensor names
+ * gguf/tensor_info.rs:211-230; configuration keys crates/oxibonsai-core/src/config.rs:41-118 with head_dim =
+ * hidden / heads and the vocabulary taken from token_embd's shape; norm vectors F32 or F16 widened,
+ * model/weight_loaders.rs:24-46; shapes in GGUF order [in, out]).  Every projection matrix and output.weight must be
+ * Q1_0_g128 (type 41) or TQ2_0_g128 (type 42), one format for the whole file; anything else is InvalidArgument. */
+typedef struct {
+    uint32_t version, alignment;
+    uint64_t n_tensors, n_metadata;
+    int fmt;                        /* OXB_HIP_FMT_* of the projection matrices (type of blk.0.attn_q.weight) */
+    int embedding_type;             /* GGUF type id of token_embd.weight: 0 F32, 1 F16, 41 Q1_0_g128, 42 TQ2_0_g128 */
+    uint32_t n_layers, h, inter, nq, nkv, hd, vocab, context_length;
+    float eps, rope_theta;
+    char architecture[32], name[64];
+} oxb_gguf_info;
+int  oxb_hip_gguf_info(const char* path, oxb_gguf_info* info);
+/* Uploads every tensor, creates the model (max_seq == 0: the file's context length) and the embedding table.  The
+ * model owns its weights: oxb_hip_model_destroy frees them; the embedding is freed with oxb_hip_free_embedding. */
+int  oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64_t* model, uint64_t* embedding,
+                       oxb_gguf_info* info_or_null);
+/* Token embedding table kept on the device in its stored form: vocab rows of h values, gguf_type 0 (F32), 1 (F16),
+ * 41 or 42 (rows of h/128 blocks); a row is widened / dequantised when it is looked up, with the values
+ * load_f32_tensor produces (model/weight_loaders.rs:24-86). */
+int  oxb_hip_upload_embedding(uint64_t* id, const void* table, size_t n_bytes, int gguf_type, uint32_t vocab, uint32_t h);
+int  oxb_hip_free_embedding(uint64_t id);
+int  oxb_hip_embedding_rows(uint64_t embedding, const uint32_t* ids, uint32_t n, float* out);   /* out: [n][h] */
+/* Greedy decode without a host round trip per token: the embedding row copy that precedes the forward
+ * (model/types/mod.rs:647-658) and the argmax that follows it (temperature 0, crates/oxibonsai-runtime/src/sampling.rs:182)
+ * stay on the device.  tokens[batch] are the ids to feed at pos[batch]; n_steps forwards run back to back, each
+ * feeding the previous step's argmax; tokens_out[n_steps][batch] receives every step's ids. */
+int  oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
+                           uint32_t n_steps, uint32_t* tokens_out);
+/* oxb_hip_prefill with the embedding rows gathered on the device from token ids. */
+int  oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, const uint32_t* ids, uint32_t n_tokens,
+                            uint32_t pos_start, float* logits_or_null, uint32_t* token_out_or_null);
+
 /* ---- host-only helpers (no GPU needed): the upload-time repack, exposed so it can be checked on any machine.
  * reformat_q1_aos_to_soa / reformat_tq2_blocks_to_soa (KG/cuda_graph/cudagraph_reformat_*_group.rs). */
 int  oxb_hip_repack_sizes(int fmt, uint32_t n_rows, uint32_t k, size_t* codes_bytes, size_t* scales_bytes);

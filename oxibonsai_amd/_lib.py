@@ -50,6 +50,13 @@ _SIGNATURES = {
     "oxb_hip_decode": ([C.c_uint64, f32p, u32p, f32p, u32p], C.c_int),
     "oxb_hip_prefill": ([C.c_uint64, C.c_uint32, f32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_model_uses_graph": ([C.c_uint64], C.c_int),
+    "oxb_hip_gguf_info": ([C.c_char_p, C.c_void_p], C.c_int),
+    "oxb_hip_load_gguf": ([C.c_char_p, C.c_uint32, C.c_uint32, u64p, u64p, C.c_void_p], C.c_int),
+    "oxb_hip_upload_embedding": ([u64p, C.c_void_p, C.c_size_t, C.c_int, C.c_uint32, C.c_uint32], C.c_int),
+    "oxb_hip_free_embedding": ([C.c_uint64], C.c_int),
+    "oxb_hip_embedding_rows": ([C.c_uint64, u32p, C.c_uint32, f32p], C.c_int),
+    "oxb_hip_decode_tokens": ([C.c_uint64, C.c_uint64, u32p, u32p, C.c_uint32, u32p], C.c_int),
+    "oxb_hip_prefill_tokens": ([C.c_uint64, C.c_uint64, C.c_uint32, u32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_repack_sizes": ([C.c_int, C.c_uint32, C.c_uint32, szp, szp], C.c_int),
     "oxb_hip_repack": ([C.c_int, u8p, C.c_size_t, C.c_uint32, C.c_uint32, u8p, C.c_size_t, u8p, C.c_size_t], C.c_int),
     "oxb_hip_unpack": ([C.c_int, u8p, C.c_size_t, u8p, C.c_size_t, C.c_uint32, C.c_uint32, u8p, C.c_size_t], C.c_int),

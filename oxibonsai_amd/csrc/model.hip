@@ -21,6 +21,7 @@
 
 #include "../../include/oxb_hip.h"
 #include "gemm_kernels.h"
+#include "gguf.h"
 #include "gemv_kernels.h"
 #include "layer_kernels.h"
 #include "prefill_kernels.h"
@@ -57,7 +58,18 @@ struct Model {
     float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
     std::vector<void*> pf_allocs;
     GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
+    // a model loaded from a file owns the weights it uploaded
+    std::vector<uint64_t> owned_mats, owned_vecs;
+    DevBuf tok_hist, tok_ids;  // token history of the on-device greedy loop; prompt ids of a token prefill
 };
+
+struct Embedding {  // token embedding table in its stored form
+    void* d = nullptr;
+    int type = 0;   // GGUF tensor type id: 0 F32, 1 F16, 41 Q1_0_g128, 42 TQ2_0_g128
+    uint32_t vocab = 0, h = 0;
+    size_t bytes = 0;
+};
+static std::unordered_map<uint64_t, Embedding> g_embeddings;
 
 static std::unordered_map<uint64_t, std::unique_ptr<Model>> g_models;
 static uint64_t g_next_model = 1;
@@ -79,11 +91,15 @@ static void free_model(Model& m) {
     m.pf_allocs.clear();
     m.pf_cap = 0;
     m.gws.release();
+    m.tok_hist.release();
+    m.tok_ids.release();
 }
 
 void shutdown_models() {
     for (auto& kv : g_models) free_model(*kv.second);
     g_models.clear();
+    for (auto& kv : g_embeddings) (void)hipFree(kv.second.d);
+    g_embeddings.clear();
 }
 
 static const float* vec_ptr(uint64_t id, uint32_t n, const char* what, int* rc) {
@@ -567,7 +583,10 @@ int oxb_hip_model_destroy(uint64_t model) {
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
     (void)hipStreamSynchronize(g_rt.stream);
     free_model(*m);
+    const std::vector<uint64_t> mats = std::move(m->owned_mats), vecs = std::move(m->owned_vecs);
     g_models.erase(model);
+    for (uint64_t id : mats) (void)oxb_hip_free_weight(id);
+    for (uint64_t id : vecs) (void)oxb_hip_free_f32(id);
     return OXB_HIP_OK;
 }
 
@@ -580,19 +599,10 @@ int oxb_hip_model_reset(uint64_t model) {
     return OXB_HIP_OK;
 }
 
-int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out) {
-    std::lock_guard<std::recursive_mutex> lk(g_mu);
-    Model* mp = find_model(model);
-    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
-    Model& m = *mp;
-    const oxb_model_desc& d = m.d;
-    if (!hidden || !pos) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden or pos");
-    for (uint32_t b = 0; b < d.batch; b++)
-        if (pos[b] >= d.max_seq)
-            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+// One decode step on m.hidden / m.pos (device): replayed from the captured graph, captured on first use, or launched
+// kernel by kernel when capture is off or failed.
+static int run_decode_step(Model& m) {
     hipStream_t st = g_rt.stream;
-    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
-    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
     if (m.graph_exec) {
         OXB_TRY_HIP(hipGraphLaunch(m.graph_exec, st), "graph launch");
     } else if (!m.graph_failed && st == g_rt.own_stream) {
@@ -619,6 +629,23 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     } else {
         OXB_TRY(encode_decode_step(m, true));
     }
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (!hidden || !pos) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden or pos");
+    for (uint32_t b = 0; b < d.batch; b++)
+        if (pos[b] >= d.max_seq)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    OXB_TRY(run_decode_step(m));
     if (token_out) OXB_TRY_HIP(hipMemcpyAsync(token_out, m.tokens, (size_t)d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
     if (logits_or_null)
         OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits, (size_t)d.batch * d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
@@ -692,6 +719,351 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     OXB_TRY_HIP(hipMemcpyAsync(hidden, d_hidden, (size_t)h * 4, hipMemcpyDeviceToHost, st), "hidden download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+}
+
+// ---------------------------------------------------------------------------
+// Token embedding tables, the on-device greedy loop, and the GGUF loader.
+// ---------------------------------------------------------------------------
+static Embedding* find_embedding(uint64_t id) {
+    auto it = g_embeddings.find(id);
+    return it == g_embeddings.end() ? nullptr : &it->second;
+}
+
+int oxb_hip_upload_embedding(uint64_t* id, const void* table, size_t n_bytes, int gguf_type, uint32_t vocab, uint32_t h) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!id || !table) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null id or table");
+    if (gguf_type != GGUF_F32 && gguf_type != GGUF_F16 && gguf_type != GGUF_Q1_0_G128 && gguf_type != GGUF_TQ2_0_G128)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: embedding tensor type %d (supported: 0 F32, 1 F16, 41, 42)", gguf_type);
+    if (vocab == 0 || h == 0 || (gguf_type >= 41 && h % 128))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: embedding of %u rows x %u values", vocab, h);
+    const size_t need = (size_t)gguf_tensor_bytes((uint32_t)gguf_type, (uint64_t)vocab * h);
+    if (n_bytes < need)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: embedding buffer holds %zu bytes, %zu needed", n_bytes, need);
+    OXB_TRY(ensure_init());
+    Embedding e;
+    e.type = gguf_type, e.vocab = vocab, e.h = h, e.bytes = need;
+    if (hipMalloc(&e.d, need) != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", need, g_rt.device);
+    hipError_t he = hipMemcpy(e.d, table, need, hipMemcpyHostToDevice);
+    if (he != hipSuccess) {
+        (void)hipFree(e.d);
+        return hip_fail(he, "embedding upload");
+    }
+    if (*id == 0) *id = g_rt.next_id++;
+    if (Embedding* old = find_embedding(*id)) (void)hipFree(old->d);
+    g_embeddings[*id] = e;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_free_embedding(uint64_t id) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Embedding* e = find_embedding(id);
+    if (!e) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (embedding) not found", (unsigned long long)id);
+    (void)hipStreamSynchronize(g_rt.stream);
+    (void)hipFree(e->d);
+    g_embeddings.erase(id);
+    return OXB_HIP_OK;
+}
+
+static int check_ids(const Embedding& e, const uint32_t* ids, size_t n) {
+    for (size_t i = 0; i < n; i++)
+        if (ids[i] >= e.vocab)  // model/types/mod.rs:649-657
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: token_id %u out of range (vocab=%u)", ids[i], e.vocab);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_embedding_rows(uint64_t embedding, const uint32_t* ids, uint32_t n, float* out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Embedding* e = find_embedding(embedding);
+    if (!e) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (embedding) not found", (unsigned long long)embedding);
+    if (n == 0) return OXB_HIP_OK;
+    if (!ids || !out) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null ids or out");
+    OXB_TRY(check_ids(*e, ids, n));
+    OXB_TRY(g_rt.ws_x.ensure((size_t)n * 4));
+    OXB_TRY(g_rt.ws_y.ensure((size_t)n * e->h * 4));
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(g_rt.ws_x.ptr, ids, (size_t)n * 4, hipMemcpyHostToDevice, st), "token id upload");
+    OXB_TRY_HIP(oxb_launch_embedding_gather(e->d, e->type, e->vocab, e->h, (const uint32_t*)g_rt.ws_x.ptr, n, (float*)g_rt.ws_y.ptr, st),
+                "kernel launch failed: embedding_gather");
+    OXB_TRY_HIP(hipMemcpyAsync(out, g_rt.ws_y.ptr, (size_t)n * e->h * 4, hipMemcpyDeviceToHost, st), "embedding download");
+    hipError_t he = hipStreamSynchronize(st);
+    if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: embedding_rows: %s", hipGetErrorString(he));
+    return OXB_HIP_OK;
+}
+
+static int model_and_embedding(uint64_t model, uint64_t embedding, Model** m, Embedding** e) {
+    *m = find_model(model);
+    if (!*m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    *e = find_embedding(embedding);
+    if (!*e) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (embedding) not found", (unsigned long long)embedding);
+    if ((*e)->h != (*m)->d.h)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: embedding rows hold %u values, the model's hidden size is %u", (*e)->h, (*m)->d.h);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
+                          uint32_t* tokens_out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp;
+    Embedding* e;
+    OXB_TRY(model_and_embedding(model, embedding, &mp, &e));
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (n_steps == 0) return OXB_HIP_OK;
+    if (!tokens || !pos || !tokens_out) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null tokens, pos or tokens_out");
+    if (e->vocab < d.vocab)  // every argmax result must name a row of the table
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: embedding has %u rows, the LM head %u", e->vocab, d.vocab);
+    OXB_TRY(check_ids(*e, tokens, d.batch));
+    for (uint32_t b = 0; b < d.batch; b++)
+        if ((uint64_t)pos[b] + n_steps > d.max_seq)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos[b],
+                        (unsigned long long)pos[b] + n_steps - 1, d.max_seq);
+    OXB_TRY(m.tok_hist.ensure((size_t)n_steps * d.batch * 4));
+    hipStream_t st = g_rt.stream;
+    uint32_t* hist = (uint32_t*)m.tok_hist.ptr;
+    OXB_TRY_HIP(hipMemcpyAsync(m.tokens, tokens, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "token upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    for (uint32_t i = 0; i < n_steps; i++) {
+        OXB_TRY_HIP(oxb_launch_embedding_gather(e->d, e->type, e->vocab, d.h, m.tokens, d.batch, m.hidden, st),
+                    "kernel launch failed: embedding_gather");
+        OXB_TRY(run_decode_step(m));  // m.tokens <- argmax
+        OXB_TRY_HIP(oxb_launch_token_step(m.tokens, hist + (size_t)i * d.batch, m.pos, d.batch, st), "kernel launch failed: token_step");
+    }
+    OXB_TRY_HIP(hipMemcpyAsync(tokens_out, hist, (size_t)n_steps * d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
+    hipError_t he = hipStreamSynchronize(st);
+    if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode_tokens: %s", hipGetErrorString(he));
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, const uint32_t* ids, uint32_t n_tokens,
+                           uint32_t pos_start, float* logits_or_null, uint32_t* token_out_or_null) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp;
+    Embedding* e;
+    OXB_TRY(model_and_embedding(model, embedding, &mp, &e));
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (!ids || n_tokens == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null ids or no tokens");
+    if (seq >= d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, d.batch);
+    if ((uint64_t)pos_start + n_tokens > d.max_seq)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
+                    (unsigned long long)pos_start + n_tokens - 1, d.max_seq);
+    OXB_TRY(check_ids(*e, ids, n_tokens));
+    OXB_TRY(ensure_prefill_buffers(m, n_tokens));
+    OXB_TRY(m.tok_ids.ensure((size_t)n_tokens * 4));
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(m.tok_ids.ptr, ids, (size_t)n_tokens * 4, hipMemcpyHostToDevice, st), "token id upload");
+    OXB_TRY_HIP(oxb_launch_embedding_gather(e->d, e->type, e->vocab, d.h, (const uint32_t*)m.tok_ids.ptr, n_tokens, m.pf_hidden, st),
+                "kernel launch failed: embedding_gather");
+    OXB_TRY(encode_prefill(m, seq, n_tokens, pos_start));
+    if (token_out_or_null) OXB_TRY_HIP(hipMemcpyAsync(token_out_or_null, m.tokens + seq, 4, hipMemcpyDeviceToHost, st), "token download");
+    if (logits_or_null)
+        OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits + (size_t)seq * d.vocab, (size_t)d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
+    hipError_t he = hipStreamSynchronize(st);
+    if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: prefill_tokens: %s", hipGetErrorString(he));
+    return OXB_HIP_OK;
+}
+
+// --- GGUF ---------------------------------------------------------------------------------------------------
+static int gguf_fail(const std::string& why) { return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: GGUF: %s", why.c_str()); }
+
+// Configuration the way Qwen3Config::from_metadata reads it (crates/oxibonsai-core/src/config.rs:41-118):
+// "<architecture>.<key>" first, then "llm.<key>", then the Bonsai-8B default.
+static int gguf_describe(const GgufFile& g, oxb_gguf_info* info) {
+    memset(info, 0, sizeof *info);
+    info->version = g.version;
+    info->alignment = g.alignment;
+    info->n_tensors = g.n_tensors;
+    info->n_metadata = g.n_kv;
+    std::string arch = "qwen3", name = "Bonsai-8B";
+    (void)g.get_str("general.architecture", &arch);
+    (void)g.get_str("general.name", &name);
+    snprintf(info->architecture, sizeof info->architecture, "%s", arch.c_str());
+    snprintf(info->name, sizeof info->name, "%s", name.c_str());
+    auto u32 = [&](const char* key, uint32_t dflt) {
+        uint32_t v = dflt;
+        if (!g.get_u32(arch + "." + key, &v)) (void)g.get_u32(std::string("llm.") + key, &v);
+        return v;
+    };
+    auto f32 = [&](const char* key, float dflt) {
+        float v = dflt;
+        if (!g.get_f32(arch + "." + key, &v)) (void)g.get_f32(std::string("llm.") + key, &v);
+        return v;
+    };
+    info->h = u32("embedding_length", 4096);
+    info->n_layers = u32("block_count", 36);
+    info->nq = u32("attention.head_count", 32);
+    info->nkv = u32("attention.head_count_kv", 8);
+    info->inter = u32("feed_forward_length", 14336);
+    info->vocab = u32("vocab_size", 151936);
+    info->context_length = u32("context_length", 65536);
+    info->eps = f32("attention.layer_norm_rms_epsilon", 1e-6f);
+    info->rope_theta = f32("rope.freq_base", 1000000.0f);
+    if (info->nq == 0) return gguf_fail("attention.head_count is 0");
+    info->hd = info->h / info->nq;
+    // the embedding tensor's row count overrides the metadata (model/types/mod.rs:73-86)
+    const GgufTensor* emb = g.find("token_embd.weight");
+    if (!emb) return gguf_fail("tensor not found: token_embd.weight");
+    if (emb->shape.size() >= 2 && emb->shape[1] <= UINT32_MAX) info->vocab = (uint32_t)emb->shape[1];
+    info->embedding_type = (int)emb->type;
+    const GgufTensor* q = g.find("blk.0.attn_q.weight");
+    if (!q) return gguf_fail("tensor not found: blk.0.attn_q.weight");
+    if (q->type == GGUF_Q1_0_G128) info->fmt = OXB_FMT_Q1;
+    else if (q->type == GGUF_TQ2_0_G128) info->fmt = OXB_FMT_TQ2;
+    else return gguf_fail("blk.0.attn_q.weight has tensor type " + std::to_string(q->type) + "; this tier runs Q1_0_g128 (41) and TQ2_0_g128 (42)");
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_gguf_info(const char* path, oxb_gguf_info* info) {
+    if (!info) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null info");
+    GgufFile g;
+    std::string err;
+    if (!g.open(path, &err)) return gguf_fail(err);
+    return gguf_describe(g, info);
+}
+
+// A tensor that must exist with the given type(s) and GGUF shape [in (, out)].
+static int gguf_require(const GgufFile& g, const std::string& name, uint32_t type_a, uint32_t type_b, uint64_t in, uint64_t out,
+                        const GgufTensor** t) {
+    *t = g.find(name);
+    if (!*t) return gguf_fail("tensor not found: " + name);
+    const GgufTensor& x = **t;
+    if (x.type != type_a && x.type != type_b)
+        return gguf_fail(name + " has tensor type " + std::to_string(x.type) + ", expected " + std::to_string(type_a) +
+                         (type_b != type_a ? " or " + std::to_string(type_b) : ""));
+    const bool shape_ok = out ? (x.shape.size() == 2 && x.shape[0] == in && x.shape[1] == out) : (x.shape.size() == 1 && x.shape[0] == in);
+    if (!shape_ok) {
+        std::string sh;
+        for (uint64_t v : x.shape) sh += (sh.empty() ? "" : ", ") + std::to_string(v);
+        return gguf_fail(name + " has shape [" + sh + "], expected [" + std::to_string(in) + (out ? ", " + std::to_string(out) : "") + "]");
+    }
+    if (!x.data) return gguf_fail("unexpected end of file at offset " + std::to_string(g.data_offset + x.offset + x.bytes) + " (tensor " + name + ")");
+    return OXB_HIP_OK;
+}
+
+// Norm vector, F32 or F16 widened (model/weight_loaders.rs:24-46) -> resident fp32 vector owned by the model.
+static int gguf_vector(const GgufFile& g, Model& m, const std::string& name, uint32_t n, uint64_t* id) {
+    const GgufTensor* t;
+    OXB_TRY(gguf_require(g, name, GGUF_F32, GGUF_F16, n, 0, &t));
+    std::vector<float> v(n);
+    if (t->type == GGUF_F32) memcpy(v.data(), t->data, (size_t)n * 4);
+    else
+        for (uint32_t i = 0; i < n; i++) {
+            uint16_t b;
+            memcpy(&b, t->data + 2 * (size_t)i, 2);
+            v[i] = __half2float(__ushort_as_half(b));
+        }
+    *id = 0;
+    OXB_TRY(oxb_hip_upload_f32(id, v.data(), n));
+    m.owned_vecs.push_back(*id);
+    return OXB_HIP_OK;
+}
+
+// Row concatenation of projection matrices that share k (Q|K|V, gate|up): their AoS block arrays back to back
+// (crates/oxibonsai-model/src/block/types/upload.rs:21-39) -> one resident matrix owned by the model.
+static int gguf_matrix(const GgufFile& g, Model& m, int fmt, const std::vector<std::pair<std::string, uint32_t>>& parts, uint32_t k,
+                       uint64_t* id) {
+    const uint32_t type = fmt == OXB_FMT_Q1 ? GGUF_Q1_0_G128 : GGUF_TQ2_0_G128;
+    std::vector<const GgufTensor*> ts(parts.size());
+    uint32_t rows = 0;
+    size_t bytes = 0;
+    for (size_t i = 0; i < parts.size(); i++) {
+        OXB_TRY(gguf_require(g, parts[i].first, type, type, k, parts[i].second, &ts[i]));
+        rows += parts[i].second;
+        bytes += ts[i]->bytes;
+    }
+    *id = 0;
+    int rc;
+    if (parts.size() == 1) {
+        rc = upload_weight(id, fmt, ts[0]->data, ts[0]->bytes, rows, k);
+    } else {
+        std::vector<uint8_t> cat(bytes);
+        size_t off = 0;
+        for (const GgufTensor* t : ts) {
+            memcpy(cat.data() + off, t->data, t->bytes);
+            off += t->bytes;
+        }
+        rc = upload_weight(id, fmt, cat.data(), bytes, rows, k);
+    }
+    if (rc) return rc;
+    m.owned_mats.push_back(*id);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64_t* model, uint64_t* embedding,
+                      oxb_gguf_info* info_or_null) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!model || !embedding) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null model or embedding pointer");
+    GgufFile g;
+    std::string err;
+    if (!g.open(path, &err)) return gguf_fail(err);
+    oxb_gguf_info info;
+    OXB_TRY(gguf_describe(g, &info));
+    if (info_or_null) *info_or_null = info;
+    if (info.h % 128 || info.inter % 128 || info.hd == 0 || info.h != info.nq * info.hd)
+        return gguf_fail("hidden " + std::to_string(info.h) + " / heads " + std::to_string(info.nq) + " / intermediate " +
+                         std::to_string(info.inter) + " do not fit this tier (multiples of 128, hidden = heads x head_dim)");
+    OXB_TRY(ensure_init());
+
+    // uploads are collected in a scratch model so that any failure frees what was uploaded so far
+    Model owner;
+    std::vector<oxb_layer_ids> layers(info.n_layers);
+    uint64_t final_norm = 0, lm_head = 0;
+    const uint32_t qd = info.nq * info.hd, kd = info.nkv * info.hd;
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < info.n_layers && !rc; L++) {
+        const std::string b = "blk." + std::to_string(L) + ".";
+        oxb_layer_ids& ly = layers[L];
+        (rc = gguf_vector(g, owner, b + "attn_norm.weight", info.h, &ly.attn_norm)) ||
+            (rc = gguf_vector(g, owner, b + "ffn_norm.weight", info.h, &ly.ffn_norm)) ||
+            (rc = gguf_vector(g, owner, b + "attn_q_norm.weight", info.hd, &ly.q_norm)) ||
+            (rc = gguf_vector(g, owner, b + "attn_k_norm.weight", info.hd, &ly.k_norm)) ||
+            (rc = gguf_matrix(g, owner, info.fmt, {{b + "attn_q.weight", qd}, {b + "attn_k.weight", kd}, {b + "attn_v.weight", kd}}, info.h, &ly.qkv)) ||
+            (rc = gguf_matrix(g, owner, info.fmt, {{b + "attn_output.weight", info.h}}, qd, &ly.o)) ||
+            (rc = gguf_matrix(g, owner, info.fmt, {{b + "ffn_gate.weight", info.inter}, {b + "ffn_up.weight", info.inter}}, info.h, &ly.gate_up)) ||
+            (rc = gguf_matrix(g, owner, info.fmt, {{b + "ffn_down.weight", info.h}}, info.inter, &ly.down));
+    }
+    if (!rc) rc = gguf_vector(g, owner, "output_norm.weight", info.h, &final_norm);
+    // the LM head's row count comes from its own shape (model/weight_loaders.rs:654-666)
+    uint32_t lm_rows = info.vocab;
+    if (!rc) {
+        const GgufTensor* out = g.find("output.weight");
+        if (!out) rc = gguf_fail("tensor not found: output.weight");
+        else if (out->shape.size() >= 2 && out->shape[1] <= UINT32_MAX) lm_rows = (uint32_t)out->shape[1];
+    }
+    if (!rc) rc = gguf_matrix(g, owner, info.fmt, {{"output.weight", lm_rows}}, info.h, &lm_head);
+    uint64_t emb_id = 0;
+    if (!rc) {
+        const GgufTensor* emb;
+        rc = gguf_require(g, "token_embd.weight", (uint32_t)info.embedding_type, (uint32_t)info.embedding_type, info.h, info.vocab, &emb);
+        if (!rc) rc = oxb_hip_upload_embedding(&emb_id, emb->data, emb->bytes, info.embedding_type, info.vocab, info.h);
+    }
+    uint64_t mid = 0;
+    if (!rc) {
+        oxb_model_desc d;
+        memset(&d, 0, sizeof d);
+        d.fmt = info.fmt;
+        d.n_layers = info.n_layers, d.h = info.h, d.inter = info.inter, d.nq = info.nq, d.nkv = info.nkv, d.hd = info.hd;
+        d.vocab = lm_rows;
+        d.max_seq = max_seq ? max_seq : info.context_length;
+        d.batch = batch;
+        d.eps = info.eps, d.rope_theta = info.rope_theta;
+        d.layers = layers.data();
+        d.final_norm = final_norm, d.lm_head = lm_head;
+        rc = oxb_hip_model_create(&d, &mid);
+    }
+    if (rc) {
+        for (uint64_t id : owner.owned_mats) (void)oxb_hip_free_weight(id);
+        for (uint64_t id : owner.owned_vecs) (void)oxb_hip_free_f32(id);
+        if (emb_id) (void)oxb_hip_free_embedding(emb_id);
+        return rc;
+    }
+    Model* m = find_model(mid);
+    m->owned_mats = std::move(owner.owned_mats);
+    m->owned_vecs = std::move(owner.owned_vecs);
+    *model = mid;
+    *embedding = emb_id;
     return OXB_HIP_OK;
 }
 

@@ -27,6 +27,53 @@ class _ModelDesc(C.Structure):
                 ("final_norm", C.c_uint64), ("lm_head", C.c_uint64)]
 
 
+class GgufInfo(C.Structure):
+    """oxb_gguf_info: what GgufFile::parse + Qwen3Config::from_metadata tell about a checkpoint."""
+    _fields_ = [("version", C.c_uint32), ("alignment", C.c_uint32), ("n_tensors", C.c_uint64), ("n_metadata", C.c_uint64),
+                ("fmt", C.c_int), ("embedding_type", C.c_int)] + \
+               [(n, C.c_uint32) for n in ("n_layers", "h", "inter", "nq", "nkv", "hd", "vocab", "context_length")] + \
+               [("eps", C.c_float), ("rope_theta", C.c_float), ("architecture", C.c_char * 32), ("name", C.c_char * 64)]
+
+    def as_dict(self) -> dict:
+        d = {n: getattr(self, n) for n, _ in self._fields_}
+        d["architecture"], d["name"] = self.architecture.decode(), self.name.decode()
+        return d
+
+
+def gguf_info(path: str) -> dict:
+    """Header, configuration and formats of a GGUF checkpoint; needs no GPU
+    (GgufFile::parse, crates/oxibonsai-core/src/gguf/reader.rs:25-66; Qwen3Config::from_metadata, config.rs:41-118)."""
+    info = GgufInfo()
+    _check(_lib.lib().oxb_hip_gguf_info(str(path).encode(), C.byref(info)))
+    return info.as_dict()
+
+
+class Embedding:
+    """Token embedding table resident on the device in its stored form (F32, F16, Q1_0_g128 or TQ2_0_g128)."""
+
+    def __init__(self, table, gguf_type: int, vocab: int, h: int, _id: int = 0):
+        self._lib = _lib.lib()
+        if _id:
+            self.id = _id
+        else:
+            a = np.ascontiguousarray(table)
+            eid = C.c_uint64(0)
+            _check(self._lib.oxb_hip_upload_embedding(C.byref(eid), a.ctypes.data_as(C.c_void_p), a.nbytes, gguf_type, vocab, h))
+            self.id = eid.value
+        self.vocab, self.h, self.gguf_type = vocab, h, gguf_type
+
+    def rows(self, ids) -> np.ndarray:
+        iv = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+        out = np.empty((iv.size, self.h), dtype=np.float32)
+        _check(self._lib.oxb_hip_embedding_rows(self.id, iv.ctypes.data_as(_lib.u32p), iv.size, out.ctypes.data_as(_lib.f32p)))
+        return out
+
+    def close(self):
+        if self.id:
+            _check(self._lib.oxb_hip_free_embedding(self.id))
+            self.id = 0
+
+
 class HipModel:
     """cfg: fmt, n_layers, h, inter, nq, nkv, hd, vocab, max_seq, eps, rope_theta.
     weights: dict of oxibonsai_amd.synth.make_model (reference AoS blocks + f32 norm vectors)."""
@@ -51,6 +98,22 @@ class HipModel:
         mid = C.c_uint64(0)
         _check(self._lib.oxb_hip_model_create(C.byref(desc), C.byref(mid)))
         self.id = mid.value
+
+    @classmethod
+    def from_gguf(cls, backend: NativeHipBackend, path: str, max_seq: int = 0, batch: int = 1):
+        """BonsaiModel::from_gguf (crates/oxibonsai-model/src/model/types/mod.rs:71-160) on the device:
+        -> (model, embedding, info dict).  The model owns the weights it uploaded."""
+        self = cls.__new__(cls)
+        self.be, self.batch = backend, batch
+        self._lib = _lib.lib()
+        self._mats, self._vecs = [], []
+        info, mid, eid = GgufInfo(), C.c_uint64(0), C.c_uint64(0)
+        _check(self._lib.oxb_hip_load_gguf(str(path).encode(), max_seq, batch, C.byref(mid), C.byref(eid), C.byref(info)))
+        d = info.as_dict()
+        self.cfg = dict(fmt=d["fmt"], n_layers=d["n_layers"], h=d["h"], inter=d["inter"], nq=d["nq"], nkv=d["nkv"], hd=d["hd"],
+                        vocab=d["vocab"], max_seq=max_seq or d["context_length"], eps=d["eps"], rope_theta=d["rope_theta"])
+        self.id = mid.value
+        return self, Embedding(None, d["embedding_type"], d["vocab"], d["h"], _id=eid.value), d
 
     def _mat(self, blocks, n_rows, k):
         fmt = self.cfg["fmt"]
@@ -86,6 +149,26 @@ class HipModel:
         _check(self._lib.oxb_hip_prefill(self.id, seq, hv.ctypes.data_as(_lib.f32p), hv.shape[0], pos_start,
                                          logits.ctypes.data_as(_lib.f32p) if want_logits else None,
                                          token.ctypes.data_as(_lib.u32p)))
+        return logits, int(token[0])
+
+    def generate(self, embedding: Embedding, tokens, pos, n_steps: int) -> np.ndarray:
+        """Greedy decode of n_steps tokens per sequence without a host round trip per token: tokens [batch] are fed
+        at pos [batch], every further step feeds the previous argmax -> ids [n_steps, batch]."""
+        tv = np.ascontiguousarray(np.broadcast_to(np.asarray(tokens, dtype=np.uint32), (self.batch,)))
+        pv = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, dtype=np.uint32), (self.batch,)))
+        out = np.empty((n_steps, self.batch), dtype=np.uint32)
+        _check(self._lib.oxb_hip_decode_tokens(self.id, embedding.id, tv.ctypes.data_as(_lib.u32p), pv.ctypes.data_as(_lib.u32p),
+                                               n_steps, out.ctypes.data_as(_lib.u32p)))
+        return out
+
+    def prefill_tokens(self, embedding: Embedding, ids, pos_start: int = 0, seq: int = 0, want_logits: bool = True):
+        """prefill() with the embedding rows gathered on the device from token ids."""
+        iv = np.ascontiguousarray(ids, dtype=np.uint32).reshape(-1)
+        logits = np.empty(self.cfg["vocab"], dtype=np.float32) if want_logits else None
+        token = np.empty(1, dtype=np.uint32)
+        _check(self._lib.oxb_hip_prefill_tokens(self.id, embedding.id, seq, iv.ctypes.data_as(_lib.u32p), iv.size, pos_start,
+                                                logits.ctypes.data_as(_lib.f32p) if want_logits else None,
+                                                token.ctypes.data_as(_lib.u32p)))
         return logits, int(token[0])
 
     def uses_graph(self) -> bool:
