@@ -74,7 +74,7 @@ DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd
                   max_seq=32768, eps=1e-6, rope_theta=1e6)   # BASELINE.json configs[4]: Qwen3-8B shape, Q1_0_g128
 
 
-def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32)) -> dict:
+def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32), with_gguf: bool = True) -> dict:
     """Greedy batch-1 decode of the random-init 8B-shape Q1 model: one batched prefill of `prompt_len` random
     token ids fills the context (timed on its own), then `n_tokens` greedy steps are timed.  The per-token time
     is what the caller of the fused entry point sees: embedding row H2D, the replayed HIP graph (36 layers,
@@ -119,7 +119,37 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
            "kv_bytes_per_token_at_end": 2 * cfg["n_layers"] * cfg["nkv"] * cfg["hd"] * 2 * (prompt_len + n_tokens),
            "weight_stream_GBps": round(weight_bytes / (spent / n_tokens) / 1e9, 1),
            "distinct_tokens": len(set(tokens))}
+    # the same loop without a host round trip per token: embedding lookup (a Q1_0_g128 table here), forward and
+    # argmax stay on the device, the host gets all ids at the end (oxb_hip_decode_tokens)
+    from oxibonsai_amd.model import Embedding
+    emb_blocks = synth.make_q1_blocks(0xB0A5A104E0, cfg["vocab"] * (cfg["h"] // 128), 0.01, 0.1)
+    emb_tab = Embedding(emb_blocks, 41, cfg["vocab"], cfg["h"])
+    m.generate(emb_tab, [tok], [prompt_len + n_tokens], 2)
+    t0 = time.perf_counter()
+    ids_dev = m.generate(emb_tab, [tok], [prompt_len + n_tokens], n_tokens)
+    t_dev = time.perf_counter() - t0
+    res["device_loop"] = {"tokens": n_tokens, "tok_per_s": round(n_tokens / t_dev, 2),
+                          "ms_per_token": round(t_dev / n_tokens * 1e3, 4), "embedding": "Q1_0_g128 table on the device"}
     m.close()
+    if with_gguf:
+        # checkpoint file -> device: the same tensors written as a GGUF file (page cache), loaded by oxb_hip_load_gguf
+        import tempfile
+        from oxibonsai_amd.gguf import model_gguf
+        with tempfile.TemporaryDirectory() as td:
+            path = os.path.join(td, "bonsai8b_shape_q1.gguf")
+            with open(path, "wb") as f:
+                f.write(model_gguf(cfg, w, 41, emb_blocks))
+            size = os.path.getsize(path)
+            t0 = time.perf_counter()
+            mg, eg, _ = HipModel.from_gguf(be, path, max_seq=prompt_len + 2 * n_tokens + 8)
+            t_load = time.perf_counter() - t0
+        mg.prefill_tokens(eg, ids, want_logits=False)
+        ids_file = mg.generate(eg, [int(ids_dev[0, 0])], [prompt_len], 16)
+        mg.close()
+        eg.close()
+        res["gguf_load"] = {"file_bytes": size, "seconds": round(t_load, 3), "GB_per_s": round(size / t_load / 1e9, 2),
+                            "first_tokens": [int(t) for t in ids_file[:4, 0]]}
+    emb_tab.close()
     # the same model decoding several sequences at once (weights stream once per step for the whole batch); each
     # sequence gets its own prefilled context of `prompt_len` positions
     res["batched"] = []
@@ -211,6 +241,7 @@ def main() -> int:
     ap.add_argument("--decode-context", type=int, default=2048)
     ap.add_argument("--decode-tokens", type=int, default=128)
     ap.add_argument("--decode-batches", type=str, default="8,32", help="batch sizes of the batched decode runs ('' = none)")
+    ap.add_argument("--no-gguf", action="store_true", help="skip the checkpoint-file load of the decode leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (multi-GPU sharding is design-only)",
@@ -355,7 +386,7 @@ def main() -> int:
         out["prefill_gemm"] = prefill_gemm_leg(be, L, torch)
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
-                                   tuple(int(b) for b in args.decode_batches.split(",") if b))
+                                   tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf)
     print(json.dumps(out), flush=True)
     return 0
 
