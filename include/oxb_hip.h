@@ -158,6 +158,14 @@ typedef struct {
     char architecture[32], name[64];
 } oxb_gguf_info;
 int  oxb_hip_gguf_info(const char* path, oxb_gguf_info* info);
+/* Directory access without a GPU: one metadata value rendered as text (integers, floats with %.9g, strings as they
+ * are, bools as true/false, arrays as "[<count> x type <id>]"), and one tensor's entry (GGUF type id, shape in file
+ * order, absolute file offset of its data = data section start + tensor offset, byte size; size 0 for a type this
+ * tier does not read).  A missing key / tensor is OXB_HIP_WEIGHT_NOT_FOUND (BonsaiError::TensorNotFound,
+ * gguf/tensor_info.rs:86-91). */
+int  oxb_hip_gguf_metadata(const char* path, const char* key, char* out, size_t out_cap);
+int  oxb_hip_gguf_tensor(const char* path, const char* name, int* type, uint32_t* n_dims, uint64_t shape4[4],
+                         uint64_t* file_offset, uint64_t* n_bytes);
 /* Uploads every tensor, creates the model (max_seq == 0: the file's context length) and the embedding table.  The
  * model owns its weights: oxb_hip_model_destroy frees them; the embedding is freed with oxb_hip_free_embedding. */
 int  oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64_t* model, uint64_t* embedding,

@@ -923,6 +923,42 @@ int oxb_hip_gguf_info(const char* path, oxb_gguf_info* info) {
     return gguf_describe(g, info);
 }
 
+int oxb_hip_gguf_metadata(const char* path, const char* key, char* out, size_t out_cap) {
+    if (!key || !out || out_cap == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null key or output");
+    GgufFile g;
+    std::string err;
+    if (!g.open(path, &err)) return gguf_fail(err);
+    auto it = g.meta.find(key);
+    if (it == g.meta.end()) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "metadata key %s not found", key);
+    const GgufValue& v = it->second;
+    switch (v.type) {
+        case 0: case 2: case 4: case 10: snprintf(out, out_cap, "%llu", (unsigned long long)v.u); break;
+        case 1: case 3: case 5: case 11: snprintf(out, out_cap, "%lld", (long long)v.i); break;
+        case 6: case 12: snprintf(out, out_cap, "%.9g", v.f); break;
+        case 7: snprintf(out, out_cap, "%s", v.u ? "true" : "false"); break;
+        case 8: snprintf(out, out_cap, "%s", v.s.c_str()); break;
+        default: snprintf(out, out_cap, "[%llu x type %u]", (unsigned long long)v.count, v.elem_type); break;
+    }
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_gguf_tensor(const char* path, const char* name, int* type, uint32_t* n_dims, uint64_t shape4[4],
+                        uint64_t* file_offset, uint64_t* n_bytes) {
+    if (!name) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null name");
+    GgufFile g;
+    std::string err;
+    if (!g.open(path, &err)) return gguf_fail(err);
+    const GgufTensor* t = g.find(name);
+    if (!t) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "tensor not found: %s", name);
+    if (type) *type = (int)t->type;
+    if (n_dims) *n_dims = (uint32_t)t->shape.size();
+    if (shape4)
+        for (size_t i = 0; i < 4; i++) shape4[i] = i < t->shape.size() ? t->shape[i] : 0;
+    if (file_offset) *file_offset = g.data_offset + t->offset;
+    if (n_bytes) *n_bytes = t->bytes;
+    return OXB_HIP_OK;
+}
+
 // A tensor that must exist with the given type(s) and GGUF shape [in (, out)].
 static int gguf_require(const GgufFile& g, const std::string& name, uint32_t type_a, uint32_t type_b, uint64_t in, uint64_t out,
                         const GgufTensor** t) {

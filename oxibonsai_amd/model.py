@@ -48,6 +48,22 @@ def gguf_info(path: str) -> dict:
     return info.as_dict()
 
 
+def gguf_metadata(path: str, key: str) -> str:
+    """One metadata value of a GGUF file as text (MetadataStore::get, crates/oxibonsai-core/src/gguf/metadata.rs:94)."""
+    buf = C.create_string_buffer(4096)
+    _check(_lib.lib().oxb_hip_gguf_metadata(str(path).encode(), key.encode(), buf, len(buf)))
+    return buf.value.decode()
+
+
+def gguf_tensor(path: str, name: str) -> dict:
+    """Directory entry of one tensor (TensorStore::require, gguf/tensor_info.rs:86): type id, shape in file order,
+    absolute file offset of the data and its size in bytes."""
+    t, nd, sh, off, nb = C.c_int(0), C.c_uint32(0), (C.c_uint64 * 4)(), C.c_uint64(0), C.c_uint64(0)
+    _check(_lib.lib().oxb_hip_gguf_tensor(str(path).encode(), name.encode(), C.byref(t), C.byref(nd), sh, C.byref(off), C.byref(nb)))
+    return {"type": t.value, "shape": [int(sh[i]) for i in range(min(nd.value, 4))], "n_dims": nd.value,
+            "file_offset": off.value, "bytes": nb.value}
+
+
 class Embedding:
     """Token embedding table resident on the device in its stored form (F32, F16, Q1_0_g128 or TQ2_0_g128)."""
 

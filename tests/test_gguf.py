@@ -95,3 +95,77 @@ def test_missing_and_unsupported_tensors(tmp_path):
     assert "token_embd.weight" in _err(tmp_path, gguf_bytes([], []))
     q4 = ("blk.0.attn_q.weight", [128, 32], 2, b"")          # Q4_0: a format of the reference this tier does not run
     assert "tensor type 2" in _err(tmp_path, gguf_bytes([], ts + [q4]))
+
+
+# ---------------------------------------------------------------------------
+# The byte strings of the reference's own parser tests (crates/oxibonsai-core/tests/gguf_edge_cases.rs:19-91 build
+# them field by field; they are rebuilt here the same way, independently of the package's writer).
+# ---------------------------------------------------------------------------
+from oxibonsai_amd.model import gguf_metadata, gguf_tensor
+
+
+def _hdr(magic, version, tensors, metadata):
+    return struct.pack("<I", magic) + struct.pack("<I", version) + struct.pack("<Q", tensors) + struct.pack("<Q", metadata)
+
+
+def _s(x):
+    return struct.pack("<Q", len(x)) + x.encode()
+
+
+def _tinfo(name, shape, type_id, offset):
+    return _s(name) + struct.pack("<I", len(shape)) + b"".join(struct.pack("<Q", d) for d in shape) + \
+        struct.pack("<I", type_id) + struct.pack("<Q", offset)
+
+
+def test_reference_edge_case_files(tmp_path):
+    # gguf_file_parse_with_one_metadata_entry (:506-520): "test.key" = 42u32
+    data = _hdr(0x46554747, 3, 0, 1) + _s("test.key") + struct.pack("<I", 4) + struct.pack("<I", 42)
+    data += b"\0" * (64 - len(data))
+    p = _write(tmp_path, data)
+    assert gguf_metadata(p, "test.key") == "42"
+    with pytest.raises(GpuError) as e:
+        gguf_metadata(p, "absent.key")
+    assert e.value.kind == "WeightNotFound"
+    # metadata_value_type_conversions (:274-306) through the configuration reader: a u64 that does not fit u32 and a
+    # negative i32 are not usable as u32 (the default stays), f64 narrows to f32
+    emb = np.zeros((4, 128), np.float32).tobytes()
+    q = np.zeros(4 * 18, np.uint8).tobytes()
+    md = [("qwen3.block_count", "u64", 2**64 - 1), ("qwen3.attention.head_count", "i32", -1),
+          ("qwen3.embedding_length", "u64", 128), ("qwen3.rope.freq_base", "f64", 2.718281828459045)]
+    ts = [("token_embd.weight", [128, 4], GGUF_F32, emb), ("blk.0.attn_q.weight", [128, 4], GGUF_Q1, q)]
+    info = gguf_info(_write(tmp_path, gguf_bytes(md, ts), "conv.gguf"))
+    assert (info["n_layers"], info["nq"], info["h"]) == (36, 32, 128) and info["rope_theta"] == np.float32(2.718281828459045)
+    # metadata_duplicate_keys_last_wins (:329-336), metadata_bool_entry, metadata_array_u32 (:355-371)
+    data = _hdr(0x46554747, 3, 0, 4) + _s("k") + struct.pack("<II", 4, 1) + _s("k") + struct.pack("<II", 4, 2)
+    data += _s("flag") + struct.pack("<I", 7) + b"\x01"
+    data += _s("arr") + struct.pack("<I", 9) + struct.pack("<I", 4) + struct.pack("<Q", 3) + struct.pack("<III", 10, 20, 30)
+    p = _write(tmp_path, data + b"\0" * 64, "dup.gguf")
+    assert gguf_metadata(p, "k") == "2" and gguf_metadata(p, "flag") == "true" and gguf_metadata(p, "arr") == "[3 x type 4]"
+
+
+def test_data_section_alignment_and_tensor_offsets(tmp_path):
+    # gguf_file_parse_minimal_valid (:491-503): header only -> the data section starts at 32; align_offset table (:465-484)
+    for name_len, align, want in ((1, 32, None), (7, 32, None), (8, 32, None), (9, 64, None), (40, 1, None)):
+        name = "t" * name_len
+        md = [] if align == 32 else [("general.alignment", "u32", align)]
+        head = _hdr(0x46554747, 3, 1, len(md))
+        for k, _, v in md:
+            head += _s(k) + struct.pack("<II", 4, v)
+        head += _tinfo(name, [128, 2], 41, 96 if align != 1 else 5)
+        start = (len(head) + align - 1) & ~(align - 1)          # the reference's formula
+        off = 96 if align != 1 else 5
+        payload = bytes(range(36))
+        data = head + b"\0" * (start - len(head)) + b"\xEE" * off + payload
+        t = gguf_tensor(_write(tmp_path, data, f"a{name_len}.gguf"), name)
+        assert t == {"type": 41, "shape": [128, 2], "n_dims": 2, "file_offset": start + off, "bytes": 36}
+        assert data[t["file_offset"]:t["file_offset"] + t["bytes"]] == payload
+    with pytest.raises(GpuError) as e:                           # tensor_store_missing_tensor (:405-411)
+        gguf_tensor(_write(tmp_path, _hdr(0x46554747, 3, 0, 0) + b"\0" * 8, "none.gguf"), "nope")
+    assert e.value.kind == "WeightNotFound"
+    # tensor_info_zero_dimensions / single_dimension / type sizes (types.rs block_bytes): F32 4, F16 2, 41 18, 42 34 per unit
+    head = _hdr(0x46554747, 3, 4, 0) + _tinfo("s", [], 0, 0) + _tinfo("v", [5], 1, 32) + _tinfo("m", [256, 3], 42, 64) + \
+        _tinfo("x", [32, 2], 2, 0)
+    p = _write(tmp_path, head + b"\0" * 1024, "dims.gguf")
+    assert gguf_tensor(p, "s")["bytes"] == 4 and gguf_tensor(p, "s")["n_dims"] == 0
+    assert gguf_tensor(p, "v")["bytes"] == 10 and gguf_tensor(p, "m")["bytes"] == 6 * 34
+    assert gguf_tensor(p, "x")["bytes"] == 0 and gguf_tensor(p, "x")["type"] == 2          # Q4_0: listed, not read
