@@ -128,8 +128,12 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
     t0 = time.perf_counter()
     ids_dev = m.generate(emb_tab, [tok], [prompt_len + n_tokens], n_tokens)
     t_dev = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    m.generate_sampled(emb_tab, [tok], [prompt_len + n_tokens], n_tokens, 0.7, 40, 0.9, [0xB0A5A1])   # the reference's defaults
+    t_smp = time.perf_counter() - t0
     res["device_loop"] = {"tokens": n_tokens, "tok_per_s": round(n_tokens / t_dev, 2),
-                          "ms_per_token": round(t_dev / n_tokens * 1e3, 4), "embedding": "Q1_0_g128 table on the device"}
+                          "ms_per_token": round(t_dev / n_tokens * 1e3, 4), "embedding": "Q1_0_g128 table on the device",
+                          "sampled_tok_per_s": round(n_tokens / t_smp, 2), "sampling": "temperature 0.7, top-k 40, top-p 0.9"}
     m.close()
     if with_gguf:
         # checkpoint file -> device: the same tensors written as a GGUF file (page cache), loaded by oxb_hip_load_gguf

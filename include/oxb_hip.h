@@ -182,6 +182,20 @@ int  oxb_hip_embedding_rows(uint64_t embedding, const uint32_t* ids, uint32_t n,
  * feeding the previous step's argmax; tokens_out[n_steps][batch] receives every step's ids. */
 int  oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
                            uint32_t n_steps, uint32_t* tokens_out);
+/* The same loop with Sampler::sample (crates/oxibonsai-runtime/src/sampling.rs:84-177) on the device instead of the
+ * argmax: v / temperature, the top_k largest, softmax, top-p cut with renormalisation, one xorshift64 draw
+ * (sampling.rs:73-80) per step and sequence, cumulative pick.  rng_state[batch] holds one generator state per
+ * sequence (the reference's Sampler seed) and is advanced in place.  temperature < 1e-6 is the greedy loop (the
+ * device argmax keeps the FIRST maximum, the reference's host argmax the last; they differ only on exact ties).
+ * The device sampler takes 1 <= top_k <= 128 and works on the candidates in descending order, where the reference
+ * keeps whatever order its partial selection leaves when top_p == 1 (its pick is then an equally valid draw from
+ * the same distribution, not the same token).  Repetition penalty is not part of Sampler::sample. */
+typedef struct { float temperature; uint32_t top_k; float top_p; } oxb_sampling;
+int  oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
+                                   uint32_t n_steps, const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out);
+/* The sampler alone on host logits [batch][vocab] (vocab <= 524288). */
+int  oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params,
+                           uint64_t* rng_state, uint32_t* tokens_out);
 /* oxb_hip_prefill with the embedding rows gathered on the device from token ids. */
 int  oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, const uint32_t* ids, uint32_t n_tokens,
                             uint32_t pos_start, float* logits_or_null, uint32_t* token_out_or_null);

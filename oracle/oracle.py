@@ -66,6 +66,9 @@ def lib() -> C.CDLL:
             getattr(L, n).argtypes = [f32p, sz]
             getattr(L, n).restype = C.c_uint32
         L.oxb_state_new.restype = C.c_void_p
+        L.oxb_sample.restype = C.c_uint32
+        L.oxb_sample.argtypes = [f32p, sz, C.c_float, sz, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), f32p, sz,
+                                 C.POINTER(sz), f32p]
         L.oxb_state_new.argtypes = [C.c_void_p]
         L.oxb_state_free.argtypes = [C.c_void_p]
         L.oxb_state_free.restype = None
@@ -212,6 +215,19 @@ def attention_head(q, keys, values, seq_len: int, head_dim: int) -> np.ndarray:
 def argmax_last(v) -> int:
     a = _vec(v)
     return int(lib().oxb_argmax_last(_f32(a), a.size))
+
+
+def sample(logits, temperature: float, top_k: int, top_p: float, rng_state: int):
+    """Sampler::sample (crates/oxibonsai-runtime/src/sampling.rs:84-177) -> (token, new rng state, candidate ids,
+    candidate probabilities, random draw); the last three are empty / None for the greedy branch."""
+    a = _vec(logits)
+    st = C.c_uint64(rng_state)
+    cap = a.size
+    ci, cp = np.zeros(cap, dtype=np.uint32), np.zeros(cap, dtype=np.float32)
+    nc, r = C.c_size_t(0), C.c_float(0.0)
+    tok = lib().oxb_sample(_f32(a), a.size, temperature, top_k, top_p, C.byref(st), ci.ctypes.data_as(C.POINTER(C.c_uint32)),
+                           _f32(cp), cap, C.byref(nc), C.byref(r))
+    return int(tok), int(st.value), ci[:nc.value].copy(), cp[:nc.value].copy(), (float(r.value) if nc.value else None)
 
 
 def argmax_first(v) -> int:

@@ -295,6 +295,91 @@ uint32_t oxb_argmax_first(const float* v, size_t n) {
 }
 
 /* ------------------------------------------------------------------------- */
+/* Sampler::sample, crates/oxibonsai-runtime/src/sampling.rs:84-177 (xorshift64 next_u64 :73-80).
+ * temperature < 1e-6: greedy, the LAST maximum (Iterator::max_by).  Otherwise: v / temperature; keep the top_k
+ * largest (top_k == 0 or >= n: all); softmax over the kept values; if top_p < 1: sort by probability descending,
+ * keep the shortest prefix whose cumulative sum exceeds top_p (all but none if it never does), renormalise;
+ * draw r = (next_u64 / u64::MAX) as f32 and return the first candidate whose cumulative probability reaches r
+ * (the first candidate if none does).
+ * The reference leaves the candidates in the order select_nth_unstable_by happens to produce when top_p == 1 and
+ * sums the softmax in that order; this restatement always works in descending order of value, ties by ascending
+ * index (a stable sort of the index-ordered buffer).  cand_idx / cand_p (capacity cap, may be NULL) receive the
+ * final candidate list, *n_cand its length, *r_out the random draw. */
+static uint64_t xorshift64(uint64_t* state) {
+    uint64_t x = *state;
+    x ^= x << 13;
+    x ^= x >> 7;
+    x ^= x << 17;
+    *state = x;
+    return x;
+}
+
+uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top_k, float top_p, uint64_t* rng_state,
+                    uint32_t* cand_idx, float* cand_p, size_t cap, size_t* n_cand, float* r_out) {
+    if (n_cand) *n_cand = 0;
+    if (n == 0) return 0;
+    if (temperature < 1e-6f) return oxb_argmax_last(logits, n);
+    size_t k = (top_k > 0 && top_k < n) ? top_k : n;
+    uint32_t* idx = (uint32_t*)malloc(k * sizeof(uint32_t));
+    float* p = (float*)malloc(k * sizeof(float));
+    unsigned char* taken = (unsigned char*)calloc(n, 1);
+    /* k largest scaled values in descending order, ties by ascending index (selection; n * k compares) */
+    for (size_t j = 0; j < k; j++) {
+        size_t best = n;
+        float bv = 0.0f;
+        for (size_t i = 0; i < n; i++) {
+            if (taken[i]) continue;
+            const float v = logits[i] / temperature;
+            if (best == n || v > bv) best = i, bv = v;
+        }
+        taken[best] = 1;
+        idx[j] = (uint32_t)best;
+        p[j] = bv;
+    }
+    free(taken);
+    const float max_val = p[0];
+    float sum = 0.0f;
+    for (size_t j = 0; j < k; j++) {
+        p[j] = expf(p[j] - max_val);
+        sum += p[j];
+    }
+    for (size_t j = 0; j < k; j++) p[j] /= sum;
+    if (top_p < 1.0f) {
+        float cum = 0.0f;
+        size_t cutoff = k ? k - 1 : 0;
+        for (size_t j = 0; j < k; j++) {
+            cum += p[j];
+            if (cum > top_p) {
+                cutoff = j;
+                break;
+            }
+        }
+        k = cutoff + 1;
+        float s2 = 0.0f;
+        for (size_t j = 0; j < k; j++) s2 += p[j];
+        for (size_t j = 0; j < k; j++) p[j] /= s2;
+    }
+    const float r = (float)((double)xorshift64(rng_state) / (double)UINT64_MAX);
+    if (r_out) *r_out = r;
+    if (n_cand) *n_cand = k;
+    for (size_t j = 0; j < k && j < cap; j++) {
+        if (cand_idx) cand_idx[j] = idx[j];
+        if (cand_p) cand_p[j] = p[j];
+    }
+    uint32_t tok = idx[0];
+    float cum = 0.0f;
+    for (size_t j = 0; j < k; j++) {
+        cum += p[j];
+        if (r <= cum) {
+            tok = idx[j];
+            break;
+        }
+    }
+    free(idx);
+    free(p);
+    return tok;
+}
+
 /* Whole-model decode step: model/src/model/types/mod.rs:633-934 (embedding   */
 /* row -> blocks -> output_norm -> LM head) around                            */
 /* model/src/block/types/forward.rs:92-408 (one transformer block).           */

@@ -22,6 +22,13 @@
  *   model forward      float64 numpy restatement on the tiny test geometry
  *                      (no stored logits exist in the reference: end-to-end
  *                      token strings of the real binary are parity unpinned)
+ *   sample             the reference's sampler unit tests (greedy, valid index,
+ *                      top-k range), the xorshift64 recurrence and the draw formula
+ *                      recomputed with Python integers, candidates / probabilities
+ *                      against a float64 numpy softmax, draw frequencies.  Parity
+ *                      unpinned: the candidate order the reference's partial
+ *                      selection leaves when top_p == 1 (implementation-defined)
+ *                      and the last place of exp()
  */
 #ifndef OXB_ORACLE_H
 #define OXB_ORACLE_H
@@ -71,6 +78,9 @@ void  oxb_attention_head(const float* q, const float* keys, const float* values,
                          size_t seq_len, size_t head_dim);
 uint32_t oxb_argmax_last(const float* v, size_t n);   /* Sampler greedy: last max on ties */
 uint32_t oxb_argmax_first(const float* v, size_t n);  /* GPU argmax_f32: first max        */
+/* Sampler::sample (runtime/src/sampling.rs:84-177); see the definition for the candidate order it fixes. */
+uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top_k, float top_p, uint64_t* rng_state,
+                    uint32_t* cand_idx, float* cand_p, size_t cap, size_t* n_cand, float* r_out);
 
 /* One linear layer in the reference's AoS block format. fmt: 0 = Q1_0_g128, 1 = TQ2_0_g128. */
 typedef struct {

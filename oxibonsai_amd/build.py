@@ -15,7 +15,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "lib")
-SOURCES = ["runtime.hip", "gemv_kernels.hip", "gemm_kernels.hip", "layer_kernels.hip", "prefill_kernels.hip", "model.hip", "repack.cpp", "gguf.cpp"]
+SOURCES = ["runtime.hip", "gemv_kernels.hip", "gemm_kernels.hip", "layer_kernels.hip", "prefill_kernels.hip", "token_kernels.hip", "model.hip", "repack.cpp", "gguf.cpp"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          # packed-FP32 VALU forms are kept out of every kernel

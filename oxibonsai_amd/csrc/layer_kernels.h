@@ -50,12 +50,3 @@ hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.
 #define OXB_ARGMAX_MAX_PARTS 256u
 hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st);
-
-// Token embedding lookup: out[i][0..h) = row ids[i] of the table kept in its stored form (gguf_type 0 F32, 1 F16,
-// 41 Q1_0_g128 blocks, 42 TQ2_0_g128 blocks), widened / dequantised as the reference's loader does.  ids are device
-// memory; an id >= vocab yields a row of NaN (host-supplied ids are validated before the launch).
-hipError_t oxb_launch_embedding_gather(const void* d_table, int gguf_type, uint32_t vocab, uint32_t h, const uint32_t* d_ids,
-                                       uint32_t n, float* d_out, hipStream_t st);
-// End of one step of the on-device greedy loop: history[b] = tokens[b]; pos[b] += 1.
-hipError_t oxb_launch_token_step(const uint32_t* d_tokens, uint32_t* d_history, uint32_t* d_pos, uint32_t batch, hipStream_t st);
-

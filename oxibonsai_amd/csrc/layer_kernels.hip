@@ -496,56 +496,6 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
 // ---------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------
-// ---------------------------------------------------------------------------
-// Token embedding lookup (the row copy that precedes the forward, crates/oxibonsai-model/src/model/types/mod.rs:647-658)
-// from the table in its stored form; values as load_f32_tensor widens / dequantises them
-// (crates/oxibonsai-model/src/model/weight_loaders.rs:24-86): F16 -> f32 exactly; Q1_0_g128 bit ? d : -d;
-// TQ2_0_g128 codes 00 -> -d, 01 -> 0, 10 -> +d, 11 -> 0.  Grid = rows, 256 threads.
-// ---------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void embedding_gather_kernel(const uint8_t* __restrict__ table, int type, uint32_t vocab,
-                                                                uint32_t h, const uint32_t* __restrict__ ids,
-                                                                float* __restrict__ out) {
-    const uint32_t row = blockIdx.x, id = ids[row];
-    float* o = out + (size_t)row * h;
-    if (id >= vocab) {
-        for (uint32_t i = threadIdx.x; i < h; i += 256) o[i] = __int_as_float(0x7FC00000);
-        return;
-    }
-    if (type == 0) {
-        const float* src = reinterpret_cast<const float*>(table) + (size_t)id * h;
-        for (uint32_t i = threadIdx.x; i < h; i += 256) o[i] = src[i];
-    } else if (type == 1) {
-        const __half* src = reinterpret_cast<const __half*>(table) + (size_t)id * h;
-        for (uint32_t i = threadIdx.x; i < h; i += 256) o[i] = __half2float(src[i]);
-    } else {
-        const uint32_t bb = type == 41 ? 18u : 34u;
-        const uint8_t* src = table + (size_t)id * (h / 128u) * bb;
-        for (uint32_t i = threadIdx.x; i < h; i += 256) {
-            const uint8_t* blk = src + (size_t)(i >> 7) * bb;
-            const uint32_t j = i & 127u;
-            float v;
-            if (type == 41) {  // [d f16][qs 16]
-                const float d = __half2float(__ushort_as_half((unsigned short)(blk[0] | (blk[1] << 8))));
-                v = ((blk[2 + (j >> 3)] >> (j & 7u)) & 1u) ? d : -d;
-            } else {           // [qs 32][d f16]
-                const float d = __half2float(__ushort_as_half((unsigned short)(blk[32] | (blk[33] << 8))));
-                const uint32_t code = (blk[j >> 2] >> (2u * (j & 3u))) & 3u;
-                v = code == 0u ? -d : (code == 2u ? d : 0.0f);
-            }
-            o[i] = v;
-        }
-    }
-}
-
-__global__ void token_step_kernel(const uint32_t* __restrict__ tokens, uint32_t* __restrict__ history,
-                                  uint32_t* __restrict__ pos, uint32_t batch) {
-    const uint32_t b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b < batch) {
-        history[b] = tokens[b];
-        pos[b] += 1u;
-    }
-}
-
 template <int FMT>
 static hipError_t launch_rmsnorm_fmt(const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
                                      uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed,
@@ -643,18 +593,3 @@ hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, 
     hipLaunchKernelGGL(argmax_final_kernel, dim3(batch), dim3(64), 0, st, pv, pi, parts, d_out);
     return hipGetLastError();
 }
-
-hipError_t oxb_launch_embedding_gather(const void* d_table, int gguf_type, uint32_t vocab, uint32_t h, const uint32_t* d_ids,
-                                       uint32_t n, float* d_out, hipStream_t st) {
-    if (n == 0) return hipSuccess;
-    if ((gguf_type != 0 && gguf_type != 1 && gguf_type != 41 && gguf_type != 42) || (gguf_type >= 41 && h % 128u)) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(embedding_gather_kernel, dim3(n), dim3(256), 0, st, static_cast<const uint8_t*>(d_table), gguf_type, vocab, h,
-                       d_ids, d_out);
-    return hipGetLastError();
-}
-
-hipError_t oxb_launch_token_step(const uint32_t* d_tokens, uint32_t* d_history, uint32_t* d_pos, uint32_t batch, hipStream_t st) {
-    hipLaunchKernelGGL(token_step_kernel, dim3((batch + 63) / 64), dim3(64), 0, st, d_tokens, d_history, d_pos, batch);
-    return hipGetLastError();
-}
-

@@ -26,6 +26,7 @@
 #include "layer_kernels.h"
 #include "prefill_kernels.h"
 #include "runtime_internal.h"
+#include "token_kernels.h"
 
 namespace oxb {
 
@@ -60,7 +61,8 @@ struct Model {
     GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
     // a model loaded from a file owns the weights it uploaded
     std::vector<uint64_t> owned_mats, owned_vecs;
-    DevBuf tok_hist, tok_ids;  // token history of the on-device greedy loop; prompt ids of a token prefill
+    DevBuf tok_hist, tok_ids;  // token history of the on-device generation loop; prompt ids of a token prefill
+    DevBuf sample_ws, rng;     // sampler scratch and per-sequence xorshift64 states
 };
 
 struct Embedding {  // token embedding table in its stored form
@@ -93,6 +95,8 @@ static void free_model(Model& m) {
     m.gws.release();
     m.tok_hist.release();
     m.tok_ids.release();
+    m.sample_ws.release();
+    m.rng.release();
 }
 
 void shutdown_models() {
@@ -802,8 +806,17 @@ static int model_and_embedding(uint64_t model, uint64_t embedding, Model** m, Em
     return OXB_HIP_OK;
 }
 
-int oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
-                          uint32_t* tokens_out) {
+static int check_sampling(const oxb_sampling& sp) {
+    if (!(sp.temperature >= 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: temperature %g", (double)sp.temperature);
+    if (sp.temperature >= 1e-6f && (sp.top_k == 0 || sp.top_k > OXB_SAMPLE_MAX_TOP_K))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_k %u (the device sampler takes 1..%u; sample on the host from the logits otherwise)",
+                    sp.top_k, OXB_SAMPLE_MAX_TOP_K);
+    if (!(sp.top_p > 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_p %g", (double)sp.top_p);
+    return OXB_HIP_OK;
+}
+
+static int decode_tokens_impl(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
+                              const oxb_sampling* sp, uint64_t* rng_state, uint32_t* tokens_out) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* mp;
     Embedding* e;
@@ -819,20 +832,76 @@ int oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* to
         if ((uint64_t)pos[b] + n_steps > d.max_seq)
             return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos[b],
                         (unsigned long long)pos[b] + n_steps - 1, d.max_seq);
+    const bool sampled = sp && sp->temperature >= 1e-6f;  // below: greedy (sampling.rs:89-92)
+    if (sp) OXB_TRY(check_sampling(*sp));
+    if (sampled && !rng_state) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null rng_state");
     OXB_TRY(m.tok_hist.ensure((size_t)n_steps * d.batch * 4));
     hipStream_t st = g_rt.stream;
+    if (sampled) {
+        OXB_TRY(m.sample_ws.ensure(oxb_sample_ws_bytes(d.vocab, d.batch)));
+        OXB_TRY(m.rng.ensure((size_t)d.batch * 8));
+        OXB_TRY_HIP(hipMemcpyAsync(m.rng.ptr, rng_state, (size_t)d.batch * 8, hipMemcpyHostToDevice, st), "rng state upload");
+    }
     uint32_t* hist = (uint32_t*)m.tok_hist.ptr;
     OXB_TRY_HIP(hipMemcpyAsync(m.tokens, tokens, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "token upload");
     OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
     for (uint32_t i = 0; i < n_steps; i++) {
         OXB_TRY_HIP(oxb_launch_embedding_gather(e->d, e->type, e->vocab, d.h, m.tokens, d.batch, m.hidden, st),
                     "kernel launch failed: embedding_gather");
-        OXB_TRY(run_decode_step(m));  // m.tokens <- argmax
+        OXB_TRY(run_decode_step(m));  // m.logits, m.tokens <- argmax
+        if (sampled)
+            OXB_TRY_HIP(oxb_launch_sample(m.logits, d.vocab, d.batch, sp->temperature, sp->top_k, sp->top_p, (uint64_t*)m.rng.ptr,
+                                          m.tokens, m.sample_ws.ptr, st),
+                        "kernel launch failed: sample");
         OXB_TRY_HIP(oxb_launch_token_step(m.tokens, hist + (size_t)i * d.batch, m.pos, d.batch, st), "kernel launch failed: token_step");
     }
     OXB_TRY_HIP(hipMemcpyAsync(tokens_out, hist, (size_t)n_steps * d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
+    if (sampled) OXB_TRY_HIP(hipMemcpyAsync(rng_state, m.rng.ptr, (size_t)d.batch * 8, hipMemcpyDeviceToHost, st), "rng state download");
     hipError_t he = hipStreamSynchronize(st);
     if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode_tokens: %s", hipGetErrorString(he));
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
+                          uint32_t* tokens_out) {
+    return decode_tokens_impl(model, embedding, tokens, pos, n_steps, nullptr, nullptr, tokens_out);
+}
+
+int oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
+                                  const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out) {
+    if (!params) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null sampling parameters");
+    return decode_tokens_impl(model, embedding, tokens, pos, n_steps, params, rng_state, tokens_out);
+}
+
+int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params, uint64_t* rng_state,
+                          uint32_t* tokens_out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!logits || !params || !rng_state || !tokens_out || vocab == 0 || batch == 0)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or empty logits");
+    OXB_TRY(check_sampling(*params));
+    if ((vocab + 2047u) / 2048u > 256u) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u logits per row (at most 524288)", vocab);
+    OXB_TRY(ensure_init());
+    const size_t lb = (size_t)batch * vocab * 4, wb = oxb_sample_ws_bytes(vocab, batch);
+    OXB_TRY(g_rt.ws_y.ensure(lb + wb + 256));
+    OXB_TRY(g_rt.ws_x.ensure((size_t)batch * 16));
+    float* d_logits = (float*)g_rt.ws_y.ptr;
+    void* d_ws = (uint8_t*)g_rt.ws_y.ptr + ((lb + 255) & ~(size_t)255);
+    uint64_t* d_rng = (uint64_t*)g_rt.ws_x.ptr;
+    uint32_t* d_tok = (uint32_t*)(d_rng + batch);
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(d_logits, logits, lb, hipMemcpyHostToDevice, st), "logits upload");
+    OXB_TRY_HIP(hipMemcpyAsync(d_rng, rng_state, (size_t)batch * 8, hipMemcpyHostToDevice, st), "rng state upload");
+    if (params->temperature < 1e-6f) {
+        OXB_TRY(g_rt.ws_xq.ensure((size_t)batch * OXB_ARGMAX_MAX_PARTS * 8));
+        OXB_TRY_HIP(oxb_launch_argmax(d_logits, vocab, batch, d_tok, g_rt.ws_xq.ptr, st), "kernel launch failed: argmax");
+    } else {
+        OXB_TRY_HIP(oxb_launch_sample(d_logits, vocab, batch, params->temperature, params->top_k, params->top_p, d_rng, d_tok, d_ws, st),
+                    "kernel launch failed: sample");
+    }
+    OXB_TRY_HIP(hipMemcpyAsync(tokens_out, d_tok, (size_t)batch * 4, hipMemcpyDeviceToHost, st), "token download");
+    OXB_TRY_HIP(hipMemcpyAsync(rng_state, d_rng, (size_t)batch * 8, hipMemcpyDeviceToHost, st), "rng state download");
+    hipError_t he = hipStreamSynchronize(st);
+    if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: sample_logits: %s", hipGetErrorString(he));
     return OXB_HIP_OK;
 }
 

@@ -64,6 +64,23 @@ def gguf_tensor(path: str, name: str) -> dict:
             "file_offset": off.value, "bytes": nb.value}
 
 
+class Sampling(C.Structure):
+    """oxb_sampling: the SamplingParams fields Sampler::sample reads (crates/oxibonsai-runtime/src/sampling.rs:14-27)."""
+    _fields_ = [("temperature", C.c_float), ("top_k", C.c_uint32), ("top_p", C.c_float)]
+
+
+def sample_logits(logits, temperature: float, top_k: int, top_p: float, rng_state):
+    """Sampler::sample on the device for rows of host logits -> (tokens [batch], advanced rng states [batch])."""
+    a = np.ascontiguousarray(logits, dtype=np.float32)
+    a = a.reshape(1, -1) if a.ndim == 1 else a
+    st = np.ascontiguousarray(np.broadcast_to(np.asarray(rng_state, dtype=np.uint64), (a.shape[0],))).copy()
+    out = np.empty(a.shape[0], dtype=np.uint32)
+    sp = Sampling(temperature, top_k, top_p)
+    _check(_lib.lib().oxb_hip_sample_logits(a.ctypes.data_as(_lib.f32p), a.shape[1], a.shape[0], C.byref(sp),
+                                            st.ctypes.data_as(_lib.u64p), out.ctypes.data_as(_lib.u32p)))
+    return out, st
+
+
 class Embedding:
     """Token embedding table resident on the device in its stored form (F32, F16, Q1_0_g128 or TQ2_0_g128)."""
 
@@ -176,6 +193,18 @@ class HipModel:
         _check(self._lib.oxb_hip_decode_tokens(self.id, embedding.id, tv.ctypes.data_as(_lib.u32p), pv.ctypes.data_as(_lib.u32p),
                                                n_steps, out.ctypes.data_as(_lib.u32p)))
         return out
+
+    def generate_sampled(self, embedding: Embedding, tokens, pos, n_steps: int, temperature: float, top_k: int, top_p: float,
+                         rng_state):
+        """generate() with Sampler::sample instead of the argmax -> (ids [n_steps, batch], advanced rng states [batch])."""
+        tv = np.ascontiguousarray(np.broadcast_to(np.asarray(tokens, dtype=np.uint32), (self.batch,)))
+        pv = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, dtype=np.uint32), (self.batch,)))
+        st = np.ascontiguousarray(np.broadcast_to(np.asarray(rng_state, dtype=np.uint64), (self.batch,))).copy()
+        out = np.empty((n_steps, self.batch), dtype=np.uint32)
+        sp = Sampling(temperature, top_k, top_p)
+        _check(self._lib.oxb_hip_decode_tokens_sampled(self.id, embedding.id, tv.ctypes.data_as(_lib.u32p), pv.ctypes.data_as(_lib.u32p),
+                                                       n_steps, C.byref(sp), st.ctypes.data_as(_lib.u64p), out.ctypes.data_as(_lib.u32p)))
+        return out, st
 
     def prefill_tokens(self, embedding: Embedding, ids, pos_start: int = 0, seq: int = 0, want_logits: bool = True):
         """prefill() with the embedding rows gathered on the device from token ids."""

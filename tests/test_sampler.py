@@ -1,0 +1,149 @@
+"""Sampler::sample (crates/oxibonsai-runtime/src/sampling.rs:84-177): the CPU restatement against the reference's own
+unit tests and what the mathematics fixes, then the device sampler against the restatement."""
+import numpy as np
+import pytest
+
+from oracle import oracle
+from oxibonsai_amd import synth
+
+
+def _xorshift(x):
+    m = (1 << 64) - 1
+    x ^= (x << 13) & m
+    x ^= x >> 7
+    x ^= (x << 17) & m
+    return x
+
+
+def test_reference_unit_tests():
+    # greedy_sampling (:195-204), argmax_basic (:219-222)
+    assert oracle.sample([0.1, 0.5, 0.3, 0.9, 0.2], 0.0, 40, 0.9, 42)[0] == 3
+    assert oracle.sample([1.0, 3.0, 2.0], 0.0, 40, 0.9, 1)[0] == 1 and oracle.sample([5.0], 0.0, 40, 0.9, 1)[0] == 0
+    # sampling_returns_valid_index (:206-216): defaults, seed 12345, 50 draws over 100 equal logits
+    st = 12345
+    for _ in range(50):
+        tok, st, *_ = oracle.sample(np.zeros(100, np.float32), 0.7, 40, 0.9, st)
+        assert tok < 100
+    # buffer_reuse_across_calls (:224-243): top_k = 5 over ascending logits -> only 195..199
+    st, logits = 99, np.arange(200, dtype=np.float32) * np.float32(0.01)
+    seen = set()
+    for _ in range(20):
+        tok, st, ids, p, r = oracle.sample(logits, 0.7, 5, 1.0, st)
+        assert tok >= 195 and sorted(ids) == [195, 196, 197, 198, 199]
+        seen.add(tok)
+    assert len(seen) > 1
+
+
+def test_generator_and_draw():
+    # xorshift64 with shifts 13 / 7 / 17 (:73-80), r = (x as f64 / u64::MAX as f64) as f32 (:160)
+    st = 42
+    for _ in range(5):
+        tok, new, ids, p, r = oracle.sample(np.zeros(8, np.float32), 1.0, 0, 1.0, st)
+        assert new == _xorshift(st)
+        assert r == np.float32(np.float64(new) / np.float64(2**64 - 1))
+        st = new
+    # a zero state stays zero: the draw is 0 and the first candidate wins
+    tok, new, ids, *_ = oracle.sample([0.0, 5.0, 1.0], 1.0, 0, 1.0, 0)
+    assert new == 0 and tok == 1
+
+
+def test_candidates_follow_the_definition():
+    logits = synth.normal_f32(3, 500) * 3.0
+    T, k, tp = 0.8, 50, 0.9
+    tok, _, ids, p, r = oracle.sample(logits, T, k, tp, 777)
+    scaled = (logits / np.float32(T)).astype(np.float64)
+    order = np.argsort(-scaled, kind="stable")[:k]
+    sm = np.exp(scaled[order] - scaled[order[0]])
+    sm /= sm.sum()
+    cut = int(np.argmax(np.cumsum(sm) > tp)) + 1
+    assert list(ids) == list(order[:cut])
+    assert np.allclose(p, sm[:cut] / sm[:cut].sum(), rtol=1e-5) and abs(float(p.sum()) - 1.0) < 1e-5
+    assert tok == ids[int(np.argmax(np.cumsum(p) >= r))]
+    # top_p that is never exceeded keeps everything; a tiny one keeps the best candidate only; low temperature -> argmax
+    assert len(oracle.sample(logits, T, k, 1.5, 1)[2]) == k
+    assert list(oracle.sample(logits, T, k, 1e-6, 1)[2]) == [order[0]]
+    assert all(oracle.sample(logits, 1e-3, 40, 0.9, s)[0] == int(np.argmax(logits)) for s in (1, 2, 3))
+    # frequencies of many draws follow the probabilities (top-p off)
+    lg = np.array([2.0, 1.0, 0.0, -1.0], np.float32)
+    want = np.exp(lg - 2.0) / np.exp(lg - 2.0).sum()
+    st, counts = 0x9E3779B97F4A7C15, np.zeros(4)
+    for _ in range(20000):
+        tok, st, *_ = oracle.sample(lg, 1.0, 0, 1.0, st)
+        counts[tok] += 1
+    assert np.max(np.abs(counts / counts.sum() - want)) < 0.01
+
+
+# --------------------------------------------------------------------------- GPU
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,T,k,tp", [(151936, 0.7, 40, 0.9), (5000, 1.0, 128, 1.0), (33, 0.5, 40, 0.95), (4096, 2.0, 1, 0.9),
+                                      (2049, 0.7, 5, 1.0), (100000, 1e-3, 40, 0.9)])
+def test_device_sampler_matches_restatement(backend, n, T, k, tp):
+    from oxibonsai_amd.model import sample_logits
+    rows = 6
+    logits = (synth.normal_f32(n + k, rows * n) * 4.0).reshape(rows, n)
+    logits[1, 7] = logits[1, 99 % n] = logits[1].max() + 1.0          # an exact tie at the top
+    seeds = np.array([1, 42, 2**63 + 5, 12345, 99, 0], dtype=np.uint64)
+    toks, states = sample_logits(logits, T, k, tp, seeds)
+    for b in range(rows):
+        tok, new, ids, p, r = oracle.sample(logits[b], T, k, tp, int(seeds[b]))
+        assert int(states[b]) == new
+        if int(toks[b]) != tok:
+            # libm and device exp may differ in the last place: then the draw must sit on a cumulative boundary
+            cum = np.cumsum(p.astype(np.float64))
+            assert int(toks[b]) in ids and np.min(np.abs(cum - r)) < 1e-5, (b, int(toks[b]), tok)
+    # a second call continues the generators
+    toks2, states2 = sample_logits(logits, T, k, tp, states)
+    for b in range(rows):
+        assert int(states2[b]) == _xorshift(int(states[b]))
+
+
+@pytest.mark.gpu
+def test_device_sampler_statistics_and_errors(backend):
+    from oxibonsai_amd import GpuError
+    from oxibonsai_amd.model import sample_logits
+    lg = np.tile(np.array([2.0, 1.0, 0.0, -1.0] + [-30.0] * 60, np.float32), (512, 1))
+    want = np.exp(lg[0, :4] - 2.0) / np.exp(lg[0, :4] - 2.0).sum()
+    st = (np.arange(512, dtype=np.uint64) + 1) * np.uint64(0x9E3779B97F4A7C15)
+    counts = np.zeros(64)
+    for _ in range(20):
+        toks, st = sample_logits(lg, 1.0, 8, 1.0, st)
+        counts += np.bincount(toks, minlength=64)
+    assert counts[4:].sum() == 0 and np.max(np.abs(counts[:4] / counts.sum() - want)) < 0.02
+    assert sample_logits([0.1, 0.5, 0.3, 0.9, 0.2], 0.0, 40, 0.9, 42)[0][0] == 3          # greedy_sampling
+    for bad in ((0.7, 0, 0.9), (0.7, 129, 0.9), (-1.0, 40, 0.9), (0.7, 40, 0.0)):
+        with pytest.raises(GpuError) as e:
+            sample_logits(lg[:2], *bad, [1, 2])
+        assert e.value.kind == "InvalidArgument"
+
+
+@pytest.mark.gpu
+def test_sampled_generation_loop(backend, tmp_path):
+    """Token loop with the sampler: every step's token is the sampler's pick from that step's logits."""
+    from helpers import GGUF_F16, TQ2, model_gguf
+    from oxibonsai_amd.model import HipModel
+    cfg = dict(fmt=TQ2, n_layers=2, h=512, inter=1024, nq=8, nkv=2, hd=64, vocab=300, max_seq=128, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 9)
+    table = (synth.embedding_rows(3, range(cfg["vocab"]), cfg["h"]) * 50.0).astype(np.float16)
+    (tmp_path / "m.gguf").write_bytes(model_gguf(cfg, w, GGUF_F16, table))
+    a, emb, _ = HipModel.from_gguf(backend, str(tmp_path / "m.gguf"), batch=2)
+    b = HipModel(backend, cfg, w, batch=2)
+    try:
+        T, k, tp = 0.9, 20, 0.95
+        seeds = np.array([7, 1234567], dtype=np.uint64)
+        ids, states = a.generate_sampled(emb, [5, 17], [0, 0], 12, T, k, tp, seeds)
+        toks, st = np.array([5, 17], dtype=np.uint32), [int(s) for s in seeds]
+        for i in range(12):
+            logits, _ = b.forward(table[toks].astype(np.float32), [i, i])
+            for s in range(2):
+                tok, st[s], cand, p, r = oracle.sample(logits[s], T, k, tp, st[s])
+                if int(ids[i, s]) != tok:
+                    assert int(ids[i, s]) in cand and np.min(np.abs(np.cumsum(p.astype(np.float64)) - r)) < 1e-5
+            toks = ids[i].copy()                                       # follow the device's own tokens
+        assert [int(s) for s in states] == st
+        greedy = a.generate(emb, [5, 17], [0, 0], 4)
+        same, _ = a.generate_sampled(emb, [5, 17], [0, 0], 4, 0.0, 40, 0.9, seeds)      # temperature 0 = the greedy loop
+        assert np.array_equal(greedy, same)
+    finally:
+        a.close()
+        b.close()
+        emb.close()
