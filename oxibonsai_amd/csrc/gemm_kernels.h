@@ -5,8 +5,8 @@
 
 #include "layout.h"
 
-// STORE: y = W a;  RESIDUAL: y = residual + W a;  SWIGLU (at most OXB_GEMM_NARROW_MAX_M token rows): W = gate || up
-// (n_rows = 2 * inter), y[m][i] = silu(gate_i . a) * (up_i . a) for i < inter, ldy >= inter.
+// STORE: y = W a;  RESIDUAL: y = residual + W a;  SWIGLU: W = gate || up (n_rows = 2 * inter, a multiple of 32),
+// y[m][i] = silu(gate_i . a) * (up_i . a) for i < inter, ldy >= inter.
 enum { OXB_GEMM_STORE = 0, OXB_GEMM_RESIDUAL = 2, OXB_GEMM_SWIGLU = 3 };
 #define OXB_GEMM_NARROW_MAX_M 32  // up to this many token rows the narrow kernel (K split over waves) is used
 

@@ -345,6 +345,11 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     const uint32_t t0 = wg_t0 + wave * per;
     const uint32_t t1 = min(t0 + per, wg_t1);
     const uint32_t n_valid = t1 > t0 ? t1 - t0 : 0u;
+    // SWIGLU mode (the matrix is gate || up): the tile sequence interleaves gate tile j and up tile j, and every
+    // wave starts on a gate tile (the launcher gives it an even count), so accumulators 2q and 2q+1 hold both
+    // factors of 16 output rows.
+    const bool sw = p.mode == OXB_GEMM_SWIGLU;
+    auto tile_of = [&](uint32_t u) -> uint32_t { return sw ? ((u & 1u) ? p.n_tiles / 2 + (u >> 1) : (u >> 1)) : u; };
 
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.codes, p.codes_bytes), rs = make_rsrc(p.scales, p.scales_bytes);
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.xh, p.xh_bytes);
@@ -378,8 +383,8 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     stage_x(sb0 * 4, xs0);
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
-        load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
+        load_half<FMT>(H[rt][0], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
+        load_half<FMT>(H[rt][1], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
     }
     publish();
     BlockDec bd[RT], bdn[RT];
@@ -406,7 +411,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             bdn[rt] = prepare_block<FMT>(H[rt][1], 0);
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
         publish();
         // block 2
@@ -426,7 +431,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             bdn[rt] = prepare_block<FMT>(H[rt][0], 0);
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, t0 + rt, (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
         publish();
 #pragma unroll
@@ -446,11 +451,21 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             if ((uint32_t)rt >= n_valid) continue;
-            const uint32_t n = (t0 + rt) * 16 + 4 * g;
+            if (sw && (rt & 1)) continue;  // the up factor: consumed with its gate tile
+            const uint32_t n = sw ? ((t0 + rt) >> 1) * 16 + 4 * g : (t0 + rt) * 16 + 4 * g;
+            const uint32_t n_lim = sw ? p.n_rows / 2 : p.n_rows;
             float o[4];
 #pragma unroll
             for (int v = 0; v < 4; v++) o[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(acc[rt][ct][v], e);
-            if (vec_ok && n + 3 < p.n_rows) {
+            if (sw) {
+                constexpr int ru = RT > 1 ? 1 : 0;  // (RT = 1 is never launched in this mode)
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float u = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(acc[rt + ru < RT ? rt + ru : rt][ct][v], e);
+                    o[v] = silu_mul(o[v], u);
+                }
+            }
+            if (vec_ok && n + 3 < n_lim) {
                 if (rr) {
                     const float4 q4 = *reinterpret_cast<const float4*>(rr + n);
                     o[0] += q4.x, o[1] += q4.y, o[2] += q4.z, o[3] += q4.w;
@@ -459,7 +474,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             } else {
 #pragma unroll
                 for (int v = 0; v < 4; v++)
-                    if (n + v < p.n_rows) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
+                    if (n + v < n_lim) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
             }
         }
     }
@@ -676,13 +691,16 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
     const uint32_t n_mt = (p.M + BM - 1) / BM;
     static const uint32_t rts[] = {5, 4, 3, 2, 1};
     GemmPlan best = {1, 4, 1, p.n_sb};
+    if (p.mode == OXB_GEMM_SWIGLU) best = {2, 8, 1, p.n_sb};
     uint64_t best_cost = ~0ull;
-    const bool can_split = (p.ldy & 3u) == 0;
+    const bool sw = p.mode == OXB_GEMM_SWIGLU;  // even tile counts per wave, no K split (the epilogue is not linear)
+    const bool can_split = (p.ldy & 3u) == 0 && !sw;
     for (uint32_t ks = 1; ks <= (can_split ? 8u : 1u) && ks <= p.n_sb; ks++) {
         const uint32_t spk = (p.n_sb + ks - 1) / ks;
         if (ks > 1 && (p.n_sb + spk - 1) / spk != ks) continue;  // same slices as a smaller count
         for (uint32_t rt : rts) {
-            for (uint32_t tpw = 4 * rt; tpw > 4 * rt - 4; tpw--) {
+            if (sw && (rt & 1u)) continue;
+            for (uint32_t tpw = 4 * rt; tpw > (sw ? 4 * rt - 1 : 4 * rt - 4); tpw--) {
                 const uint32_t groups = (p.n_tiles + tpw - 1) / tpw;
                 const uint64_t wgs = (uint64_t)groups * n_mt * ks;
                 uint64_t cost = ((wgs + n_cus - 1) / n_cus) * ((uint64_t)spk * (rt + 1) + 2 * rt + 2);
@@ -733,7 +751,7 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     if (p.n_sb == 0 || (uint64_t)p.n_tiles * p.n_sb * 2048ull >= 0xFFFFFFF0ull) return hipErrorInvalidValue;
     p.M_pad = (p.M + 15u) / 16u * 16u;
     if (p.M <= OXB_GEMM_NARROW_MAX_M) return launch_gemm_narrow(fmt, p, n_cus, st);
-    if (p.mode == OXB_GEMM_SWIGLU) return hipErrorInvalidValue;  // only the narrow kernel has that epilogue
+    if (p.mode == OXB_GEMM_SWIGLU && (p.n_rows & 31u) != 0) return hipErrorInvalidValue;  // whole gate and up row tiles
     constexpr uint32_t CT = 8, BM = 16 * CT;
     p.n_mt = (p.M + BM - 1) / BM;
     const GemmPlan plan = plan_gemm(p, n_cus);

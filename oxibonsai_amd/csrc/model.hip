@@ -254,13 +254,9 @@ static int encode_decode_step_gemm(Model& m) {
         OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
                     "kernel launch failed: attn_combine");
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
-        if (B <= OXB_GEMM_NARROW_MAX_M) {  // SwiGLU in the epilogue of the gate || up product
-            OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
-            OXB_TRY(gemm_device(*wdn, m.gu, d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
-        } else {
-            OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
-            OXB_TRY(gemm_device(*wdn, m.gu, 2 * d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_SWIGLU, nullptr, 0.f, &m.gws));
-        }
+        // SwiGLU in the epilogue of the gate || up product
+        OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
+        OXB_TRY(gemm_device(*wdn, m.gu, d.inter, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
     }
     const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
     const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
@@ -333,7 +329,7 @@ static int ensure_prefill_buffers(Model& m, uint32_t rows) {
     const oxb_model_desc& d = m.d;
     const size_t R = (rows + 127u) / 128u * 128u, qd = (size_t)d.nq * d.hd, qkv_rows = qd + 2 * (size_t)d.nkv * d.hd;
     struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_qkv, R * qkv_rows}, {&m.pf_q, R * qd},
-                                             {&m.pf_attn, R * qd},    {&m.pf_gu, R * 2 * d.inter}};
+                                             {&m.pf_attn, R * qd},    {&m.pf_gu, R * d.inter}};
     for (auto& b : bufs) {
         if (hipMalloc((void**)b.p, b.n * sizeof(float)) != hipSuccess) {
             for (void* p : m.pf_allocs) (void)hipFree(p);
@@ -402,8 +398,9 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         ap.scale = 1.0f / sqrtf((float)d.hd);
         OXB_TRY_HIP(oxb_launch_attn_prefill(ap, st), "kernel launch failed: attn_prefill");
         OXB_TRY(gemm_device(*wo, m.pf_attn, qd, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_IDENT, nullptr, 0.f));
-        OXB_TRY(gemm_device(*wgu, m.pf_hidden, d.h, m.pf_gu, M, 2 * d.inter, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps));
-        OXB_TRY(gemm_device(*wdn, m.pf_gu, 2 * d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_SWIGLU, nullptr, 0.f));
+        // SwiGLU in the epilogue of the gate || up product: the activation [M][inter] is all that is written
+        OXB_TRY(gemm_device(*wgu, m.pf_hidden, d.h, m.pf_gu, M, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps));
+        OXB_TRY(gemm_device(*wdn, m.pf_gu, d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_IDENT, nullptr, 0.f));
     }
     // last token: final norm, LM head, greedy token (fp32-exact products, as in a decode step)
     const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
