@@ -34,9 +34,9 @@ size_t oxb_xh_bytes(uint32_t k, uint32_t M);
 
 // Activations a[M][k] -> fp16 in MFMA B-operand order, each row scaled by a power of two so that its largest
 // element lies in [2^14, 2^15).  The activations are computed on the fly from x[M][ldx] by `op`:
-//   IDENT: a = x;  RMSNORM: a = w * x / rms(x) (w = d_w[k]);  SWIGLU: a = silu(x[.. k)) * x[k .. 2k) (ldx >= 2k).
+//   IDENT: a = x;  RMSNORM: a = w * x / rms(x) (w = d_w[k]).
 // d_rowmul: M floats of scratch (the multiplier applied to every row).
-enum { OXB_PACK_IDENT = 0, OXB_PACK_RMSNORM = 1, OXB_PACK_SWIGLU = 2 };
+enum { OXB_PACK_IDENT = 0, OXB_PACK_RMSNORM = 1 };
 hipError_t oxb_launch_xh_pack(int fmt, int op, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, float eps,
                               uint32_t M, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st);
 // Number of K slices the launcher will use for this shape (1: no workspace needed).

@@ -35,11 +35,11 @@ typedef _Float16 v2h __attribute__((ext_vector_type(2)));
 // Activation packer, fused with the row-wise producer of the activations:
 //   OXB_PACK_IDENT   a[m][k] = x[m][k]
 //   OXB_PACK_RMSNORM a[m][k] = w[k] * x[m][k] / sqrt(mean_k x[m][k]^2 + eps)      (simd_float_ops.rs:204-215)
-//   OXB_PACK_SWIGLU  a[m][k] = silu(x[m][k]) * x[m][k + K],  x = [gate | up]        (simd_float_ops.rs:217-236)
 // Two kernels: row_stats (one workgroup per token row) finds the row's multiplier - the producer's scalar
 // times the power of two that puts the row's largest |a| into [2^14, 2^15) - and the exponent that undoes the
 // power of two; xh_pack (one workgroup = 16 token rows x a share of the blocks) recomputes a from x and writes
-// fp16 in MFMA B-operand order.  The fp32 activations never go to memory.  A few token rows (decode batches)
+// fp16 in MFMA B-operand order.  The normalised activations never go to memory in fp32.  (SwiGLU is not a packer
+// operation: the gate || up GEMM applies it in its epilogue, simd_float_ops.rs:217-236.)  A few token rows (decode batches)
 // take both steps in one launch, xh_pack_rows, one workgroup per row.
 // ---------------------------------------------------------------------------
 __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
@@ -62,9 +62,6 @@ __device__ __forceinline__ void row_stats(const float* __restrict__ xr, const fl
             const float4 g = *reinterpret_cast<const float4*>(w + i);
             ss = fmaf(v.x, v.x, fmaf(v.y, v.y, fmaf(v.z, v.z, fmaf(v.w, v.w, ss))));
             a = make_float4(g.x * v.x, g.y * v.y, g.z * v.z, g.w * v.w);
-        } else if (OP == OXB_PACK_SWIGLU) {
-            const float4 u = *reinterpret_cast<const float4*>(xr + k + i);
-            a = make_float4(silu_mul(v.x, u.x), silu_mul(v.y, u.y), silu_mul(v.z, u.z), silu_mul(v.w, u.w));
         }
         bad |= !(fabsf(a.x) <= 3.402823466e38f) | !(fabsf(a.y) <= 3.402823466e38f) | !(fabsf(a.z) <= 3.402823466e38f) |
                !(fabsf(a.w) <= 3.402823466e38f);
@@ -123,10 +120,6 @@ __device__ __forceinline__ uint4 pack_item(const float* __restrict__ xr, const f
         const float4 wa = *reinterpret_cast<const float4*>(w + blk * 128 + k0), wb = *reinterpret_cast<const float4*>(w + blk * 128 + k1);
         a = make_float4(wa.x * a.x, wa.y * a.y, wa.z * a.z, wa.w * a.w);
         b = make_float4(wb.x * b.x, wb.y * b.y, wb.z * b.z, wb.w * b.w);
-    } else if (OP == OXB_PACK_SWIGLU) {
-        const float4 ua = *reinterpret_cast<const float4*>(xb + k + k0), ub = *reinterpret_cast<const float4*>(xb + k + k1);
-        a = make_float4(silu_mul(a.x, ua.x), silu_mul(a.y, ua.y), silu_mul(a.z, ua.z), silu_mul(a.w, ua.w));
-        b = make_float4(silu_mul(b.x, ub.x), silu_mul(b.y, ub.y), silu_mul(b.z, ub.z), silu_mul(b.w, ub.w));
     }
     return make_uint4(pack_h2(a.x * mul, b.x * mul), pack_h2(a.y * mul, b.y * mul), pack_h2(a.z * mul, b.z * mul),
                       pack_h2(a.w * mul, b.w * mul));
@@ -668,7 +661,6 @@ hipError_t oxb_launch_xh_pack(int fmt, int op, const float* d_x, const float* d_
     switch (op) {
         case OXB_PACK_IDENT: launch_pack_op<OXB_PACK_IDENT>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
         case OXB_PACK_RMSNORM: launch_pack_op<OXB_PACK_RMSNORM>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
-        case OXB_PACK_SWIGLU: launch_pack_op<OXB_PACK_SWIGLU>(fmt, d_x, d_w, ldx, k, M, M_pad, nblk_pad, eps, d_rowmul, d_xh, d_xsh, st); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
