@@ -265,10 +265,12 @@ class OracleModel:
     ``final_norm`` and ``lm_head``.
     """
 
-    def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False):
+    def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False, dot_f64: bool = False):
+        """dot_f64: every linear layer sums in double (not the reference's arithmetic; a yardstick for how far the
+        fp32 summation order moves the result at a given model size)."""
         self.cfg = cfg
         self._keep = []
-        fmt = cfg["fmt"]
+        fmt = cfg["fmt"] + (2 if dot_f64 else 0)
         h, inter, nq, nkv, hd = cfg["h"], cfg["inter"], cfg["nq"], cfg["nkv"], cfg["hd"]
 
         def lin(arr, n_rows, k):

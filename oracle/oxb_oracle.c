@@ -154,6 +154,7 @@ int oxb_gemv_q1(const uint8_t* blocks, size_t n_blocks, const float* x, size_t x
     if (y_len < n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
     size_t bpr = k / OXB_QK;
     if (n_blocks < n_rows * bpr) return OXB_ERR_BUFFER_TOO_SMALL;
+#pragma omp parallel for schedule(static) if (n_rows * bpr > 4096)  /* rows are independent: same bits, less waiting */
     for (size_t r = 0; r < n_rows; r++)
         y[r] = q1_row_dot(blocks + r * bpr * OXB_Q1_BYTES, bpr, x);
     return OXB_OK;
@@ -167,6 +168,7 @@ int oxb_gemv_tq2(const uint8_t* blocks, size_t n_blocks, const float* x, size_t 
     if (y_len < n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
     size_t bpr = k / OXB_QK;
     if (n_blocks < n_rows * bpr) return OXB_ERR_DIMENSION_MISMATCH;
+#pragma omp parallel for schedule(static) if (n_rows * bpr > 4096)
     for (size_t r = 0; r < n_rows; r++)
         y[r] = tq2_row_dot(blocks + r * bpr * OXB_TQ2_BYTES, bpr, x);
     return OXB_OK;
@@ -391,7 +393,37 @@ struct oxb_state {
     float *hidden, *normed, *q, *k, *v, *qn, *kn, *qr, *kr, *attn, *proj, *gate, *up, *act, *down;
 };
 
+/* The same row products with every sum kept in double (block sums and the row total), rounded to float once:
+ * not the reference's arithmetic but a check on it - with 24 more bits the order of the additions no longer
+ * matters, so this is what any correct tier converges to. */
+static void linear_fwd_f64(int fmt, const oxb_linear* l, const float* x, float* y) {
+    const size_t bpr = l->k / OXB_QK, bb = fmt == 0 ? OXB_Q1_BYTES : OXB_TQ2_BYTES;
+#pragma omp parallel for schedule(static) if (l->n_rows * bpr > 4096)
+    for (size_t r = 0; r < l->n_rows; r++) {
+        const uint8_t* row = l->blocks + r * bpr * bb;
+        double sum = 0.0;
+        for (size_t bi = 0; bi < bpr; bi++) {
+            const uint8_t* b = row + bi * bb;
+            const float* xb = x + bi * OXB_QK;
+            double bs = 0.0;
+            if (fmt == 0) {
+                for (size_t j = 0; j < OXB_QK; j++) bs += ((b[2 + j / 8] >> (j % 8)) & 1u) ? (double)xb[j] : -(double)xb[j];
+                sum += (double)q1_scale(b) * bs;
+            } else {
+                for (size_t byte = 0; byte < 32; byte++)
+                    for (unsigned lane = 0; lane < 4; lane++) bs += (double)tq2_code(b[byte], lane) * (double)xb[byte * 4 + lane];
+                sum += (double)tq2_scale(b) * bs;
+            }
+        }
+        y[r] = (float)sum;
+    }
+}
+
 static int linear_fwd(int fmt, const oxb_linear* l, const float* x, float* y) {
+    if (fmt >= 2) {
+        linear_fwd_f64(fmt - 2, l, x, y);
+        return OXB_OK;
+    }
     size_t nb = l->n_rows * (l->k / OXB_QK);
     return fmt == 0 ? oxb_gemv_q1(l->blocks, nb, x, l->k, y, l->n_rows, l->n_rows, l->k)
                     : oxb_gemv_tq2(l->blocks, nb, x, l->k, y, l->n_rows, l->n_rows, l->k);

@@ -97,7 +97,7 @@ typedef struct {
 } oxb_layer;
 
 typedef struct {
-    int fmt;
+    int fmt;                  /* 0 / 1 as above; 2 / 3: the same formats with every linear layer summed in double */
     size_t n_layers, h, inter, nq, nkv, hd, vocab, max_seq;
     float eps, rope_theta;
     const oxb_layer* layers;

@@ -199,3 +199,53 @@ def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt, B):
         assert gpu.uses_graph()
     finally:
         gpu.close()
+
+
+@pytest.mark.parametrize("name,cfg", [
+    ("qwen3-8b-shape-q1", dict(fmt=Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd=128, vocab=151936, max_seq=256,
+                               eps=1e-6, rope_theta=1e6)),
+    ("qwen3-1.7b-shape-ternary", dict(fmt=TQ2, n_layers=28, h=2048, inter=6144, nq=16, nkv=8, hd=128, vocab=151936, max_seq=256,
+                                      eps=1e-6, rope_theta=1e6)),
+])
+def test_full_size_shapes_match_oracle(backend, name, cfg):
+    """The two model shapes the measurements are quoted on, at their real sizes: three decode steps, then a batched
+    prefill of eight more positions, against the oracle.
+
+    At 28-36 layers of width 2048-4096 the reference's 1e-3 gate no longer separates right from wrong: its own
+    scalar fp32 sums sit 1.4-1.9e-3 (abs, logits up to 20) from the same forward with double sums, and every value
+    that rounds differently into the f16 KV cache - a last-bit difference before the rounding is enough - moves the
+    logits by 2-5e-4, for this path and for any other.  Measured here: 1.5e-3 at position 0 (no attention history;
+    the scalar oracle itself: 1.9e-3), up to 4e-3 afterwards.  The bar: 5e-4 of the largest logit (about 1e-2
+    absolute), the greedy token equal wherever the oracle's margin exceeds that, and at position 0 no further from
+    the double-sum forward than the scalar oracle is."""
+    w = synth.make_model(cfg, 0xB0A5A104)
+    cpu = oracle.OracleModel(cfg, w, kv_f16=True)
+    c64 = oracle.OracleModel(cfg, w, kv_f16=True, dot_f64=True)
+    gpu = HipModel(backend, cfg, w, batch=1)
+    try:
+        toks = [11, 70000, 151935]
+        rows = [synth.embedding_rows(0xE3B, [t], cfg["h"])[0] * 50.0 for t in toks]
+        for pos, r in enumerate(rows):
+            want = cpu.forward(r, pos)
+            got, tok = gpu.forward(r, pos)
+            tol = 5e-4 * float(np.max(np.abs(want)))
+            err = float(np.max(np.abs(got[0] - want)))
+            assert err < tol, (name, pos, err, tol)
+            top2 = np.sort(want)[-2:]
+            if top2[1] - top2[0] > 2 * tol:
+                assert tok[0] == oracle.argmax_first(want)
+            if pos == 0:
+                w64 = c64.forward(r, pos)
+                assert np.max(np.abs(got[0] - w64)) <= 1.1 * np.max(np.abs(want - w64)), (name, "position 0 vs double sums")
+        more = synth.embedding_rows(0xE3B, [5, 6, 7, 8, 9, 10, 12, 13], cfg["h"]) * 50.0
+        got, _ = gpu.prefill(more, pos_start=3)
+        for i, r in enumerate(more):
+            want = cpu.forward(r, 3 + i, want_logits=i == len(more) - 1)
+        # the prefill GEMMs round every activation to fp16 (11 bits): about 2.8e-4 of relative noise per product,
+        # four products per layer in quadrature - 3.4e-3 of the logit scale after 36 layers (measured: 0.068 on
+        # logits up to 20), the same order as what the f16 KV cache alone does to the logits
+        tol = 5e-3 * float(np.max(np.abs(want)))
+        err = float(np.max(np.abs(got - want)))
+        assert err < tol, (name, "prefill", err, tol)
+    finally:
+        gpu.close()

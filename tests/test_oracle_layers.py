@@ -142,6 +142,15 @@ def test_model_forward_matches_float64_numpy():
         for pos, hid in enumerate(hiddens):
             got = m.forward(hid, pos)
             assert np.max(np.abs(got - want[pos])) < 2e-4 * max(1.0, np.max(np.abs(want[pos]))), (fmt, pos)
+        # the double-sum variant of the linear layers (a yardstick, not the reference's arithmetic) sits closer to
+        # the float64 forward than the fp32 sums do
+        m64 = oracle.OracleModel(cfg, w, kv_f16=False, dot_f64=True)
+        e32 = e64 = 0.0
+        m = oracle.OracleModel(cfg, w, kv_f16=False)
+        for pos, hid in enumerate(hiddens):
+            e32 = max(e32, float(np.max(np.abs(m.forward(hid, pos) - want[pos]))))
+            e64 = max(e64, float(np.max(np.abs(m64.forward(hid, pos) - want[pos]))))
+        assert e64 <= e32 and e64 < 2e-5 * max(1.0, max(float(np.max(np.abs(x))) for x in want))
         # with the f16 KV rounding of the reference's GPU cache the logits move, but only slightly
         m16 = oracle.OracleModel(cfg, w, kv_f16=True)
         d = max(np.max(np.abs(m16.forward(hid, pos) - want[pos])) for pos, hid in enumerate(hiddens))
