@@ -65,9 +65,19 @@ def cpu_baseline(blocks: dict, xs: dict, budget_s: float = 12.0) -> dict:
         times.append(time.perf_counter() - t0)
     med = float(np.median(times))
     total = sum(algorithmic_bytes(r, k) for _, r, k in SHAPES)
+    # the reference's scalar tier on one thread: two passes over the same set, the faster one
+    oracle.set_threads(1)
+    t_scalar = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        for name, n_rows, k in SHAPES:
+            oracle.gemv(FMT_Q1, blocks[name], xs[name], n_rows, k)
+        t_scalar.append(time.perf_counter() - t0)
+    oracle.set_threads(0)
     return {"value": round(total / med / 1e9, 3), "unit": "GB/s", "cores": oracle.simd_threads(),
             "kind": "port", "tier": oracle.simd_tier(),
-            "sample": f"{reps} passes over the same 3-GEMV set (median), {sum(times):.1f} s of CPU time"}
+            "sample": f"{reps} passes over the same 3-GEMV set (median), {sum(times):.1f} s of CPU time",
+            "scalar_tier_1_thread_GBps": round(total / min(t_scalar) / 1e9, 3)}
 
 
 DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd=128, vocab=151936,
@@ -197,6 +207,44 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
         res["cpu_linear_layers_only_tok_per_s"] = round(1.0 / (36 * t_layer + t_lm), 2)
         res["cpu_cores"] = oracle.simd_threads()
     return res
+
+
+TERNARY_CFG = dict(fmt=FMT_TQ2, n_layers=28, h=2048, inter=6144, nq=16, nkv=8, hd=128, vocab=151936,
+                   max_seq=4096, eps=1e-6, rope_theta=1e6)   # BASELINE.json configs[3]: Qwen3-1.7B shape, TQ2_0_g128
+
+
+def decode_ternary_leg(be, prompt_len: int, n_tokens: int) -> dict:
+    """Greedy batch-1 decode of the random-init ternary 1.7B-shape model after a batched prefill, as decode_leg."""
+    from oxibonsai_amd import synth
+    from oxibonsai_amd.model import HipModel
+    cfg = TERNARY_CFG
+    w = synth.make_model(cfg, 0xB0A5A103)
+    m = HipModel(be, cfg, w, batch=1)
+    ids = (synth.splitmix64(0xB0A5A1030F, prompt_len) % np.uint64(cfg["vocab"])).astype(np.int64)
+    table = {}
+
+    def emb(t):
+        if t not in table:
+            table[t] = synth.embedding_rows(0xE3C, [t], cfg["h"])[0] * 50.0
+        return table[t]
+
+    rows = np.stack([emb(int(t)) for t in ids])
+    m.prefill(rows, want_logits=False)
+    t0 = time.perf_counter()
+    _, tok = m.prefill(rows, want_logits=False)
+    t_prefill = time.perf_counter() - t0
+    spent = 0.0
+    for i in range(n_tokens):
+        hidden = emb(tok)
+        t0 = time.perf_counter()
+        _, out = m.forward(hidden, prompt_len + i, want_logits=False)
+        spent += time.perf_counter() - t0
+        tok = int(out[0])
+    m.close()
+    return {"model": "random-init Qwen3-1.7B shape, TQ2_0_g128 (28 layers, h 2048, 16/8 heads, inter 6144, vocab 151936)",
+            "batch": 1, "context_before": prompt_len, "prefill_ms": round(t_prefill * 1e3, 2),
+            "prefill_tok_per_s": round(prompt_len / t_prefill, 1), "tokens": n_tokens,
+            "tok_per_s": round(n_tokens / spent, 2), "ms_per_token": round(spent / n_tokens * 1e3, 4)}
 
 
 PREFILL_SHAPES = [("qkv", 5120, 2560), ("gate_up", 19456, 2560), ("down", 2560, 9728)]   # BASELINE.json configs[2]
@@ -358,6 +406,26 @@ def main() -> int:
                                          "GB/s": round(algorithmic_bytes(lm_rows, lm_k) / (us.value * 1e-6) / 1e9, 1)}
     for h in lm_ids:
         be.free_weights(h)
+    # the same three shapes with ONE resident copy: every launch re-reads what the last one left in the caches
+    # (a cache-resident figure, reported apart from the rotating-copies one above)
+    cache_resident = {}
+    for nm, r, kk in SHAPES:
+        arr = (C.c_uint64 * 1)(int(ids[nm][0]))
+        L.oxb_hip_profile_gemv(arr, 1, d_x[nm].data_ptr(), d_y[nm].data_ptr(), r, kk, 20, 200, C.byref(us))
+        cache_resident[nm] = {"us": round(us.value, 3), "GB/s": round(algorithmic_bytes(r, kk) / (us.value * 1e-6) / 1e9, 1)}
+    # BASELINE.json configs[0]: TQ2_0_g128 GEMV 12288 x 2048, batch 1, 96 rotating copies (642 MB)
+    c0_rows, c0_k, c0_copies = 12288, 2048, 96
+    c0_blocks = synth.make_tq2_blocks(0xB0A5A10000, c0_rows * (c0_k // 128))
+    c0_ids = [be.upload_weights_ternary(c0_blocks, c0_rows, c0_k) for _ in range(c0_copies)]
+    c0_x = torch.from_numpy(synth.normal_f32(0xB0A5A10080, c0_k)).cuda()
+    c0_y = torch.zeros(c0_rows, dtype=torch.float32, device="cuda")
+    arr = (C.c_uint64 * c0_copies)(*[int(h) for h in c0_ids])
+    L.oxb_hip_profile_gemv(arr, c0_copies, c0_x.data_ptr(), c0_y.data_ptr(), c0_rows, c0_k, 20, 400, C.byref(us))
+    c0_bytes = algorithmic_bytes(c0_rows, c0_k, 1, 34)
+    per_kernel["tq2_12288x2048"] = {"us": round(us.value, 3), "GB/s": round(c0_bytes / (us.value * 1e-6) / 1e9, 1),
+                                    "bytes_per_launch": c0_bytes}
+    for h in c0_ids:
+        be.free_weights(h)
 
     out = {
         "metric": "quant GEMV HBM GB/s", "value": round(value, 2), "unit": "GB/s",
@@ -371,7 +439,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                      "kernel": "gemv_mfma_kernel<Q1> gate||up 24576x4096", "bytes_per_launch": kbytes,
-                     "avg_launch_us": round(avg_us.value, 3), "per_kernel": per_kernel},
+                     "avg_launch_us": round(avg_us.value, 3), "per_kernel": per_kernel,
+                     "per_kernel_cache_resident": cache_resident},
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(blocks, xs)
@@ -391,6 +460,7 @@ def main() -> int:
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
                                    tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf)
+        out["decode_ternary_1p7b"] = decode_ternary_leg(be, args.decode_context, args.decode_tokens)
     print(json.dumps(out), flush=True)
     return 0
 

@@ -66,6 +66,8 @@ def lib() -> C.CDLL:
             getattr(L, n).argtypes = [f32p, sz]
             getattr(L, n).restype = C.c_uint32
         L.oxb_state_new.restype = C.c_void_p
+        L.oxb_oracle_set_threads.argtypes = [C.c_int]
+        L.oxb_oracle_set_threads.restype = None
         L.oxb_sample.restype = C.c_uint32
         L.oxb_sample.argtypes = [f32p, sz, C.c_float, sz, C.c_float, C.POINTER(C.c_uint64), C.POINTER(C.c_uint32), f32p, sz,
                                  C.POINTER(sz), f32p]
@@ -160,6 +162,11 @@ def simd_gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int) -> np.ndarray:
 
 def simd_tier() -> str:
     return {0: "scalar", 1: "avx2+fma", 2: "avx512"}[lib().oxb_simd_tier()]
+
+
+def set_threads(n: int) -> None:
+    """Threads for the row loops of the scalar kernels (0 = all cores); results do not depend on it."""
+    lib().oxb_oracle_set_threads(n)
 
 
 def simd_threads() -> int:

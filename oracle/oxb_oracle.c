@@ -6,6 +6,9 @@
 
 #include <math.h>
 #include <stdlib.h>
+#ifdef _OPENMP
+#include <omp.h>
+#endif
 #include <string.h>
 
 /* ------------------------------------------------------------------------- */
@@ -144,6 +147,16 @@ static float tq2_row_dot(const uint8_t* row_blocks, size_t blocks_per_row, const
         sum += d * block_sum;
     }
     return sum;
+}
+
+/* Threads the row loops of the scalar kernels may use (rows are independent, so the results do not depend on it);
+ * 1 gives the single-thread time of the reference's scalar tier. */
+void oxb_oracle_set_threads(int n) {
+#ifdef _OPENMP
+    omp_set_num_threads(n > 0 ? n : omp_get_num_procs());
+#else
+    (void)n;
+#endif
 }
 
 /* kernels/src/gemv.rs:25-87 (validation order :32-58) */

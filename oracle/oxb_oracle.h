@@ -52,6 +52,7 @@ enum {
 #define OXB_Q1_BYTES 18     /* [d: f16 LE][qs: 16 B]                        */
 #define OXB_TQ2_BYTES 34    /* [qs: 32 B][d: f16 LE]                        */
 
+void     oxb_oracle_set_threads(int n);  /* row-loop threads of the scalar kernels; 0 = all cores */
 float    oxb_f16_to_f32(uint16_t h);
 uint16_t oxb_f32_to_f16(float f);  /* round-to-nearest-even, as half::f16::from_f32 */
 
