@@ -406,6 +406,17 @@ __global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
     const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
+    // The first slots' partial outputs of this thread's first four elements do not depend on the slot weights:
+    // request them before the weights are worked out, so that both round trips to memory overlap.
+    constexpr int PRE = 8;
+    float4 pre[PRE];
+    {
+        const uint32_t e = e0 + tid * 4;
+        const float* ph = part + (size_t)(e / hd) * p.n_splits * stride + e % hd;
+#pragma unroll
+        for (int u = 0; u < PRE; u++)
+            pre[u] = (e < e1 && (uint32_t)u < used) ? *reinterpret_cast<const float4*>(ph + (size_t)u * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
     for (uint32_t hh = tid >> 6; hh < nh; hh += 4) {
         const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
         const float mv = lane < used ? ph[0] : -INFINITY, lv = lane < used ? ph[1] : 0.f;
@@ -424,16 +435,24 @@ __global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p
         const uint32_t h = e / hd, d = e % hd, hh = h - h_first;
         const float* ph = part + (size_t)h * p.n_splits * stride + d;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        uint32_t s = 0;
-        for (; s + 4 <= used; s += 4) {
-            float4 v[4];
+        // slots are added in ascending order, PRE requests in flight at a time
+        auto fold = [&](const float4 (&v)[PRE], uint32_t s0) {
 #pragma unroll
-            for (int u = 0; u < 4; u++) v[u] = *reinterpret_cast<const float4*>(ph + (size_t)(s + u) * stride);
-#pragma unroll
-            for (int u = 0; u < 4; u++) {
-                const float w = wts[hh * 64 + s + u];
+            for (int u = 0; u < PRE; u++) {
+                const float w = s0 + u < used ? wts[hh * 64 + s0 + u] : 0.f;  // (slots past `used` were loaded as zeros)
                 acc.x = fmaf(v[u].x, w, acc.x), acc.y = fmaf(v[u].y, w, acc.y), acc.z = fmaf(v[u].z, w, acc.z), acc.w = fmaf(v[u].w, w, acc.w);
             }
+        };
+        uint32_t s = 0;
+        if (e == e0 + tid * 4) {  // the element group whose first slots are already here
+            fold(pre, 0);
+            s = PRE;
+        }
+        for (; s + PRE <= used; s += PRE) {
+            float4 v[PRE];
+#pragma unroll
+            for (int u = 0; u < PRE; u++) v[u] = *reinterpret_cast<const float4*>(ph + (size_t)(s + u) * stride);
+            fold(v, s);
         }
         for (; s < used; s++) {
             const float4 v = *reinterpret_cast<const float4*>(ph + (size_t)s * stride);
