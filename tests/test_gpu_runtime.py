@@ -1,0 +1,87 @@
+"""Runtime behaviour of the native-hip library through the C ABI: calls from several host threads, device memory
+given back when handles and models are released (the reference serialises its CUDA graph singleton behind a Mutex,
+gpu_backend/cuda_graph/cudagraph_type.rs:18-32; weights live until freed, gpu_backend/mod.rs:445-472)."""
+import threading
+
+import numpy as np
+import pytest
+
+from helpers import Q1, TQ2
+from oracle import oracle
+from oxibonsai_amd import synth
+from oxibonsai_amd.model import HipModel
+
+pytestmark = pytest.mark.gpu
+
+
+def test_calls_from_several_threads_are_serialised(backend):
+    shapes = [(Q1, 640, 1024), (TQ2, 384, 2048), (Q1, 100, 512), (TQ2, 1000, 256)]
+    work = []
+    for i, (fmt, n, k) in enumerate(shapes):
+        a = synth.make_blocks(fmt, 300 + i, n, k)
+        h = backend.upload_weights_raw(a, n, k) if fmt == Q1 else backend.upload_weights_ternary(a, n, k)
+        x = synth.normal_f32(400 + i, k)
+        call = backend.gemv_q1_g128_cached if fmt == Q1 else backend.gemv_tq2_g128_cached
+        work.append((call, h, x, n, k, call(h, x, n, k)))
+    errors = []
+
+    def worker(idx):
+        call, h, x, n, k, want = work[idx]
+        try:
+            for _ in range(60):
+                got = call(h, x, n, k)
+                if not np.array_equal(got, want):
+                    errors.append((idx, "result changed"))
+                    return
+        except Exception as e:   # noqa: BLE001
+            errors.append((idx, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(len(work))]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    for _, h, *_ in work:
+        backend.free_weights(h)
+    assert not errors, errors
+
+
+def test_device_memory_returns_when_models_and_weights_go(backend):
+    cfg = dict(fmt=TQ2, n_layers=2, h=512, inter=1024, nq=8, nkv=2, hd=64, vocab=1000, max_seq=2048, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 5)
+    rows = synth.embedding_rows(3, range(40), cfg["h"]) * 50.0
+
+    def cycle():
+        m = HipModel(backend, cfg, w, batch=4)
+        m.prefill(rows, seq=1, want_logits=False)
+        m.forward(np.stack([rows[0]] * 4), [0, 40, 0, 0], want_logits=False)
+        m.close()
+
+    cycle()                                  # the library's own grow-only workspaces reach their size here
+    backend.synchronize()
+    free0, total = backend.memory_info()
+    for _ in range(5):
+        cycle()
+    backend.synchronize()
+    free1, _ = backend.memory_info()
+    assert total > 0 and abs(free0 - free1) < 8 << 20, (free0, free1)     # within one allocator granule or two
+
+
+def test_two_models_share_the_device(backend):
+    # two resident models with their own caches and graphs, used alternately
+    cfgs = [dict(fmt=TQ2, n_layers=2, h=128, inter=256, nq=4, nkv=2, hd=32, vocab=32, max_seq=64, eps=1e-6, rope_theta=1e6),
+            dict(fmt=Q1, n_layers=3, h=256, inter=512, nq=4, nkv=4, hd=64, vocab=64, max_seq=64, eps=1e-6, rope_theta=1e4)]
+    ws = [synth.make_model(c, 10 + i) for i, c in enumerate(cfgs)]
+    gpus = [HipModel(backend, c, w) for c, w in zip(cfgs, ws)]
+    cpus = [oracle.OracleModel(c, w, kv_f16=True) for c, w in zip(cfgs, ws)]
+    try:
+        for pos in range(8):
+            for i in ((0, 1) if pos % 2 else (1, 0)):
+                r = synth.embedding_rows(20 + i, [pos], cfgs[i]["h"])[0] * 50.0
+                got, _ = gpus[i].forward(r, pos)
+                want = cpus[i].forward(r, pos)
+                assert np.max(np.abs(got[0] - want)) < 1e-3 * max(1.0, float(np.max(np.abs(want)))), (i, pos)
+        assert all(g.uses_graph() for g in gpus)
+    finally:
+        for g in gpus:
+            g.close()
