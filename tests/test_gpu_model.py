@@ -249,3 +249,32 @@ def test_full_size_shapes_match_oracle(backend, name, cfg):
         assert err < tol, (name, "prefill", err, tol)
     finally:
         gpu.close()
+
+
+def test_attention_slots_walk_several_chunks(backend):
+    """Many sequences leave few attention slots per sequence (here two), so that a slot walks several 128-position
+    chunks of the KV sequence with the next chunk's keys and values already requested: positions 600..602 span five
+    chunks, slot 0 takes chunks 0, 2, 4 and slot 1 chunks 1, 3."""
+    cfg = dict(fmt=TQ2, n_layers=2, h=512, inter=1024, nq=16, nkv=8, hd=64, vocab=512, max_seq=700, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 91)
+    B, n = 64, 600
+    gpu = HipModel(backend, cfg, w, batch=B)
+    ctx = [synth.embedding_rows(200 + s, [(5 * i + s) % 251 for i in range(n)], cfg["h"]) * 50.0 for s in (0, 1)]
+    cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in (0, 1)]
+    try:
+        for b in range(B):                       # even sequences share context 0, odd ones context 1
+            gpu.prefill(ctx[b % 2], seq=b, want_logits=False)
+        for s in (0, 1):
+            for i, r in enumerate(ctx[s]):
+                cpus[s].forward(r, i, want_logits=False)
+        for step in range(3):
+            rows = [synth.embedding_rows(300 + s, [step], cfg["h"])[0] * 50.0 for s in (0, 1)]
+            got, toks = gpu.forward(np.stack([rows[b % 2] for b in range(B)]), np.full(B, n + step, dtype=np.uint32))
+            for s in (0, 1):
+                want = cpus[s].forward(rows[s], n + step)
+                assert parity_violations(got[s], want, 1e-2) == 0, (step, s, float(np.max(np.abs(got[s] - want))))
+                for b in range(s, B, 2):        # every sequence with the same inputs gives the same result
+                    assert np.allclose(got[b], got[s], rtol=0, atol=1e-5), (step, b)
+        assert gpu.uses_graph()
+    finally:
+        gpu.close()
