@@ -278,3 +278,34 @@ def test_attention_slots_walk_several_chunks(backend):
         assert gpu.uses_graph()
     finally:
         gpu.close()
+
+
+@pytest.mark.parametrize("fmt", [TQ2, Q1])
+def test_wide_ffn_takes_four_row_tiles_per_workgroup(backend, fmt):
+    """An intermediate size of 8192 gives the gate || up product 1024 row tiles: the narrow GEMM then takes four per
+    workgroup (two gate tiles with their up tiles) and the prefill GEMM its widest SwiGLU tiling - the tilings the
+    8B-shape model runs with - on a model small enough for the oracle."""
+    cfg = dict(fmt=fmt, n_layers=1, h=256, inter=8192, nq=4, nkv=2, hd=64, vocab=128, max_seq=96, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 17 + fmt)
+    for B in (9, 20):
+        gpu = HipModel(backend, cfg, w, batch=B)
+        cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
+        try:
+            for step in range(2):
+                hidden = np.stack([synth.embedding_rows(80 + b, [step + b], cfg["h"])[0] * 50.0 for b in range(B)])
+                got, _ = gpu.forward(hidden, np.full(B, step, dtype=np.uint32))
+                for b in range(B):
+                    want = cpus[b].forward(hidden[b], step)
+                    assert parity_violations(got[b], want, 1e-2) == 0, (B, step, b)
+        finally:
+            gpu.close()
+    gpu = HipModel(backend, cfg, w)
+    cpu = oracle.OracleModel(cfg, w, kv_f16=True)
+    try:
+        rows = synth.embedding_rows(5, range(70), cfg["h"]) * 50.0
+        got, _ = gpu.prefill(rows)
+        for i, r in enumerate(rows):
+            want = cpu.forward(r, i, want_logits=i == len(rows) - 1)
+        assert parity_violations(got, want, 1e-2) == 0
+    finally:
+        gpu.close()
