@@ -66,6 +66,19 @@ def lib() -> C.CDLL:
             getattr(L, n).argtypes = [f32p, sz]
             getattr(L, n).restype = C.c_uint32
         L.oxb_state_new.restype = C.c_void_p
+        L.oxb_state_cache.restype = C.c_void_p
+        L.oxb_state_cache.argtypes = [C.c_void_p, C.c_int]
+        L.oxb_in_window.argtypes = [sz, sz, sz, sz]
+        L.oxb_attention_head_windowed.argtypes = [f32p, f32p, f32p, f32p, sz, sz, sz, sz]
+        L.oxb_attention_head_windowed.restype = None
+        for n in ("oxb_fp8_e4m3_encode", "oxb_fp8_e5m2_encode"):
+            getattr(L, n).argtypes = [C.c_float]
+            getattr(L, n).restype = C.c_uint8
+        for n in ("oxb_fp8_e4m3_decode", "oxb_fp8_e5m2_decode"):
+            getattr(L, n).argtypes = [C.c_uint8]
+            getattr(L, n).restype = C.c_float
+        L.oxb_kv_quantize_row.argtypes = [C.c_int, f32p, sz, u8p, C.POINTER(C.c_float)]
+        L.oxb_kv_dequantize_row.argtypes = [C.c_int, u8p, sz, C.c_float, f32p]
         L.oxb_oracle_set_threads.argtypes = [C.c_int]
         L.oxb_oracle_set_threads.restype = None
         L.oxb_sample.restype = C.c_uint32
@@ -219,6 +232,49 @@ def attention_head(q, keys, values, seq_len: int, head_dim: int) -> np.ndarray:
     return out
 
 
+def in_window(key: int, query: int, window: int, sinks: int) -> bool:
+    """is_in_window (crates/oxibonsai-model/src/layers/sliding_window.rs:173-189)."""
+    return bool(lib().oxb_in_window(key, query, window, sinks))
+
+
+def attention_head_windowed(q, keys, values, seq_len: int, head_dim: int, window: int, sinks: int) -> np.ndarray:
+    qv, kv, vv = _vec(q), _vec(keys).reshape(-1), _vec(values).reshape(-1)
+    out = np.empty(head_dim, dtype=np.float32)
+    lib().oxb_attention_head_windowed(_f32(qv), _f32(kv), _f32(vv), _f32(out), seq_len, head_dim, window, sinks)
+    return out
+
+
+KV_F32, KV_F16, KV_I8, KV_FP8_E4M3, KV_FP8_E5M2 = range(5)
+
+
+def fp8_encode(x, e5m2: bool = False) -> np.ndarray:
+    """fp8_e4m3_encode / fp8_e5m2_encode (crates/oxibonsai-core/src/quant_fp8.rs:47-160, 208-301), elementwise."""
+    a = _vec(x)
+    f = lib().oxb_fp8_e5m2_encode if e5m2 else lib().oxb_fp8_e4m3_encode
+    return np.array([f(float(v)) for v in a], dtype=np.uint8)
+
+
+def fp8_decode(codes, e5m2: bool = False) -> np.ndarray:
+    f = lib().oxb_fp8_e5m2_decode if e5m2 else lib().oxb_fp8_e4m3_decode
+    return np.array([f(int(c)) for c in np.asarray(codes, dtype=np.uint8).reshape(-1)], dtype=np.float32)
+
+
+def kv_quantize_row(mode: int, row):
+    """quantize_row_i8 / quantize_row_fp8 (crates/oxibonsai-model/src/kv_cache_quant.rs:46-62, 519-540) -> (codes, scale)."""
+    a = _vec(row)
+    codes = np.empty(a.size, dtype=np.uint8)
+    scale = C.c_float(0.0)
+    _check(lib().oxb_kv_quantize_row(mode, _f32(a), a.size, _u8(codes), C.byref(scale)))
+    return codes, np.float32(scale.value)
+
+
+def kv_dequantize_row(mode: int, codes, scale) -> np.ndarray:
+    c = np.ascontiguousarray(codes, dtype=np.uint8).reshape(-1)
+    out = np.empty(c.size, dtype=np.float32)
+    _check(lib().oxb_kv_dequantize_row(mode, _u8(c), c.size, float(scale), _f32(out)))
+    return out
+
+
 def argmax_last(v) -> int:
     a = _vec(v)
     return int(lib().oxb_argmax_last(_f32(a), a.size))
@@ -260,7 +316,8 @@ class _Model(C.Structure):
     _fields_ = [("fmt", C.c_int)] + [(n, C.c_size_t) for n in
                                       ("n_layers", "h", "inter", "nq", "nkv", "hd", "vocab", "max_seq")] + \
                [("eps", C.c_float), ("rope_theta", C.c_float), ("layers", C.POINTER(_Layer)),
-                ("final_norm", C.POINTER(C.c_float)), ("lm_head", _Linear), ("kv_f16", C.c_int)]
+                ("final_norm", C.POINTER(C.c_float)), ("lm_head", _Linear), ("kv_mode", C.c_int),
+                ("window", C.c_size_t), ("sinks", C.c_size_t)]
 
 
 class OracleModel:
@@ -272,9 +329,14 @@ class OracleModel:
     ``final_norm`` and ``lm_head``.
     """
 
-    def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False, dot_f64: bool = False):
+    def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False, dot_f64: bool = False, kv_mode: int = None,
+                 window: int = 0, sinks: int = 0):
         """dot_f64: every linear layer sums in double (not the reference's arithmetic; a yardstick for how far the
-        fp32 summation order moves the result at a given model size)."""
+        fp32 summation order moves the result at a given model size).  kv_mode: one of KV_* (default f32, or f16 with
+        kv_f16); window / sinks: sliding-window attention (window 0 = every earlier position is visible)."""
+        if kv_mode is None:
+            kv_mode = KV_F16 if kv_f16 else KV_F32
+        self.kv_mode = kv_mode
         self.cfg = cfg
         self._keep = []
         fmt = cfg["fmt"] + (2 if dot_f64 else 0)
@@ -299,7 +361,7 @@ class OracleModel:
         self._layers = layers
         self._model = _Model(fmt, cfg["n_layers"], h, inter, nq, nkv, hd, cfg["vocab"], cfg["max_seq"],
                              cfg["eps"], cfg["rope_theta"], layers, vec(weights["final_norm"]),
-                             lin(weights["lm_head"], cfg["vocab"], h), 1 if kv_f16 else 0)
+                             lin(weights["lm_head"], cfg["vocab"], h), kv_mode, window, sinks)
         self._state = lib().oxb_state_new(C.byref(self._model))
 
     def forward(self, hidden, pos: int, want_normed: bool = False, want_logits: bool = True):
@@ -309,6 +371,22 @@ class OracleModel:
         _check(lib().oxb_forward_ex(C.byref(self._model), self._state, _f32(hv), pos,
                                     _f32(logits) if want_logits else None, _f32(normed)))
         return (logits, normed) if want_normed else logits
+
+    def cache(self):
+        """K and V as attention reads them, [layer][kv_head][max_seq][hd] f32; for a quantised cache also the codes
+        (uint8, same shape) and the scales [layer][kv_head][max_seq]: (k, v, k_codes, v_codes, k_scale, v_scale)."""
+        c = self.cfg
+        shape = (c["n_layers"], c["nkv"], c["max_seq"], c["hd"])
+        n = int(np.prod(shape))
+        def view(which, ctype, count, dtype, shp):
+            ptr = lib().oxb_state_cache(self._state, which)
+            if not ptr:
+                return None
+            return np.ctypeslib.as_array(C.cast(ptr, C.POINTER(ctype)), shape=(count,)).view(dtype).reshape(shp).copy()
+
+        return (view(0, C.c_float, n, np.float32, shape), view(1, C.c_float, n, np.float32, shape),
+                view(2, C.c_uint8, n, np.uint8, shape), view(3, C.c_uint8, n, np.uint8, shape),
+                view(4, C.c_float, n // c["hd"], np.float32, shape[:3]), view(5, C.c_float, n // c["hd"], np.float32, shape[:3]))
 
     def reset(self):
         lib().oxb_state_free(self._state)

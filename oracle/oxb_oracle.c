@@ -4,6 +4,7 @@
  */
 #include "oxb_oracle.h"
 
+#include <float.h>
 #include <math.h>
 #include <stdlib.h>
 #ifdef _OPENMP
@@ -264,17 +265,30 @@ void oxb_rope_apply(const float* in, float* out, const float* c, const float* s,
     }
 }
 
+/* model/src/layers/sliding_window.rs:173-189 (is_in_window; attention_range :53-98 lists the same positions):
+ * the first `sinks` keys are always visible, the others while query - key < window - sinks. */
+int oxb_in_window(size_t key, size_t query, size_t window, size_t sinks) {
+    if (window == 0) return 0;
+    if (key < sinks) return 1;
+    if (query < key) return 0;
+    const size_t budget = window > sinks ? window - sinks : 0;
+    return query - key < budget;
+}
+
 /* model/src/layers/attention_fused.rs:166-226 (online softmax state) and :329-400
  * (contiguous K/V walk).  The reference's dot product is AVX dual-accumulator on
  * x86 (:139-164); the plain index-order sum is used here, the difference being a
- * summation order the tolerances cover. */
-void oxb_attention_head(const float* q, const float* keys, const float* values, float* out,
-                        size_t seq_len, size_t hd) {
+ * summation order the tolerances cover.  window > 0 restricts the keys of the query at
+ * position seq_len - 1 to those oxb_in_window admits (masked keys get weight 0, which
+ * is what apply_sliding_window_mask's -inf scores amount to, sliding_window.rs:109-135). */
+void oxb_attention_head_windowed(const float* q, const float* keys, const float* values, float* out,
+                                 size_t seq_len, size_t hd, size_t window, size_t sinks) {
     for (size_t d = 0; d < hd; d++) out[d] = 0.0f;
     if (seq_len == 0) return;
     float scale = 1.0f / sqrtf((float)hd);
     float max_val = -INFINITY, sum_exp = 0.0f;
     for (size_t t = 0; t < seq_len; t++) {
+        if (window && !oxb_in_window(t, seq_len - 1, window, sinks)) continue;
         const float* kt = keys + t * hd;
         float dot = 0.0f;
         for (size_t d = 0; d < hd; d++) dot += q[d] * kt[d];
@@ -294,6 +308,100 @@ void oxb_attention_head(const float* q, const float* keys, const float* values, 
         float inv = 1.0f / sum_exp;
         for (size_t d = 0; d < hd; d++) out[d] *= inv;
     }
+}
+
+void oxb_attention_head(const float* q, const float* keys, const float* values, float* out,
+                        size_t seq_len, size_t hd) {
+    oxb_attention_head_windowed(q, keys, values, out, seq_len, hd, 0, 0);
+}
+
+/* ------------------------------------------------------------------------- */
+/* Quantised KV rows.                                                         */
+/* FP8 codes: core/src/quant_fp8.rs:47-160 (E4M3FN: s eeee mmm, bias 7, no infinity, NaN = 0x7f, |x| >= 448
+ * saturates to 0x7e) and :208-301 (E5M2: s eeeee mm, bias 15, |x| > 57344 becomes infinity 0x7c, NaN = 0x7e);
+ * both round to nearest, ties to even, including into and inside the subnormal range.  One routine covers both:
+ * man_bits / bias / the code of the largest finite value / what lies beyond it. */
+static uint8_t fp8_encode(float x, int man_bits, int bias, float max_finite, int at_max_saturates,
+                          uint8_t code_max, uint8_t code_over, uint8_t code_nan) {
+    uint32_t bits;
+    memcpy(&bits, &x, 4);
+    const uint8_t sign = (uint8_t)((bits >> 31) << 7);
+    const uint32_t mag = bits & 0x7FFFFFFFu;
+    if (mag > 0x7F800000u) return code_nan;             /* NaN: canonical, positive */
+    if (mag == 0x7F800000u) return sign | code_over;
+    if (mag == 0) return sign;
+    float a;
+    memcpy(&a, &mag, 4);
+    if (at_max_saturates ? a >= max_finite : a > max_finite) return sign | (at_max_saturates ? code_max : code_over);
+    const int e = (int)(mag >> 23) - 127 + bias;        /* biased exponent in the target format */
+    uint32_t code;
+    if (e >= 1) {
+        const int shift = 23 - man_bits;
+        const uint32_t man = mag & 0x7FFFFFu, rem = man & ((1u << shift) - 1u), halfway = 1u << (shift - 1);
+        code = ((uint32_t)e << man_bits) | (man >> shift);
+        if (rem > halfway || (rem == halfway && (code & 1u))) code++;   /* a carry runs into the exponent field */
+        if (code > code_max) code = at_max_saturates ? code_max : code_over;
+    } else {
+        /* subnormal target: multiples of 2^(1 - bias - man_bits); the product is exact, rintf rounds to even,
+         * and 2^man_bits is the code of the smallest normal value */
+        code = (uint32_t)rintf(ldexpf(a, bias - 1 + man_bits));
+    }
+    return sign | (uint8_t)code;
+}
+
+static float fp8_decode(uint8_t b, int man_bits, int bias, int has_inf) {
+    const int exp_bits = 7 - man_bits;
+    const uint32_t e = (b >> man_bits) & ((1u << exp_bits) - 1u), m = b & ((1u << man_bits) - 1u);
+    const float sgn = (b & 0x80) ? -1.0f : 1.0f;
+    if (e == (1u << exp_bits) - 1u) {
+        if (has_inf) return m == 0 ? sgn * INFINITY : NAN;
+        if (m == (1u << man_bits) - 1u) return NAN;
+    }
+    if (e == 0) return sgn * ldexpf((float)m, 1 - bias - man_bits);
+    return sgn * ldexpf((float)((1u << man_bits) | m), (int)e - bias - man_bits);
+}
+
+uint8_t oxb_fp8_e4m3_encode(float x) { return fp8_encode(x, 3, 7, 448.0f, 1, 0x7e, 0x7e, 0x7f); }
+uint8_t oxb_fp8_e5m2_encode(float x) { return fp8_encode(x, 2, 15, 57344.0f, 0, 0x7b, 0x7c, 0x7e); }
+float oxb_fp8_e4m3_decode(uint8_t b) { return fp8_decode(b, 3, 7, 0); }
+float oxb_fp8_e5m2_decode(uint8_t b) { return fp8_decode(b, 2, 15, 1); }
+
+/* One row (one position of one kv head) -> codes + scale.
+ * INT8: model/src/kv_cache_quant.rs:46-62  scale = max(max|x| / 127, f32::EPSILON), q = round(x / scale) (half away
+ *       from zero) clamped to +-127.
+ * FP8:  model/src/kv_cache_quant.rs:519-540  scale = max(max|x| / FP8_MAX, f32::EPSILON), code = encode(x / scale).
+ * Dequantisation (:69-71, :545-556) is code * scale in f32. */
+int oxb_kv_quantize_row(int mode, const float* row, size_t n, uint8_t* codes, float* scale_out) {
+    if (mode != OXB_KV_I8 && mode != OXB_KV_FP8_E4M3 && mode != OXB_KV_FP8_E5M2) return OXB_ERR_DIMENSION_MISMATCH;
+    float max_abs = 0.0f;
+    for (size_t i = 0; i < n; i++) max_abs = fmaxf(max_abs, fabsf(row[i]));
+    const float top = mode == OXB_KV_I8 ? 127.0f : mode == OXB_KV_FP8_E4M3 ? 448.0f : 57344.0f;
+    float scale = max_abs / top;
+    if (!(scale >= FLT_EPSILON)) scale = FLT_EPSILON;
+    for (size_t i = 0; i < n; i++) {
+        const float t = row[i] / scale;
+        if (mode == OXB_KV_I8) {
+            float r = roundf(t);
+            r = r < -127.0f ? -127.0f : r > 127.0f ? 127.0f : r;
+            codes[i] = (uint8_t)(int8_t)r;
+        } else {
+            codes[i] = mode == OXB_KV_FP8_E4M3 ? oxb_fp8_e4m3_encode(t) : oxb_fp8_e5m2_encode(t);
+        }
+    }
+    *scale_out = scale;
+    return OXB_OK;
+}
+
+int oxb_kv_dequantize_row(int mode, const uint8_t* codes, size_t n, float scale, float* out) {
+    for (size_t i = 0; i < n; i++) {
+        switch (mode) {
+            case OXB_KV_I8: out[i] = (float)(int8_t)codes[i] * scale; break;
+            case OXB_KV_FP8_E4M3: out[i] = oxb_fp8_e4m3_decode(codes[i]) * scale; break;
+            case OXB_KV_FP8_E5M2: out[i] = oxb_fp8_e5m2_decode(codes[i]) * scale; break;
+            default: return OXB_ERR_DIMENSION_MISMATCH;
+        }
+    }
+    return OXB_OK;
 }
 
 /* runtime/src/sampling.rs:84-91,182-189: Iterator::max_by keeps the LAST maximum. */
@@ -401,7 +509,9 @@ uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top
 /* KV layout: model/src/kv_cache.rs:118-120  [layer][kv_head][pos][d].        */
 /* ------------------------------------------------------------------------- */
 struct oxb_state {
-    float *k_cache, *v_cache;     /* [L][nkv][max_seq][hd] */
+    float *k_cache, *v_cache;     /* [L][nkv][max_seq][hd], as attention reads them (after the cache's rounding) */
+    uint8_t *k_codes, *v_codes;   /* quantised caches only: codes [L][nkv][max_seq][hd], scales [L][nkv][max_seq] */
+    float *k_scale, *v_scale;
     float *cos_t, *sin_t;         /* [max_seq][hd/2] */
     float *hidden, *normed, *q, *k, *v, *qn, *kn, *qr, *kr, *attn, *proj, *gate, *up, *act, *down;
 };
@@ -449,6 +559,12 @@ oxb_state* oxb_state_new(const oxb_model* m) {
     size_t qd = m->nq * m->hd, kd = m->nkv * m->hd;
     s->k_cache = (float*)calloc(kv, 4);
     s->v_cache = (float*)calloc(kv, 4);
+    if (m->kv_mode >= OXB_KV_I8) {
+        s->k_codes = (uint8_t*)calloc(kv, 1);
+        s->v_codes = (uint8_t*)calloc(kv, 1);
+        s->k_scale = (float*)calloc(kv / m->hd, 4);
+        s->v_scale = (float*)calloc(kv / m->hd, 4);
+    }
     s->cos_t = (float*)malloc(m->max_seq * (m->hd / 2) * 4);
     s->sin_t = (float*)malloc(m->max_seq * (m->hd / 2) * 4);
     oxb_rope_table(s->cos_t, s->sin_t, m->hd, m->max_seq, m->rope_theta);
@@ -469,6 +585,7 @@ oxb_state* oxb_state_new(const oxb_model* m) {
 void oxb_state_free(oxb_state* s) {
     if (!s) return;
     free(s->k_cache); free(s->v_cache); free(s->cos_t); free(s->sin_t);
+    free(s->k_codes); free(s->v_codes); free(s->k_scale); free(s->v_scale);
     free(s->hidden); free(s->normed); free(s->q); free(s->qn); free(s->qr);
     free(s->k); free(s->kn); free(s->kr); free(s->v); free(s->attn); free(s->proj);
     free(s->gate); free(s->up); free(s->act); free(s->down);
@@ -500,9 +617,17 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
         }
         for (size_t hh = 0; hh < nkv; hh++) {                                     /* :209-213 */
             size_t off = ((L * nkv + hh) * m->max_seq + pos) * hd;
+            if (m->kv_mode >= OXB_KV_I8) { /* a quantised cache: attention reads back code * scale */
+                const size_t row = (L * nkv + hh) * m->max_seq + pos;
+                oxb_kv_quantize_row(m->kv_mode, s->kr + hh * hd, hd, s->k_codes + off, &s->k_scale[row]);
+                oxb_kv_quantize_row(m->kv_mode, s->v + hh * hd, hd, s->v_codes + off, &s->v_scale[row]);
+                oxb_kv_dequantize_row(m->kv_mode, s->k_codes + off, hd, s->k_scale[row], s->k_cache + off);
+                oxb_kv_dequantize_row(m->kv_mode, s->v_codes + off, hd, s->v_scale[row], s->v_cache + off);
+                continue;
+            }
             for (size_t d = 0; d < hd; d++) {
                 float kv = s->kr[hh * hd + d], vv = s->v[hh * hd + d];
-                if (m->kv_f16) { /* cuda_attn_kernels.rs:228-251 rounds to f16 on store */
+                if (m->kv_mode == OXB_KV_F16) { /* cuda_attn_kernels.rs:228-251 rounds to f16 on store */
                     kv = oxb_f16_to_f32(oxb_f32_to_f16(kv));
                     vv = oxb_f16_to_f32(oxb_f32_to_f16(vv));
                 }
@@ -513,8 +638,8 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
         for (size_t qh = 0; qh < nq; qh++) {                                      /* block/functions.rs:78-127 */
             size_t kvh = qh / group;
             size_t base = (L * nkv + kvh) * m->max_seq * hd;
-            oxb_attention_head(s->qr + qh * hd, s->k_cache + base, s->v_cache + base,
-                               s->attn + qh * hd, pos + 1, hd);
+            oxb_attention_head_windowed(s->qr + qh * hd, s->k_cache + base, s->v_cache + base,
+                                        s->attn + qh * hd, pos + 1, hd, m->window, m->sinks);
         }
         if ((rc = linear_fwd(m->fmt, &ly->o, s->attn, s->proj))) return rc;      /* :389-392 */
         for (size_t i = 0; i < h; i++) s->hidden[i] += s->proj[i];
@@ -529,6 +654,18 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
     if (normed_out) memcpy(normed_out, s->normed, h * 4);
     if (logits) return linear_fwd(m->fmt, &m->lm_head, s->normed, logits);       /* mod.rs:874-880 */
     return OXB_OK;
+}
+
+const void* oxb_state_cache(const oxb_state* s, int which) {
+    switch (which) {
+        case 0: return s->k_cache;
+        case 1: return s->v_cache;
+        case 2: return s->k_codes;
+        case 3: return s->v_codes;
+        case 4: return s->k_scale;
+        case 5: return s->v_scale;
+        default: return NULL;
+    }
 }
 
 int oxb_forward(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos, float* logits) {

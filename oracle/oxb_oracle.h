@@ -29,6 +29,11 @@
  *                      unpinned: the candidate order the reference's partial
  *                      selection leaves when top_p == 1 (implementation-defined)
  *                      and the last place of exp()
+ *   fp8 codes, kv rows the reference's encode / decode unit tests (0, -0, NaN, infinities, 448, 2^-9, 1000, ...),
+ *                      every byte's value and every representable value's code against torch's float8 types,
+ *                      round-to-nearest-even against a float64 search over the code table; INT8 rows against the
+ *                      reference's [127, -127, 0] test and a float64 numpy restatement
+ *   in_window          the reference's attention_range / is_in_window unit tests (positions listed there)
  */
 #ifndef OXB_ORACLE_H
 #define OXB_ORACLE_H
@@ -77,6 +82,20 @@ void  oxb_rope_table(float* cos_t, float* sin_t, size_t head_dim, size_t max_seq
 void  oxb_rope_apply(const float* in, float* out, const float* cos_row, const float* sin_row, size_t half_dim);
 void  oxb_attention_head(const float* q, const float* keys, const float* values, float* out,
                          size_t seq_len, size_t head_dim);
+/* Sliding window with attention sinks (model/src/layers/sliding_window.rs); window == 0 in the attention call: off. */
+int   oxb_in_window(size_t key, size_t query, size_t window, size_t sinks);
+void  oxb_attention_head_windowed(const float* q, const float* keys, const float* values, float* out,
+                                  size_t seq_len, size_t head_dim, size_t window, size_t sinks);
+
+/* How a KV cache keeps its rows. */
+enum { OXB_KV_F32 = 0, OXB_KV_F16 = 1, OXB_KV_I8 = 2, OXB_KV_FP8_E4M3 = 3, OXB_KV_FP8_E5M2 = 4 };
+uint8_t oxb_fp8_e4m3_encode(float x);
+uint8_t oxb_fp8_e5m2_encode(float x);
+float   oxb_fp8_e4m3_decode(uint8_t b);
+float   oxb_fp8_e5m2_decode(uint8_t b);
+/* One row of head_dim values -> codes (i8 as its byte, or FP8) and the row scale; and back (code * scale). */
+int oxb_kv_quantize_row(int mode, const float* row, size_t n, uint8_t* codes, float* scale_out);
+int oxb_kv_dequantize_row(int mode, const uint8_t* codes, size_t n, float scale, float* out);
 uint32_t oxb_argmax_last(const float* v, size_t n);   /* Sampler greedy: last max on ties */
 uint32_t oxb_argmax_first(const float* v, size_t n);  /* GPU argmax_f32: first max        */
 /* Sampler::sample (runtime/src/sampling.rs:84-177); see the definition for the candidate order it fixes. */
@@ -104,12 +123,17 @@ typedef struct {
     const oxb_layer* layers;
     const float* final_norm;  /* [h] */
     oxb_linear lm_head;       /* vocab x h */
-    int kv_f16;               /* 1: round K/V through f16 as the reference's GPU cache does */
+    int kv_mode;              /* OXB_KV_*: F16 rounds K/V through f16 as the reference's GPU cache does; I8 / FP8 store
+                                 codes + a scale per (position, kv head) as model/src/kv_cache_quant.rs does */
+    size_t window, sinks;     /* sliding-window attention; window == 0: every earlier position is visible */
 } oxb_model;
 
 typedef struct oxb_state oxb_state;   /* KV cache + scratch */
 oxb_state* oxb_state_new(const oxb_model* m);
 void       oxb_state_free(oxb_state* s);
+/* which: 0 / 1 K / V as attention reads them (f32 [L][nkv][max_seq][hd]); 2 / 3 their codes (u8, same shape) and
+ * 4 / 5 their scales (f32 [L][nkv][max_seq]) when the cache is quantised, else NULL. */
+const void* oxb_state_cache(const oxb_state* s, int which);
 /* One decode step: hidden[h] (embedding row) at position pos -> logits[vocab]. */
 int oxb_forward(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos, float* logits);
 /* Same but also returns the hidden state after the final norm (may be NULL). */

@@ -83,9 +83,10 @@ def test_argmax_tie_rules():
 
 
 # ---- whole-model decode against an independent float64 numpy forward -------------------------------
-def _f64_forward(cfg, w, hiddens):
+def _f64_forward(cfg, w, hiddens, kv_round=None, visible=None):
     """Textbook Qwen3 decode in float64 from the dequantised matrices (no oracle code involved except dequant,
-    which test_oracle.py pins bit for bit)."""
+    which test_oracle.py pins bit for bit).  kv_round(row) -> the row as a cache of limited precision returns it;
+    visible(key, query) -> whether the query's attention may look at the key."""
     from helpers import dense_f64
     fmt, h, hd, nq, nkv = cfg["fmt"], cfg["h"], cfg["hd"], cfg["nq"], cfg["nkv"]
     inter, half = cfg["inter"], cfg["hd"] // 2
@@ -112,13 +113,16 @@ def _f64_forward(cfg, w, hiddens):
             n = rms(x, lw["attn_norm"].astype(np.float64))
             q, k, v = mats[L]["q"] @ n, mats[L]["k"] @ n, mats[L]["v"] @ n
             for kh in range(nkv):
-                K[L][kh].append(rope(rms(k[kh * hd:(kh + 1) * hd], lw["k_norm"].astype(np.float64)), pos))
-                V[L][kh].append(v[kh * hd:(kh + 1) * hd])
+                kr, vr = rope(rms(k[kh * hd:(kh + 1) * hd], lw["k_norm"].astype(np.float64)), pos), v[kh * hd:(kh + 1) * hd]
+                K[L][kh].append(kv_round(kr) if kv_round else kr)
+                V[L][kh].append(kv_round(vr) if kv_round else vr)
             att = np.zeros(nq * hd)
             for qh in range(nq):
                 qv = rope(rms(q[qh * hd:(qh + 1) * hd], lw["q_norm"].astype(np.float64)), pos)
                 kh = qh // (nq // nkv)
                 sc = np.array(K[L][kh]) @ qv / np.sqrt(hd)
+                if visible:
+                    sc = np.where([visible(t, pos) for t in range(pos + 1)], sc, -np.inf)
                 p = np.exp(sc - sc.max())
                 att[qh * hd:(qh + 1) * hd] = (p / p.sum()) @ np.array(V[L][kh])
             x = x + mats[L]["o"] @ att
