@@ -140,6 +140,39 @@ int  oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t
                      float* logits_or_null, uint32_t* token_out_or_null);
 int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is replayed from a captured graph */
 
+/* ---- long-context options of the attention kernels (decode and prefill), modelled on what the reference's CPU
+ * library offers beside its plain cache:
+ *  - sliding window with attention sinks: SlidingWindowConfig { window_size, sink_tokens } and is_in_window
+ *    (crates/oxibonsai-model/src/layers/sliding_window.rs:11-43, 173-189): the query at position p sees key k iff
+ *    k < sink_tokens or p - k < window_size - sink_tokens.  window_size 0 switches the window off (every key up to
+ *    p is visible).  The cache keeps every row (no eviction); chunks outside the window are not read.
+ *  - quantised KV rows: one byte per value and one f32 scale per (position, kv head).  OXB_KV_DTYPE_I8 follows
+ *    QuantizedKvLayer / quantize_row_i8 (crates/oxibonsai-model/src/kv_cache_quant.rs:46-62, 98-195),
+ *    OXB_KV_DTYPE_FP8_E4M3 follows Fp8KvLayer / quantize_row_fp8 with Fp8KvFormat::E4M3 (:502-540) and
+ *    fp8_e4m3_encode (crates/oxibonsai-core/src/quant_fp8.rs:47-160); attention reads code * scale (:69-71, :545-556).
+ *    Device layout: codes [batch][layer][kv_head][max_seq][hd] (head-major, where the reference's layer keeps
+ *    [token][head][dim]), scales [batch][layer][kv_head][max_seq rounded up to 128].  Fp8KvFormat::E5M2 is not
+ *    offered: its row quantiser turns the row maximum into infinity whenever max / scale rounds above 57344
+ *    (quant_fp8.rs:229-231), about one row in five.
+ * oxb_hip_model_set_attention may be called at any time between steps; changing kv_dtype replaces the cache, so
+ * the sequences start again at position 0. */
+enum { OXB_KV_DTYPE_F16 = 0, OXB_KV_DTYPE_I8 = 1, OXB_KV_DTYPE_FP8_E4M3 = 2 };
+typedef struct {
+    int32_t kv_dtype;       /* OXB_KV_DTYPE_* */
+    uint32_t window_size;   /* 0 = no window */
+    uint32_t sink_tokens;
+} oxb_attention_options;
+int  oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt);
+int  oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt);
+/* Cache rows of positions pos .. pos + n_pos - 1 of one kv head as stored (QuantizedKvLayer::get_key / get_value
+ * without the dequantisation, kv_cache_quant.rs:204-228): k_rows / v_rows receive n_pos * hd elements (2-byte fp16
+ * or 1-byte codes), k_scales / v_scales n_pos row scales (1.0 for an fp16 cache).  Any pointer may be NULL. */
+int  oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t kv_head, uint32_t pos, uint32_t n_pos,
+                           void* k_rows, void* v_rows, float* k_scales, float* v_scales);
+/* quantize_row_i8 / quantize_row_fp8 on the device for n_rows rows of n values each (host buffers): the same
+ * routine the attention kernels store new rows with. */
+int  oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, uint32_t n, uint8_t* codes, float* scales);
+
 /* ---- the steps either side of the fused forward: checkpoint file -> device, token ids in, token ids out.
  * oxb_hip_gguf_info (no GPU needed) and oxb_hip_load_gguf read a GGUF file the way GgufFile::parse does
  * (crates/oxibonsai-core/src/gguf/reader.rs:11-80, header.rs, metadata.rs, tensor_info.rs) and assemble the model

@@ -68,6 +68,10 @@ def lib() -> C.CDLL:
         L.oxb_state_new.restype = C.c_void_p
         L.oxb_state_cache.restype = C.c_void_p
         L.oxb_state_cache.argtypes = [C.c_void_p, C.c_int]
+        L.oxb_state_load_rows.argtypes = [C.c_void_p, C.c_void_p, sz, sz, sz, sz, f32p, f32p]
+        L.oxb_state_load_rows.restype = None
+        L.oxb_state_freeze.argtypes = [C.c_void_p, C.c_int]
+        L.oxb_state_freeze.restype = None
         L.oxb_in_window.argtypes = [sz, sz, sz, sz]
         L.oxb_attention_head_windowed.argtypes = [f32p, f32p, f32p, f32p, sz, sz, sz, sz]
         L.oxb_attention_head_windowed.restype = None
@@ -387,6 +391,17 @@ class OracleModel:
         return (view(0, C.c_float, n, np.float32, shape), view(1, C.c_float, n, np.float32, shape),
                 view(2, C.c_uint8, n, np.uint8, shape), view(3, C.c_uint8, n, np.uint8, shape),
                 view(4, C.c_float, n // c["hd"], np.float32, shape[:3]), view(5, C.c_float, n // c["hd"], np.float32, shape[:3]))
+
+    def load_rows(self, layer: int, kv_head: int, pos0: int, k_rows, v_rows):
+        """Cache rows as attention shall read them (f32 [n][hd]), e.g. the rows another implementation stored."""
+        k = np.ascontiguousarray(k_rows, dtype=np.float32)
+        v = np.ascontiguousarray(v_rows, dtype=np.float32)
+        assert k.shape == v.shape and k.shape[1] == self.cfg["hd"] and pos0 + k.shape[0] <= self.cfg["max_seq"]
+        lib().oxb_state_load_rows(C.byref(self._model), self._state, layer, kv_head, pos0, k.shape[0], _f32(k), _f32(v))
+
+    def freeze(self, frozen: bool = True):
+        """While frozen a forward stores nothing: attention runs over the rows given by load_rows."""
+        lib().oxb_state_freeze(self._state, 1 if frozen else 0)
 
     def reset(self):
         lib().oxb_state_free(self._state)

@@ -510,6 +510,7 @@ uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top
 /* ------------------------------------------------------------------------- */
 struct oxb_state {
     float *k_cache, *v_cache;     /* [L][nkv][max_seq][hd], as attention reads them (after the cache's rounding) */
+    int frozen;                   /* 1: the cache rows are given (oxb_state_load_rows); a forward stores nothing */
     uint8_t *k_codes, *v_codes;   /* quantised caches only: codes [L][nkv][max_seq][hd], scales [L][nkv][max_seq] */
     float *k_scale, *v_scale;
     float *cos_t, *sin_t;         /* [max_seq][hd/2] */
@@ -615,7 +616,7 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
             oxb_rms_norm(s->k + hh * hd, ly->k_norm, s->kn + hh * hd, hd, m->eps);
             oxb_rope_apply(s->kn + hh * hd, s->kr + hh * hd, c, sn, half);
         }
-        for (size_t hh = 0; hh < nkv; hh++) {                                     /* :209-213 */
+        for (size_t hh = 0; hh < nkv && !s->frozen; hh++) {                       /* :209-213 */
             size_t off = ((L * nkv + hh) * m->max_seq + pos) * hd;
             if (m->kv_mode >= OXB_KV_I8) { /* a quantised cache: attention reads back code * scale */
                 const size_t row = (L * nkv + hh) * m->max_seq + pos;
@@ -655,6 +656,17 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
     if (logits) return linear_fwd(m->fmt, &m->lm_head, s->normed, logits);       /* mod.rs:874-880 */
     return OXB_OK;
 }
+
+/* Test aid: rows pos0 .. pos0 + n - 1 of one (layer, kv head) as attention shall read them, e.g. the rows another
+ * implementation stored; with oxb_state_freeze(s, 1) the forward then leaves the cache alone, so that its attention
+ * runs over exactly those rows (its own K and V of the current position included). */
+void oxb_state_load_rows(const oxb_model* m, oxb_state* s, size_t layer, size_t kv_head, size_t pos0, size_t n,
+                         const float* k_rows, const float* v_rows) {
+    const size_t off = ((layer * m->nkv + kv_head) * m->max_seq + pos0) * m->hd;
+    memcpy(s->k_cache + off, k_rows, n * m->hd * 4);
+    memcpy(s->v_cache + off, v_rows, n * m->hd * 4);
+}
+void oxb_state_freeze(oxb_state* s, int frozen) { s->frozen = frozen; }
 
 const void* oxb_state_cache(const oxb_state* s, int which) {
     switch (which) {

@@ -134,6 +134,11 @@ void       oxb_state_free(oxb_state* s);
 /* which: 0 / 1 K / V as attention reads them (f32 [L][nkv][max_seq][hd]); 2 / 3 their codes (u8, same shape) and
  * 4 / 5 their scales (f32 [L][nkv][max_seq]) when the cache is quantised, else NULL. */
 const void* oxb_state_cache(const oxb_state* s, int which);
+/* Test aid: give the cache rows of one (layer, kv head) as attention shall read them; while frozen, a forward stores
+ * nothing (its attention then runs over exactly the given rows). */
+void oxb_state_load_rows(const oxb_model* m, oxb_state* s, size_t layer, size_t kv_head, size_t pos0, size_t n,
+                         const float* k_rows, const float* v_rows);
+void oxb_state_freeze(oxb_state* s, int frozen);
 /* One decode step: hidden[h] (embedding row) at position pos -> logits[vocab]. */
 int oxb_forward(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos, float* logits);
 /* Same but also returns the hidden state after the final norm (may be NULL). */

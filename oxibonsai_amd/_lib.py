@@ -50,6 +50,11 @@ _SIGNATURES = {
     "oxb_hip_decode": ([C.c_uint64, f32p, u32p, f32p, u32p], C.c_int),
     "oxb_hip_prefill": ([C.c_uint64, C.c_uint32, f32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_model_uses_graph": ([C.c_uint64], C.c_int),
+    "oxb_hip_model_set_attention": ([C.c_uint64, C.c_void_p], C.c_int),
+    "oxb_hip_model_get_attention": ([C.c_uint64, C.c_void_p], C.c_int),
+    "oxb_hip_model_read_kv": ([C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p,
+                               f32p, f32p], C.c_int),
+    "oxb_hip_kv_quantize_rows": ([C.c_int, f32p, C.c_uint32, C.c_uint32, u8p, f32p], C.c_int),
     "oxb_hip_gguf_info": ([C.c_char_p, C.c_void_p], C.c_int),
     "oxb_hip_gguf_metadata": ([C.c_char_p, C.c_char_p, C.c_char_p, C.c_size_t], C.c_int),
     "oxb_hip_gguf_tensor": ([C.c_char_p, C.c_char_p, C.POINTER(C.c_int), u32p, u64p, u64p, u64p], C.c_int),

@@ -12,7 +12,9 @@ struct OxbQkParams {
     const uint32_t* pos;           // [batch], device; null: row b is token pos_base + b of sequence `seq` (prefill)
     uint32_t pos_base, seq;
     float* q_rope;                 // [batch][nq][hd]
-    __half *k_cache, *v_cache;     // [batch][n_layers][nkv][max_seq][hd]
+    void *k_cache, *v_cache;       // [batch][n_layers][nkv][max_seq][hd]: fp16, or one-byte codes (kv_mode)
+    float *k_scale, *v_scale;      // quantised cache: row scales [batch][n_layers][nkv][sc_stride]
+    uint32_t kv_mode, sc_stride;
     uint32_t nq, nkv, hd, max_seq, n_layers, layer;
     float eps;
 };
@@ -24,7 +26,10 @@ struct OxbAttnParams {
     const float *q_norm, *k_norm;        // [hd]
     const float *cos_t, *sin_t;          // [max_seq][hd/2]
     float eps;
-    __half *k_cache, *v_cache;           // [batch][n_layers][nkv][max_seq][hd]
+    void *k_cache, *v_cache;             // [batch][n_layers][nkv][max_seq][hd]: fp16, or one-byte codes (kv_mode)
+    float *k_scale, *v_scale;            // quantised cache: row scales [batch][n_layers][nkv][sc_stride]
+    uint32_t kv_mode, sc_stride;         // OXB_KV_* (kv_quant_device.h); sc_stride: a multiple of the chunk, >= max_seq
+    uint32_t window, sinks;              // sliding window with attention sinks; window 0 = off
     float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
@@ -37,6 +42,9 @@ hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w,
                                     float* d_normed_or_null, hipStream_t st);
 hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
                                    int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
+// n_rows rows of n values -> one-byte codes [n_rows][n] and a scale per row (kv_mode: OXB_KV_I8 or OXB_KV_FP8_E4M3).
+hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n_rows, uint32_t n, uint8_t* d_codes, float* d_scales,
+                                       hipStream_t st);
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);
 #define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers at a time
 #define OXB_ATTN_MAX_SPLITS 64        // slots the KV sequence is split over; slot s walks chunks s, s + n_splits, ...

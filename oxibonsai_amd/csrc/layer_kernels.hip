@@ -10,6 +10,9 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <type_traits>
+
+#include "kv_quant_device.h"
 #include "layer_kernels.h"
 #include "quant_device.h"
 
@@ -22,6 +25,17 @@ __device__ __forceinline__ float block_sum(float v, float* red) {  // two barrie
     __syncthreads();
     float s = 0.f;
     for (uint32_t i = 0; i < (blockDim.x >> 6); i++) s += red[i];
+    __syncthreads();
+    return s;
+}
+
+__device__ __forceinline__ float block_max(float v, float* red) {  // of non-negative values; same protocol
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    float s = 0.f;
+    for (uint32_t i = 0; i < (blockDim.x >> 6); i++) s = fmaxf(s, red[i]);
     __syncthreads();
     return s;
 }
@@ -123,14 +137,16 @@ __global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const 
 }
 
 // ---------------------------------------------------------------------------
-// Per-head QK-RMSNorm + half-split RoPE + FP16 KV store
+// Per-head QK-RMSNorm + half-split RoPE + KV store (fp16, or quantised rows: kv_quant_device.h)
 // (fused_qk_norm_rope + fused_kv_store, gpu_backend/cuda_attn_kernels.rs:160-251;
 //  CPU: block/types/forward.rs:179-213, rope pairs (d, d + hd/2) simd_float_ops.rs:240-253).
 // Grid (nq + nkv, batch); block = 128 threads.  Q heads go to q_rope (fp32), K heads (after RoPE)
 // and the raw V head go to the cache at position pos[b], rounded to f16 (round-to-nearest-even).
 // Cache layout: [seq][layer][kv_head][max_seq][hd], K and V in separate arrays.
 // ---------------------------------------------------------------------------
+template <int KVM>
 __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) {
+    constexpr bool QC = KVM != OXB_KV_F16;
     __shared__ float red[2];
     const uint32_t head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, hd = p.hd, half = hd >> 1;
     const bool is_q = head < p.nq;
@@ -145,24 +161,76 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
     const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
     const float* cs = p.cos_t + (size_t)pos * half;
     const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t cache_off = ((((size_t)seq * p.n_layers + p.layer) * p.nkv + hh) * p.max_seq + pos) * hd;
-    for (uint32_t d = tid; d < half; d += 128) {
-        const float lo = w[d] * in[d] * inv_rms, hi = w[d + half] * in[d + half] * inv_rms;
-        const float c = cs[d], s = sn[d];
-        const float o_lo = lo * c - hi * s, o_hi = lo * s + hi * c;
-        if (is_q) {
+    const size_t head_row = ((size_t)seq * p.n_layers + p.layer) * p.nkv + hh;
+    const size_t cache_off = (head_row * p.max_seq + pos) * hd;
+    // head_dim <= 256: a thread owns at most one rotation pair and two V values
+    float o_lo = 0.f, o_hi = 0.f;
+    if (tid < half) {
+        const float lo = w[tid] * in[tid] * inv_rms, hi = w[tid + half] * in[tid + half] * inv_rms;
+        const float c = cs[tid], s = sn[tid];
+        o_lo = lo * c - hi * s;
+        o_hi = lo * s + hi * c;
+    }
+    if (is_q) {
+        if (tid < half) {
             float* q = p.q_rope + ((size_t)b * p.nq + hh) * hd;
-            q[d] = o_lo;
-            q[d + half] = o_hi;
-        } else {
-            p.k_cache[cache_off + d] = __float2half_rn(o_lo);
-            p.k_cache[cache_off + d + half] = __float2half_rn(o_hi);
+            q[tid] = o_lo;
+            q[tid + half] = o_hi;
         }
+        return;
     }
-    if (!is_q) {
-        const float* v = p.qkv + (size_t)b * p.qkv_stride + (size_t)(p.nq + p.nkv + hh) * hd;
-        for (uint32_t d = tid; d < hd; d += 128) p.v_cache[cache_off + d] = __float2half_rn(v[d]);
+    const float* v = p.qkv + (size_t)b * p.qkv_stride + (size_t)(p.nq + p.nkv + hh) * hd;
+    const float v0 = tid < hd ? v[tid] : 0.f, v1 = tid + 128 < hd ? v[tid + 128] : 0.f;
+    if constexpr (QC) {
+        uint8_t* kc = reinterpret_cast<uint8_t*>(p.k_cache) + cache_off;
+        uint8_t* vc = reinterpret_cast<uint8_t*>(p.v_cache) + cache_off;
+        const float ks = kv_row_scale<KVM>(block_max(fmaxf(fabsf(o_lo), fabsf(o_hi)), red));
+        const float vs = kv_row_scale<KVM>(block_max(fmaxf(fabsf(v0), fabsf(v1)), red));
+        if (tid < half) {
+            kc[tid] = (uint8_t)kv_encode<KVM>(o_lo, ks);
+            kc[tid + half] = (uint8_t)kv_encode<KVM>(o_hi, ks);
+        }
+        if (tid < hd) vc[tid] = (uint8_t)kv_encode<KVM>(v0, vs);
+        if (tid + 128 < hd) vc[tid + 128] = (uint8_t)kv_encode<KVM>(v1, vs);
+        if (tid == 0) {
+            p.k_scale[head_row * p.sc_stride + pos] = ks;
+            p.v_scale[head_row * p.sc_stride + pos] = vs;
+        }
+    } else {
+        __half* kc = reinterpret_cast<__half*>(p.k_cache) + cache_off;
+        __half* vc = reinterpret_cast<__half*>(p.v_cache) + cache_off;
+        if (tid < half) {
+            kc[tid] = __float2half_rn(o_lo);
+            kc[tid + half] = __float2half_rn(o_hi);
+        }
+        if (tid < hd) vc[tid] = __float2half_rn(v0);
+        if (tid + 128 < hd) vc[tid + 128] = __float2half_rn(v1);
     }
+}
+
+// Rows of f32 values -> quantised cache rows (codes + scale), one wave per row; the arithmetic of the attention
+// kernels' own stores, exposed for callers that fill a cache themselves and for tests.
+template <int KVM>
+__global__ __launch_bounds__(64) void kv_quantize_rows_kernel(const float* __restrict__ x, uint32_t n, uint8_t* __restrict__ codes,
+                                                               float* __restrict__ scales) {
+    const float* row = x + (size_t)blockIdx.x * n;
+    float mx = 0.f;
+    for (uint32_t d = threadIdx.x; d < n; d += 64) mx = fmaxf(mx, fabsf(row[d]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    const float scale = kv_row_scale<KVM>(mx);
+    for (uint32_t d = threadIdx.x; d < n; d += 64) codes[(size_t)blockIdx.x * n + d] = (uint8_t)kv_encode<KVM>(row[d], scale);
+    if (threadIdx.x == 0) scales[blockIdx.x] = scale;
+}
+
+hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n_rows, uint32_t n, uint8_t* d_codes, float* d_scales,
+                                       hipStream_t st) {
+    if (n_rows == 0 || n == 0) return hipErrorInvalidValue;
+    if (kv_mode == OXB_KV_I8) hipLaunchKernelGGL(kv_quantize_rows_kernel<OXB_KV_I8>, dim3(n_rows), dim3(64), 0, st, d_x, n, d_codes, d_scales);
+    else if (kv_mode == OXB_KV_FP8_E4M3)
+        hipLaunchKernelGGL(kv_quantize_rows_kernel<OXB_KV_FP8_E4M3>, dim3(n_rows), dim3(64), 0, st, d_x, n, d_codes, d_scales);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
 }
 
 #define OXB_ATTN_CHUNK 128  // KV positions per chunk of the split-KV decode attention
@@ -187,9 +255,21 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
 // ---------------------------------------------------------------------------
 typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 
-template <int HD>
+// Options of the kernel (template KVM, fields window / sinks):
+//  * quantised cache rows (kv_quant_device.h): one byte per value plus an f32 scale per row.  The codes enter the
+//    matrix cores as exact fp16 numbers; the K row scale multiplies the score, the V row scale the probability
+//    (relative to a running largest scale `u`, so that the fp16 hi + lo pair of the product stays in range; the
+//    accumulator is kept in units of u and rescaled like the running maximum of the softmax).  A lane takes a
+//    contiguous quarter of a K row (hd / 4 bytes), so the Q operand follows that order.
+//  * sliding window with attention sinks (is_in_window, crates/oxibonsai-model/src/layers/sliding_window.rs:173-189):
+//    the first `sinks` keys stay visible, the others while pos - key < window - sinks; chunks without a visible key
+//    are not walked.  window == 0: every key up to pos is visible.
+template <int HD, int KVM>
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p) {
-    constexpr int KS = HD / 32, NS = HD / 16, VL = HD / 16, VSTR = HD + 8;
+    constexpr bool QC = KVM != OXB_KV_F16;
+    constexpr int KS = HD / 32, NS = HD / 16, VSTR = HD + 8;
+    constexpr int VPR = QC ? HD / 16 : HD / 8;  // 16-byte pieces per V row
+    constexpr int VL = 32 * VPR / 64;           // pieces of the wave's 32-row V block per lane
     // V block per wave; before the loop its start holds Q * scale of the group's heads, after it the merge buffers
     __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];
     static_assert(sizeof(vs_all) >= 16 * HD * sizeof(float), "Q must fit in the V slices");
@@ -201,32 +281,75 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     const uint32_t pos = p.pos[b], seq_len = pos + 1;
     const uint32_t n_chunks = (seq_len + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK;
     if (slot >= n_chunks) return;  // never read by the merge
+    // visible keys: [0, sink_n) and [lo, seq_len)
+    const uint32_t budget = p.window > p.sinks ? p.window - p.sinks : 0u;
+    const uint32_t lo = p.window ? (seq_len > budget ? seq_len - budget : 0u) : 0u;
+    const uint32_t sink_n = p.window ? min(p.sinks, seq_len) : 0u;
+    const uint32_t sink_chunks = (sink_n + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK, lo_chunk = lo / OXB_ATTN_CHUNK;
+    auto next_needed = [&](uint32_t c) {  // first chunk >= c of this slot's walk that holds a visible key
+        if (c >= sink_chunks && c < lo_chunk) c += (lo_chunk - c + p.n_splits - 1) / p.n_splits * p.n_splits;
+        return c;
+    };
+    const bool owner = (pos / OXB_ATTN_CHUNK) % p.n_splits == slot;  // this workgroup stores the new position
+    const uint32_t first = next_needed(slot);
+    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + slot) * (HD + OXB_ATTN_PART_PAD);
+    const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
+    if (first >= n_chunks && !owner) {  // nothing visible in this slot's chunks: an empty result for the merge
+        for (uint32_t i = tid; i < G * HD; i += 256) {
+            const uint32_t h = i / HD, d = i % HD;
+            part[h * part_head + d] = 0.f;
+            if (d == 0) {
+                part[h * part_head + HD] = -INFINITY;
+                part[h * part_head + HD + 1] = 0.f;
+            }
+        }
+        return;
+    }
     const float* qkv = p.qkv + (size_t)b * p.qkv_stride;
     const float* cs = p.cos_t + (size_t)pos * half;
     const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t base = (((size_t)b * p.n_layers + p.layer) * p.nkv + kvh) * p.max_seq * HD;
-    _Float16* Kc = reinterpret_cast<_Float16*>(p.k_cache) + base;
-    _Float16* Vc = reinterpret_cast<_Float16*>(p.v_cache) + base;
+    const size_t head_row = ((size_t)b * p.n_layers + p.layer) * p.nkv + kvh;
+    const size_t base = head_row * p.max_seq * HD;
+    typedef typename std::conditional<QC, uint8_t, _Float16>::type cache_t;
+    cache_t* Kc = reinterpret_cast<cache_t*>(p.k_cache) + base;
+    cache_t* Vc = reinterpret_cast<cache_t*>(p.v_cache) + base;
+    float* Ksc = QC ? p.k_scale + head_row * p.sc_stride : nullptr;  // one scale per position; the stride is a multiple of the chunk
+    float* Vsc = QC ? p.v_scale + head_row * p.sc_stride : nullptr;
 
     // K rows of the two 16-key tiles (A operands) and this lane's pieces of the 32-key V block of a chunk.
     // Rows past the last key repeat it; their scores are masked.
-    v8h_t k0r[KS], k1r[KS];
+    v8h_t k0r[QC ? 1 : KS], k1r[QC ? 1 : KS];
+    kvi2_t k0q[QC ? KS : 1], k1q[QC ? KS : 1];
+    float4 ksc0, ksc1, vsc0, vsc1;  // row scales of the lane's keys 4g .. 4g+3 and 16+4g .. 16+4g+3
     v4i vr[VL];
     auto load_k = [&](uint32_t chunk) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
         const uint32_t kr0 = min(key0 + qi, seq_len - 1), kr1 = min(key0 + 16 + qi, seq_len - 1);
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-            k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
-            k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
+            if constexpr (QC) {
+                k0q[s] = *reinterpret_cast<const kvi2_t*>(Kc + (size_t)kr0 * HD + (HD / 4) * g + 8 * s);
+                k1q[s] = *reinterpret_cast<const kvi2_t*>(Kc + (size_t)kr1 * HD + (HD / 4) * g + 8 * s);
+            } else {
+                k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
+                k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
+            }
+        }
+        if constexpr (QC) {
+            ksc0 = *reinterpret_cast<const float4*>(Ksc + key0 + 4 * g);
+            ksc1 = *reinterpret_cast<const float4*>(Ksc + key0 + 16 + 4 * g);
         }
     };
     auto load_v = [&](uint32_t chunk) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
 #pragma unroll
         for (int i = 0; i < VL; i++) {
-            const uint32_t id = i * 64 + lane, row = min(key0 + id / (HD / 8), seq_len - 1), col = id % (HD / 8);
-            vr[i] = *reinterpret_cast<const v4i*>(Vc + (size_t)row * HD + col * 8);
+            const uint32_t id = i * 64 + lane, row = min(key0 + id / VPR, seq_len - 1), col = id % VPR;
+            vr[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(Vc + (size_t)row * HD) + col * 16);
+        }
+        if constexpr (QC) {
+            vsc0 = *reinterpret_cast<const float4*>(Vsc + key0 + 4 * g);
+            vsc1 = *reinterpret_cast<const float4*>(Vsc + key0 + 16 + 4 * g);
         }
     };
 
@@ -239,13 +362,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
         const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
         for (uint32_t d = lane; d < half; d += 64) {
-            const float lo = p.q_norm[d] * in[d] * inv, hi = p.q_norm[d + half] * in[d + half] * inv;
-            qs[h * HD + d] = (lo * cs[d] - hi * sn[d]) * p.scale;
-            qs[h * HD + d + half] = (lo * sn[d] + hi * cs[d]) * p.scale;
+            const float lo_ = p.q_norm[d] * in[d] * inv, hi_ = p.q_norm[d + half] * in[d + half] * inv;
+            qs[h * HD + d] = (lo_ * cs[d] - hi_ * sn[d]) * p.scale;
+            qs[h * HD + d + half] = (lo_ * sn[d] + hi_ * cs[d]) * p.scale;
         }
     }
     // --- K and V of the new position, by the workgroup whose slot walks its chunk (wave 0 and wave 1) ---
-    if ((pos / OXB_ATTN_CHUNK) % p.n_splits == slot) {
+    if (owner) {
         if (wave == 0) {
             const float* in = qkv + (size_t)(p.nq + kvh) * HD;
             float ss = 0.f;
@@ -253,27 +376,80 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
             const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
-            for (uint32_t d = lane; d < half; d += 64) {
-                const float lo = p.k_norm[d] * in[d] * inv, hi = p.k_norm[d + half] * in[d + half] * inv;
-                Kc[(size_t)pos * HD + d] = (_Float16)(lo * cs[d] - hi * sn[d]);
-                Kc[(size_t)pos * HD + d + half] = (_Float16)(lo * sn[d] + hi * cs[d]);
+            constexpr int KI = (HD / 2 + 63) / 64;
+            float klo[KI], khi[KI], mx = 0.f;
+#pragma unroll
+            for (int it = 0; it < KI; it++) {
+                const uint32_t d = lane + 64 * it;
+                klo[it] = khi[it] = 0.f;
+                if (d < half) {
+                    const float lo_ = p.k_norm[d] * in[d] * inv, hi_ = p.k_norm[d + half] * in[d + half] * inv;
+                    klo[it] = lo_ * cs[d] - hi_ * sn[d];
+                    khi[it] = lo_ * sn[d] + hi_ * cs[d];
+                    mx = fmaxf(mx, fmaxf(fabsf(klo[it]), fabsf(khi[it])));
+                }
+            }
+            float scale = 1.f;
+            if constexpr (QC) {
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                scale = kv_row_scale<KVM>(mx);
+                if (lane == 0) Ksc[pos] = scale;
+            }
+#pragma unroll
+            for (int it = 0; it < KI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < half) {
+                    if constexpr (QC) {
+                        Kc[(size_t)pos * HD + d] = (uint8_t)kv_encode<KVM>(klo[it], scale);
+                        Kc[(size_t)pos * HD + d + half] = (uint8_t)kv_encode<KVM>(khi[it], scale);
+                    } else {
+                        Kc[(size_t)pos * HD + d] = (_Float16)klo[it];
+                        Kc[(size_t)pos * HD + d + half] = (_Float16)khi[it];
+                    }
+                }
             }
         } else if (wave == 1) {
             const float* in = qkv + (size_t)(p.nq + p.nkv + kvh) * HD;
-            for (uint32_t d = lane; d < HD; d += 64) Vc[(size_t)pos * HD + d] = (_Float16)in[d];
+            constexpr int VI = (HD + 63) / 64;
+            float vv[VI], mx = 0.f;
+#pragma unroll
+            for (int it = 0; it < VI; it++) {
+                const uint32_t d = lane + 64 * it;
+                vv[it] = d < HD ? in[d] : 0.f;
+                mx = fmaxf(mx, fabsf(vv[it]));
+            }
+            float scale = 1.f;
+            if constexpr (QC) {
+#pragma unroll
+                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                scale = kv_row_scale<KVM>(mx);
+                if (lane == 0) Vsc[pos] = scale;
+            }
+#pragma unroll
+            for (int it = 0; it < VI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < HD) {
+                    if constexpr (QC) Vc[(size_t)pos * HD + d] = (uint8_t)kv_encode<KVM>(vv[it], scale);
+                    else Vc[(size_t)pos * HD + d] = (_Float16)vv[it];
+                }
+            }
         }
     }
     __syncthreads();  // publishes qs and, within this workgroup, the new cache rows
-    load_k(slot);
-    load_v(slot);
+    if (first < n_chunks) {
+        load_k(first);
+        load_v(first);
+    }
 
-    // B operands: lane (head = qi, g) holds Q[head][32 s + 8 g .. + 7] as hi + lo
+    // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo
     v8h_t qh[KS], ql[KS];
 #pragma unroll
     for (int s = 0; s < KS; s++)
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float x = qi < G ? qs[qi * HD + 32 * s + 8 * g + e] : 0.f;
+            const uint32_t d = QC ? (HD / 4) * g + 8 * s + e : 32 * s + 8 * g + e;
+            const float x = qi < G ? qs[qi * HD + d] : 0.f;
             const _Float16 hi = (_Float16)x;
             qh[s][e] = hi;
             ql[s][e] = (_Float16)(x - (float)hi);
@@ -282,56 +458,114 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     v4f O[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
-    float m_run = -INFINITY, l_run = 0.f;
+    float m_run = -INFINITY, l_run = 0.f, u_run = QC ? 0.f : 1.f;  // u_run: the unit of O (largest V row scale so far)
     _Float16* vs = vs_all[wave];
 
-    for (uint32_t chunk = slot; chunk < n_chunks; chunk += p.n_splits) {
+    for (uint32_t chunk = first; chunk < n_chunks;) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
-        const bool more = chunk + p.n_splits < n_chunks;
+        const uint32_t nxt = next_needed(chunk + p.n_splits);
+        const bool more = nxt < n_chunks;
+        chunk = nxt;
         // stage the V block in the wave's LDS slice (the previous block's gathers were issued before: LDS runs in
         // order) and request the next chunk's
 #pragma unroll
         for (int i = 0; i < VL; i++) {
             const uint32_t id = i * 64 + lane;
-            *reinterpret_cast<v4i*>(vs + (id / (HD / 8)) * VSTR + (id % (HD / 8)) * 8) = vr[i];
+            if constexpr (QC) {
+                uint32_t d[8];
+                kv_dec4<KVM>((uint32_t)vr[i].x, d[0], d[1]);
+                kv_dec4<KVM>((uint32_t)vr[i].y, d[2], d[3]);
+                kv_dec4<KVM>((uint32_t)vr[i].z, d[4], d[5]);
+                kv_dec4<KVM>((uint32_t)vr[i].w, d[6], d[7]);
+                _Float16* dst = vs + (id / VPR) * VSTR + (id % VPR) * 16;
+                *reinterpret_cast<v4i*>(dst) = (v4i){(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
+                *reinterpret_cast<v4i*>(dst + 8) = (v4i){(int)d[4], (int)d[5], (int)d[6], (int)d[7]};
+            } else {
+                *reinterpret_cast<v4i*>(vs + (id / VPR) * VSTR + (id % VPR) * 8) = vr[i];
+            }
         }
-        if (more) load_v(chunk + p.n_splits);
+        const float4 vc0 = vsc0, vc1 = vsc1;
+        if (more) load_v(nxt);
         v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; s++) {
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], qh[s], s0, 0, 0, 0);
-            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k0r[s], ql[s], s0, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], qh[s], s1, 0, 0, 0);
-            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1r[s], ql[s], s1, 0, 0, 0);
+            v8h_t a0, a1;
+            if constexpr (QC) {
+                a0 = kv_dec8<KVM>(k0q[s]);
+                a1 = kv_dec8<KVM>(k1q[s]);
+            } else {
+                a0 = k0r[s];
+                a1 = k1r[s];
+            }
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qh[s], s0, 0, 0, 0);
+            s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ql[s], s0, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, qh[s], s1, 0, 0, 0);
+            s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ql[s], s1, 0, 0, 0);
         }
-        if (more) load_k(chunk + p.n_splits);
-        if (key0 >= seq_len) continue;  // this wave's quarter of the last chunk is empty
+        const float4 kc0 = ksc0, kc1 = ksc1;
+        if (more) load_k(nxt);
+        // this wave's quarter of the chunk holds no visible key (past the end, or outside the window)
+        if (!(key0 < sink_n || max(key0, lo) < min(key0 + 32, seq_len))) continue;
         // this lane: head qi, keys key0 + 4g + v and key0 + 16 + 4g + v
         float sv[8];
+        bool vis[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            sv[v] = key0 + 4 * g + v < seq_len ? s0[v] : -INFINITY;
-            sv[4 + v] = key0 + 16 + 4 * g + v < seq_len ? s1[v] : -INFINITY;
+            const uint32_t ka = key0 + 4 * g + v, kb = ka + 16;
+            vis[v] = ka < sink_n || (ka >= lo && ka < seq_len);
+            vis[4 + v] = kb < sink_n || (kb >= lo && kb < seq_len);
+        }
+        if constexpr (QC) {
+            const float ka[8] = {kc0.x, kc0.y, kc0.z, kc0.w, kc1.x, kc1.y, kc1.z, kc1.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                s0[v] *= ka[v];
+                s1[v] *= ka[4 + v];
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            sv[v] = vis[v] ? s0[v] : -INFINITY;
+            sv[4 + v] = vis[4 + v] ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);      // finite: key0 < seq_len
-        const float alpha = expf(m_run - m_new);   // 0 for the wave's first block
+        const float m_new = fmaxf(m_run, mx);      // finite: the block holds a visible key
+        float alpha = expf(m_run - m_new);         // 0 for the wave's first block
+        float vw[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // V row scales of the lane's keys in units of u_run
+        if constexpr (QC) {
+            const float va[8] = {vc0.x, vc0.y, vc0.z, vc0.w, vc1.x, vc1.y, vc1.z, vc1.w};
+            float vmx = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; e++) vmx = fmaxf(vmx, vis[e] ? va[e] : 0.f);
+            vmx = fmaxf(vmx, __shfl_xor(vmx, 16, 64));
+            vmx = fmaxf(vmx, __shfl_xor(vmx, 32, 64));
+            const float u_new = fmaxf(u_run, vmx);  // > 0: a visible row's scale is at least f32::EPSILON
+            const float inv_u = 1.0f / u_new;
+#pragma unroll
+            for (int e = 0; e < 8; e++) vw[e] = vis[e] ? va[e] * inv_u : 0.f;
+            l_run = l_run * alpha;                  // the sum is rescaled by the softmax factor only
+            alpha *= u_run * inv_u;                 // the accumulator also changes its unit
+            u_run = u_new;
+        } else {
+            l_run = l_run * alpha;
+        }
         float sum = 0.f;
         v8h_t ph, pl;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             const float pe = expf(sv[e] - m_new);
             sum += pe;
-            const _Float16 hi = (_Float16)pe;
+            const float pv = QC ? pe * vw[e] : pe;
+            const _Float16 hi = (_Float16)pv;
             ph[e] = hi;
-            pl[e] = (_Float16)(pe - (float)hi);
+            pl[e] = (_Float16)(pv - (float)hi);
         }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
-        l_run = l_run * alpha + sum;
+        l_run += sum;
         m_run = m_new;
         // O^T += V^T P^T; A operand gathered from the staged block
 #pragma unroll
@@ -353,21 +587,20 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     float* ml = mm + 4 * 16;
 #pragma unroll
     for (int sl = 0; sl < NS; sl++)
-        *reinterpret_cast<float4*>(&mo[(wave * 16 + qi) * HD + 16 * sl + 4 * g]) = make_float4(O[sl][0], O[sl][1], O[sl][2], O[sl][3]);
+        *reinterpret_cast<float4*>(&mo[(wave * 16 + qi) * HD + 16 * sl + 4 * g]) =
+            make_float4(O[sl][0] * u_run, O[sl][1] * u_run, O[sl][2] * u_run, O[sl][3] * u_run);
     if (g == 0) {
         mm[wave * 16 + qi] = m_run;
         ml[wave * 16 + qi] = l_run;
     }
     __syncthreads();
-    float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + slot) * (HD + OXB_ATTN_PART_PAD);
-    const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
     for (uint32_t i = tid; i < G * HD; i += 256) {
         const uint32_t h = i / HD, d = i % HD;
         const float M = fmaxf(fmaxf(mm[h], mm[16 + h]), fmaxf(mm[32 + h], mm[48 + h]));
         float o = 0.f, l = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float wgt = expf(mm[w * 16 + h] - M);  // 0 for a wave that saw no key
+            const float wgt = mm[w * 16 + h] == -INFINITY ? 0.f : expf(mm[w * 16 + h] - M);  // a wave that saw no key
             o = fmaf(mo[(w * 16 + h) * HD + d], wgt, o);
             l = fmaf(ml[w * 16 + h], wgt, l);
         }
@@ -557,20 +790,33 @@ hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, u
 }
 
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st) {
-    hipLaunchKernelGGL(qk_norm_rope_store_kernel, dim3(p.nq + p.nkv, batch), dim3(128), 0, st, p);
+    if (p.hd > 256 || p.kv_mode > OXB_KV_FP8_E4M3 || (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
+    const dim3 grid(p.nq + p.nkv, batch), block(128);
+    if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_I8>, grid, block, 0, st, p);
+    else if (p.kv_mode == OXB_KV_FP8_E4M3) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_FP8_E4M3>, grid, block, 0, st, p);
+    else hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_F16>, grid, block, 0, st, p);
     return hipGetLastError();
 }
 
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
     if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
-        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t)
+        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 ||
+        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale || p.sc_stride % OXB_ATTN_CHUNK || p.sc_stride < p.max_seq)))
         return hipErrorInvalidValue;
     const dim3 grid(p.n_splits, p.nkv, batch), block(256);
     switch (p.hd) {
-        case 32: hipLaunchKernelGGL(attn_decode_fused_kernel<32>, grid, block, 0, st, p); break;
-        case 64: hipLaunchKernelGGL(attn_decode_fused_kernel<64>, grid, block, 0, st, p); break;
-        case 128: hipLaunchKernelGGL(attn_decode_fused_kernel<128>, grid, block, 0, st, p); break;
-        case 256: hipLaunchKernelGGL(attn_decode_fused_kernel<256>, grid, block, 0, st, p); break;
+#define OXB_ATTN_CASE(HD_)                                                                                                  \
+    case HD_:                                                                                                            \
+        if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_I8>), grid, block, 0, st, p);  \
+        else if (p.kv_mode == OXB_KV_FP8_E4M3)                                                                           \
+            hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_FP8_E4M3>), grid, block, 0, st, p);                  \
+        else hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_F16>), grid, block, 0, st, p);                      \
+        break;
+        OXB_ATTN_CASE(32)
+        OXB_ATTN_CASE(64)
+        OXB_ATTN_CASE(128)
+        OXB_ATTN_CASE(256)
+#undef OXB_ATTN_CASE
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

@@ -23,6 +23,7 @@
 #include "gemm_kernels.h"
 #include "gguf.h"
 #include "gemv_kernels.h"
+#include "kv_quant_device.h"
 #include "layer_kernels.h"
 #include "prefill_kernels.h"
 #include "runtime_internal.h"
@@ -44,7 +45,11 @@ struct Model {
           *gu = nullptr, *logits = nullptr;
     uint32_t *tokens = nullptr, *pos = nullptr;
     void* argmax_ws = nullptr;
-    __half *k_cache = nullptr, *v_cache = nullptr;
+    // KV cache: fp16 values or one-byte codes [batch][n_layers][nkv][max_seq][hd]; a quantised cache also keeps one
+    // f32 scale per row, [batch][n_layers][nkv][sc_stride]
+    void *k_cache = nullptr, *v_cache = nullptr;
+    float *k_scale = nullptr, *v_scale = nullptr;
+    uint32_t kv_mode = OXB_KV_F16, sc_stride = 0, window = 0, sinks = 0;
     float *cos_t = nullptr, *sin_t = nullptr;
     void* xq_mem = nullptr;
     XqBuf xq;
@@ -84,6 +89,15 @@ static int dev_alloc(Model& m, void** p, size_t bytes) {
     return OXB_HIP_OK;
 }
 
+static void free_kv_cache(Model& m) {
+    void* bufs[4] = {m.k_cache, m.v_cache, m.k_scale, m.v_scale};
+    for (void* p : bufs)
+        if (p) (void)hipFree(p);
+    m.k_cache = m.v_cache = nullptr;
+    m.k_scale = m.v_scale = nullptr;
+    m.sc_stride = 0;
+}
+
 static void free_model(Model& m) {
     if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
     m.graph_exec = nullptr;
@@ -93,6 +107,7 @@ static void free_model(Model& m) {
     m.pf_allocs.clear();
     m.pf_cap = 0;
     m.gws.release();
+    free_kv_cache(m);
     m.tok_hist.release();
     m.tok_ids.release();
     m.sample_ws.release();
@@ -211,6 +226,12 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.eps = d.eps;
     ap.k_cache = m.k_cache;
     ap.v_cache = m.v_cache;
+    ap.k_scale = m.k_scale;
+    ap.v_scale = m.v_scale;
+    ap.kv_mode = m.kv_mode;
+    ap.sc_stride = m.sc_stride;
+    ap.window = m.window;
+    ap.sinks = m.sinks;
     ap.part = m.attn_part;
     ap.pos = m.pos;
     ap.nq = d.nq;
@@ -375,6 +396,10 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.q_rope = m.pf_q;
         qp.k_cache = m.k_cache;
         qp.v_cache = m.v_cache;
+        qp.k_scale = m.k_scale;
+        qp.v_scale = m.v_scale;
+        qp.kv_mode = m.kv_mode;
+        qp.sc_stride = m.sc_stride;
         qp.nq = d.nq;
         qp.nkv = d.nkv;
         qp.hd = d.hd;
@@ -384,10 +409,17 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.eps = d.eps;
         OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, M, st), "kernel launch failed: qk_norm_rope_store");
         OxbPrefillAttnParams ap;
-        const size_t layer_off = (((size_t)seq * d.n_layers + L) * d.nkv) * (size_t)d.max_seq * d.hd;
+        const size_t layer_row = ((size_t)seq * d.n_layers + L) * d.nkv;
+        const size_t layer_off = layer_row * (size_t)d.max_seq * d.hd * (m.kv_mode == OXB_KV_F16 ? 2 : 1);  // bytes
         ap.q = m.pf_q;
-        ap.k_cache = m.k_cache + layer_off;
-        ap.v_cache = m.v_cache + layer_off;
+        ap.k_cache = (const uint8_t*)m.k_cache + layer_off;
+        ap.v_cache = (const uint8_t*)m.v_cache + layer_off;
+        ap.k_scale = m.k_scale ? m.k_scale + layer_row * m.sc_stride : nullptr;
+        ap.v_scale = m.v_scale ? m.v_scale + layer_row * m.sc_stride : nullptr;
+        ap.kv_mode = m.kv_mode;
+        ap.sc_stride = m.sc_stride;
+        ap.window = m.window;
+        ap.sinks = m.sinks;
         ap.out = m.pf_attn;
         ap.M = M;
         ap.pos_start = pos_start;
@@ -461,6 +493,33 @@ int oxb_hip_free_f32(uint64_t id) {
     return OXB_HIP_OK;
 }
 
+// (Re)allocates the KV cache in the given storage form.  Row scales start at 0 so that a row never written reads
+// as zeros; the scale stride is a whole number of attention chunks, which keeps the kernels' 16-byte scale loads
+// inside the row and aligned.
+static int alloc_kv_cache(Model& m, uint32_t kv_mode) {
+    const oxb_model_desc& d = m.d;
+    const size_t rows = (size_t)d.batch * d.n_layers * d.nkv;
+    const size_t bytes = rows * d.max_seq * d.hd * (kv_mode == OXB_KV_F16 ? 2 : 1);
+    free_kv_cache(m);
+    auto grab = [&](void** p, size_t n) -> int {
+        if (hipMalloc(p, n ? n : 16) == hipSuccess) return OXB_HIP_OK;
+        *p = nullptr;
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes of KV cache on device %d", n, g_rt.device);
+    };
+    OXB_TRY(grab(&m.k_cache, bytes));
+    OXB_TRY(grab(&m.v_cache, bytes));
+    if (kv_mode != OXB_KV_F16) {
+        m.sc_stride = (d.max_seq + OXB_ATTN_CHUNK_POSITIONS - 1) / OXB_ATTN_CHUNK_POSITIONS * OXB_ATTN_CHUNK_POSITIONS;
+        const size_t sb = rows * m.sc_stride * sizeof(float);
+        OXB_TRY(grab((void**)&m.k_scale, sb));
+        OXB_TRY(grab((void**)&m.v_scale, sb));
+        OXB_TRY_HIP(hipMemset(m.k_scale, 0, sb), "scale clear");
+        OXB_TRY_HIP(hipMemset(m.v_scale, 0, sb), "scale clear");
+    }
+    m.kv_mode = kv_mode;
+    return OXB_HIP_OK;
+}
+
 int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!desc || !model || !desc->layers) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
@@ -508,7 +567,6 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     if (m.n_splits > want) m.n_splits = want;
     if (m.n_splits > OXB_ATTN_MAX_SPLITS) m.n_splits = OXB_ATTN_MAX_SPLITS;
     const size_t B = d.batch;
-    const size_t kv_elems = B * d.n_layers * d.nkv * (size_t)d.max_seq * d.hd;
     uint32_t kmax = d.h > d.inter ? d.h : d.inter;
     if (qd > kmax) kmax = qd;
     const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
@@ -516,8 +574,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = dev_alloc(m, (void**)&m.k_cache, kv_elems * 2)) ||
-        (rc = dev_alloc(m, (void**)&m.v_cache, kv_elems * 2)) ||
+        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + OXB_XEXP_BYTES))) {
@@ -589,6 +646,94 @@ int oxb_hip_model_destroy(uint64_t model) {
     for (uint64_t id : mats) (void)oxb_hip_free_weight(id);
     for (uint64_t id : vecs) (void)oxb_hip_free_f32(id);
     return OXB_HIP_OK;
+}
+
+int oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (!opt) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
+    if (opt->kv_dtype != OXB_KV_DTYPE_F16 && opt->kv_dtype != OXB_KV_DTYPE_I8 && opt->kv_dtype != OXB_KV_DTYPE_FP8_E4M3)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown KV cache type %d", opt->kv_dtype);
+    OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
+    // the captured decode step holds the cache pointers and the options: it is captured again on the next step
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    m->graph_exec = nullptr;
+    if ((uint32_t)opt->kv_dtype != m->kv_mode) {
+        const int rc = alloc_kv_cache(*m, (uint32_t)opt->kv_dtype);
+        if (rc) {  // leave the model usable: back to the fp16 cache
+            if (alloc_kv_cache(*m, OXB_KV_F16)) m->k_cache = m->v_cache = nullptr;
+            return rc;
+        }
+    }
+    m->window = opt->window_size;
+    m->sinks = opt->sink_tokens;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (!opt) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
+    opt->kv_dtype = (int32_t)m->kv_mode;
+    opt->window_size = m->window;
+    opt->sink_tokens = m->sinks;
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t kv_head, uint32_t pos, uint32_t n_pos,
+                          void* k_rows, void* v_rows, float* k_scales, float* v_scales) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    const oxb_model_desc& d = m->d;
+    if (seq >= d.batch || layer >= d.n_layers || kv_head >= d.nkv || (uint64_t)pos + n_pos > d.max_seq)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: cache rows (sequence %u, layer %u, head %u, positions %u..%llu) out of range",
+                    seq, layer, kv_head, pos, (unsigned long long)pos + n_pos);
+    if (!m->k_cache) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: the model has no KV cache");
+    if (n_pos == 0) return OXB_HIP_OK;
+    OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
+    const size_t esz = m->kv_mode == OXB_KV_F16 ? 2 : 1;
+    const size_t head_row = ((size_t)seq * d.n_layers + layer) * d.nkv + kv_head;
+    const size_t off = (head_row * d.max_seq + pos) * d.hd * esz, bytes = (size_t)n_pos * d.hd * esz;
+    if (k_rows) OXB_TRY_HIP(hipMemcpy(k_rows, (const uint8_t*)m->k_cache + off, bytes, hipMemcpyDeviceToHost), "cache read");
+    if (v_rows) OXB_TRY_HIP(hipMemcpy(v_rows, (const uint8_t*)m->v_cache + off, bytes, hipMemcpyDeviceToHost), "cache read");
+    if (m->kv_mode != OXB_KV_F16) {
+        const size_t so = head_row * m->sc_stride + pos;
+        if (k_scales) OXB_TRY_HIP(hipMemcpy(k_scales, m->k_scale + so, (size_t)n_pos * 4, hipMemcpyDeviceToHost), "scale read");
+        if (v_scales) OXB_TRY_HIP(hipMemcpy(v_scales, m->v_scale + so, (size_t)n_pos * 4, hipMemcpyDeviceToHost), "scale read");
+    } else {
+        for (uint32_t i = 0; i < n_pos; i++) {
+            if (k_scales) k_scales[i] = 1.0f;
+            if (v_scales) v_scales[i] = 1.0f;
+        }
+    }
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, uint32_t n, uint8_t* codes, float* scales) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!rows || !codes || !scales) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
+    if (kv_dtype != OXB_KV_DTYPE_I8 && kv_dtype != OXB_KV_DTYPE_FP8_E4M3)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: KV cache type %d has no quantised rows", kv_dtype);
+    if (n_rows == 0 || n == 0) return OXB_HIP_OK;
+    OXB_TRY(ensure_init());
+    DevBuf x, c, sc;
+    int rc = OXB_HIP_OK;
+    const size_t cnt = (size_t)n_rows * n;
+    if (!(rc = x.ensure(cnt * 4)) && !(rc = c.ensure(cnt)) && !(rc = sc.ensure((size_t)n_rows * 4))) {
+        hipError_t e = hipMemcpyAsync(x.ptr, rows, cnt * 4, hipMemcpyHostToDevice, g_rt.stream);
+        if (e == hipSuccess) e = oxb_launch_kv_quantize_rows(kv_dtype, (const float*)x.ptr, n_rows, n, (uint8_t*)c.ptr, (float*)sc.ptr, g_rt.stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(codes, c.ptr, cnt, hipMemcpyDeviceToHost, g_rt.stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(scales, sc.ptr, (size_t)n_rows * 4, hipMemcpyDeviceToHost, g_rt.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(g_rt.stream);
+        if (e != hipSuccess) rc = hip_fail(e, "kv row quantisation");
+    }
+    x.release();
+    c.release();
+    sc.release();
+    return rc;
 }
 
 int oxb_hip_model_reset(uint64_t model) {

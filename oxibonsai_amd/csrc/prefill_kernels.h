@@ -6,7 +6,10 @@
 
 struct OxbPrefillAttnParams {
     const float* q;                   // [M][nq][hd], after QK-norm and RoPE
-    const __half *k_cache, *v_cache;  // this sequence's, this layer's cache: [nkv][max_seq][hd]
+    const void *k_cache, *v_cache;    // this sequence's, this layer's cache: [nkv][max_seq][hd], fp16 or one-byte codes
+    const float *k_scale, *v_scale;   // quantised cache: this sequence's, this layer's row scales [nkv][sc_stride]
+    uint32_t kv_mode, sc_stride;      // OXB_KV_* (kv_quant_device.h)
+    uint32_t window, sinks;           // sliding window with attention sinks; window 0 = off
     float* out;                       // [M][nq * hd]
     uint32_t M, pos_start;            // query t sits at position pos_start + t and sees keys 0 .. pos_start + t
     uint32_t nq, nkv, hd, max_seq;

@@ -1,4 +1,4 @@
-// prefill_kernels.hip — causal attention of the prefill pipeline over the FP16 KV cache on the matrix cores
+// prefill_kernels.hip — causal attention of the prefill pipeline over the KV cache (fp16 or quantised rows) on the matrix cores
 // (the row-wise RMSNorm of the pipeline lives in the GEMM's activation packer, SwiGLU in the gate || up GEMM's
 // epilogue, gemm_kernels.hip).
 //
@@ -9,7 +9,10 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "device_utils.h"
+#include "kv_quant_device.h"
 #include "prefill_kernels.h"
 
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -34,14 +37,21 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // written to the other buffer before the barrier that ends the block.  Waves of an earlier query tile see the
 // last block(s) fully masked.
 // ---------------------------------------------------------------------------
-template <int HD>
+// Options as in the decode attention: quantised cache rows (template KVM; the codes are widened to exact fp16
+// numbers on their way into LDS, V already multiplied by its row scale there, the K row scale multiplies the
+// score) and a sliding window with attention sinks (key visible to the query at qpos iff key < sinks or
+// qpos - key < window - sinks; blocks no query of the workgroup can see are skipped).
+template <int HD, int KVM>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams p, uint32_t hpw) {
+    constexpr bool QC = KVM != OXB_KV_F16;
     constexpr int KS = HD / 32, NS = HD / 16;
     constexpr int STR = HD + 8;                      // LDS row stride in fp16 (16 bytes of padding: conflict-free rows)
-    constexpr int PIECES = 32 * HD / 8;              // 16-byte pieces of a 32-key block
+    constexpr int PPR = QC ? HD / 16 : HD / 8;       // 16-byte pieces per cache row
+    constexpr int PIECES = 32 * PPR;                 // pieces of a 32-key block
     constexpr int PP = (PIECES + 255) / 256;         // pieces per thread
     __shared__ __attribute__((aligned(16))) _Float16 ks[2][32 * STR];
     __shared__ __attribute__((aligned(16))) _Float16 vs[2][32 * STR];
+    __shared__ __attribute__((aligned(16))) float kscale[2][32];                // K row scales of the block (quantised cache)
     const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t n_qt = (p.M + 15u) / 16u, hq = p.nq / hpw, tpw = 4u / hpw, n_tg = (n_qt + tpw - 1) / tpw;
@@ -54,8 +64,21 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
     const uint32_t t_q = min(qt * 16 + qi, p.M - 1);                      // rows past M repeat the last one and are not stored
     const uint32_t qpos = p.pos_start + t_q;
     const uint32_t kv_len = p.pos_start + min((tg * tpw + tpw - 1) * 16 + 15, p.M - 1) + 1;  // keys the workgroup's last query sees
-    const _Float16* K = reinterpret_cast<const _Float16*>(p.k_cache) + (size_t)kvh * p.max_seq * HD;
-    const _Float16* V = reinterpret_cast<const _Float16*>(p.v_cache) + (size_t)kvh * p.max_seq * HD;
+    typedef typename std::conditional<QC, uint8_t, _Float16>::type cache_t;
+    const cache_t* K = reinterpret_cast<const cache_t*>(p.k_cache) + (size_t)kvh * p.max_seq * HD;
+    const cache_t* V = reinterpret_cast<const cache_t*>(p.v_cache) + (size_t)kvh * p.max_seq * HD;
+    const float* Ksc = QC ? p.k_scale + (size_t)kvh * p.sc_stride : nullptr;
+    const float* Vsc = QC ? p.v_scale + (size_t)kvh * p.sc_stride : nullptr;
+    // sliding window: this query sees [0, sinks) and (qpos - budget, qpos]; the workgroup's earliest query sits at
+    // q_first, so no query of it sees a key in [sinks, q_first + 1 - budget): whole 32-key blocks in there are skipped
+    const uint32_t budget = p.window > p.sinks ? p.window - p.sinks : 0u;
+    const uint32_t q_first = p.pos_start + tg * tpw * 16;
+    const uint32_t skip_from = p.window ? (p.sinks + 31u) & ~31u : 0u;
+    const uint32_t skip_to = p.window && q_first + 1 > budget ? (q_first + 1 - budget) & ~31u : 0u;
+    auto next_block = [&](uint32_t key0) {  // the block after key0 that some query may see
+        key0 += 32;
+        return key0 >= skip_from && key0 < skip_to ? skip_to : key0;
+    };
 
     v8h qh[KS], ql[KS];
     {
@@ -78,37 +101,67 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
 
-    // this thread's pieces of a block: piece id = i * 256 + tid -> row id / (HD / 8), 16-byte column id % (HD / 8);
+    // this thread's pieces of a block: piece id = i * 256 + tid -> row id / PPR, 16-byte column id % PPR;
     // rows past the last key repeat it (their scores are masked, their probabilities 0)
     v4i kreg[PP], vreg[PP];
+    float vsreg[PP], ksreg = 0.f;  // quantised cache: the V row scale of each piece, one K row scale (threads 0..31)
     auto fetch = [&](uint32_t key0) {
 #pragma unroll
         for (int i = 0; i < PP; i++) {
             const uint32_t id = i * 256 + tid;
             if (PIECES % 256 == 0 || id < (uint32_t)PIECES) {
-                const uint32_t row = min(key0 + id / (HD / 8), kv_len - 1), col = id % (HD / 8);
-                kreg[i] = *reinterpret_cast<const v4i*>(K + (size_t)row * HD + col * 8);
-                vreg[i] = *reinterpret_cast<const v4i*>(V + (size_t)row * HD + col * 8);
+                const uint32_t row = min(key0 + id / PPR, kv_len - 1), col = id % PPR;
+                kreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(K + (size_t)row * HD) + col * 16);
+                vreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(V + (size_t)row * HD) + col * 16);
+                if constexpr (QC) vsreg[i] = Vsc[row];
             }
         }
+        if constexpr (QC)
+            if (tid < 32) ksreg = Ksc[min(key0 + tid, kv_len - 1)];
     };
     auto stash = [&](int buf) {
 #pragma unroll
         for (int i = 0; i < PP; i++) {
             const uint32_t id = i * 256 + tid;
             if (PIECES % 256 == 0 || id < (uint32_t)PIECES) {
-                *reinterpret_cast<v4i*>(&ks[buf][(id / (HD / 8)) * STR + (id % (HD / 8)) * 8]) = kreg[i];
-                *reinterpret_cast<v4i*>(&vs[buf][(id / (HD / 8)) * STR + (id % (HD / 8)) * 8]) = vreg[i];
+                if constexpr (QC) {
+                    uint32_t kd[8], vd[8];
+                    kv_dec4<KVM>((uint32_t)kreg[i].x, kd[0], kd[1]);
+                    kv_dec4<KVM>((uint32_t)kreg[i].y, kd[2], kd[3]);
+                    kv_dec4<KVM>((uint32_t)kreg[i].z, kd[4], kd[5]);
+                    kv_dec4<KVM>((uint32_t)kreg[i].w, kd[6], kd[7]);
+                    kv_dec4<KVM>((uint32_t)vreg[i].x, vd[0], vd[1]);
+                    kv_dec4<KVM>((uint32_t)vreg[i].y, vd[2], vd[3]);
+                    kv_dec4<KVM>((uint32_t)vreg[i].z, vd[4], vd[5]);
+                    kv_dec4<KVM>((uint32_t)vreg[i].w, vd[6], vd[7]);
+                    // V leaves for LDS as code * scale in fp16 (the probabilities it meets are fp16 as well)
+                    const _Float16 sc = (_Float16)vsreg[i];
+                    const kvh2_t sc2 = {sc, sc};
+#pragma unroll
+                    for (int e = 0; e < 8; e++) vd[e] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(kvh2_t, vd[e]) * sc2);
+                    _Float16* kd_ = &ks[buf][(id / PPR) * STR + (id % PPR) * 16];
+                    _Float16* vd_ = &vs[buf][(id / PPR) * STR + (id % PPR) * 16];
+                    *reinterpret_cast<v4i*>(kd_) = (v4i){(int)kd[0], (int)kd[1], (int)kd[2], (int)kd[3]};
+                    *reinterpret_cast<v4i*>(kd_ + 8) = (v4i){(int)kd[4], (int)kd[5], (int)kd[6], (int)kd[7]};
+                    *reinterpret_cast<v4i*>(vd_) = (v4i){(int)vd[0], (int)vd[1], (int)vd[2], (int)vd[3]};
+                    *reinterpret_cast<v4i*>(vd_ + 8) = (v4i){(int)vd[4], (int)vd[5], (int)vd[6], (int)vd[7]};
+                } else {
+                    *reinterpret_cast<v4i*>(&ks[buf][(id / PPR) * STR + (id % PPR) * 8]) = kreg[i];
+                    *reinterpret_cast<v4i*>(&vs[buf][(id / PPR) * STR + (id % PPR) * 8]) = vreg[i];
+                }
             }
         }
+        if constexpr (QC)
+            if (tid < 32) kscale[buf][tid] = ksreg;
     };
     fetch(0);
     stash(0);
-    if (32 < kv_len) fetch(32);
+    if (next_block(0) < kv_len) fetch(next_block(0));
     __syncthreads();
 
     int buf = 0;
-    for (uint32_t key0 = 0; key0 < kv_len; key0 += 32) {
+    for (uint32_t key0 = 0; key0 < kv_len;) {
+        const uint32_t key1 = next_block(key0), key2 = next_block(key1);
         const _Float16* kb = ks[buf];
         const _Float16* vb = vs[buf];
         v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
@@ -121,23 +174,34 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, qh[s], s1, 0, 0, 0);
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(k1, ql[s], s1, 0, 0, 0);
         }
+        if constexpr (QC) {
+            const float4 a = *reinterpret_cast<const float4*>(&kscale[buf][4 * g]), b = *reinterpret_cast<const float4*>(&kscale[buf][16 + 4 * g]);
+            s0[0] *= a.x, s0[1] *= a.y, s0[2] *= a.z, s0[3] *= a.w;
+            s1[0] *= b.x, s1[1] *= b.y, s1[2] *= b.z, s1[3] *= b.w;
+        }
         float sv[8];
         float mx = -INFINITY;
 #pragma unroll
         for (int v = 0; v < 4; v++) {
-            sv[v] = key0 + 4 * g + v <= qpos ? s0[v] : -INFINITY;
-            sv[4 + v] = key0 + 16 + 4 * g + v <= qpos ? s1[v] : -INFINITY;
+            const uint32_t ka = key0 + 4 * g + v, kb_ = ka + 16;
+            const bool va = ka <= qpos && (!p.window || ka < p.sinks || qpos - ka < budget);
+            const bool vb_ = kb_ <= qpos && (!p.window || kb_ < p.sinks || qpos - kb_ < budget);
+            sv[v] = va ? s0[v] : -INFINITY;
+            sv[4 + v] = vb_ ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
         }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-        const float m_new = fmaxf(m_run, mx);       // finite from the first block on: key 0 is visible to every query
-        const float alpha = __expf(m_run - m_new);  // 0 for the first block
+        // without a window key 0 is visible to every query, so the maximum is finite from the first block on; with
+        // one, a query may see nothing yet: it keeps its empty state (all probabilities 0)
+        const float m_new = fmaxf(m_run, mx);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float alpha = __expf(m_run - m_ref);  // 0 for the first block
         float sum = 0.f;
         v8h pb;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float pe = __expf(sv[e] - m_new);
+            const float pe = __expf(sv[e] - m_ref);
             sum += pe;
             pb[e] = (_Float16)pe;
         }
@@ -156,15 +220,16 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         }
         // the next block goes into the other buffer (last read one block ago, before the previous barrier);
         // the block after it is requested now
-        if (key0 + 32 < kv_len) {
+        if (key1 < kv_len) {
             stash(buf ^ 1);
-            if (key0 + 64 < kv_len) fetch(key0 + 64);
+            if (key2 < kv_len) fetch(key2);
         }
         __syncthreads();
         buf ^= 1;
+        key0 = key1;
     }
     if (active && qt * 16 + qi < p.M) {
-        const float inv = 1.0f / l_run;
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
         float* o = p.out + ((size_t)(qt * 16 + qi) * p.nq + head) * HD + 4 * g;
 #pragma unroll
         for (int sl = 0; sl < NS; sl++)
@@ -173,14 +238,24 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
 }
 
 hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st) {
-    if (p.M == 0 || p.nq == 0 || p.nkv == 0 || p.nq % p.nkv || p.pos_start + p.M > p.max_seq) return hipErrorInvalidValue;
+    if (p.M == 0 || p.nq == 0 || p.nkv == 0 || p.nq % p.nkv || p.pos_start + p.M > p.max_seq || p.kv_mode > OXB_KV_FP8_E4M3 ||
+        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)))
+        return hipErrorInvalidValue;
     const uint32_t G = p.nq / p.nkv, hpw = G % 4u == 0 ? 4u : (G % 2u == 0 ? 2u : 1u), tpw = 4u / hpw;
     const uint32_t n_qt = (p.M + 15u) / 16u, grid = ((n_qt + tpw - 1) / tpw) * (p.nq / hpw);
     switch (p.hd) {
-        case 32: hipLaunchKernelGGL(attn_prefill_kernel<32>, dim3(grid), dim3(256), 0, st, p, hpw); break;
-        case 64: hipLaunchKernelGGL(attn_prefill_kernel<64>, dim3(grid), dim3(256), 0, st, p, hpw); break;
-        case 128: hipLaunchKernelGGL(attn_prefill_kernel<128>, dim3(grid), dim3(256), 0, st, p, hpw); break;
-        case 256: hipLaunchKernelGGL(attn_prefill_kernel<256>, dim3(grid), dim3(256), 0, st, p, hpw); break;
+#define OXB_PF_CASE(HD_)                                                                                                          \
+    case HD_:                                                                                                                    \
+        if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_I8>), dim3(grid), dim3(256), 0, st, p, hpw); \
+        else if (p.kv_mode == OXB_KV_FP8_E4M3)                                                                                   \
+            hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_FP8_E4M3>), dim3(grid), dim3(256), 0, st, p, hpw);                \
+        else hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_F16>), dim3(grid), dim3(256), 0, st, p, hpw);                    \
+        break;
+        OXB_PF_CASE(32)
+        OXB_PF_CASE(64)
+        OXB_PF_CASE(128)
+        OXB_PF_CASE(256)
+#undef OXB_PF_CASE
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();

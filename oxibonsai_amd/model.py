@@ -81,6 +81,29 @@ def sample_logits(logits, temperature: float, top_k: int, top_p: float, rng_stat
     return out, st
 
 
+KV_F16, KV_I8, KV_FP8_E4M3 = 0, 1, 2   # OXB_KV_DTYPE_*
+
+
+class AttentionOptions(C.Structure):
+    """oxb_attention_options: KV cache storage type and SlidingWindowConfig { window_size, sink_tokens }
+    (crates/oxibonsai-model/src/layers/sliding_window.rs:11-43; window_size 0 = no window)."""
+    _fields_ = [("kv_dtype", C.c_int32), ("window_size", C.c_uint32), ("sink_tokens", C.c_uint32)]
+
+
+def kv_quantize_rows(kv_dtype: int, rows):
+    """quantize_row_i8 / quantize_row_fp8 (crates/oxibonsai-model/src/kv_cache_quant.rs:46-62, 519-540) on the device
+    -> (codes uint8 [n_rows][n], scales f32 [n_rows])."""
+    lib = _lib.lib()
+    a = np.ascontiguousarray(rows, dtype=np.float32)
+    if a.ndim != 2:
+        raise ValueError("rows must be a 2-D array")
+    codes = np.empty(a.shape, dtype=np.uint8)
+    scales = np.empty(a.shape[0], dtype=np.float32)
+    _check(lib.oxb_hip_kv_quantize_rows(kv_dtype, a.ctypes.data_as(_lib.f32p), a.shape[0], a.shape[1],
+                                        codes.ctypes.data_as(_lib.u8p), scales.ctypes.data_as(_lib.f32p)))
+    return codes, scales
+
+
 class Embedding:
     """Token embedding table resident on the device in its stored form (F32, F16, Q1_0_g128 or TQ2_0_g128)."""
 
@@ -218,6 +241,26 @@ class HipModel:
 
     def uses_graph(self) -> bool:
         return bool(self._lib.oxb_hip_model_uses_graph(self.id))
+
+    def set_attention(self, kv_dtype: int = KV_F16, window_size: int = 0, sink_tokens: int = 0):
+        """Long-context options of the attention kernels; changing kv_dtype replaces the cache (start again at 0)."""
+        opt = AttentionOptions(kv_dtype, window_size, sink_tokens)
+        _check(self._lib.oxb_hip_model_set_attention(self.id, C.byref(opt)))
+
+    def attention(self) -> AttentionOptions:
+        opt = AttentionOptions()
+        _check(self._lib.oxb_hip_model_get_attention(self.id, C.byref(opt)))
+        return opt
+
+    def read_kv(self, layer: int, kv_head: int, pos: int, n_pos: int, seq: int = 0):
+        """Cache rows as stored -> (k, v, k_scales, v_scales): fp16 rows (scales 1.0) or uint8 codes with row scales."""
+        dt = np.float16 if self.attention().kv_dtype == KV_F16 else np.uint8
+        hd = self.cfg["hd"]
+        k, v = np.empty((n_pos, hd), dtype=dt), np.empty((n_pos, hd), dtype=dt)
+        ks, vs = np.empty(n_pos, dtype=np.float32), np.empty(n_pos, dtype=np.float32)
+        _check(self._lib.oxb_hip_model_read_kv(self.id, seq, layer, kv_head, pos, n_pos, k.ctypes.data, v.ctypes.data,
+                                               ks.ctypes.data_as(_lib.f32p), vs.ctypes.data_as(_lib.f32p)))
+        return k, v, ks, vs
 
     def reset(self):
         _check(self._lib.oxb_hip_model_reset(self.id))
