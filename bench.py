@@ -84,7 +84,8 @@ DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd
                   max_seq=32768, eps=1e-6, rope_theta=1e6)   # BASELINE.json configs[4]: Qwen3-8B shape, Q1_0_g128
 
 
-def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32), with_gguf: bool = True) -> dict:
+def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32), with_gguf: bool = True,
+               long_context: int = 0) -> dict:
     """Greedy batch-1 decode of the random-init 8B-shape Q1 model: one batched prefill of `prompt_len` random
     token ids fills the context (timed on its own), then `n_tokens` greedy steps are timed.  The per-token time
     is what the caller of the fused entry point sees: embedding row H2D, the replayed HIP graph (36 layers,
@@ -170,21 +171,51 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
     for B in batches:
         cfg_b = dict(cfg, max_seq=prompt_len + 64)
         mb = HipModel(be, cfg_b, w, batch=B)
-        for sq in range(B):
-            mb.prefill(np.roll(rows, sq, axis=0), seq=sq, want_logits=False)
-        toks = [int(ids[sq]) for sq in range(B)]
-        steps_b, spent = 32, 0.0
-        for i in range(steps_b + 2):
-            hidden = np.stack([emb(t) for t in toks])
-            t0 = time.perf_counter()
-            _, out = mb.forward(hidden, np.full(B, prompt_len + i, dtype=np.uint32), want_logits=False)
-            if i >= 2:      # the first step records the graph, the second replays it for the first time
-                spent += time.perf_counter() - t0
-            toks = [int(t) for t in out]
-        res["batched"].append({"batch": B, "context_before": prompt_len, "steps": steps_b,
-                               "ms_per_step": round(spent / steps_b * 1e3, 4),
-                               "tok_per_s": round(B * steps_b / spent, 1), "hip_graph": mb.uses_graph()})
+        for cache, kv_mode in (("fp16", 0), ("int8", 1)) if B == max(batches) else (("fp16", 0),):
+            mb.set_attention(kv_mode, 0, 0)
+            for sq in range(B):
+                mb.prefill(np.roll(rows, sq, axis=0), seq=sq, want_logits=False)
+            toks = [int(ids[sq]) for sq in range(B)]
+            steps_b, spent = 32, 0.0
+            for i in range(steps_b + 2):
+                hidden = np.stack([emb(t) for t in toks])
+                t0 = time.perf_counter()
+                _, out = mb.forward(hidden, np.full(B, prompt_len + i, dtype=np.uint32), want_logits=False)
+                if i >= 2:      # the first step records the graph, the second replays it for the first time
+                    spent += time.perf_counter() - t0
+                toks = [int(t) for t in out]
+            res["batched"].append({"batch": B, "context_before": prompt_len, "kv_cache": cache, "steps": steps_b,
+                                   "ms_per_step": round(spent / steps_b * 1e3, 4),
+                                   "tok_per_s": round(B * steps_b / spent, 1), "hip_graph": mb.uses_graph()})
         mb.close()
+    if long_context:
+        # one sequence deep into the 32 768-position context: fp16 cache, quantised caches, sliding window
+        from oxibonsai_amd.model import KV_F16, KV_FP8_E4M3, KV_I8
+        ml = HipModel(be, dict(cfg, max_seq=long_context + 64), w, batch=1)
+        reps = -(-long_context // prompt_len)
+        res["long_context"] = []
+        for name, mode, window, sinks in (("fp16 cache", KV_F16, 0, 0), ("int8 cache", KV_I8, 0, 0), ("fp8-e4m3 cache", KV_FP8_E4M3, 0, 0),
+                                          ("fp16 cache, window 4096 + 4 sinks", KV_F16, 4096, 4)):
+            ml.set_attention(mode, window, sinks)
+            t0 = time.perf_counter()
+            for c in range(reps):       # the prompt rows again and again until the context is full
+                n = min(prompt_len, long_context - c * prompt_len)
+                ml.prefill(rows[:n], pos_start=c * prompt_len, want_logits=False)
+            t_fill = time.perf_counter() - t0
+            t, spent, steps_l = int(ids[0]), 0.0, 32
+            for i in range(steps_l + 2):
+                hidden = emb(t)
+                t0 = time.perf_counter()
+                _, out = ml.forward(hidden, long_context + i, want_logits=False)
+                if i >= 2:
+                    spent += time.perf_counter() - t0
+                t = int(out[0])
+            kv_row = cfg["hd"] * (2 if mode == KV_F16 else 1) + (0 if mode == KV_F16 else 4)
+            seen = long_context if not window else min(window, long_context)
+            res["long_context"].append({"cache": name, "context_before": long_context, "fill_s": round(t_fill, 2),
+                                        "ms_per_token": round(spent / steps_l * 1e3, 4), "tok_per_s": round(steps_l / spent, 1),
+                                        "kv_bytes_read_per_token": 2 * cfg["n_layers"] * cfg["nkv"] * kv_row * seen})
+        ml.close()
     if with_cpu:
         # CPU SIMD tier on the same matrices: linear layers only (one layer x 36 + LM head), an upper bound on its tok/s
         from oracle import oracle
@@ -294,6 +325,8 @@ def main() -> int:
     ap.add_argument("--decode-tokens", type=int, default=128)
     ap.add_argument("--decode-batches", type=str, default="8,32", help="batch sizes of the batched decode runs ('' = none)")
     ap.add_argument("--no-gguf", action="store_true", help="skip the checkpoint-file load of the decode leg")
+    ap.add_argument("--long-context", type=int, default=32000,
+                    help="context of the long-context decode runs (fp16 / int8 / fp8 cache, sliding window); 0 = skip")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (multi-GPU sharding is design-only)",
@@ -459,7 +492,8 @@ def main() -> int:
         out["prefill_gemm"] = prefill_gemm_leg(be, L, torch)
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
-                                   tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf)
+                                   tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf,
+                                   args.long_context)
         out["decode_ternary_1p7b"] = decode_ternary_leg(be, args.decode_context, args.decode_tokens)
     print(json.dumps(out), flush=True)
     return 0
