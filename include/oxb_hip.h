@@ -154,13 +154,24 @@ int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is re
  *    [token][head][dim]), scales [batch][layer][kv_head][max_seq rounded up to 128].  Fp8KvFormat::E5M2 is not
  *    offered: its row quantiser turns the row maximum into infinity whenever max / scale rounds above 57344
  *    (quant_fp8.rs:229-231), about one row in five.
- * oxb_hip_model_set_attention may be called at any time between steps; changing kv_dtype replaces the cache, so
- * the sequences start again at position 0. */
+ *  - paged cache: PagedKvCache / BlockPool / BlockTable (crates/oxibonsai-model/src/paged_kv_cache.rs:70-160, 187-236,
+ *    294-345).  The cache is a pool of n_pages pages of page_size positions (DEFAULT_BLOCK_SIZE = 16, :33); a page holds
+ *    those positions for every layer and kv head ([layer][kv_head][position][hd], where the reference allocates one
+ *    page per layer in lockstep), so one table of page numbers per sequence serves all layers.  The model's `batch`
+ *    sequence slots take the place of the reference's sequence ids.  Pages are handed out lazily: decode and prefill
+ *    calls reserve what the positions they write need, as write_kv does (:447-470); when the pool is empty they fail
+ *    with OXB_HIP_OUT_OF_MEMORY ("out of memory: no free KV blocks", PagedKvError::OutOfMemory) and the pages taken
+ *    so far stay with the sequence, as in ensure_capacity (:394-433).  The kernels look the page of a position up in
+ *    the table; everything else (window, quantised rows) combines freely.
+ * oxb_hip_model_set_attention may be called at any time between steps; changing kv_dtype, page_size or n_pages
+ * replaces the cache, so the sequences start again at position 0. */
 enum { OXB_KV_DTYPE_F16 = 0, OXB_KV_DTYPE_I8 = 1, OXB_KV_DTYPE_FP8_E4M3 = 2 };
 typedef struct {
     int32_t kv_dtype;       /* OXB_KV_DTYPE_* */
     uint32_t window_size;   /* 0 = no window */
     uint32_t sink_tokens;
+    uint32_t page_size;     /* paged cache: positions per page (16, 32, 64 or 128); 0 = contiguous cache */
+    uint32_t n_pages;       /* paged cache: pages in the pool, shared by the model's sequences; 0 = contiguous cache */
 } oxb_attention_options;
 int  oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt);
 int  oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt);
@@ -169,6 +180,15 @@ int  oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt);
  * or 1-byte codes), k_scales / v_scales n_pos row scales (1.0 for an fp16 cache).  Any pointer may be NULL. */
 int  oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t kv_head, uint32_t pos, uint32_t n_pos,
                            void* k_rows, void* v_rows, float* k_scales, float* v_scales);
+/* Paged cache bookkeeping (each is a no-op / trivial answer for a contiguous cache):
+ * reserve  = PagedKvCache::ensure_capacity (:394-433): pages for positions 0 .. n_tokens - 1 of sequence slot `seq`;
+ * release  = drop_sequence (:362-375): the slot's pages return to the pool (oxb_hip_model_reset releases every slot);
+ * pool     = BlockPool::free_count / total_count (:138-146); capacity = BlockTable::token_capacity (:233-236). */
+typedef struct { uint32_t page_size, total_pages, free_pages; } oxb_kv_pool_info;
+int  oxb_hip_model_kv_reserve(uint64_t model, uint32_t seq, uint32_t n_tokens);
+int  oxb_hip_model_kv_release(uint64_t model, uint32_t seq);
+int  oxb_hip_model_kv_pool(uint64_t model, oxb_kv_pool_info* info);
+int  oxb_hip_model_kv_capacity(uint64_t model, uint32_t seq, uint32_t* n_tokens);
 /* quantize_row_i8 / quantize_row_fp8 on the device for n_rows rows of n values each (host buffers): the same
  * routine the attention kernels store new rows with. */
 int  oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, uint32_t n, uint8_t* codes, float* scales);

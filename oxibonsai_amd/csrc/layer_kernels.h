@@ -4,6 +4,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include "kv_quant_device.h"
+
 struct OxbQkParams {
     const float* qkv;      // [batch][qkv_stride]: q heads | k heads | v heads
     uint32_t qkv_stride;
@@ -12,9 +14,10 @@ struct OxbQkParams {
     const uint32_t* pos;           // [batch], device; null: row b is token pos_base + b of sequence `seq` (prefill)
     uint32_t pos_base, seq;
     float* q_rope;                 // [batch][nq][hd]
-    void *k_cache, *v_cache;       // [batch][n_layers][nkv][max_seq][hd]: fp16, or one-byte codes (kv_mode)
-    float *k_scale, *v_scale;      // quantised cache: row scales [batch][n_layers][nkv][sc_stride]
-    uint32_t kv_mode, sc_stride;
+    void *k_cache, *v_cache;       // cache rows of hd values each (fp16, or one-byte codes: kv_mode), placed by `kv`
+    float *k_scale, *v_scale;      // quantised cache: one scale per row
+    uint32_t kv_mode;
+    OxbKvLayout kv;
     uint32_t nq, nkv, hd, max_seq, n_layers, layer;
     float eps;
 };
@@ -26,9 +29,10 @@ struct OxbAttnParams {
     const float *q_norm, *k_norm;        // [hd]
     const float *cos_t, *sin_t;          // [max_seq][hd/2]
     float eps;
-    void *k_cache, *v_cache;             // [batch][n_layers][nkv][max_seq][hd]: fp16, or one-byte codes (kv_mode)
-    float *k_scale, *v_scale;            // quantised cache: row scales [batch][n_layers][nkv][sc_stride]
-    uint32_t kv_mode, sc_stride;         // OXB_KV_* (kv_quant_device.h); sc_stride: a multiple of the chunk, >= max_seq
+    void *k_cache, *v_cache;             // cache rows of hd values each (fp16, or one-byte codes: kv_mode), placed by `kv`
+    float *k_scale, *v_scale;            // quantised cache: one scale per row
+    uint32_t kv_mode;                    // OXB_KV_* (kv_quant_device.h)
+    OxbKvLayout kv;                      // contiguous (row_stride a multiple of the chunk, >= max_seq) or paged (pages of 16..128 positions)
     uint32_t window, sinks;              // sliding window with attention sinks; window 0 = off
     float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1

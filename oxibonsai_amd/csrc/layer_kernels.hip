@@ -161,8 +161,8 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
     const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
     const float* cs = p.cos_t + (size_t)pos * half;
     const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t head_row = ((size_t)seq * p.n_layers + p.layer) * p.nkv + hh;
-    const size_t cache_off = (head_row * p.max_seq + pos) * hd;
+    const size_t row = is_q ? 0 : kv_row(p.kv, seq, p.layer, hh, pos);
+    const size_t cache_off = row * hd;
     // head_dim <= 256: a thread owns at most one rotation pair and two V values
     float o_lo = 0.f, o_hi = 0.f;
     if (tid < half) {
@@ -193,8 +193,8 @@ __global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) 
         if (tid < hd) vc[tid] = (uint8_t)kv_encode<KVM>(v0, vs);
         if (tid + 128 < hd) vc[tid + 128] = (uint8_t)kv_encode<KVM>(v1, vs);
         if (tid == 0) {
-            p.k_scale[head_row * p.sc_stride + pos] = ks;
-            p.v_scale[head_row * p.sc_stride + pos] = vs;
+            p.k_scale[row] = ks;
+            p.v_scale[row] = vs;
         }
     } else {
         __half* kc = reinterpret_cast<__half*>(p.k_cache) + cache_off;
@@ -308,13 +308,16 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     const float* qkv = p.qkv + (size_t)b * p.qkv_stride;
     const float* cs = p.cos_t + (size_t)pos * half;
     const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t head_row = ((size_t)b * p.n_layers + p.layer) * p.nkv + kvh;
-    const size_t base = head_row * p.max_seq * HD;
     typedef typename std::conditional<QC, uint8_t, _Float16>::type cache_t;
-    cache_t* Kc = reinterpret_cast<cache_t*>(p.k_cache) + base;
-    cache_t* Vc = reinterpret_cast<cache_t*>(p.v_cache) + base;
-    float* Ksc = QC ? p.k_scale + head_row * p.sc_stride : nullptr;  // one scale per position; the stride is a multiple of the chunk
-    float* Vsc = QC ? p.v_scale + head_row * p.sc_stride : nullptr;
+    cache_t* Kc = reinterpret_cast<cache_t*>(p.k_cache);
+    cache_t* Vc = reinterpret_cast<cache_t*>(p.v_cache);
+    float* Ksc = p.k_scale;  // one scale per row
+    float* Vsc = p.v_scale;
+    // row of a position of this (sequence, layer, kv head): an offset in a contiguous cache, a table lookup in a paged
+    // one (four consecutive positions from a multiple of four never straddle a page: pages hold 16 positions or more)
+    const bool paged = p.kv.page_table != nullptr;
+    const size_t row0 = paged ? 0 : kv_row(p.kv, b, p.layer, kvh, 0);
+    auto row_of = [&](uint32_t key) -> size_t { return paged ? kv_row(p.kv, b, p.layer, kvh, key) : row0 + key; };
 
     // K rows of the two 16-key tiles (A operands) and this lane's pieces of the 32-key V block of a chunk.
     // Rows past the last key repeat it; their scores are masked.
@@ -324,32 +327,33 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     v4i vr[VL];
     auto load_k = [&](uint32_t chunk) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
-        const uint32_t kr0 = min(key0 + qi, seq_len - 1), kr1 = min(key0 + 16 + qi, seq_len - 1);
+        const size_t kr0 = row_of(min(key0 + qi, seq_len - 1)), kr1 = row_of(min(key0 + 16 + qi, seq_len - 1));
 #pragma unroll
         for (int s = 0; s < KS; s++) {
             if constexpr (QC) {
-                k0q[s] = *reinterpret_cast<const kvi2_t*>(Kc + (size_t)kr0 * HD + (HD / 4) * g + 8 * s);
-                k1q[s] = *reinterpret_cast<const kvi2_t*>(Kc + (size_t)kr1 * HD + (HD / 4) * g + 8 * s);
+                k0q[s] = *reinterpret_cast<const kvi2_t*>(Kc + kr0 * HD + (HD / 4) * g + 8 * s);
+                k1q[s] = *reinterpret_cast<const kvi2_t*>(Kc + kr1 * HD + (HD / 4) * g + 8 * s);
             } else {
-                k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr0 * HD + 32 * s + 8 * g);
-                k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + (size_t)kr1 * HD + 32 * s + 8 * g);
+                k0r[s] = *reinterpret_cast<const v8h_t*>(Kc + kr0 * HD + 32 * s + 8 * g);
+                k1r[s] = *reinterpret_cast<const v8h_t*>(Kc + kr1 * HD + 32 * s + 8 * g);
             }
         }
-        if constexpr (QC) {
-            ksc0 = *reinterpret_cast<const float4*>(Ksc + key0 + 4 * g);
-            ksc1 = *reinterpret_cast<const float4*>(Ksc + key0 + 16 + 4 * g);
+        if constexpr (QC) {  // scales of positions past the last key are never used (their scores are masked)
+            ksc0 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u)));
+            ksc1 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u)));
         }
     };
     auto load_v = [&](uint32_t chunk) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
 #pragma unroll
         for (int i = 0; i < VL; i++) {
-            const uint32_t id = i * 64 + lane, row = min(key0 + id / VPR, seq_len - 1), col = id % VPR;
-            vr[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(Vc + (size_t)row * HD) + col * 16);
+            const uint32_t id = i * 64 + lane, col = id % VPR;
+            const size_t row = row_of(min(key0 + id / VPR, seq_len - 1));
+            vr[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(Vc + row * HD) + col * 16);
         }
         if constexpr (QC) {
-            vsc0 = *reinterpret_cast<const float4*>(Vsc + key0 + 4 * g);
-            vsc1 = *reinterpret_cast<const float4*>(Vsc + key0 + 16 + 4 * g);
+            vsc0 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u)));
+            vsc1 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u)));
         }
     };
 
@@ -368,6 +372,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     }
     // --- K and V of the new position, by the workgroup whose slot walks its chunk (wave 0 and wave 1) ---
+    const size_t new_row = row_of(pos);
     if (owner) {
         if (wave == 0) {
             const float* in = qkv + (size_t)(p.nq + kvh) * HD;
@@ -394,18 +399,18 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
 #pragma unroll
                 for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
                 scale = kv_row_scale<KVM>(mx);
-                if (lane == 0) Ksc[pos] = scale;
+                if (lane == 0) Ksc[new_row] = scale;
             }
 #pragma unroll
             for (int it = 0; it < KI; it++) {
                 const uint32_t d = lane + 64 * it;
                 if (d < half) {
                     if constexpr (QC) {
-                        Kc[(size_t)pos * HD + d] = (uint8_t)kv_encode<KVM>(klo[it], scale);
-                        Kc[(size_t)pos * HD + d + half] = (uint8_t)kv_encode<KVM>(khi[it], scale);
+                        Kc[new_row * HD + d] = (uint8_t)kv_encode<KVM>(klo[it], scale);
+                        Kc[new_row * HD + d + half] = (uint8_t)kv_encode<KVM>(khi[it], scale);
                     } else {
-                        Kc[(size_t)pos * HD + d] = (_Float16)klo[it];
-                        Kc[(size_t)pos * HD + d + half] = (_Float16)khi[it];
+                        Kc[new_row * HD + d] = (_Float16)klo[it];
+                        Kc[new_row * HD + d + half] = (_Float16)khi[it];
                     }
                 }
             }
@@ -424,14 +429,14 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
 #pragma unroll
                 for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
                 scale = kv_row_scale<KVM>(mx);
-                if (lane == 0) Vsc[pos] = scale;
+                if (lane == 0) Vsc[new_row] = scale;
             }
 #pragma unroll
             for (int it = 0; it < VI; it++) {
                 const uint32_t d = lane + 64 * it;
                 if (d < HD) {
-                    if constexpr (QC) Vc[(size_t)pos * HD + d] = (uint8_t)kv_encode<KVM>(vv[it], scale);
-                    else Vc[(size_t)pos * HD + d] = (_Float16)vv[it];
+                    if constexpr (QC) Vc[new_row * HD + d] = (uint8_t)kv_encode<KVM>(vv[it], scale);
+                    else Vc[new_row * HD + d] = (_Float16)vv[it];
                 }
             }
         }
@@ -801,7 +806,8 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
     if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
         !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 ||
-        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale || p.sc_stride % OXB_ATTN_CHUNK || p.sc_stride < p.max_seq)))
+        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)) ||
+        (p.kv.page_table ? (p.kv.page_shift < 4 || p.kv.page_shift > 7) : (p.kv.row_stride % OXB_ATTN_CHUNK != 0 || p.kv.row_stride < p.max_seq)))
         return hipErrorInvalidValue;
     const dim3 grid(p.n_splits, p.nkv, batch), block(256);
     switch (p.hd) {

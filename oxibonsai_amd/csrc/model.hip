@@ -45,11 +45,18 @@ struct Model {
           *gu = nullptr, *logits = nullptr;
     uint32_t *tokens = nullptr, *pos = nullptr;
     void* argmax_ws = nullptr;
-    // KV cache: fp16 values or one-byte codes [batch][n_layers][nkv][max_seq][hd]; a quantised cache also keeps one
-    // f32 scale per row, [batch][n_layers][nkv][sc_stride]
+    // KV cache: rows of hd fp16 values or one-byte codes, a quantised cache also one f32 scale per row.  Contiguous:
+    // [batch][n_layers][nkv][row_stride] rows; paged: a pool [n_pages][n_layers][nkv][2^page_shift] rows and, per
+    // sequence, a table of page numbers (kv_quant_device.h: OxbKvLayout)
     void *k_cache = nullptr, *v_cache = nullptr;
     float *k_scale = nullptr, *v_scale = nullptr;
-    uint32_t kv_mode = OXB_KV_F16, sc_stride = 0, window = 0, sinks = 0;
+    uint32_t kv_mode = OXB_KV_F16, row_stride = 0, window = 0, sinks = 0;
+    uint32_t page_shift = 0, n_pages = 0, table_stride = 0;   // n_pages 0: contiguous
+    std::vector<uint32_t> free_pages;                          // stack of free physical pages
+    std::vector<std::vector<uint32_t>> seq_pages;              // pages of each sequence slot, in position order
+    std::vector<uint32_t> h_table;                             // [batch][table_stride], mirrored in d_table
+    uint32_t* d_table = nullptr;
+    bool table_dirty = false;
     float *cos_t = nullptr, *sin_t = nullptr;
     void* xq_mem = nullptr;
     XqBuf xq;
@@ -90,12 +97,17 @@ static int dev_alloc(Model& m, void** p, size_t bytes) {
 }
 
 static void free_kv_cache(Model& m) {
-    void* bufs[4] = {m.k_cache, m.v_cache, m.k_scale, m.v_scale};
+    void* bufs[5] = {m.k_cache, m.v_cache, m.k_scale, m.v_scale, m.d_table};
     for (void* p : bufs)
         if (p) (void)hipFree(p);
     m.k_cache = m.v_cache = nullptr;
     m.k_scale = m.v_scale = nullptr;
-    m.sc_stride = 0;
+    m.d_table = nullptr;
+    m.n_pages = m.page_shift = m.table_stride = 0;
+    m.free_pages.clear();
+    m.seq_pages.clear();
+    m.h_table.clear();
+    m.table_dirty = false;
 }
 
 static void free_model(Model& m) {
@@ -212,6 +224,54 @@ static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn
     return OXB_HIP_OK;
 }
 
+static OxbKvLayout kv_layout(const Model& m) {
+    OxbKvLayout L;
+    L.page_table = m.n_pages ? m.d_table : nullptr;
+    L.page_shift = m.page_shift;
+    L.table_stride = m.table_stride;
+    L.n_layers = m.d.n_layers;
+    L.nkv = m.d.nkv;
+    L.row_stride = m.row_stride;
+    return L;
+}
+
+// Paged cache: make sure sequence `seq` owns pages for positions 0 .. n_tokens - 1 (PagedKvCache::ensure_capacity,
+// crates/oxibonsai-model/src/paged_kv_cache.rs:394-433: pages are taken from the free list one by one; when the pool
+// runs dry the pages taken so far stay with the sequence).  A contiguous cache needs nothing.
+static int kv_reserve(Model& m, uint32_t seq, uint64_t n_tokens) {
+    if (!m.k_cache) return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: the model has no KV cache (its last reallocation failed)");
+    if (!m.n_pages) return OXB_HIP_OK;
+    const size_t need = (size_t)((n_tokens + (1u << m.page_shift) - 1) >> m.page_shift);
+    std::vector<uint32_t>& pg = m.seq_pages[seq];
+    while (pg.size() < need) {
+        if (m.free_pages.empty())
+            return fail(OXB_HIP_OUT_OF_MEMORY, "out of memory: no free KV blocks (sequence %u needs %zu pages of %u positions, it holds %zu, pool of %u)",
+                        seq, need, 1u << m.page_shift, pg.size(), m.n_pages);
+        const uint32_t page = m.free_pages.back();
+        m.free_pages.pop_back();
+        m.h_table[(size_t)seq * m.table_stride + pg.size()] = page;
+        pg.push_back(page);
+        m.table_dirty = true;
+    }
+    return OXB_HIP_OK;
+}
+
+static void kv_release(Model& m, uint32_t seq) {  // PagedKvCache::drop_sequence (:362-375): pages go back to the pool
+    if (!m.n_pages) return;
+    std::vector<uint32_t>& pg = m.seq_pages[seq];
+    for (size_t i = pg.size(); i-- > 0;) m.free_pages.push_back(pg[i]);
+    pg.clear();
+}
+
+// The device copy of the page tables follows the host's before the next launch reads it (never inside a capture).
+static int kv_sync_table(Model& m) {
+    if (!m.n_pages || !m.table_dirty) return OXB_HIP_OK;
+    OXB_TRY_HIP(hipMemcpyAsync(m.d_table, m.h_table.data(), m.h_table.size() * 4, hipMemcpyHostToDevice, g_rt.stream), "page table upload");
+    OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "page table upload");
+    m.table_dirty = false;
+    return OXB_HIP_OK;
+}
+
 // QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch, one launch; leaves the
 // slot results in m.attn_part and the parameters the merge needs in *ap.
 static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out) {
@@ -229,7 +289,7 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.k_scale = m.k_scale;
     ap.v_scale = m.v_scale;
     ap.kv_mode = m.kv_mode;
-    ap.sc_stride = m.sc_stride;
+    ap.kv = kv_layout(m);
     ap.window = m.window;
     ap.sinks = m.sinks;
     ap.part = m.attn_part;
@@ -399,7 +459,7 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.k_scale = m.k_scale;
         qp.v_scale = m.v_scale;
         qp.kv_mode = m.kv_mode;
-        qp.sc_stride = m.sc_stride;
+        qp.kv = kv_layout(m);
         qp.nq = d.nq;
         qp.nkv = d.nkv;
         qp.hd = d.hd;
@@ -409,15 +469,15 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.eps = d.eps;
         OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, M, st), "kernel launch failed: qk_norm_rope_store");
         OxbPrefillAttnParams ap;
-        const size_t layer_row = ((size_t)seq * d.n_layers + L) * d.nkv;
-        const size_t layer_off = layer_row * (size_t)d.max_seq * d.hd * (m.kv_mode == OXB_KV_F16 ? 2 : 1);  // bytes
         ap.q = m.pf_q;
-        ap.k_cache = (const uint8_t*)m.k_cache + layer_off;
-        ap.v_cache = (const uint8_t*)m.v_cache + layer_off;
-        ap.k_scale = m.k_scale ? m.k_scale + layer_row * m.sc_stride : nullptr;
-        ap.v_scale = m.v_scale ? m.v_scale + layer_row * m.sc_stride : nullptr;
+        ap.k_cache = m.k_cache;
+        ap.v_cache = m.v_cache;
+        ap.k_scale = m.k_scale;
+        ap.v_scale = m.v_scale;
         ap.kv_mode = m.kv_mode;
-        ap.sc_stride = m.sc_stride;
+        ap.kv = kv_layout(m);
+        ap.seq = seq;
+        ap.layer = L;
         ap.window = m.window;
         ap.sinks = m.sinks;
         ap.out = m.pf_attn;
@@ -493,14 +553,15 @@ int oxb_hip_free_f32(uint64_t id) {
     return OXB_HIP_OK;
 }
 
-// (Re)allocates the KV cache in the given storage form.  Row scales start at 0 so that a row never written reads
-// as zeros; the scale stride is a whole number of attention chunks, which keeps the kernels' 16-byte scale loads
-// inside the row and aligned.
-static int alloc_kv_cache(Model& m, uint32_t kv_mode) {
+// (Re)allocates the KV cache in the given storage form, contiguous (n_pages 0) or as a pool of n_pages pages of
+// page_size positions.  Row scales start at 0 so that a row never written reads as zeros.  A contiguous head holds a
+// whole number of attention chunks of rows, which keeps the kernels' 16-byte scale loads aligned and inside it.
+static int alloc_kv_cache(Model& m, uint32_t kv_mode, uint32_t page_size, uint32_t n_pages) {
     const oxb_model_desc& d = m.d;
-    const size_t rows = (size_t)d.batch * d.n_layers * d.nkv;
-    const size_t bytes = rows * d.max_seq * d.hd * (kv_mode == OXB_KV_F16 ? 2 : 1);
     free_kv_cache(m);
+    m.row_stride = (d.max_seq + OXB_ATTN_CHUNK_POSITIONS - 1) / OXB_ATTN_CHUNK_POSITIONS * OXB_ATTN_CHUNK_POSITIONS;
+    const size_t rows = n_pages ? (size_t)n_pages * d.n_layers * d.nkv * page_size : (size_t)d.batch * d.n_layers * d.nkv * m.row_stride;
+    const size_t bytes = rows * d.hd * (kv_mode == OXB_KV_F16 ? 2 : 1);
     auto grab = [&](void** p, size_t n) -> int {
         if (hipMalloc(p, n ? n : 16) == hipSuccess) return OXB_HIP_OK;
         *p = nullptr;
@@ -509,12 +570,24 @@ static int alloc_kv_cache(Model& m, uint32_t kv_mode) {
     OXB_TRY(grab(&m.k_cache, bytes));
     OXB_TRY(grab(&m.v_cache, bytes));
     if (kv_mode != OXB_KV_F16) {
-        m.sc_stride = (d.max_seq + OXB_ATTN_CHUNK_POSITIONS - 1) / OXB_ATTN_CHUNK_POSITIONS * OXB_ATTN_CHUNK_POSITIONS;
-        const size_t sb = rows * m.sc_stride * sizeof(float);
+        const size_t sb = rows * sizeof(float);
         OXB_TRY(grab((void**)&m.k_scale, sb));
         OXB_TRY(grab((void**)&m.v_scale, sb));
         OXB_TRY_HIP(hipMemset(m.k_scale, 0, sb), "scale clear");
         OXB_TRY_HIP(hipMemset(m.v_scale, 0, sb), "scale clear");
+    }
+    if (n_pages) {
+        uint32_t shift = 0;
+        while ((1u << shift) < page_size) shift++;
+        m.page_shift = shift;
+        m.n_pages = n_pages;
+        m.table_stride = (d.max_seq + page_size - 1) / page_size;
+        m.h_table.assign((size_t)d.batch * m.table_stride, 0u);   // entries of unreserved blocks name page 0: never read
+        m.seq_pages.assign(d.batch, {});
+        m.free_pages.resize(n_pages);
+        for (uint32_t i = 0; i < n_pages; i++) m.free_pages[i] = n_pages - 1 - i;   // page 0 is handed out first
+        OXB_TRY(grab((void**)&m.d_table, m.h_table.size() * 4));
+        OXB_TRY_HIP(hipMemset(m.d_table, 0, m.h_table.size() * 4), "page table clear");
     }
     m.kv_mode = kv_mode;
     return OXB_HIP_OK;
@@ -574,7 +647,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16)) ||
+        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + OXB_XEXP_BYTES))) {
@@ -659,10 +732,15 @@ int oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt
     // the captured decode step holds the cache pointers and the options: it is captured again on the next step
     if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
     m->graph_exec = nullptr;
-    if ((uint32_t)opt->kv_dtype != m->kv_mode) {
-        const int rc = alloc_kv_cache(*m, (uint32_t)opt->kv_dtype);
-        if (rc) {  // leave the model usable: back to the fp16 cache
-            if (alloc_kv_cache(*m, OXB_KV_F16)) m->k_cache = m->v_cache = nullptr;
+    const uint32_t cur_page = m->n_pages ? 1u << m->page_shift : 0u;
+    if ((opt->n_pages != 0) != (opt->page_size != 0))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: page_size and n_pages must both be given (paged cache) or both be 0");
+    if (opt->n_pages && opt->page_size != 16 && opt->page_size != 32 && opt->page_size != 64 && opt->page_size != 128)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: page_size %u (supported: 16, 32, 64, 128 positions)", opt->page_size);
+    if ((uint32_t)opt->kv_dtype != m->kv_mode || opt->n_pages != m->n_pages || opt->page_size != cur_page) {
+        const int rc = alloc_kv_cache(*m, (uint32_t)opt->kv_dtype, opt->page_size, opt->n_pages);
+        if (rc) {  // leave the model usable: back to the contiguous fp16 cache
+            if (alloc_kv_cache(*m, OXB_KV_F16, 0, 0)) free_kv_cache(*m);
             return rc;
         }
     }
@@ -679,6 +757,8 @@ int oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt) {
     opt->kv_dtype = (int32_t)m->kv_mode;
     opt->window_size = m->window;
     opt->sink_tokens = m->sinks;
+    opt->page_size = m->n_pages ? 1u << m->page_shift : 0u;
+    opt->n_pages = m->n_pages;
     return OXB_HIP_OK;
 }
 
@@ -694,21 +774,75 @@ int oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t
     if (!m->k_cache) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: the model has no KV cache");
     if (n_pos == 0) return OXB_HIP_OK;
     OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
-    const size_t esz = m->kv_mode == OXB_KV_F16 ? 2 : 1;
-    const size_t head_row = ((size_t)seq * d.n_layers + layer) * d.nkv + kv_head;
-    const size_t off = (head_row * d.max_seq + pos) * d.hd * esz, bytes = (size_t)n_pos * d.hd * esz;
-    if (k_rows) OXB_TRY_HIP(hipMemcpy(k_rows, (const uint8_t*)m->k_cache + off, bytes, hipMemcpyDeviceToHost), "cache read");
-    if (v_rows) OXB_TRY_HIP(hipMemcpy(v_rows, (const uint8_t*)m->v_cache + off, bytes, hipMemcpyDeviceToHost), "cache read");
-    if (m->kv_mode != OXB_KV_F16) {
-        const size_t so = head_row * m->sc_stride + pos;
-        if (k_scales) OXB_TRY_HIP(hipMemcpy(k_scales, m->k_scale + so, (size_t)n_pos * 4, hipMemcpyDeviceToHost), "scale read");
-        if (v_scales) OXB_TRY_HIP(hipMemcpy(v_scales, m->v_scale + so, (size_t)n_pos * 4, hipMemcpyDeviceToHost), "scale read");
-    } else {
+    const size_t esz = m->kv_mode == OXB_KV_F16 ? 2 : 1, row_bytes = (size_t)d.hd * esz;
+    const uint32_t run_max = m->n_pages ? 1u << m->page_shift : n_pos;   // rows of one page are contiguous
+    for (uint32_t i = 0; i < n_pos;) {
+        const uint32_t p0 = pos + i;
+        uint32_t run = m->n_pages ? run_max - (p0 & (run_max - 1)) : n_pos;
+        if (run > n_pos - i) run = n_pos - i;
+        size_t row;
+        if (m->n_pages) {
+            const std::vector<uint32_t>& pg = m->seq_pages[seq];
+            const size_t blk = p0 >> m->page_shift;
+            if (blk >= pg.size())
+                return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u of sequence %u lies outside its %zu pages", p0, seq, pg.size());
+            row = ((((size_t)pg[blk] * d.n_layers + layer) * d.nkv + kv_head) << m->page_shift) + (p0 & (run_max - 1));
+        } else {
+            row = (((size_t)seq * d.n_layers + layer) * d.nkv + kv_head) * m->row_stride + p0;
+        }
+        if (k_rows) OXB_TRY_HIP(hipMemcpy((uint8_t*)k_rows + i * row_bytes, (const uint8_t*)m->k_cache + row * row_bytes, run * row_bytes, hipMemcpyDeviceToHost), "cache read");
+        if (v_rows) OXB_TRY_HIP(hipMemcpy((uint8_t*)v_rows + i * row_bytes, (const uint8_t*)m->v_cache + row * row_bytes, run * row_bytes, hipMemcpyDeviceToHost), "cache read");
+        if (m->kv_mode != OXB_KV_F16) {
+            if (k_scales) OXB_TRY_HIP(hipMemcpy(k_scales + i, m->k_scale + row, (size_t)run * 4, hipMemcpyDeviceToHost), "scale read");
+            if (v_scales) OXB_TRY_HIP(hipMemcpy(v_scales + i, m->v_scale + row, (size_t)run * 4, hipMemcpyDeviceToHost), "scale read");
+        }
+        i += run;
+    }
+    if (m->kv_mode == OXB_KV_F16)
         for (uint32_t i = 0; i < n_pos; i++) {
             if (k_scales) k_scales[i] = 1.0f;
             if (v_scales) v_scales[i] = 1.0f;
         }
-    }
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_kv_reserve(uint64_t model, uint32_t seq, uint32_t n_tokens) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (seq >= m->d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, m->d.batch);
+    if (n_tokens > m->d.max_seq)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u positions exceed the context of %u", n_tokens, m->d.max_seq);
+    return kv_reserve(*m, seq, n_tokens);
+}
+
+int oxb_hip_model_kv_release(uint64_t model, uint32_t seq) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (seq >= m->d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, m->d.batch);
+    OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
+    kv_release(*m, seq);
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_kv_pool(uint64_t model, oxb_kv_pool_info* info) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (!info) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
+    info->page_size = m->n_pages ? 1u << m->page_shift : 0u;
+    info->total_pages = m->n_pages;
+    info->free_pages = (uint32_t)m->free_pages.size();
+    return OXB_HIP_OK;
+}
+
+int oxb_hip_model_kv_capacity(uint64_t model, uint32_t seq, uint32_t* n_tokens) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* m = find_model(model);
+    if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    if (seq >= m->d.batch || !n_tokens) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, m->d.batch);
+    *n_tokens = m->n_pages ? (uint32_t)(m->seq_pages[seq].size() << m->page_shift) : m->d.max_seq;
     return OXB_HIP_OK;
 }
 
@@ -740,8 +874,10 @@ int oxb_hip_model_reset(uint64_t model) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
-    // positions are supplied per call and attention reads only 0..pos, so nothing has to be cleared
+    // positions are supplied per call and attention reads only 0..pos, so nothing has to be cleared; a paged cache
+    // takes the sequences' pages back
     (void)hipStreamSynchronize(g_rt.stream);
+    for (uint32_t b = 0; b < m->d.batch; b++) kv_release(*m, b);
     return OXB_HIP_OK;
 }
 
@@ -788,6 +924,8 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     for (uint32_t b = 0; b < d.batch; b++)
         if (pos[b] >= d.max_seq)
             return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+    for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + 1));
+    OXB_TRY(kv_sync_table(m));
     hipStream_t st = g_rt.stream;
     OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
     OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
@@ -812,6 +950,8 @@ int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t 
     if ((uint64_t)pos_start + n_tokens > d.max_seq)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
                     (unsigned long long)pos_start + n_tokens - 1, d.max_seq);
+    OXB_TRY(kv_reserve(m, seq, (uint64_t)pos_start + n_tokens));
+    OXB_TRY(kv_sync_table(m));
     OXB_TRY(ensure_prefill_buffers(m, n_tokens));
     hipStream_t st = g_rt.stream;
     OXB_TRY_HIP(hipMemcpyAsync(m.pf_hidden, hidden, (size_t)n_tokens * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
@@ -974,6 +1114,8 @@ static int decode_tokens_impl(uint64_t model, uint64_t embedding, const uint32_t
         if ((uint64_t)pos[b] + n_steps > d.max_seq)
             return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos[b],
                         (unsigned long long)pos[b] + n_steps - 1, d.max_seq);
+    for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + n_steps));
+    OXB_TRY(kv_sync_table(m));
     const bool sampled = sp && sp->temperature >= 1e-6f;  // below: greedy (sampling.rs:89-92)
     if (sp) OXB_TRY(check_sampling(*sp));
     if (sampled && !rng_state) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null rng_state");
@@ -1061,6 +1203,8 @@ int oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, con
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
                     (unsigned long long)pos_start + n_tokens - 1, d.max_seq);
     OXB_TRY(check_ids(*e, ids, n_tokens));
+    OXB_TRY(kv_reserve(m, seq, (uint64_t)pos_start + n_tokens));
+    OXB_TRY(kv_sync_table(m));
     OXB_TRY(ensure_prefill_buffers(m, n_tokens));
     OXB_TRY(m.tok_ids.ensure((size_t)n_tokens * 4));
     hipStream_t st = g_rt.stream;

@@ -4,11 +4,15 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include "kv_quant_device.h"
+
 struct OxbPrefillAttnParams {
     const float* q;                   // [M][nq][hd], after QK-norm and RoPE
-    const void *k_cache, *v_cache;    // this sequence's, this layer's cache: [nkv][max_seq][hd], fp16 or one-byte codes
-    const float *k_scale, *v_scale;   // quantised cache: this sequence's, this layer's row scales [nkv][sc_stride]
-    uint32_t kv_mode, sc_stride;      // OXB_KV_* (kv_quant_device.h)
+    const void *k_cache, *v_cache;    // cache rows of hd values each (fp16 or one-byte codes), placed by `kv`
+    const float *k_scale, *v_scale;   // quantised cache: one scale per row
+    uint32_t kv_mode;                 // OXB_KV_* (kv_quant_device.h)
+    OxbKvLayout kv;
+    uint32_t seq, layer;              // whose rows the queries attend to
     uint32_t window, sinks;           // sliding window with attention sinks; window 0 = off
     float* out;                       // [M][nq * hd]
     uint32_t M, pos_start;            // query t sits at position pos_start + t and sees keys 0 .. pos_start + t

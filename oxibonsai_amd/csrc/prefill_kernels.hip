@@ -65,10 +65,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
     const uint32_t qpos = p.pos_start + t_q;
     const uint32_t kv_len = p.pos_start + min((tg * tpw + tpw - 1) * 16 + 15, p.M - 1) + 1;  // keys the workgroup's last query sees
     typedef typename std::conditional<QC, uint8_t, _Float16>::type cache_t;
-    const cache_t* K = reinterpret_cast<const cache_t*>(p.k_cache) + (size_t)kvh * p.max_seq * HD;
-    const cache_t* V = reinterpret_cast<const cache_t*>(p.v_cache) + (size_t)kvh * p.max_seq * HD;
-    const float* Ksc = QC ? p.k_scale + (size_t)kvh * p.sc_stride : nullptr;
-    const float* Vsc = QC ? p.v_scale + (size_t)kvh * p.sc_stride : nullptr;
+    const cache_t* K = reinterpret_cast<const cache_t*>(p.k_cache);
+    const cache_t* V = reinterpret_cast<const cache_t*>(p.v_cache);
+    const float* Ksc = p.k_scale;
+    const float* Vsc = p.v_scale;
+    const bool paged = p.kv.page_table != nullptr;
+    const size_t row0 = paged ? 0 : kv_row(p.kv, p.seq, p.layer, kvh, 0);
+    auto row_of = [&](uint32_t key) -> size_t { return paged ? kv_row(p.kv, p.seq, p.layer, kvh, key) : row0 + key; };
     // sliding window: this query sees [0, sinks) and (qpos - budget, qpos]; the workgroup's earliest query sits at
     // q_first, so no query of it sees a key in [sinks, q_first + 1 - budget): whole 32-key blocks in there are skipped
     const uint32_t budget = p.window > p.sinks ? p.window - p.sinks : 0u;
@@ -110,14 +113,15 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         for (int i = 0; i < PP; i++) {
             const uint32_t id = i * 256 + tid;
             if (PIECES % 256 == 0 || id < (uint32_t)PIECES) {
-                const uint32_t row = min(key0 + id / PPR, kv_len - 1), col = id % PPR;
-                kreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(K + (size_t)row * HD) + col * 16);
-                vreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(V + (size_t)row * HD) + col * 16);
+                const uint32_t col = id % PPR;
+                const size_t row = row_of(min(key0 + id / PPR, kv_len - 1));
+                kreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(K + row * HD) + col * 16);
+                vreg[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(V + row * HD) + col * 16);
                 if constexpr (QC) vsreg[i] = Vsc[row];
             }
         }
         if constexpr (QC)
-            if (tid < 32) ksreg = Ksc[min(key0 + tid, kv_len - 1)];
+            if (tid < 32) ksreg = Ksc[row_of(min(key0 + tid, kv_len - 1))];
     };
     auto stash = [&](int buf) {
 #pragma unroll
@@ -239,7 +243,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
 
 hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st) {
     if (p.M == 0 || p.nq == 0 || p.nkv == 0 || p.nq % p.nkv || p.pos_start + p.M > p.max_seq || p.kv_mode > OXB_KV_FP8_E4M3 ||
-        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)))
+        (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)) || (p.kv.page_table && (p.kv.page_shift < 4 || p.kv.page_shift > 7)))
         return hipErrorInvalidValue;
     const uint32_t G = p.nq / p.nkv, hpw = G % 4u == 0 ? 4u : (G % 2u == 0 ? 2u : 1u), tpw = 4u / hpw;
     const uint32_t n_qt = (p.M + 15u) / 16u, grid = ((n_qt + tpw - 1) / tpw) * (p.nq / hpw);

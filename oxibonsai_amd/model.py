@@ -85,9 +85,15 @@ KV_F16, KV_I8, KV_FP8_E4M3 = 0, 1, 2   # OXB_KV_DTYPE_*
 
 
 class AttentionOptions(C.Structure):
-    """oxb_attention_options: KV cache storage type and SlidingWindowConfig { window_size, sink_tokens }
-    (crates/oxibonsai-model/src/layers/sliding_window.rs:11-43; window_size 0 = no window)."""
-    _fields_ = [("kv_dtype", C.c_int32), ("window_size", C.c_uint32), ("sink_tokens", C.c_uint32)]
+    """oxb_attention_options: KV cache storage type, SlidingWindowConfig { window_size, sink_tokens }
+    (crates/oxibonsai-model/src/layers/sliding_window.rs:11-43; window_size 0 = no window) and the page pool of a paged
+    cache (crates/oxibonsai-model/src/paged_kv_cache.rs; page_size = n_pages = 0: contiguous cache)."""
+    _fields_ = [("kv_dtype", C.c_int32), ("window_size", C.c_uint32), ("sink_tokens", C.c_uint32),
+                ("page_size", C.c_uint32), ("n_pages", C.c_uint32)]
+
+
+class KvPoolInfo(C.Structure):
+    _fields_ = [("page_size", C.c_uint32), ("total_pages", C.c_uint32), ("free_pages", C.c_uint32)]
 
 
 def kv_quantize_rows(kv_dtype: int, rows):
@@ -242,10 +248,30 @@ class HipModel:
     def uses_graph(self) -> bool:
         return bool(self._lib.oxb_hip_model_uses_graph(self.id))
 
-    def set_attention(self, kv_dtype: int = KV_F16, window_size: int = 0, sink_tokens: int = 0):
-        """Long-context options of the attention kernels; changing kv_dtype replaces the cache (start again at 0)."""
-        opt = AttentionOptions(kv_dtype, window_size, sink_tokens)
+    def set_attention(self, kv_dtype: int = KV_F16, window_size: int = 0, sink_tokens: int = 0, page_size: int = 0,
+                      n_pages: int = 0):
+        """Long-context options of the attention kernels; changing kv_dtype or the paging replaces the cache (start
+        again at 0)."""
+        opt = AttentionOptions(kv_dtype, window_size, sink_tokens, page_size, n_pages)
         _check(self._lib.oxb_hip_model_set_attention(self.id, C.byref(opt)))
+
+    def kv_reserve(self, seq: int, n_tokens: int):
+        """PagedKvCache::ensure_capacity: pages for positions 0 .. n_tokens - 1 of a sequence slot."""
+        _check(self._lib.oxb_hip_model_kv_reserve(self.id, seq, n_tokens))
+
+    def kv_release(self, seq: int):
+        """PagedKvCache::drop_sequence: the slot's pages return to the pool."""
+        _check(self._lib.oxb_hip_model_kv_release(self.id, seq))
+
+    def kv_pool(self) -> KvPoolInfo:
+        info = KvPoolInfo()
+        _check(self._lib.oxb_hip_model_kv_pool(self.id, C.byref(info)))
+        return info
+
+    def kv_capacity(self, seq: int) -> int:
+        n = C.c_uint32(0)
+        _check(self._lib.oxb_hip_model_kv_capacity(self.id, seq, C.byref(n)))
+        return int(n.value)
 
     def attention(self) -> AttentionOptions:
         opt = AttentionOptions()

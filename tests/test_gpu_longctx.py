@@ -266,3 +266,126 @@ def test_prefill_with_options_matches_sequential_oracle(backend, mode, window, s
             assert parity_violations(got2, held.forward(more[-1], n + 3 + len(more) - 1), 1e-2) == 0
     finally:
         gpu.close()
+
+
+# ---- paged cache -----------------------------------------------------------------------------------------------
+# Paging moves rows, it does not change arithmetic: the kernels read the same keys in the same order, so a paged run
+# must reproduce the contiguous run bit for bit (which the tests above hold to the oracle), however the pages of the
+# sequences interleave in the pool.
+def _interleaved_decode(gpu, cfg, steps, seed):
+    """Two sequences advancing at different speeds (sequence 1 moves every step, sequence 0 every third), so that
+    their pages alternate irregularly in the pool; returns every step's logits."""
+    out = []
+    p0 = 0
+    for i in range(steps):
+        hidden = np.stack([synth.embedding_rows(seed + b, [(i * 5 + b) % 97], cfg["h"])[0] * 50.0 for b in (0, 1)])
+        got, tok = gpu.forward(hidden, [p0, i])
+        out.append((got.copy(), tok.copy()))
+        if i % 3 == 2:
+            p0 += 1
+    return out
+
+
+@pytest.mark.parametrize("mode,window,sinks", [(KV_F16, 0, 0), (KV_I8, 0, 0), (KV_FP8_E4M3, 20, 2), (KV_F16, 150, 4)])
+@pytest.mark.parametrize("page_size", [16, 32, 64, 128])
+def test_paged_decode_equals_contiguous_bit_for_bit(backend, mode, window, sinks, page_size):
+    cfg = dict(SMALL, fmt=Q1)
+    w = synth.make_model(cfg, 91)
+    gpu = HipModel(backend, cfg, w, batch=2)
+    try:
+        steps = 290
+        gpu.set_attention(mode, window, sinks)
+        want = _interleaved_decode(gpu, cfg, steps, 7)
+        n_pages = -(-steps // page_size) + -(-(steps // 3 + 1) // page_size)     # exactly what the two sequences need
+        gpu.set_attention(mode, window, sinks, page_size, n_pages)
+        o = gpu.attention()
+        assert (o.page_size, o.n_pages) == (page_size, n_pages)
+        got = _interleaved_decode(gpu, cfg, steps, 7)
+        for i, ((gl, gt), (wl, wt)) in enumerate(zip(got, want)):
+            assert np.array_equal(gl, wl) and np.array_equal(gt, wt), i
+        assert gpu.kv_pool().free_pages == 0
+        assert gpu.kv_capacity(1) == -(-steps // page_size) * page_size
+    finally:
+        gpu.close()
+
+
+@pytest.mark.parametrize("mode,window,sinks", [(KV_F16, 0, 0), (KV_I8, 60, 3)])
+@pytest.mark.parametrize("page_size", [16, 128])
+def test_paged_prefill_equals_contiguous_bit_for_bit(backend, mode, window, sinks, page_size):
+    cfg = dict(MID, fmt=TQ2)
+    w = synth.make_model(cfg, 93)
+    gpu = HipModel(backend, cfg, w, batch=2)
+    try:
+        def run():
+            res = []
+            gpu.prefill(_rows(2, 37, cfg["h"]), seq=1)                  # the other slot takes pages first
+            res.append(gpu.prefill(_rows(5, 150, cfg["h"]), seq=0))
+            res.append(gpu.prefill(_rows(3, 61, cfg["h"]), seq=1, pos_start=37))
+            res.append(gpu.prefill(_rows(9, 45, cfg["h"]), seq=0, pos_start=150))
+            hidden = np.stack([_rows(12, 1, cfg["h"])[0], _rows(13, 1, cfg["h"])[0]])
+            res.append(gpu.forward(hidden, [195, 98]))
+            rows = [gpu.read_kv(L, hh, 0, 196, seq=0) for L in range(cfg["n_layers"]) for hh in range(cfg["nkv"])]
+            return res, rows
+        gpu.set_attention(mode, window, sinks)
+        want, want_rows = run()
+        gpu.set_attention(mode, window, sinks, page_size, 2 * (-(-200 // page_size)))
+        got, got_rows = run()
+        for (gl, gt), (wl, wt) in zip(got, want):
+            assert np.array_equal(gl, wl) and np.array_equal(np.asarray(gt), np.asarray(wt))
+        for g, wnt in zip(got_rows, want_rows):
+            assert all(np.array_equal(a, b) for a, b in zip(g, wnt))
+    finally:
+        gpu.close()
+
+
+def test_page_pool_accounting(backend):
+    """The bookkeeping of crates/oxibonsai-model/tests/paged_kv_cache_tests.rs: lazy allocation, capacity in whole
+    pages, exhaustion, pages returning to the pool when a sequence is dropped."""
+    cfg = dict(TINY, fmt=Q1)
+    w = synth.make_model(cfg, 95)
+    gpu = HipModel(backend, cfg, w, batch=3)
+    cpu = oracle.OracleModel(cfg, w, kv_mode=oracle.KV_F16)
+    try:
+        info = gpu.kv_pool()
+        assert (info.page_size, info.total_pages, info.free_pages) == (0, 0, 0)      # contiguous: no pool
+        assert gpu.kv_capacity(0) == cfg["max_seq"]
+        gpu.kv_reserve(0, 5)                                                         # a no-op there
+        gpu.set_attention(KV_F16, 0, 0, 16, 5)
+        info = gpu.kv_pool()
+        assert (info.page_size, info.total_pages, info.free_pages) == (16, 5, 5)
+        assert [gpu.kv_capacity(s) for s in range(3)] == [0, 0, 0]                   # sequences start without pages
+        gpu.kv_reserve(0, 1)
+        assert gpu.kv_capacity(0) == 16 and gpu.kv_pool().free_pages == 4
+        gpu.kv_reserve(0, 16)                                                        # still one page
+        assert gpu.kv_capacity(0) == 16 and gpu.kv_pool().free_pages == 4
+        gpu.kv_reserve(0, 17)
+        assert gpu.kv_capacity(0) == 32 and gpu.kv_pool().free_pages == 3
+        gpu.kv_reserve(1, 48)
+        assert gpu.kv_capacity(1) == 48 and gpu.kv_pool().free_pages == 0
+        with pytest.raises(GpuError) as e:                                           # block_pool_oom / paged_cache_oom_error
+            gpu.kv_reserve(2, 1)
+        assert e.value.kind == "OutOfMemory" and "no free KV blocks" in str(e.value)
+        with pytest.raises(GpuError):
+            gpu.kv_reserve(0, cfg["max_seq"] + 1)
+        with pytest.raises(GpuError):
+            gpu.kv_release(3)
+        # a decode step that needs a page the pool no longer has fails the same way and leaves the model usable
+        hidden = np.stack([synth.embedding_rows(1, [t], cfg["h"])[0] * 50.0 for t in (1, 2, 3)])
+        with pytest.raises(GpuError) as e:
+            gpu.forward(hidden, [0, 0, 0])
+        assert e.value.kind == "OutOfMemory"
+        gpu.kv_release(1)                                                            # drop_sequence frees its blocks
+        assert gpu.kv_pool().free_pages == 3 and gpu.kv_capacity(1) == 0
+        for pos in range(20):                                                        # sequence 2 grows into the freed pages
+            got, _ = gpu.forward(hidden, [pos, 0, pos])
+            want = cpu.forward(hidden[2], pos)
+            assert parity_violations(got[2], want) == 0, pos
+        assert gpu.kv_capacity(2) == 32 and gpu.kv_capacity(1) == 16      # slot 1 wrote position 0 again: one page
+        gpu.reset()                                                                  # every slot's pages go back
+        info = gpu.kv_pool()
+        assert info.free_pages == info.total_pages == 5
+        for bad in (dict(page_size=24, n_pages=4), dict(page_size=16, n_pages=0), dict(page_size=0, n_pages=3), dict(page_size=256, n_pages=2)):
+            with pytest.raises(GpuError):
+                gpu.set_attention(KV_F16, 0, 0, **bad)
+    finally:
+        gpu.close()
