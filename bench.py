@@ -85,7 +85,7 @@ DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd
 
 
 def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32), with_gguf: bool = True,
-               long_context: int = 0) -> dict:
+               long_context: int = 0, long_only: str = "") -> dict:
     """Greedy batch-1 decode of the random-init 8B-shape Q1 model: one batched prefill of `prompt_len` random
     token ids fills the context (timed on its own), then `n_tokens` greedy steps are timed.  The per-token time
     is what the caller of the fused entry point sees: embedding row H2D, the replayed HIP graph (36 layers,
@@ -194,9 +194,15 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
         ml = HipModel(be, dict(cfg, max_seq=long_context + 64), w, batch=1)
         reps = -(-long_context // prompt_len)
         res["long_context"] = []
-        for name, mode, window, sinks in (("fp16 cache", KV_F16, 0, 0), ("int8 cache", KV_I8, 0, 0), ("fp8-e4m3 cache", KV_FP8_E4M3, 0, 0),
-                                          ("fp16 cache, window 4096 + 4 sinks", KV_F16, 4096, 4)):
-            ml.set_attention(mode, window, sinks)
+        n_pages16 = -(-(long_context + 64) // 16)
+        for name, mode, window, sinks, page, pages in (
+                ("fp16 cache", KV_F16, 0, 0, 0, 0), ("int8 cache", KV_I8, 0, 0, 0, 0), ("fp8-e4m3 cache", KV_FP8_E4M3, 0, 0, 0, 0),
+                ("fp16 cache, window 4096 + 4 sinks", KV_F16, 4096, 4, 0, 0),
+                ("fp16 cache in pages of 16 positions", KV_F16, 0, 0, 16, n_pages16),
+                ("int8 cache in pages of 128 positions", KV_I8, 0, 0, 128, -(-(long_context + 64) // 128))):
+            if long_only and name != long_only:
+                continue
+            ml.set_attention(mode, window, sinks, page, pages)
             t0 = time.perf_counter()
             for c in range(reps):       # the prompt rows again and again until the context is full
                 n = min(prompt_len, long_context - c * prompt_len)
@@ -327,6 +333,8 @@ def main() -> int:
     ap.add_argument("--no-gguf", action="store_true", help="skip the checkpoint-file load of the decode leg")
     ap.add_argument("--long-context", type=int, default=32000,
                     help="context of the long-context decode runs (fp16 / int8 / fp8 cache, sliding window); 0 = skip")
+    ap.add_argument("--long-context-only", type=str, default="", help="run only the long-context option of this name")
+    ap.add_argument("--no-ternary", action="store_true", help="skip the ternary 1.7B-shape decode leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build targets one GPU; run with --gpus 1 (multi-GPU sharding is design-only)",
@@ -493,8 +501,9 @@ def main() -> int:
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
                                    tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf,
-                                   args.long_context)
-        out["decode_ternary_1p7b"] = decode_ternary_leg(be, args.decode_context, args.decode_tokens)
+                                   args.long_context, args.long_context_only)
+        if not args.no_ternary:
+            out["decode_ternary_1p7b"] = decode_ternary_leg(be, args.decode_context, args.decode_tokens)
     print(json.dumps(out), flush=True)
     return 0
 

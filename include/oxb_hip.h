@@ -155,9 +155,9 @@ int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is re
  *    offered: its row quantiser turns the row maximum into infinity whenever max / scale rounds above 57344
  *    (quant_fp8.rs:229-231), about one row in five.
  *  - paged cache: PagedKvCache / BlockPool / BlockTable (crates/oxibonsai-model/src/paged_kv_cache.rs:70-160, 187-236,
- *    294-345).  The cache is a pool of n_pages pages of page_size positions (DEFAULT_BLOCK_SIZE = 16, :33); a page holds
- *    those positions for every layer and kv head ([layer][kv_head][position][hd], where the reference allocates one
- *    page per layer in lockstep), so one table of page numbers per sequence serves all layers.  The model's `batch`
+ *    294-345).  The cache is a pool of n_pages pages of page_size positions (DEFAULT_BLOCK_SIZE = 16, :33); a page number
+ *    stands for those positions in every layer and kv head (device rows [layer][kv_head][page][position][hd], where the
+ *    reference allocates one page per layer in lockstep), so one table of page numbers per sequence serves all layers.  The model's `batch`
  *    sequence slots take the place of the reference's sequence ids.  Pages are handed out lazily: decode and prefill
  *    calls reserve what the positions they write need, as write_kv does (:447-470); when the pool is empty they fail
  *    with OXB_HIP_OUT_OF_MEMORY ("out of memory: no free KV blocks", PagedKvError::OutOfMemory) and the pages taken

@@ -18,19 +18,21 @@
 
 // Where the rows of a KV cache lie.  Contiguous: [sequence][layer][kv_head][row_stride] rows (row_stride = the context
 // rounded up to a whole number of 128-position attention chunks).  Paged (PagedKvCache / BlockTable,
-// crates/oxibonsai-model/src/paged_kv_cache.rs:187-236, 294-345): a pool of pages of 2^page_shift positions each,
-// [page][layer][kv_head][position in page] rows, and per sequence a table of physical page numbers indexed by
-// position >> page_shift.  A row index addresses both the data (row * head_dim elements) and the row scales.
+// crates/oxibonsai-model/src/paged_kv_cache.rs:187-236, 294-345): a pool of n_pages pages of 2^page_shift positions
+// each, [layer][kv_head][page][position in page] rows - the pages of one (layer, head) lie side by side, so a walk
+// over a sequence stays inside n_pages * page bytes of address space, as it does in the contiguous cache - and per
+// sequence a table of physical page numbers indexed by position >> page_shift.  A row index addresses both the data
+// (row * head_dim elements) and the row scales.
 struct OxbKvLayout {
     const uint32_t* page_table;  // null: contiguous
-    uint32_t page_shift, table_stride;
+    uint32_t page_shift, table_stride, n_pages;
     uint32_t n_layers, nkv, row_stride;
 };
 #if defined(__HIPCC__)
 __device__ __forceinline__ size_t kv_row(const OxbKvLayout& L, uint32_t seq, uint32_t layer, uint32_t kvh, uint32_t pos) {
     if (L.page_table) {
         const uint32_t page = L.page_table[(size_t)seq * L.table_stride + (pos >> L.page_shift)];
-        return ((((size_t)page * L.n_layers + layer) * L.nkv + kvh) << L.page_shift) + (pos & ((1u << L.page_shift) - 1u));
+        return ((((size_t)layer * L.nkv + kvh) * L.n_pages + page) << L.page_shift) + (pos & ((1u << L.page_shift) - 1u));
     }
     return (((size_t)seq * L.n_layers + layer) * L.nkv + kvh) * L.row_stride + pos;
 }

@@ -264,7 +264,7 @@ typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 //  * sliding window with attention sinks (is_in_window, crates/oxibonsai-model/src/layers/sliding_window.rs:173-189):
 //    the first `sinks` keys stay visible, the others while pos - key < window - sinks; chunks without a visible key
 //    are not walked.  window == 0: every key up to pos is visible.
-template <int HD, int KVM>
+template <int HD, int KVM, bool OPT>  // OPT: a window and / or a paged cache may be in use (else neither costs anything)
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p) {
     constexpr bool QC = KVM != OXB_KV_F16;
     constexpr int KS = HD / 32, NS = HD / 16, VSTR = HD + 8;
@@ -282,9 +282,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     const uint32_t n_chunks = (seq_len + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK;
     if (slot >= n_chunks) return;  // never read by the merge
     // visible keys: [0, sink_n) and [lo, seq_len)
-    const uint32_t budget = p.window > p.sinks ? p.window - p.sinks : 0u;
-    const uint32_t lo = p.window ? (seq_len > budget ? seq_len - budget : 0u) : 0u;
-    const uint32_t sink_n = p.window ? min(p.sinks, seq_len) : 0u;
+    const uint32_t window = OPT ? p.window : 0u;
+    const uint32_t budget = window > p.sinks ? window - p.sinks : 0u;
+    const uint32_t lo = window ? (seq_len > budget ? seq_len - budget : 0u) : 0u;
+    const uint32_t sink_n = window ? min(p.sinks, seq_len) : 0u;
     const uint32_t sink_chunks = (sink_n + OXB_ATTN_CHUNK - 1) / OXB_ATTN_CHUNK, lo_chunk = lo / OXB_ATTN_CHUNK;
     auto next_needed = [&](uint32_t c) {  // first chunk >= c of this slot's walk that holds a visible key
         if (c >= sink_chunks && c < lo_chunk) c += (lo_chunk - c + p.n_splits - 1) / p.n_splits * p.n_splits;
@@ -313,11 +314,28 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     cache_t* Vc = reinterpret_cast<cache_t*>(p.v_cache);
     float* Ksc = p.k_scale;  // one scale per row
     float* Vsc = p.v_scale;
-    // row of a position of this (sequence, layer, kv head): an offset in a contiguous cache, a table lookup in a paged
-    // one (four consecutive positions from a multiple of four never straddle a page: pages hold 16 positions or more)
-    const bool paged = p.kv.page_table != nullptr;
-    const size_t row0 = paged ? 0 : kv_row(p.kv, b, p.layer, kvh, 0);
-    auto row_of = [&](uint32_t key) -> size_t { return paged ? kv_row(p.kv, b, p.layer, kvh, key) : row0 + key; };
+    // Row of a position of this (sequence, layer, kv head): an offset in a contiguous cache; in a paged one the page
+    // number comes from the sequence's table.  Pages hold 16 positions or more, so the 32 keys of a wave's block lie in
+    // at most two pages - those of keys key0 .. key0 + 15 and key0 + 16 .. key0 + 31, the same for every lane - which
+    // are looked up (one broadcast load each) one chunk before the rows are requested, so that no row load waits for
+    // a lookup.  (Keeping the table in LDS instead was measured slower: the 8 KB cost a workgroup per CU.)
+    const bool paged = OPT && p.kv.page_table != nullptr;
+    const uint32_t pshift = p.kv.page_shift, pmask = (1u << pshift) - 1u;
+    const size_t row0 = paged ? ((size_t)(p.layer * p.nkv + kvh) * p.kv.n_pages) << pshift : kv_row(p.kv, b, p.layer, kvh, 0);
+    const uint32_t* tbl = paged ? p.kv.page_table + (size_t)b * p.kv.table_stride : nullptr;  // covers whole chunks
+    auto pages_of = [&](uint32_t chunk, uint32_t& pa, uint32_t& pb) {
+        pa = pb = 0;
+        if (!paged) return;
+        const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave, i0 = key0 >> pshift, i1 = (key0 + 16) >> pshift;
+        pa = (uint32_t)__builtin_amdgcn_readfirstlane((int)tbl[i0]);
+        pb = (uint32_t)__builtin_amdgcn_readfirstlane((int)tbl[i1]);
+    };
+    // key: a position of the block that starts at key0 (or, for a block past the end, the last position, whose row
+    // is then read from a wrong but existing page: such a block is masked as a whole)
+    auto row_of = [&](uint32_t key, uint32_t key0, uint32_t pa, uint32_t pb) -> size_t {
+        if (!paged) return row0 + key;
+        return row0 + ((size_t)(((key - key0) & 16u) ? pb : pa) << pshift) + (key & pmask);
+    };
 
     // K rows of the two 16-key tiles (A operands) and this lane's pieces of the 32-key V block of a chunk.
     // Rows past the last key repeat it; their scores are masked.
@@ -325,9 +343,9 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     kvi2_t k0q[QC ? KS : 1], k1q[QC ? KS : 1];
     float4 ksc0, ksc1, vsc0, vsc1;  // row scales of the lane's keys 4g .. 4g+3 and 16+4g .. 16+4g+3
     v4i vr[VL];
-    auto load_k = [&](uint32_t chunk) {
+    auto load_k = [&](uint32_t chunk, uint32_t pa, uint32_t pb) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
-        const size_t kr0 = row_of(min(key0 + qi, seq_len - 1)), kr1 = row_of(min(key0 + 16 + qi, seq_len - 1));
+        const size_t kr0 = row_of(min(key0 + qi, seq_len - 1), key0, pa, pb), kr1 = row_of(min(key0 + 16 + qi, seq_len - 1), key0, pa, pb);
 #pragma unroll
         for (int s = 0; s < KS; s++) {
             if constexpr (QC) {
@@ -339,21 +357,21 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             }
         }
         if constexpr (QC) {  // scales of positions past the last key are never used (their scores are masked)
-            ksc0 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u)));
-            ksc1 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u)));
+            ksc0 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u), key0, pa, pb));
+            ksc1 = *reinterpret_cast<const float4*>(Ksc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u), key0, pa, pb));
         }
     };
-    auto load_v = [&](uint32_t chunk) {
+    auto load_v = [&](uint32_t chunk, uint32_t pa, uint32_t pb) {
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
 #pragma unroll
         for (int i = 0; i < VL; i++) {
             const uint32_t id = i * 64 + lane, col = id % VPR;
-            const size_t row = row_of(min(key0 + id / VPR, seq_len - 1));
+            const size_t row = row_of(min(key0 + id / VPR, seq_len - 1), key0, pa, pb);
             vr[i] = *reinterpret_cast<const v4i*>(reinterpret_cast<const uint8_t*>(Vc + row * HD) + col * 16);
         }
         if constexpr (QC) {
-            vsc0 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u)));
-            vsc1 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u)));
+            vsc0 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 4 * g, (seq_len - 1) & ~3u), key0, pa, pb));
+            vsc1 = *reinterpret_cast<const float4*>(Vsc + row_of(min(key0 + 16 + 4 * g, (seq_len - 1) & ~3u), key0, pa, pb));
         }
     };
 
@@ -372,7 +390,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     }
     // --- K and V of the new position, by the workgroup whose slot walks its chunk (wave 0 and wave 1) ---
-    const size_t new_row = row_of(pos);
+    const size_t new_row = kv_row(p.kv, b, p.layer, kvh, pos);
     if (owner) {
         if (wave == 0) {
             const float* in = qkv + (size_t)(p.nq + kvh) * HD;
@@ -442,9 +460,14 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     }
     __syncthreads();  // publishes qs and, within this workgroup, the new cache rows
+    uint32_t na = 0, nb = 0;  // pages of the chunk whose rows are requested next
     if (first < n_chunks) {
-        load_k(first);
-        load_v(first);
+        uint32_t pa, pb;
+        pages_of(first, pa, pb);
+        load_k(first, pa, pb);
+        load_v(first, pa, pb);
+        const uint32_t second = next_needed(first + p.n_splits);
+        if (second < n_chunks) pages_of(second, na, nb);
     }
 
     // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo
@@ -490,7 +513,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             }
         }
         const float4 vc0 = vsc0, vc1 = vsc1;
-        if (more) load_v(nxt);
+        if (more) load_v(nxt, na, nb);
         v4f s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int s = 0; s < KS; s++) {
@@ -508,7 +531,11 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             s1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a1, ql[s], s1, 0, 0, 0);
         }
         const float4 kc0 = ksc0, kc1 = ksc1;
-        if (more) load_k(nxt);
+        if (more) {
+            load_k(nxt, na, nb);
+            const uint32_t after = next_needed(nxt + p.n_splits);
+            if (after < n_chunks) pages_of(after, na, nb);  // used by the next iteration's requests
+        }
         // this wave's quarter of the chunk holds no visible key (past the end, or outside the window)
         if (!(key0 < sink_n || max(key0, lo) < min(key0 + 32, seq_len))) continue;
         // this lane: head qi, keys key0 + 4g + v and key0 + 16 + 4g + v
@@ -810,18 +837,26 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
         (p.kv.page_table ? (p.kv.page_shift < 4 || p.kv.page_shift > 7) : (p.kv.row_stride % OXB_ATTN_CHUNK != 0 || p.kv.row_stride < p.max_seq)))
         return hipErrorInvalidValue;
     const dim3 grid(p.n_splits, p.nkv, batch), block(256);
+    const bool opt = p.window != 0 || p.kv.page_table != nullptr;
     switch (p.hd) {
-#define OXB_ATTN_CASE(HD_)                                                                                                  \
-    case HD_:                                                                                                            \
-        if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_I8>), grid, block, 0, st, p);  \
-        else if (p.kv_mode == OXB_KV_FP8_E4M3)                                                                           \
-            hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_FP8_E4M3>), grid, block, 0, st, p);                  \
-        else hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, OXB_KV_F16>), grid, block, 0, st, p);                      \
+#define OXB_ATTN_LAUNCH(HD_, KVM_)                                                                                   \
+    if (opt) hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, KVM_, true>), grid, block, 0, st, p);                 \
+    else hipLaunchKernelGGL((attn_decode_fused_kernel<HD_, KVM_, false>), grid, block, 0, st, p);
+#define OXB_ATTN_CASE(HD_)                                         \
+    case HD_:                                                      \
+        if (p.kv_mode == OXB_KV_I8) {                              \
+            OXB_ATTN_LAUNCH(HD_, OXB_KV_I8)                        \
+        } else if (p.kv_mode == OXB_KV_FP8_E4M3) {                 \
+            OXB_ATTN_LAUNCH(HD_, OXB_KV_FP8_E4M3)                  \
+        } else {                                                   \
+            OXB_ATTN_LAUNCH(HD_, OXB_KV_F16)                       \
+        }                                                          \
         break;
         OXB_ATTN_CASE(32)
         OXB_ATTN_CASE(64)
         OXB_ATTN_CASE(128)
         OXB_ATTN_CASE(256)
+#undef OXB_ATTN_LAUNCH
 #undef OXB_ATTN_CASE
         default: return hipErrorInvalidValue;
     }

@@ -229,6 +229,7 @@ static OxbKvLayout kv_layout(const Model& m) {
     L.page_table = m.n_pages ? m.d_table : nullptr;
     L.page_shift = m.page_shift;
     L.table_stride = m.table_stride;
+    L.n_pages = m.n_pages;
     L.n_layers = m.d.n_layers;
     L.nkv = m.d.nkv;
     L.row_stride = m.row_stride;
@@ -581,7 +582,7 @@ static int alloc_kv_cache(Model& m, uint32_t kv_mode, uint32_t page_size, uint32
         while ((1u << shift) < page_size) shift++;
         m.page_shift = shift;
         m.n_pages = n_pages;
-        m.table_stride = (d.max_seq + page_size - 1) / page_size;
+        m.table_stride = m.row_stride / page_size;   // whole attention chunks: the kernels look up every block of a chunk
         m.h_table.assign((size_t)d.batch * m.table_stride, 0u);   // entries of unreserved blocks name page 0: never read
         m.seq_pages.assign(d.batch, {});
         m.free_pages.resize(n_pages);
@@ -786,7 +787,7 @@ int oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t
             const size_t blk = p0 >> m->page_shift;
             if (blk >= pg.size())
                 return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u of sequence %u lies outside its %zu pages", p0, seq, pg.size());
-            row = ((((size_t)pg[blk] * d.n_layers + layer) * d.nkv + kv_head) << m->page_shift) + (p0 & (run_max - 1));
+            row = ((((size_t)layer * d.nkv + kv_head) * m->n_pages + pg[blk]) << m->page_shift) + (p0 & (run_max - 1));
         } else {
             row = (((size_t)seq * d.n_layers + layer) * d.nkv + kv_head) * m->row_stride + p0;
         }

@@ -41,7 +41,7 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 // numbers on their way into LDS, V already multiplied by its row scale there, the K row scale multiplies the
 // score) and a sliding window with attention sinks (key visible to the query at qpos iff key < sinks or
 // qpos - key < window - sinks; blocks no query of the workgroup can see are skipped).
-template <int HD, int KVM>
+template <int HD, int KVM, bool OPT>  // OPT: a window and / or a paged cache may be in use (else neither costs anything)
 __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams p, uint32_t hpw) {
     constexpr bool QC = KVM != OXB_KV_F16;
     constexpr int KS = HD / 32, NS = HD / 16;
@@ -69,15 +69,16 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
     const cache_t* V = reinterpret_cast<const cache_t*>(p.v_cache);
     const float* Ksc = p.k_scale;
     const float* Vsc = p.v_scale;
-    const bool paged = p.kv.page_table != nullptr;
+    const bool paged = OPT && p.kv.page_table != nullptr;
+    const uint32_t window = OPT ? p.window : 0u;
     const size_t row0 = paged ? 0 : kv_row(p.kv, p.seq, p.layer, kvh, 0);
     auto row_of = [&](uint32_t key) -> size_t { return paged ? kv_row(p.kv, p.seq, p.layer, kvh, key) : row0 + key; };
     // sliding window: this query sees [0, sinks) and (qpos - budget, qpos]; the workgroup's earliest query sits at
     // q_first, so no query of it sees a key in [sinks, q_first + 1 - budget): whole 32-key blocks in there are skipped
-    const uint32_t budget = p.window > p.sinks ? p.window - p.sinks : 0u;
+    const uint32_t budget = window > p.sinks ? window - p.sinks : 0u;
     const uint32_t q_first = p.pos_start + tg * tpw * 16;
-    const uint32_t skip_from = p.window ? (p.sinks + 31u) & ~31u : 0u;
-    const uint32_t skip_to = p.window && q_first + 1 > budget ? (q_first + 1 - budget) & ~31u : 0u;
+    const uint32_t skip_from = window ? (p.sinks + 31u) & ~31u : 0u;
+    const uint32_t skip_to = window && q_first + 1 > budget ? (q_first + 1 - budget) & ~31u : 0u;
     auto next_block = [&](uint32_t key0) {  // the block after key0 that some query may see
         key0 += 32;
         return key0 >= skip_from && key0 < skip_to ? skip_to : key0;
@@ -188,8 +189,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
 #pragma unroll
         for (int v = 0; v < 4; v++) {
             const uint32_t ka = key0 + 4 * g + v, kb_ = ka + 16;
-            const bool va = ka <= qpos && (!p.window || ka < p.sinks || qpos - ka < budget);
-            const bool vb_ = kb_ <= qpos && (!p.window || kb_ < p.sinks || qpos - kb_ < budget);
+            const bool va = ka <= qpos && (!window || ka < p.sinks || qpos - ka < budget);
+            const bool vb_ = kb_ <= qpos && (!window || kb_ < p.sinks || qpos - kb_ < budget);
             sv[v] = va ? s0[v] : -INFINITY;
             sv[4 + v] = vb_ ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
@@ -247,18 +248,26 @@ hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st
         return hipErrorInvalidValue;
     const uint32_t G = p.nq / p.nkv, hpw = G % 4u == 0 ? 4u : (G % 2u == 0 ? 2u : 1u), tpw = 4u / hpw;
     const uint32_t n_qt = (p.M + 15u) / 16u, grid = ((n_qt + tpw - 1) / tpw) * (p.nq / hpw);
+    const bool opt = p.window != 0 || p.kv.page_table != nullptr;
     switch (p.hd) {
-#define OXB_PF_CASE(HD_)                                                                                                          \
-    case HD_:                                                                                                                    \
-        if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_I8>), dim3(grid), dim3(256), 0, st, p, hpw); \
-        else if (p.kv_mode == OXB_KV_FP8_E4M3)                                                                                   \
-            hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_FP8_E4M3>), dim3(grid), dim3(256), 0, st, p, hpw);                \
-        else hipLaunchKernelGGL((attn_prefill_kernel<HD_, OXB_KV_F16>), dim3(grid), dim3(256), 0, st, p, hpw);                    \
+#define OXB_PF_LAUNCH(HD_, KVM_)                                                                                     \
+    if (opt) hipLaunchKernelGGL((attn_prefill_kernel<HD_, KVM_, true>), dim3(grid), dim3(256), 0, st, p, hpw);        \
+    else hipLaunchKernelGGL((attn_prefill_kernel<HD_, KVM_, false>), dim3(grid), dim3(256), 0, st, p, hpw);
+#define OXB_PF_CASE(HD_)                                           \
+    case HD_:                                                      \
+        if (p.kv_mode == OXB_KV_I8) {                              \
+            OXB_PF_LAUNCH(HD_, OXB_KV_I8)                          \
+        } else if (p.kv_mode == OXB_KV_FP8_E4M3) {                 \
+            OXB_PF_LAUNCH(HD_, OXB_KV_FP8_E4M3)                    \
+        } else {                                                   \
+            OXB_PF_LAUNCH(HD_, OXB_KV_F16)                         \
+        }                                                          \
         break;
         OXB_PF_CASE(32)
         OXB_PF_CASE(64)
         OXB_PF_CASE(128)
         OXB_PF_CASE(256)
+#undef OXB_PF_LAUNCH
 #undef OXB_PF_CASE
         default: return hipErrorInvalidValue;
     }
