@@ -283,8 +283,8 @@ def test_attention_slots_walk_several_chunks(backend):
 @pytest.mark.parametrize("fmt", [TQ2, Q1])
 def test_wide_ffn_takes_four_row_tiles_per_workgroup(backend, fmt):
     """An intermediate size of 8192 gives the gate || up product 1024 row tiles: the narrow GEMM then takes four per
-    workgroup (two gate tiles with their up tiles) and the prefill GEMM its widest SwiGLU tiling - the tilings the
-    8B-shape model runs with - on a model small enough for the oracle."""
+    workgroup (two gate tiles with their up tiles) and the prefill GEMM its SwiGLU tiling (one gate / up pair per wave)
+    - the tilings the 8B-shape model runs with - on a model small enough for the oracle."""
     cfg = dict(fmt=fmt, n_layers=1, h=256, inter=8192, nq=4, nkv=2, hd=64, vocab=128, max_seq=96, eps=1e-6, rope_theta=1e6)
     w = synth.make_model(cfg, 17 + fmt)
     for B in (9, 20):
