@@ -29,17 +29,6 @@ __device__ __forceinline__ float block_sum(float v, float* red) {  // two barrie
     return s;
 }
 
-__device__ __forceinline__ float block_max(float v, float* red) {  // of non-negative values; same protocol
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = 0.f;
-    for (uint32_t i = 0; i < (blockDim.x >> 6); i++) s = fmaxf(s, red[i]);
-    __syncthreads();
-    return s;
-}
-
 // ---------------------------------------------------------------------------
 // RMSNorm fused with the activation quantiser (rms_norm: crates/oxibonsai-kernels/src/
 // simd_float_ops.rs:204-215; GPU twin rmsnorm_weighted_v2, gpu_backend/cuda_kernels.rs:335-374).
@@ -140,71 +129,118 @@ __global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const 
 // Per-head QK-RMSNorm + half-split RoPE + KV store (fp16, or quantised rows: kv_quant_device.h)
 // (fused_qk_norm_rope + fused_kv_store, gpu_backend/cuda_attn_kernels.rs:160-251;
 //  CPU: block/types/forward.rs:179-213, rope pairs (d, d + hd/2) simd_float_ops.rs:240-253).
-// Grid (nq + nkv, batch); block = 128 threads.  Q heads go to q_rope (fp32), K heads (after RoPE)
-// and the raw V head go to the cache at position pos[b], rounded to f16 (round-to-nearest-even).
-// Cache layout: [seq][layer][kv_head][max_seq][hd], K and V in separate arrays.
+// Grid (head groups, rows); block = 256 threads = 4 waves, a wave takes OXB_QK_HEADS_PER_WAVE heads of one row one
+// after the other: a lane holds the rotation pairs (d, d + hd/2) for d = lane, lane + 64, every reduction stays inside
+// the wave.  Q heads go to q_rope (fp32), K heads (after RoPE) and the raw V head go to the cache row of position
+// pos[b], rounded to f16 (round-to-nearest-even) or quantised.
 // ---------------------------------------------------------------------------
+#define OXB_QK_HEADS_PER_WAVE 2
 template <int KVM>
-__global__ __launch_bounds__(128) void qk_norm_rope_store_kernel(OxbQkParams p) {
+__global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(OxbQkParams p) {
     constexpr bool QC = KVM != OXB_KV_F16;
-    __shared__ float red[2];
-    const uint32_t head = blockIdx.x, b = blockIdx.y, tid = threadIdx.x, hd = p.hd, half = hd >> 1;
-    const bool is_q = head < p.nq;
-    const uint32_t hh = is_q ? head : head - p.nq;
-    const float* in = p.qkv + (size_t)b * p.qkv_stride + (is_q ? (size_t)hh * hd : (size_t)(p.nq + hh) * hd);
-    const float* w = is_q ? p.q_norm : p.k_norm;
+    constexpr int KI = 2, VI = 4;  // pairs / values per lane at head_dim 256
+    const uint32_t b = blockIdx.y, lane = threadIdx.x & 63u, hd = p.hd, half = hd >> 1;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const uint32_t pos = p.pos ? p.pos[b] : p.pos_base + b;
     const uint32_t seq = p.pos ? b : p.seq;
-    float ss = 0.f;
-    for (uint32_t d = tid; d < hd; d += 128) ss += in[d] * in[d];
-    ss = block_sum(ss, red);
-    const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
-    const float* cs = p.cos_t + (size_t)pos * half;
-    const float* sn = p.sin_t + (size_t)pos * half;
-    const size_t row = is_q ? 0 : kv_row(p.kv, seq, p.layer, hh, pos);
-    const size_t cache_off = row * hd;
-    // head_dim <= 256: a thread owns at most one rotation pair and two V values
-    float o_lo = 0.f, o_hi = 0.f;
-    if (tid < half) {
-        const float lo = w[tid] * in[tid] * inv_rms, hi = w[tid + half] * in[tid + half] * inv_rms;
-        const float c = cs[tid], s = sn[tid];
-        o_lo = lo * c - hi * s;
-        o_hi = lo * s + hi * c;
+    const float* row_in = p.qkv + (size_t)b * p.qkv_stride;
+    float cs[KI], sn[KI];
+#pragma unroll
+    for (int it = 0; it < KI; it++) {
+        const uint32_t d = lane + 64 * it;
+        cs[it] = d < half ? p.cos_t[(size_t)pos * half + d] : 0.f;
+        sn[it] = d < half ? p.sin_t[(size_t)pos * half + d] : 0.f;
     }
-    if (is_q) {
-        if (tid < half) {
+    const uint32_t head0 = (blockIdx.x * 4 + wave) * OXB_QK_HEADS_PER_WAVE;
+#pragma unroll
+    for (uint32_t j = 0; j < OXB_QK_HEADS_PER_WAVE; j++) {
+        const uint32_t head = head0 + j;
+        if (head >= p.nq + p.nkv) break;  // wave-uniform
+        const bool is_q = head < p.nq;
+        const uint32_t hh = is_q ? head : head - p.nq;
+        const float* in = row_in + (size_t)head * hd;  // q heads, then k heads
+        const float* w = is_q ? p.q_norm : p.k_norm;
+        float lo[KI], hi[KI], ss = 0.f;
+#pragma unroll
+        for (int it = 0; it < KI; it++) {
+            const uint32_t d = lane + 64 * it;
+            lo[it] = d < half ? in[d] : 0.f;
+            hi[it] = d < half ? in[d + half] : 0.f;
+            ss = fmaf(lo[it], lo[it], fmaf(hi[it], hi[it], ss));
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
+        float o_lo[KI], o_hi[KI], kmax = 0.f;
+#pragma unroll
+        for (int it = 0; it < KI; it++) {
+            const uint32_t d = lane + 64 * it;
+            const float a = d < half ? w[d] * lo[it] * inv_rms : 0.f, c = d < half ? w[d + half] * hi[it] * inv_rms : 0.f;
+            o_lo[it] = a * cs[it] - c * sn[it];
+            o_hi[it] = a * sn[it] + c * cs[it];
+            kmax = fmaxf(kmax, fmaxf(fabsf(o_lo[it]), fabsf(o_hi[it])));
+        }
+        if (is_q) {
             float* q = p.q_rope + ((size_t)b * p.nq + hh) * hd;
-            q[tid] = o_lo;
-            q[tid + half] = o_hi;
+#pragma unroll
+            for (int it = 0; it < KI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < half) q[d] = o_lo[it], q[d + half] = o_hi[it];
+            }
+            continue;
         }
-        return;
-    }
-    const float* v = p.qkv + (size_t)b * p.qkv_stride + (size_t)(p.nq + p.nkv + hh) * hd;
-    const float v0 = tid < hd ? v[tid] : 0.f, v1 = tid + 128 < hd ? v[tid + 128] : 0.f;
-    if constexpr (QC) {
-        uint8_t* kc = reinterpret_cast<uint8_t*>(p.k_cache) + cache_off;
-        uint8_t* vc = reinterpret_cast<uint8_t*>(p.v_cache) + cache_off;
-        const float ks = kv_row_scale<KVM>(block_max(fmaxf(fabsf(o_lo), fabsf(o_hi)), red));
-        const float vs = kv_row_scale<KVM>(block_max(fmaxf(fabsf(v0), fabsf(v1)), red));
-        if (tid < half) {
-            kc[tid] = (uint8_t)kv_encode<KVM>(o_lo, ks);
-            kc[tid + half] = (uint8_t)kv_encode<KVM>(o_hi, ks);
+        const size_t row = kv_row(p.kv, seq, p.layer, hh, pos), cache_off = row * hd;
+        const float* v = row_in + (size_t)(p.nq + p.nkv + hh) * hd;
+        float vv[VI], vmax = 0.f;
+#pragma unroll
+        for (int it = 0; it < VI; it++) {
+            const uint32_t d = lane + 64 * it;
+            vv[it] = d < hd ? v[d] : 0.f;
+            vmax = fmaxf(vmax, fabsf(vv[it]));
         }
-        if (tid < hd) vc[tid] = (uint8_t)kv_encode<KVM>(v0, vs);
-        if (tid + 128 < hd) vc[tid + 128] = (uint8_t)kv_encode<KVM>(v1, vs);
-        if (tid == 0) {
-            p.k_scale[row] = ks;
-            p.v_scale[row] = vs;
+        if constexpr (QC) {
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) {
+                kmax = fmaxf(kmax, __shfl_xor(kmax, o, 64));
+                vmax = fmaxf(vmax, __shfl_xor(vmax, o, 64));
+            }
+            const float ks = kv_row_scale<KVM>(kmax), vs = kv_row_scale<KVM>(vmax);
+            uint8_t* kc = reinterpret_cast<uint8_t*>(p.k_cache) + cache_off;
+            uint8_t* vc = reinterpret_cast<uint8_t*>(p.v_cache) + cache_off;
+#pragma unroll
+            for (int it = 0; it < KI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < half) {
+                    kc[d] = (uint8_t)kv_encode<KVM>(o_lo[it], ks);
+                    kc[d + half] = (uint8_t)kv_encode<KVM>(o_hi[it], ks);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < VI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < hd) vc[d] = (uint8_t)kv_encode<KVM>(vv[it], vs);
+            }
+            if (lane == 0) {
+                p.k_scale[row] = ks;
+                p.v_scale[row] = vs;
+            }
+        } else {
+            __half* kc = reinterpret_cast<__half*>(p.k_cache) + cache_off;
+            __half* vc = reinterpret_cast<__half*>(p.v_cache) + cache_off;
+#pragma unroll
+            for (int it = 0; it < KI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < half) {
+                    kc[d] = __float2half_rn(o_lo[it]);
+                    kc[d + half] = __float2half_rn(o_hi[it]);
+                }
+            }
+#pragma unroll
+            for (int it = 0; it < VI; it++) {
+                const uint32_t d = lane + 64 * it;
+                if (d < hd) vc[d] = __float2half_rn(vv[it]);
+            }
         }
-    } else {
-        __half* kc = reinterpret_cast<__half*>(p.k_cache) + cache_off;
-        __half* vc = reinterpret_cast<__half*>(p.v_cache) + cache_off;
-        if (tid < half) {
-            kc[tid] = __float2half_rn(o_lo);
-            kc[tid + half] = __float2half_rn(o_hi);
-        }
-        if (tid < hd) vc[tid] = __float2half_rn(v0);
-        if (tid + 128 < hd) vc[tid + 128] = __float2half_rn(v1);
     }
 }
 
@@ -823,7 +859,8 @@ hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, u
 
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st) {
     if (p.hd > 256 || p.kv_mode > OXB_KV_FP8_E4M3 || (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
-    const dim3 grid(p.nq + p.nkv, batch), block(128);
+    const uint32_t per_wg = 4 * OXB_QK_HEADS_PER_WAVE;
+    const dim3 grid((p.nq + p.nkv + per_wg - 1) / per_wg, batch), block(256);
     if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_I8>, grid, block, 0, st, p);
     else if (p.kv_mode == OXB_KV_FP8_E4M3) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_FP8_E4M3>, grid, block, 0, st, p);
     else hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_F16>, grid, block, 0, st, p);
