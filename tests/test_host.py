@@ -135,3 +135,31 @@ def test_device_arithmetic_model_reference_generators_and_outliers():
     assert np.all(kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 256), 16, 256, np.zeros(256, np.float32)) == 0)
     x[3] = np.inf
     assert np.all(np.isnan(kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 16, 256), 16, 256, x)))
+
+
+def test_ctypes_structs_match_the_header_layout(tmp_path):
+    """Size and field offsets of every struct of the C ABI, as a C compiler sees the header, against the ctypes
+    mirrors the Python host side passes across the boundary."""
+    import shutil
+    import subprocess
+    from oxibonsai_amd import model as M
+    mirrors = {"oxb_layer_ids": M._LayerIds, "oxb_model_desc": M._ModelDesc, "oxb_gguf_info": M.GgufInfo,
+               "oxb_sampling": M.Sampling, "oxb_attention_options": M.AttentionOptions, "oxb_kv_pool_info": M.KvPoolInfo}
+    cc = shutil.which("gcc") or shutil.which("cc")
+    if not cc:
+        pytest.skip("no C compiler")
+    lines = ['#include <stdio.h>', '#include <stddef.h>', '#include "oxb_hip.h"', 'int main(void) {']
+    for cname, cls in mirrors.items():
+        lines.append(f'  printf("{cname} %zu\\n", sizeof({cname}));')
+        for fname, _ in cls._fields_:
+            lines.append(f'  printf("{cname}.{fname} %zu\\n", offsetof({cname}, {fname}));')
+    lines += ['  return 0;', '}']
+    src = tmp_path / "layout.c"
+    src.write_text("\n".join(lines))
+    exe = tmp_path / "layout"
+    subprocess.run([cc, "-std=c99", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    seen = dict(l.split() for l in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.splitlines())
+    for cname, cls in mirrors.items():
+        assert int(seen[cname]) == C.sizeof(cls), cname
+        for fname, _ in cls._fields_:
+            assert int(seen[f"{cname}.{fname}"]) == getattr(cls, fname).offset, (cname, fname)
