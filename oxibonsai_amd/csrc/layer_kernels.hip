@@ -151,7 +151,9 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(OxbQkParams p) 
         cs[it] = d < half ? p.cos_t[(size_t)pos * half + d] : 0.f;
         sn[it] = d < half ? p.sin_t[(size_t)pos * half + d] : 0.f;
     }
-    const uint32_t head0 = (blockIdx.x * 4 + wave) * OXB_QK_HEADS_PER_WAVE;
+    // without a q_rope buffer only the K and V heads are handled (the consumer of Q does its own norm + RoPE)
+    const uint32_t first_head = p.q_rope ? 0u : p.nq;
+    const uint32_t head0 = first_head + (blockIdx.x * 4 + wave) * OXB_QK_HEADS_PER_WAVE;
 #pragma unroll
     for (uint32_t j = 0; j < OXB_QK_HEADS_PER_WAVE; j++) {
         const uint32_t head = head0 + j;
@@ -860,7 +862,7 @@ hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, u
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st) {
     if (p.hd > 256 || p.kv_mode > OXB_KV_FP8_E4M3 || (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
     const uint32_t per_wg = 4 * OXB_QK_HEADS_PER_WAVE;
-    const dim3 grid((p.nq + p.nkv + per_wg - 1) / per_wg, batch), block(256);
+    const dim3 grid(((p.q_rope ? p.nq : 0u) + p.nkv + per_wg - 1) / per_wg, batch), block(256);
     if (p.kv_mode == OXB_KV_I8) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_I8>, grid, block, 0, st, p);
     else if (p.kv_mode == OXB_KV_FP8_E4M3) hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_FP8_E4M3>, grid, block, 0, st, p);
     else hipLaunchKernelGGL(qk_norm_rope_store_kernel<OXB_KV_F16>, grid, block, 0, st, p);

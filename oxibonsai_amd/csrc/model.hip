@@ -68,7 +68,7 @@ struct Model {
     std::vector<void*> allocs;
     // prefill activations for up to pf_cap token rows (allocated on first use)
     uint32_t pf_cap = 0;
-    float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_q = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
+    float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
     std::vector<void*> pf_allocs;
     GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
     // a model loaded from a file owns the weights it uploaded
@@ -410,7 +410,7 @@ static int ensure_prefill_buffers(Model& m, uint32_t rows) {
     m.pf_cap = 0;
     const oxb_model_desc& d = m.d;
     const size_t R = (rows + 127u) / 128u * 128u, qd = (size_t)d.nq * d.hd, qkv_rows = qd + 2 * (size_t)d.nkv * d.hd;
-    struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_qkv, R * qkv_rows}, {&m.pf_q, R * qd},
+    struct { float** p; size_t n; } bufs[] = {{&m.pf_hidden, R * d.h}, {&m.pf_qkv, R * qkv_rows},
                                              {&m.pf_attn, R * qd},    {&m.pf_gu, R * d.inter}};
     for (auto& b : bufs) {
         if (hipMalloc((void**)b.p, b.n * sizeof(float)) != hipSuccess) {
@@ -454,7 +454,7 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.pos = nullptr;
         qp.pos_base = pos_start;
         qp.seq = seq;
-        qp.q_rope = m.pf_q;
+        qp.q_rope = nullptr;  // the attention kernel norms and rotates Q itself
         qp.k_cache = m.k_cache;
         qp.v_cache = m.v_cache;
         qp.k_scale = m.k_scale;
@@ -470,7 +470,12 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         qp.eps = d.eps;
         OXB_TRY_HIP(oxb_launch_qk_norm_rope_store(qp, M, st), "kernel launch failed: qk_norm_rope_store");
         OxbPrefillAttnParams ap;
-        ap.q = m.pf_q;
+        ap.qkv = m.pf_qkv;
+        ap.qkv_stride = qkv_rows;
+        ap.q_norm = q_norm;
+        ap.cos_t = m.cos_t;
+        ap.sin_t = m.sin_t;
+        ap.eps = d.eps;
         ap.k_cache = m.k_cache;
         ap.v_cache = m.v_cache;
         ap.k_scale = m.k_scale;

@@ -7,7 +7,11 @@
 #include "kv_quant_device.h"
 
 struct OxbPrefillAttnParams {
-    const float* q;                   // [M][nq][hd], after QK-norm and RoPE
+    const float* qkv;                 // [M][qkv_stride]: the raw projections, q heads first (QK-norm and RoPE happen in the kernel)
+    uint32_t qkv_stride;
+    const float* q_norm;              // [hd]
+    const float *cos_t, *sin_t;       // [max_seq][hd/2]
+    float eps;
     const void *k_cache, *v_cache;    // cache rows of hd values each (fp16 or one-byte codes), placed by `kv`
     const float *k_scale, *v_scale;   // quantised cache: one scale per row
     uint32_t kv_mode;                 // OXB_KV_* (kv_quant_device.h)

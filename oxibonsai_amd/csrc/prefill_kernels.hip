@@ -84,21 +84,63 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         return key0 >= skip_from && key0 < skip_to ? skip_to : key0;
     };
 
+    // Q of this lane's query: per-head RMSNorm, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd)
+    // (fused_qk_norm_rope, gpu_backend/cuda_attn_kernels.rs:160-226), then split into fp16 hi + lo.  The lane holds
+    // elements 32 s + 8 g + e; for hd >= 64 both elements of a pair are its own (steps s and s + KS / 2), for hd = 32
+    // the partner sits in lane g ^ 2.
     v8h qh[KS], ql[KS];
     {
-        const float* qr = p.q + ((size_t)t_q * p.nq + head) * HD + 8 * g;
+        constexpr int half = HD / 2;
+        const float* qr = p.qkv + (size_t)t_q * p.qkv_stride + (size_t)head * HD + 8 * g;
+        float x[KS][8], ss = 0.f;
 #pragma unroll
         for (int s = 0; s < KS; s++) {
             const float4 a = *reinterpret_cast<const float4*>(qr + 32 * s), b = *reinterpret_cast<const float4*>(qr + 32 * s + 4);
             const float f[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
 #pragma unroll
             for (int e = 0; e < 8; e++) {
-                const float x = f[e] * p.scale;
-                const _Float16 hi = (_Float16)x;
-                qh[s][e] = hi;
-                ql[s][e] = (_Float16)(x - (float)hi);
+                x[s][e] = f[e];
+                ss = fmaf(f[e], f[e], ss);
             }
         }
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) x[s][e] = p.q_norm[32 * s + 8 * g + e] * x[s][e] * inv;
+        const float* cs = p.cos_t + (size_t)qpos * half;
+        const float* sn = p.sin_t + (size_t)qpos * half;
+        float r[KS][8];
+        if constexpr (KS >= 2) {
+#pragma unroll
+            for (int s = 0; s < KS / 2; s++)
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int d = 32 * s + 8 * (int)g + e;  // < half
+                    const float lo = x[s][e], hi = x[s + KS / 2][e], c = cs[d], sv = sn[d];
+                    r[s][e] = lo * c - hi * sv;
+                    r[s + KS / 2][e] = lo * sv + hi * c;
+                }
+        } else {  // hd = 32: lanes g = 0, 1 hold the first half, g = 2, 3 the second
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float mine = x[0][e], other = __shfl_xor(mine, 32, 64);
+                const int d = 8 * (int)(g & 1u) + e;
+                const float c = cs[d], sv = sn[d];
+                r[0][e] = g < 2 ? mine * c - other * sv : other * sv + mine * c;
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < KS; s++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const float v = r[s][e] * p.scale;
+                const _Float16 hi = (_Float16)v;
+                qh[s][e] = hi;
+                ql[s][e] = (_Float16)(v - (float)hi);
+            }
     }
     v4f O[NS];
 #pragma unroll
@@ -243,7 +285,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
 }
 
 hipError_t oxb_launch_attn_prefill(const OxbPrefillAttnParams& p, hipStream_t st) {
-    if (p.M == 0 || p.nq == 0 || p.nkv == 0 || p.nq % p.nkv || p.pos_start + p.M > p.max_seq || p.kv_mode > OXB_KV_FP8_E4M3 ||
+    if (p.M == 0 || p.nq == 0 || p.nkv == 0 || p.nq % p.nkv || !p.qkv || !p.q_norm || !p.cos_t || !p.sin_t || p.pos_start + p.M > p.max_seq || p.kv_mode > OXB_KV_FP8_E4M3 ||
         (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)) || (p.kv.page_table && (p.kv.page_shift < 4 || p.kv.page_shift > 7)))
         return hipErrorInvalidValue;
     const uint32_t G = p.nq / p.nkv, hpw = G % 4u == 0 ? 4u : (G % 2u == 0 ? 2u : 1u), tpw = 4u / hpw;
