@@ -119,7 +119,7 @@ typedef struct {
     const oxb_layer_ids* layers;   /* [n_layers], read during the call only */
     uint64_t final_norm, lm_head;
 } oxb_model_desc;
-/* Allocates the FP16 KV cache [batch][layer][kv_head][max_seq][hd] (CudaKvCache, KG/cuda_full_layer/mod.rs:112-139),
+/* Allocates the FP16 KV cache [batch][layer][kv_head][max_seq rounded up to 128][hd] (CudaKvCache, KG/cuda_full_layer/mod.rs:112-139),
  * the activation buffers (mod.rs:149-181) and the RoPE table (crates/oxibonsai-model/src/layers/rope.rs:27-48). */
 int  oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model);
 int  oxb_hip_model_reset(uint64_t model);
@@ -150,7 +150,7 @@ int  oxb_hip_model_uses_graph(uint64_t model);   /* 1 once the decode step is re
  *    QuantizedKvLayer / quantize_row_i8 (crates/oxibonsai-model/src/kv_cache_quant.rs:46-62, 98-195),
  *    OXB_KV_DTYPE_FP8_E4M3 follows Fp8KvLayer / quantize_row_fp8 with Fp8KvFormat::E4M3 (:502-540) and
  *    fp8_e4m3_encode (crates/oxibonsai-core/src/quant_fp8.rs:47-160); attention reads code * scale (:69-71, :545-556).
- *    Device layout: codes [batch][layer][kv_head][max_seq][hd] (head-major, where the reference's layer keeps
+ *    Device layout: codes [batch][layer][kv_head][max_seq rounded up to 128][hd] (head-major, where the reference's layer keeps
  *    [token][head][dim]), scales [batch][layer][kv_head][max_seq rounded up to 128].  Fp8KvFormat::E5M2 is not
  *    offered: its row quantiser turns the row maximum into infinity whenever max / scale rounds above 57344
  *    (quant_fp8.rs:229-231), about one row in five.
