@@ -559,6 +559,21 @@ int oxb_hip_free_f32(uint64_t id) {
     return OXB_HIP_OK;
 }
 
+// Slots of the split-KV attention: about one workgroup (slot x kv head x sequence) per CU for the fp16 cache, two for a
+// quantised one (widening the codes adds arithmetic that a second resident workgroup hides), no more: every slot pays
+// the Q arithmetic and a merge, and walks its chunks with a prefetch.  Measured, 8B shape: four per CU are slower
+// everywhere (batch 8 at context 2048 by 12 %, batch 16 by 7 %, one sequence at context 32 000 by 3 %); two per CU
+// gain 4 % at batch 32 with the INT8 cache and lose 1-3 % with the fp16 cache.
+static uint32_t attn_slots(const Model& m, uint32_t kv_mode) {
+    const oxb_model_desc& d = m.d;
+    uint32_t n = (d.max_seq + m.chunk - 1) / m.chunk;
+    const uint32_t per_cu = kv_mode == OXB_KV_F16 ? 1u : 2u;
+    const uint32_t want = (per_cu * g_rt.n_cus + d.nkv * d.batch - 1) / (d.nkv * d.batch);
+    if (n > want) n = want;
+    if (n > OXB_ATTN_MAX_SPLITS) n = OXB_ATTN_MAX_SPLITS;
+    return n;
+}
+
 // (Re)allocates the KV cache in the given storage form, contiguous (n_pages 0) or as a pool of n_pages pages of
 // page_size positions.  Row scales start at 0 so that a row never written reads as zeros.  A contiguous head holds a
 // whole number of attention chunks of rows, which keeps the kernels' 16-byte scale loads aligned and inside it.
@@ -639,19 +654,14 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     if (rc) return rc;
 
     m.chunk = OXB_ATTN_CHUNK_POSITIONS;
-    // Slots of the split-KV attention: about one workgroup (slot x kv head x sequence) per CU, no more: every slot pays
-    // the Q arithmetic and a merge, and walks its chunks with a prefetch.  (Four per CU measured slower everywhere:
-    // batch 8 at context 2048 by 12 %, batch 16 by 7 %, one sequence at context 32 000 by 3 %.)
-    m.n_splits = (d.max_seq + m.chunk - 1) / m.chunk;
-    const uint32_t want = (g_rt.n_cus + d.nkv * d.batch - 1) / (d.nkv * d.batch);
-    if (m.n_splits > want) m.n_splits = want;
-    if (m.n_splits > OXB_ATTN_MAX_SPLITS) m.n_splits = OXB_ATTN_MAX_SPLITS;
+    m.n_splits = attn_slots(m, OXB_KV_F16);
+    const uint32_t max_slots = attn_slots(m, OXB_KV_I8);  // what any cache type may ask for: sizes the slot results
     const size_t B = d.batch;
     uint32_t kmax = d.h > d.inter ? d.h : d.inter;
     if (qd > kmax) kmax = qd;
     const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
     if ((rc = dev_alloc(m, (void**)&m.hidden, B * d.h * 4)) || (rc = dev_alloc(m, (void**)&m.qkv, B * qkv_rows * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * m.n_splits * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * max_slots * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
         (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
@@ -751,6 +761,7 @@ int oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt
             return rc;
         }
     }
+    m->n_splits = attn_slots(*m, m->kv_mode);
     m->window = opt->window_size;
     m->sinks = opt->sink_tokens;
     return OXB_HIP_OK;
