@@ -35,6 +35,7 @@ struct OxbAttnParams {
     OxbKvLayout kv;                      // contiguous (row_stride a multiple of the chunk, >= max_seq) or paged (pages of 16..128 positions)
     uint32_t window, sinks;              // sliding window with attention sinks; window 0 = off
     float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
+    float* out_single;                   // optional, n_splits == 1 only: [batch][nq*hd] receives the finished output (no merge launch)
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
     float scale;                         // 1 / sqrt(hd)

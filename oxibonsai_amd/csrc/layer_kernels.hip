@@ -674,6 +674,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             o = fmaf(mo[(w * 16 + h) * HD + d], wgt, o);
             l = fmaf(ml[w * 16 + h], wgt, l);
         }
+        if (p.out_single) {  // the only slot: what the merge would compute (weight 1, times 1 / sum)
+            p.out_single[((size_t)b * p.nq + h0 + h) * HD + d] = o * (l > 0.f ? 1.0f / l : 0.f);
+            continue;
+        }
         part[h * part_head + d] = o;
         if (d == 0) {
             part[h * part_head + HD] = M;
@@ -871,7 +875,7 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
     if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
-        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 ||
+        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 || (p.out_single && p.n_splits != 1) ||
         (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)) ||
         (p.kv.page_table ? (p.kv.page_shift < 4 || p.kv.page_shift > 7) : (p.kv.row_stride % OXB_ATTN_CHUNK != 0 || p.kv.row_stride < p.max_seq)))
         return hipErrorInvalidValue;

@@ -275,7 +275,8 @@ static int kv_sync_table(Model& m) {
 
 // QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch, one launch; leaves the
 // slot results in m.attn_part and the parameters the merge needs in *ap.
-static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out) {
+static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out,
+                                   float* out_single = nullptr) {
     const oxb_model_desc& d = m.d;
     OxbAttnParams ap;
     ap.qkv = m.qkv;
@@ -294,6 +295,7 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.window = m.window;
     ap.sinks = m.sinks;
     ap.part = m.attn_part;
+    ap.out_single = out_single;
     ap.pos = m.pos;
     ap.nq = d.nq;
     ap.nkv = d.nkv;
@@ -332,9 +334,13 @@ static int encode_decode_step_gemm(Model& m) {
         if (rc) return rc;
         OXB_TRY(gemm_device(*wqkv, m.hidden, d.h, m.qkv, B, qkv_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, attn_norm, d.eps, &m.gws));
         OxbAttnParams ap;
-        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
-        OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
-                    "kernel launch failed: attn_combine");
+        if (m.n_splits == 1) {  // one slot per sequence: the attention kernel finishes its output itself
+            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap, m.attn_out));
+        } else {
+            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
+            OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
+                        "kernel launch failed: attn_combine");
+        }
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
         // SwiGLU in the epilogue of the gate || up product
         OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));

@@ -251,13 +251,15 @@ def test_full_size_shapes_match_oracle(backend, name, cfg):
         gpu.close()
 
 
-def test_attention_slots_walk_several_chunks(backend):
-    """Many sequences leave few attention slots per sequence (here two: 8 kv heads x 16 sequences on 256 CUs), so that
-    a slot walks several 128-position chunks of the KV sequence with the next chunk's keys and values already
-    requested: positions 600..602 span five chunks, slot 0 takes chunks 0, 2, 4 and slot 1 chunks 1, 3."""
+@pytest.mark.parametrize("B", [16, 32])
+def test_attention_slots_walk_several_chunks(backend, B):
+    """Many sequences leave few attention slots per sequence, so that a slot walks several 128-position chunks of the
+    KV sequence with the next chunk's keys and values already requested.  16 sequences x 8 kv heads on 256 CUs: two
+    slots - positions 600..602 span five chunks, slot 0 takes chunks 0, 2, 4 and slot 1 chunks 1, 3.  32 sequences:
+    one slot walks all five, and the attention kernel finishes its output itself (no merge launch)."""
     cfg = dict(fmt=TQ2, n_layers=2, h=512, inter=1024, nq=16, nkv=8, hd=64, vocab=512, max_seq=700, eps=1e-6, rope_theta=1e6)
     w = synth.make_model(cfg, 91)
-    B, n = 16, 600
+    n = 600
     gpu = HipModel(backend, cfg, w, batch=B)
     ctx = [synth.embedding_rows(200 + s, [(5 * i + s) % 251 for i in range(n)], cfg["h"]) * 50.0 for s in (0, 1)]
     cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in (0, 1)]
