@@ -98,6 +98,29 @@ def test_device_sampler_matches_restatement(backend, n, T, k, tp):
 
 
 @pytest.mark.gpu
+def test_device_sampler_orders_signs_zeros_ties_and_infinities(backend):
+    # the selection compares the logits as integer keys: negative numbers, both zeros, -inf and long runs of equal
+    # values must come out in the order the restatement's (value descending, index ascending) sort gives
+    from oxibonsai_amd.model import sample_logits
+    n, k = 6000, 64
+    base = np.round(synth.normal_f32(3, 4 * n).reshape(4, n) * 3.0) / 2.0      # half-integers: many exact ties
+    base[0, ::7] = -np.inf
+    base[1] = -np.abs(base[1]) - 1.0                                             # all negative
+    base[2, :] = 0.0
+    base[2, 1::2] = -0.0                                                        # only zeros of both signs
+    base[3, :] = -np.inf
+    base[3, [5, 4097, 2048]] = [-2.0, -2.0, -7.5]                                # three finite candidates
+    seeds = np.array([2**63 + 5, 12345678901234567, 0x9E3779B97F4A7C15, 42424242424242], dtype=np.uint64)
+    toks, states = sample_logits(base.astype(np.float32), 1.0, k, 1.0, seeds)
+    for b in range(4):
+        tok, new, ids, p, r = oracle.sample(base[b].astype(np.float32), 1.0, k, 1.0, int(seeds[b]))
+        assert int(states[b]) == new
+        if int(toks[b]) != tok:
+            cum = np.cumsum(p.astype(np.float64))
+            assert int(toks[b]) in ids and np.min(np.abs(cum - r)) < 1e-5, (b, int(toks[b]), tok)
+
+
+@pytest.mark.gpu
 def test_device_sampler_statistics_and_errors(backend):
     from oxibonsai_amd import GpuError
     from oxibonsai_amd.model import sample_logits
