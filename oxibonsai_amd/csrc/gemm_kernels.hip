@@ -371,6 +371,10 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
                                                      (int)xoff[it], (int)soff, 0, 0);
     };
     auto publish = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
+    // In the blocks that also request the next superblock's weights, those 3 RT loads are issued after the stage's
+    // loads (memory reads return in order) and stay in flight across the barrier: they come from HBM and have until
+    // the end of the following block, instead of stalling the whole workgroup at the end of this one.
+    auto publish_keep_weights = [&]() { asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * RT) : "memory"); };
 
     HalfRegs<FMT> H[RT][2];
     stage_x(sb0 * 4, xs0);
@@ -398,6 +402,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
         publish();
         // block 1: half 0 is consumed; reload it for the next superblock
         stage_x(sb * 4 + 2, xs0);
+        __builtin_amdgcn_sched_barrier(0);  // the stage's loads first, then the weights (see publish_keep_weights)
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             bd[rt] = bdn[rt];
@@ -405,8 +410,9 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
         }
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
+        __builtin_amdgcn_sched_barrier(0);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
-        publish();
+        publish_keep_weights();
         // block 2
         stage_x(sb * 4 + 3, xs1);
 #pragma unroll
@@ -418,6 +424,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
         publish();
         // block 3: half 1 is consumed; the next block is block 0 of the next superblock (half 0, already reloaded)
         stage_x(sb * 4 + 4, xs0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             bd[rt] = bdn[rt];
@@ -425,8 +432,9 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
         }
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
+        __builtin_amdgcn_sched_barrier(0);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
-        publish();
+        publish_keep_weights();
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) bd[rt] = bdn[rt];
     }
