@@ -333,6 +333,40 @@ def prefill_gemm_leg(be, L, torch, m_tokens: int = 512) -> dict:
     return res
 
 
+def measure_launch_context(torch, stream, nbytes: int, copies: int) -> dict:
+    """What any launch of this size costs on this GPU, to read roofline.frac against: a kernel that does next to
+    nothing, and a device copy that moves the same number of bytes (half read, half written), each replayed from a
+    HIP graph of `copies` launches over rotating buffers - the way the GEMV itself is timed."""
+    tiny = torch.zeros(64, device="cuda")
+    half = nbytes // 8
+    src = [torch.ones(half, dtype=torch.float32, device="cuda") for _ in range(copies)]
+    dst = [torch.empty(half, dtype=torch.float32, device="cuda") for _ in range(copies)]
+
+    def timed(fn) -> float:
+        for i in range(3):
+            fn(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=stream):
+            for i in range(copies):
+                fn(i)
+        g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(8):
+            g.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / (8 * copies)
+
+    empty_us = timed(lambda i: tiny.add_(1.0))
+    copy_us = timed(lambda i: dst[i].copy_(src[i]))
+    return {"near_empty_kernel_us": round(empty_us, 3), "device_copy_same_bytes_us": round(copy_us, 3),
+            "device_copy_GB/s": round(half * 8 / (copy_us * 1e-6) / 1e9, 1),
+            "note": "torch elementwise kernels in a replayed HIP graph; the copy moves the GEMV's algorithmic byte count"}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -485,6 +519,8 @@ def main() -> int:
     for h in c0_ids:
         be.free_weights(h)
 
+    launch_context = measure_launch_context(torch, stream, kbytes, args.copies)
+
     out = {
         "metric": "quant GEMV HBM GB/s", "value": round(value, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 6),
@@ -497,7 +533,7 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
                      "kernel": "gemv_mfma_kernel<Q1> gate||up 24576x4096", "bytes_per_launch": kbytes,
-                     "avg_launch_us": round(avg_us.value, 3), "per_kernel": per_kernel,
+                     "avg_launch_us": round(avg_us.value, 3), "launch_context": launch_context, "per_kernel": per_kernel,
                      "per_kernel_cache_resident": cache_resident},
     }
     if not args.no_cpu:
