@@ -165,6 +165,25 @@ def test_gemm_prefill_shape_q1_8b_gate_up(backend):
     assert np.max(np.abs(got[rows] - want)) < 3e-3 * np.sqrt(np.mean(want.astype(np.float64) ** 2))
 
 
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+def test_gemm_prefill_shape_8b_qkv_2048_tokens(backend, fmt):
+    """6144 x 4096 at 2048 tokens: the shape the planner gives three row tiles per wave, whose weight loads stay in
+    flight across the block barrier.  A sample of rows against the CPU restatement, equal token rows in different
+    token tiles and workgroups must give equal output rows, and the whole result is finite."""
+    m, n, k = 2048, 6144, 4096
+    a = synth.make_blocks(fmt, 8100 + fmt, n, k)
+    x = synth.normal_f32(8101, m * k).reshape(m, k).copy()
+    x[1999] = x[3]
+    x[1024] = x[127]
+    got = _gemm(backend, fmt, a, x, m, n, k)
+    rows = [0, 3, 127, 128, 1023, 1500, 2047]
+    want = oracle.simd_gemm(fmt, a, np.ascontiguousarray(x[rows]), len(rows), n, k)
+    assert parity_violations(got[rows], want, GEMM_REL_TOL) == 0
+    assert np.max(np.abs(got[rows] - want)) < 3e-3 * np.sqrt(np.mean(want.astype(np.float64) ** 2))
+    assert np.array_equal(got[1999], got[3]) and np.array_equal(got[1024], got[127])
+    assert np.all(np.isfinite(got))
+
+
 def test_trait_gemm_paths(backend):
     # the trait-level call: m <= 16 takes the fp32-exact route, larger m the matrix cores
     n, k = 64, 512
