@@ -442,25 +442,33 @@ uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top
     if (n_cand) *n_cand = 0;
     if (n == 0) return 0;
     if (temperature < 1e-6f) return oxb_argmax_last(logits, n);
-    size_t k = (top_k > 0 && top_k < n) ? top_k : n;
+    const int filtered = top_k > 0 && top_k < n;
+    size_t k = filtered ? top_k : n;
     uint32_t* idx = (uint32_t*)malloc(k * sizeof(uint32_t));
     float* p = (float*)malloc(k * sizeof(float));
-    unsigned char* taken = (unsigned char*)calloc(n, 1);
-    /* k largest scaled values in descending order, ties by ascending index (selection; n * k compares) */
-    for (size_t j = 0; j < k; j++) {
-        size_t best = n;
-        float bv = 0.0f;
-        for (size_t i = 0; i < n; i++) {
-            if (taken[i]) continue;
-            const float v = logits[i] / temperature;
-            if (best == n || v > bv) best = i, bv = v;
+    float max_val = -INFINITY;
+    if (filtered) {
+        /* sampling.rs:111-118 keeps the k largest in the order select_nth_unstable_by leaves them, which is
+         * implementation-defined; here: descending, ties by ascending index (selection; n * k compares) */
+        unsigned char* taken = (unsigned char*)calloc(n, 1);
+        for (size_t j = 0; j < k; j++) {
+            size_t best = n;
+            float bv = 0.0f;
+            for (size_t i = 0; i < n; i++) {
+                if (taken[i]) continue;
+                const float v = logits[i] / temperature;
+                if (best == n || v > bv) best = i, bv = v;
+            }
+            taken[best] = 1;
+            idx[j] = (uint32_t)best;
+            p[j] = bv;
         }
-        taken[best] = 1;
-        idx[j] = (uint32_t)best;
-        p[j] = bv;
+        free(taken);
+    } else {
+        /* top-k off (or k >= n): the buffer stays in index order (sampling.rs:98-104) */
+        for (size_t i = 0; i < n; i++) idx[i] = (uint32_t)i, p[i] = logits[i] / temperature;
     }
-    free(taken);
-    const float max_val = p[0];
+    for (size_t j = 0; j < k; j++) max_val = fmaxf(max_val, p[j]);  /* fold(NEG_INFINITY, f32::max), :121-125 */
     float sum = 0.0f;
     for (size_t j = 0; j < k; j++) {
         p[j] = expf(p[j] - max_val);
@@ -468,6 +476,28 @@ uint32_t oxb_sample(const float* logits, size_t n, float temperature, size_t top
     }
     for (size_t j = 0; j < k; j++) p[j] /= sum;
     if (top_p < 1.0f) {
+        if (!filtered) {
+            /* sort_by(|a, b| b.1.partial_cmp(&a.1)) is a stable sort (:136-137): descending probability, equal
+             * probabilities keep index order.  Bottom-up merge sort. */
+            uint32_t* ti = (uint32_t*)malloc(k * sizeof(uint32_t));
+            float* tp = (float*)malloc(k * sizeof(float));
+            for (size_t w = 1; w < k; w *= 2) {
+                for (size_t lo = 0; lo < k; lo += 2 * w) {
+                    const size_t mid = lo + w < k ? lo + w : k, hi = lo + 2 * w < k ? lo + 2 * w : k;
+                    size_t a = lo, b = mid, o = lo;
+                    while (a < mid && b < hi) {
+                        if (p[b] > p[a]) tp[o] = p[b], ti[o++] = idx[b++];
+                        else tp[o] = p[a], ti[o++] = idx[a++];
+                    }
+                    while (a < mid) tp[o] = p[a], ti[o++] = idx[a++];
+                    while (b < hi) tp[o] = p[b], ti[o++] = idx[b++];
+                }
+                float* sp = p; p = tp; tp = sp;
+                uint32_t* si = idx; idx = ti; ti = si;
+            }
+            free(ti);
+            free(tp);
+        }
         float cum = 0.0f;
         size_t cutoff = k ? k - 1 : 0;
         for (size_t j = 0; j < k; j++) {

@@ -42,9 +42,13 @@ def test_generator_and_draw():
         assert new == _xorshift(st)
         assert r == np.float32(np.float64(new) / np.float64(2**64 - 1))
         st = new
-    # a zero state stays zero: the draw is 0 and the first candidate wins
+    # a zero state stays zero: the draw is 0 and the first entry of the buffer wins - with top-k and top-p off the
+    # buffer is still in index order (:98-104; no select, no sort), so that is token 0, not the most likely one
     tok, new, ids, *_ = oracle.sample([0.0, 5.0, 1.0], 1.0, 0, 1.0, 0)
-    assert new == 0 and tok == 1
+    assert new == 0 and tok == 0 and list(ids) == [0, 1, 2]
+    # top-p on: the stable descending sort (:136-137) puts the most likely token first
+    tok, new, ids, *_ = oracle.sample([0.0, 5.0, 1.0], 1.0, 0, 0.999, 0)
+    assert new == 0 and tok == 1 and list(ids) == [1, 2, 0]
 
 
 def test_candidates_follow_the_definition():
@@ -71,6 +75,52 @@ def test_candidates_follow_the_definition():
         tok, st, *_ = oracle.sample(lg, 1.0, 0, 1.0, st)
         counts[tok] += 1
     assert np.max(np.abs(counts / counts.sum() - want)) < 0.01
+
+
+def test_unfiltered_path_follows_the_definition():
+    """top_k = 0 (the Creative preset, presets.rs:57-63): softmax over the whole vocabulary summed in index order,
+    stable descending sort for top-p, cumulative cut, renormalisation, pick - against numpy with the same f32 sums."""
+    n, T, tp = 5000, 1.0, 0.95
+    logits = (synth.normal_f32(11, n) * 2.0).astype(np.float32)
+    logits[17] = logits[4000] = logits[3]                       # equal probabilities keep index order in the sort
+    tok, new, ids, p, r = oracle.sample(logits, T, 0, tp, 0x9E3779B97F4A7C15)
+    scaled = logits / np.float32(T)
+    e = np.exp((scaled - scaled.max()).astype(np.float32)).astype(np.float32)
+    s = np.float32(0.0)
+    for v in e:
+        s = np.float32(s + v)
+    prob = (e / s).astype(np.float32)
+    order = np.argsort(-prob.astype(np.float64), kind="stable")
+    cum, cut = np.float32(0.0), n - 1
+    for j, i in enumerate(order):
+        cum = np.float32(cum + prob[i])
+        if cum > np.float32(tp):
+            cut = j
+            break
+    assert list(ids) == list(order[:cut + 1])
+    s2 = np.float32(0.0)
+    for i in order[:cut + 1]:
+        s2 = np.float32(s2 + prob[i])
+    want = (prob[order[:cut + 1]] / s2).astype(np.float32)
+    assert np.max(np.abs(p - want)) <= 1.2e-7 * float(want.max())      # libm expf against numpy's exp: last place
+    cum = np.float32(0.0)
+    pick = ids[0]
+    for i, q in zip(ids, p):
+        cum = np.float32(cum + q)
+        if r <= cum:
+            pick = i
+            break
+    assert tok == pick
+    # top-p off as well: index order throughout
+    tok, _, ids, p, r = oracle.sample(logits, T, 0, 1.0, 777)
+    assert list(ids) == list(range(n))
+    cum, pick = np.float32(0.0), 0
+    for i, q in enumerate(p):
+        cum = np.float32(cum + q)
+        if r <= cum:
+            pick = i
+            break
+    assert tok == pick and pick != int(np.argmax(logits))       # an ordinary draw lands somewhere in the middle
 
 
 # --------------------------------------------------------------------------- GPU
