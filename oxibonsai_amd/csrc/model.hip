@@ -1112,10 +1112,11 @@ static int model_and_embedding(uint64_t model, uint64_t embedding, Model** m, Em
     return OXB_HIP_OK;
 }
 
-static int check_sampling(const oxb_sampling& sp) {
+static int check_sampling(const oxb_sampling& sp, uint32_t vocab) {
     if (!(sp.temperature >= 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: temperature %g", (double)sp.temperature);
-    if (sp.temperature >= 1e-6f && (sp.top_k == 0 || sp.top_k > OXB_SAMPLE_MAX_TOP_K))
-        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_k %u (the device sampler takes 1..%u; sample on the host from the logits otherwise)",
+    // top_k = 0 or >= the vocabulary switches the filter off (sampling.rs:111): the whole-vocabulary route
+    if (sp.temperature >= 1e-6f && sp.top_k > OXB_SAMPLE_MAX_TOP_K && sp.top_k < vocab)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_k %u (the device sampler takes 1..%u, or 0 for no filter; sample on the host from the logits otherwise)",
                     sp.top_k, OXB_SAMPLE_MAX_TOP_K);
     if (!(sp.top_p > 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_p %g", (double)sp.top_p);
     return OXB_HIP_OK;
@@ -1141,7 +1142,7 @@ static int decode_tokens_impl(uint64_t model, uint64_t embedding, const uint32_t
     for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + n_steps));
     OXB_TRY(kv_sync_table(m));
     const bool sampled = sp && sp->temperature >= 1e-6f;  // below: greedy (sampling.rs:89-92)
-    if (sp) OXB_TRY(check_sampling(*sp));
+    if (sp) OXB_TRY(check_sampling(*sp, d.vocab));
     if (sampled && !rng_state) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null rng_state");
     OXB_TRY(m.tok_hist.ensure((size_t)n_steps * d.batch * 4));
     hipStream_t st = g_rt.stream;
@@ -1186,7 +1187,7 @@ int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, c
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!logits || !params || !rng_state || !tokens_out || vocab == 0 || batch == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or empty logits");
-    OXB_TRY(check_sampling(*params));
+    OXB_TRY(check_sampling(*params, vocab));
     if ((vocab + 2047u) / 2048u > 256u) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u logits per row (at most 524288)", vocab);
     OXB_TRY(ensure_init());
     const size_t lb = (size_t)batch * vocab * 4, wb = oxb_sample_ws_bytes(vocab, batch);

@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
+#include <hipcub/hipcub.hpp>
 
 #include "device_utils.h"
 #include "token_kernels.h"
@@ -237,6 +238,152 @@ __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restric
     tokens[row] = tok;
 }
 
+// ---------------------------------------------------------------------------
+// Sampler::sample with top-k off (top_k = 0 or >= the vocabulary: the Creative preset, presets.rs:57-63).  The
+// reference then works on the whole vocabulary in index order (sampling.rs:98-104): softmax with the sum taken
+// element by element in f32 (:121-133), for top-p a stable descending sort (:136-137), the cumulative cut and the
+// renormalising sum again element by element (:138-152), and the cumulative pick (:160-171).  f32 addition is not
+// associative and over 150 000 nearly equal probabilities the order of the additions decides which token a draw
+// lands on, so every one of these sums runs here as one chain in the reference's order (one wave per row: 64
+// elements per load, added lane by lane); only the element-wise steps and the sort are parallel.
+// ---------------------------------------------------------------------------
+#define OXB_FULL_SPAN 2048u
+
+__device__ __forceinline__ float block_max_256(float v, float* sm4) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    if ((threadIdx.x & 63u) == 0) sm4[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return fmaxf(fmaxf(sm4[0], sm4[1]), fmaxf(sm4[2], sm4[3]));  // f32::max semantics: a NaN operand is dropped
+}
+
+__global__ __launch_bounds__(256) void full_max_kernel(const float* __restrict__ logits, uint32_t n, float* __restrict__ pmax) {
+    __shared__ float sm4[4];
+    const float* v = logits + (size_t)blockIdx.y * n;
+    float mx = -INFINITY;
+    for (uint32_t i = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; i < min(n, (blockIdx.x + 1) * OXB_FULL_SPAN); i += 256) mx = fmaxf(mx, v[i]);
+    mx = block_max_256(mx, sm4);
+    if (threadIdx.x == 0) pmax[(size_t)blockIdx.y * gridDim.x + blockIdx.x] = mx;
+}
+
+// e[i] = exp(v[i] / T - max / T): the quotient and the difference in f32 as the reference forms them, the exponential
+// through double precision, which rounds to the nearest f32 like libm's expf does in all but very rare cases.
+__global__ __launch_bounds__(256) void full_exp_kernel(const float* __restrict__ logits, uint32_t n, float temperature,
+                                                        const float* __restrict__ pmax, float* __restrict__ e_out,
+                                                        uint32_t* __restrict__ iota) {
+    __shared__ float sm4[4];
+    const uint32_t row = blockIdx.y, parts = gridDim.x;
+    float mx = -INFINITY;
+    for (uint32_t j = threadIdx.x; j < parts; j += 256) mx = fmaxf(mx, pmax[(size_t)row * parts + j]);
+    const float ms = block_max_256(mx, sm4) / temperature;  // max of the quotients = quotient of the max (T > 0, division is monotone)
+    const float* v = logits + (size_t)row * n;
+    for (uint32_t i = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; i < min(n, (blockIdx.x + 1) * OXB_FULL_SPAN); i += 256) {
+        const float x = v[i] / temperature;
+        e_out[(size_t)row * n + i] = (float)exp((double)(x - ms));
+        if (row == 0) iota[i] = i;
+    }
+}
+
+// acc + x(lane 0) + x(lane 1) + ... + x(lane 63), added in that order.
+__device__ __forceinline__ float chain64(float acc, float x) {
+#pragma unroll
+    for (int l = 0; l < 64; l++) acc += __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), l));
+    return acc;
+}
+
+// sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One wave per row.
+__global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ e, uint32_t n, float* __restrict__ sum) {
+    const float* x = e + (size_t)blockIdx.x * n;
+    const uint32_t lane = threadIdx.x;
+    float acc = 0.0f;
+    float cur[4], nxt[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) cur[c] = lane + 64u * c < n ? x[lane + 64u * c] : 0.0f;
+    for (uint32_t base = 0; base < n; base += 256) {
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const uint32_t i = base + 256u + 64u * c + lane;
+            nxt[c] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
+#pragma unroll
+        for (int c = 0; c < 4; c++) cur[c] = nxt[c];
+    }
+    if (lane == 0) sum[blockIdx.x] = acc;
+}
+
+__global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t n, const float* __restrict__ sum) {
+    const float s = sum[blockIdx.y];
+    float* x = e + (size_t)blockIdx.y * n;
+    for (uint32_t i = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; i < min(n, (blockIdx.x + 1) * OXB_FULL_SPAN); i += 256) x[i] /= s;
+}
+
+// Top-p cut, renormalisation, draw and pick over the row's probabilities p (sorted descending with their token ids
+// when top-p is on, else in index order with ids = null).  One wave per row; every sum is a chain in element order.
+__global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t n,
+                                                        float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
+    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+    const float* p = p_all + (size_t)row * n;
+    const uint32_t* ids = ids_all ? ids_all + (size_t)row * n : nullptr;
+    auto lane_value = [](float x, uint32_t l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), (int)l)); };
+    uint32_t m = n;
+    float s2 = 1.0f;
+    const bool cut = top_p < 1.0f;
+    if (cut) {
+        // position(|p| { cum += p; cum > top_p }).unwrap_or(len - 1), sampling.rs:138-146
+        uint32_t cutoff = n - 1;
+        float cum = 0.0f;
+        for (uint32_t base = 0; base < n; base += 64) {
+            const float x = base + lane < n ? p[base + lane] : 0.0f;
+            const float end = chain64(cum, x);
+            if (end > top_p) {  // probabilities are >= 0, the running sum does not fall: the crossing is in this chunk
+                float c = cum;
+                for (uint32_t l = 0; l < 64; l++) {
+                    c += lane_value(x, l);
+                    if (c > top_p) {
+                        cutoff = base + l;
+                        break;
+                    }
+                }
+                break;
+            }
+            cum = end;
+        }
+        m = cutoff + 1;
+        s2 = 0.0f;  // the renormalising sum over the kept entries, :150-152
+        for (uint32_t base = 0; base < m; base += 64) s2 = chain64(s2, base + lane < m ? p[base + lane] : 0.0f);
+    }
+    uint64_t x64 = rng[row];
+    x64 ^= x64 << 13;
+    x64 ^= x64 >> 7;
+    x64 ^= x64 << 17;
+    const float r = (float)((double)x64 / 18446744073709551615.0);
+    uint32_t pick = 0;  // the fallback is the buffer's first entry, :173-174
+    float cum = 0.0f;
+    for (uint32_t base = 0; base < m; base += 64) {
+        float x = base + lane < m ? p[base + lane] : 0.0f;
+        if (cut) x /= s2;
+        const float end = chain64(cum, x);
+        if (r <= end) {
+            float c = cum;
+            for (uint32_t l = 0; l < 64; l++) {
+                c += lane_value(x, l);
+                if (r <= c) {
+                    pick = base + l;
+                    break;
+                }
+            }
+            break;
+        }
+        cum = end;
+    }
+    if (lane == 0) {
+        rng[row] = x64;
+        tokens[row] = ids ? ids[pick] : pick;
+    }
+}
+
 hipError_t oxb_launch_embedding_gather(const void* d_table, int gguf_type, uint32_t vocab, uint32_t h, const uint32_t* d_ids,
                                        uint32_t n, float* d_out, hipStream_t st) {
     if (n == 0) return hipSuccess;
@@ -253,15 +400,76 @@ hipError_t oxb_launch_token_step(const uint32_t* d_tokens, uint32_t* d_history, 
 
 static uint32_t sample_parts(uint32_t n) { return (n + OXB_TOPK_SPAN - 1) / OXB_TOPK_SPAN; }
 
+static size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
+
+// Scratch of the top-k-off route: e / p [batch][n], sorted p [batch][n], sorted ids [batch][n], iota [n],
+// part maxima [batch][parts], sums [batch], the sort's temporary storage.
+struct FullWs { size_t e, ps, is, iota, pmax, sum, tmp, tmp_bytes, total; };
+static hipError_t full_ws_layout(uint32_t n, uint32_t batch, FullWs* w) {
+    size_t tmp = 0;
+    hipError_t err = hipcub::DeviceRadixSort::SortPairsDescending(nullptr, tmp, (const float*)nullptr, (float*)nullptr,
+                                                                 (const uint32_t*)nullptr, (uint32_t*)nullptr, (int)n);
+    if (err != hipSuccess) return err;
+    const size_t rows = align256((size_t)n * 4 * batch), parts = (n + OXB_FULL_SPAN - 1) / OXB_FULL_SPAN;
+    w->e = 0;
+    w->ps = w->e + rows;
+    w->is = w->ps + rows;
+    w->iota = w->is + rows;
+    w->pmax = w->iota + align256((size_t)n * 4);
+    w->sum = w->pmax + align256((size_t)batch * parts * 4);
+    w->tmp = w->sum + align256((size_t)batch * 4);
+    w->tmp_bytes = tmp;
+    w->total = w->tmp + align256(tmp);
+    return hipSuccess;
+}
+
 size_t oxb_sample_ws_bytes(uint32_t n, uint32_t batch) {
-    return (size_t)batch * sample_parts(n) * OXB_SAMPLE_MAX_TOP_K * 8;
+    const size_t topk = (size_t)batch * sample_parts(n) * OXB_SAMPLE_MAX_TOP_K * 8;
+    FullWs w;
+    if (n > 0x7FFFFFFFu || full_ws_layout(n, batch, &w) != hipSuccess) return topk;
+    return topk > w.total ? topk : w.total;
+}
+
+static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t batch, float temperature, float top_p,
+                                     uint64_t* d_rng, uint32_t* d_tokens, void* d_ws, hipStream_t st) {
+    FullWs w;
+    if (n > 0x7FFFFFFFu) return hipErrorInvalidValue;
+    hipError_t err = full_ws_layout(n, batch, &w);
+    if (err != hipSuccess) return err;
+    uint8_t* base = static_cast<uint8_t*>(d_ws);
+    float* e = reinterpret_cast<float*>(base + w.e);
+    float* ps = reinterpret_cast<float*>(base + w.ps);
+    uint32_t* is = reinterpret_cast<uint32_t*>(base + w.is);
+    uint32_t* iota = reinterpret_cast<uint32_t*>(base + w.iota);
+    float* pmax = reinterpret_cast<float*>(base + w.pmax);
+    float* sum = reinterpret_cast<float*>(base + w.sum);
+    const uint32_t parts = (n + OXB_FULL_SPAN - 1) / OXB_FULL_SPAN;
+    hipLaunchKernelGGL(full_max_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, pmax);
+    hipLaunchKernelGGL(full_exp_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, pmax, e, iota);
+    hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, sum);
+    hipLaunchKernelGGL(full_prob_kernel, dim3(parts, batch), dim3(256), 0, st, e, n, sum);
+    if (top_p < 1.0f) {
+        // stable: equal probabilities keep index order, as the reference's sort_by does
+        for (uint32_t b = 0; b < batch; b++) {
+            size_t tmp = w.tmp_bytes;
+            err = hipcub::DeviceRadixSort::SortPairsDescending(base + w.tmp, tmp, e + (size_t)b * n, ps + (size_t)b * n, iota,
+                                                               is + (size_t)b * n, (int)n, 0, 32, st);
+            if (err != hipSuccess) return err;
+        }
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, ps, is, n, top_p, d_rng, d_tokens);
+    } else {
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, (const uint32_t*)nullptr, n, top_p, d_rng, d_tokens);
+    }
+    return hipGetLastError();
 }
 
 hipError_t oxb_launch_sample(const float* d_logits, uint32_t n, uint32_t batch, float temperature, uint32_t top_k, float top_p,
                              uint64_t* d_rng, uint32_t* d_tokens, void* d_ws, hipStream_t st) {
     const uint32_t parts = sample_parts(n);
-    if (n == 0 || batch == 0 || top_k == 0 || top_k > OXB_SAMPLE_MAX_TOP_K || parts > 64 * OXB_SAMPLE_LISTS_PER_LANE || !(temperature >= 1e-6f) || !d_ws)
-        return hipErrorInvalidValue;
+    if (n == 0 || batch == 0 || !(temperature >= 1e-6f) || !d_ws) return hipErrorInvalidValue;
+    if (top_k == 0 || top_k >= n)  // the filter is off (sampling.rs:111)
+        return launch_sample_full(d_logits, n, batch, temperature, top_p, d_rng, d_tokens, d_ws, st);
+    if (top_k > OXB_SAMPLE_MAX_TOP_K || parts > 64 * OXB_SAMPLE_LISTS_PER_LANE) return hipErrorInvalidValue;
     float* cv = reinterpret_cast<float*>(d_ws);
     uint32_t* ci = reinterpret_cast<uint32_t*>(d_ws) + (size_t)batch * parts * top_k;
     hipLaunchKernelGGL(topk_partial_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, top_k, cv, ci);

@@ -183,10 +183,45 @@ def test_device_sampler_statistics_and_errors(backend):
         counts += np.bincount(toks, minlength=64)
     assert counts[4:].sum() == 0 and np.max(np.abs(counts[:4] / counts.sum() - want)) < 0.02
     assert sample_logits([0.1, 0.5, 0.3, 0.9, 0.2], 0.0, 40, 0.9, 42)[0][0] == 3          # greedy_sampling
-    for bad in ((0.7, 0, 0.9), (0.7, 129, 0.9), (-1.0, 40, 0.9), (0.7, 40, 0.0)):
+    wide = np.zeros((2, 300), np.float32)
+    for rows, bad in ((wide, (0.7, 129, 0.9)), (wide, (0.7, 299, 0.9)), (lg[:2], (-1.0, 40, 0.9)), (lg[:2], (0.7, 40, 0.0))):
         with pytest.raises(GpuError) as e:
-            sample_logits(lg[:2], *bad, [1, 2])
+            sample_logits(rows, *bad, [1, 2])
         assert e.value.kind == "InvalidArgument"
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("n,T,tp", [(151936, 1.0, 0.95), (151936, 0.7, 1.0), (5000, 1.0, 0.95), (5000, 2.0, 1.0),
+                                    (33, 0.5, 0.95), (33, 0.5, 1.0), (1, 1.0, 0.9), (64, 1.0, 0.5), (2049, 0.05, 0.9)])
+def test_device_sampler_with_the_filter_off(backend, n, T, tp):
+    """top_k = 0 (and top_k >= the vocabulary, which the reference treats alike): softmax, sort, cut and pick over the
+    whole vocabulary with every sum taken in the reference's order.  The device must return the restatement's token;
+    where they differ, the two tokens must be neighbours in the buffer and the draw must sit on their boundary (the
+    device's exponential goes through double precision, libm's expf is not always the nearest f32)."""
+    from oxibonsai_amd.model import sample_logits
+    rows = 6
+    spread = 4.0 if n < 100000 else 0.05                 # the large rows are nearly flat: 150 000 comparable probabilities
+    logits = (synth.normal_f32(n + 7, rows * n) * spread).reshape(rows, n)
+    if n > 100:
+        logits[1, 7] = logits[1, 99] = logits[1].max() + 1.0       # equal probabilities: the sort keeps index order
+        logits[2, 50:60] = 3.0 * spread + logits[2].max()            # a peaked row
+    seeds = np.array([1, 42, 2**63 + 5, 0x9E3779B97F4A7C15, 99, 0], dtype=np.uint64)
+    top_k = 0 if n != 33 else 40                                   # 40 >= 33: the filter is off as well
+    toks, states = sample_logits(logits, T, top_k, tp, seeds)
+    differing = 0
+    for b in range(rows):
+        tok, new, ids, p, r = oracle.sample(logits[b], T, top_k, tp, int(seeds[b]))
+        assert int(states[b]) == new
+        if int(toks[b]) != tok:
+            differing += 1
+            ids = list(ids)
+            assert int(toks[b]) in ids, (b, int(toks[b]), tok)
+            a, c = sorted((ids.index(int(toks[b])), ids.index(tok)))
+            cum = np.float32(0.0)
+            for q in p[:a + 1]:
+                cum = np.float32(cum + q)
+            assert c - a == 1 and abs(float(cum) - float(r)) < 1e-6, (b, a, c, float(cum), float(r))
+    assert differing <= 1
 
 
 @pytest.mark.gpu
