@@ -244,8 +244,9 @@ int  oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* t
  * keeps whatever order its partial selection leaves when top_p == 1 (its pick is then an equally valid draw from
  * the same distribution, not the same token).  top_k = 0 or >= vocab switches the filter off as in the reference
  * (sampling.rs:111; the Creative preset): the whole vocabulary in index order, every f32 sum taken element by
- * element in the reference's order, a stable descending sort for top-p.  A top_k between 129 and vocab - 1 is
- * INVALID_ARGUMENT (sample on the host from the logits).  Repetition penalty is not part of Sampler::sample. */
+ * element in the reference's order, a stable descending sort for top-p.  A top_k between 129 and vocab - 1 sorts
+ * the whole row (descending, stable) and continues with its first top_k entries in that order.  Repetition penalty
+ * is not part of Sampler::sample. */
 typedef struct { float temperature; uint32_t top_k; float top_p; } oxb_sampling;
 int  oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
                                    uint32_t n_steps, const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out);

@@ -1112,12 +1112,8 @@ static int model_and_embedding(uint64_t model, uint64_t embedding, Model** m, Em
     return OXB_HIP_OK;
 }
 
-static int check_sampling(const oxb_sampling& sp, uint32_t vocab) {
+static int check_sampling(const oxb_sampling& sp, uint32_t /*vocab*/) {
     if (!(sp.temperature >= 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: temperature %g", (double)sp.temperature);
-    // top_k = 0 or >= the vocabulary switches the filter off (sampling.rs:111): the whole-vocabulary route
-    if (sp.temperature >= 1e-6f && sp.top_k > OXB_SAMPLE_MAX_TOP_K && sp.top_k < vocab)
-        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_k %u (the device sampler takes 1..%u, or 0 for no filter; sample on the host from the logits otherwise)",
-                    sp.top_k, OXB_SAMPLE_MAX_TOP_K);
     if (!(sp.top_p > 0.0f)) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: top_p %g", (double)sp.top_p);
     return OXB_HIP_OK;
 }

@@ -292,8 +292,8 @@ __device__ __forceinline__ float chain64(float acc, float x) {
 }
 
 // sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One wave per row.
-__global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ e, uint32_t n, float* __restrict__ sum) {
-    const float* x = e + (size_t)blockIdx.x * n;
+__global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
+    const float* x = e + (size_t)blockIdx.x * stride;
     const uint32_t lane = threadIdx.x;
     float acc = 0.0f;
     float cur[4], nxt[4];
@@ -313,19 +313,37 @@ __global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ 
     if (lane == 0) sum[blockIdx.x] = acc;
 }
 
-__global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t n, const float* __restrict__ sum) {
+__global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t stride, uint32_t n, const float* __restrict__ sum) {
     const float s = sum[blockIdx.y];
-    float* x = e + (size_t)blockIdx.y * n;
+    float* x = e + (size_t)blockIdx.y * stride;
     for (uint32_t i = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; i < min(n, (blockIdx.x + 1) * OXB_FULL_SPAN); i += 256) x[i] /= s;
+}
+
+// A top-k beyond what the selection kernels hold (129 .. vocabulary - 1): the whole row is sorted by v / T, descending and
+// stable (equal values keep index order, -0 counted as +0: the order the selection route produces), and the first
+// top_k entries go through the same softmax, cut and pick as above, in that order.
+__global__ __launch_bounds__(256) void full_scale_kernel(const float* __restrict__ logits, uint32_t n, float temperature,
+                                                          float* __restrict__ out, uint32_t* __restrict__ iota) {
+    const float* v = logits + (size_t)blockIdx.y * n;
+    for (uint32_t i = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; i < min(n, (blockIdx.x + 1) * OXB_FULL_SPAN); i += 256) {
+        out[(size_t)blockIdx.y * n + i] = v[i] / temperature + 0.0f;
+        if (blockIdx.y == 0) iota[i] = i;
+    }
+}
+__global__ __launch_bounds__(256) void sorted_exp_kernel(const float* __restrict__ sorted, uint32_t stride, uint32_t k, float* __restrict__ e_out) {
+    const float* x = sorted + (size_t)blockIdx.y * stride;
+    const float mx = x[0];
+    for (uint32_t j = blockIdx.x * OXB_FULL_SPAN + threadIdx.x; j < min(k, (blockIdx.x + 1) * OXB_FULL_SPAN); j += 256)
+        e_out[(size_t)blockIdx.y * stride + j] = (float)exp((double)(x[j] - mx));
 }
 
 // Top-p cut, renormalisation, draw and pick over the row's probabilities p (sorted descending with their token ids
 // when top-p is on, else in index order with ids = null).  One wave per row; every sum is a chain in element order.
-__global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t n,
-                                                        float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
+__global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t stride,
+                                                        uint32_t n, float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
     const uint32_t row = blockIdx.x, lane = threadIdx.x;
-    const float* p = p_all + (size_t)row * n;
-    const uint32_t* ids = ids_all ? ids_all + (size_t)row * n : nullptr;
+    const float* p = p_all + (size_t)row * stride;
+    const uint32_t* ids = ids_all ? ids_all + (size_t)row * stride : nullptr;
     auto lane_value = [](float x, uint32_t l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), (int)l)); };
     uint32_t m = n;
     float s2 = 1.0f;
@@ -430,7 +448,8 @@ size_t oxb_sample_ws_bytes(uint32_t n, uint32_t batch) {
     return topk > w.total ? topk : w.total;
 }
 
-static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t batch, float temperature, float top_p,
+// top_k = 0: the filter is off; otherwise 128 < top_k < n.
+static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t batch, float temperature, uint32_t top_k, float top_p,
                                      uint64_t* d_rng, uint32_t* d_tokens, void* d_ws, hipStream_t st) {
     FullWs w;
     if (n > 0x7FFFFFFFu) return hipErrorInvalidValue;
@@ -444,21 +463,34 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
     float* pmax = reinterpret_cast<float*>(base + w.pmax);
     float* sum = reinterpret_cast<float*>(base + w.sum);
     const uint32_t parts = (n + OXB_FULL_SPAN - 1) / OXB_FULL_SPAN;
-    hipLaunchKernelGGL(full_max_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, pmax);
-    hipLaunchKernelGGL(full_exp_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, pmax, e, iota);
-    hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, sum);
-    hipLaunchKernelGGL(full_prob_kernel, dim3(parts, batch), dim3(256), 0, st, e, n, sum);
-    if (top_p < 1.0f) {
-        // stable: equal probabilities keep index order, as the reference's sort_by does
+    auto sort_rows = [&]() -> hipError_t {  // e -> ps (descending, stable), iota -> is
         for (uint32_t b = 0; b < batch; b++) {
             size_t tmp = w.tmp_bytes;
-            err = hipcub::DeviceRadixSort::SortPairsDescending(base + w.tmp, tmp, e + (size_t)b * n, ps + (size_t)b * n, iota,
-                                                               is + (size_t)b * n, (int)n, 0, 32, st);
-            if (err != hipSuccess) return err;
+            hipError_t r = hipcub::DeviceRadixSort::SortPairsDescending(base + w.tmp, tmp, e + (size_t)b * n, ps + (size_t)b * n, iota,
+                                                                        is + (size_t)b * n, (int)n, 0, 32, st);
+            if (r != hipSuccess) return r;
         }
-        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, ps, is, n, top_p, d_rng, d_tokens);
+        return hipSuccess;
+    };
+    if (top_k != 0) {
+        const uint32_t kparts = (top_k + OXB_FULL_SPAN - 1) / OXB_FULL_SPAN;
+        hipLaunchKernelGGL(full_scale_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, e, iota);
+        if ((err = sort_rows()) != hipSuccess) return err;
+        hipLaunchKernelGGL(sorted_exp_kernel, dim3(kparts, batch), dim3(256), 0, st, ps, n, top_k, e);
+        hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, top_k, sum);
+        hipLaunchKernelGGL(full_prob_kernel, dim3(kparts, batch), dim3(256), 0, st, e, n, top_k, sum);
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, is, n, top_k, top_p, d_rng, d_tokens);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(full_max_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, pmax);
+    hipLaunchKernelGGL(full_exp_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, pmax, e, iota);
+    hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, n, sum);
+    hipLaunchKernelGGL(full_prob_kernel, dim3(parts, batch), dim3(256), 0, st, e, n, n, sum);
+    if (top_p < 1.0f) {
+        if ((err = sort_rows()) != hipSuccess) return err;  // stable: equal probabilities keep index order, as sort_by does
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, ps, is, n, n, top_p, d_rng, d_tokens);
     } else {
-        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, (const uint32_t*)nullptr, n, top_p, d_rng, d_tokens);
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, (const uint32_t*)nullptr, n, n, top_p, d_rng, d_tokens);
     }
     return hipGetLastError();
 }
@@ -468,8 +500,9 @@ hipError_t oxb_launch_sample(const float* d_logits, uint32_t n, uint32_t batch, 
     const uint32_t parts = sample_parts(n);
     if (n == 0 || batch == 0 || !(temperature >= 1e-6f) || !d_ws) return hipErrorInvalidValue;
     if (top_k == 0 || top_k >= n)  // the filter is off (sampling.rs:111)
-        return launch_sample_full(d_logits, n, batch, temperature, top_p, d_rng, d_tokens, d_ws, st);
-    if (top_k > OXB_SAMPLE_MAX_TOP_K || parts > 64 * OXB_SAMPLE_LISTS_PER_LANE) return hipErrorInvalidValue;
+        return launch_sample_full(d_logits, n, batch, temperature, 0, top_p, d_rng, d_tokens, d_ws, st);
+    if (top_k > OXB_SAMPLE_MAX_TOP_K) return launch_sample_full(d_logits, n, batch, temperature, top_k, top_p, d_rng, d_tokens, d_ws, st);
+    if (parts > 64 * OXB_SAMPLE_LISTS_PER_LANE) return hipErrorInvalidValue;
     float* cv = reinterpret_cast<float*>(d_ws);
     uint32_t* ci = reinterpret_cast<uint32_t*>(d_ws) + (size_t)batch * parts * top_k;
     hipLaunchKernelGGL(topk_partial_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, top_k, cv, ci);

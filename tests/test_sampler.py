@@ -183,17 +183,20 @@ def test_device_sampler_statistics_and_errors(backend):
         counts += np.bincount(toks, minlength=64)
     assert counts[4:].sum() == 0 and np.max(np.abs(counts[:4] / counts.sum() - want)) < 0.02
     assert sample_logits([0.1, 0.5, 0.3, 0.9, 0.2], 0.0, 40, 0.9, 42)[0][0] == 3          # greedy_sampling
-    wide = np.zeros((2, 300), np.float32)
-    for rows, bad in ((wide, (0.7, 129, 0.9)), (wide, (0.7, 299, 0.9)), (lg[:2], (-1.0, 40, 0.9)), (lg[:2], (0.7, 40, 0.0))):
+    for bad in ((-1.0, 40, 0.9), (0.7, 40, 0.0), (float("nan"), 40, 0.9)):
         with pytest.raises(GpuError) as e:
-            sample_logits(rows, *bad, [1, 2])
+            sample_logits(lg[:2], *bad, [1, 2])
         assert e.value.kind == "InvalidArgument"
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("n,T,tp", [(151936, 1.0, 0.95), (151936, 0.7, 1.0), (5000, 1.0, 0.95), (5000, 2.0, 1.0),
-                                    (33, 0.5, 0.95), (33, 0.5, 1.0), (1, 1.0, 0.9), (64, 1.0, 0.5), (2049, 0.05, 0.9)])
-def test_device_sampler_with_the_filter_off(backend, n, T, tp):
+@pytest.mark.parametrize("n,T,tp,top_k", [(151936, 1.0, 0.95, 0), (151936, 0.7, 1.0, 0), (5000, 1.0, 0.95, 0), (5000, 2.0, 1.0, 0),
+                                          (33, 0.5, 0.95, 40), (33, 0.5, 1.0, 40), (1, 1.0, 0.9, 0), (64, 1.0, 0.5, 0),
+                                          (2049, 0.05, 0.9, 0),
+                                          # a top-k beyond the selection kernels: whole-row sort, the first top_k entries
+                                          (151936, 0.8, 0.95, 1000), (151936, 1.0, 1.0, 129), (5000, 1.0, 0.9, 300),
+                                          (300, 1.0, 0.9, 299), (5000, 0.7, 1.0, 4999)])
+def test_device_sampler_with_the_filter_off(backend, n, T, tp, top_k):
     """top_k = 0 (and top_k >= the vocabulary, which the reference treats alike): softmax, sort, cut and pick over the
     whole vocabulary with every sum taken in the reference's order.  The device must return the restatement's token;
     where they differ, the two tokens must be neighbours in the buffer and the draw must sit on their boundary (the
@@ -206,7 +209,6 @@ def test_device_sampler_with_the_filter_off(backend, n, T, tp):
         logits[1, 7] = logits[1, 99] = logits[1].max() + 1.0       # equal probabilities: the sort keeps index order
         logits[2, 50:60] = 3.0 * spread + logits[2].max()            # a peaked row
     seeds = np.array([1, 42, 2**63 + 5, 0x9E3779B97F4A7C15, 99, 0], dtype=np.uint64)
-    top_k = 0 if n != 33 else 40                                   # 40 >= 33: the filter is off as well
     toks, states = sample_logits(logits, T, top_k, tp, seeds)
     differing = 0
     for b in range(rows):
