@@ -12,9 +12,11 @@ hipError_t oxb_launch_embedding_gather(const void* d_table, int gguf_type, uint3
 hipError_t oxb_launch_token_step(const uint32_t* d_tokens, uint32_t* d_history, uint32_t* d_pos, uint32_t batch, hipStream_t st);
 
 // Sampler::sample on the device (crates/oxibonsai-runtime/src/sampling.rs:84-177) for `batch` rows of logits:
-// the top_k largest logits (1 <= top_k <= OXB_SAMPLE_MAX_TOP_K) in descending order (ties: lower index first),
-// v / temperature, softmax, top-p cut and renormalisation, one xorshift64 draw per row from d_rng[row]
-// (updated in place), cumulative pick -> d_tokens[row].  d_ws: oxb_sample_ws_bytes(n, batch) bytes of scratch.
+// the top_k largest logits in descending order (ties: lower index first; up to OXB_SAMPLE_MAX_TOP_K by selection
+// kernels, beyond that by a stable sort of the whole row), v / temperature, softmax, top-p cut and renormalisation,
+// one xorshift64 draw per row from d_rng[row] (updated in place), cumulative pick -> d_tokens[row].  top_k = 0 or
+// >= n: the filter is off and the row is taken in index order, as the reference does (sampling.rs:111).
+// d_ws: oxb_sample_ws_bytes(n, batch) bytes of scratch.
 #define OXB_SAMPLE_MAX_TOP_K 128
 size_t oxb_sample_ws_bytes(uint32_t n, uint32_t batch);
 hipError_t oxb_launch_sample(const float* d_logits, uint32_t n, uint32_t batch, float temperature, uint32_t top_k, float top_p,
