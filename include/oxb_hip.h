@@ -250,6 +250,10 @@ int  oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* t
 typedef struct { float temperature; uint32_t top_k; float top_p; } oxb_sampling;
 int  oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
                                    uint32_t n_steps, const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out);
+/* The f32 sum of x[0..n) taken element by element from 0, as the loop `sum += *v` of the reference's softmax does
+ * (sampling.rs:126-130); all x >= 0.  The filter-off sampler depends on this order bit for bit; exposed so that it can
+ * be checked on its own. */
+int  oxb_hip_sum_in_order(const float* x, uint32_t n, float* sum_out);
 /* The sampler alone on host logits [batch][vocab] (vocab <= 524288). */
 int  oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params,
                            uint64_t* rng_state, uint32_t* tokens_out);

@@ -1178,6 +1178,22 @@ int oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint
     return decode_tokens_impl(model, embedding, tokens, pos, n_steps, params, rng_state, tokens_out);
 }
 
+int oxb_hip_sum_in_order(const float* x, uint32_t n, float* sum_out) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!x || !sum_out || n == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or no elements");
+    OXB_TRY(ensure_init());
+    OXB_TRY(g_rt.ws_y.ensure((size_t)n * 4 + 256));
+    float* d_x = (float*)g_rt.ws_y.ptr;
+    float* d_sum = (float*)((uint8_t*)g_rt.ws_y.ptr + (((size_t)n * 4 + 255) & ~(size_t)255));
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(d_x, x, (size_t)n * 4, hipMemcpyHostToDevice, st), "upload");
+    OXB_TRY_HIP(oxb_launch_sum_in_order(d_x, n, d_sum, st), "kernel launch failed: sum_in_order");
+    OXB_TRY_HIP(hipMemcpyAsync(sum_out, d_sum, 4, hipMemcpyDeviceToHost, st), "download");
+    hipError_t he = hipStreamSynchronize(st);
+    if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: sum_in_order: %s", hipGetErrorString(he));
+    return OXB_HIP_OK;
+}
+
 int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params, uint64_t* rng_state,
                           uint32_t* tokens_out) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);

@@ -21,3 +21,6 @@ hipError_t oxb_launch_token_step(const uint32_t* d_tokens, uint32_t* d_history, 
 size_t oxb_sample_ws_bytes(uint32_t n, uint32_t batch);
 hipError_t oxb_launch_sample(const float* d_logits, uint32_t n, uint32_t batch, float temperature, uint32_t top_k, float top_p,
                              uint64_t* d_rng, uint32_t* d_tokens, void* d_ws, hipStream_t st);
+// d_sum[0] = ((0 + x[0]) + x[1]) + ... in f32, element by element: the softmax denominator as the reference's loop
+// forms it (sampling.rs:126-130).  All x >= 0.
+hipError_t oxb_launch_sum_in_order(const float* d_x, uint32_t n, float* d_sum, hipStream_t st);

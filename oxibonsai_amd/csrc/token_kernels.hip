@@ -291,6 +291,54 @@ __device__ __forceinline__ float chain64(float acc, float x) {
     return acc;
 }
 
+__device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
+    v += dpp_u32<OXB_DPP_ROW_SHR(1)>(v);
+    v += dpp_u32<OXB_DPP_ROW_SHR(2)>(v);
+    v += dpp_u32<OXB_DPP_ROW_SHR(4)>(v);
+    v += dpp_u32<OXB_DPP_ROW_SHR(8)>(v);  // lane 16 r + 15 holds the total of its row of 16 lanes
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 15) + (uint32_t)__builtin_amdgcn_readlane((int)v, 31) +
+           (uint32_t)__builtin_amdgcn_readlane((int)v, 47) + (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// The same result as C x chain64 (elements c * 64 + lane in ascending order) without the chain, where that is
+// provable.  While the running sum s stays inside one binade its ulp u is fixed, and fl(s + x) = s + u * R(x / u) with
+// R = round to nearest: the sum is an integer accumulation T += R_i of the mantissa T = s / u, whose increments do
+// not depend on the order - unless x / u ends in exactly one half, where the tie goes to the even mantissa and
+// so depends on T.  So: every lane forms its increments from the bits of x; if no element is a tie, none is negative,
+// NaN, infinite or as large as u * 2^23, and T + sum of the increments stays below 2^24 (the binade is not left,
+// and since the terms are >= 0 no partial sum leaves it either), the new sum is s with the mantissa T + sum.
+// Otherwise false is returned and the caller adds these elements one by one.
+template <int C>
+__device__ __forceinline__ bool chain_fast(float& acc, const float (&x)[C]) {
+    const uint32_t sb = __float_as_uint(acc), es = sb >> 23;  // acc >= 0 here
+    if (es == 0 || es >= 255) return false;                   // zero, subnormal, infinite or NaN running sum
+    const uint32_t T = (sb & 0x7FFFFFu) | 0x800000u;
+    uint32_t f_sum = 0;
+    bool bad = false;
+#pragma unroll
+    for (int c = 0; c < C; c++) {
+        const uint32_t b = __float_as_uint(x[c]), ex0 = b >> 23;  // a set sign bit makes ex0 >= 256
+        uint32_t m = b & 0x7FFFFFu;
+        const uint32_t ex = ex0 ? ex0 : 1u;
+        if (ex0) m |= 0x800000u;
+        // x = m * 2^(ex - 150), u = 2^(es - 150): x / u = m >> shr with shr = es - ex
+        const int shr = (int)es - (int)ex;
+        if (m == 0u) continue;  // +0 (a -0 has ex0 = 256 and is refused below)
+        if (ex0 >= 255u || shr <= 0) {
+            bad = true;
+        } else if (shr <= 24) {
+            const uint32_t rem = m & ((1u << shr) - 1u), half = 1u << (shr - 1);
+            f_sum += (m >> shr) + (rem > half ? 1u : 0u);
+            bad |= rem == half;
+        }  // shr >= 25: less than half an ulp, the sum does not move
+    }
+    if (__builtin_amdgcn_ballot_w64(bad) != 0ull) return false;
+    const uint32_t total = T + wave_sum_u32(f_sum);  // <= 2^24 + 64 C * 2^23: no overflow
+    if (total >= 0x1000000u) return false;
+    acc = __uint_as_float((es << 23) | (total & 0x7FFFFFu));
+    return true;
+}
+
 // sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One wave per row.
 __global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
     const float* x = e + (size_t)blockIdx.x * stride;
@@ -305,8 +353,10 @@ __global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ 
             const uint32_t i = base + 256u + 64u * c + lane;
             nxt[c] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
         }
+        if (!chain_fast<4>(acc, cur)) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
+            for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
+        }
 #pragma unroll
         for (int c = 0; c < 4; c++) cur[c] = nxt[c];
     }
@@ -492,6 +542,11 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
     } else {
         hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, (const uint32_t*)nullptr, n, n, top_p, d_rng, d_tokens);
     }
+    return hipGetLastError();
+}
+
+hipError_t oxb_launch_sum_in_order(const float* d_x, uint32_t n, float* d_sum, hipStream_t st) {
+    hipLaunchKernelGGL(full_sum_kernel, dim3(1), dim3(64), 0, st, d_x, n, n, d_sum);
     return hipGetLastError();
 }
 

@@ -81,6 +81,14 @@ def sample_logits(logits, temperature: float, top_k: int, top_p: float, rng_stat
     return out, st
 
 
+def sum_in_order(x) -> np.float32:
+    """((0 + x[0]) + x[1]) + ... in f32 on the device, the order of the reference's softmax loop (sampling.rs:126-130)."""
+    a = np.ascontiguousarray(x, dtype=np.float32).ravel()
+    out = np.zeros(1, dtype=np.float32)
+    _check(_lib.lib().oxb_hip_sum_in_order(a.ctypes.data_as(_lib.f32p), a.size, out.ctypes.data_as(_lib.f32p)))
+    return out[0]
+
+
 KV_F16, KV_I8, KV_FP8_E4M3 = 0, 1, 2   # OXB_KV_DTYPE_*
 
 

@@ -257,3 +257,33 @@ def test_sampled_generation_loop(backend, tmp_path):
         a.close()
         b.close()
         emb.close()
+
+
+@pytest.mark.gpu
+def test_device_sum_in_order_is_bit_exact(backend):
+    """The softmax denominator must be the reference's element-by-element f32 sum.  The device takes 256 elements at
+    a time without a chain where it can prove the result (no rounding tie, binade not left) and one by one elsewhere:
+    both routes and the switches between them against numpy's sequential cumsum."""
+    from oxibonsai_amd.model import sum_in_order
+    rng = np.random.default_rng(5)
+
+    def ref(x):
+        return np.cumsum(np.asarray(x, dtype=np.float32), dtype=np.float32)[-1]
+
+    cases = {
+        "softmax terms, flat": np.exp(rng.normal(0, 0.05, 151936)).astype(np.float32) * np.float32(0.9),
+        "softmax terms, peaked": np.exp(rng.normal(0, 4.0, 151936) - 16).astype(np.float32),
+        "many ties": np.concatenate([[np.float32(2.0**24)], rng.integers(1, 8, 100000).astype(np.float32)]),  # ulp 2 and up: odd terms tie
+        "ties at every scale": np.ldexp(rng.integers(1, 4, 70000).astype(np.float32), rng.integers(-30, 2, 70000)).astype(np.float32),
+        "one large element late": np.concatenate([np.full(5000, 1e-3, np.float32), [np.float32(900.0)], np.full(5000, 1e-3, np.float32)]),
+        "zeros and subnormals": np.concatenate([np.zeros(300, np.float32), np.full(300, 1e-42, np.float32), np.ones(300, np.float32)]),
+        "short": np.array([0.1, 0.2, 0.3], np.float32),
+        "single": np.array([7.25], np.float32),
+        "all zero": np.zeros(1000, np.float32),
+        "crosses many binades": np.full(200000, 1.0, np.float32),
+        "random magnitudes": np.exp(rng.normal(0, 6.0, 120001)).astype(np.float32),
+        "odd length": np.exp(rng.normal(0, 1.0, 65537)).astype(np.float32),
+    }
+    for name, x in cases.items():
+        got, want = sum_in_order(x), ref(x)
+        assert got.tobytes() == want.tobytes(), (name, float(got), float(want))
