@@ -302,18 +302,21 @@ __device__ __forceinline__ uint32_t wave_sum_u32(uint32_t v) {
 
 // The same result as C x chain64 (elements c * 64 + lane in ascending order) without the chain, where that is
 // provable.  While the running sum s stays inside one binade its ulp u is fixed, and fl(s + x) = s + u * R(x / u) with
-// R = round to nearest: the sum is an integer accumulation T += R_i of the mantissa T = s / u, whose increments do
-// not depend on the order - unless x / u ends in exactly one half, where the tie goes to the even mantissa and
-// so depends on T.  So: every lane forms its increments from the bits of x; if no element is a tie, none is negative,
-// NaN, infinite or as large as u * 2^23, and T + sum of the increments stays below 2^24 (the binade is not left,
-// and since the terms are >= 0 no partial sum leaves it either), the new sum is s with the mantissa T + sum.
-// Otherwise false is returned and the caller adds these elements one by one.
+// R = round to nearest: the sum is an integer accumulation T += R_i of the mantissa T = s / u.  The increments do
+// not depend on T except where x / u ends in exactly one half: such a tie goes to the even mantissa, so it adds
+// floor(x / u) plus one if T + floor(x / u) is odd - and leaves T even.  Parity is therefore all the state there is:
+// before a tie it is the parity of T at the previous tie (even) or at the start, flipped once per odd increment in
+// between.  Every lane forms its increment from the bits of x; the odd increments and the ties of a chunk become two
+// 64-bit lane masks, over which the carries of the ties are worked out with scalar bit operations; one wave-wide
+// integer sum finishes the group.  Refused (false: the caller adds the elements one by one) if an element is negative,
+// NaN, infinite or at least u * 2^23, if s is zero, subnormal or not finite, or if the mantissa would reach 2^24 (the
+// binade is left; the terms are >= 0, so then and only then some partial sum leaves it too).
 template <int C>
 __device__ __forceinline__ bool chain_fast(float& acc, const float (&x)[C]) {
     const uint32_t sb = __float_as_uint(acc), es = sb >> 23;  // acc >= 0 here
-    if (es == 0 || es >= 255) return false;                   // zero, subnormal, infinite or NaN running sum
+    if (es == 0 || es >= 255) return false;
     const uint32_t T = (sb & 0x7FFFFFu) | 0x800000u;
-    uint32_t f_sum = 0;
+    uint32_t f_sum = 0, carries = 0, par = T & 1u;
     bool bad = false;
 #pragma unroll
     for (int c = 0; c < C; c++) {
@@ -321,46 +324,91 @@ __device__ __forceinline__ bool chain_fast(float& acc, const float (&x)[C]) {
         uint32_t m = b & 0x7FFFFFu;
         const uint32_t ex = ex0 ? ex0 : 1u;
         if (ex0) m |= 0x800000u;
-        // x = m * 2^(ex - 150), u = 2^(es - 150): x / u = m >> shr with shr = es - ex
+        // x = m * 2^(ex - 150), u = 2^(es - 150): x / u = m / 2^shr with shr = es - ex
         const int shr = (int)es - (int)ex;
-        if (m == 0u) continue;  // +0 (a -0 has ex0 = 256 and is refused below)
-        if (ex0 >= 255u || shr <= 0) {
-            bad = true;
-        } else if (shr <= 24) {
-            const uint32_t rem = m & ((1u << shr) - 1u), half = 1u << (shr - 1);
-            f_sum += (m >> shr) + (rem > half ? 1u : 0u);
-            bad |= rem == half;
-        }  // shr >= 25: less than half an ulp, the sum does not move
+        uint32_t f = 0;
+        bool tie = false;
+        if (m != 0u) {  // (a -0 counts as +0)
+            if (ex0 >= 255u || shr <= 0) {
+                bad = true;
+            } else if (shr <= 24) {
+                const uint32_t rem = m & ((1u << shr) - 1u), half = 1u << (shr - 1);
+                f = (m >> shr) + (rem > half ? 1u : 0u);
+                tie = rem == half;
+            }  // shr >= 25: less than half an ulp, the sum does not move
+        }
+        f_sum += f;
+        const uint64_t odd = __builtin_amdgcn_ballot_w64((f & 1u) != 0u);
+        uint64_t ties = __builtin_amdgcn_ballot_w64(tie);
+        uint64_t done = 0;  // lanes up to and including the last tie handled
+        while (ties) {
+            const uint32_t i = (uint32_t)__builtin_ctzll(ties);
+            ties &= ties - 1;
+            const uint64_t below = (1ull << i) - 1ull;
+            const uint32_t before = par ^ ((uint32_t)__builtin_popcountll(odd & below & ~done) & 1u);
+            carries += before ^ (uint32_t)((odd >> i) & 1ull);  // T + floor odd -> one more, and T is even afterwards
+            par = 0;
+            done = below | (1ull << i);
+        }
+        par ^= (uint32_t)__builtin_popcountll(odd & ~done) & 1u;
     }
     if (__builtin_amdgcn_ballot_w64(bad) != 0ull) return false;
-    const uint32_t total = T + wave_sum_u32(f_sum);  // <= 2^24 + 64 C * 2^23: no overflow
+    const uint32_t total = T + wave_sum_u32(f_sum) + carries;  // <= 2^24 + 64 C * (2^23 + 1): no overflow for C <= 4
     if (total >= 0x1000000u) return false;
     acc = __uint_as_float((es << 23) | (total & 0x7FFFFFu));
     return true;
 }
 
-// sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One wave per row.
-__global__ __launch_bounds__(64) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
+// acc + the wave's 64 values in lane order.
+__device__ __forceinline__ float add64(float acc, float x) {
+    float a = acc;
+    const float xs[1] = {x};
+    if (chain_fast<1>(a, xs)) return a;
+    return chain64(acc, x);
+}
+
+// sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One workgroup per row: all four
+// waves bring the row in, 4096 elements at a time, through two LDS tiles (the next tile's loads are in flight while
+// the current one is added up); the first wave does the adding, 256 elements per step.
+#define OXB_SUM_TILE 4096u
+__global__ __launch_bounds__(256) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
+    __shared__ float tile[2][OXB_SUM_TILE];
     const float* x = e + (size_t)blockIdx.x * stride;
-    const uint32_t lane = threadIdx.x;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    float r[16];
+    auto fetch = [&](uint32_t base) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t i = base + 256u * j + tid;
+            r[j] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
+        }
+    };
+    auto stash = [&](uint32_t buf) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) tile[buf][256u * j + tid] = r[j];
+    };
+    fetch(0);
+    stash(0);
+    __syncthreads();
     float acc = 0.0f;
-    float cur[4], nxt[4];
+    for (uint32_t base = 0, buf = 0; base < n; base += OXB_SUM_TILE, buf ^= 1u) {
+        const bool more = base + OXB_SUM_TILE < n;  // uniform
+        if (more) fetch(base + OXB_SUM_TILE);
+        if (wave == 0) {
+            for (uint32_t g = 0; g < OXB_SUM_TILE / 256u && base + 256u * g < n; g++) {
+                float cur[4];
 #pragma unroll
-    for (int c = 0; c < 4; c++) cur[c] = lane + 64u * c < n ? x[lane + 64u * c] : 0.0f;
-    for (uint32_t base = 0; base < n; base += 256) {
+                for (int c = 0; c < 4; c++) cur[c] = tile[buf][256u * g + 64u * c + lane];
+                if (!chain_fast<4>(acc, cur)) {
 #pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const uint32_t i = base + 256u + 64u * c + lane;
-            nxt[c] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
+                    for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
+                }
+            }
         }
-        if (!chain_fast<4>(acc, cur)) {
-#pragma unroll
-            for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
-        }
-#pragma unroll
-        for (int c = 0; c < 4; c++) cur[c] = nxt[c];
+        if (more) stash(buf ^ 1u);
+        __syncthreads();
     }
-    if (lane == 0) sum[blockIdx.x] = acc;
+    if (tid == 0) sum[blockIdx.x] = acc;
 }
 
 __global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t stride, uint32_t n, const float* __restrict__ sum) {
@@ -404,7 +452,7 @@ __global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__
         float cum = 0.0f;
         for (uint32_t base = 0; base < n; base += 64) {
             const float x = base + lane < n ? p[base + lane] : 0.0f;
-            const float end = chain64(cum, x);
+            const float end = add64(cum, x);
             if (end > top_p) {  // probabilities are >= 0, the running sum does not fall: the crossing is in this chunk
                 float c = cum;
                 for (uint32_t l = 0; l < 64; l++) {
@@ -420,7 +468,7 @@ __global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__
         }
         m = cutoff + 1;
         s2 = 0.0f;  // the renormalising sum over the kept entries, :150-152
-        for (uint32_t base = 0; base < m; base += 64) s2 = chain64(s2, base + lane < m ? p[base + lane] : 0.0f);
+        for (uint32_t base = 0; base < m; base += 64) s2 = add64(s2, base + lane < m ? p[base + lane] : 0.0f);
     }
     uint64_t x64 = rng[row];
     x64 ^= x64 << 13;
@@ -432,7 +480,7 @@ __global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__
     for (uint32_t base = 0; base < m; base += 64) {
         float x = base + lane < m ? p[base + lane] : 0.0f;
         if (cut) x /= s2;
-        const float end = chain64(cum, x);
+        const float end = add64(cum, x);
         if (r <= end) {
             float c = cum;
             for (uint32_t l = 0; l < 64; l++) {
@@ -527,14 +575,14 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
         hipLaunchKernelGGL(full_scale_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, e, iota);
         if ((err = sort_rows()) != hipSuccess) return err;
         hipLaunchKernelGGL(sorted_exp_kernel, dim3(kparts, batch), dim3(256), 0, st, ps, n, top_k, e);
-        hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, top_k, sum);
+        hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(256), 0, st, e, n, top_k, sum);
         hipLaunchKernelGGL(full_prob_kernel, dim3(kparts, batch), dim3(256), 0, st, e, n, top_k, sum);
         hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, is, n, top_k, top_p, d_rng, d_tokens);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(full_max_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, pmax);
     hipLaunchKernelGGL(full_exp_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, temperature, pmax, e, iota);
-    hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(64), 0, st, e, n, n, sum);
+    hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(256), 0, st, e, n, n, sum);
     hipLaunchKernelGGL(full_prob_kernel, dim3(parts, batch), dim3(256), 0, st, e, n, n, sum);
     if (top_p < 1.0f) {
         if ((err = sort_rows()) != hipSuccess) return err;  // stable: equal probabilities keep index order, as sort_by does
@@ -546,7 +594,7 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
 }
 
 hipError_t oxb_launch_sum_in_order(const float* d_x, uint32_t n, float* d_sum, hipStream_t st) {
-    hipLaunchKernelGGL(full_sum_kernel, dim3(1), dim3(64), 0, st, d_x, n, n, d_sum);
+    hipLaunchKernelGGL(full_sum_kernel, dim3(1), dim3(256), 0, st, d_x, n, n, d_sum);
     return hipGetLastError();
 }
 
