@@ -367,48 +367,72 @@ __device__ __forceinline__ float add64(float acc, float x) {
     return chain64(acc, x);
 }
 
-// sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One workgroup per row: all four
-// waves bring the row in, 4096 elements at a time, through two LDS tiles (the next tile's loads are in flight while
-// the current one is added up); the first wave does the adding, 256 elements per step.
+// Brings x[0 .. n) to the first wave in element order, 256 elements per call of visit(base, cur) with
+// cur[c] = x[base + 64 c + lane] (+0 past n); visit returns true to end the walk.  All four waves load, 4096 elements at
+// a time, through two LDS tiles: the next tile's loads are in flight while the current one is visited.  Every thread
+// of the workgroup must call it (barriers inside); what visit changes is valid in the first wave only.
 #define OXB_SUM_TILE 4096u
-__global__ __launch_bounds__(256) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
-    __shared__ float tile[2][OXB_SUM_TILE];
-    const float* x = e + (size_t)blockIdx.x * stride;
+struct RowTiles {
+    float t[2][OXB_SUM_TILE];
+    uint32_t stop;
+};
+template <class Visit>
+__device__ __forceinline__ void walk_row(const float* __restrict__ x, uint32_t n, RowTiles& L, Visit&& visit) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     float r[16];
     auto fetch = [&](uint32_t base) {
 #pragma unroll
         for (int j = 0; j < 16; j++) {
             const uint32_t i = base + 256u * j + tid;
-            r[j] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
+            r[j] = i < n ? x[i] : 0.0f;
         }
     };
     auto stash = [&](uint32_t buf) {
 #pragma unroll
-        for (int j = 0; j < 16; j++) tile[buf][256u * j + tid] = r[j];
+        for (int j = 0; j < 16; j++) L.t[buf][256u * j + tid] = r[j];
     };
+    if (tid == 0) L.stop = 0u;
     fetch(0);
     stash(0);
     __syncthreads();
-    float acc = 0.0f;
     for (uint32_t base = 0, buf = 0; base < n; base += OXB_SUM_TILE, buf ^= 1u) {
         const bool more = base + OXB_SUM_TILE < n;  // uniform
         if (more) fetch(base + OXB_SUM_TILE);
         if (wave == 0) {
-            for (uint32_t g = 0; g < OXB_SUM_TILE / 256u && base + 256u * g < n; g++) {
+            bool stop = false;
+            for (uint32_t g = 0; g < OXB_SUM_TILE / 256u && base + 256u * g < n && !stop; g++) {
                 float cur[4];
 #pragma unroll
-                for (int c = 0; c < 4; c++) cur[c] = tile[buf][256u * g + 64u * c + lane];
-                if (!chain_fast<4>(acc, cur)) {
-#pragma unroll
-                    for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
-                }
+                for (int c = 0; c < 4; c++) cur[c] = L.t[buf][256u * g + 64u * c + lane];
+                stop = visit(base + 256u * g, cur);
             }
+            if (stop && lane == 0) L.stop = 1u;
         }
         if (more) stash(buf ^ 1u);
         __syncthreads();
+        if (L.stop) break;
     }
-    if (tid == 0) sum[blockIdx.x] = acc;
+    __syncthreads();  // everybody has read the flag and the tiles before the next walk rewrites them
+}
+
+// acc + the 256 values of cur in element order.
+__device__ __forceinline__ float add256(float acc, const float (&cur)[4]) {
+    float a = acc;
+    if (chain_fast<4>(a, cur)) return a;
+#pragma unroll
+    for (int c = 0; c < 4; c++) acc = chain64(acc, cur[c]);
+    return acc;
+}
+
+// sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One workgroup per row.
+__global__ __launch_bounds__(256) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
+    __shared__ RowTiles L;
+    float acc = 0.0f;
+    walk_row(e + (size_t)blockIdx.x * stride, n, L, [&](uint32_t, const float (&cur)[4]) {
+        acc = add256(acc, cur);
+        return false;
+    });
+    if (threadIdx.x == 0) sum[blockIdx.x] = acc;
 }
 
 __global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t stride, uint32_t n, const float* __restrict__ sum) {
@@ -436,13 +460,48 @@ __global__ __launch_bounds__(256) void sorted_exp_kernel(const float* __restrict
 }
 
 // Top-p cut, renormalisation, draw and pick over the row's probabilities p (sorted descending with their token ids
-// when top-p is on, else in index order with ids = null).  One wave per row; every sum is a chain in element order.
-__global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t stride,
-                                                        uint32_t n, float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
-    const uint32_t row = blockIdx.x, lane = threadIdx.x;
+// when top-p is on or top-k was taken by sorting, else in index order with ids = null).  One workgroup per row; every
+// sum runs in element order (walk_row; 256 elements at a time where chain_fast can, one by one around the element a
+// threshold is crossed at).
+__global__ __launch_bounds__(256) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t stride,
+                                                         uint32_t n, float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
+    __shared__ RowTiles L;
+    __shared__ uint32_t sh_m;
+    __shared__ float sh_s2;
+    const uint32_t row = blockIdx.x, tid = threadIdx.x;
     const float* p = p_all + (size_t)row * stride;
     const uint32_t* ids = ids_all ? ids_all + (size_t)row * stride : nullptr;
     auto lane_value = [](float x, uint32_t l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), (int)l)); };
+    uint64_t x64 = rng[row];  // read by everybody before the first barrier; written once at the very end
+    x64 ^= x64 << 13;
+    x64 ^= x64 >> 7;
+    x64 ^= x64 << 17;
+    const float r = (float)((double)x64 / 18446744073709551615.0);
+    // First position at which the running sum of q (taken from `cum`) satisfies pred, within the 256 elements of q;
+    // cum is advanced over the chunks before it.  Returns false if there is none (cum then covers all 256).
+    auto cross = [&](float& cum, const float (&q)[4], uint32_t base, auto pred, uint32_t& where) -> bool {
+        const float all = add256(cum, q);
+        if (!pred(all)) {  // the terms are >= 0: no partial sum is larger than the last
+            cum = all;
+            return false;
+        }
+#pragma unroll
+        for (int c = 0; c < 4; c++) {
+            const float end = add64(cum, q[c]);
+            if (pred(end)) {
+                float s = cum;
+                for (uint32_t l = 0; l < 64; l++) {
+                    s += lane_value(q[c], l);
+                    if (pred(s)) {
+                        where = base + 64u * c + l;
+                        return true;
+                    }
+                }
+            }
+            cum = end;
+        }
+        return false;  // not reached: add256 and the chunk-wise sums agree bit for bit
+    };
     uint32_t m = n;
     float s2 = 1.0f;
     const bool cut = top_p < 1.0f;
@@ -450,51 +509,30 @@ __global__ __launch_bounds__(64) void full_pick_kernel(const float* __restrict__
         // position(|p| { cum += p; cum > top_p }).unwrap_or(len - 1), sampling.rs:138-146
         uint32_t cutoff = n - 1;
         float cum = 0.0f;
-        for (uint32_t base = 0; base < n; base += 64) {
-            const float x = base + lane < n ? p[base + lane] : 0.0f;
-            const float end = add64(cum, x);
-            if (end > top_p) {  // probabilities are >= 0, the running sum does not fall: the crossing is in this chunk
-                float c = cum;
-                for (uint32_t l = 0; l < 64; l++) {
-                    c += lane_value(x, l);
-                    if (c > top_p) {
-                        cutoff = base + l;
-                        break;
-                    }
-                }
-                break;
-            }
-            cum = end;
-        }
-        m = cutoff + 1;
-        s2 = 0.0f;  // the renormalising sum over the kept entries, :150-152
-        for (uint32_t base = 0; base < m; base += 64) s2 = add64(s2, base + lane < m ? p[base + lane] : 0.0f);
+        walk_row(p, n, L, [&](uint32_t base, const float (&cur)[4]) {
+            return cross(cum, cur, base, [&](float v) { return v > top_p; }, cutoff);
+        });
+        if (tid == 0) sh_m = cutoff + 1;
+        __syncthreads();
+        m = sh_m;
+        float acc = 0.0f;  // the renormalising sum over the kept entries, :150-152
+        walk_row(p, m, L, [&](uint32_t, const float (&cur)[4]) {
+            acc = add256(acc, cur);
+            return false;
+        });
+        if (tid == 0) sh_s2 = acc;
+        __syncthreads();
+        s2 = sh_s2;
     }
-    uint64_t x64 = rng[row];
-    x64 ^= x64 << 13;
-    x64 ^= x64 >> 7;
-    x64 ^= x64 << 17;
-    const float r = (float)((double)x64 / 18446744073709551615.0);
     uint32_t pick = 0;  // the fallback is the buffer's first entry, :173-174
     float cum = 0.0f;
-    for (uint32_t base = 0; base < m; base += 64) {
-        float x = base + lane < m ? p[base + lane] : 0.0f;
-        if (cut) x /= s2;
-        const float end = add64(cum, x);
-        if (r <= end) {
-            float c = cum;
-            for (uint32_t l = 0; l < 64; l++) {
-                c += lane_value(x, l);
-                if (r <= c) {
-                    pick = base + l;
-                    break;
-                }
-            }
-            break;
-        }
-        cum = end;
-    }
-    if (lane == 0) {
+    walk_row(p, m, L, [&](uint32_t base, const float (&cur)[4]) {
+        float q[4];
+#pragma unroll
+        for (int c = 0; c < 4; c++) q[c] = cut ? cur[c] / s2 : cur[c];
+        return cross(cum, q, base, [&](float v) { return r <= v; }, pick);
+    });
+    if (tid == 0) {
         rng[row] = x64;
         tokens[row] = ids ? ids[pick] : pick;
     }
@@ -577,7 +615,7 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
         hipLaunchKernelGGL(sorted_exp_kernel, dim3(kparts, batch), dim3(256), 0, st, ps, n, top_k, e);
         hipLaunchKernelGGL(full_sum_kernel, dim3(batch), dim3(256), 0, st, e, n, top_k, sum);
         hipLaunchKernelGGL(full_prob_kernel, dim3(kparts, batch), dim3(256), 0, st, e, n, top_k, sum);
-        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, is, n, top_k, top_p, d_rng, d_tokens);
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(256), 0, st, e, is, n, top_k, top_p, d_rng, d_tokens);
         return hipGetLastError();
     }
     hipLaunchKernelGGL(full_max_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, pmax);
@@ -586,9 +624,9 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
     hipLaunchKernelGGL(full_prob_kernel, dim3(parts, batch), dim3(256), 0, st, e, n, n, sum);
     if (top_p < 1.0f) {
         if ((err = sort_rows()) != hipSuccess) return err;  // stable: equal probabilities keep index order, as sort_by does
-        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, ps, is, n, n, top_p, d_rng, d_tokens);
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(256), 0, st, ps, is, n, n, top_p, d_rng, d_tokens);
     } else {
-        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(64), 0, st, e, (const uint32_t*)nullptr, n, n, top_p, d_rng, d_tokens);
+        hipLaunchKernelGGL(full_pick_kernel, dim3(batch), dim3(256), 0, st, e, (const uint32_t*)nullptr, n, n, top_p, d_rng, d_tokens);
     }
     return hipGetLastError();
 }
