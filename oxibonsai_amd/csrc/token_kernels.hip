@@ -367,54 +367,6 @@ __device__ __forceinline__ float add64(float acc, float x) {
     return chain64(acc, x);
 }
 
-// Brings x[0 .. n) to the first wave in element order, 256 elements per call of visit(base, cur) with
-// cur[c] = x[base + 64 c + lane] (+0 past n); visit returns true to end the walk.  All four waves load, 4096 elements at
-// a time, through two LDS tiles: the next tile's loads are in flight while the current one is visited.  Every thread
-// of the workgroup must call it (barriers inside); what visit changes is valid in the first wave only.
-#define OXB_SUM_TILE 4096u
-struct RowTiles {
-    float t[2][OXB_SUM_TILE];
-    uint32_t stop;
-};
-template <class Visit>
-__device__ __forceinline__ void walk_row(const float* __restrict__ x, uint32_t n, RowTiles& L, Visit&& visit) {
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    float r[16];
-    auto fetch = [&](uint32_t base) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t i = base + 256u * j + tid;
-            r[j] = i < n ? x[i] : 0.0f;
-        }
-    };
-    auto stash = [&](uint32_t buf) {
-#pragma unroll
-        for (int j = 0; j < 16; j++) L.t[buf][256u * j + tid] = r[j];
-    };
-    if (tid == 0) L.stop = 0u;
-    fetch(0);
-    stash(0);
-    __syncthreads();
-    for (uint32_t base = 0, buf = 0; base < n; base += OXB_SUM_TILE, buf ^= 1u) {
-        const bool more = base + OXB_SUM_TILE < n;  // uniform
-        if (more) fetch(base + OXB_SUM_TILE);
-        if (wave == 0) {
-            bool stop = false;
-            for (uint32_t g = 0; g < OXB_SUM_TILE / 256u && base + 256u * g < n && !stop; g++) {
-                float cur[4];
-#pragma unroll
-                for (int c = 0; c < 4; c++) cur[c] = L.t[buf][256u * g + 64u * c + lane];
-                stop = visit(base + 256u * g, cur);
-            }
-            if (stop && lane == 0) L.stop = 1u;
-        }
-        if (more) stash(buf ^ 1u);
-        __syncthreads();
-        if (L.stop) break;
-    }
-    __syncthreads();  // everybody has read the flag and the tiles before the next walk rewrites them
-}
-
 // acc + the 256 values of cur in element order.
 __device__ __forceinline__ float add256(float acc, const float (&cur)[4]) {
     float a = acc;
@@ -424,15 +376,149 @@ __device__ __forceinline__ float add256(float acc, const float (&cur)[4]) {
     return acc;
 }
 
+// What chain_fast needs from 256 elements when none of them is a rounding tie: the sum of the mantissa increments for a
+// running sum with biased exponent es.  `refuse` is set if chain_fast would refuse the elements or if one is a tie.
+__device__ __forceinline__ uint32_t increments256(uint32_t es, const float (&x)[4], bool& refuse) {
+    uint32_t f_sum = 0;
+    bool bad = es == 0 || es >= 255;
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        const uint32_t b = __float_as_uint(x[c]), ex0 = b >> 23;
+        uint32_t m = b & 0x7FFFFFu;
+        const uint32_t ex = ex0 ? ex0 : 1u;
+        if (ex0) m |= 0x800000u;
+        const int shr = (int)es - (int)ex;
+        if (m != 0u) {
+            if (ex0 >= 255u || shr <= 0) {
+                bad = true;
+            } else if (shr <= 24) {
+                const uint32_t rem = m & ((1u << shr) - 1u), half = 1u << (shr - 1);
+                f_sum += (m >> shr) + (rem > half ? 1u : 0u);
+                bad |= rem == half;
+            }
+        }
+    }
+    refuse = __builtin_amdgcn_ballot_w64(bad) != 0ull;
+    return wave_sum_u32(f_sum);
+}
+
+// The running f32 sum of x[0 .. n) (each element divided by `divisor` first if `divide`), taken in element order
+// from L.acc, up to the first element at which pred(sum) holds: returns true and its position in `where`, or false
+// with the whole sum.  L.acc holds the sum reached in either case.  One workgroup of four waves, all threads call:
+//  * the row comes through two LDS tiles of 4096 elements, the next tile's loads in flight while this one is summed;
+//  * the four waves take the four 256-element groups of a 1024-element batch at once, each forming its group's mantissa
+//    increments for the binade the sum is in at the start of the batch (increments256).  If no group refuses and the
+//    mantissa stays inside the binade, the batch's result is the integer sum - the order does not matter then;
+//  * otherwise, or when pred holds after the batch, the first wave redoes the batch group by group in order
+//    (add256, add64, and lane by lane around the crossing).
+struct RowSum {
+    float t[2][4096];
+    uint32_t inc[4], refuse[4];
+    float acc;
+    uint32_t stop, where;
+};
+template <class Pred>
+__device__ __forceinline__ bool run_sum(const float* __restrict__ x, uint32_t n, bool divide, float divisor, RowSum& L, Pred pred,
+                                        uint32_t& where) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    auto lane_value = [](float v, uint32_t l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), (int)l)); };
+    float r[16];
+    auto fetch = [&](uint32_t base) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t i = base + 256u * j + tid;
+            r[j] = i < n ? x[i] : 0.0f;  // adding +0 past the end changes nothing
+        }
+    };
+    auto stash = [&](uint32_t buf) {
+#pragma unroll
+        for (int j = 0; j < 16; j++) L.t[buf][256u * j + tid] = divide ? r[j] / divisor : r[j];
+    };
+    if (tid == 0) L.stop = 0u;
+    fetch(0);
+    stash(0);
+    __syncthreads();
+    for (uint32_t base = 0, buf = 0; base < n; base += 4096u, buf ^= 1u) {
+        const bool more = base + 4096u < n;  // uniform
+        if (more) fetch(base + 4096u);
+        for (uint32_t bb = 0; bb < 4096u && base + bb < n; bb += 1024u) {
+            float cur[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) cur[c] = L.t[buf][bb + 256u * wave + 64u * c + lane];
+            const uint32_t sb = __float_as_uint(L.acc), es = sb >> 23;
+            bool refuse;
+            const uint32_t inc = increments256(es, cur, refuse);
+            if (lane == 0) L.inc[wave] = inc, L.refuse[wave] = refuse ? 1u : 0u;
+            __syncthreads();
+            if (wave == 0) {
+                uint32_t total = (sb & 0x7FFFFFu) | 0x800000u;
+                bool slow = false;
+                for (uint32_t w = 0; w < 4 && base + bb + 256u * w < n; w++) {
+                    total += L.inc[w];  // each < 2^30: no overflow before the check
+                    slow |= L.refuse[w] != 0u || total >= 0x1000000u;
+                }
+                const float fast = __uint_as_float((es << 23) | (total & 0x7FFFFFu));
+                if (!slow && !pred(fast)) {  // the terms are >= 0: no partial sum exceeds the last
+                    if (lane == 0) L.acc = fast;
+                } else {
+                    float cum = L.acc;
+                    bool found = false;
+                    uint32_t at = 0;
+                    for (uint32_t w = 0; w < 4 && base + bb + 256u * w < n && !found; w++) {
+                        float q[4];
+#pragma unroll
+                        for (int c = 0; c < 4; c++) q[c] = L.t[buf][bb + 256u * w + 64u * c + lane];
+                        const float all = add256(cum, q);
+                        if (!pred(all)) {
+                            cum = all;
+                            continue;
+                        }
+                        for (uint32_t c = 0; c < 4 && !found; c++) {
+                            const float qc = c == 0 ? q[0] : (c == 1 ? q[1] : (c == 2 ? q[2] : q[3]));
+                            const float end = add64(cum, qc);
+                            if (pred(end)) {
+                                float s2 = cum;
+                                for (uint32_t l = 0; l < 64; l++) {
+                                    s2 += lane_value(qc, l);
+                                    if (pred(s2)) {
+                                        at = base + bb + 256u * w + 64u * c + l;
+                                        cum = s2;
+                                        found = true;
+                                        break;
+                                    }
+                                }
+                            } else {
+                                cum = end;
+                            }
+                        }
+                    }
+                    if (lane == 0) {
+                        L.acc = cum;
+                        if (found) L.stop = 1u, L.where = at;
+                    }
+                }
+            }
+            __syncthreads();
+            if (L.stop) break;
+        }
+        if (L.stop) break;  // uniform
+        if (more) stash(buf ^ 1u);
+        __syncthreads();
+    }
+    const bool hit = L.stop != 0u;
+    if (hit) where = L.where;
+    __syncthreads();  // everybody has read the result before the next run rewrites the flags and tiles
+    return hit;
+}
+
 // sum[row] = e[row][0] + e[row][1] + ... in element order (sampling.rs:126-130).  One workgroup per row.
 __global__ __launch_bounds__(256) void full_sum_kernel(const float* __restrict__ e, uint32_t stride, uint32_t n, float* __restrict__ sum) {
-    __shared__ RowTiles L;
-    float acc = 0.0f;
-    walk_row(e + (size_t)blockIdx.x * stride, n, L, [&](uint32_t, const float (&cur)[4]) {
-        acc = add256(acc, cur);
-        return false;
-    });
-    if (threadIdx.x == 0) sum[blockIdx.x] = acc;
+    __shared__ RowSum L;
+    if (threadIdx.x == 0) L.acc = 0.0f;
+    __syncthreads();
+    uint32_t unused = 0;
+    run_sum(e + (size_t)blockIdx.x * stride, n, false, 1.0f, L, [](float) { return false; }, unused);
+    if (threadIdx.x == 0) sum[blockIdx.x] = L.acc;
 }
 
 __global__ __launch_bounds__(256) void full_prob_kernel(float* __restrict__ e, uint32_t stride, uint32_t n, const float* __restrict__ sum) {
@@ -461,46 +547,21 @@ __global__ __launch_bounds__(256) void sorted_exp_kernel(const float* __restrict
 
 // Top-p cut, renormalisation, draw and pick over the row's probabilities p (sorted descending with their token ids
 // when top-p is on or top-k was taken by sorting, else in index order with ids = null).  One workgroup per row; every
-// sum runs in element order (walk_row; 256 elements at a time where chain_fast can, one by one around the element a
-// threshold is crossed at).
+// sum runs in element order (run_sum).
 __global__ __launch_bounds__(256) void full_pick_kernel(const float* __restrict__ p_all, const uint32_t* __restrict__ ids_all, uint32_t stride,
                                                          uint32_t n, float top_p, uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
-    __shared__ RowTiles L;
-    __shared__ uint32_t sh_m;
-    __shared__ float sh_s2;
+    __shared__ RowSum L;
     const uint32_t row = blockIdx.x, tid = threadIdx.x;
     const float* p = p_all + (size_t)row * stride;
     const uint32_t* ids = ids_all ? ids_all + (size_t)row * stride : nullptr;
-    auto lane_value = [](float x, uint32_t l) { return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, x), (int)l)); };
     uint64_t x64 = rng[row];  // read by everybody before the first barrier; written once at the very end
     x64 ^= x64 << 13;
     x64 ^= x64 >> 7;
     x64 ^= x64 << 17;
     const float r = (float)((double)x64 / 18446744073709551615.0);
-    // First position at which the running sum of q (taken from `cum`) satisfies pred, within the 256 elements of q;
-    // cum is advanced over the chunks before it.  Returns false if there is none (cum then covers all 256).
-    auto cross = [&](float& cum, const float (&q)[4], uint32_t base, auto pred, uint32_t& where) -> bool {
-        const float all = add256(cum, q);
-        if (!pred(all)) {  // the terms are >= 0: no partial sum is larger than the last
-            cum = all;
-            return false;
-        }
-#pragma unroll
-        for (int c = 0; c < 4; c++) {
-            const float end = add64(cum, q[c]);
-            if (pred(end)) {
-                float s = cum;
-                for (uint32_t l = 0; l < 64; l++) {
-                    s += lane_value(q[c], l);
-                    if (pred(s)) {
-                        where = base + 64u * c + l;
-                        return true;
-                    }
-                }
-            }
-            cum = end;
-        }
-        return false;  // not reached: add256 and the chunk-wise sums agree bit for bit
+    auto restart = [&]() {
+        if (tid == 0) L.acc = 0.0f;
+        __syncthreads();
     };
     uint32_t m = n;
     float s2 = 1.0f;
@@ -508,30 +569,18 @@ __global__ __launch_bounds__(256) void full_pick_kernel(const float* __restrict_
     if (cut) {
         // position(|p| { cum += p; cum > top_p }).unwrap_or(len - 1), sampling.rs:138-146
         uint32_t cutoff = n - 1;
-        float cum = 0.0f;
-        walk_row(p, n, L, [&](uint32_t base, const float (&cur)[4]) {
-            return cross(cum, cur, base, [&](float v) { return v > top_p; }, cutoff);
-        });
-        if (tid == 0) sh_m = cutoff + 1;
+        restart();
+        run_sum(p, n, false, 1.0f, L, [&](float v) { return v > top_p; }, cutoff);
+        m = cutoff + 1;
+        restart();  // the renormalising sum over the kept entries, :150-152
+        uint32_t unused = 0;
+        run_sum(p, m, false, 1.0f, L, [](float) { return false; }, unused);
+        s2 = L.acc;
         __syncthreads();
-        m = sh_m;
-        float acc = 0.0f;  // the renormalising sum over the kept entries, :150-152
-        walk_row(p, m, L, [&](uint32_t, const float (&cur)[4]) {
-            acc = add256(acc, cur);
-            return false;
-        });
-        if (tid == 0) sh_s2 = acc;
-        __syncthreads();
-        s2 = sh_s2;
     }
     uint32_t pick = 0;  // the fallback is the buffer's first entry, :173-174
-    float cum = 0.0f;
-    walk_row(p, m, L, [&](uint32_t base, const float (&cur)[4]) {
-        float q[4];
-#pragma unroll
-        for (int c = 0; c < 4; c++) q[c] = cut ? cur[c] / s2 : cur[c];
-        return cross(cum, q, base, [&](float v) { return r <= v; }, pick);
-    });
+    restart();
+    run_sum(p, m, cut, s2, L, [&](float v) { return r <= v; }, pick);
     if (tid == 0) {
         rng[row] = x64;
         tokens[row] = ids ? ids[pick] : pick;
