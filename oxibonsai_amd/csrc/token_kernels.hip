@@ -65,7 +65,7 @@ __global__ void token_step_kernel(const uint32_t* __restrict__ tokens, uint32_t*
 // barrier in the loop); the four sorted lists meet in LDS and wave 0 merges them the same way: the span's top_k
 // in descending order, ties to the lower index.  Stage 2, one wave per row: a lane walks up to four of the parts'
 // sorted lists (the next element of each already requested) and the same pop yields the row's top_k in descending
-// order; lane 0 then walks the reference's arithmetic over those <= 128 values: v / temperature, exp(v - max),
+// order; lane 0 then walks the reference's arithmetic over those <= 128 values: v / temperature, exp(v - max) (formed by all lanes),
 // sum, divide, top-p cut, renormalise, r = (xorshift64 / u64::MAX) as f32, cumulative pick (first candidate if
 // none reaches r).  The reference leaves the candidates in whatever order its partial selection produces when
 // top_p == 1; here the order is always descending.
@@ -195,15 +195,27 @@ __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restric
         if (lane == 0) pv[j] = key_value(best), pi[j] = key_index(best);
         k = j + 1;
     }
-    if (lane != 0) return;
-    // pv[0..k) descending.  From here on: sampling.rs:104-176 on the k candidates.
-    for (uint32_t j = 0; j < k; j++) pv[j] = pv[j] / temperature;
-    const float max_val = pv[0];
-    float sum = 0.0f;
-    for (uint32_t j = 0; j < k; j++) {
-        pv[j] = expf(pv[j] - max_val);
-        sum += pv[j];
+    // pv[0..k) descending.  From here on: sampling.rs:104-176 on the k candidates.  The element-wise part on all
+    // lanes (the exponential through double precision: the nearest f32, as libm's expf gives in all but rare cases),
+    // the sums by lane 0 in the reference's order.
+    __syncthreads();
+    if (k > 0) {
+        const float max_val = pv[0] / temperature;
+        float e[(OXB_SAMPLE_MAX_TOP_K + 63) / 64];
+#pragma unroll
+        for (uint32_t q = 0; q < (OXB_SAMPLE_MAX_TOP_K + 63) / 64; q++) {
+            const uint32_t j = lane + 64u * q;
+            e[q] = j < k ? (float)exp((double)(pv[j] / temperature - max_val)) : 0.0f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t q = 0; q < (OXB_SAMPLE_MAX_TOP_K + 63) / 64; q++)
+            if (lane + 64u * q < k) pv[lane + 64u * q] = e[q];
     }
+    __syncthreads();
+    if (lane != 0) return;
+    float sum = 0.0f;
+    for (uint32_t j = 0; j < k; j++) sum += pv[j];
     for (uint32_t j = 0; j < k; j++) pv[j] /= sum;
     if (top_p < 1.0f) {
         float cum = 0.0f;
