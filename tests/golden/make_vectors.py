@@ -50,6 +50,18 @@ def build() -> dict:
                         ("e4m3", dict(kv_mode=oracle.KV_FP8_E4M3)), ("f16_w4_1", dict(kv_mode=oracle.KV_F16, window=4, sinks=1))):
             mdl = oracle.OracleModel(cfg, w, **kw)
             out[f"model_{name}_{tag}_logits"] = np.stack([mdl.forward(h, p) for p, h in enumerate(hid)])
+    # Sampler::sample: logits, parameters, seeds -> tokens and advanced generator states, for the three routes
+    # (top-k by selection, top-k by sorting, filter off)
+    lg = (synth.normal_f32(70, 4 * 3000) * 3.0).reshape(4, 3000)
+    lg[1, 5] = lg[1, 1234] = lg[1].max() + 0.5
+    seeds = np.array([1, 2**63 + 5, 0x9E3779B97F4A7C15, 424242], dtype=np.uint64)
+    out["sample_logits"], out["sample_seeds"] = lg, seeds
+    for tag, (T, k, tp) in (("k40", (0.7, 40, 0.9)), ("k300", (1.0, 300, 0.95)), ("off_p95", (1.0, 0, 0.95)), ("off_p1", (0.8, 0, 1.0))):
+        res = [oracle.sample(lg[b], T, k, tp, int(seeds[b])) for b in range(4)]
+        out[f"sample_{tag}_params"] = np.array([T, k, tp], dtype=np.float64)
+        out[f"sample_{tag}_tokens"] = np.array([r[0] for r in res], dtype=np.uint32)
+        out[f"sample_{tag}_states"] = np.array([r[1] for r in res], dtype=np.uint64)
+        out[f"sample_{tag}_draws"] = np.array([r[4] for r in res], dtype=np.float32)
     return out
 
 
