@@ -156,8 +156,7 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
     t0 = time.perf_counter()
     m.generate_sampled(emb_tab, [tok], [prompt_len + n_tokens], n_tokens, 0.7, 40, 0.9, [0xB0A5A1])   # the reference's defaults
     t_smp = time.perf_counter() - t0
-    # the Creative preset: top-k off, softmax / sort / top-p over the whole vocabulary (random-init logits are nearly
-    # flat, so the nucleus holds most of the 151 936 tokens: the slowest case of the sequential sums)
+    # the Creative preset: top-k off, softmax / sort / top-p over the whole vocabulary of 151 936 logits
     t0 = time.perf_counter()
     m.generate_sampled(emb_tab, [tok], [prompt_len + 2 * n_tokens], n_tokens, 1.0, 0, 0.95, [0xB0A5A1])
     t_full = time.perf_counter() - t0
@@ -165,7 +164,7 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
                           "ms_per_token": round(t_dev / n_tokens * 1e3, 4), "embedding": "Q1_0_g128 table on the device",
                           "sampled_tok_per_s": round(n_tokens / t_smp, 2), "sampling": "temperature 0.7, top-k 40, top-p 0.9",
                           "sampled_filter_off_tok_per_s": round(n_tokens / t_full, 2),
-                          "sampling_filter_off": "temperature 1.0, top-k 0, top-p 0.95 over 151936 nearly flat logits"}
+                          "sampling_filter_off": "temperature 1.0, top-k 0 (filter off), top-p 0.95 over the 151936 logits"}
     m.close()
     if with_gguf:
         # checkpoint file -> device: the same tensors written as a GGUF file (page cache), loaded by oxb_hip_load_gguf
