@@ -227,8 +227,10 @@ def test_device_sampler_with_the_filter_off(backend, n, T, tp, top_k):
 
 
 @pytest.mark.gpu
-def test_sampled_generation_loop(backend, tmp_path):
-    """Token loop with the sampler: every step's token is the sampler's pick from that step's logits."""
+@pytest.mark.parametrize("T,k,tp", [(0.9, 20, 0.95), (1.0, 0, 0.95), (0.8, 0, 1.0), (0.9, 200, 0.9)])
+def test_sampled_generation_loop(backend, tmp_path, T, k, tp):
+    """Token loop with the sampler (top-k by selection, filter off with and without top-p, top-k by sorting): every
+    step's token is the sampler's pick from that step's logits."""
     from helpers import GGUF_F16, TQ2, model_gguf
     from oxibonsai_amd.model import HipModel
     cfg = dict(fmt=TQ2, n_layers=2, h=512, inter=1024, nq=8, nkv=2, hd=64, vocab=300, max_seq=128, eps=1e-6, rope_theta=1e6)
@@ -238,7 +240,6 @@ def test_sampled_generation_loop(backend, tmp_path):
     a, emb, _ = HipModel.from_gguf(backend, str(tmp_path / "m.gguf"), batch=2)
     b = HipModel(backend, cfg, w, batch=2)
     try:
-        T, k, tp = 0.9, 20, 0.95
         seeds = np.array([7, 1234567], dtype=np.uint64)
         ids, states = a.generate_sampled(emb, [5, 17], [0, 0], 12, T, k, tp, seeds)
         toks, st = np.array([5, 17], dtype=np.uint32), [int(s) for s in seeds]
@@ -247,7 +248,8 @@ def test_sampled_generation_loop(backend, tmp_path):
             for s in range(2):
                 tok, st[s], cand, p, r = oracle.sample(logits[s], T, k, tp, st[s])
                 if int(ids[i, s]) != tok:
-                    assert int(ids[i, s]) in cand and np.min(np.abs(np.cumsum(p.astype(np.float64)) - r)) < 1e-5
+                    cum = np.cumsum(p, dtype=np.float32)                # sequential f32, the sampler's own sums
+                    assert int(ids[i, s]) in cand and np.min(np.abs(cum - r)) < 1e-5
             toks = ids[i].copy()                                       # follow the device's own tokens
         assert [int(s) for s in states] == st
         greedy = a.generate(emb, [5, 17], [0, 0], 4)
