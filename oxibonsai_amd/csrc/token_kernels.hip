@@ -156,19 +156,42 @@ __global__ __launch_bounds__(256) void topk_partial_kernel(const float* __restri
 }
 
 #define OXB_SAMPLE_LISTS_PER_LANE 4  // stage 2 walks up to 256 parts with one wave
+#define OXB_SAMPLE_LDS_KEYS 6144     // the parts' lists are walked out of LDS when they fit (48 KB of keys)
+template <bool IN_LDS>
 __global__ __launch_bounds__(64) void sample_final_kernel(const float* __restrict__ cv, const uint32_t* __restrict__ ci,
                                                            uint32_t parts, uint32_t top_k, float temperature, float top_p,
                                                            uint64_t* __restrict__ rng, uint32_t* __restrict__ tokens) {
     __shared__ float pv[OXB_SAMPLE_MAX_TOP_K];
     __shared__ uint32_t pi[OXB_SAMPLE_MAX_TOP_K];
+    __shared__ uint64_t keys[IN_LDS ? OXB_SAMPLE_LDS_KEYS : 1];
     const uint32_t row = blockIdx.x, lane = threadIdx.x;
     const float* lv = cv + (size_t)row * parts * top_k;
     const uint32_t* li = ci + (size_t)row * parts * top_k;
+    if (IN_LDS) {  // one pass over the lists with every load in flight, instead of a trip to memory per pop
+        const uint32_t total = parts * top_k;
+        for (uint32_t e0 = 0; e0 < total; e0 += 64 * 16) {  // sixteen loads of each array in flight per lane
+            uint32_t i[16];
+            float v[16];
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const uint32_t e = e0 + 64u * u + lane;
+                i[u] = e < total ? li[e] : 0xFFFFFFFFu;
+                v[u] = e < total ? lv[e] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 16; u++) {
+                const uint32_t e = e0 + 64u * u + lane;
+                if (e < total) keys[e] = i[u] == 0xFFFFFFFFu ? 0ull : cand_key(v[u], i[u]);
+            }
+        }
+        __syncthreads();
+    }
     // lane t walks the sorted lists of parts t, t + 64, ...: `cur` is each list's head, `nxt` the element behind it
     uint64_t cur[OXB_SAMPLE_LISTS_PER_LANE], nxt[OXB_SAMPLE_LISTS_PER_LANE];
     uint32_t head[OXB_SAMPLE_LISTS_PER_LANE];
     auto fetch = [&](uint32_t part, uint32_t at) -> uint64_t {
         if (part >= parts || at >= top_k) return 0ull;
+        if (IN_LDS) return keys[part * top_k + at];
         const uint32_t i = li[(size_t)part * top_k + at];
         return i == 0xFFFFFFFFu ? 0ull : cand_key(lv[(size_t)part * top_k + at], i);
     };
@@ -708,6 +731,9 @@ hipError_t oxb_launch_sample(const float* d_logits, uint32_t n, uint32_t batch, 
     float* cv = reinterpret_cast<float*>(d_ws);
     uint32_t* ci = reinterpret_cast<uint32_t*>(d_ws) + (size_t)batch * parts * top_k;
     hipLaunchKernelGGL(topk_partial_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, top_k, cv, ci);
-    hipLaunchKernelGGL(sample_final_kernel, dim3(batch), dim3(64), 0, st, cv, ci, parts, top_k, temperature, top_p, d_rng, d_tokens);
+    if (parts * top_k <= OXB_SAMPLE_LDS_KEYS)
+        hipLaunchKernelGGL(sample_final_kernel<true>, dim3(batch), dim3(64), 0, st, cv, ci, parts, top_k, temperature, top_p, d_rng, d_tokens);
+    else
+        hipLaunchKernelGGL(sample_final_kernel<false>, dim3(batch), dim3(64), 0, st, cv, ci, parts, top_k, temperature, top_p, d_rng, d_tokens);
     return hipGetLastError();
 }

@@ -126,7 +126,7 @@ def test_unfiltered_path_follows_the_definition():
 # --------------------------------------------------------------------------- GPU
 @pytest.mark.gpu
 @pytest.mark.parametrize("n,T,k,tp", [(151936, 0.7, 40, 0.9), (5000, 1.0, 128, 1.0), (33, 0.5, 40, 0.95), (4096, 2.0, 1, 0.9),
-                                      (2049, 0.7, 5, 1.0), (100000, 1e-3, 40, 0.9)])
+                                      (2049, 0.7, 5, 1.0), (100000, 1e-3, 40, 0.9), (151936, 1.0, 128, 0.9), (151936, 0.9, 82, 1.0)])
 def test_device_sampler_matches_restatement(backend, n, T, k, tp):
     from oxibonsai_amd.model import sample_logits
     rows = 6
