@@ -209,6 +209,7 @@ typedef struct {
     uint32_t n_layers, h, inter, nq, nkv, hd, vocab, context_length;
     float eps, rope_theta;
     char architecture[32], name[64];
+    uint32_t lm_head_rows;          /* rows of output.weight = logits per position (model/weight_loaders.rs:654-666); `vocab` counts the rows of token_embd.weight */
 } oxb_gguf_info;
 int  oxb_hip_gguf_info(const char* path, oxb_gguf_info* info);
 /* Directory access without a GPU: one metadata value rendered as text (integers, floats with %.9g, strings as they

@@ -63,6 +63,7 @@ struct Model {
     uint32_t chunk = 0, n_splits = 0;
     // graph
     hipGraphExec_t graph_exec = nullptr;
+    uint64_t graph_gen = 0;  // g_rt.weights_gen at capture: the graph holds the weights' device pointers of that moment
     bool graph_failed = false;
     bool want_logits_in_graph = true;
     std::vector<void*> allocs;
@@ -532,6 +533,7 @@ using namespace oxb;
 extern "C" {
 
 int oxb_hip_upload_f32(uint64_t* id, const float* w, size_t n) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!id || !w || n == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or empty vector");
     OXB_TRY(ensure_init());
@@ -550,19 +552,27 @@ int oxb_hip_upload_f32(uint64_t* id, const float* w, size_t n) {
     }
     if (*id == 0) *id = g_rt.next_id++;
     auto it = g_rt.vectors.find(*id);
-    if (it != g_rt.vectors.end()) (void)hipFree(it->second.d);
+    if (it != g_rt.vectors.end()) {
+        (void)hipStreamSynchronize(g_rt.stream);
+        (void)hipFree(it->second.d);
+        g_rt.weights_gen++;
+    }
     g_rt.vectors[*id] = v;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_free_f32(uint64_t id) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     auto it = g_rt.vectors.find(id);
     if (it == g_rt.vectors.end()) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
     if (g_rt.ready) (void)hipStreamSynchronize(g_rt.stream);
     (void)hipFree(it->second.d);
     g_rt.vectors.erase(it);
+    g_rt.weights_gen++;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 // Slots of the split-KV attention: about one workgroup (slot x kv head x sequence) per CU for the fp16 cache, two for a
@@ -621,6 +631,7 @@ static int alloc_kv_cache(Model& m, uint32_t kv_mode, uint32_t page_size, uint32
 }
 
 int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!desc || !model || !desc->layers) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer");
     OXB_TRY(ensure_init());
@@ -729,9 +740,11 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     *model = g_next_model++;
     g_models[*model] = std::move(mp);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_destroy(uint64_t model) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -742,9 +755,11 @@ int oxb_hip_model_destroy(uint64_t model) {
     for (uint64_t id : mats) (void)oxb_hip_free_weight(id);
     for (uint64_t id : vecs) (void)oxb_hip_free_f32(id);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -771,9 +786,11 @@ int oxb_hip_model_set_attention(uint64_t model, const oxb_attention_options* opt
     m->window = opt->window_size;
     m->sinks = opt->sink_tokens;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -784,10 +801,12 @@ int oxb_hip_model_get_attention(uint64_t model, oxb_attention_options* opt) {
     opt->page_size = m->n_pages ? 1u << m->page_shift : 0u;
     opt->n_pages = m->n_pages;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t kv_head, uint32_t pos, uint32_t n_pos,
                           void* k_rows, void* v_rows, float* k_scales, float* v_scales) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -828,9 +847,11 @@ int oxb_hip_model_read_kv(uint64_t model, uint32_t seq, uint32_t layer, uint32_t
             if (v_scales) v_scales[i] = 1.0f;
         }
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_kv_reserve(uint64_t model, uint32_t seq, uint32_t n_tokens) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -838,9 +859,11 @@ int oxb_hip_model_kv_reserve(uint64_t model, uint32_t seq, uint32_t n_tokens) {
     if (n_tokens > m->d.max_seq)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %u positions exceed the context of %u", n_tokens, m->d.max_seq);
     return kv_reserve(*m, seq, n_tokens);
+    OXB_API_END
 }
 
 int oxb_hip_model_kv_release(uint64_t model, uint32_t seq) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -848,9 +871,11 @@ int oxb_hip_model_kv_release(uint64_t model, uint32_t seq) {
     OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
     kv_release(*m, seq);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_kv_pool(uint64_t model, oxb_kv_pool_info* info) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -859,18 +884,22 @@ int oxb_hip_model_kv_pool(uint64_t model, oxb_kv_pool_info* info) {
     info->total_pages = m->n_pages;
     info->free_pages = (uint32_t)m->free_pages.size();
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_kv_capacity(uint64_t model, uint32_t seq, uint32_t* n_tokens) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
     if (seq >= m->d.batch || !n_tokens) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, m->d.batch);
     *n_tokens = m->n_pages ? (uint32_t)(m->seq_pages[seq].size() << m->page_shift) : m->d.max_seq;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, uint32_t n, uint8_t* codes, float* scales) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!rows || !codes || !scales) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
     if (kv_dtype != OXB_KV_DTYPE_I8 && kv_dtype != OXB_KV_DTYPE_FP8_E4M3)
@@ -892,9 +921,11 @@ int oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, u
     c.release();
     sc.release();
     return rc;
+    OXB_API_END
 }
 
 int oxb_hip_model_reset(uint64_t model) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     if (!m) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -903,17 +934,24 @@ int oxb_hip_model_reset(uint64_t model) {
     (void)hipStreamSynchronize(g_rt.stream);
     for (uint32_t b = 0; b < m->d.batch; b++) kv_release(*m, b);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 // One decode step on m.hidden / m.pos (device): replayed from the captured graph, captured on first use, or launched
 // kernel by kernel when capture is off or failed.
 static int run_decode_step(Model& m) {
     hipStream_t st = g_rt.stream;
+    if (m.graph_exec && m.graph_gen != g_rt.weights_gen) {
+        // a weight or norm vector was freed or replaced since the capture: look every handle up again
+        (void)hipGraphExecDestroy(m.graph_exec);
+        m.graph_exec = nullptr;
+    }
     if (m.graph_exec) {
         OXB_TRY_HIP(hipGraphLaunch(m.graph_exec, st), "graph launch");
     } else if (!m.graph_failed && st == g_rt.own_stream) {
         // capture the whole token once; on any capture problem fall back to plain launches for good
         hipGraph_t graph = nullptr;
+        m.graph_gen = g_rt.weights_gen;
         hipError_t e = hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal);
         int rc = OXB_HIP_OK;
         if (e == hipSuccess) {
@@ -939,6 +977,7 @@ static int run_decode_step(Model& m) {
 }
 
 int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* mp = find_model(model);
     if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -960,10 +999,12 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode: %s", hipGetErrorString(e));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t n_tokens, uint32_t pos_start,
                     float* logits_or_null, uint32_t* token_out_or_null) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* mp = find_model(model);
     if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
@@ -986,16 +1027,20 @@ int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t 
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: prefill: %s", hipGetErrorString(e));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_model_uses_graph(uint64_t model) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     return m && m->graph_exec ? 1 : 0;
+    OXB_API_END
 }
 
 int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float* norm_w, float eps, uint64_t o_id,
                       uint64_t gate_up_id, uint64_t down_id, uint32_t h, uint32_t inter, uint32_t attn_k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!hidden || !attn_out || !norm_w) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
     if (h % 128 || inter % 128 || attn_k % 128) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: dimensions must be multiples of 128");
@@ -1030,6 +1075,7 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 // ---------------------------------------------------------------------------
@@ -1041,6 +1087,7 @@ static Embedding* find_embedding(uint64_t id) {
 }
 
 int oxb_hip_upload_embedding(uint64_t* id, const void* table, size_t n_bytes, int gguf_type, uint32_t vocab, uint32_t h) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!id || !table) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null id or table");
     if (gguf_type != GGUF_F32 && gguf_type != GGUF_F16 && gguf_type != GGUF_Q1_0_G128 && gguf_type != GGUF_TQ2_0_G128)
@@ -1064,9 +1111,11 @@ int oxb_hip_upload_embedding(uint64_t* id, const void* table, size_t n_bytes, in
     if (Embedding* old = find_embedding(*id)) (void)hipFree(old->d);
     g_embeddings[*id] = e;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_free_embedding(uint64_t id) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Embedding* e = find_embedding(id);
     if (!e) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (embedding) not found", (unsigned long long)id);
@@ -1074,6 +1123,7 @@ int oxb_hip_free_embedding(uint64_t id) {
     (void)hipFree(e->d);
     g_embeddings.erase(id);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 static int check_ids(const Embedding& e, const uint32_t* ids, size_t n) {
@@ -1084,6 +1134,7 @@ static int check_ids(const Embedding& e, const uint32_t* ids, size_t n) {
 }
 
 int oxb_hip_embedding_rows(uint64_t embedding, const uint32_t* ids, uint32_t n, float* out) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Embedding* e = find_embedding(embedding);
     if (!e) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (embedding) not found", (unsigned long long)embedding);
@@ -1100,6 +1151,7 @@ int oxb_hip_embedding_rows(uint64_t embedding, const uint32_t* ids, uint32_t n, 
     hipError_t he = hipStreamSynchronize(st);
     if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: embedding_rows: %s", hipGetErrorString(he));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 static int model_and_embedding(uint64_t model, uint64_t embedding, Model** m, Embedding** e) {
@@ -1169,16 +1221,21 @@ static int decode_tokens_impl(uint64_t model, uint64_t embedding, const uint32_t
 
 int oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
                           uint32_t* tokens_out) {
+    OXB_API_BEGIN
     return decode_tokens_impl(model, embedding, tokens, pos, n_steps, nullptr, nullptr, tokens_out);
+    OXB_API_END
 }
 
 int oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos, uint32_t n_steps,
                                   const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out) {
+    OXB_API_BEGIN
     if (!params) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null sampling parameters");
     return decode_tokens_impl(model, embedding, tokens, pos, n_steps, params, rng_state, tokens_out);
+    OXB_API_END
 }
 
 int oxb_hip_sum_in_order(const float* x, uint32_t n, float* sum_out) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!x || !sum_out || n == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or no elements");
     OXB_TRY(ensure_init());
@@ -1192,10 +1249,12 @@ int oxb_hip_sum_in_order(const float* x, uint32_t n, float* sum_out) {
     hipError_t he = hipStreamSynchronize(st);
     if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: sum_in_order: %s", hipGetErrorString(he));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params, uint64_t* rng_state,
                           uint32_t* tokens_out) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!logits || !params || !rng_state || !tokens_out || vocab == 0 || batch == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null pointer or empty logits");
@@ -1224,10 +1283,12 @@ int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, c
     hipError_t he = hipStreamSynchronize(st);
     if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: sample_logits: %s", hipGetErrorString(he));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, const uint32_t* ids, uint32_t n_tokens,
                            uint32_t pos_start, float* logits_or_null, uint32_t* token_out_or_null) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* mp;
     Embedding* e;
@@ -1255,6 +1316,7 @@ int oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, con
     hipError_t he = hipStreamSynchronize(st);
     if (he != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: prefill_tokens: %s", hipGetErrorString(he));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 // --- GGUF ---------------------------------------------------------------------------------------------------
@@ -1299,6 +1361,9 @@ static int gguf_describe(const GgufFile& g, oxb_gguf_info* info) {
     if (!emb) return gguf_fail("tensor not found: token_embd.weight");
     if (emb->shape.size() >= 2 && emb->shape[1] <= UINT32_MAX) info->vocab = (uint32_t)emb->shape[1];
     info->embedding_type = (int)emb->type;
+    info->lm_head_rows = info->vocab;
+    if (const GgufTensor* out = g.find("output.weight"))
+        if (out->shape.size() >= 2 && out->shape[1] <= UINT32_MAX) info->lm_head_rows = (uint32_t)out->shape[1];
     const GgufTensor* q = g.find("blk.0.attn_q.weight");
     if (!q) return gguf_fail("tensor not found: blk.0.attn_q.weight");
     if (q->type == GGUF_Q1_0_G128) info->fmt = OXB_FMT_Q1;
@@ -1308,14 +1373,17 @@ static int gguf_describe(const GgufFile& g, oxb_gguf_info* info) {
 }
 
 int oxb_hip_gguf_info(const char* path, oxb_gguf_info* info) {
+    OXB_API_BEGIN
     if (!info) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null info");
     GgufFile g;
     std::string err;
     if (!g.open(path, &err)) return gguf_fail(err);
     return gguf_describe(g, info);
+    OXB_API_END
 }
 
 int oxb_hip_gguf_metadata(const char* path, const char* key, char* out, size_t out_cap) {
+    OXB_API_BEGIN
     if (!key || !out || out_cap == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null key or output");
     GgufFile g;
     std::string err;
@@ -1332,10 +1400,12 @@ int oxb_hip_gguf_metadata(const char* path, const char* key, char* out, size_t o
         default: snprintf(out, out_cap, "[%llu x type %u]", (unsigned long long)v.count, v.elem_type); break;
     }
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_gguf_tensor(const char* path, const char* name, int* type, uint32_t* n_dims, uint64_t shape4[4],
                         uint64_t* file_offset, uint64_t* n_bytes) {
+    OXB_API_BEGIN
     if (!name) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null name");
     GgufFile g;
     std::string err;
@@ -1349,6 +1419,7 @@ int oxb_hip_gguf_tensor(const char* path, const char* name, int* type, uint32_t*
     if (file_offset) *file_offset = g.data_offset + t->offset;
     if (n_bytes) *n_bytes = t->bytes;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 // A tensor that must exist with the given type(s) and GGUF shape [in (, out)].
@@ -1421,6 +1492,7 @@ static int gguf_matrix(const GgufFile& g, Model& m, int fmt, const std::vector<s
 
 int oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64_t* model, uint64_t* embedding,
                       oxb_gguf_info* info_or_null) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!model || !embedding) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null model or embedding pointer");
     GgufFile g;
@@ -1429,6 +1501,10 @@ int oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64
     oxb_gguf_info info;
     OXB_TRY(gguf_describe(g, &info));
     if (info_or_null) *info_or_null = info;
+    // every layer brings nine tensors of its own: a block count beyond that (or beyond any model this tier could hold)
+    // is a damaged or hostile header, not a model; nothing is allocated for it
+    if (info.n_layers == 0 || info.n_layers > 4096 || (uint64_t)info.n_layers * 9 > g.n_tensors)
+        return gguf_fail("block_count " + std::to_string(info.n_layers) + " does not fit a file of " + std::to_string(g.n_tensors) + " tensors");
     if (info.h % 128 || info.inter % 128 || info.hd == 0 || info.h != info.nq * info.hd)
         return gguf_fail("hidden " + std::to_string(info.h) + " / heads " + std::to_string(info.nq) + " / intermediate " +
                          std::to_string(info.inter) + " do not fit this tier (multiples of 128, hidden = heads x head_dim)");
@@ -1454,12 +1530,8 @@ int oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64
     }
     if (!rc) rc = gguf_vector(g, owner, "output_norm.weight", info.h, &final_norm);
     // the LM head's row count comes from its own shape (model/weight_loaders.rs:654-666)
-    uint32_t lm_rows = info.vocab;
-    if (!rc) {
-        const GgufTensor* out = g.find("output.weight");
-        if (!out) rc = gguf_fail("tensor not found: output.weight");
-        else if (out->shape.size() >= 2 && out->shape[1] <= UINT32_MAX) lm_rows = (uint32_t)out->shape[1];
-    }
+    const uint32_t lm_rows = info.lm_head_rows;
+    if (!rc && !g.find("output.weight")) rc = gguf_fail("tensor not found: output.weight");
     if (!rc) rc = gguf_matrix(g, owner, info.fmt, {{"output.weight", lm_rows}}, info.h, &lm_head);
     uint64_t emb_id = 0;
     if (!rc) {
@@ -1493,6 +1565,7 @@ int oxb_hip_load_gguf(const char* path, uint32_t max_seq, uint32_t batch, uint64
     *model = mid;
     *embedding = emb_id;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 }  // extern "C"

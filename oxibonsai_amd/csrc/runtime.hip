@@ -110,7 +110,11 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
     w.d_codes = reinterpret_cast<uint32_t*>(w.d_base);
     w.d_scales = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(w.d_base) + w.L.codes_bytes);
     if (*id == 0) *id = g_rt.next_id++;
-    if (Weight* old = find_weight(*id)) free_weight_mem(*old);
+    if (Weight* old = find_weight(*id)) {
+        (void)hipStreamSynchronize(g_rt.stream);  // a launch in flight may still read the old copy
+        free_weight_mem(*old);
+        g_rt.weights_gen++;
+    }
     g_rt.weights[*id] = w;
     return OXB_HIP_OK;
 }
@@ -241,6 +245,7 @@ int oxb_hip_device_count(void) {
 }
 
 int oxb_hip_init(int device_ordinal) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (g_rt.ready) {
         if (device_ordinal != g_rt.device)
@@ -266,6 +271,7 @@ int oxb_hip_init(int device_ordinal) {
     snprintf(g_rt.name, sizeof g_rt.name, "%s (%s)", prop.name, prop.gcnArchName);
     g_rt.ready = true;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 void oxb_hip_shutdown(void) {
@@ -290,6 +296,7 @@ void oxb_hip_shutdown(void) {
 }
 
 int oxb_hip_device_info(char* name, size_t name_cap, size_t* free_bytes, size_t* total_bytes) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     int rc = ensure_init();
     if (rc) return rc;
@@ -300,44 +307,57 @@ int oxb_hip_device_info(char* name, size_t name_cap, size_t* free_bytes, size_t*
     if (free_bytes) *free_bytes = f;
     if (total_bytes) *total_bytes = t;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_synchronize(void) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     int rc = ensure_init();
     if (rc) return rc;
     return sync_stream("synchronize");
+    OXB_API_END
 }
 
 int oxb_hip_set_stream(void* hip_stream) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     int rc = ensure_init();
     if (rc) return rc;
     g_rt.stream = hip_stream ? (hipStream_t)hip_stream : g_rt.own_stream;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_upload_q1(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     return upload_weight(id, OXB_FMT_Q1, aos, n_bytes, n_rows, k);
+    OXB_API_END
 }
 
 int oxb_hip_upload_tq2(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     return upload_weight(id, OXB_FMT_TQ2, aos, n_bytes, n_rows, k);
+    OXB_API_END
 }
 
 int oxb_hip_free_weight(uint64_t id) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
     if (g_rt.ready) (void)hipStreamSynchronize(g_rt.stream);
     free_weight_mem(*w);
     g_rt.weights.erase(id);
+    g_rt.weights_gen++;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, size_t* resident_bytes) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -346,9 +366,11 @@ int oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, si
     if (k) *k = w->L.k;
     if (resident_bytes) *resident_bytes = w->L.codes_bytes + w->L.scales_bytes;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_dequant(uint64_t id, float* out, size_t out_len) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -361,9 +383,11 @@ int oxb_hip_dequant(uint64_t id, float* out, size_t out_len) {
     e = hipMemcpyAsync(out, g_rt.ws_y.ptr, n * sizeof(float), hipMemcpyDeviceToHost, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "dequant download");
     return sync_stream("dequant");
+    OXB_API_END
 }
 
 int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -371,10 +395,12 @@ int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows,
     if (rc) return rc;
     if (!d_x || !d_y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
     return gemv_device(*w, d_x, d_y, batch, n_rows, OXB_GEMV_STORE, nullptr);
+    OXB_API_END
 }
 
 int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,
                          uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     if (!ids || n_ids == 0 || !d_x || !d_y || !avg_us || iters == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
@@ -440,9 +466,11 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
     return rc;
+    OXB_API_END
 }
 
 int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -450,9 +478,11 @@ int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint
     if (rc) return rc;
     if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
     return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f);
+    OXB_API_END
 }
 
 int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -469,10 +499,12 @@ int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_r
     e = hipMemcpyAsync(y, g_rt.ws_y.ptr, yb, hipMemcpyDeviceToHost, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "output download");
     return sync_stream("gemm");
+    OXB_API_END
 }
 
 int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
                          uint32_t warmup, uint32_t iters, float* avg_us) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -520,9 +552,11 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
     return rc;
+    OXB_API_END
 }
 
 int oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
@@ -539,18 +573,23 @@ int oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_
     e = hipMemcpyAsync(y, g_rt.ws_y.ptr, yb, hipMemcpyDeviceToHost, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "output download");
     return sync_stream("gemv");
+    OXB_API_END
 }
 
 int oxb_hip_gemv_q1_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len, float* y, size_t y_len,
                          uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     return oneshot_gemv(OXB_FMT_Q1, aos, n_bytes, x, x_len, y, y_len, n_rows, k);
+    OXB_API_END
 }
 
 int oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, size_t x_len, float* y, size_t y_len,
                           uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     return oneshot_gemv(OXB_FMT_TQ2, aos, n_bytes, x, x_len, y, y_len, n_rows, k);
+    OXB_API_END
 }
 
 // ---- host-only repack helpers -------------------------------------------------
@@ -562,16 +601,19 @@ static int repack_args(int fmt, uint32_t n_rows, uint32_t k) {
 }
 
 int oxb_hip_repack_sizes(int fmt, uint32_t n_rows, uint32_t k, size_t* codes_bytes, size_t* scales_bytes) {
+    OXB_API_BEGIN
     int rc = repack_args(fmt, n_rows, k);
     if (rc) return rc;
     OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
     if (codes_bytes) *codes_bytes = L.codes_bytes;
     if (scales_bytes) *scales_bytes = L.scales_bytes;
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_repack(int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k, uint8_t* codes,
                    size_t codes_cap, uint8_t* scales, size_t scales_cap) {
+    OXB_API_BEGIN
     int rc = repack_args(fmt, n_rows, k);
     if (rc) return rc;
     OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
@@ -581,10 +623,12 @@ int oxb_hip_repack(int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows,
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: output sections too small");
     oxb_repack_aos_to_tiled(L, aos, reinterpret_cast<uint32_t*>(codes), reinterpret_cast<uint16_t*>(scales));
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 int oxb_hip_unpack(int fmt, const uint8_t* codes, size_t codes_len, const uint8_t* scales, size_t scales_len,
                    uint32_t n_rows, uint32_t k, uint8_t* aos, size_t aos_cap) {
+    OXB_API_BEGIN
     int rc = repack_args(fmt, n_rows, k);
     if (rc) return rc;
     OxbLayout L = oxb_make_layout((uint32_t)fmt, n_rows, k);
@@ -593,6 +637,7 @@ int oxb_hip_unpack(int fmt, const uint8_t* codes, size_t codes_len, const uint8_
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: buffer sizes do not match the layout");
     oxb_repack_tiled_to_aos(L, reinterpret_cast<const uint32_t*>(codes), reinterpret_cast<const uint16_t*>(scales), aos);
     return OXB_HIP_OK;
+    OXB_API_END
 }
 
 }  // extern "C"

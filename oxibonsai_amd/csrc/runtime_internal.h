@@ -2,7 +2,9 @@
 #pragma once
 #include <hip/hip_runtime.h>
 
+#include <exception>
 #include <mutex>
+#include <new>
 #include <string>
 #include <unordered_map>
 
@@ -47,6 +49,9 @@ struct Runtime {
     std::unordered_map<uint64_t, Weight> weights;
     std::unordered_map<uint64_t, Vector> vectors;
     uint64_t next_id = 1ull << 40;  // library-allocated handles stay clear of caller-chosen ids
+    // Counts every free or replacement of a resident matrix or vector.  A captured decode graph holds their device
+    // pointers; a model compares the count it captured under with this one and captures again when they differ.
+    uint64_t weights_gen = 0;
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
     GemmWorkspace gemm_ws;  // shared by every GEMM call that does not bring its own
 };
@@ -67,5 +72,14 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
 int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uint32_t m, uint32_t ldy, int mode,
                 const float* d_residual, int pack_op, const float* d_pack_w, float eps, GemmWorkspace* ws = nullptr);
 void shutdown_models();
+
+// Every `int` entry point of the C ABI runs its body between these two, so that no C++ exception (a failed host
+// allocation in a std container, above all) unwinds into the caller.
+#define OXB_API_BEGIN try {
+#define OXB_API_END                                                                                          \
+    }                                                                                                        \
+    catch (const std::bad_alloc&) { return oxb::fail(OXB_HIP_OUT_OF_MEMORY, "out of host memory"); }        \
+    catch (const std::exception& e_) { return oxb::fail(OXB_HIP_INVALID_ARGUMENT, "internal error: %s", e_.what()); } \
+    catch (...) { return oxb::fail(OXB_HIP_INVALID_ARGUMENT, "internal error: unknown C++ exception"); }
 
 }  // namespace oxb

@@ -63,10 +63,12 @@ def gguf_bytes(metadata, tensors, version: int = 3, alignment: int = 32, packed:
 
 
 def model_gguf(cfg: dict, w: dict, emb_type: int, emb_table, arch: str = "qwen3", norm_f16: bool = False,
-               meta_override: dict | None = None, type_override: dict | None = None, **kw) -> bytes:
+               meta_override: dict | None = None, type_override: dict | None = None, emb_rows: int | None = None,
+               **kw) -> bytes:
     """The synthetic checkpoint of the reference's parity test
     (crates/oxibonsai-model/tests/metal_prefill_ternary_parity_tests.rs:79-224) for any geometry / format:
-    cfg and w as for oxibonsai_amd.synth.make_model; emb_table = the stored bytes of token_embd.weight."""
+    cfg and w as for oxibonsai_amd.synth.make_model; emb_table = the stored bytes of token_embd.weight, which holds
+    emb_rows rows (default: as many as the LM head, cfg["vocab"])."""
     h, inter, hd = cfg["h"], cfg["inter"], cfg["hd"]
     qd, kd = cfg["nq"] * hd, cfg["nkv"] * hd
     mt = GGUF_Q1 if cfg["fmt"] == Q1 else GGUF_TQ2
@@ -85,7 +87,7 @@ def model_gguf(cfg: dict, w: dict, emb_type: int, emb_table, arch: str = "qwen3"
         a = np.asarray(v, dtype=np.float32)
         return (GGUF_F16, a.astype(np.float16).tobytes()) if norm_f16 else (GGUF_F32, a.tobytes())
 
-    ts = [("token_embd.weight", [h, cfg["vocab"]], emb_type, np.ascontiguousarray(emb_table).tobytes()),
+    ts = [("token_embd.weight", [h, emb_rows or cfg["vocab"]], emb_type, np.ascontiguousarray(emb_table).tobytes()),
           ("output_norm.weight", [h], *vec(w["final_norm"])),
           ("output.weight", [h, cfg["vocab"]], mt, w["lm_head"].tobytes())]
     for i, lw in enumerate(w["layers"]):

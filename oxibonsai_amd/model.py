@@ -32,7 +32,8 @@ class GgufInfo(C.Structure):
     _fields_ = [("version", C.c_uint32), ("alignment", C.c_uint32), ("n_tensors", C.c_uint64), ("n_metadata", C.c_uint64),
                 ("fmt", C.c_int), ("embedding_type", C.c_int)] + \
                [(n, C.c_uint32) for n in ("n_layers", "h", "inter", "nq", "nkv", "hd", "vocab", "context_length")] + \
-               [("eps", C.c_float), ("rope_theta", C.c_float), ("architecture", C.c_char * 32), ("name", C.c_char * 64)]
+               [("eps", C.c_float), ("rope_theta", C.c_float), ("architecture", C.c_char * 32), ("name", C.c_char * 64),
+                ("lm_head_rows", C.c_uint32)]
 
     def as_dict(self) -> dict:
         d = {n: getattr(self, n) for n, _ in self._fields_}
@@ -181,7 +182,7 @@ class HipModel:
         _check(self._lib.oxb_hip_load_gguf(str(path).encode(), max_seq, batch, C.byref(mid), C.byref(eid), C.byref(info)))
         d = info.as_dict()
         self.cfg = dict(fmt=d["fmt"], n_layers=d["n_layers"], h=d["h"], inter=d["inter"], nq=d["nq"], nkv=d["nkv"], hd=d["hd"],
-                        vocab=d["vocab"], max_seq=max_seq or d["context_length"], eps=d["eps"], rope_theta=d["rope_theta"])
+                        vocab=d["lm_head_rows"], max_seq=max_seq or d["context_length"], eps=d["eps"], rope_theta=d["rope_theta"])
         self.id = mid.value
         return self, Embedding(None, d["embedding_type"], d["vocab"], d["h"], _id=eid.value), d
 

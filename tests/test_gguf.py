@@ -169,3 +169,22 @@ def test_data_section_alignment_and_tensor_offsets(tmp_path):
     assert gguf_tensor(p, "s")["bytes"] == 4 and gguf_tensor(p, "s")["n_dims"] == 0
     assert gguf_tensor(p, "v")["bytes"] == 10 and gguf_tensor(p, "m")["bytes"] == 6 * 34
     assert gguf_tensor(p, "x")["bytes"] == 0 and gguf_tensor(p, "x")["type"] == 2          # Q4_0: listed, not read
+
+
+def test_loader_rejects_an_absurd_block_count_before_allocating(tmp_path):
+    # a header that claims 2^32 - 1 layers must be refused by the loader itself (no GPU is touched, nothing is
+    # allocated for it), and so must a count the file's tensor directory cannot cover
+    import ctypes as C
+    from oxibonsai_amd import _lib
+    from oxibonsai_amd.model import GgufInfo
+    emb = np.zeros((4, 128), np.float32).tobytes()
+    q = np.zeros(4 * 18, np.uint8).tobytes()
+    ts = [("token_embd.weight", [128, 4], GGUF_F32, emb), ("blk.0.attn_q.weight", [128, 4], GGUF_Q1, q)]
+    for count in (0xFFFFFFFF, 4097, 1, 0):
+        md = [("qwen3.block_count", "u32", count), ("qwen3.embedding_length", "u32", 128), ("qwen3.attention.head_count", "u32", 1)]
+        p = _write(tmp_path, gguf_bytes(md, ts), f"layers{count}.gguf")
+        assert gguf_info(p)["n_layers"] == count          # the directory reader reports what the file says
+        mid, eid, info = C.c_uint64(0), C.c_uint64(0), GgufInfo()
+        rc = _lib.lib().oxb_hip_load_gguf(p.encode(), 0, 1, C.byref(mid), C.byref(eid), C.byref(info))
+        assert rc == 5 and "block_count" in _lib.last_error(), (count, _lib.last_error())
+        assert info.lm_head_rows == 4                      # no output.weight: falls back to the embedding's rows

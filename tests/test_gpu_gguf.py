@@ -76,6 +76,33 @@ def test_loaded_model_equals_hand_assembled_model_and_oracle(backend, tmp_path, 
         ref.close()
 
 
+def test_lm_head_with_fewer_rows_than_the_embedding_table(backend, tmp_path):
+    # token_embd.weight and output.weight need not have the same row count: the logits have one entry per LM-head
+    # row, the embedding lookup accepts every row of the table
+    cfg = dict(TINY, fmt=Q1)
+    w = synth.make_model(cfg, 77)
+    big = dict(cfg, vocab=48)
+    stored, rows = _table(big, GGUF_F16)
+    path = tmp_path / "m.gguf"
+    path.write_bytes(model_gguf(cfg, w, GGUF_F16, stored, emb_rows=48))
+    ref = HipModel(backend, dict(cfg, max_seq=64), w)
+    gpu, emb, info = HipModel.from_gguf(backend, str(path), max_seq=64)
+    try:
+        assert (info["vocab"], info["lm_head_rows"], gpu.cfg["vocab"], emb.vocab) == (48, 32, 32, 48)
+        hidden = emb.rows([47])[0]
+        assert np.array_equal(hidden, rows[47])
+        a, ta = gpu.forward(hidden, 0)
+        b, tb = ref.forward(hidden, 0)
+        assert a.shape == (1, 32) and np.array_equal(a, b) and ta[0] == tb[0]
+        logits, tok = gpu.prefill_tokens(emb, [47, 3, 40], pos_start=1)
+        assert logits.shape == (32,) and tok == int(np.argmax(logits))
+        assert gpu.generate(emb, [47], [4], 3).max() < 32
+    finally:
+        gpu.close()
+        emb.close()
+        ref.close()
+
+
 @pytest.mark.parametrize("batch", [1, 2, 4])
 def test_on_device_greedy_loop_equals_host_driven_loop(backend, tmp_path, batch):
     cfg = dict(SMALL, fmt=TQ2)

@@ -85,3 +85,52 @@ def test_two_models_share_the_device(backend):
     finally:
         for g in gpus:
             g.close()
+
+
+def test_replacing_or_freeing_a_weight_of_a_live_model(backend):
+    # The captured decode step holds device pointers: after a weight is replaced under its id the next step must
+    # compute with the new copy (as a model built from the new weights does), and after it is freed the step must
+    # report the missing handle instead of replaying a graph over freed memory.
+    import ctypes as C
+
+    from oxibonsai_amd import GpuError, _lib
+    cfg = dict(fmt=Q1, n_layers=2, h=128, inter=256, nq=4, nkv=2, hd=32, vocab=32, max_seq=64, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 61)
+    w2 = synth.make_model(cfg, 62)
+    gpu = HipModel(backend, cfg, w)
+    rows = synth.embedding_rows(7, range(8), cfg["h"]) * 50.0
+    try:
+        for pos in range(3):
+            gpu.forward(rows[pos], pos)
+        assert gpu.uses_graph()
+        # replace layer 1's down projection and the final norm vector under their ids
+        down_id, norm_id = int(gpu._ids[1].down), int(gpu._vecs[-1])
+        backend.upload_weights_raw(w2["layers"][1]["down"], cfg["h"], cfg["inter"], handle_id=down_id)
+        nv = np.ascontiguousarray(w2["final_norm"], dtype=np.float32)
+        hid = C.c_uint64(norm_id)
+        assert _lib.lib().oxb_hip_upload_f32(C.byref(hid), nv.ctypes.data_as(_lib.f32p), nv.size) == 0 and hid.value == norm_id
+        mixed = dict(w, final_norm=w2["final_norm"], layers=[w["layers"][0], dict(w["layers"][1], down=w2["layers"][1]["down"])])
+        ref = HipModel(backend, cfg, mixed)
+        try:
+            for pos in range(3):
+                ref.forward(rows[pos], pos)
+            a, _ = gpu.forward(rows[3], 3)
+            b, _ = ref.forward(rows[3], 3)
+            # the last layer's down projection and the final norm feed no cache row, so both models hold the same
+            # cache for positions 0..2 and must agree bit for bit at position 3
+            assert np.array_equal(a, b)
+            assert gpu.uses_graph()
+        finally:
+            ref.close()
+        backend.free_weights(down_id)
+        gpu._mats.remove(down_id)
+        with pytest.raises(GpuError) as e:
+            gpu.forward(rows[4], 4)
+        assert e.value.kind == "WeightNotFound"
+        # the handle comes back: the model works again
+        backend.upload_weights_raw(w["layers"][1]["down"], cfg["h"], cfg["inter"], handle_id=down_id)
+        gpu._mats.append(down_id)
+        got, _ = gpu.forward(rows[4], 4)
+        assert np.all(np.isfinite(got))
+    finally:
+        gpu.close()
