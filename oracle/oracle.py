@@ -93,6 +93,8 @@ def lib() -> C.CDLL:
         L.oxb_state_free.restype = None
         L.oxb_forward_ex.argtypes = [C.c_void_p, C.c_void_p, f32p, sz, f32p, f32p]
         L.oxb_simd_tier.restype = C.c_int
+        L.oxb_simd_set_tier.argtypes = [C.c_int]
+        L.oxb_simd_set_tier.restype = C.c_int
         L.oxb_simd_threads.restype = C.c_int
         L.oxb_simd_set_threads.argtypes = [C.c_int]
         L.oxb_simd_set_threads.restype = None
@@ -177,8 +179,17 @@ def simd_gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int) -> np.ndarray:
     return y.reshape(m, n_rows)
 
 
+SIMD_TIERS = {0: "scalar", 1: "avx2+fma", 2: "avx512"}
+
+
 def simd_tier() -> str:
-    return {0: "scalar", 1: "avx2+fma", 2: "avx512"}[lib().oxb_simd_tier()]
+    return SIMD_TIERS[lib().oxb_simd_tier()]
+
+
+def simd_set_tier(tier: int) -> int:
+    """Lower (or restore) the SIMD tier of the CPU baseline: 0 scalar, 1 AVX2+FMA, 2 AVX-512.  Returns the tier in use,
+    -1 when the host CPU lacks the requested one."""
+    return lib().oxb_simd_set_tier(int(tier))
 
 
 def set_threads(n: int) -> None:

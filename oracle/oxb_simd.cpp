@@ -25,6 +25,7 @@
 #include <algorithm>
 #include <atomic>
 #include <condition_variable>
+#include <cstdlib>
 #include <cstring>
 #include <functional>
 #include <mutex>
@@ -258,6 +259,15 @@ unsigned g_threads_req = 0;
 void ensure_init() {
     std::call_once(g_once, [] {
         g_tier = detect_tier();
+        /* OXB_SIMD_TIER=scalar|avx2|avx512 lowers the tier below what the CPU offers (never above it), so that
+         * the AVX2 path can be run and checked on an AVX-512 host. */
+        if (const char* want = std::getenv("OXB_SIMD_TIER")) {
+            Tier t = g_tier;
+            if (!std::strcmp(want, "scalar")) t = TIER_SCALAR;
+            else if (!std::strcmp(want, "avx2")) t = TIER_AVX2;
+            else if (!std::strcmp(want, "avx512")) t = TIER_AVX512;
+            if (t < g_tier) g_tier = t;
+        }
         unsigned n = g_threads_req ? g_threads_req : std::thread::hardware_concurrency();
         g_pool = new Pool(n ? n : 1);
     });
@@ -295,6 +305,15 @@ extern "C" {
 /* 0 scalar, 1 AVX2+FMA, 2 AVX-512 — what dispatch.rs:143-175 would pick on this host. */
 int oxb_simd_tier(void) { ensure_init(); return (int)g_tier; }
 int oxb_simd_threads(void) { ensure_init(); return (int)g_pool->size(); }
+/* Lower the tier at run time (0 scalar, 1 AVX2+FMA, 2 AVX-512); a tier the CPU lacks is refused (-1).
+ * Returns the tier now in use.  The reference fixes its tier once per process (dispatch.rs:143-175); this
+ * switch exists so that one test process can hold every tier the host offers to the scalar oracle. */
+int oxb_simd_set_tier(int tier) {
+    ensure_init();
+    if (tier < 0 || tier > (int)detect_tier()) return -1;
+    g_tier = (Tier)tier;
+    return (int)g_tier;
+}
 /* Must be called before the first kernel call to take effect (0 = all host cores). */
 void oxb_simd_set_threads(int n) { g_threads_req = n > 0 ? (unsigned)n : 0; }
 

@@ -188,3 +188,45 @@ def test_gemv_large_k_edge_case():
     k = 12800
     blocks = np.concatenate([q1_block(0.5, 0xFF)] * (k // 128))
     assert oracle.gemv(Q1, blocks, np.ones(k, np.float32), 1, k)[0] == 0.5 * k
+
+
+# ---- every SIMD tier the host offers, forced in turn ---------------------------------------------
+@pytest.mark.parametrize("tier", [0, 1, 2])
+def test_each_simd_tier_against_the_scalar_oracle(tier):
+    """The CPU baseline picks its tier by CPUID (dispatch.rs:143-175), so on an AVX-512 host the AVX2 kernels would
+    never run: force each tier and hold it to the scalar oracle with the reference's own SIMD-vs-scalar gates
+    (MSE < 1e-6 on the generator of simd_avx2.rs:1147-1180; < 1.0 absolute on cross_tier.rs:18-93) and to the
+    float64 product."""
+    best = oracle.lib().oxb_simd_tier()
+    top = oracle.simd_set_tier(2)
+    top = top if top >= 0 else (1 if oracle.simd_set_tier(1) >= 0 else 0)
+    try:
+        if tier > top:
+            pytest.skip(f"host CPU offers no tier above {oracle.SIMD_TIERS[top]}")
+        assert oracle.simd_set_tier(tier) == tier and oracle.lib().oxb_simd_tier() == tier
+        blocks, x = simd_parity_tq2(64, 128)
+        assert np.mean((oracle.simd_gemv(TQ2, blocks, x, 64, 128) - oracle.gemv(TQ2, blocks, x, 64, 128)) ** 2) < 1e-6
+        n, k = 128, 1024
+        blocks = cross_tier_q1(n, k)
+        x = np.array([(i % 17) * 0.25 - 2.0 for i in range(k)], dtype=np.float32)
+        assert np.max(np.abs(oracle.simd_gemv(Q1, blocks, x, n, k) - oracle.gemv(Q1, blocks, x, n, k))) < 1.0
+        for fmt in (Q1, TQ2):
+            # odd block counts (the AVX2 Q1 kernel takes two blocks per iteration and a tail), row counts on both
+            # sides of the direct / threaded switch, and the batched entry point
+            for n, k in ((5, 128), (33, 384), (300, 640), (70, 2048)):
+                blocks = synth.make_blocks(fmt, 900 + n, n, k)
+                x = synth.normal_f32(901 + k, k)
+                want = dense_f64(fmt, blocks, n, k) @ x.astype(np.float64)
+                got = oracle.simd_gemv(fmt, blocks, x, n, k)
+                scale = np.max(np.abs(want))
+                assert np.max(np.abs(got - want)) < 2e-6 * scale, (tier, fmt, n, k)
+                assert np.max(np.abs(got - oracle.gemv(fmt, blocks, x, n, k))) < 4e-6 * scale
+            m, n, k = 5, 40, 256
+            blocks = synth.make_blocks(fmt, 77, n, k)
+            xs = synth.normal_f32(78, m * k).reshape(m, k)
+            got = oracle.simd_gemm(fmt, blocks, xs, m, n, k)
+            want = xs.astype(np.float64) @ dense_f64(fmt, blocks, n, k).T
+            assert np.max(np.abs(got - want)) < 2e-6 * np.max(np.abs(want))
+        assert oracle.simd_set_tier(3) == -1 and oracle.lib().oxb_simd_tier() == tier      # an unknown tier changes nothing
+    finally:
+        oracle.simd_set_tier(best)
