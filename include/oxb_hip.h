@@ -96,6 +96,13 @@ int  oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_
 int  oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k);
 int  oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
                           uint32_t warmup, uint32_t iters, float* avg_us);
+/* oxb_hip_gemm_dev for callers that cannot allocate (no counterpart in the reference): code under HIP graph capture,
+ * serving loops and harnesses that forbid hipMalloc.  Same kernels and results, but the call's scratch - packed fp16
+ * activations, per-row exponents, the partial sums of a K split - lies in a 32 MiB array inside the library's code
+ * object instead of a workspace that grows on demand; no allocation or free of device memory happens in the call.  A shape
+ * whose scratch exceeds the array is OXB_HIP_INVALID_ARGUMENT (the message gives both sizes).  Every call on a GPU
+ * uses that GPU's one array: calls that overlap in time (different streams) race. */
+int  oxb_hip_gemm_dev_static(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k);
 
 /* ---- batch_ffn_phase (KG/mod.rs:519; CUDA: KG/cuda_graph/nativecudabackend_traits.rs:122-188 -> encode_ffn_phase,
  * KG/cuda_graph/cudagraph_encoding.rs:72-160): hidden += O * attn_out; normed = RMSNorm(hidden); hidden += down * SwiGLU(gate||up * normed),

@@ -36,6 +36,7 @@ _SIGNATURES = {
                               C.c_uint32, f32p], C.c_int),
     "oxb_hip_gemm": ([C.c_uint64, f32p, f32p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_gemm_dev": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
+    "oxb_hip_gemm_dev_static": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_profile_gemm": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
                               C.c_uint32, C.c_uint32, f32p], C.c_int),
     "oxb_hip_gemv_q1_g128": ([u8p, C.c_size_t, f32p, C.c_size_t, f32p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),

@@ -44,8 +44,16 @@ int hip_fail(hipError_t e, const char* what) {
 Runtime g_rt;
 std::recursive_mutex g_mu;
 
+// Scratch of the allocation-free GEMM entry point (oxb_hip_gemm_dev_static): packed fp16 activations, per-row
+// exponents and multipliers, and the partial sums of a K split.  It lives in the code object, so the GPU the library
+// runs on holds it from the first use of the library until the process ends.  In host code the array's name only
+// stands for the symbol; its device address is looked up once in oxb_hip_init and kept in g_rt.static_scratch.
+#define OXB_STATIC_SCRATCH_BYTES (32u << 20)
+static __device__ __align__(256) unsigned char oxb_static_scratch[OXB_STATIC_SCRATCH_BYTES];
+
 int DevBuf::ensure(size_t bytes) {
     if (bytes <= cap) return OXB_HIP_OK;
+    if (fixed) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %zu bytes of scratch needed, the fixed buffer holds %zu", bytes, cap);
     if (ptr) (void)hipFree(ptr);
     ptr = nullptr;
     cap = 0;
@@ -61,7 +69,7 @@ int DevBuf::ensure(size_t bytes) {
 }
 
 void DevBuf::release() {
-    if (ptr) (void)hipFree(ptr);
+    if (ptr && !fixed) (void)hipFree(ptr);
     ptr = nullptr;
     cap = 0;
 }
@@ -263,6 +271,10 @@ int oxb_hip_init(int device_ordinal) {
         return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: %s", hipGetErrorString(e));
     if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
         return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: kernels are built for gfx950, device is %s", prop.gcnArchName);
+    void* scratch_addr = nullptr;
+    if ((e = hipGetSymbolAddress(&scratch_addr, HIP_SYMBOL(oxb_static_scratch))) != hipSuccess || !scratch_addr)
+        return hip_fail(e, "static scratch lookup");
+    g_rt.static_scratch = scratch_addr;
     if ((e = hipStreamCreateWithFlags(&g_rt.own_stream, hipStreamNonBlocking)) != hipSuccess)
         return hip_fail(e, "stream creation");
     g_rt.stream = g_rt.own_stream;
@@ -290,6 +302,7 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_xexp.release();
     g_rt.gemm_ws.release();
     (void)hipStreamDestroy(g_rt.own_stream);
+    g_rt.static_scratch = nullptr;
     g_rt.own_stream = nullptr;
     g_rt.stream = nullptr;
     g_rt.ready = false;
@@ -478,6 +491,43 @@ int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint
     if (rc) return rc;
     if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
     return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f);
+    OXB_API_END
+}
+
+int oxb_hip_gemm_dev_static(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Weight* w = find_weight(id);
+    if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    int rc = check_shape(*w, n_rows, k);
+    if (rc) return rc;
+    if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
+    if (!g_rt.ready || !g_rt.static_scratch) return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: the library is not initialised");
+    // Carve the file-scope array into the four buffers of a GEMM call.  Every byte the kernels read from them is
+    // written earlier in the same call (the packer fills its padding rows and blocks with zeros, every K slice
+    // writes all of its partial sums), so nothing needs clearing between calls.
+    OxbGemmParams gp;
+    memset(&gp, 0, sizeof gp);
+    gp.n_rows = n_rows, gp.n_tiles = w->L.n_tiles, gp.n_sb = w->L.n_sb, gp.M = m, gp.ldy = n_rows;
+    const uint32_t ksplit = oxb_gemm_ksplit(gp, g_rt.n_cus);
+    auto up = [](size_t v) { return (v + 255) & ~(size_t)255; };
+    const size_t need[4] = {up(oxb_xh_bytes(k, m)), up(((size_t)m + 16) * sizeof(int32_t)), up(((size_t)m + 16) * sizeof(float)),
+                            ksplit > 1 ? up((size_t)ksplit * m * n_rows * sizeof(float)) : 0};
+    const size_t total = need[0] + need[1] + need[2] + need[3];
+    if (total > OXB_STATIC_SCRATCH_BYTES)
+        return fail(OXB_HIP_INVALID_ARGUMENT,
+                    "invalid argument: a GEMM of %u rows x %u x %u needs %zu bytes of scratch, the allocation-free entry point holds %u",
+                    m, n_rows, k, total, OXB_STATIC_SCRATCH_BYTES);
+    GemmWorkspace ws;
+    DevBuf* bufs[4] = {&ws.xh, &ws.xsh, &ws.rowmul, &ws.part};
+    size_t off = 0;
+    for (int i = 0; i < 4; i++) {
+        bufs[i]->ptr = need[i] ? (unsigned char*)g_rt.static_scratch + off : nullptr;
+        bufs[i]->cap = need[i];
+        bufs[i]->fixed = true;
+        off += need[i];
+    }
+    return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f, &ws);
     OXB_API_END
 }
 

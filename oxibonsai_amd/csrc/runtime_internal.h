@@ -15,6 +15,7 @@ namespace oxb {
 struct DevBuf {  // grow-only device scratch
     void* ptr = nullptr;
     size_t cap = 0;
+    bool fixed = false;  // a view of memory owned elsewhere: never grown, never freed
     int ensure(size_t bytes);
     void release();
 };
@@ -53,6 +54,7 @@ struct Runtime {
     // pointers; a model compares the count it captured under with this one and captures again when they differ.
     uint64_t weights_gen = 0;
     DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
+    void* static_scratch = nullptr;  // device address of the library's file-scope scratch array on g_rt.device
     GemmWorkspace gemm_ws;  // shared by every GEMM call that does not bring its own
 };
 

@@ -109,3 +109,51 @@ def parity_violations(a: np.ndarray, b: np.ndarray, tol: float = 1e-3) -> int:
 
 
 from oxibonsai_amd.gguf import GGUF_F16, GGUF_F32, GGUF_MAGIC, GGUF_Q1, GGUF_TQ2, gguf_bytes, model_gguf  # noqa: E402,F401
+
+
+class DeviceBuffer:
+    """A device allocation made through the HIP runtime the library itself links (libamdhip64.so.7), for the
+    entry points that take device pointers; no second runtime (torch ships its own) enters the process."""
+    _hip = None
+
+    @classmethod
+    def hip(cls):
+        if cls._hip is None:
+            import ctypes as C
+            h = C.CDLL("libamdhip64.so.7")
+            h.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+            h.hipFree.argtypes = [C.c_void_p]
+            h.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+            h.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
+            h.hipDeviceSynchronize.argtypes = []
+            cls._hip = h
+        return cls._hip
+
+    def __init__(self, nbytes: int):
+        import ctypes as C
+        p = C.c_void_p(0)
+        assert self.hip().hipMalloc(C.byref(p), max(int(nbytes), 16)) == 0, "hipMalloc failed"
+        self.ptr, self.nbytes = p.value, int(nbytes)
+
+    @classmethod
+    def from_numpy(cls, a: np.ndarray) -> "DeviceBuffer":
+        a = np.ascontiguousarray(a)
+        b = cls(a.nbytes)
+        assert cls.hip().hipMemcpy(b.ptr, a.ctypes.data, a.nbytes, 1) == 0       # hipMemcpyHostToDevice
+        return b
+
+    def fill(self, byte: int) -> None:
+        assert self.hip().hipMemset(self.ptr, byte, self.nbytes) == 0
+        assert self.hip().hipDeviceSynchronize() == 0
+
+    def to_numpy(self, dtype, shape) -> np.ndarray:
+        out = np.empty(shape, dtype=dtype)
+        assert out.nbytes <= self.nbytes
+        assert self.hip().hipDeviceSynchronize() == 0
+        assert self.hip().hipMemcpy(out.ctypes.data, self.ptr, out.nbytes, 2) == 0     # hipMemcpyDeviceToHost
+        return out
+
+    def free(self) -> None:
+        if self.ptr:
+            self.hip().hipFree(self.ptr)
+            self.ptr = 0

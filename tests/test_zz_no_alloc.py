@@ -1,0 +1,69 @@
+"""The allocation-free GEMM entry point (oxb_hip_gemm_dev_static) against oxb_hip_gemm_dev, through the C ABI.
+
+Same kernels and launch plan, so the results must be equal bit for bit; the second call of each pair is smaller than
+the first and runs on the scratch the first call left behind."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import Q1, TQ2, DeviceBuffer
+from oxibonsai_amd import _lib, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _both(L, h, x, m, n, k):
+    d_x = DeviceBuffer.from_numpy(x)
+    d_y = DeviceBuffer(m * n * 4)
+    outs = []
+    try:
+        for fn in (L.oxb_hip_gemm_dev, L.oxb_hip_gemm_dev_static):
+            d_y.fill(0xFF)                              # NaN patterns: every output must be written by the call
+            rc = fn(int(h), d_x.ptr, d_y.ptr, m, n, k)
+            assert rc == 0, _lib.last_error()
+            assert L.oxb_hip_synchronize() == 0
+            outs.append(d_y.to_numpy(np.float32, (m, n)))
+    finally:
+        d_x.free()
+        d_y.free()
+    return outs
+
+
+@pytest.mark.parametrize("fmt,shapes", [
+    (TQ2, [(512, 2560, 9728), (130, 250, 1152)]),      # wide kernel with a K split, then a ragged small case
+    (Q1, [(300, 4096, 4096), (20, 4100, 1152)]),       # wide kernel, then the narrow (few token rows) kernel
+    (Q1, [(64, 333, 640), (1, 16, 128)]),
+])
+def test_static_scratch_gemm_equals_the_allocating_entry_point(backend, fmt, shapes):
+    L = _lib.lib()
+    for i, (m, n, k) in enumerate(shapes):             # two calls in a row, the second one smaller
+        a = synth.make_blocks(fmt, 50 + i + n, n, k)
+        x = synth.normal_f32(60 + i + k, m * k).reshape(m, k)
+        h = backend.upload_weights_raw(a, n, k) if fmt == Q1 else backend.upload_weights_ternary(a, n, k)
+        try:
+            want, got = _both(L, h, x, m, n, k)
+        finally:
+            backend.free_weights(h)
+        assert np.all(np.isfinite(want))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (fmt, m, n, k)
+
+
+def test_static_scratch_gemm_rejects_what_does_not_fit(backend):
+    L = _lib.lib()
+    n, k, m = 256, 4096, 4096                           # packed activations alone: 32 * 16 * 4096 * 16 B = 32 MiB + the rest
+    a = synth.make_blocks(Q1, 9, n, k)
+    h = backend.upload_weights_raw(a, n, k)
+    try:
+        d_x, d_y = DeviceBuffer(m * k * 4), DeviceBuffer(m * n * 4)
+        d_x.fill(0)
+        rc = L.oxb_hip_gemm_dev_static(int(h), d_x.ptr, d_y.ptr, m, n, k)
+        assert rc == 5 and "allocation-free entry point holds" in _lib.last_error()
+        assert L.oxb_hip_gemm_dev(int(h), d_x.ptr, d_y.ptr, m, n, k) == 0     # the allocating one takes it
+        assert L.oxb_hip_synchronize() == 0
+        assert L.oxb_hip_gemm_dev_static(int(h), d_x.ptr, d_y.ptr, 16, n, k) == 0   # and small shapes still run
+        assert L.oxb_hip_synchronize() == 0
+        d_x.free()
+        d_y.free()
+    finally:
+        backend.free_weights(h)
