@@ -116,3 +116,8 @@ def embedding_rows(seed: int, token_ids, h: int) -> np.ndarray:
     """Embedding rows N(0, 0.02) through f16, generated per token id so a 151 936-row
     table never has to exist on the host."""
     return np.stack([f16_round(normal_f32((seed << 20) ^ int(t), h, 0.02)) for t in token_ids])
+
+
+def token_ids(seed: int, n: int, vocab: int) -> np.ndarray:
+    """n token ids, uniform over 0 .. vocab - 1 (a seeded random prompt)."""
+    return (splitmix64(seed, n) % np.uint64(vocab)).astype(np.uint32)
