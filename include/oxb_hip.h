@@ -67,17 +67,21 @@ int  oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, s
 int  oxb_hip_dequant(uint64_t id, float* out, size_t out_len);
 
 /* ---- GEMV / GEMM on resident weights: gemv_q1_g128_cached (KG/mod.rs:457), gemv_tq2_g128_cached (:484).
- * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per two vectors). */
+ * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per four vectors). */
 int  oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch);
 /* Same with device-resident x / y, asynchronous on the current stream. */
 int  oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch);
 
 /* Measurement aid (the reference's counterpart is its CUDA_PROFILE / OXIBONSAI_PROFILE_GPU instrumentation,
- * KG/cuda_full_layer/mod.rs:339-344, KG/metal_full_layer/functions.rs:17-35): quantise d_x once, then launch the
- * GEMV kernel alone `iters` times, launch i on weight ids[i % n_ids] (same shape and format), bracketed by HIP
- * events on the stream the kernel runs on.  *avg_us = mean time per launch in microseconds. */
+ * KG/cuda_full_layer/mod.rs:339-344, KG/metal_full_layer/functions.rs:17-35): launch the GEMV kernel (which quantises
+ * d_x in its prologue) `iters` times, launch i on weight ids[i % n_ids] (same shape and format), bracketed by HIP
+ * events on the stream the kernel runs on.  *avg_us = mean time per launch in microseconds.
+ * _floor launches, in place of the GEMV, a kernel that only reads the same codes and scales with the same grid, waves and
+ * load ring: the time below which no kernel that streams these bytes can finish on this GPU. */
 int  oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y,
                           uint32_t n_rows, uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us);
+int  oxb_hip_profile_gemv_floor(const uint64_t* ids, uint32_t n_ids, uint32_t n_rows, uint32_t k, uint32_t warmup,
+                                uint32_t iters, float* avg_us);
 
 /* ---- uncached one-shot calls: gemv_q1_g128 (KG/mod.rs:412), gemm_q1_g128 (:425) and their ternary twins.
  * Validation follows the scalar kernels (crates/oxibonsai-kernels/src/gemv.rs:32-58): k % 128, buffer lengths. */
@@ -134,8 +138,8 @@ int  oxb_hip_model_destroy(uint64_t model);
 /* One token for each of the `batch` sequences: hidden[batch][h] are the embedding rows, pos[batch] the positions.
  * Runs all layers, the final norm, the LM head and a first-maximum argmax on the device (a HIP graph after the first
  * call).  logits_or_null: [batch][vocab]; token_out: [batch] greedy ids (either may be NULL).
- * Batches of 1 and 2 use the fp32-exact GEMV; from 3 sequences on the projections run as fp16 matrix-core GEMMs
- * (the arithmetic of oxb_hip_gemm / oxb_hip_prefill). */
+ * Batches of up to 4 use the fp32-exact GEMV (one pass over the weights); from 5 sequences on the projections run as
+ * fp16 matrix-core GEMMs (the arithmetic of oxb_hip_gemm / oxb_hip_prefill). */
 int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out);
 /* Batched prefill: try_cuda_prefill / try_cuda_prefill_ternary (KG/cuda_prefill/try_apis.rs:42, 318; per layer
  * encode_prefill_layer[_ternary], KG/cuda_prefill/encode_q1.rs:123, encode_ternary.rs:114).  hidden = [n_tokens][h]

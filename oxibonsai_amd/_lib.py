@@ -34,6 +34,7 @@ _SIGNATURES = {
     "oxb_hip_gemv_dev": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_profile_gemv": ([u64p, C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
                               C.c_uint32, f32p], C.c_int),
+    "oxb_hip_profile_gemv_floor": ([u64p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, f32p], C.c_int),
     "oxb_hip_gemm": ([C.c_uint64, f32p, f32p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_gemm_dev": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_gemm_dev_static": ([C.c_uint64, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32], C.c_int),

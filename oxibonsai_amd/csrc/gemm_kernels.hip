@@ -192,10 +192,10 @@ __device__ __forceinline__ void load_half(HalfRegs<FMT>& H, __amdgpu_buffer_rsrc
         H.c[0] = (uint32_t)v.x, H.c[1] = (uint32_t)v.y, H.c[FMT == OXB_FMT_Q1 ? 0 : 2] = (uint32_t)v.z,
         H.c[FMT == OXB_FMT_Q1 ? 1 : 3] = (uint32_t)v.w;
     }
-    const uint32_t sv = ((r >> 2) * 16u + (r & 3u)) * 2u + half * 16u;  // scale of block 2*half, then +8 bytes
-#pragma unroll
-    for (int e = 0; e < 2; e++)
-        H.d[e] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rs, (int)(ok ? sv + e * 8u : OXB_OOB), (int)(unit * 128u), 0);
+    // scales of blocks 2 * half and 2 * half + 1 of this lane's row lie side by side
+    const uint32_t sv = __builtin_amdgcn_raw_buffer_load_b32(rs, (int)(ok ? r * 8u + half * 4u : OXB_OOB), (int)(unit * 128u), 0);
+    H.d[0] = sv & 0xFFFFu;
+    H.d[1] = sv >> 16;
 }
 
 // Per (row tile, block) state prepared once and used by the four MFMA steps of the block.

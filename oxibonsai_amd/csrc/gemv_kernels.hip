@@ -1,64 +1,45 @@
 // gemv_kernels.hip — Q1_0_g128 / TQ2_0_g128 GEMV for gfx950 (MI355X).
 //
 // What it computes (reference: crates/oxibonsai-kernels/src/gemv.rs:60-84,
-// gemv_ternary.rs:83-102):  y[row] = sum_blocks f16(d) * sum_128 code(w) * x.
+// gemv_ternary.rs:83-102):  y[row] = sum_blocks f16(d) * sum_128 code(w) * x,
+// optionally with RMSNorm in front (simd_float_ops.rs:204-215) and a residual add or SwiGLU
+// (simd_float_ops.rs:217-236) behind it, as the reference's fused kernels gemv_*_residual and
+// fused_gate_up_swiglu_q1 do (gpu_backend/cuda_kernels.rs:130-178, 456-543).
 //
-// Why int8 MFMA and not per-weight VALU decode.  At 8 TB/s a Q1 stream delivers
-// 64e12 weights/s, but the chip retires only ~39e12 non-packed VALU lane-ops/s
-// (256 CU x 64 lanes x 2.4 GHz), so any scheme that spends >= 1 VALU op per
-// weight is compute-bound at < 61 % of the HBM roofline.  Here a weight costs
-// 1/4 VALU op: one AND with 0x01010101 << j (Q1) or 0x03030303 << 2jj (TQ2)
-// turns a code dword into four int8 MFMA operands worth 2^j (4^jj) each, and the
-// activation vector is pre-divided by the same power of two when it is
-// quantised.  The fp32 activation is carried exactly: each x is scaled by a
-// per-vector power of two to a 54-bit integer (every element within 2^22 of the
-// largest one keeps all 24 mantissa bits) and split into eight balanced int8
-// digits which occupy eight MFMA columns, so one 16x16x64 MFMA multiplies 16
-// rows x 64 weights by all eight digits of up to two activation vectors.
-// Block sums are exact integers; the per-block f16 scale is applied in fp32.
+// Why int8 MFMA and not per-weight VALU decode.  At 8 TB/s a Q1 stream delivers 64e12 weights/s, but
+// the chip retires about 33e12 VALU lane-operations/s, so any scheme that spends one VALU operation
+// per weight is compute-bound far below the HBM roofline.  Here a weight costs 1/4 VALU operation: one
+// AND with 0x01010101 << j (Q1) or 0x03030303 << 2jj (TQ2) turns a code dword into four int8 MFMA
+// operands worth 2^j (4^jj) each, and the activation that meets them was divided by the same power of
+// two when it was quantised.
+//
+// One kernel does everything.  The weights are the MFMA's B operand (16 weight rows = 16 columns), the
+// activations its A operand: every activation is scaled by a power of two - one per K slice of a wave,
+// 512 to 1536 values - to a 30-bit integer and cut into four balanced base-256 digits, which occupy four
+// of the sixteen A rows, so up to four activation vectors share one pass over the weights.  A lane then
+// holds the four digit sums of one (vector, weight row) pair: they are joined by two shift-adds, two
+// conversions and one FMA, the fp16 block scale is applied by one mixed-precision FMA, the slice's power
+// of two comes back with one ldexp per tile.  Block sums are exact integers; the rounding of the
+// activations to 2^-26 .. 2^-30 of their slice's largest element is below what the fp32 sums of the
+// reference lose (Q1 masks the high nibble of a code byte after a shift by 4, so that no operand byte
+// is worth more than 8 and no activation gives up more than three bits to it).
+// The quantisation happens in the kernel's prologue: the waves of a workgroup split K, and each wave
+// quantises exactly the K slice it owns (the activations are requested before the weight stream, so
+// they arrive while the first weight tiles are still on their way) - no quantiser kernel, no digit
+// planes in memory.  Every workgroup repeats that work; it hides behind the first HBM round trip.
 //
 // Kernels:
-//   quant_x_kernel   x[batch][k] fp32 -> int8 digit planes in MFMA B-operand order
-//   gemv_mfma_kernel codes/scales (tiled SoA, see layout.h) x digit planes -> y
-//   dequant_kernel   resident layout -> fp32 weights (bit-exactness check)
+//   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y
+//   stream_floor_kernel  the same loads and nothing else (measurement aid)
+//   dequant_kernel       resident layout -> fp32 weights (bit-exactness check)
+//   swiglu_kernel        silu(gate) * up on fp32 vectors (rows too long for one GEMV launch)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "device_utils.h"
 #include "gemv_kernels.h"
 #include "layout.h"
-#include "quant_device.h"
 
-
-// The activation quantiser (quant_device.h) produces the MFMA B operands ("digit planes").
-#define OXB_QUANT_THREADS 256
-
-// Grid (vectors, parts): each workgroup takes whole exponent groups of one vector, finds their maxima and
-// quantises them; no workgroup needs anything from another.
-template <int FMT>
-__global__ __launch_bounds__(OXB_QUANT_THREADS) void quant_x_kernel(const float* __restrict__ x, uint32_t k, uint32_t NC,
-                                                                     uint32_t gsb, uint32_t n_groups,
-                                                                     uint32_t* __restrict__ xq,
-                                                                     int32_t* __restrict__ cneg,
-                                                                     int32_t* __restrict__ xexp) {
-    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
-    const uint32_t n = blockIdx.x;
-    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
-    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
-    if (g0 >= g1) return;
-    const float* xn = x + (size_t)n * k;
-    gstat_scan(xn, k, gsb, g0, g1, gstat);
-    quantise_groups<FMT>(xn, k, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
-}
-
-// ---------------------------------------------------------------------------
-// GEMV.  One workgroup = S waves; wave s owns superblocks
-// [sb_begin + s*NSBW, +NSBW) of every row tile the workgroup processes and keeps
-// the matching slice of the digit planes in registers for the whole kernel, so
-// the inner loop is: one coalesced 1 KiB code load per superblock, 4 ANDs + 1
-// MFMA per 64 weights of 16 rows, 4 cvt + 4 fma per block for the scale.
-// Partial row sums of the S waves meet in LDS; the last step weighs and adds the eight digit
-// columns (DPP) and applies the epilogue (store / +=).
-// ---------------------------------------------------------------------------
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
     return (float)__builtin_bit_cast(_Float16, (unsigned short)h);
 }
@@ -68,7 +49,7 @@ template <int FMT, int NSBW>
 struct TileRegs {
     static constexpr int UNITS = (FMT == OXB_FMT_Q1) ? 1 : 2;  // 1 KiB code units per superblock
     v4i w[NSBW][UNITS];
-    uint32_t sc[NSBW];  // lane (c, rg): f16 pair (c & 7) of row group rg, pair 2q+p = scales of block q, rows 2p, 2p+1
+    v2u sc[NSBW];  // the four f16 scales (blocks 0..3 of the superblock) of this lane's weight row
 };
 
 // `valid`, `tile` and the unit index are wave-uniform: they travel in scalar registers, the lane
@@ -84,143 +65,337 @@ __device__ __forceinline__ void load_tile(TileRegs<FMT, NSBW>& t, __amdgpu_buffe
         const uint32_t unit = __builtin_amdgcn_readfirstlane(tile * n_sb + sb0 + (uint32_t)i);
 #pragma unroll
         for (int u = 0; u < UNITS; u++) t.w[i][u] = buf_load_b128(codes, ok ? lane_c : OXB_OOB, (unit * UNITS + u) * 1024u);
-        t.sc[i] = buf_load_b32(scales, ok ? lane_s : OXB_OOB, unit * 128u);
+        t.sc[i] = __builtin_amdgcn_raw_buffer_load_b64(scales, (int)(ok ? lane_s : OXB_OOB), (int)(unit * 128u), 0);
     }
 }
 
-// One block: two MFMAs over its 128 weights, then the f16 scale in fp32.
-template <int FMT, int Q>
-__device__ __forceinline__ void block_mac(v4f& accf, uint32_t d0, uint32_t d1, const v4i& b0, const v4i& b1,
-                                          const v4i& c4, uint32_t scdw) {
-    v4i a0, a1;
-    if (FMT == OXB_FMT_Q1) {  // d0 == d1: 32 sign bits
-        a0 = (v4i){(int)(d0 & 0x01010101u), (int)(d0 & 0x02020202u), (int)(d0 & 0x04040404u), (int)(d0 & 0x08080808u)};
-        a1 = (v4i){(int)(d0 & 0x10101010u), (int)(d0 & 0x20202020u), (int)(d0 & 0x40404040u), (int)(d0 & 0x80808080u)};
-    } else {  // 16 two-bit fields each
-        a0 = (v4i){(int)(d0 & 0x03030303u), (int)(d0 & 0x0C0C0C0Cu), (int)(d0 & 0x30303030u), (int)(d0 & 0xC0C0C0C0u)};
-        a1 = (v4i){(int)(d1 & 0x03030303u), (int)(d1 & 0x0C0C0C0Cu), (int)(d1 & 0x30303030u), (int)(d1 & 0xC0C0C0C0u)};
-    }
-    v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a0, b0, c4, 0, 0, 0);
-    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(a1, b1, acc, 0, 0, 0);
-    const uint32_t p0 = dpp_u32<OXB_DPP_ROW_NEWBCAST(2 * Q)>(scdw);      // scales of rows 4g+0, 4g+1
-    const uint32_t p1 = dpp_u32<OXB_DPP_ROW_NEWBCAST(2 * Q + 1)>(scdw);  // rows 4g+2, 4g+3
-    accf[0] = fmaf((float)acc[0], f16_bits_to_f32(p0 & 0xFFFFu), accf[0]);
-    accf[1] = fmaf((float)acc[1], f16_bits_to_f32(p0 >> 16), accf[1]);
-    accf[2] = fmaf((float)acc[2], f16_bits_to_f32(p1 & 0xFFFFu), accf[2]);
-    accf[3] = fmaf((float)acc[3], f16_bits_to_f32(p1 >> 16), accf[3]);
+// 4 x 4 byte transpose: o[d] = { t[0].byte d, t[1].byte d, t[2].byte d, t[3].byte d }.
+__device__ __forceinline__ void transpose_bytes4(const uint32_t t[4], uint32_t o[4]) {
+    const uint32_t p01l = __builtin_amdgcn_perm(t[1], t[0], 0x05010400u), p01h = __builtin_amdgcn_perm(t[1], t[0], 0x07030602u);
+    const uint32_t p23l = __builtin_amdgcn_perm(t[3], t[2], 0x05010400u), p23h = __builtin_amdgcn_perm(t[3], t[2], 0x07030602u);
+    o[0] = __builtin_amdgcn_perm(p23l, p01l, 0x05040100u);
+    o[1] = __builtin_amdgcn_perm(p23l, p01l, 0x07060302u);
+    o[2] = __builtin_amdgcn_perm(p23h, p01h, 0x05040100u);
+    o[3] = __builtin_amdgcn_perm(p23h, p01h, 0x07060302u);
 }
 
-// Workgroup wg handles row tiles [wg * groups * TG, +groups * TG); TG tiles are in flight per
-// wave at any time and are recombined together.  All control flow is uniform and branch-free
-// inside a group, so the compiler can wait for exactly the tile it is about to use.
-template <int FMT, int NSBW, int TG>
-__global__ __launch_bounds__(512, (NSBW == 1 ? 4 : 2)) void gemv_mfma_kernel(const OxbGemvParams p) {
-    extern __shared__ float part[];  // [2][TG][S][NC][16]
-    constexpr int UNITS = TileRegs<FMT, NSBW>::UNITS;
+// Unsigned maximum / integer sum over the 32 lanes of a half wave (lanes 0-31, 32-63), result in every lane.  Zero is
+// the identity of both, so the DPP moves (which hand 0 to a lane without a source) fold into the arithmetic.
+__device__ __forceinline__ uint32_t half_umax(uint32_t v) {
+    v = max(v, dpp_u32<0xB1>(v));    // quad_perm [1,0,3,2]
+    v = max(v, dpp_u32<0x4E>(v));    // quad_perm [2,3,0,1]
+    v = max(v, dpp_u32<0x141>(v));   // row_half_mirror
+    v = max(v, dpp_u32<0x140>(v));   // row_mirror
+    return max(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F));  // lane ^ 16
+}
+__device__ __forceinline__ int half_isum(int v) {
+    v += dpp_i32<0xB1>(v);
+    v += dpp_i32<0x4E>(v);
+    v += dpp_i32<0x141>(v);
+    v += dpp_i32<0x140>(v);
+    return v + __builtin_amdgcn_ds_swizzle(v, 0x401F);
+}
+
+// Fixed point of the quantised activations.  2^E > max |x| of a wave's K slice, r = rint(x * 2^(P - E - s)) with s the
+// power of two the weight's operand byte carries (Q1: bit j of a code byte is worth 2^(j & 3), the high nibble being
+// masked after a shift by 4; TQ2: field jj is worth 4^jj).  Q1 operands hold 2 r (weights are 2 b - 1), so
+// |operand| < 2^30 needs P = 29; TQ2 P = 30.
+template <int FMT>
+struct Fix {
+    static constexpr int P = (FMT == OXB_FMT_Q1) ? 29 : 30;
+    __device__ static __forceinline__ int shift_of(uint32_t j) { return FMT == OXB_FMT_Q1 ? (int)(j & 3u) : 2 * (int)(j & 3u); }
+};
+
+#define OXB_GEMV_META 4  // ints of per-block metadata a wave leaves in LDS: the four accumulator start values
+
+// Dynamic LDS of a launch: [S][NSBW * 512] staging dwords | [S][NSBW * 4][META] | part [4][TG][S][64] floats | red [16] | flags [4]
+__host__ __device__ inline size_t oxb_gemv_lds_bytes(uint32_t S, uint32_t nsbw, uint32_t tg) {
+    return ((size_t)S * nsbw * 512 + (size_t)S * nsbw * 4 * OXB_GEMV_META + (size_t)4 * tg * S * 64 + 16 + 4) * 4;
+}
+
+// Workgroup wg handles tile slots [wg * tpw, +tpw) in groups of TG (TG tiles are in flight per wave).  For the SwiGLU
+// epilogue the groups alternate between TG gate tiles and the TG up tiles of the same rows.  All control flow is
+// uniform and branch-free inside a group, so the compiler waits for exactly the tile it is about to use.
+template <int FMT, int NSBW, int TG, int PRO>
+__global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
+    extern __shared__ uint32_t smem[];
     const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
-    const uint32_t c = lane & 15u, g = lane >> 4;  // B operand: column c, k-group g; D: column c, rows 4g..4g+3
-    const uint32_t NC = p.NC;
-    const bool col_on = c < NC;
+    const uint32_t c = lane & 15u, g = lane >> 4;  // D: weight row c of the tile, activation vector g
+    const uint32_t nvec = p.nvec;
+    const bool swiglu = p.epi == OXB_GEMV_SWIGLU;
+    uint32_t* stage = smem + (size_t)s * NSBW * 512;
+    int* meta = (int*)(smem + (size_t)S * NSBW * 512) + (size_t)s * NSBW * 4 * OXB_GEMV_META;
+    float* part = (float*)(smem + (size_t)S * NSBW * 512 + (size_t)S * NSBW * 4 * OXB_GEMV_META);
+    float* red = part + (size_t)4 * TG * S * 64;
+    int* flags = (int*)(red + 16);
 
-    const uint32_t lane_c = lane * 16u, lane_s = ((lane >> 4) * 8u + (lane & 7u)) * 4u;
+    const uint32_t lane_c = lane * 16u, lane_s = c * 8u;
     const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
     const int sb_lim = (int)(p.sb_begin + p.sb_count) - (int)sb0;  // superblocks of this wave's slice that exist
-
     const __amdgpu_buffer_rsrc_t r_codes = make_rsrc(p.codes, p.codes_bytes);
     const __amdgpu_buffer_rsrc_t r_scales = make_rsrc(p.scales, p.scales_bytes);
-    const __amdgpu_buffer_rsrc_t r_xq = make_rsrc(p.xq, p.xq_bytes);
-    const __amdgpu_buffer_rsrc_t r_cneg = make_rsrc(p.cneg, p.cneg_bytes);
 
-    // Digit planes and accumulator start values of this wave's K slice (L2-resident), issued
-    // first so that the weight stream behind them can be consumed tile by tile as it arrives.
-    v4i B[NSBW][4][2];
-    v4i C4[NSBW][4];
+    // slot (group, t) -> row tile
+    const uint32_t half_tiles = p.n_tiles >> 1;
+    const uint32_t n_units = swiglu ? half_tiles : p.n_tiles;                // gate tiles, or all tiles
+    const uint32_t upw = swiglu ? (p.tpw >> 1) : p.tpw, u_begin = blockIdx.x * upw;
+    const uint32_t groups = p.tpw / TG;
+    auto unit_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return u_begin + (swiglu ? (grp >> 1) : grp) * TG + t; };
+    auto tile_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return unit_of(grp, t) + ((swiglu && (grp & 1u)) ? half_tiles : 0u); };
+    auto slot_ok = [&](uint32_t grp, uint32_t t) -> bool { return grp < groups && unit_of(grp, t) < n_units && unit_of(grp, t) < u_begin + upw; };
+
+    // ---- prologue: this wave's K slice of every vector -> MFMA A operands ----
+    // Loads complete in issue order, so the activations of the first vector are requested before the weight stream.
+    constexpr uint32_t KS = FMT == OXB_FMT_Q1 ? 8 : 4;
+    // lane -> (block of the superblock half, 32-weight group, bit position / field) of its four activations per pass:
+    // Q1 k = 128 blk + 32 gg + 8 bb + j;  TQ2 k = 128 blk + 32 gg + 16 (j >> 2) + 4 bb + (j & 3),  bb = 0..3
+    const uint32_t j = lane & 7u, gg = (lane >> 3) & 3u, blh = lane >> 5;
+    const uint32_t koff = (FMT == OXB_FMT_Q1 ? 32 * gg + j : 32 * gg + 16 * (j >> 2) + (j & 3u)) * 4u;
+    const int js = Fix<FMT>::shift_of(j);
+    const __amdgpu_buffer_rsrc_t r_w = make_rsrc(p.norm_w, PRO == OXB_GEMV_PRO_RMSNORM ? p.k * 4u : 0u);
+    float xe[NSBW][2][4], we[NSBW][2][4];
+    // Only requests: nothing here waits for the values, so the weight stream can be requested right behind them.
+    auto load_x = [&](uint32_t v) {
+        const __amdgpu_buffer_rsrc_t r_x = make_rsrc(p.x + (size_t)v * p.ldx, p.k * 4u);
 #pragma unroll
-    for (int i = 0; i < NSBW; i++)
+        for (int i = 0; i < NSBW; i++)
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const bool ok = col_on && i < sb_lim;
-            const uint32_t blk = (sb0 + (uint32_t)i) * 4 + q;
-            B[i][q][0] = buf_load_b128(r_xq, ok ? (((blk * 2 + 0) * 4 + g) * NC + c) * 16u : OXB_OOB);
-            B[i][q][1] = buf_load_b128(r_xq, ok ? (((blk * 2 + 1) * 4 + g) * NC + c) * 16u : OXB_OOB);
-            C4[i][q] = buf_load_b128(r_cneg, ok ? (blk * NC + c) * 16u : OXB_OOB);
-        }
-    // In the recombination, thread t handles column (t % NC): digit (t % 8) of vector (t % NC) / 8, and needs
-    // the exponent of every wave's K slice (= exponent group) of that vector.
-    __shared__ int xes[2 * 8];  // [vector][wave]; published by the first barrier of the tile loop
-    if (threadIdx.x < 16) {
-        const uint32_t vec = threadIdx.x >> 3, w = threadIdx.x & 7u;
-        xes[threadIdx.x] = (vec * 8 < NC && w < S) ? p.xexp[vec * p.n_groups + p.sb_begin / NSBW + w] : 0;
-    }
-    const uint32_t my_vec = (threadIdx.x % NC) >> 3;
-
-    const uint32_t tpw = p.groups * TG, t_begin = blockIdx.x * tpw;
-    const uint32_t t_end = (t_begin + tpw) < p.n_tiles ? (t_begin + tpw) : p.n_tiles;
-
-    // The scheduling barriers pin the issue order of the loads: memory returns in issue order, so
-    // "tile t has arrived" is a wait for all but the loads issued after it.
+            for (int pass = 0; pass < 2; pass++) {
+                const uint32_t blk = (sb0 + i) * 4 + pass * 2 + blh;
+                const uint32_t off = i < sb_lim ? blk * 512u + koff : OXB_OOB;  // beyond k the buffer returns 0
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) {
+                    xe[i][pass][bb] = __uint_as_float(buf_load_b32(r_x, off + KS * 4u * bb));
+                    if (PRO == OXB_GEMV_PRO_RMSNORM) we[i][pass][bb] = __uint_as_float(buf_load_b32(r_w, off + KS * 4u * bb));
+                }
+            }
+    };
+    load_x(0);
     __builtin_amdgcn_sched_barrier(0);
     TileRegs<FMT, NSBW> ring[TG];
 #pragma unroll
     for (int t = 0; t < TG; t++) {
-        load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, t_begin + t, t_begin + t < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+        load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
         __builtin_amdgcn_sched_barrier(0);
     }
+    if (threadIdx.x < 4) flags[threadIdx.x] = 0;
 
-    for (uint32_t grp = 0; grp < p.groups; grp++) {
-        float* buf = part + (size_t)(grp & 1u) * TG * S * NC * 16;
+    v4i A[NSBW][4][2];  // [superblock][block][MFMA]: digit d of vector v in lanes with c = 4 v + d
+    v4i C4[NSBW][4];    // accumulator start values (they cancel the bias of the unsigned code encodings), lanes with g = v
+    int EX = 0;         // E - P of this wave's K slice of vector g
+#pragma unroll
+    for (int i = 0; i < NSBW; i++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            A[i][q][0] = (v4i){0, 0, 0, 0};
+            A[i][q][1] = (v4i){0, 0, 0, 0};
+            C4[i][q] = (v4i){0, 0, 0, 0};
+        }
+    auto quantise_vector = [&](const uint32_t v) {
+        uint32_t bad = 0;
+        float inv_rms = 1.f;
+        if (PRO == OXB_GEMV_PRO_RMSNORM) {
+            // Sum of squares over the whole vector: every wave adds its own slice (in registers already); what the
+            // waves of this launch do not cover between them is added by a strided loop.
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < NSBW; i++)
+#pragma unroll
+                for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+                    for (int bb = 0; bb < 4; bb++) {
+                        ss = fmaf(xe[i][pass][bb], xe[i][pass][bb], ss);
+                        xe[i][pass][bb] *= we[i][pass][bb];
+                    }
+            const uint32_t c0 = p.sb_begin * 512u, c1 = (p.sb_begin + S * NSBW) * 512u;
+            if (c0 > 0 || c1 < p.k) {
+                const float* xv = p.x + (size_t)v * p.ldx;
+                for (uint32_t i = threadIdx.x; i < p.k; i += blockDim.x)
+                    if (i < c0 || i >= c1) ss = fmaf(xv[i], xv[i], ss);
+            }
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            if (lane == 0) red[s] = ss;
+            __syncthreads();
+            float tot = 0.f;
+            for (uint32_t w = 0; w < S; w++) tot += red[w];
+            inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+            bad |= !(fabsf(inv_rms) <= 3.402823466e38f);
+            __syncthreads();
+        } else if (v == 0) {
+            __syncthreads();  // flags cleared
+        }
+        // exponent of the slice: |x| as integers are ordered like the floats, NaN and infinity on top
+        uint32_t mxb = 0;
+#pragma unroll
+        for (int i = 0; i < NSBW; i++)
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) {
+                    if (PRO == OXB_GEMV_PRO_RMSNORM) xe[i][pass][bb] *= inv_rms;
+                    mxb = max(mxb, __float_as_uint(xe[i][pass][bb]) & 0x7FFFFFFFu);
+                }
+        mxb = half_umax(mxb);
+        mxb = max((uint32_t)__builtin_amdgcn_readlane((int)mxb, 0), (uint32_t)__builtin_amdgcn_readlane((int)mxb, 32));
+        bad |= mxb >= 0x7F800000u;
+        const uint32_t be = mxb >> 23;
+        const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x| (subnormal maxima share the smallest E)
+        const int sh = Fix<FMT>::P - E - js;
+#pragma unroll
+        for (int i = 0; i < NSBW; i++) {
+#pragma unroll
+            for (int pass = 0; pass < 2; pass++) {
+                const uint32_t bl = pass * 2 + blh;
+                int r[4];
+#pragma unroll
+                for (int bb = 0; bb < 4; bb++) r[bb] = (int)rintf(ldexpf(xe[i][pass][bb], sh));
+                uint32_t tb[4];
+                // block sum of 2^js r, in two parts that cannot overflow (|r| <= 2^30)
+                int cl = (r[0] & 0x7FFF) + (r[1] & 0x7FFF) + (r[2] & 0x7FFF) + (r[3] & 0x7FFF);
+                int ch = (r[0] >> 15) + (r[1] >> 15) + (r[2] >> 15) + (r[3] >> 15);
+                if (FMT == OXB_FMT_Q1) {
+#pragma unroll
+                    for (int bb = 0; bb < 4; bb++) tb[bb] = (((uint32_t)r[bb] << 1) + 0x00808080u) ^ 0x00808080u;
+                } else {
+#pragma unroll
+                    for (int bb = 0; bb < 4; bb++) tb[bb] = ((uint32_t)r[bb] + 0x00808080u) ^ 0x00808080u;
+                    if ((j & 3u) == 3u) cl = 0, ch = 0;  // field 3 is two's complement: no bias
+                }
+                cl = half_isum(cl << js), ch = half_isum(ch << js);
+                uint32_t D[4];
+                transpose_bytes4(tb, D);
+                const uint32_t m = j >> 2, jj = j & 3u;
+#pragma unroll
+                for (int d = 0; d < 4; d++) stage[((((i * 4 + bl) * 2 + m) * 16 + gg * 4 + d) << 2) + jj] = D[d];
+                if ((lane & 31u) == 0) {
+                    const long long nc = -(((long long)ch << 15) + cl);  // as three balanced digits and a remainder
+                    const unsigned long long t = ((unsigned long long)nc + 0x808080ull) ^ 0x808080ull;
+                    *reinterpret_cast<v4i*>(meta + (i * 4 + bl) * OXB_GEMV_META) =
+                        (v4i){(int)(signed char)(t & 0xFF), (int)(signed char)((t >> 8) & 0xFF), (int)(signed char)((t >> 16) & 0xFF),
+                              (int)((long long)t >> 24)};
+                }
+            }
+        }
+        if (__builtin_amdgcn_ballot_w64(bad != 0) != 0 && lane == 0) atomicOr(&flags[v], 1);
+        // the staging area is this wave's own: LDS operations of a wave execute in order
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if ((c >> 2) == v) {
+#pragma unroll
+            for (int i = 0; i < NSBW; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++)
+#pragma unroll
+                    for (int m = 0; m < 2; m++)
+                        A[i][q][m] = *reinterpret_cast<const v4i*>(&stage[(((i * 4 + q) * 2 + m) * 16 + g * 4 + (c & 3u)) << 2]);
+        }
+        if (g == v) {
+#pragma unroll
+            for (int i = 0; i < NSBW; i++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) C4[i][q] = *reinterpret_cast<const v4i*>(meta + (i * 4 + q) * OXB_GEMV_META);
+            EX = mxb ? E - Fix<FMT>::P : 0;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+    };
+    quantise_vector(0);  // on the activations requested ahead of the weight stream
+    for (uint32_t v = 1; v < nvec; v++) {
+        load_x(v);
+        quantise_vector(v);
+    }
+
+    // ---- main loop ----
+    for (uint32_t grp = 0; grp < groups; grp++) {
+        float* buf = part + (size_t)(grp & 3u) * TG * S * 64;
 #pragma unroll
         for (int t = 0; t < TG; t++) {
-            const uint32_t tile = t_begin + grp * TG + t;
-            v4f accf = {0.f, 0.f, 0.f, 0.f};
+            float accf = 0.f;
             const TileRegs<FMT, NSBW>& r = ring[t];
 #pragma unroll
             for (int i = 0; i < NSBW; i++) {
-                if (FMT == OXB_FMT_Q1) {
-                    block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][0], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
-                    block_mac<FMT, 1>(accf, r.w[i][0][1], r.w[i][0][1], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
-                    block_mac<FMT, 2>(accf, r.w[i][0][2], r.w[i][0][2], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
-                    block_mac<FMT, 3>(accf, r.w[i][0][3], r.w[i][0][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
-                } else {
-                    block_mac<FMT, 0>(accf, r.w[i][0][0], r.w[i][0][1], B[i][0][0], B[i][0][1], C4[i][0], r.sc[i]);
-                    block_mac<FMT, 1>(accf, r.w[i][0][2], r.w[i][0][3], B[i][1][0], B[i][1][1], C4[i][1], r.sc[i]);
-                    block_mac<FMT, 2>(accf, r.w[i][UNITS - 1][0], r.w[i][UNITS - 1][1], B[i][2][0], B[i][2][1], C4[i][2], r.sc[i]);
-                    block_mac<FMT, 3>(accf, r.w[i][UNITS - 1][2], r.w[i][UNITS - 1][3], B[i][3][0], B[i][3][1], C4[i][3], r.sc[i]);
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i b0, b1;
+                    if (FMT == OXB_FMT_Q1) {  // 32 sign bits: low nibbles of the four bytes, then the high nibbles
+                        const uint32_t d0 = (uint32_t)r.w[i][0][q], d1 = d0 >> 4;
+                        b0 = (v4i){(int)(d0 & 0x01010101u), (int)(d0 & 0x02020202u), (int)(d0 & 0x04040404u), (int)(d0 & 0x08080808u)};
+                        b1 = (v4i){(int)(d1 & 0x01010101u), (int)(d1 & 0x02020202u), (int)(d1 & 0x04040404u), (int)(d1 & 0x08080808u)};
+                    } else {  // 16 two-bit fields each
+                        const uint32_t d0 = (uint32_t)r.w[i][q >> 1][(q & 1) * 2], d1 = (uint32_t)r.w[i][q >> 1][(q & 1) * 2 + 1];
+                        b0 = (v4i){(int)(d0 & 0x03030303u), (int)(d0 & 0x0C0C0C0Cu), (int)(d0 & 0x30303030u), (int)(d0 & 0xC0C0C0C0u)};
+                        b1 = (v4i){(int)(d1 & 0x03030303u), (int)(d1 & 0x0C0C0C0Cu), (int)(d1 & 0x30303030u), (int)(d1 & 0xC0C0C0C0u)};
+                    }
+                    v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][q][0], b0, C4[i][q], 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(A[i][q][1], b1, acc, 0, 0, 0);
+                    // four digit sums of (vector g, weight row c): sum_d 256^d acc[d], then the block scale
+                    const int lo = acc[0] + (acc[1] << 8), hi = acc[2] + (acc[3] << 8);
+                    const float val = fmaf((float)hi, 65536.0f, (float)lo);
+                    const uint32_t scw = (q < 2) ? r.sc[i].x : r.sc[i].y;
+                    accf = fmaf(val, f16_bits_to_f32((q & 1) ? scw >> 16 : scw & 0xFFFFu), accf);
                 }
             }
-            // refill this ring slot with the tile TG ahead (reads nothing past the workgroup's range)
-            load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile + TG, tile + TG < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+            // refill this ring slot with the same slot of the next group (reads nothing past the workgroup's range)
+            load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(grp + 1, t), slot_ok(grp + 1, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
             __builtin_amdgcn_sched_barrier(0);
-            if (col_on) *reinterpret_cast<v4f*>(&buf[(((size_t)t * S + s) * NC + c) * 16 + g * 4]) = accf;
+            buf[((size_t)t * S + s) * 64 + lane] = ldexpf(accf, EX);  // the slice's 2^(E - P)
         }
         lds_barrier();
-        // thread -> (slot, row, column): add the S partial sums in a fixed order, weigh the digit
-        // by 2^(8 digit + E - P), then add the eight digit columns of a vector across lanes.
-        for (uint32_t idx = threadIdx.x; idx < (uint32_t)TG * 16 * NC; idx += blockDim.x) {
-            const uint32_t cc = idx % NC, rr = (idx / NC) & 15u, slot = idx / (16 * NC);
-            float v = 0.f;
-            bool nan = false;
-#pragma unroll
-            for (int w = 0; w < 8; w++)
-                if ((uint32_t)w < S) {
-                    const int xe = xes[my_vec * 8 + w];
-                    nan |= xe == INT32_MIN;
-                    v += ldexpf(buf[(((size_t)slot * S + w) * NC + cc) * 16 + rr], xe + 8 * (int)(cc & 7u));
-                }
-            if (nan) v = __int_as_float(0x7FC00000);
-            v += dpp_f32<OXB_DPP_ROW_SHR(1)>(v);
-            v += dpp_f32<OXB_DPP_ROW_SHR(2)>(v);
-            v += dpp_f32<OXB_DPP_ROW_SHR(4)>(v);
-            const uint32_t tile = t_begin + grp * TG + slot, row = tile * 16 + rr;
-            if ((cc & 7u) == 7u && tile < t_end && row < p.n_rows) {
-                const size_t o = (size_t)(cc >> 3) * p.ldy + row;
-                if (p.mode == OXB_GEMV_ACCUM) v += p.y[o];
-                else if (p.mode == OXB_GEMV_RESIDUAL) v += p.residual[o];
-                p.y[o] = v;
-            }
+        if (swiglu && !(grp & 1u)) continue;  // the gate sums wait for the up sums of the same rows
+        // thread -> (slot, vector, row): add the S partial sums in wave order, then the epilogue.  No second barrier:
+        // the next groups write other quarters of `part`, and a quarter is reused only after two more barriers.
+        const float* gbuf = part + (size_t)((grp - 1) & 3u) * TG * S * 64;
+        for (uint32_t idx = threadIdx.x; idx < (uint32_t)TG * 64; idx += blockDim.x) {
+            const uint32_t t = idx >> 6, ln = idx & 63u, cc = ln & 15u, vv = ln >> 4;
+            if (vv >= nvec || !slot_ok(grp, t)) continue;
+            float v0 = 0.f, v1 = 0.f;
+            for (uint32_t w = 0; w < S; w++) v0 += buf[((size_t)t * S + w) * 64 + ln];
+            if (swiglu)
+                for (uint32_t w = 0; w < S; w++) v1 += gbuf[((size_t)t * S + w) * 64 + ln];
+            if (flags[vv]) v0 = __int_as_float(0x7FC00000);
+            const uint32_t row = unit_of(grp, t) * 16 + cc;
+            if (row >= (swiglu ? (p.n_rows >> 1) : p.n_rows)) continue;
+            const size_t o = (size_t)vv * p.ldy + row;
+            if (swiglu) v0 = (v1 / (1.0f + expf(-v1))) * v0;  // v1 = gate, v0 = up
+            else if (p.epi == OXB_GEMV_ACCUM) v0 += p.y[o];
+            else if (p.epi == OXB_GEMV_RESIDUAL) v0 += p.residual[o];
+            p.y[o] = v0;
         }
-        // no second barrier: the next group writes the other half of `part`
     }
+}
+
+// The same grid, waves, ring and addresses as gemv_kernel, and no arithmetic beyond an OR.
+template <int FMT, int NSBW, int TG>
+__global__ __launch_bounds__(512) void stream_floor_kernel(const OxbGemvParams p) {
+    const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6;
+    const uint32_t lane_c = lane * 16u, lane_s = (lane & 15u) * 8u;
+    const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
+    const int sb_lim = (int)(p.sb_begin + p.sb_count) - (int)sb0;
+    const __amdgpu_buffer_rsrc_t r_codes = make_rsrc(p.codes, p.codes_bytes);
+    const __amdgpu_buffer_rsrc_t r_scales = make_rsrc(p.scales, p.scales_bytes);
+    const uint32_t t_begin = blockIdx.x * p.tpw;
+    const uint32_t t_end = (t_begin + p.tpw) < p.n_tiles ? (t_begin + p.tpw) : p.n_tiles;
+    TileRegs<FMT, NSBW> ring[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++) load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, t_begin + t, t_begin + t < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+    uint32_t acc = 0;
+    for (uint32_t grp = 0; grp < p.tpw / TG; grp++) {
+#pragma unroll
+        for (int t = 0; t < TG; t++) {
+            const uint32_t slot = t_begin + grp * TG + t;
+#pragma unroll
+            for (int i = 0; i < NSBW; i++) {
+#pragma unroll
+                for (int u = 0; u < TileRegs<FMT, NSBW>::UNITS; u++)
+                    acc |= (uint32_t)(ring[t].w[i][u][0] | ring[t].w[i][u][1] | ring[t].w[i][u][2] | ring[t].w[i][u][3]);
+                acc |= ring[t].sc[i].x | ring[t].sc[i].y;
+            }
+            load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, slot + TG, slot + TG < t_end, p.n_sb, sb0, sb_lim, lane_c, lane_s);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    if (acc == 0x12345678u && p.y) p.y[threadIdx.x] = 1.f;  // practically never true; keeps the loads alive
 }
 
 // ---------------------------------------------------------------------------
@@ -249,82 +424,104 @@ __global__ __launch_bounds__(256) void dequant_kernel(OxbLayout L, const uint32_
     }
 }
 
+// silu(gate) * up (simd_float_ops.rs:217-236) for rows whose GEMV took several launches.
+__global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gu, uint32_t inter, float* __restrict__ out, uint32_t ldo) {
+    const uint32_t v = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= inter) return;
+    const float g = gu[(size_t)v * 2 * inter + i], u = gu[(size_t)v * 2 * inter + inter + i];
+    out[(size_t)v * ldo + i] = (g / (1.0f + expf(-g))) * u;
+}
+
 // ---------------------------------------------------------------------------
 // Host-side launchers.
 // ---------------------------------------------------------------------------
-size_t oxb_xq_bytes(uint32_t k, uint32_t batch) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
-    return (size_t)nblk_pad * 8 * NC * 16;
-}
-size_t oxb_cneg_bytes(uint32_t k, uint32_t batch) {
-    const uint32_t nblk_pad = ((k + 511u) / 512u) * 4u, NC = OXB_XQ_DIGITS * batch;
-    return (size_t)nblk_pad * NC * 16;
+struct GemvPlan {
+    uint32_t nsbw, S, tg, tpw, grid;
+};
+
+// Waves split K (one to three superblocks each, eight waves at most); about one workgroup per CU, each taking whole
+// groups of TG tiles.  TG is limited by the registers the ring needs; among the allowed values the one with the least
+// padded work wins, weighted by how well a ring of that depth hides the load latency.
+static bool plan_gemv(int fmt, const OxbGemvParams& p, uint32_t n_cus, GemvPlan* pl) {
+    if (p.sb_count == 0 || p.sb_count > OXB_GEMV_MAX_SB) return false;
+    pl->nsbw = (p.sb_count + 7u) / 8u;
+    pl->S = (p.sb_count + pl->nsbw - 1) / pl->nsbw;
+    const bool swiglu = p.epi == OXB_GEMV_SWIGLU;
+    if (swiglu && ((p.n_tiles & 1u) || (p.n_rows & 31u))) return false;  // whole gate and up tiles
+    const uint32_t units = swiglu ? p.n_tiles / 2 : p.n_tiles;
+    uint32_t tg_max = 1;
+    if (pl->nsbw == 1) tg_max = fmt == OXB_FMT_Q1 ? 4u : 3u;
+    else if (pl->nsbw == 2) tg_max = fmt == OXB_FMT_Q1 ? 2u : 1u;
+    const uint32_t per = (units + n_cus - 1) / n_cus;
+    static const uint32_t ring_weight[5] = {0, 130, 108, 103, 100};
+    uint32_t best = 0xFFFFFFFFu;
+    for (uint32_t t = tg_max; t >= 1; t--) {
+        const uint32_t padded = (per + t - 1) / t * t, cost = padded * ring_weight[t];
+        if (cost < best) best = cost, pl->tg = t, pl->tpw = padded;
+    }
+    pl->grid = (units + pl->tpw - 1) / pl->tpw;
+    if (swiglu) pl->tpw *= 2;
+    return true;
 }
 
-hipError_t oxb_launch_quant_x(int fmt, const float* d_x, uint32_t k, uint32_t batch, uint32_t* d_xq, int32_t* d_cneg,
-                              int32_t* d_xexp, hipStream_t st) {
-    const uint32_t n_sb = (k + 511u) / 512u, NC = OXB_XQ_DIGITS * batch;
-    const uint32_t gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
-    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
-    const dim3 grid(batch, n_groups < 16 ? n_groups : 16);
-    if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_Q1>, grid, dim3(OXB_QUANT_THREADS), 0, st, d_x, k, NC, gsb, n_groups, d_xq, d_cneg,
-                           d_xexp);
+template <int FMT, int NSBW, int TG>
+static hipError_t launch_gemv_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    const size_t shm = oxb_gemv_lds_bytes(pl.S, NSBW, TG);
+    if (p.pro == OXB_GEMV_PRO_RMSNORM)
+        hipLaunchKernelGGL((gemv_kernel<FMT, NSBW, TG, OXB_GEMV_PRO_RMSNORM>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
     else
-        hipLaunchKernelGGL(quant_x_kernel<OXB_FMT_TQ2>, grid, dim3(OXB_QUANT_THREADS), 0, st, d_x, k, NC, gsb, n_groups, d_xq, d_cneg,
-                           d_xexp);
+        hipLaunchKernelGGL((gemv_kernel<FMT, NSBW, TG, OXB_GEMV_PRO_F32>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
     return hipGetLastError();
 }
 
 template <int FMT, int NSBW, int TG>
-static hipError_t launch_gemv_t(OxbGemvParams p, uint32_t S, uint32_t grid, hipStream_t st) {
-    const size_t shm = 2 * (size_t)TG * S * p.NC * 64u;
-    hipLaunchKernelGGL((gemv_mfma_kernel<FMT, NSBW, TG>), dim3(grid), dim3(S * 64), shm, st, p);
+static hipError_t launch_floor_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    hipLaunchKernelGGL((stream_floor_kernel<FMT, NSBW, TG>), dim3(pl.grid), dim3(pl.S * 64), 0, st, p);
     return hipGetLastError();
 }
 
+#define OXB_GEMV_CASES(LAUNCH)                                                                                        \
+    OXB_CASE(OXB_FMT_Q1, 1, 1, LAUNCH) OXB_CASE(OXB_FMT_Q1, 1, 2, LAUNCH) OXB_CASE(OXB_FMT_Q1, 1, 3, LAUNCH)         \
+    OXB_CASE(OXB_FMT_Q1, 1, 4, LAUNCH) OXB_CASE(OXB_FMT_Q1, 2, 1, LAUNCH) OXB_CASE(OXB_FMT_Q1, 2, 2, LAUNCH)         \
+    OXB_CASE(OXB_FMT_Q1, 3, 1, LAUNCH) OXB_CASE(OXB_FMT_TQ2, 1, 1, LAUNCH) OXB_CASE(OXB_FMT_TQ2, 1, 2, LAUNCH)       \
+    OXB_CASE(OXB_FMT_TQ2, 1, 3, LAUNCH) OXB_CASE(OXB_FMT_TQ2, 2, 1, LAUNCH) OXB_CASE(OXB_FMT_TQ2, 3, 1, LAUNCH)
+#define OXB_CASE(F, N, T, LAUNCH) \
+    if (fmt == F && pl.nsbw == N && pl.tg == T) return LAUNCH<F, N, T>(p, pl, st);
+
+static bool check_gemv_args(const OxbGemvParams& p) {
+    if (p.nvec == 0 || p.nvec > OXB_GEMV_MAX_BATCH) return false;
+    if (p.codes_bytes >= 0x7FFFFFFFull || (uint64_t)p.k * 4 >= 0x7FFFFFFFull) return false;
+    if (p.pro != OXB_GEMV_PRO_F32 && p.pro != OXB_GEMV_PRO_RMSNORM) return false;
+    if (p.pro == OXB_GEMV_PRO_RMSNORM && !p.norm_w) return false;
+    if (p.epi == OXB_GEMV_RESIDUAL && !p.residual) return false;
+    if (p.epi == OXB_GEMV_SWIGLU && (p.sb_begin != 0 || p.sb_count != p.n_sb)) return false;  // needs the whole K
+    return p.epi >= OXB_GEMV_STORE && p.epi <= OXB_GEMV_SWIGLU;
+}
+
 hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {
-    // K slice per wave = one exponent group of the quantised input: NSBW superblocks; S <= 8 waves per workgroup.
-    const uint32_t nsbw = oxb_xq_gsb(p.n_sb);
-    p.n_groups = oxb_xq_groups(p.n_sb);
-    if (p.sb_count > 8 * nsbw || p.sb_begin % nsbw) return hipErrorInvalidValue;  // caller splits K into chunks of OXB_GEMV_MAX_SB superblocks
-    const uint32_t S = (p.sb_count + nsbw - 1) / nsbw;
     if (p.n_tiles == 0) return hipSuccess;
-    if (p.codes_bytes >= 0x7FFFFFFFull || p.xq_bytes >= 0x7FFFFFFFull) return hipErrorInvalidValue;
-    // Choose workgroups per CU (j), tiles in flight per wave (TG) and groups of TG tiles per
-    // workgroup so that the busiest CU computes the fewest tile slots; prefer more waves, then
-    // a deeper ring.  The partial-sum buffers 2 x TG x S x NC x 64 B stay <= 64 KiB.
-    const uint32_t units = fmt == OXB_FMT_Q1 ? 1u : 2u;
-    const uint32_t occ = nsbw == 1 ? 2u : 1u;  // what the register budget of the variant allows
-    uint32_t tg_max = nsbw == 1 ? 4u : (nsbw == 2 ? 4u / units : 1u);
-    while (tg_max > 1 && 2u * tg_max * S * p.NC * 64u > 64u * 1024u) tg_max--;
-    uint32_t best_cost = 0xFFFFFFFFu, tg = 1, grid = 1;
-    for (uint32_t j = occ; j >= 1; j--)
-        for (uint32_t t = tg_max; t >= 1; t--) {
-            const uint32_t tpw0 = (p.n_tiles + n_cus * j - 1) / (n_cus * j);
-            const uint32_t groups = (tpw0 + t - 1) / t, tpw = groups * t;
-            const uint32_t g = (p.n_tiles + tpw - 1) / tpw;
-            // tile slots of the busiest CU, weighted by how well a ring of t tiles hides the load latency
-            // (measured on 14 MB and 87 MB matrices: one tile in flight costs about 30 %, two 8 %, three 3 %)
-            static const uint32_t ring_weight[5] = {0, 130, 108, 103, 100};
-            const uint32_t cost = ((g + n_cus - 1) / n_cus) * tpw * ring_weight[t];
-            if (cost < best_cost || (cost == best_cost && g > grid)) {  // ties: more workgroups in flight
-                best_cost = cost;
-                tg = t;
-                grid = g;
-                p.groups = groups;
-            }
-        }
-#define OXB_CASE(F, N, T)                                                \
-    if (fmt == F && nsbw == N && tg == T) return launch_gemv_t<F, N, T>(p, S, grid, st);
-    OXB_CASE(OXB_FMT_Q1, 1, 1) OXB_CASE(OXB_FMT_Q1, 1, 2) OXB_CASE(OXB_FMT_Q1, 1, 3) OXB_CASE(OXB_FMT_Q1, 1, 4)
-    OXB_CASE(OXB_FMT_Q1, 2, 1) OXB_CASE(OXB_FMT_Q1, 2, 2) OXB_CASE(OXB_FMT_Q1, 2, 3) OXB_CASE(OXB_FMT_Q1, 2, 4)
-    OXB_CASE(OXB_FMT_Q1, 3, 1)
-    OXB_CASE(OXB_FMT_TQ2, 1, 1) OXB_CASE(OXB_FMT_TQ2, 1, 2) OXB_CASE(OXB_FMT_TQ2, 1, 3) OXB_CASE(OXB_FMT_TQ2, 1, 4)
-    OXB_CASE(OXB_FMT_TQ2, 2, 1) OXB_CASE(OXB_FMT_TQ2, 2, 2)
-    OXB_CASE(OXB_FMT_TQ2, 3, 1)
-#undef OXB_CASE
+    GemvPlan pl;
+    if (!check_gemv_args(p) || !plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
+    p.tpw = pl.tpw;
+    OXB_GEMV_CASES(launch_gemv_t)
     return hipErrorInvalidValue;
+}
+
+hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {
+    if (p.n_tiles == 0) return hipSuccess;
+    GemvPlan pl;
+    p.epi = OXB_GEMV_STORE;
+    if (!plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
+    p.tpw = pl.tpw;
+    OXB_GEMV_CASES(launch_floor_t)
+    return hipErrorInvalidValue;
+}
+#undef OXB_CASE
+
+hipError_t oxb_launch_swiglu(const float* d_gu, uint32_t inter, uint32_t nvec, float* d_out, uint32_t ldo, hipStream_t st) {
+    if (inter == 0 || nvec == 0) return hipSuccess;
+    hipLaunchKernelGGL(swiglu_kernel, dim3((inter + 255) / 256, nvec), dim3(256), 0, st, d_gu, inter, d_out, ldo);
+    return hipGetLastError();
 }
 
 hipError_t oxb_launch_dequant(const OxbLayout& L, const uint32_t* d_codes, const uint16_t* d_scales, float* d_out,

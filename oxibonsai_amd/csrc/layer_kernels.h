@@ -41,12 +41,6 @@ struct OxbAttnParams {
     float scale;                         // 1 / sqrt(hd)
 };
 
-// w_absmax = max |w[i]|, known when the norm weights are uploaded.
-hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
-                                    uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp,
-                                    float* d_normed_or_null, hipStream_t st);
-hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
-                                   int32_t* d_cneg, int32_t* d_xexp, hipStream_t st);
 // n_rows rows of n values -> one-byte codes [n_rows][n] and a scale per row (kv_mode: OXB_KV_I8 or OXB_KV_FP8_E4M3).
 hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n_rows, uint32_t n, uint8_t* d_codes, float* d_scales,
                                        hipStream_t st);
@@ -55,11 +49,9 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 #define OXB_ATTN_MAX_SPLITS 64        // slots the KV sequence is split over; slot s walks chunks s, s + n_splits, ...
 #define OXB_ATTN_PART_PAD 4           // floats after the hd outputs of a slot: maximum, sum, 2 unused (16-byte rows)
 // QK-norm, RoPE, KV store of the new position and split-KV attention (at most 16 q heads per kv head) into
-// p.part, then the merge of the slots fused with the quantiser of the O projection's input for sequences
-// b0 .. b0 + nb - 1 (nb <= 2); d_out_or_null also receives the fp32 attention output [batch][nq*hd].
+// p.part; then the merge of the slots into the fp32 attention output d_out [batch][nq * hd].
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
-hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
-                                         int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st);
+hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.
 #define OXB_ARGMAX_MAX_PARTS 256u
 hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st);

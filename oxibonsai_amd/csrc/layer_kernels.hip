@@ -4,126 +4,17 @@
 // cuda_full_layer/encode_ternary.rs:142-290, CPU twin crates/oxibonsai-model/src/block/types/forward.rs:92-408):
 //   RMSNorm -> QKV GEMV -> per-head QK-RMSNorm + half-split RoPE -> FP16 KV store ->
 //   attention over seq_len -> O GEMV + residual -> RMSNorm -> gate||up GEMV -> SiLU(g)*u -> down GEMV + residual.
-// Every kernel that produces a GEMV input writes the int8 digit planes directly
-// (quant_device.h) instead of an fp32 vector, so no separate quantisation pass runs.
+// RMSNorm, the residual adds and SwiGLU live in the GEMV kernel's prologue and epilogues (gemv_kernels.hip); here
+// are the attention kernels, the merge of their slots, the KV row quantiser and the greedy selection.
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
 #include <type_traits>
 
+#include "device_utils.h"
 #include "kv_quant_device.h"
 #include "layer_kernels.h"
-#include "quant_device.h"
-
-#define OXB_LAYER_THREADS 256
-
-__device__ __forceinline__ float block_sum(float v, float* red) {  // two barriers; red: blockDim.x / 64 floats
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    if ((threadIdx.x & 63u) == 0) red[threadIdx.x >> 6] = v;
-    __syncthreads();
-    float s = 0.f;
-    for (uint32_t i = 0; i < (blockDim.x >> 6); i++) s += red[i];
-    __syncthreads();
-    return s;
-}
-
-// ---------------------------------------------------------------------------
-// RMSNorm fused with the activation quantiser (rms_norm: crates/oxibonsai-kernels/src/
-// simd_float_ops.rs:204-215; GPU twin rmsnorm_weighted_v2, gpu_backend/cuda_kernels.rs:335-374).
-// out[i] = w[i] * x[i] * (1 / sqrt(mean(x^2) + eps)); the normalised vector lives only in LDS.
-// Grid (vectors of the pass, parts): every part repeats the reduction (the vector is a few KB in
-// L2) and quantises its share of the blocks.  x and w are fetched together, EPT elements per thread.
-// The quantiser's exponent does not need the exact maximum, only a bound: |out[i]| <= max|w| * sqrt(h)
-// because |x[i]| / rms <= sqrt(h).  With 54-bit fixed point the slack of sqrt(h) costs no mantissa bit
-// of any element within 2^22 / sqrt(h) of the largest one.
-// ---------------------------------------------------------------------------
-template <int FMT, int EPT>
-__global__ __launch_bounds__(OXB_LAYER_THREADS) void rmsnorm_quant_kernel(const float* __restrict__ x,
-                                                                           const float* __restrict__ w, float eps,
-                                                                           float w_absmax, uint32_t h, uint32_t NC,
-                                                                           uint32_t* __restrict__ xq,
-                                                                           int32_t* __restrict__ cneg,
-                                                                           int32_t* __restrict__ xexp,
-                                                                           float* __restrict__ normed_out) {
-    extern __shared__ float lds_x[];  // [h]
-    __shared__ float red[OXB_LAYER_THREADS / 64];
-    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
-    const uint32_t n = blockIdx.x, tid = threadIdx.x;
-    const float* xn = x + (size_t)n * h;
-    float xv[EPT], wv[EPT];
-#pragma unroll
-    for (int e = 0; e < EPT; e++) {
-        const uint32_t i = tid + (uint32_t)e * OXB_LAYER_THREADS;
-        xv[e] = i < h ? xn[i] : 0.f;
-        wv[e] = i < h ? w[i] : 0.f;
-    }
-    float ss = 0.f;
-#pragma unroll
-    for (int e = 0; e < EPT; e++) ss = fmaf(xv[e], xv[e], ss);
-    ss = block_sum(ss, red);
-    const float inv_rms = 1.0f / sqrtf(ss / (float)h + eps);
-#pragma unroll
-    for (int e = 0; e < EPT; e++) {
-        const uint32_t i = tid + (uint32_t)e * OXB_LAYER_THREADS;
-        const float v = wv[e] * xv[e] * inv_rms;
-        if (i < h) {
-            lds_x[i] = v;
-            if (normed_out && blockIdx.y == 0) normed_out[(size_t)n * h + i] = v;
-        }
-    }
-    // This workgroup's exponent groups.  Their exponent does not need the exact maximum, only a bound:
-    // |out[i]| <= max|w| * sqrt(h) because |x[i]| / rms <= sqrt(h); with 54-bit fixed point the slack costs no
-    // mantissa bit of any element within 2^22 / sqrt(h) of the largest one, and it saves a pass over the slice.
-    // A NaN or infinity anywhere in x or w shows up in the sum of squares or in the bound.
-    const uint32_t n_sb = (h + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
-    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
-    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
-    if (g0 >= g1) return;
-    const float bound = w_absmax * sqrtf((float)h);
-    const bool any_bad = oxb_not_finite(ss) || oxb_not_finite(bound);
-    for (uint32_t i = tid; i < g1 - g0; i += OXB_LAYER_THREADS) {
-        gstat[2 * i] = __float_as_uint(ss > 0.f && !any_bad ? bound : 0.f);
-        gstat[2 * i + 1] = any_bad ? 1u : 0u;
-    }
-    __syncthreads();  // publishes lds_x and gstat
-    quantise_groups<FMT>(lds_x, h, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
-}
-
-// ---------------------------------------------------------------------------
-// SwiGLU fused with the quantiser: act[i] = silu(gate[i]) * up[i], silu(x) = x / (1 + exp(-x))
-// (crates/oxibonsai-kernels/src/simd_float_ops.rs:217-236; GPU twin swiglu_fused, cuda_kernels.rs:394-401).
-// gu = [gate: inter | up: inter] per vector.  Grid (vectors, parts), 1024 threads.
-// ---------------------------------------------------------------------------
-#define OXB_SWIGLU_THREADS 256
-template <int FMT>
-__global__ __launch_bounds__(OXB_SWIGLU_THREADS) void swiglu_quant_kernel(const float* __restrict__ gu, uint32_t inter,
-                                                                           uint32_t NC, uint32_t* __restrict__ xq,
-                                                                           int32_t* __restrict__ cneg,
-                                                                           int32_t* __restrict__ xexp) {
-    extern __shared__ float lds_x[];  // [inter]; a workgroup fills only the span of its exponent groups
-    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
-    const uint32_t n = blockIdx.x, tid = threadIdx.x;
-    const uint32_t n_sb = (inter + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
-    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
-    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
-    if (g0 >= g1) return;
-    const uint32_t e0 = g0 * gsb * 512u, e1 = g1 * gsb * 512u < inter ? g1 * gsb * 512u : inter;
-    const float* g = gu + (size_t)n * 2 * inter;
-    const float* u = g + inter;
-    for (uint32_t i = e0 + tid * 4; i < e1; i += OXB_SWIGLU_THREADS * 4) {  // inter % 128 == 0
-        const float4 g4 = *reinterpret_cast<const float4*>(g + i), u4 = *reinterpret_cast<const float4*>(u + i);
-        float4 a;
-        a.x = (g4.x / (1.0f + expf(-g4.x))) * u4.x;
-        a.y = (g4.y / (1.0f + expf(-g4.y))) * u4.y;
-        a.z = (g4.z / (1.0f + expf(-g4.z))) * u4.z;
-        a.w = (g4.w / (1.0f + expf(-g4.w))) * u4.w;
-        *reinterpret_cast<float4*>(lds_x + i) = a;
-    }
-    gstat_scan(lds_x, inter, gsb, g0, g1, gstat);  // its first barrier publishes lds_x
-    quantise_groups<FMT>(lds_x, inter, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
-}
 
 // ---------------------------------------------------------------------------
 // Per-head QK-RMSNorm + half-split RoPE + KV store (fp16, or quantised rows: kv_quant_device.h)
@@ -686,30 +577,20 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     }
 }
 
-// Merge the slot results of the q heads and quantise the attention output for the O projection.  Grid
-// (vectors of the pass, parts), 256 threads: a workgroup takes whole exponent groups of the output vector
-// (nq * hd values), i.e. a run of dimensions that it merges (softmax weights of the slots per head: one wave
-// per head, one slot per lane; then the weighted sum, four outputs per thread) and quantises on its own.
-// Sequence b0 + blockIdx.x becomes vector blockIdx.x of the quantised pass.
-template <int FMT>
-__global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p, uint32_t b0, uint32_t NC,
-                                                                  uint32_t* __restrict__ xq, int32_t* __restrict__ cneg,
-                                                                  int32_t* __restrict__ xexp,
-                                                                  float* __restrict__ out_or_null) {
-    extern __shared__ float sm[];  // [span] outputs of this workgroup | [heads here][64] slot weights | [heads here] 1 / sum
-    __shared__ uint32_t gstat[2 * OXB_XQ_MAX_GROUPS];
-    const uint32_t n = blockIdx.x, b = b0 + n, tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
-    const uint32_t n_sb = (qd + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
-    const uint32_t per = (n_groups + gridDim.y - 1) / gridDim.y, g0 = blockIdx.y * per;
-    const uint32_t g1 = g0 + per < n_groups ? g0 + per : n_groups;
-    if (g0 >= g1) return;
-    const uint32_t e0 = g0 * gsb * 512u, e1 = g1 * gsb * 512u < qd ? g1 * gsb * 512u : qd;
-    const uint32_t h_first = e0 / hd, h_last = (e1 - 1) / hd, nh = h_last - h_first + 1;  // heads touched by the span
+// Merge the slot results of the q heads into the attention output [batch][nq * hd] (fp32), the input of the O
+// projection.  Grid (sequences, parts), 256 threads: a workgroup takes a run of whole heads; per head one wave works out
+// the softmax weights of the slots (one slot per lane), then every thread adds the weighted slot outputs of four
+// dimensions in ascending slot order.
+__global__ __launch_bounds__(256) void attn_combine_kernel(OxbAttnParams p, uint32_t heads_per, float* __restrict__ out) {
+    extern __shared__ float sm[];  // [heads here][64] slot weights | [heads here] 1 / sum
+    const uint32_t b = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
+    const uint32_t h_first = blockIdx.y * heads_per;
+    if (h_first >= p.nq) return;
+    const uint32_t nh = (h_first + heads_per <= p.nq ? heads_per : p.nq - h_first);
+    const uint32_t e0 = h_first * hd, e1 = e0 + nh * hd;
     const uint32_t stride = hd + OXB_ATTN_PART_PAD;
-    const uint32_t span_pad = gsb * 512u * per;
-    float* o = sm;  // o[e - e0]
-    float* wts = sm + span_pad;
-    float* inv_l = wts + nh * 64;
+    float* wts = sm;
+    float* inv_l = wts + heads_per * 64;
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
     const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
@@ -768,13 +649,8 @@ __global__ __launch_bounds__(256) void attn_combine_quant_kernel(OxbAttnParams p
         }
         const float il = inv_l[hh];
         acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
-        *reinterpret_cast<float4*>(o + (e - e0)) = acc;
-        if (out_or_null) *reinterpret_cast<float4*>(out_or_null + (size_t)b * qd + e) = acc;
+        *reinterpret_cast<float4*>(out + (size_t)b * qd + e) = acc;
     }
-    if (!xq) return;  // merge only: the caller consumes the fp32 output
-    // the quantiser indexes the vector from its start: hand it the span shifted back by e0
-    gstat_scan(o - e0, qd, gsb, g0, g1, gstat);  // its first barrier publishes the outputs
-    quantise_groups<FMT>(o - e0, qd, NC, n, gsb, n_groups, g0, g1, gstat, xq, cneg, xexp);
 }
 
 // ---------------------------------------------------------------------------
@@ -822,47 +698,6 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
 // ---------------------------------------------------------------------------
 // Launchers
 // ---------------------------------------------------------------------------
-template <int FMT>
-static hipError_t launch_rmsnorm_fmt(const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
-                                     uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp, float* d_normed,
-                                     hipStream_t st) {
-    const size_t shm = (size_t)h * sizeof(float);
-    const uint32_t n_groups = oxb_xq_groups((h + 511u) / 512u);
-    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
-    const dim3 grid(nb, n_groups < 8 ? n_groups : 8), block(OXB_LAYER_THREADS);
-    const uint32_t ept = (h + OXB_LAYER_THREADS - 1) / OXB_LAYER_THREADS;
-#define OXB_RMS_CASE(E)                                                                                              \
-    if (ept <= E) {                                                                                                  \
-        hipLaunchKernelGGL((rmsnorm_quant_kernel<FMT, E>), grid, block, shm, st, d_x, d_w, eps, w_absmax, h, 8 * nb, \
-                           d_xq, d_cneg, d_xexp, d_normed);                                                          \
-        return hipGetLastError();                                                                                    \
-    }
-    OXB_RMS_CASE(4) OXB_RMS_CASE(8) OXB_RMS_CASE(16) OXB_RMS_CASE(32) OXB_RMS_CASE(64)
-#undef OXB_RMS_CASE
-    return hipErrorInvalidValue;  // h > 16384
-}
-
-hipError_t oxb_launch_rmsnorm_quant(int fmt, const float* d_x, const float* d_w, float eps, float w_absmax, uint32_t h,
-                                    uint32_t nb, uint32_t* d_xq, int32_t* d_cneg, int32_t* d_xexp,
-                                    float* d_normed_or_null, hipStream_t st) {
-    return fmt == OXB_FMT_Q1
-               ? launch_rmsnorm_fmt<OXB_FMT_Q1>(d_x, d_w, eps, w_absmax, h, nb, d_xq, d_cneg, d_xexp, d_normed_or_null, st)
-               : launch_rmsnorm_fmt<OXB_FMT_TQ2>(d_x, d_w, eps, w_absmax, h, nb, d_xq, d_cneg, d_xexp, d_normed_or_null, st);
-}
-
-hipError_t oxb_launch_swiglu_quant(int fmt, const float* d_gu, uint32_t inter, uint32_t nb, uint32_t* d_xq,
-                                   int32_t* d_cneg, int32_t* d_xexp, hipStream_t st) {
-    const size_t shm = (size_t)inter * sizeof(float);
-    const uint32_t n_groups = oxb_xq_groups((inter + 511u) / 512u);
-    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
-    const dim3 grid(nb, n_groups < 16 ? n_groups : 16), block(OXB_SWIGLU_THREADS);
-    if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_Q1>, grid, block, shm, st, d_gu, inter, 8 * nb, d_xq, d_cneg, d_xexp);
-    else
-        hipLaunchKernelGGL(swiglu_quant_kernel<OXB_FMT_TQ2>, grid, block, shm, st, d_gu, inter, 8 * nb, d_xq, d_cneg, d_xexp);
-    return hipGetLastError();
-}
-
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st) {
     if (p.hd > 256 || p.kv_mode > OXB_KV_FP8_E4M3 || (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale))) return hipErrorInvalidValue;
     const uint32_t per_wg = 4 * OXB_QK_HEADS_PER_WAVE;
@@ -906,25 +741,12 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
     return hipGetLastError();
 }
 
-hipError_t oxb_launch_attn_combine_quant(int fmt, const OxbAttnParams& p, uint32_t b0, uint32_t nb, uint32_t* d_xq,
-                                         int32_t* d_cneg, int32_t* d_xexp, float* d_out_or_null, hipStream_t st) {
-    const uint32_t qd = p.nq * p.hd;
-    // with d_xq == nullptr the kernel only merges (any nb) and d_out_or_null must be given
-    if (nb == 0 || (d_xq && nb > 2) || (!d_xq && !d_out_or_null) || (qd % OXB_QK) != 0 || p.n_splits > OXB_ATTN_MAX_SPLITS)
-        return hipErrorInvalidValue;
-    const uint32_t n_sb = (qd + 511u) / 512u, gsb = oxb_xq_gsb(n_sb), n_groups = oxb_xq_groups(n_sb);
-    if (n_groups > OXB_XQ_MAX_GROUPS) return hipErrorInvalidValue;
-    const uint32_t parts = n_groups < 16 ? n_groups : 16, per = (n_groups + parts - 1) / parts;
-    const uint32_t span = gsb * 512u * per, heads = span / p.hd + 2;
-    const size_t shm = ((size_t)span + heads * 65) * sizeof(float);
-    if (shm > 60 * 1024) return hipErrorInvalidValue;
-    const uint32_t NC = OXB_XQ_DIGITS * nb;
-    if (fmt == OXB_FMT_Q1)
-        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_Q1>, dim3(nb, parts), dim3(256), shm, st, p, b0, NC, d_xq, d_cneg, d_xexp,
-                           d_out_or_null);
-    else
-        hipLaunchKernelGGL(attn_combine_quant_kernel<OXB_FMT_TQ2>, dim3(nb, parts), dim3(256), shm, st, p, b0, NC, d_xq, d_cneg, d_xexp,
-                           d_out_or_null);
+hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st) {
+    if (batch == 0 || !d_out || (p.hd & 3u) || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
+    // about 16 workgroups per sequence, whole heads each
+    const uint32_t heads_per = (p.nq + 15u) / 16u, parts = (p.nq + heads_per - 1) / heads_per;
+    const size_t shm = (size_t)heads_per * 65 * sizeof(float);
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(batch, parts), dim3(256), shm, st, p, heads_per, d_out);
     return hipGetLastError();
 }
 

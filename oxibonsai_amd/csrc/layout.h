@@ -24,8 +24,9 @@
 //                    i%4 == 3: field = value as 2-bit two's complement (3,0,1)
 //     The reserved reference code 0b11 decodes to 0 like 0b01 and is stored as 0.
 //
-//  scales (both)   : unit (tile, sb) = 4 row-groups x 16 f16 = 128 B.
-//     element [rg][q][v] = f16 scale of block 4*sb+q, row 16*tile + 4*rg + v.
+//  scales (both)   : unit (tile, sb) = 16 rows x 4 f16 = 128 B.
+//     element [r][q] = f16 scale of block 4*sb+q, row 16*tile + r: the four scales a lane needs for one
+//     superblock of its row are one 8-byte load.
 //
 // Rows are padded to a multiple of 16 and blocks to a multiple of 4 with zero
 // scales and zero codes; padded entries contribute exactly 0.
@@ -85,7 +86,7 @@ OXB_HD uint64_t oxb_tq2_dword_index(const OxbLayout& L, uint32_t row, uint32_t b
 // f16 index (within the scales section) of the scale of block `blk`, row `row`.
 OXB_HD uint64_t oxb_scale_index(const OxbLayout& L, uint32_t row, uint32_t blk) {
     uint32_t tile = row >> 4, r = row & 15u, sb = blk >> 2, q = blk & 3u;
-    return ((uint64_t)tile * L.n_sb + sb) * 64u + (r >> 2) * 16u + q * 4u + (r & 3u);
+    return ((uint64_t)tile * L.n_sb + sb) * 64u + r * 4u + q;
 }
 
 // TQ2 field encoding: reference code (00 -> -1, 01 -> 0, 10 -> +1, 11 -> 0) to

@@ -31,18 +31,12 @@
 
 namespace oxb {
 
-struct XqBuf {  // quantised activation of one GEMV pass (<= OXB_GEMV_MAX_BATCH vectors)
-    uint32_t* xq = nullptr;
-    int32_t* cneg = nullptr;
-    int32_t* xexp = nullptr;
-};
-
 struct Model {
     oxb_model_desc d;
     std::vector<oxb_layer_ids> layers;
     // activations
     float *hidden = nullptr, *qkv = nullptr, *attn_part = nullptr, *attn_out = nullptr,
-          *gu = nullptr, *logits = nullptr;
+          *gu = nullptr, *act = nullptr, *logits = nullptr;  // gu: [batch][2 inter] gate || up sums, act: [batch][inter] SwiGLU output
     uint32_t *tokens = nullptr, *pos = nullptr;
     void* argmax_ws = nullptr;
     // KV cache: rows of hd fp16 values or one-byte codes, a quantised cache also one f32 scale per row.  Contiguous:
@@ -58,8 +52,6 @@ struct Model {
     uint32_t* d_table = nullptr;
     bool table_dirty = false;
     float *cos_t = nullptr, *sin_t = nullptr;
-    void* xq_mem = nullptr;
-    XqBuf xq;
     uint32_t chunk = 0, n_splits = 0;
     // graph
     hipGraphExec_t graph_exec = nullptr;
@@ -147,11 +139,6 @@ static const float* vec_ptr(uint64_t id, uint32_t n, const char* what, int* rc) 
     return it->second.d;
 }
 
-static float vec_absmax(uint64_t id) {
-    auto it = g_rt.vectors.find(id);
-    return it == g_rt.vectors.end() ? 0.f : it->second.absmax;
-}
-
 static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, const char* what, int* rc) {
     const Weight* w = find_weight(id);
     if (!w) {
@@ -166,37 +153,6 @@ static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, 
     return w;
 }
 
-// GEMV on an already quantised input.
-static int gemv_xq(const Weight& w, const XqBuf& xb, uint32_t nb, float* d_y, uint32_t ldy, int mode,
-                   const float* d_res) {
-    OxbGemvParams p;
-    memset(&p, 0, sizeof p);
-    p.codes = w.d_codes;
-    p.scales = w.d_scales;
-    p.xq = xb.xq;
-    p.cneg = xb.cneg;
-    p.xexp = xb.xexp;
-    p.y = d_y;
-    p.residual = d_res;
-    p.n_rows = w.L.n_rows;
-    p.n_tiles = w.L.n_tiles;
-    p.n_sb = w.L.n_sb;
-    p.NC = 8 * nb;
-    p.ldy = ldy;
-    p.codes_bytes = (uint32_t)w.L.codes_bytes;
-    p.scales_bytes = (uint32_t)w.L.scales_bytes;
-    p.xq_bytes = (uint32_t)oxb_xq_bytes(w.L.k, nb);
-    p.cneg_bytes = (uint32_t)oxb_cneg_bytes(w.L.k, nb);
-    for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
-        p.sb_begin = sb;
-        p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
-        p.mode = sb == 0 ? mode : OXB_GEMV_ACCUM;
-        hipError_t e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
-        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
-    }
-    return OXB_HIP_OK;
-}
-
 #define OXB_TRY_HIP(expr, what)                               \
     do {                                                      \
         hipError_t e_ = (expr);                               \
@@ -208,20 +164,25 @@ static int gemv_xq(const Weight& w, const XqBuf& xb, uint32_t nb, float* d_y, ui
         if (rc_) return rc_;     \
     } while (0)
 
-// The FFN half of a layer on vectors [b0, b0+nb): O-proj + residual, RMSNorm, gate||up, SwiGLU, down + residual.
-static int encode_ffn(int fmt, const XqBuf& xb, float* hidden, const float* attn_out, const float* ffn_norm,
-                      float ffn_norm_absmax, float eps,
-                      const Weight& o, const Weight& gate_up, const Weight& down, float* gu, uint32_t h,
-                      uint32_t inter, uint32_t attn_k, uint32_t nb) {
-    hipStream_t st = g_rt.stream;
-    if (attn_out)  // null: xb already holds the quantised attention output
-        OXB_TRY_HIP(oxb_launch_quant_x(fmt, attn_out, attn_k, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: quant_x");
-    OXB_TRY(gemv_xq(o, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
-    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(fmt, hidden, ffn_norm, eps, ffn_norm_absmax, h, nb, xb.xq, xb.cneg, xb.xexp, nullptr, st),
-                "kernel launch failed: rmsnorm_quant");
-    OXB_TRY(gemv_xq(gate_up, xb, nb, gu, 2 * inter, OXB_GEMV_STORE, nullptr));
-    OXB_TRY_HIP(oxb_launch_swiglu_quant(fmt, gu, inter, nb, xb.xq, xb.cneg, xb.xexp, st), "kernel launch failed: swiglu_quant");
-    OXB_TRY(gemv_xq(down, xb, nb, hidden, h, OXB_GEMV_RESIDUAL, hidden));
+// gate || up with SwiGLU behind it: one launch when K fits one GEMV launch (the epilogue needs whole row sums),
+// else the plain product into gu and a separate SwiGLU.
+static int gate_up_swiglu(const Weight& gate_up, const float* x, uint32_t ldx, uint32_t nb, const float* norm_w, float eps,
+                          float* gu, float* act, uint32_t inter) {
+    if (gate_up.L.n_sb <= OXB_GEMV_MAX_SB)
+        return gemv_launch(gate_up, x, ldx, nb, act, inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_SWIGLU, nullptr);
+    OXB_TRY(gemv_launch(gate_up, x, ldx, nb, gu, 2 * inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_STORE, nullptr));
+    OXB_TRY_HIP(oxb_launch_swiglu(gu, inter, nb, act, inter, g_rt.stream), "kernel launch failed: swiglu");
+    return OXB_HIP_OK;
+}
+
+// The FFN half of a layer on nb <= OXB_GEMV_MAX_BATCH vectors: O-proj + residual, RMSNorm -> gate || up -> SwiGLU,
+// down + residual: three launches (RMSNorm rides in the gate || up kernel's prologue, SwiGLU in its epilogue).
+static int encode_ffn(float* hidden, const float* attn_out, const float* ffn_norm, float eps, const Weight& o,
+                      const Weight& gate_up, const Weight& down, float* gu, float* act, uint32_t h, uint32_t inter,
+                      uint32_t attn_k, uint32_t nb) {
+    OXB_TRY(gemv_launch(o, attn_out, attn_k, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden));
+    OXB_TRY(gate_up_swiglu(gate_up, hidden, h, nb, ffn_norm, eps, gu, act, inter));
+    OXB_TRY(gemv_launch(down, act, inter, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden));
     return OXB_HIP_OK;
 }
 
@@ -314,8 +275,8 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
 
 // Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
 // matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
-// the weights once per two sequences.
-#define OXB_DECODE_GEMM_MIN_BATCH 3
+// the weights once per four sequences.
+#define OXB_DECODE_GEMM_MIN_BATCH (OXB_GEMV_MAX_BATCH + 1)
 
 static int encode_decode_step_gemm(Model& m) {
     const oxb_model_desc& d = m.d;
@@ -339,8 +300,7 @@ static int encode_decode_step_gemm(Model& m) {
             OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap, m.attn_out));
         } else {
             OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
-            OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, 0, B, nullptr, nullptr, nullptr, m.attn_out, st),
-                        "kernel launch failed: attn_combine");
+            OXB_TRY_HIP(oxb_launch_attn_combine(ap, B, m.attn_out, st), "kernel launch failed: attn_combine");
         }
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
         // SwiGLU in the epilogue of the gate || up product
@@ -373,23 +333,23 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
         const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
         if (rc) return rc;
-        // attention input: RMSNorm -> QKV, two sequences per pass over the weights
+        // attention input: RMSNorm -> QKV in one launch per pass of OXB_GEMV_MAX_BATCH sequences
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, attn_norm, d.eps, vec_absmax(ly.attn_norm), d.h, nb, m.xq.xq,
-                                                 m.xq.cneg, m.xq.xexp, nullptr, st),
-                        "kernel launch failed: rmsnorm_quant");
-            OXB_TRY(gemv_xq(*wqkv, m.xq, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows, OXB_GEMV_STORE, nullptr));
+            OXB_TRY(gemv_launch(*wqkv, m.hidden + (size_t)b0 * d.h, d.h, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows,
+                                OXB_GEMV_PRO_RMSNORM, attn_norm, d.eps, OXB_GEMV_STORE, nullptr));
         }
         OxbAttnParams ap;
-        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
+        if (m.n_splits == 1) {  // one slot per sequence: the attention kernel finishes its output itself
+            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap, m.attn_out));
+        } else {
+            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
+            OXB_TRY_HIP(oxb_launch_attn_combine(ap, d.batch, m.attn_out, st), "kernel launch failed: attn_combine");
+        }
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY_HIP(oxb_launch_attn_combine_quant(d.fmt, ap, b0, nb, m.xq.xq, m.xq.cneg, m.xq.xexp, nullptr, st),
-                        "kernel launch failed: attn_combine_quant");
-            OXB_TRY(encode_ffn(d.fmt, m.xq, m.hidden + (size_t)b0 * d.h, nullptr, ffn_norm,
-                               vec_absmax(ly.ffn_norm), d.eps, *wo,
-                               *wgu, *wdn, m.gu + (size_t)b0 * 2 * d.inter, d.h, d.inter, qd, nb));
+            OXB_TRY(encode_ffn(m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo, *wgu, *wdn,
+                               m.gu + (size_t)b0 * 2 * d.inter, m.act + (size_t)b0 * d.inter, d.h, d.inter, qd, nb));
         }
     }
     if (with_lm_head) {
@@ -398,10 +358,8 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         if (rc) return rc;
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, m.hidden + (size_t)b0 * d.h, final_norm, d.eps, vec_absmax(d.final_norm), d.h, nb, m.xq.xq,
-                                                 m.xq.cneg, m.xq.xexp, nullptr, st),
-                        "kernel launch failed: rmsnorm_quant");
-            OXB_TRY(gemv_xq(*lm, m.xq, nb, m.logits + (size_t)b0 * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
+            OXB_TRY(gemv_launch(*lm, m.hidden + (size_t)b0 * d.h, d.h, nb, m.logits + (size_t)b0 * d.vocab, d.vocab,
+                                OXB_GEMV_PRO_RMSNORM, final_norm, d.eps, OXB_GEMV_STORE, nullptr));
         }
         OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, m.argmax_ws, st), "kernel launch failed: argmax");
     }
@@ -513,10 +471,8 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
     if (rc) return rc;
     float* last = m.hidden + (size_t)seq * d.h;
     OXB_TRY_HIP(hipMemcpyAsync(last, m.pf_hidden + (size_t)(M - 1) * d.h, (size_t)d.h * 4, hipMemcpyDeviceToDevice, st), "last row copy");
-    OXB_TRY_HIP(oxb_launch_rmsnorm_quant(d.fmt, last, final_norm, d.eps, vec_absmax(d.final_norm), d.h, 1, m.xq.xq, m.xq.cneg, m.xq.xexp,
-                                         nullptr, st),
-                "kernel launch failed: rmsnorm_quant");
-    OXB_TRY(gemv_xq(*lm, m.xq, 1, m.logits + (size_t)seq * d.vocab, d.vocab, OXB_GEMV_STORE, nullptr));
+    OXB_TRY(gemv_launch(*lm, last, d.h, 1, m.logits + (size_t)seq * d.vocab, d.vocab, OXB_GEMV_PRO_RMSNORM, final_norm, d.eps,
+                        OXB_GEMV_STORE, nullptr));
     OXB_TRY_HIP(oxb_launch_argmax(m.logits + (size_t)seq * d.vocab, d.vocab, 1, m.tokens + seq, m.argmax_ws, st), "kernel launch failed: argmax");
     return OXB_HIP_OK;
 }
@@ -674,23 +630,17 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     m.n_splits = attn_slots(m, OXB_KV_F16);
     const uint32_t max_slots = attn_slots(m, OXB_KV_I8);  // what any cache type may ask for: sizes the slot results
     const size_t B = d.batch;
-    uint32_t kmax = d.h > d.inter ? d.h : d.inter;
-    if (qd > kmax) kmax = qd;
-    const size_t xq_b = oxb_xq_bytes(kmax, OXB_GEMV_MAX_BATCH), cn_b = oxb_cneg_bytes(kmax, OXB_GEMV_MAX_BATCH);
     if ((rc = dev_alloc(m, (void**)&m.hidden, B * d.h * 4)) || (rc = dev_alloc(m, (void**)&m.qkv, B * qkv_rows * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * max_slots * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.act, B * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
         (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
-        (rc = dev_alloc(m, &m.xq_mem, xq_b + cn_b + OXB_XEXP_BYTES))) {
+        (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4))) {
         free_model(m);
         return rc;
     }
-    m.xq.xq = (uint32_t*)m.xq_mem;
-    m.xq.cneg = (int32_t*)((uint8_t*)m.xq_mem + xq_b);
-    m.xq.xexp = (int32_t*)((uint8_t*)m.xq_mem + xq_b + cn_b);
     // RoPE table, computed as RopeTable::new does (crates/oxibonsai-model/src/layers/rope.rs:27-48): all in f32.
     {
         const size_t half = d.hd / 2;
@@ -1049,28 +999,18 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     const Weight* wgu = mat_ptr(gate_up_id, fmt, 2 * inter, h, "gate_up", &rc);
     const Weight* wdn = mat_ptr(down_id, fmt, h, inter, "down", &rc);
     if (rc) return rc;
-    uint32_t kmax = h > inter ? h : inter;
-    if (attn_k > kmax) kmax = attn_k;
-    const size_t xq_b = oxb_xq_bytes(kmax, 1), cn_b = oxb_cneg_bytes(kmax, 1);
-    OXB_TRY(g_rt.ws_xq.ensure(xq_b + cn_b + OXB_XEXP_BYTES));
     OXB_TRY(g_rt.ws_x.ensure(((size_t)h * 2 + attn_k) * 4));
-    OXB_TRY(g_rt.ws_y.ensure((size_t)2 * inter * 4));
-    XqBuf xb;
-    xb.xq = (uint32_t*)g_rt.ws_xq.ptr;
-    xb.cneg = (int32_t*)((uint8_t*)g_rt.ws_xq.ptr + xq_b);
-    xb.xexp = (int32_t*)((uint8_t*)g_rt.ws_xq.ptr + xq_b + cn_b);
+    OXB_TRY(g_rt.ws_y.ensure((size_t)3 * inter * 4));
     float* d_hidden = (float*)g_rt.ws_x.ptr;
     float* d_norm = d_hidden + h;
     float* d_attn = d_norm + h;
+    float* d_gu = (float*)g_rt.ws_y.ptr;
+    float* d_act = d_gu + 2 * (size_t)inter;
     hipStream_t st = g_rt.stream;
     OXB_TRY_HIP(hipMemcpyAsync(d_hidden, hidden, (size_t)h * 4, hipMemcpyHostToDevice, st), "hidden upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_norm, norm_w, (size_t)h * 4, hipMemcpyHostToDevice, st), "norm upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_attn, attn_out, (size_t)attn_k * 4, hipMemcpyHostToDevice, st), "attn_out upload");
-    float nw_absmax = 0.f;
-    for (uint32_t i = 0; i < h; i++) nw_absmax = fmaxf(nw_absmax, fabsf(norm_w[i]));  // NaN-free maximum; a NaN weight yields NaN outputs
-    for (uint32_t i = 0; i < h; i++)
-        if (norm_w[i] != norm_w[i]) nw_absmax = norm_w[i];
-    OXB_TRY(encode_ffn(fmt, xb, d_hidden, d_attn, d_norm, nw_absmax, eps, *wo, *wgu, *wdn, (float*)g_rt.ws_y.ptr, h, inter, attn_k, 1));
+    OXB_TRY(encode_ffn(d_hidden, d_attn, d_norm, eps, *wo, *wgu, *wdn, d_gu, d_act, h, inter, attn_k, 1));
     OXB_TRY_HIP(hipMemcpyAsync(hidden, d_hidden, (size_t)h * 4, hipMemcpyDeviceToHost, st), "hidden download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));
@@ -1272,8 +1212,8 @@ int oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, c
     OXB_TRY_HIP(hipMemcpyAsync(d_logits, logits, lb, hipMemcpyHostToDevice, st), "logits upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_rng, rng_state, (size_t)batch * 8, hipMemcpyHostToDevice, st), "rng state upload");
     if (params->temperature < 1e-6f) {
-        OXB_TRY(g_rt.ws_xq.ensure((size_t)batch * OXB_ARGMAX_MAX_PARTS * 8));
-        OXB_TRY_HIP(oxb_launch_argmax(d_logits, vocab, batch, d_tok, g_rt.ws_xq.ptr, st), "kernel launch failed: argmax");
+        OXB_TRY(g_rt.ws_aux.ensure((size_t)batch * OXB_ARGMAX_MAX_PARTS * 8));
+        OXB_TRY_HIP(oxb_launch_argmax(d_logits, vocab, batch, d_tok, g_rt.ws_aux.ptr, st), "kernel launch failed: argmax");
     } else {
         OXB_TRY_HIP(oxb_launch_sample(d_logits, vocab, batch, params->temperature, params->top_k, params->top_p, d_rng, d_tok, d_ws, st),
                     "kernel launch failed: sample");

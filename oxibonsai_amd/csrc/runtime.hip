@@ -127,44 +127,48 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
     return OXB_HIP_OK;
 }
 
-// x (device, [batch][k]) -> y (device, [batch][ldy]) through quantiser + GEMV, OXB_GEMV_MAX_BATCH vectors per pass.
+// One GEMV over resident weights, any K: launches of at most OXB_GEMV_MAX_SB superblocks, the first with the wanted
+// epilogue, the rest accumulating.  nvec <= OXB_GEMV_MAX_BATCH vectors share each pass over the weights.
+int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, float* d_y, uint32_t ldy, int pro,
+                const float* d_norm_w, float eps, int epi, const float* d_residual) {
+    OxbGemvParams p;
+    memset(&p, 0, sizeof p);
+    p.codes = w.d_codes;
+    p.scales = w.d_scales;
+    p.x = d_x;
+    p.norm_w = d_norm_w;
+    p.eps = eps;
+    p.y = d_y;
+    p.residual = d_residual;
+    p.n_rows = w.L.n_rows;
+    p.n_tiles = w.L.n_tiles;
+    p.n_sb = w.L.n_sb;
+    p.k = w.L.k;
+    p.nvec = nvec;
+    p.ldx = ldx;
+    p.ldy = ldy;
+    p.codes_bytes = (uint32_t)w.L.codes_bytes;
+    p.scales_bytes = (uint32_t)w.L.scales_bytes;
+    p.pro = pro;
+    for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
+        p.sb_begin = sb;
+        p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
+        p.epi = sb == 0 ? epi : OXB_GEMV_ACCUM;
+        hipError_t e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
+        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
+    }
+    return OXB_HIP_OK;
+}
+
+// x (device, [batch][k]) -> y (device, [batch][ldy]), OXB_GEMV_MAX_BATCH vectors per pass over the weights.
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual) {
     const uint32_t k = w.L.k;
     for (uint32_t b0 = 0; b0 < batch; b0 += OXB_GEMV_MAX_BATCH) {
         const uint32_t nb = (batch - b0) < OXB_GEMV_MAX_BATCH ? (batch - b0) : OXB_GEMV_MAX_BATCH;
-        int rc;
-        if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-        if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-        if ((rc = g_rt.ws_xexp.ensure(OXB_XEXP_BYTES))) return rc;
-        hipError_t e = oxb_launch_quant_x((int)w.L.fmt, d_x + (size_t)b0 * k, k, nb, (uint32_t*)g_rt.ws_xq.ptr,
-                                          (int32_t*)g_rt.ws_cneg.ptr, (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
-        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: quant_x");
-        OxbGemvParams p;
-        memset(&p, 0, sizeof p);
-        p.codes = w.d_codes;
-        p.scales = w.d_scales;
-        p.xq = (const uint32_t*)g_rt.ws_xq.ptr;
-        p.cneg = (const int32_t*)g_rt.ws_cneg.ptr;
-        p.xexp = (const int32_t*)g_rt.ws_xexp.ptr;
-        p.y = d_y + (size_t)b0 * ldy;
-        p.residual = d_residual ? d_residual + (size_t)b0 * ldy : nullptr;
-        p.n_rows = w.L.n_rows;
-        p.n_tiles = w.L.n_tiles;
-        p.n_sb = w.L.n_sb;
-        p.NC = 8 * nb;
-        p.ldy = ldy;
-        p.codes_bytes = (uint32_t)w.L.codes_bytes;
-        p.scales_bytes = (uint32_t)w.L.scales_bytes;
-        p.xq_bytes = (uint32_t)oxb_xq_bytes(k, nb);
-        p.cneg_bytes = (uint32_t)oxb_cneg_bytes(k, nb);
-        for (uint32_t sb = 0; sb < w.L.n_sb; sb += OXB_GEMV_MAX_SB) {
-            p.sb_begin = sb;
-            p.sb_count = (w.L.n_sb - sb) < OXB_GEMV_MAX_SB ? (w.L.n_sb - sb) : OXB_GEMV_MAX_SB;
-            p.mode = sb == 0 ? mode : OXB_GEMV_ACCUM;
-            e = oxb_launch_gemv((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
-            if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv");
-        }
+        int rc = gemv_launch(w, d_x + (size_t)b0 * k, k, nb, d_y + (size_t)b0 * ldy, ldy, OXB_GEMV_PRO_F32, nullptr, 0.f, mode,
+                             d_residual ? d_residual + (size_t)b0 * ldy : nullptr);
+        if (rc) return rc;
     }
     return OXB_HIP_OK;
 }
@@ -297,9 +301,7 @@ void oxb_hip_shutdown(void) {
     g_rt.vectors.clear();
     g_rt.ws_x.release();
     g_rt.ws_y.release();
-    g_rt.ws_xq.release();
-    g_rt.ws_cneg.release();
-    g_rt.ws_xexp.release();
+    g_rt.ws_aux.release();
     g_rt.gemm_ws.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.static_scratch = nullptr;
@@ -411,11 +413,10 @@ int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows,
     OXB_API_END
 }
 
-int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,
-                         uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us) {
-    OXB_API_BEGIN
+static int profile_gemv_impl(bool floor_only, const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,
+                             uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
-    if (!ids || n_ids == 0 || !d_x || !d_y || !avg_us || iters == 0)
+    if (!ids || n_ids == 0 || (!floor_only && (!d_x || !d_y)) || !avg_us || iters == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
     std::vector<const Weight*> ws;
     for (uint32_t i = 0; i < n_ids; i++) {
@@ -428,34 +429,27 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
         ws.push_back(w);
     }
     if (ws[0]->L.n_sb > OXB_GEMV_MAX_SB) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k too large for a single launch");
-    int rc;
-    if ((rc = g_rt.ws_xq.ensure(oxb_xq_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-    if ((rc = g_rt.ws_cneg.ensure(oxb_cneg_bytes(k, OXB_GEMV_MAX_BATCH)))) return rc;
-    if ((rc = g_rt.ws_xexp.ensure(OXB_XEXP_BYTES))) return rc;
     const int fmt = (int)ws[0]->L.fmt;
-    hipError_t e = oxb_launch_quant_x(fmt, d_x, k, 1, (uint32_t*)g_rt.ws_xq.ptr, (int32_t*)g_rt.ws_cneg.ptr,
-                                      (int32_t*)g_rt.ws_xexp.ptr, g_rt.stream);
-    if (e != hipSuccess) return hip_fail(e, "kernel launch failed: quant_x");
     OxbGemvParams p;
     memset(&p, 0, sizeof p);
-    p.xq = (const uint32_t*)g_rt.ws_xq.ptr;
-    p.cneg = (const int32_t*)g_rt.ws_cneg.ptr;
-    p.xexp = (const int32_t*)g_rt.ws_xexp.ptr;
+    p.x = d_x;
     p.y = d_y;
     p.n_rows = n_rows;
     p.n_tiles = ws[0]->L.n_tiles;
     p.n_sb = ws[0]->L.n_sb;
+    p.k = k;
     p.sb_begin = 0;
     p.sb_count = p.n_sb;
-    p.NC = 8;
+    p.nvec = 1;
+    p.ldx = k;
     p.ldy = n_rows;
-    p.xq_bytes = (uint32_t)oxb_xq_bytes(k, 1);
-    p.cneg_bytes = (uint32_t)oxb_cneg_bytes(k, 1);
-    p.mode = OXB_GEMV_STORE;
+    p.pro = OXB_GEMV_PRO_F32;
+    p.epi = OXB_GEMV_STORE;
     hipEvent_t ev0, ev1;
+    hipError_t e;
     if ((e = hipEventCreate(&ev0)) != hipSuccess) return hip_fail(e, "event creation");
     if ((e = hipEventCreate(&ev1)) != hipSuccess) { (void)hipEventDestroy(ev0); return hip_fail(e, "event creation"); }
-    rc = OXB_HIP_OK;
+    int rc = OXB_HIP_OK;
     for (uint32_t i = 0; i < warmup + iters && rc == OXB_HIP_OK; i++) {
         if (i == warmup) (void)hipEventRecord(ev0, g_rt.stream);
         const Weight* w = ws[i % n_ids];
@@ -463,7 +457,7 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
         p.scales = w->d_scales;
         p.codes_bytes = (uint32_t)w->L.codes_bytes;
         p.scales_bytes = (uint32_t)w->L.scales_bytes;
-        e = oxb_launch_gemv(fmt, p, g_rt.n_cus, g_rt.stream);
+        e = floor_only ? oxb_launch_gemv_stream_floor(fmt, p, g_rt.n_cus, g_rt.stream) : oxb_launch_gemv(fmt, p, g_rt.n_cus, g_rt.stream);
         if (e != hipSuccess) rc = hip_fail(e, "kernel launch failed: gemv");
     }
     (void)hipEventRecord(ev1, g_rt.stream);
@@ -479,6 +473,19 @@ int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, 
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
     return rc;
+}
+
+int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,
+                         uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us) {
+    OXB_API_BEGIN
+    return profile_gemv_impl(false, ids, n_ids, d_x, d_y, n_rows, k, warmup, iters, avg_us);
+    OXB_API_END
+}
+
+int oxb_hip_profile_gemv_floor(const uint64_t* ids, uint32_t n_ids, uint32_t n_rows, uint32_t k, uint32_t warmup,
+                               uint32_t iters, float* avg_us) {
+    OXB_API_BEGIN
+    return profile_gemv_impl(true, ids, n_ids, nullptr, nullptr, n_rows, k, warmup, iters, avg_us);
     OXB_API_END
 }
 

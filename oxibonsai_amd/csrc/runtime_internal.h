@@ -53,7 +53,7 @@ struct Runtime {
     // Counts every free or replacement of a resident matrix or vector.  A captured decode graph holds their device
     // pointers; a model compares the count it captured under with this one and captures again when they differ.
     uint64_t weights_gen = 0;
-    DevBuf ws_x, ws_y, ws_xq, ws_cneg, ws_xexp;
+    DevBuf ws_x, ws_y, ws_aux;
     void* static_scratch = nullptr;  // device address of the library's file-scope scratch array on g_rt.device
     GemmWorkspace gemm_ws;  // shared by every GEMM call that does not bring its own
 };
@@ -68,6 +68,10 @@ Weight* find_weight(uint64_t id);
 int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual);
+// nvec <= OXB_GEMV_MAX_BATCH vectors x [nvec][ldx] through one pass over the weights: pro / epi are OXB_GEMV_PRO_* /
+// OXB_GEMV_* (RMSNorm with d_norm_w and eps in front; store, residual add or SwiGLU behind).
+int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, float* d_y, uint32_t ldy, int pro,
+                const float* d_norm_w, float eps, int epi, const float* d_residual);
 // x (device, [m][ldx]) -> y (device, [m][ldy]) through the fp16 packer + MFMA GEMM.  pack_op (OXB_PACK_*) names the
 // row-wise producer fused into the packer: RMSNorm with weights d_pack_w and eps, or SwiGLU of x = [gate | up].
 // ws = nullptr uses (and may grow) the runtime's shared workspace.

@@ -1,113 +1,118 @@
-"""numpy model of the device GEMV arithmetic (quantiser + int8 MFMA + recombination).
+"""numpy model of the device GEMV arithmetic (in-kernel activation quantiser + int8 MFMA + recombination).
 
-It reads the *resident* sections produced by the library's host repacker and
-reproduces, step by step, what quant_x_kernel and gemv_mfma_kernel compute:
-int8 operands made by AND-masks, eight balanced base-256 activation digits scaled per
-exponent group (the K slice of one GEMV wave), the accumulator start values and the fp32 epilogue.  The CPU test suite holds it to
-the oracle, which pins the arithmetic design where no GPU is present."""
+It reads the *resident* sections produced by the library's host repacker and reproduces, step by step, what
+gemv_kernel computes: int8 weight operands made by AND-masks, four balanced base-256 activation digits scaled per
+K slice of a wave, the accumulator start values that cancel the bias of the unsigned code encodings, the joining of
+the digit sums, the fp16 block scale, the slice exponent, the waves' partial sums added in wave order.  The CPU test
+suite holds it to the oracle, which pins the arithmetic design where no GPU is present; the GPU tests can hold the
+kernel to this model bit for bit."""
 from __future__ import annotations
 
 import numpy as np
 
-P = 53
-ND = 8
+P = {0: 29, 1: 30}          # fixed-point bits below 2^E (Q1 operands hold 2 r)
+MAX_SB = 24                  # superblocks of K per launch
 
 
-def _digits(v: np.ndarray) -> np.ndarray:
-    """int64 array -> balanced signed base-256 digits [..., 8]."""
-    bias = np.uint64(0x0080808080808080)
-    with np.errstate(over="ignore"):
-        t = (v.astype(np.int64).view(np.uint64) + bias) ^ bias
-    d = np.stack([(t >> np.uint64(8 * i)) & np.uint64(0xFF) for i in range(ND)], axis=-1).astype(np.int64)
+def _digits32(v: np.ndarray) -> np.ndarray:
+    """int64 values in int32 range -> four balanced signed base-256 digits [..., 4] (the top one takes the rest)."""
+    t = ((v.astype(np.int64) + 0x808080) & 0xFFFFFFFF) ^ 0x808080
+    d = np.stack([(t >> (8 * i)) & 0xFF for i in range(4)], axis=-1)
     return np.where(d >= 128, d - 256, d)
 
 
-def group_sb(n_sb: int) -> int:
-    """Superblocks per exponent group = K slice of one GEMV wave (oxb_xq_gsb)."""
-    return min(3, max(1, (n_sb + 7) // 8))
+def _f32(x):
+    return np.asarray(x, dtype=np.float32)
 
 
-def quant_x(fmt: int, x: np.ndarray, nblk_pad: int):
-    """Returns (B[blk, m, g, jj, bb, digit] int, cneg[blk, digit] int, xexp[group] int with None for a
-    group that holds a NaN or an infinity).  Every exponent group is scaled by its own maximum."""
-    k = x.size
-    nblk = k // 128
-    n_sb = nblk_pad // 4
-    gsb = group_sb(n_sb)
-    n_groups = (n_sb + gsb - 1) // gsb
-    B = np.zeros((nblk_pad, 2, 4, 4, 4, ND), dtype=np.int64)
-    cneg = np.zeros((nblk_pad, ND), dtype=np.int64)
-    xexp = []
-    for gi in range(n_groups):
-        b0, b1 = gi * gsb * 4, min((gi + 1) * gsb * 4, nblk)
-        xs = x[b0 * 128:b1 * 128]
-        if not np.all(np.isfinite(xs)):
-            xexp.append(None)
-            continue
-        mx = float(np.max(np.abs(xs))) if xs.size else 0.0
-        if mx == 0.0:
-            xexp.append(0)
-            continue
-        _, E = np.frexp(np.float32(mx))
-        E = int(E)
-        xexp.append(E - P)
-        blk, m, g, jj, bb = np.meshgrid(np.arange(b0, b1), np.arange(2), np.arange(4), np.arange(4), np.arange(4),
-                                        indexing="ij")
+def _fma32(a, b, c):
+    """fp32 fused multiply-add through float64 (the product of two f32 is exact there)."""
+    return _f32(a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64))
+
+
+def slice_exponent(xs: np.ndarray):
+    """E with 2^E > max |x| over a wave's K slice (None for a slice that holds a NaN or an infinity), and whether
+    the slice is all zeros."""
+    mxb = int((xs.view(np.uint32) & 0x7FFFFFFF).max())
+    if mxb >= 0x7F800000:
+        return None, False
+    be = mxb >> 23
+    return (be if be else 1) - 126, mxb == 0
+
+
+def quantise_block(fmt: int, xb: np.ndarray, E: int):
+    """One 128-activation block at the slice exponent E -> (operand digits [128][4] in k order, start values [4])."""
+    k = np.arange(128)
+    if fmt == 0:
+        js = (k % 8) & 3                            # bit j of its code byte is worth 2^(j & 3): k = 32 g + 8 bb + j
+        r = np.rint(np.ldexp(xb.astype(np.float32), (P[0] - E - js).astype(np.int32)).astype(np.float32)).astype(np.int64)
+        xi = 2 * r
+        csum = int(np.sum(r << js))
+    else:
+        jj = k % 4                                  # field inside its code byte: k = 32 g + 16 m + 4 bb + jj
+        js = 2 * jj
+        r = np.rint(np.ldexp(xb.astype(np.float32), (P[1] - E - js).astype(np.int32)).astype(np.float32)).astype(np.int64)
+        xi = r
+        csum = int(np.sum(np.where(jj < 3, r << js, 0)))
+    t = ((-csum + 0x808080) ^ 0x808080)
+    c = [((t >> (8 * i)) & 0xFF) for i in range(3)]
+    c = [v - 256 if v >= 128 else v for v in c] + [t >> 24]
+    return _digits32(xi), np.array(c, dtype=np.int64)
+
+
+def _weight_bytes(fmt: int, codes, tile: int, sb: int, q: int) -> np.ndarray:
+    """Signed int8 operand bytes [16 rows][128 k] of block q of unit (tile, sb), as the AND masks produce them."""
+    out = np.zeros((16, 128), dtype=np.int64)
+    for g in range(4):
+        lanes = g * 16 + np.arange(16)
         if fmt == 0:
-            j = 4 * m + jj
-            kk = blk * 128 + 32 * g + 8 * bb + j
-            r = np.rint(np.ldexp(x[kk].astype(np.float64), P - E - j)).astype(np.int64)
-            xi = np.where(j == 7, -2 * r, 2 * r)
-            cr, cmul = r, (1 << j)
+            w = codes[tile, sb, lanes * 4 + q].astype(np.int64)
+            for i in range(32):                     # bit i of the dword: byte bb = i // 8, position j = i % 8
+                out[:, 32 * g + i] = ((w >> i) & 1) << (i % 4)      # high nibbles are masked after a shift by 4
         else:
-            kk = blk * 128 + 32 * g + 16 * m + 4 * bb + jj
-            xi = np.rint(np.ldexp(x[kk].astype(np.float64), P - E - 2 * jj)).astype(np.int64)
-            cr, cmul = xi, np.where(jj < 3, 1 << (2 * jj), 0)
-        B[b0:b1] = _digits(xi)
-        cneg[b0:b1] = -(_digits(cr) * cmul[..., None]).sum(axis=(1, 2, 3, 4))
-    return B, cneg, xexp
+            for m in range(2):
+                w = codes[tile, sb, (q >> 1) * 256 + lanes * 4 + (q & 1) * 2 + m].astype(np.int64)
+                for i in range(16):                 # field i: byte bb = i // 4, position jj = i % 4
+                    b = ((w >> (2 * i)) & 3) << (2 * (i % 4))
+                    out[:, 32 * g + 16 * m + i] = np.where(b >= 128, b - 256, b)
+    return out
 
 
 def gemv(fmt: int, codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
     n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512
-    nblk_pad = n_sb * 4
-    gsb = group_sb(n_sb)
-    B, cneg, xexp = quant_x(fmt, x.astype(np.float32), nblk_pad)
-    if any(e is None for e in xexp):
-        return np.full(n_rows, np.nan, dtype=np.float32)
+    x = np.asarray(x, dtype=np.float32)
+    xp = np.zeros(n_sb * 512, dtype=np.float32)
+    xp[:k] = x
     unit = 256 if fmt == 0 else 512
     codes = codes_u8.view(np.uint32).reshape(n_tiles, n_sb, unit)
-    scales = scales_u8.view(np.float16).reshape(n_tiles, n_sb, 4, 4, 4).astype(np.float32)  # [rg][q][v]
+    scales = scales_u8.view(np.float16).reshape(n_tiles, n_sb, 16, 4).astype(np.float32)  # [row][q]
     y = np.zeros(n_rows, dtype=np.float32)
-    jjs = np.arange(4)
     for tile in range(n_tiles):
-        total = np.zeros((16, ND), dtype=np.float32)  # [row][digit], groups added with their exponents
-        for gi in range(len(xexp)):
-            accf = np.zeros((16, ND), dtype=np.float32)  # one wave's partial sums
-            for sb in range(gi * gsb, min((gi + 1) * gsb, n_sb)):
-                for q in range(4):
-                    blk = sb * 4 + q
-                    I = np.tile(cneg[blk][None, :], (16, 1))  # [row][digit]
-                    for m in range(2):
-                        for g in range(4):
-                            lanes = g * 16 + np.arange(16)
-                            if fmt == 0:
-                                w = codes[tile, sb, lanes * 4 + q].astype(np.int64)
-                                a = w[:, None] & (0x01010101 << (4 * m + jjs))[None, :]
-                            else:
-                                w = codes[tile, sb, (q >> 1) * 256 + lanes * 4 + (q & 1) * 2 + m].astype(np.int64)
-                                a = w[:, None] & (0x03030303 << (2 * jjs))[None, :]
-                            ab = np.stack([(a >> (8 * b)) & 0xFF for b in range(4)], axis=-1)  # [row][jj][bb]
-                            ab = np.where(ab >= 128, ab - 256, ab)
-                            I = I + np.einsum("rjb,jbd->rd", ab, B[blk, m, g])
-                    d = scales[tile, sb, :, q, :].reshape(16)  # row = 4*rg + v
-                    accf = (accf + I.astype(np.float32) * d[:, None]).astype(np.float32)
-            weighted = np.ldexp(accf, xexp[gi] + 8 * np.arange(ND)[None, :]).astype(np.float32)
-            total = (total + weighted).astype(np.float32)
-        v = np.zeros(16, dtype=np.float32)
-        for dgt in range(ND):
-            v = (v + total[:, dgt]).astype(np.float32)
+        total = None
+        for sb_begin in range(0, n_sb, MAX_SB):                 # launches
+            sb_count = min(MAX_SB, n_sb - sb_begin)
+            nsbw = (sb_count + 7) // 8
+            S = (sb_count + nsbw - 1) // nsbw
+            launch = np.zeros(16, dtype=np.float32)
+            for s in range(S):                                  # waves, added in order
+                accf = np.zeros(16, dtype=np.float32)
+                sb_lo, sb_hi = sb_begin + s * nsbw, min(sb_begin + (s + 1) * nsbw, sb_begin + sb_count)
+                E, zero = slice_exponent(xp[sb_lo * 512:sb_hi * 512])
+                if E is None:
+                    return np.full(n_rows, np.nan, dtype=np.float32)
+                for sb in range(sb_lo, sb_hi):
+                    for q in range(4):
+                        dig, c4 = quantise_block(fmt, xp[(sb * 4 + q) * 128:(sb * 4 + q + 1) * 128], E)
+                        wb = _weight_bytes(fmt, codes, tile, sb, q)
+                        acc = c4[None, :] + wb @ dig                                    # [16 rows][4 digits], exact
+                        acc = ((acc + 2**31) % 2**32) - 2**31                           # int32 accumulators
+                        lo = (acc[:, 0] + (acc[:, 1] << 8) + 2**31) % 2**32 - 2**31
+                        hi = (acc[:, 2] + (acc[:, 3] << 8) + 2**31) % 2**32 - 2**31
+                        val = _fma32(_f32(hi), _f32(np.full(16, 65536.0)), _f32(lo))
+                        accf = _fma32(val, scales[tile, sb, :, q], accf)
+                launch = (launch + np.ldexp(accf, 0 if zero else E - P[fmt]).astype(np.float32)).astype(np.float32)
+            total = launch if total is None else (total + launch).astype(np.float32)
         rows = tile * 16 + np.arange(16)
         ok = rows < n_rows
-        y[rows[ok]] = v[ok]
+        y[rows[ok]] = total[ok]
     return y
