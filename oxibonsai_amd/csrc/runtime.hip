@@ -54,6 +54,11 @@ static __device__ __align__(256) unsigned char oxb_static_scratch[OXB_STATIC_SCR
 int DevBuf::ensure(size_t bytes) {
     if (bytes <= cap) return OXB_HIP_OK;
     if (fixed) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %zu bytes of scratch needed, the fixed buffer holds %zu", bytes, cap);
+    // Growing means hipFree + hipMalloc, which a stream capture in progress cannot take: every buffer a captured
+    // sequence uses is sized before the capture begins, so this is a bug if it ever triggers - fail, do not allocate.
+    hipStreamCaptureStatus cap_status = hipStreamCaptureStatusNone;
+    if (g_rt.stream && hipStreamIsCapturing(g_rt.stream, &cap_status) == hipSuccess && cap_status != hipStreamCaptureStatusNone)
+        return fail(OXB_HIP_KERNEL_LAUNCH, "internal error: a workspace of %zu bytes would have to grow to %zu inside a stream capture", cap, bytes);
     if (ptr) (void)hipFree(ptr);
     ptr = nullptr;
     cap = 0;
