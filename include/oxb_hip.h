@@ -60,6 +60,15 @@ const char* oxb_hip_last_error(void);
  * and replaces a weight already stored under it. */
 int  oxb_hip_upload_q1(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
 int  oxb_hip_upload_tq2(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
+/* The same uploads as the trait has them, bytes (or blocks) only: upload_weights_raw(&self, blocks: &[u8]) (KG/mod.rs:445)
+ * and upload_weights_ternary(&self, blocks: &[BlockTQ2_0_g128]) (KG/mod.rs:472; n_bytes = 34 * blocks.len()).  The weight
+ * takes its shape from the first call that names one - gemv_q1_g128_cached(handle, input, n_rows, k) (KG/mod.rs:457), a GEMM,
+ * or oxb_hip_model_create through the model's dimensions - which must satisfy n_rows * k / 128 == number of blocks; the
+ * device then repacks the bytes into the resident layout (the result is what the shaped upload stores, bit for bit) and
+ * the shape stays.  That first call must not run inside a stream capture.  Until then oxb_hip_weight_info reports
+ * 0 x 0 and oxb_hip_dequant fails. */
+int  oxb_hip_upload_q1_raw(uint64_t* id, const uint8_t* aos, size_t n_bytes);
+int  oxb_hip_upload_tq2_raw(uint64_t* id, const uint8_t* aos, size_t n_bytes);
 int  oxb_hip_free_weight(uint64_t id);
 int  oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, size_t* resident_bytes);
 /* Decode the resident copy back to fp32 [n_rows][k]: dequant_1bit_g128 / dequant_tq2_0_g128
@@ -128,7 +137,7 @@ typedef struct {
     uint32_t n_layers, h, inter, nq, nkv, hd, vocab, max_seq, batch;
     float eps, rope_theta;
     const oxb_layer_ids* layers;   /* [n_layers], read during the call only */
-    uint64_t final_norm, lm_head;
+    uint64_t final_norm, lm_head;  /* lm_head == 0: no LM head on the device (vocab is ignored; final_norm may be 0 too) */
 } oxb_model_desc;
 /* Allocates the FP16 KV cache [batch][layer][kv_head][max_seq rounded up to 128][hd] (CudaKvCache, KG/cuda_full_layer/mod.rs:112-139),
  * the activation buffers (mod.rs:149-181) and the RoPE table (crates/oxibonsai-model/src/layers/rope.rs:27-48). */
@@ -141,6 +150,17 @@ int  oxb_hip_model_destroy(uint64_t model);
  * Batches of up to 4 use the fp32-exact GEMV (one pass over the weights); from 5 sequences on the projections run as
  * fp16 matrix-core GEMMs (the arithmetic of oxb_hip_gemm / oxb_hip_prefill). */
 int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, float* logits_or_null, uint32_t* token_out);
+/* The same step without the LM head: try_cuda_full_forward / try_cuda_full_forward_ternary
+ * (KG/cuda_full_layer/encode_q1.rs:813-830, encode_ternary.rs:694-711) return the hidden state after the last layer and
+ * the final RMSNorm (final_norm_bytes: Option - a model created with final_norm == 0 returns the un-normed state);
+ * the caller runs its own LM head.  normed_out: [batch][h].  Plain launches, no graph. */
+int  oxb_hip_decode_hidden(uint64_t model, const float* hidden, const uint32_t* pos, float* normed_out);
+/* The reference's entry points receive the RoPE rows of their positions from the caller (rope_cos / rope_sin of `pos`,
+ * hd/2 values each, encode_q1.rs:816-817; cos_table / sin_table [batch_size][hd/2] for a prefill, KG/cuda_prefill/try_apis.rs:48-49).
+ * This call stores such rows for positions pos_start .. pos_start + n_pos - 1 in the model's table, in place of the
+ * values oxb_hip_model_create worked out from rope_theta, so that a caller with its own table (scaled or extended
+ * RoPE) gets its own angles. */
+int  oxb_hip_model_set_rope_rows(uint64_t model, uint32_t pos_start, uint32_t n_pos, const float* cos_rows, const float* sin_rows);
 /* Batched prefill: try_cuda_prefill / try_cuda_prefill_ternary (KG/cuda_prefill/try_apis.rs:42, 318; per layer
  * encode_prefill_layer[_ternary], KG/cuda_prefill/encode_q1.rs:123, encode_ternary.rs:114).  hidden = [n_tokens][h]
  * embedding rows of sequence `seq` (0 .. batch-1) for positions pos_start .. pos_start + n_tokens - 1; keys and

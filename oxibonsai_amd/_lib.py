@@ -27,6 +27,8 @@ _SIGNATURES = {
     "oxb_hip_last_error": ([], C.c_char_p),
     "oxb_hip_upload_q1": ([u64p, u8p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_upload_tq2": ([u64p, u8p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),
+    "oxb_hip_upload_q1_raw": ([u64p, u8p, C.c_size_t], C.c_int),
+    "oxb_hip_upload_tq2_raw": ([u64p, u8p, C.c_size_t], C.c_int),
     "oxb_hip_free_weight": ([C.c_uint64], C.c_int),
     "oxb_hip_weight_info": ([C.c_uint64, C.POINTER(C.c_int), u32p, u32p, szp], C.c_int),
     "oxb_hip_dequant": ([C.c_uint64, f32p, C.c_size_t], C.c_int),
@@ -50,6 +52,8 @@ _SIGNATURES = {
     "oxb_hip_model_reset": ([C.c_uint64], C.c_int),
     "oxb_hip_model_destroy": ([C.c_uint64], C.c_int),
     "oxb_hip_decode": ([C.c_uint64, f32p, u32p, f32p, u32p], C.c_int),
+    "oxb_hip_decode_hidden": ([C.c_uint64, f32p, u32p, f32p], C.c_int),
+    "oxb_hip_model_set_rope_rows": ([C.c_uint64, C.c_uint32, C.c_uint32, f32p, f32p], C.c_int),
     "oxb_hip_prefill": ([C.c_uint64, C.c_uint32, f32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_model_uses_graph": ([C.c_uint64], C.c_int),
     "oxb_hip_model_set_attention": ([C.c_uint64, C.c_void_p], C.c_int),

@@ -138,20 +138,26 @@ class NativeHipBackend:
     # -- resident weights -------------------------------------------------------
     def upload_weights_raw(self, block_bytes, n_rows: int | None = None, k: int | None = None,
                            handle_id: int = 0) -> GpuWeightHandle:
-        """Q1_0_g128 AoS bytes -> resident handle.  The reference passes bytes only and gives
-        the shape at GEMV time; the tiled resident layout needs it at upload, so it is an argument here."""
+        """Q1_0_g128 AoS bytes -> resident handle (GpuBackendTrait::upload_weights_raw, gpu_backend/mod.rs:445).
+        As in the reference the bytes are enough: the shape then comes with the first cached GEMV / GEMM call or
+        with the model that names the handle.  Giving (n_rows, k) here binds it at once."""
         return self._upload(Q1, block_bytes, n_rows, k, handle_id)
 
     def upload_weights_ternary(self, blocks, n_rows: int | None = None, k: int | None = None,
                                handle_id: int = 0) -> GpuWeightHandle:
-        """TQ2_0_g128 blocks (struct byte order [qs 32][d]) -> resident handle."""
+        """TQ2_0_g128 blocks (struct byte order [qs 32][d]) -> resident handle (upload_weights_ternary,
+        gpu_backend/mod.rs:472); the shape is optional as in upload_weights_raw."""
         return self._upload(TQ2, blocks, n_rows, k, handle_id)
 
     def _upload(self, fmt, block_bytes, n_rows, k, handle_id=0):
         b = _as_bytes(block_bytes)
-        if n_rows is None or k is None:
-            raise GpuError(5, "invalid argument: n_rows and k are required at upload")
         hid = C.c_uint64(handle_id)
+        if n_rows is None and k is None:
+            fn = self._lib.oxb_hip_upload_q1_raw if fmt == Q1 else self._lib.oxb_hip_upload_tq2_raw
+            _check(fn(C.byref(hid), _u8(b), b.size))
+            return GpuWeightHandle(hid.value)
+        if n_rows is None or k is None:
+            raise GpuError(5, "invalid argument: give both n_rows and k, or neither")
         fn = self._lib.oxb_hip_upload_q1 if fmt == Q1 else self._lib.oxb_hip_upload_tq2
         _check(fn(C.byref(hid), _u8(b), b.size, n_rows, k))
         return GpuWeightHandle(hid.value)

@@ -41,6 +41,9 @@ hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t
 hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st);
 hipError_t oxb_launch_dequant(const OxbLayout& L, const uint32_t* d_codes, const uint16_t* d_scales, float* d_out,
                               hipStream_t st);
+// Block bytes in the reference's order (device copy, 2-byte aligned) -> the resident codes and scales sections, every
+// padded entry included: the device twin of oxb_repack_aos_to_tiled.
+hipError_t oxb_launch_repack(const OxbLayout& L, const uint8_t* d_aos, uint32_t* d_codes, uint16_t* d_scales, hipStream_t st);
 // act[v][i] = silu(gu[v][i]) * gu[v][inter + i] for nvec vectors (rows of 2 * inter floats in, ldo floats out): the
 // separate SwiGLU for rows too long for one GEMV launch.
 hipError_t oxb_launch_swiglu(const float* d_gu, uint32_t inter, uint32_t nvec, float* d_out, uint32_t ldo, hipStream_t st);

@@ -32,6 +32,7 @@
 //   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y
 //   stream_floor_kernel  the same loads and nothing else (measurement aid)
 //   dequant_kernel       resident layout -> fp32 weights (bit-exactness check)
+//   repack_kernel        the reference's block bytes (array of structs) -> resident layout, at upload
 //   swiglu_kernel        silu(gate) * up on fp32 vectors (rows too long for one GEMV launch)
 #include <hip/hip_runtime.h>
 #include <stdint.h>
@@ -424,6 +425,51 @@ __global__ __launch_bounds__(256) void dequant_kernel(OxbLayout L, const uint32_
     }
 }
 
+// ---------------------------------------------------------------------------
+// Upload-time repack on the device: the reference's blocks (Q1 18 B [d f16][qs 16], TQ2 34 B [qs 32][d f16], row
+// after row) -> the resident codes and scales sections, padding included.  It writes what the host routine
+// oxb_repack_aos_to_tiled writes (the reformatters cuda_graph/cudagraph_reformat_q1_aos_to_soa_group.rs:21-41 and
+// cudagraph_reformat_tq2_blocks_to_soa_group.rs:16-27 are its counterparts).  One workgroup per (tile, superblock)
+// unit, one thread per output dword: stores are contiguous, the 2-byte-aligned block bytes are read as halves.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void repack_kernel(OxbLayout L, const uint16_t* __restrict__ aos,
+                                                     uint32_t* __restrict__ codes, uint16_t* __restrict__ scales) {
+    const uint32_t bpr = L.k / OXB_QK;
+    const uint32_t tile = blockIdx.x / L.n_sb, sb = blockIdx.x % L.n_sb;
+    const uint32_t t = threadIdx.x;
+    const uint32_t halves = L.fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES / 2 : OXB_TQ2_AOS_BYTES / 2;
+    if (t < 64) {  // scale [r][q]
+        const uint32_t r = t >> 2, q = t & 3u, row = tile * 16 + r, blk = sb * 4 + q;
+        uint16_t d = 0;
+        if (row < L.n_rows && blk < bpr) {
+            const uint16_t* b = aos + ((size_t)row * bpr + blk) * halves;
+            d = L.fmt == OXB_FMT_Q1 ? b[0] : b[16];
+        }
+        scales[(size_t)blockIdx.x * 64 + t] = d;
+    }
+    for (uint32_t dwi = t; dwi < L.unit_dwords; dwi += 256) {
+        uint32_t out = 0;
+        if (L.fmt == OXB_FMT_Q1) {  // dword = lane * 4 + q, lane = g * 16 + r
+            const uint32_t q = dwi & 3u, lane = dwi >> 2, r = lane & 15u, g = lane >> 4;
+            const uint32_t row = tile * 16 + r, blk = sb * 4 + q;
+            if (row < L.n_rows && blk < bpr) {
+                const uint16_t* b = aos + ((size_t)row * bpr + blk) * halves + 1 + 2 * g;
+                out = (uint32_t)b[0] | ((uint32_t)b[1] << 16);
+            }
+        } else {  // dword = half * 256 + lane * 4 + e * 2 + m
+            const uint32_t half = dwi >> 8, lane = (dwi >> 2) & 63u, e = (dwi >> 1) & 1u, m = dwi & 1u;
+            const uint32_t r = lane & 15u, g = lane >> 4;
+            const uint32_t row = tile * 16 + r, blk = sb * 4 + half * 2 + e;
+            if (row < L.n_rows && blk < bpr) {
+                const uint16_t* b = aos + ((size_t)row * bpr + blk) * halves + 2 * (2 * g + m);
+                const uint32_t w = (uint32_t)b[0] | ((uint32_t)b[1] << 16);
+                for (uint32_t i = 0; i < 16; i++) out |= oxb_tq2_encode_field((w >> (2 * i)) & 3u, i) << (2 * i);
+            }
+        }
+        codes[(size_t)blockIdx.x * L.unit_dwords + dwi] = out;
+    }
+}
+
 // silu(gate) * up (simd_float_ops.rs:217-236) for rows whose GEMV took several launches.
 __global__ __launch_bounds__(256) void swiglu_kernel(const float* __restrict__ gu, uint32_t inter, float* __restrict__ out, uint32_t ldo) {
     const uint32_t v = blockIdx.y, i = blockIdx.x * 256 + threadIdx.x;
@@ -530,5 +576,14 @@ hipError_t oxb_launch_dequant(const OxbLayout& L, const uint32_t* d_codes, const
     if (total == 0) return hipSuccess;
     const uint32_t grid = (uint32_t)((total + 255) / 256);
     hipLaunchKernelGGL(dequant_kernel, dim3(grid), dim3(256), 0, st, L, d_codes, d_scales, d_out);
+    return hipGetLastError();
+}
+
+hipError_t oxb_launch_repack(const OxbLayout& L, const uint8_t* d_aos, uint32_t* d_codes, uint16_t* d_scales, hipStream_t st) {
+    const uint64_t units = (uint64_t)L.n_tiles * L.n_sb;
+    if (units == 0) return hipSuccess;
+    if (units > 0x7FFFFFFFull) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(repack_kernel, dim3((uint32_t)units), dim3(256), 0, st, L, reinterpret_cast<const uint16_t*>(d_aos),
+                       d_codes, d_scales);
     return hipGetLastError();
 }

@@ -52,6 +52,8 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 // p.part; then the merge of the slots into the fp32 attention output d_out [batch][nq * hd].
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
 hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
+// out[v] = w * x[v] / sqrt(mean(x[v]^2) + eps) for nvec vectors of n values; d_w == nullptr copies.
+hipError_t oxb_launch_rmsnorm(const float* d_x, const float* d_w, uint32_t n, uint32_t nvec, float eps, float* d_out, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.
 #define OXB_ARGMAX_MAX_PARTS 256u
 hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st);

@@ -750,6 +750,35 @@ hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float
     return hipGetLastError();
 }
 
+// RMSNorm of `nvec` vectors of n values (simd_float_ops.rs:204-215): out = w * x / sqrt(mean(x^2) + eps), w == nullptr
+// copies x.  One workgroup per vector.  The fused paths carry their norms inside the GEMV / GEMM kernels; this one
+// finishes a forward that ends at the normed hidden state (no LM head on the device).
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ x, const float* __restrict__ w, uint32_t n,
+                                                      float eps, float* __restrict__ out) {
+    __shared__ float part[4];
+    const float* xv = x + (size_t)blockIdx.x * n;
+    float* ov = out + (size_t)blockIdx.x * n;
+    const uint32_t tid = threadIdx.x;
+    if (!w) {
+        for (uint32_t i = tid; i < n; i += 256) ov[i] = xv[i];
+        return;
+    }
+    float ss = 0.f;
+    for (uint32_t i = tid; i < n; i += 256) ss += xv[i] * xv[i];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    if ((tid & 63u) == 0) part[tid >> 6] = ss;
+    __syncthreads();
+    const float inv_rms = 1.0f / sqrtf((part[0] + part[1] + part[2] + part[3]) / (float)n + eps);
+    for (uint32_t i = tid; i < n; i += 256) ov[i] = w[i] * xv[i] * inv_rms;
+}
+
+hipError_t oxb_launch_rmsnorm(const float* d_x, const float* d_w, uint32_t n, uint32_t nvec, float eps, float* d_out, hipStream_t st) {
+    if (n == 0 || nvec == 0 || !d_x || !d_out) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(rmsnorm_kernel, dim3(nvec), dim3(256), 0, st, d_x, d_w, n, eps, d_out);
+    return hipGetLastError();
+}
+
 uint32_t oxb_argmax_parts(uint32_t n) {
     const uint32_t p = (n + 2047u) / 2048u;
     return p < 1 ? 1 : (p > OXB_ARGMAX_MAX_PARTS ? OXB_ARGMAX_MAX_PARTS : p);

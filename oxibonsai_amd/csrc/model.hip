@@ -55,6 +55,7 @@ struct Model {
     uint32_t chunk = 0, n_splits = 0;
     // graph
     hipGraphExec_t graph_exec = nullptr;
+    uint64_t checked_gen = 0;  // g_rt.weights_gen when every handle was last looked up
     uint64_t graph_gen = 0;  // g_rt.weights_gen at capture: the graph holds the weights' device pointers of that moment
     bool graph_failed = false;
     bool want_logits_in_graph = true;
@@ -140,10 +141,13 @@ static const float* vec_ptr(uint64_t id, uint32_t n, const char* what, int* rc) 
 }
 
 static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, const char* what, int* rc) {
-    const Weight* w = find_weight(id);
+    Weight* w = find_weight(id);
     if (!w) {
         *rc = fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu (%s) not found", (unsigned long long)id, what);
         return nullptr;
+    }
+    if (w->d_raw && (int)w->L.fmt == fmt) {  // uploaded as bytes alone: the model's dimensions give it its shape
+        if ((*rc = bind_shape(*w, n_rows, k))) return nullptr;
     }
     if ((int)w->L.fmt != fmt || w->L.n_rows != n_rows || w->L.k != k) {
         *rc = fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: %s is fmt %u %ux%u, model needs fmt %d %ux%u", what,
@@ -184,6 +188,30 @@ static int encode_ffn(float* hidden, const float* attn_out, const float* ffn_nor
     OXB_TRY(gate_up_swiglu(gate_up, hidden, h, nb, ffn_norm, eps, gu, act, inter));
     OXB_TRY(gemv_launch(down, act, inter, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden));
     return OXB_HIP_OK;
+}
+
+// Looks every handle of the model up with the shape the model needs (which also binds a weight that was uploaded
+// without one).  Run at creation and again whenever a weight or vector was replaced or freed since, before a decode
+// step is captured: inside the capture nothing may allocate.
+static int check_model_handles(Model& m) {
+    const oxb_model_desc& d = m.d;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    int rc = OXB_HIP_OK;
+    for (uint32_t L = 0; L < d.n_layers && !rc; L++) {
+        const oxb_layer_ids& ly = m.layers[L];
+        vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
+        if (!rc) vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
+        if (!rc) vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
+        if (!rc) vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
+        if (!rc) mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
+        if (!rc) mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
+        if (!rc) mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
+        if (!rc) mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
+    }
+    if (!rc && d.final_norm) vec_ptr(d.final_norm, d.h, "final_norm", &rc);
+    if (!rc && d.lm_head) mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+    if (!rc) m.checked_gen = g_rt.weights_gen;
+    return rc;
 }
 
 static OxbKvLayout kv_layout(const Model& m) {
@@ -465,6 +493,7 @@ static int encode_prefill(Model& m, uint32_t seq, uint32_t M, uint32_t pos_start
         OXB_TRY(gemm_device(*wgu, m.pf_hidden, d.h, m.pf_gu, M, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps));
         OXB_TRY(gemm_device(*wdn, m.pf_gu, d.inter, m.pf_hidden, M, d.h, OXB_GEMM_RESIDUAL, m.pf_hidden, OXB_PACK_IDENT, nullptr, 0.f));
     }
+    if (!d.lm_head) return OXB_HIP_OK;  // the caller asked for the cache rows only
     // last token: final norm, LM head, greedy token (fp32-exact products, as in a decode step)
     const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
     const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
@@ -593,8 +622,10 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     OXB_TRY(ensure_init());
     const oxb_model_desc& d = *desc;
     if (d.fmt != OXB_FMT_Q1 && d.fmt != OXB_FMT_TQ2) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown format %d", d.fmt);
-    if (!d.n_layers || !d.h || !d.inter || !d.nq || !d.nkv || !d.vocab || !d.max_seq || !d.batch)
+    if (!d.n_layers || !d.h || !d.inter || !d.nq || !d.nkv || !d.max_seq || !d.batch || (d.lm_head && !d.vocab))
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: a model dimension is 0");
+    if (d.lm_head && !d.final_norm)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: a model with an LM head needs the final norm vector");
     if (d.hd != 32 && d.hd != 64 && d.hd != 128 && d.hd != 256)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: head_dim %u (supported: 32, 64, 128, 256)", d.hd);
     if (d.nq % d.nkv != 0 || d.nq / d.nkv > 16)
@@ -610,20 +641,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
     m.d.layers = nullptr;
     const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
     // check every handle now, so that a decode step cannot fail half way
-    int rc = OXB_HIP_OK;
-    for (uint32_t L = 0; L < d.n_layers && !rc; L++) {
-        const oxb_layer_ids& ly = m.layers[L];
-        vec_ptr(ly.attn_norm, d.h, "attn_norm", &rc);
-        vec_ptr(ly.q_norm, d.hd, "q_norm", &rc);
-        vec_ptr(ly.k_norm, d.hd, "k_norm", &rc);
-        vec_ptr(ly.ffn_norm, d.h, "ffn_norm", &rc);
-        mat_ptr(ly.qkv, d.fmt, qkv_rows, d.h, "qkv", &rc);
-        mat_ptr(ly.o, d.fmt, d.h, qd, "o", &rc);
-        mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
-        mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
-    }
-    if (!rc) vec_ptr(d.final_norm, d.h, "final_norm", &rc);
-    if (!rc) mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
+    int rc = check_model_handles(m);
     if (rc) return rc;
 
     m.chunk = OXB_ATTN_CHUNK_POSITIONS;
@@ -634,7 +652,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         (rc = dev_alloc(m, (void**)&m.attn_part, B * d.nq * max_slots * (d.hd + OXB_ATTN_PART_PAD) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.act, B * d.inter * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.logits, B * d.vocab * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
+        (rc = dev_alloc(m, (void**)&m.logits, B * (d.lm_head ? d.vocab : 1) * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
         (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4))) {
@@ -669,6 +687,7 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
                                                                  {m.layers[0].down, d.h, d.inter}, {d.lm_head, d.vocab, d.h}};
         for (const auto& sh : shapes) {
             const Weight* w = find_weight(sh.id);
+            if (!w) continue;  // a model without an LM head
             OxbGemmParams gp;
             memset(&gp, 0, sizeof gp);
             gp.n_rows = sh.n;
@@ -891,6 +910,8 @@ int oxb_hip_model_reset(uint64_t model) {
 // kernel by kernel when capture is off or failed.
 static int run_decode_step(Model& m) {
     hipStream_t st = g_rt.stream;
+    if (!m.d.lm_head) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: the model has no LM head (oxb_hip_decode_hidden returns its normed hidden state)");
+    if (m.checked_gen != g_rt.weights_gen) OXB_TRY(check_model_handles(m));
     if (m.graph_exec && m.graph_gen != g_rt.weights_gen) {
         // a weight or norm vector was freed or replaced since the capture: look every handle up again
         (void)hipGraphExecDestroy(m.graph_exec);
@@ -952,6 +973,61 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     OXB_API_END
 }
 
+int oxb_hip_decode_hidden(uint64_t model, const float* hidden, const uint32_t* pos, float* normed_out) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    const oxb_model_desc& d = m.d;
+    if (!hidden || !pos || !normed_out) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden, pos or output");
+    for (uint32_t b = 0; b < d.batch; b++)
+        if (pos[b] >= d.max_seq)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+    if (m.checked_gen != g_rt.weights_gen) OXB_TRY(check_model_handles(m));
+    for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + 1));
+    OXB_TRY(kv_sync_table(m));
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    OXB_TRY(encode_decode_step(m, false));
+    // the normed rows go through the gate || up buffer: free once the last layer is done, 2 * inter values per sequence
+    int rc = OXB_HIP_OK;
+    const float* final_norm = d.final_norm ? vec_ptr(d.final_norm, d.h, "final_norm", &rc) : nullptr;
+    if (rc) return rc;
+    float* dst = m.gu;
+    if ((size_t)2 * d.inter < d.h) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden %u exceeds 2 x intermediate %u", d.h, d.inter);
+    OXB_TRY_HIP(oxb_launch_rmsnorm(m.hidden, final_norm, d.h, d.batch, d.eps, dst, st), "kernel launch failed: rmsnorm");
+    for (uint32_t b = 0; b < d.batch; b++)
+        OXB_TRY_HIP(hipMemcpyAsync(normed_out + (size_t)b * d.h, dst + (size_t)b * d.h, (size_t)d.h * 4, hipMemcpyDeviceToHost, st),
+                    "hidden download");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode_hidden: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+    OXB_API_END
+}
+
+int oxb_hip_model_set_rope_rows(uint64_t model, uint32_t pos_start, uint32_t n_pos, const float* cos_rows, const float* sin_rows) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    if (!cos_rows || !sin_rows || n_pos == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null table or no positions");
+    if ((uint64_t)pos_start + n_pos > m.d.max_seq)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
+                    (unsigned long long)pos_start + n_pos - 1, m.d.max_seq);
+    const size_t half = m.d.hd / 2;
+    hipStream_t st = g_rt.stream;
+    // ordered on the stream behind every step already issued; pageable host memory is staged before the call returns
+    OXB_TRY_HIP(hipMemcpyAsync(m.cos_t + (size_t)pos_start * half, cos_rows, (size_t)n_pos * half * 4, hipMemcpyHostToDevice, st), "rope rows upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.sin_t + (size_t)pos_start * half, sin_rows, (size_t)n_pos * half * 4, hipMemcpyHostToDevice, st), "rope rows upload");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: rope rows: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
+    OXB_API_END
+}
+
 int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t n_tokens, uint32_t pos_start,
                     float* logits_or_null, uint32_t* token_out_or_null) {
     OXB_API_BEGIN
@@ -961,6 +1037,9 @@ int oxb_hip_prefill(uint64_t model, uint32_t seq, const float* hidden, uint32_t 
     Model& m = *mp;
     const oxb_model_desc& d = m.d;
     if (!hidden || n_tokens == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null hidden or no tokens");
+    if (!d.lm_head && (logits_or_null || token_out_or_null))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: the model has no LM head: logits and token must be null");
+    if (m.checked_gen != g_rt.weights_gen) OXB_TRY(check_model_handles(m));
     if (seq >= d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, d.batch);
     if ((uint64_t)pos_start + n_tokens > d.max_seq)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,
@@ -1236,6 +1315,9 @@ int oxb_hip_prefill_tokens(uint64_t model, uint64_t embedding, uint32_t seq, con
     Model& m = *mp;
     const oxb_model_desc& d = m.d;
     if (!ids || n_tokens == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null ids or no tokens");
+    if (!d.lm_head && (logits_or_null || token_out_or_null))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: the model has no LM head: logits and token must be null");
+    if (m.checked_gen != g_rt.weights_gen) OXB_TRY(check_model_handles(m));
     if (seq >= d.batch) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: sequence %u of a batch of %u", seq, d.batch);
     if ((uint64_t)pos_start + n_tokens > d.max_seq)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: positions %u..%llu exceed the context of %u", pos_start,

@@ -91,7 +91,78 @@ Weight* find_weight(uint64_t id) {
 
 static void free_weight_mem(Weight& w) {
     if (w.d_base) (void)hipFree(w.d_base);
+    if (w.d_raw) (void)hipFree(w.d_raw);
     w.d_base = nullptr;
+    w.d_raw = nullptr;
+}
+
+// Block bytes -> device, shape still open.
+static int upload_weight_bytes(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes) {
+    if (!id) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: id pointer is null");
+    const size_t bb = fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES;
+    if (!aos || n_bytes == 0 || n_bytes % bb != 0)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer of %zu bytes is not a whole number of %zu-byte blocks",
+                    n_bytes, bb);
+    int rc = ensure_init();
+    if (rc) return rc;
+    Weight w;
+    w.L = oxb_make_layout((uint32_t)fmt, 0, 0);
+    w.raw_blocks = n_bytes / bb;
+    hipError_t e = hipMalloc(&w.d_raw, n_bytes);
+    if (e != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", n_bytes, g_rt.device);
+    e = hipMemcpy(w.d_raw, aos, n_bytes, hipMemcpyHostToDevice);
+    if (e != hipSuccess) {
+        (void)hipFree(w.d_raw);
+        return hip_fail(e, "weight upload");
+    }
+    if (*id == 0) *id = g_rt.next_id++;
+    if (Weight* old = find_weight(*id)) {
+        (void)hipStreamSynchronize(g_rt.stream);  // a launch in flight may still read the old copy
+        free_weight_mem(*old);
+        g_rt.weights_gen++;
+    }
+    g_rt.weights[*id] = w;
+    return OXB_HIP_OK;
+}
+
+int bind_shape(Weight& w, uint32_t n_rows, uint32_t k) {
+    if (k == 0 || k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
+    if (!w.d_raw) {
+        if (w.L.n_rows != n_rows || w.L.k != k)
+            return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight is %ux%u, call asks for %ux%u", w.L.n_rows,
+                        w.L.k, n_rows, k);
+        return OXB_HIP_OK;
+    }
+    const size_t need = (size_t)n_rows * (k / OXB_QK);
+    if (n_rows == 0 || need != w.raw_blocks)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight holds %zu blocks, %ux%u needs %zu", w.raw_blocks,
+                    n_rows, k, need);
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(g_rt.stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+        return fail(OXB_HIP_INVALID_ARGUMENT,
+                    "invalid argument: a weight uploaded without a shape cannot be bound inside a stream capture; call once before capturing");
+    const OxbLayout L = oxb_make_layout(w.L.fmt, n_rows, k);
+    const size_t total = L.codes_bytes + L.scales_bytes;
+    void* base = nullptr;
+    hipError_t e = hipMalloc(&base, total);
+    if (e != hipSuccess)
+        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", total, g_rt.device);
+    uint32_t* codes = reinterpret_cast<uint32_t*>(base);
+    uint16_t* scales = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(base) + L.codes_bytes);
+    e = oxb_launch_repack(L, reinterpret_cast<const uint8_t*>(w.d_raw), codes, scales, g_rt.stream);
+    if (e == hipSuccess) e = hipStreamSynchronize(g_rt.stream);
+    if (e != hipSuccess) {
+        (void)hipFree(base);
+        return hip_fail(e, "kernel launch failed: repack");
+    }
+    (void)hipFree(w.d_raw);
+    w.d_raw = nullptr;
+    w.L = L;
+    w.d_base = base;
+    w.d_codes = codes;
+    w.d_scales = scales;
+    return OXB_HIP_OK;
 }
 
 int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k) {
@@ -103,33 +174,16 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
     const size_t need = (size_t)n_rows * (k / OXB_QK) * bb;
     if (!aos || n_bytes < need)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer holds %zu bytes, %zu needed", n_bytes, need);
-    int rc = ensure_init();
+    const uint64_t asked = *id;
+    int rc = upload_weight_bytes(id, fmt, aos, need);
     if (rc) return rc;
-
-    Weight w;
-    w.L = oxb_make_layout((uint32_t)fmt, n_rows, k);
-    const size_t total = w.L.codes_bytes + w.L.scales_bytes;
-    std::vector<uint8_t> host(total);
-    oxb_repack_aos_to_tiled(w.L, aos, reinterpret_cast<uint32_t*>(host.data()),
-                            reinterpret_cast<uint16_t*>(host.data() + w.L.codes_bytes));
-    hipError_t e = hipMalloc(&w.d_base, total);
-    if (e != hipSuccess)
-        return fail(OXB_HIP_OUT_OF_MEMORY, "out of device memory: requested %zu bytes on device %d", total, g_rt.device);
-    e = hipMemcpy(w.d_base, host.data(), total, hipMemcpyHostToDevice);
-    if (e != hipSuccess) {
-        (void)hipFree(w.d_base);
-        return hip_fail(e, "weight upload");
+    rc = bind_shape(*find_weight(*id), n_rows, k);
+    if (rc) {
+        free_weight_mem(*find_weight(*id));
+        g_rt.weights.erase(*id);
+        *id = asked;
     }
-    w.d_codes = reinterpret_cast<uint32_t*>(w.d_base);
-    w.d_scales = reinterpret_cast<uint16_t*>(reinterpret_cast<uint8_t*>(w.d_base) + w.L.codes_bytes);
-    if (*id == 0) *id = g_rt.next_id++;
-    if (Weight* old = find_weight(*id)) {
-        (void)hipStreamSynchronize(g_rt.stream);  // a launch in flight may still read the old copy
-        free_weight_mem(*old);
-        g_rt.weights_gen++;
-    }
-    g_rt.weights[*id] = w;
-    return OXB_HIP_OK;
+    return rc;
 }
 
 // One GEMV over resident weights, any K: launches of at most OXB_GEMV_MAX_SB superblocks, the first with the wanted
@@ -215,14 +269,6 @@ int gemm_device(const Weight& w, const float* d_x, uint32_t ldx, float* d_y, uin
     }
     e = oxb_launch_gemm((int)w.L.fmt, p, g_rt.n_cus, g_rt.stream);
     if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemm");
-    return OXB_HIP_OK;
-}
-
-static int check_shape(const Weight& w, uint32_t n_rows, uint32_t k) {
-    if (k % OXB_QK != 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: k=%u is not a multiple of 128", k);
-    if (w.L.n_rows != n_rows || w.L.k != k)
-        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight is %ux%u, call asks for %ux%u", w.L.n_rows,
-                    w.L.k, n_rows, k);
     return OXB_HIP_OK;
 }
 
@@ -363,6 +409,20 @@ int oxb_hip_upload_tq2(uint64_t* id, const uint8_t* aos, size_t n_bytes, uint32_
     OXB_API_END
 }
 
+int oxb_hip_upload_q1_raw(uint64_t* id, const uint8_t* aos, size_t n_bytes) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return upload_weight_bytes(id, OXB_FMT_Q1, aos, n_bytes);
+    OXB_API_END
+}
+
+int oxb_hip_upload_tq2_raw(uint64_t* id, const uint8_t* aos, size_t n_bytes) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    return upload_weight_bytes(id, OXB_FMT_TQ2, aos, n_bytes);
+    OXB_API_END
+}
+
 int oxb_hip_free_weight(uint64_t id) {
     OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
@@ -384,7 +444,9 @@ int oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, si
     if (fmt) *fmt = (int)w->L.fmt;
     if (n_rows) *n_rows = w->L.n_rows;
     if (k) *k = w->L.k;
-    if (resident_bytes) *resident_bytes = w->L.codes_bytes + w->L.scales_bytes;
+    if (resident_bytes)
+        *resident_bytes = w->d_raw ? w->raw_blocks * (w->L.fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES)
+                                   : w->L.codes_bytes + w->L.scales_bytes;
     return OXB_HIP_OK;
     OXB_API_END
 }
@@ -394,6 +456,9 @@ int oxb_hip_dequant(uint64_t id, float* out, size_t out_len) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
+    if (w->d_raw)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight %llu was uploaded without a shape and no call has named one yet",
+                    (unsigned long long)id);
     const size_t n = (size_t)w->L.n_rows * w->L.k;
     if (!out || out_len < n) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: output holds %zu values, %zu needed", out_len, n);
     int rc = g_rt.ws_y.ensure(n * sizeof(float));
@@ -411,7 +476,7 @@ int oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows,
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!d_x || !d_y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
     return gemv_device(*w, d_x, d_y, batch, n_rows, OXB_GEMV_STORE, nullptr);
@@ -427,7 +492,7 @@ static int profile_gemv_impl(bool floor_only, const uint64_t* ids, uint32_t n_id
     for (uint32_t i = 0; i < n_ids; i++) {
         Weight* w = find_weight(ids[i]);
         if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)ids[i]);
-        int rc = check_shape(*w, n_rows, k);
+        int rc = bind_shape(*w, n_rows, k);
         if (rc) return rc;
         if (!ws.empty() && w->L.fmt != ws[0]->L.fmt)
             return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weights differ in format");
@@ -499,7 +564,7 @@ int oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
     return gemm_device(*w, d_x, k, d_y, m, n_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_IDENT, nullptr, 0.f);
@@ -511,7 +576,10 @@ int oxb_hip_gemm_dev_static(uint64_t id, const float* d_x, float* d_y, uint32_t 
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    if (w->d_raw)  // binding a shape allocates the resident copy: not in this entry point
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight %llu was uploaded without a shape; name its shape in another call first",
+                    (unsigned long long)id);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!d_x || !d_y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
     if (!g_rt.ready || !g_rt.static_scratch) return fail(OXB_HIP_NOT_AVAILABLE, "GPU not available: the library is not initialised");
@@ -548,7 +616,7 @@ int oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_r
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!x || !y || m == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or m = 0");
     const size_t xb = (size_t)m * k * sizeof(float), yb = (size_t)m * n_rows * sizeof(float);
@@ -570,7 +638,7 @@ int oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, 
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!d_x || !d_y || !avg_us || m == 0 || iters == 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or zero count");
@@ -622,7 +690,7 @@ int oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Weight* w = find_weight(id);
     if (!w) return fail(OXB_HIP_WEIGHT_NOT_FOUND, "weight handle %llu not found", (unsigned long long)id);
-    int rc = check_shape(*w, n_rows, k);
+    int rc = bind_shape(*w, n_rows, k);
     if (rc) return rc;
     if (!x || !y || batch == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer or batch 0");
     const size_t xb = (size_t)batch * k * sizeof(float), yb = (size_t)batch * n_rows * sizeof(float);

@@ -28,11 +28,16 @@ struct GemmWorkspace {
     void release() { xh.release(); xsh.release(); rowmul.release(); part.release(); }
 };
 
-struct Weight {  // one resident matrix: [codes section][scales section]
+// One resident matrix: [codes section][scales section].  A weight uploaded as bytes alone (the reference's
+// upload_weights_raw / upload_weights_ternary carry no shape) waits as a device copy of those bytes, d_raw, with
+// L.n_rows == 0, until the first call that names (n_rows, k) binds the shape and repacks it on the device.
+struct Weight {
     OxbLayout L;
     void* d_base = nullptr;
     uint32_t* d_codes = nullptr;
     uint16_t* d_scales = nullptr;
+    void* d_raw = nullptr;
+    size_t raw_blocks = 0;
 };
 
 struct Vector {  // a resident fp32 vector (norm weights)
@@ -66,6 +71,9 @@ int hip_fail(hipError_t e, const char* what);
 int ensure_init();
 Weight* find_weight(uint64_t id);
 int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uint32_t n_rows, uint32_t k);
+// Holds the weight to (n_rows, k): binds and repacks one that has no shape yet (never inside a stream capture), else
+// compares.
+int bind_shape(Weight& w, uint32_t n_rows, uint32_t k);
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual);
 // nvec <= OXB_GEMV_MAX_BATCH vectors x [nvec][ldx] through one pass over the weights: pro / epi are OXB_GEMV_PRO_* /

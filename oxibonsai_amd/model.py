@@ -149,10 +149,15 @@ class HipModel:
     """cfg: fmt, n_layers, h, inter, nq, nkv, hd, vocab, max_seq, eps, rope_theta.
     weights: dict of oxibonsai_amd.synth.make_model (reference AoS blocks + f32 norm vectors)."""
 
-    def __init__(self, backend: NativeHipBackend, cfg: dict, weights: dict, batch: int = 1):
+    def __init__(self, backend: NativeHipBackend, cfg: dict, weights: dict, batch: int = 1, lm_head: bool = True,
+                 shaped_uploads: bool = True):
+        """lm_head=False builds the model of try_cuda_full_forward (no LM head on the device: forward_hidden only);
+        shaped_uploads=False uploads every matrix as bytes alone, as the reference's callers do, and lets the model's
+        dimensions give them their shapes."""
         self.be, self.cfg, self.batch = backend, cfg, batch
         self._lib = _lib.lib()
         self._mats, self._vecs = [], []
+        self._shaped, self._has_lm = shaped_uploads, lm_head
         fmt, h, inter, hd = cfg["fmt"], cfg["h"], cfg["inter"], cfg["hd"]
         qd, kd = cfg["nq"] * hd, cfg["nkv"] * hd
         ids = (_LayerIds * cfg["n_layers"])()
@@ -165,7 +170,7 @@ class HipModel:
         self._ids = ids
         desc = _ModelDesc(fmt, cfg["n_layers"], h, inter, cfg["nq"], cfg["nkv"], hd, cfg["vocab"], cfg["max_seq"], batch,
                           cfg["eps"], cfg["rope_theta"], ids, self._vec(weights["final_norm"]),
-                          self._mat(weights["lm_head"], cfg["vocab"], h))
+                          self._mat(weights["lm_head"], cfg["vocab"], h) if lm_head else 0)
         mid = C.c_uint64(0)
         _check(self._lib.oxb_hip_model_create(C.byref(desc), C.byref(mid)))
         self.id = mid.value
@@ -178,6 +183,7 @@ class HipModel:
         self.be, self.batch = backend, batch
         self._lib = _lib.lib()
         self._mats, self._vecs = [], []
+        self._shaped, self._has_lm = True, True
         info, mid, eid = GgufInfo(), C.c_uint64(0), C.c_uint64(0)
         _check(self._lib.oxb_hip_load_gguf(str(path).encode(), max_seq, batch, C.byref(mid), C.byref(eid), C.byref(info)))
         d = info.as_dict()
@@ -188,7 +194,8 @@ class HipModel:
 
     def _mat(self, blocks, n_rows, k):
         fmt = self.cfg["fmt"]
-        h = self.be.upload_weights_raw(blocks, n_rows, k) if fmt == Q1 else self.be.upload_weights_ternary(blocks, n_rows, k)
+        shape = (n_rows, k) if self._shaped else (None, None)
+        h = self.be.upload_weights_raw(blocks, *shape) if fmt == Q1 else self.be.upload_weights_ternary(blocks, *shape)
         self._mats.append(h)
         return int(h)
 
@@ -210,6 +217,26 @@ class HipModel:
                                         tokens.ctypes.data_as(_lib.u32p)))
         return logits, tokens
 
+    def forward_hidden(self, hidden, pos) -> np.ndarray:
+        """All layers and the final norm, no LM head (try_cuda_full_forward, gpu_backend/cuda_full_layer/encode_q1.rs:813):
+        hidden [batch, h], pos [batch] -> normed hidden state [batch, h]."""
+        hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(self.batch, self.cfg["h"])
+        pv = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, dtype=np.uint32), (self.batch,)))
+        out = np.empty((self.batch, self.cfg["h"]), dtype=np.float32)
+        _check(self._lib.oxb_hip_decode_hidden(self.id, hv.ctypes.data_as(_lib.f32p), pv.ctypes.data_as(_lib.u32p),
+                                               out.ctypes.data_as(_lib.f32p)))
+        return out
+
+    def set_rope_rows(self, pos_start: int, cos_rows, sin_rows):
+        """The caller's own RoPE rows ([n_pos, hd/2] each) for positions pos_start.., as the reference's entry points
+        receive them (rope_cos / rope_sin, cos_table / sin_table)."""
+        c = np.ascontiguousarray(cos_rows, dtype=np.float32).reshape(-1, self.cfg["hd"] // 2)
+        s = np.ascontiguousarray(sin_rows, dtype=np.float32).reshape(-1, self.cfg["hd"] // 2)
+        if c.shape != s.shape:
+            raise ValueError("cos and sin rows differ in shape")
+        _check(self._lib.oxb_hip_model_set_rope_rows(self.id, pos_start, c.shape[0], c.ctypes.data_as(_lib.f32p),
+                                                     s.ctypes.data_as(_lib.f32p)))
+
     def prefill(self, hidden, pos_start: int = 0, seq: int = 0, want_logits: bool = True):
         """Batched prefill of one sequence (try_cuda_prefill, gpu_backend/cuda_prefill/try_apis.rs:42, 318).
         hidden: [n_tokens, h] embedding rows for positions pos_start.. -> (last-token logits [vocab] or None,
@@ -219,8 +246,8 @@ class HipModel:
         token = np.empty(1, dtype=np.uint32)
         _check(self._lib.oxb_hip_prefill(self.id, seq, hv.ctypes.data_as(_lib.f32p), hv.shape[0], pos_start,
                                          logits.ctypes.data_as(_lib.f32p) if want_logits else None,
-                                         token.ctypes.data_as(_lib.u32p)))
-        return logits, int(token[0])
+                                         token.ctypes.data_as(_lib.u32p) if self._has_lm else None))
+        return logits, (int(token[0]) if self._has_lm else None)
 
     def generate(self, embedding: Embedding, tokens, pos, n_steps: int) -> np.ndarray:
         """Greedy decode of n_steps tokens per sequence without a host round trip per token: tokens [batch] are fed
