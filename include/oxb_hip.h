@@ -123,6 +123,13 @@ int  oxb_hip_gemm_dev_static(uint64_t id, const float* d_x, float* d_y, uint32_t
 int  oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float* norm_w, float eps,
                        uint64_t o_id, uint64_t gate_up_id, uint64_t down_id, uint32_t h, uint32_t inter, uint32_t attn_k);
 
+/* ---- batch_attn_phase (KG/mod.rs:501-512; the Metal tier's implementation: KG/scirs2_backend.rs:1187-1232):
+ * normed = RMSNorm(hidden, norm_w, eps); [q | k | v] = qkv * normed in one launch; q receives q_rows values, k and v
+ * k_rows each.  The reference's dispatcher keeps this phase switched off (crates/oxibonsai-kernels/src/dispatch.rs:605-621)
+ * and its CUDA tier leaves the trait default (Ok(None)); offered so that the trait binds completely. */
+int  oxb_hip_attn_phase(int fmt, const float* hidden, const float* norm_w, float eps, uint64_t qkv_id, uint32_t q_rows,
+                        uint32_t k_rows, uint32_t h, float* q, float* k, float* v);
+
 /* ---- fused whole-model decode: try_cuda_full_forward[_ternary]_with_gpu_lm_head
  * (KG/cuda_full_layer/encode_q1.rs:881-900, encode_ternary.rs:755-774) with per-layer parameters as in
  * CudaFullForwardLayerParams (KG/cuda_full_layer/mod.rs:250-268): norm vectors and weight matrices are named by
@@ -155,6 +162,11 @@ int  oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, fl
  * the final RMSNorm (final_norm_bytes: Option - a model created with final_norm == 0 returns the un-normed state);
  * the caller runs its own LM head.  normed_out: [batch][h].  Plain launches, no graph. */
 int  oxb_hip_decode_hidden(uint64_t model, const float* hidden, const uint32_t* pos, float* normed_out);
+/* Gives a model its final norm vector and LM head after the fact, or other ones (lm_head == 0 takes the LM head away).
+ * The reference's entry points name them per call (final_norm_handle, lm_head_handle, lm_head_bytes, vocab_size,
+ * encode_q1.rs:881-900), and try_cuda_full_forward_with_gpu_lm_head continues on the cache try_cuda_full_forward
+ * filled: the KV cache and the positions decoded so far stay as they are. */
+int  oxb_hip_model_set_lm_head(uint64_t model, uint64_t final_norm, uint64_t lm_head, uint32_t vocab);
 /* The reference's entry points receive the RoPE rows of their positions from the caller (rope_cos / rope_sin of `pos`,
  * hd/2 values each, encode_q1.rs:816-817; cos_table / sin_table [batch_size][hd/2] for a prefill, KG/cuda_prefill/try_apis.rs:48-49).
  * This call stores such rows for positions pos_start .. pos_start + n_pos - 1 in the model's table, in place of the

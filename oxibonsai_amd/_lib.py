@@ -46,6 +46,7 @@ _SIGNATURES = {
     "oxb_hip_gemv_tq2_g128": ([u8p, C.c_size_t, f32p, C.c_size_t, f32p, C.c_size_t, C.c_uint32, C.c_uint32], C.c_int),
     "oxb_hip_ffn_phase": ([C.c_int, f32p, f32p, f32p, C.c_float, C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32,
                            C.c_uint32, C.c_uint32], C.c_int),
+    "oxb_hip_attn_phase": ([C.c_int, f32p, f32p, C.c_float, C.c_uint64, C.c_uint32, C.c_uint32, C.c_uint32, f32p, f32p, f32p], C.c_int),
     "oxb_hip_upload_f32": ([u64p, f32p, C.c_size_t], C.c_int),
     "oxb_hip_free_f32": ([C.c_uint64], C.c_int),
     "oxb_hip_model_create": ([C.c_void_p, u64p], C.c_int),
@@ -53,6 +54,7 @@ _SIGNATURES = {
     "oxb_hip_model_destroy": ([C.c_uint64], C.c_int),
     "oxb_hip_decode": ([C.c_uint64, f32p, u32p, f32p, u32p], C.c_int),
     "oxb_hip_decode_hidden": ([C.c_uint64, f32p, u32p, f32p], C.c_int),
+    "oxb_hip_model_set_lm_head": ([C.c_uint64, C.c_uint64, C.c_uint64, C.c_uint32], C.c_int),
     "oxb_hip_model_set_rope_rows": ([C.c_uint64, C.c_uint32, C.c_uint32, f32p, f32p], C.c_int),
     "oxb_hip_prefill": ([C.c_uint64, C.c_uint32, f32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_model_uses_graph": ([C.c_uint64], C.c_int),

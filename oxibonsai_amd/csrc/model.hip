@@ -59,6 +59,7 @@ struct Model {
     uint64_t graph_gen = 0;  // g_rt.weights_gen at capture: the graph holds the weights' device pointers of that moment
     bool graph_failed = false;
     bool want_logits_in_graph = true;
+    size_t logits_cap = 0;  // floats m.logits holds
     std::vector<void*> allocs;
     // prefill activations for up to pf_cap token rows (allocated on first use)
     uint32_t pf_cap = 0;
@@ -190,6 +191,11 @@ static int encode_ffn(float* hidden, const float* attn_out, const float* ffn_nor
     return OXB_HIP_OK;
 }
 
+// Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
+// matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
+// the weights once per four sequences.
+#define OXB_DECODE_GEMM_MIN_BATCH (OXB_GEMV_MAX_BATCH + 1)
+
 // Looks every handle of the model up with the shape the model needs (which also binds a weight that was uploaded
 // without one).  Run at creation and again whenever a weight or vector was replaced or freed since, before a decode
 // step is captured: inside the capture nothing may allocate.
@@ -212,6 +218,38 @@ static int check_model_handles(Model& m) {
     if (!rc && d.lm_head) mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
     if (!rc) m.checked_gen = g_rt.weights_gen;
     return rc;
+}
+
+// The GEMM-based decode step of a large batch is captured into a graph: its GEMM workspaces are sized here, before any
+// capture, for every projection shape of the model (the LM head included when there is one).
+static int size_gemm_workspaces(Model& m) {
+    const oxb_model_desc& d = m.d;
+    if (d.batch < OXB_DECODE_GEMM_MIN_BATCH) return OXB_HIP_OK;
+    const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    uint32_t kx = d.h > d.inter ? d.h : d.inter;
+    if (qd > kx) kx = qd;
+    size_t part_bytes = 0;
+    const struct { uint64_t id; uint32_t n, k; } shapes[] = {{m.layers[0].qkv, qkv_rows, d.h}, {m.layers[0].o, d.h, qd},
+                                                             {m.layers[0].gate_up, 2 * d.inter, d.h},
+                                                             {m.layers[0].down, d.h, d.inter}, {d.lm_head, d.vocab, d.h}};
+    for (const auto& sh : shapes) {
+        const Weight* w = find_weight(sh.id);
+        if (!w) continue;  // a model without an LM head
+        OxbGemmParams gp;
+        memset(&gp, 0, sizeof gp);
+        gp.n_rows = sh.n;
+        gp.n_tiles = w->L.n_tiles;
+        gp.n_sb = w->L.n_sb;
+        gp.M = d.batch;
+        gp.ldy = sh.n;
+        const size_t b = (size_t)oxb_gemm_ksplit(gp, g_rt.n_cus) * d.batch * sh.n * sizeof(float);
+        if (oxb_gemm_ksplit(gp, g_rt.n_cus) > 1 && b > part_bytes) part_bytes = b;
+    }
+    int rc;
+    if ((rc = m.gws.xh.ensure(oxb_xh_bytes(kx, d.batch))) || (rc = m.gws.xsh.ensure(((size_t)d.batch + 16) * 4)) ||
+        (rc = m.gws.rowmul.ensure(((size_t)d.batch + 16) * 4)) || (part_bytes && (rc = m.gws.part.ensure(part_bytes))))
+        return rc;
+    return OXB_HIP_OK;
 }
 
 static OxbKvLayout kv_layout(const Model& m) {
@@ -301,10 +339,6 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     return OXB_HIP_OK;
 }
 
-// Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
-// matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
-// the weights once per four sequences.
-#define OXB_DECODE_GEMM_MIN_BATCH (OXB_GEMV_MAX_BATCH + 1)
 
 static int encode_decode_step_gemm(Model& m) {
     const oxb_model_desc& d = m.d;
@@ -677,33 +711,11 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
             return hip_fail(e, "rope table upload");
         }
     }
-    if (d.batch >= OXB_DECODE_GEMM_MIN_BATCH) {
-        // the GEMM-based decode step is captured into a graph: size the library's GEMM workspaces now
-        uint32_t kx = d.h > d.inter ? d.h : d.inter;
-        if (qd > kx) kx = qd;
-        size_t part_bytes = 0;
-        const struct { uint64_t id; uint32_t n, k; } shapes[] = {{m.layers[0].qkv, qkv_rows, d.h}, {m.layers[0].o, d.h, qd},
-                                                                 {m.layers[0].gate_up, 2 * d.inter, d.h},
-                                                                 {m.layers[0].down, d.h, d.inter}, {d.lm_head, d.vocab, d.h}};
-        for (const auto& sh : shapes) {
-            const Weight* w = find_weight(sh.id);
-            if (!w) continue;  // a model without an LM head
-            OxbGemmParams gp;
-            memset(&gp, 0, sizeof gp);
-            gp.n_rows = sh.n;
-            gp.n_tiles = w->L.n_tiles;
-            gp.n_sb = w->L.n_sb;
-            gp.M = d.batch;
-            gp.ldy = sh.n;
-            const size_t b = (size_t)oxb_gemm_ksplit(gp, g_rt.n_cus) * d.batch * sh.n * sizeof(float);
-            if (oxb_gemm_ksplit(gp, g_rt.n_cus) > 1 && b > part_bytes) part_bytes = b;
-        }
-        if ((rc = m.gws.xh.ensure(oxb_xh_bytes(kx, d.batch))) || (rc = m.gws.xsh.ensure(((size_t)d.batch + 16) * 4)) ||
-            (rc = m.gws.rowmul.ensure(((size_t)d.batch + 16) * 4)) || (part_bytes && (rc = m.gws.part.ensure(part_bytes)))) {
-            free_model(m);
-            return rc;
-        }
+    if ((rc = size_gemm_workspaces(m))) {
+        free_model(m);
+        return rc;
     }
+    m.logits_cap = B * (d.lm_head ? d.vocab : 1);
     const char* no_graph = getenv("OXB_HIP_DISABLE_GRAPH");
     m.graph_failed = no_graph && no_graph[0] == '1';
     *model = g_next_model++;
@@ -973,6 +985,38 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     OXB_API_END
 }
 
+int oxb_hip_model_set_lm_head(uint64_t model, uint64_t final_norm, uint64_t lm_head, uint32_t vocab) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    Model* mp = find_model(model);
+    if (!mp) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: unknown model %llu", (unsigned long long)model);
+    Model& m = *mp;
+    if (lm_head && (!final_norm || !vocab))
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: an LM head needs the final norm vector and a vocabulary size");
+    int rc = OXB_HIP_OK;
+    if (final_norm) vec_ptr(final_norm, m.d.h, "final_norm", &rc);
+    if (!rc && lm_head) mat_ptr(lm_head, m.d.fmt, vocab, m.d.h, "lm_head", &rc);
+    if (rc) return rc;
+    OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "synchronize");
+    if (m.graph_exec) {  // the captured step ends in the old LM head (or in none)
+        (void)hipGraphExecDestroy(m.graph_exec);
+        m.graph_exec = nullptr;
+    }
+    const size_t need = (size_t)m.d.batch * (lm_head ? vocab : 1);
+    if (need > m.logits_cap) {
+        float* p = nullptr;
+        OXB_TRY(dev_alloc(m, (void**)&p, need * 4));  // the smaller buffer stays with the model until it is destroyed
+        m.logits = p;
+        m.logits_cap = need;
+    }
+    m.d.final_norm = final_norm;
+    m.d.lm_head = lm_head;
+    m.d.vocab = lm_head ? vocab : 0;
+    OXB_TRY(size_gemm_workspaces(m));
+    return check_model_handles(m);
+    OXB_API_END
+}
+
 int oxb_hip_decode_hidden(uint64_t model, const float* hidden, const uint32_t* pos, float* normed_out) {
     OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);
@@ -1064,6 +1108,34 @@ int oxb_hip_model_uses_graph(uint64_t model) {
     std::lock_guard<std::recursive_mutex> lk(g_mu);
     Model* m = find_model(model);
     return m && m->graph_exec ? 1 : 0;
+    OXB_API_END
+}
+
+int oxb_hip_attn_phase(int fmt, const float* hidden, const float* norm_w, float eps, uint64_t qkv_id, uint32_t q_rows,
+                       uint32_t k_rows, uint32_t h, float* q, float* k, float* v) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!hidden || !norm_w || !q || !k || !v) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
+    if (h % 128 || q_rows == 0 || k_rows == 0) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: h must be a multiple of 128, row counts non-zero");
+    const uint32_t rows = q_rows + 2 * k_rows;
+    int rc = OXB_HIP_OK;
+    const Weight* w = mat_ptr(qkv_id, fmt, rows, h, "qkv", &rc);
+    if (rc) return rc;
+    OXB_TRY(g_rt.ws_x.ensure((size_t)h * 2 * 4));
+    OXB_TRY(g_rt.ws_y.ensure((size_t)rows * 4));
+    float* d_hidden = (float*)g_rt.ws_x.ptr;
+    float* d_norm = d_hidden + h;
+    float* d_qkv = (float*)g_rt.ws_y.ptr;
+    hipStream_t st = g_rt.stream;
+    OXB_TRY_HIP(hipMemcpyAsync(d_hidden, hidden, (size_t)h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(d_norm, norm_w, (size_t)h * 4, hipMemcpyHostToDevice, st), "norm upload");
+    OXB_TRY(gemv_launch(*w, d_hidden, h, 1, d_qkv, rows, OXB_GEMV_PRO_RMSNORM, d_norm, eps, OXB_GEMV_STORE, nullptr));
+    OXB_TRY_HIP(hipMemcpyAsync(q, d_qkv, (size_t)q_rows * 4, hipMemcpyDeviceToHost, st), "q download");
+    OXB_TRY_HIP(hipMemcpyAsync(k, d_qkv + q_rows, (size_t)k_rows * 4, hipMemcpyDeviceToHost, st), "k download");
+    OXB_TRY_HIP(hipMemcpyAsync(v, d_qkv + q_rows + k_rows, (size_t)k_rows * 4, hipMemcpyDeviceToHost, st), "v download");
+    hipError_t e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: attn_phase: %s", hipGetErrorString(e));
+    return OXB_HIP_OK;
     OXB_API_END
 }
 

@@ -227,6 +227,15 @@ class HipModel:
                                                out.ctypes.data_as(_lib.f32p)))
         return out
 
+    def set_lm_head(self, final_norm, lm_head_blocks, vocab: int):
+        """Attach (or replace) the final norm vector and the LM head of a live model; the KV cache stays.
+        lm_head_blocks None takes the LM head away."""
+        fn = self._vec(final_norm) if final_norm is not None else 0
+        lm = self._mat(lm_head_blocks, vocab, self.cfg["h"]) if lm_head_blocks is not None else 0
+        _check(self._lib.oxb_hip_model_set_lm_head(self.id, fn, lm, vocab if lm else 0))
+        self._has_lm = bool(lm)
+        self.cfg = dict(self.cfg, vocab=vocab)
+
     def set_rope_rows(self, pos_start: int, cos_rows, sin_rows):
         """The caller's own RoPE rows ([n_pos, hd/2] each) for positions pos_start.., as the reference's entry points
         receive them (rope_cos / rope_sin, cos_table / sin_table)."""
@@ -351,3 +360,17 @@ def batch_ffn_phase(backend: NativeHipBackend, fmt: int, hidden, attn_out, norm_
                                         nv.ctypes.data_as(_lib.f32p), norm_eps, int(attn_proj_handle),
                                         int(gate_up_handle), int(down_handle), h, intermediate, attn_proj_k))
     return hv
+
+
+def batch_attn_phase(backend: NativeHipBackend, fmt: int, hidden, norm_weight, norm_eps: float, qkv_handle: int,
+                     q_rows: int, k_rows: int, h: int):
+    """GpuBackendTrait::batch_attn_phase (gpu_backend/mod.rs:501): RMSNorm + fused QKV product -> (q, k, v)."""
+    hv = np.ascontiguousarray(hidden, dtype=np.float32)
+    nv = np.ascontiguousarray(norm_weight, dtype=np.float32)
+    if hv.size < h or nv.size < h:
+        raise GpuError(5, "invalid argument: buffer shorter than its dimension")
+    q, k, v = (np.empty(n, dtype=np.float32) for n in (q_rows, k_rows, k_rows))
+    _check(_lib.lib().oxb_hip_attn_phase(fmt, hv.ctypes.data_as(_lib.f32p), nv.ctypes.data_as(_lib.f32p), norm_eps,
+                                         int(qkv_handle), q_rows, k_rows, h, q.ctypes.data_as(_lib.f32p),
+                                         k.ctypes.data_as(_lib.f32p), v.ctypes.data_as(_lib.f32p)))
+    return q, k, v

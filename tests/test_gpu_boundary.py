@@ -204,3 +204,49 @@ def test_rope_rows_come_from_the_caller(backend):
     finally:
         good.close()
         late.close()
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+def test_lm_head_joins_a_live_model(backend, fmt):
+    """try_cuda_full_forward_with_gpu_lm_head continues on the cache try_cuda_full_forward filled
+    (gpu_backend/cuda_full_layer/encode_q1.rs:881-900): positions 0..3 run without an LM head, then the head is
+    attached and position 4 must give the logits of a model that had it from the start, bit for bit."""
+    cfg = dict(CFG, fmt=fmt)
+    w = synth.make_model(cfg, 0x1A0 + fmt)
+    rows = synth.embedding_rows(21, range(6), cfg["h"]) * 50.0
+    a, b = HipModel(backend, cfg, w, lm_head=False), HipModel(backend, cfg, w)
+    try:
+        for pos in range(4):
+            a.forward_hidden(rows[pos], pos)
+            b.forward(rows[pos], pos)
+        a.set_lm_head(w["final_norm"], w["lm_head"], cfg["vocab"])
+        for pos in range(4, 6):
+            ga, ta = a.forward(rows[pos], pos)
+            gb, tb = b.forward(rows[pos], pos)
+            assert np.array_equal(ga, gb) and np.array_equal(ta, tb)
+        assert a.uses_graph()
+        a.set_lm_head(None, None, 0)
+        with pytest.raises(GpuError):
+            a.forward(rows[0], 6)
+    finally:
+        a.close()
+        b.close()
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+def test_batch_attn_phase(backend, fmt):
+    """RMSNorm + fused QKV product in one launch, against the oracle's RMSNorm and GEMV."""
+    from oxibonsai_amd.model import batch_attn_phase
+    h, qr, kr = 1024, 512, 256
+    a = synth.make_blocks(fmt, 0xA77 + fmt, qr + 2 * kr, h)
+    x = synth.normal_f32(0xA78, h)
+    nw = (1.0 + synth.normal_f32(0xA79, h, 0.02)).astype(np.float32)
+    hd = _upload(backend, fmt, a)
+    try:
+        q, k, v = batch_attn_phase(backend, fmt, x, nw, 1e-6, hd, qr, kr, h)
+        normed = oracle.rms_norm(x, nw, 1e-6)
+        want = oracle.gemv(fmt, a, normed, qr + 2 * kr, h)
+        got = np.concatenate([q, k, v])
+        assert np.max(np.abs(got - want)) < 2e-5 * float(np.max(np.abs(want)))
+    finally:
+        backend.free_weights(hd)

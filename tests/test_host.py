@@ -163,3 +163,63 @@ def test_ctypes_structs_match_the_header_layout(tmp_path):
         assert int(seen[cname]) == C.sizeof(cls), cname
         for fname, _ in cls._fields_:
             assert int(seen[f"{cname}.{fname}"]) == getattr(cls, fname).offset, (cname, fname)
+
+
+def _c_decls(text):
+    """name -> (parameter count, return type) of every oxb_hip_* prototype in the header."""
+    text = re.sub(r"/\*.*?\*/", " ", text, flags=re.S)
+    out = {}
+    for ret, name, args in re.findall(r"\b(int|void|const char\*)\s+(oxb_hip_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        args = args.strip()
+        out[name] = (0 if args in ("", "void") else args.count(",") + 1, ret)
+    return out
+
+
+def _rust_decls(text):
+    text = re.sub(r"//[^\n]*", " ", text)
+    out = {}
+    for name, args, ret in re.findall(r"pub fn (oxb_hip_[a-z0-9_]+)\s*\(([^)]*)\)\s*(->\s*[^;]+)?;", text):
+        args = args.strip().rstrip(",")
+        out[name] = (0 if not args else args.count(",") + 1, ret.replace("->", "").strip() if ret else "void")
+    return out
+
+
+def test_rust_overlay_declares_the_header_one_for_one():
+    """rust/native_hip/ffi.rs is what a maintainer links against liboxb_hip.a: every prototype of the header must be
+    there under the same name with the same number of parameters and the matching return type, and nothing else."""
+    c = _c_decls(open(os.path.join(ROOT, "include", "oxb_hip.h")).read())
+    r = _rust_decls(open(os.path.join(ROOT, "rust", "native_hip", "ffi.rs")).read())
+    assert set(c) == set(r), set(c) ^ set(r)
+    ret_map = {"int": "c_int", "void": "void", "const char*": "*const c_char"}
+    for name, (n, ret) in c.items():
+        assert r[name] == (n, ret_map[ret]), (name, c[name], r[name])
+
+
+def test_rust_overlay_mirrors_the_reference_signatures():
+    """The fused entry points keep the reference's parameter names in the reference's order (read from
+    gpu_backend/cuda_full_layer/encode_q1.rs:813-900, encode_ternary.rs:694-774, cuda_prefill/try_apis.rs:42-66,
+    cuda_graph/functions.rs:76-145)."""
+    src = open(os.path.join(ROOT, "rust", "native_hip", "full_forward.rs")).read() + open(os.path.join(ROOT, "rust", "native_hip", "prefill.rs")).read()
+
+    def params(fn):
+        m = re.search(r"pub fn %s\s*\((.*?)\)\s*->" % fn, src, flags=re.S)
+        assert m, fn
+        return [p.split(":")[0].strip() for p in m.group(1).split(",\n") if p.strip()]
+
+    forward = ["hidden", "layer_params", "rope_cos", "rope_sin", "pos", "nq", "nkv", "head_dim", "heads_per_group", "norm_eps",
+               "hidden_size", "intermediate_size", "max_seq_len", "final_norm_bytes", "final_norm_handle"]
+    lm = ["lm_head_handle", "lm_head_bytes", "vocab_size"]
+    assert params("try_hip_full_forward") == forward
+    assert params("try_hip_full_forward_ternary") == forward
+    assert params("try_hip_full_forward_with_gpu_lm_head") == forward + lm
+    assert params("try_hip_full_forward_ternary_with_gpu_lm_head") == forward + lm
+    prefill = ["hidden_batch", "batch_size", "pos_start", "n_layers", "layer_params", "cos_table", "sin_table", "hidden_size",
+               "intermediate_size", "nq", "nkv", "head_dim", "heads_per_group", "eps", "max_seq_len", "final_norm_handle",
+               "final_norm_bytes", "final_norm_eps", "lm_head_handle", "lm_head_bytes", "lm_head_out_features", "logits_out",
+               "greedy_token_id_out"]
+    assert params("try_hip_prefill") == prefill
+    assert params("try_hip_prefill_ternary") == prefill
+    assert params("try_hip_ffn") == ["hidden", "attn_out", "norm_weight", "eps", "attn_proj_handle_id", "attn_proj_bytes",
+                                     "gate_up_handle_id", "gate_bytes", "up_bytes", "down_handle_id", "down_bytes", "hidden_size",
+                                     "intermediate_size"]
+    assert params("try_hip_qkv") == ["input", "output", "weight_handle_id", "q_bytes", "k_bytes", "v_bytes", "n_rows", "k"]
