@@ -384,6 +384,8 @@ def main() -> int:
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-decode", action="store_true", help="skip the 8B-shape decode leg")
     ap.add_argument("--no-prefill-gemm", action="store_true", help="skip the prefill GEMM leg")
+    ap.add_argument("--no-batch8", action="store_true",
+                    help="skip the batch-8 run of the set (counter runs: its launches carry the same kernel names as batch 1)")
     ap.add_argument("--calibrate", action="store_true",
                     help="also run a plain 256 MiB device copy, the known-size kernel that hardware-counter runs are scaled by")
     ap.add_argument("--decode-context", type=int, default=2048)
@@ -492,21 +494,24 @@ def main() -> int:
             if rc:
                 raise RuntimeError(_lib.last_error())
 
-    for i in range(3):
+    for i in range(0 if args.no_batch8 else 3):
         step8(i)
     torch.cuda.synchronize()
     g8 = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g8, stream=stream):
-        for i in range(args.copies):
-            step8(i)
-    assert L.oxb_hip_set_stream(C.c_void_p(stream.cuda_stream)) == 0
-    g8.replay()
-    e0.record(stream)
-    for _ in range(8):
+    if args.no_batch8:
+        ms8 = float("nan")
+    else:
+        with torch.cuda.graph(g8, stream=stream):
+            for i in range(args.copies):
+                step8(i)
+        assert L.oxb_hip_set_stream(C.c_void_p(stream.cuda_stream)) == 0
         g8.replay()
-    e1.record(stream)
-    torch.cuda.synchronize()
-    ms8 = e0.elapsed_time(e1) / (8 * args.copies)
+        e0.record(stream)
+        for _ in range(8):
+            g8.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms8 = e0.elapsed_time(e1) / (8 * args.copies)
     set_bytes8 = sum(algorithmic_bytes(r, k, B8) for _, r, k in SHAPES)
     batch8 = {"batch": B8, "ms_per_step": round(ms8, 6), "algorithmic_bytes_per_step": set_bytes8,
               "GB/s": round(set_bytes8 / (ms8 * 1e-3) / 1e9, 1), "weight_passes_per_gemv": 2,

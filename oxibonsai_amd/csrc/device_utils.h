@@ -43,3 +43,18 @@ __device__ __forceinline__ uint32_t buf_load_b32(__amdgpu_buffer_rsrc_t r, uint3
 // prefetched weight tiles) stay in flight across it.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+
+// Agent-coherent accesses (the sc1 cache-policy bit): the store is written through to memory, the load is served from
+// memory and not from this CU's L1 or this XCD's L2.  Data that other workgroups of the same launch produce and
+// consume goes through these, with a counter in between, instead of through whole-cache write-backs and invalidates.
+#define OXB_AUX_SC1 16
+__device__ __forceinline__ void buf_store_b32_coherent(__amdgpu_buffer_rsrc_t r, uint32_t voff, float v) {
+    __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(v), r, (int)voff, 0, OXB_AUX_SC1);
+}
+__device__ __forceinline__ v4f buf_load_f128_coherent(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
+    const v4u v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, 0, OXB_AUX_SC1);
+    return (v4f){__uint_as_float(v.x), __uint_as_float(v.y), __uint_as_float(v.z), __uint_as_float(v.w)};
+}
+__device__ __forceinline__ float buf_load_f32_coherent(__amdgpu_buffer_rsrc_t r, uint32_t voff) {
+    return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, 0, OXB_AUX_SC1));
+}

@@ -36,6 +36,8 @@ struct OxbAttnParams {
     uint32_t window, sinks;              // sliding window with attention sinks; window 0 = off
     float* part;                         // [batch][nq][n_splits][hd + OXB_ATTN_PART_PAD]: un-normalised output, maximum, sum
     float* out_single;                   // optional, n_splits == 1 only: [batch][nq*hd] receives the finished output (no merge launch)
+    float* out_merged;                   // n_splits > 1: [batch][nq*hd], written by the last workgroup of each (sequence, kv head) to finish
+    uint32_t* done;                      // n_splits > 1: [batch][nkv] arrival counters, zero before the launch; the kernel leaves them zero
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
     float scale;                         // 1 / sqrt(hd)
@@ -48,10 +50,9 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 #define OXB_ATTN_CHUNK_POSITIONS 128  // KV positions one attention workgroup covers at a time
 #define OXB_ATTN_MAX_SPLITS 64        // slots the KV sequence is split over; slot s walks chunks s, s + n_splits, ...
 #define OXB_ATTN_PART_PAD 4           // floats after the hd outputs of a slot: maximum, sum, 2 unused (16-byte rows)
-// QK-norm, RoPE, KV store of the new position and split-KV attention (at most 16 q heads per kv head) into
-// p.part; then the merge of the slots into the fp32 attention output d_out [batch][nq * hd].
+// QK-norm, RoPE, KV store of the new position, split-KV attention (at most 16 q heads per kv head) into p.part and
+// the merge of the slots into the fp32 attention output p.out_merged [batch][nq * hd], all in one launch.
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st);
-hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st);
 // out[v] = w * x[v] / sqrt(mean(x[v]^2) + eps) for nvec vectors of n values; d_w == nullptr copies.
 hipError_t oxb_launch_rmsnorm(const float* d_x, const float* d_w, uint32_t n, uint32_t nvec, float eps, float* d_out, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.

@@ -171,8 +171,8 @@ hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n
 //  CPU: block/functions.rs:78-127 -> layers/attention_fused.rs:329-400), fused with what precedes it in the layer:
 // per-head QK-RMSNorm, RoPE and the FP16 store of the new position's K and V (fused_qk_norm_rope + fused_kv_store,
 // cuda_attn_kernels.rs:160-251).  Grid (n_splits, nkv, batch), 256 threads = 4 waves.  It writes, per q head and
-// slot, the un-normalised partial output, the running maximum and the running sum; attn_combine_quant_kernel
-// merges the slots.
+// slot, the un-normalised partial output, the running maximum and the running sum; the last workgroup of a
+// (sequence, kv head) to finish merges the slots (attn_last_arrival, attn_merge_heads).
 // A workgroup serves all q heads of one kv head (<= 16, the columns of the MFMA tiles) for one slot of the KV
 // sequence: slot s walks chunks s, s + n_splits, ... of 128 positions, wave w takes keys [32w, 32w + 32) of each.
 //   S^T[key][head] = sum_d K[key][d] Q[head][d]     A = K rows straight from the cache, B = Q * scale as fp16 hi + lo
@@ -193,6 +193,28 @@ typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 //  * sliding window with attention sinks (is_in_window, crates/oxibonsai-model/src/layers/sliding_window.rs:173-189):
 //    the first `sinks` keys stay visible, the others while pos - key < window - sinks; chunks without a visible key
 //    are not walked.  window == 0: every key up to pos is visible.
+__device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_t b, uint32_t h_first, uint32_t nh, uint32_t heads_per,
+                                                 float* sm, float* __restrict__ out);
+
+// The workgroups of one (sequence, kv head) count themselves off once their slot results are written; the last one
+// to arrive merges the slots of the group's heads into the attention output, so that no second launch is needed.
+// The counter returns to 0 for the next launch.  The slot results travel between workgroups (other CUs, other XCDs)
+// through agent-coherent stores and loads: every store of this workgroup has been acknowledged by memory before its
+// count is added, and the merge's loads bypass the caches that another workgroup's stores do not reach.
+__device__ __forceinline__ bool attn_last_arrival(const OxbAttnParams& p, uint32_t b, uint32_t kvh, uint32_t expected, uint32_t* flag) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t* ctr = p.done + (size_t)b * p.nkv + kvh;
+        const uint32_t prev = atomicAdd(ctr, 1u);
+        const uint32_t last = prev + 1u == expected ? 1u : 0u;
+        if (last) atomicExch(ctr, 0u);
+        *flag = last;
+    }
+    __syncthreads();
+    return *flag != 0u;
+}
+
 template <int HD, int KVM, bool OPT>  // OPT: a window and / or a paged cache may be in use (else neither costs anything)
 __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p) {
     constexpr bool QC = KVM != OXB_KV_F16;
@@ -201,7 +223,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     constexpr int VL = 32 * VPR / 64;           // pieces of the wave's 32-row V block per lane
     // V block per wave; before the loop its start holds Q * scale of the group's heads, after it the merge buffers
     __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];
+    __shared__ uint32_t last_flag;
+    __shared__ __attribute__((aligned(16))) _Float16 kv_new[2][HD];  // the new position's K and V rows as stored (fp16 cache)
     static_assert(sizeof(vs_all) >= 16 * HD * sizeof(float), "Q must fit in the V slices");
+    static_assert(sizeof(vs_all) >= 16 * 65 * sizeof(float), "the merge's slot weights must fit in the V slices");
     float* qs = reinterpret_cast<float*>(&vs_all[0][0]);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -224,15 +249,20 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     const uint32_t first = next_needed(slot);
     float* part = p.part + (((size_t)b * p.nq + h0) * p.n_splits + slot) * (HD + OXB_ATTN_PART_PAD);
     const size_t part_head = (size_t)p.n_splits * (HD + OXB_ATTN_PART_PAD);
+    // slot results go out through agent-coherent stores: a workgroup of this same launch merges them
+    const __amdgpu_buffer_rsrc_t r_out = make_rsrc(part, (uint32_t)(G * part_head * 4u));
+    auto put = [&](size_t idx, float v) { buf_store_b32_coherent(r_out, (uint32_t)idx * 4u, v); };
     if (first >= n_chunks && !owner) {  // nothing visible in this slot's chunks: an empty result for the merge
         for (uint32_t i = tid; i < G * HD; i += 256) {
             const uint32_t h = i / HD, d = i % HD;
-            part[h * part_head + d] = 0.f;
+            put(h * part_head + d, 0.f);
             if (d == 0) {
-                part[h * part_head + HD] = -INFINITY;
-                part[h * part_head + HD + 1] = 0.f;
+                put(h * part_head + HD, -INFINITY);
+                put(h * part_head + HD + 1, 0.f);
             }
         }
+        if (attn_last_arrival(p, b, kvh, min(n_chunks, p.n_splits), &last_flag))
+            attn_merge_heads(p, b, h0, G, G, reinterpret_cast<float*>(&vs_all[0][0]), p.out_merged);
         return;
     }
     const float* qkv = p.qkv + (size_t)b * p.qkv_stride;
@@ -304,40 +334,93 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     };
 
-    // --- Q of the group's heads: RMSNorm over the head, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd) ---
-    for (uint32_t h = wave; h < G; h += 4) {
-        const float* in = qkv + (size_t)(h0 + h) * HD;
+    // With an fp16 cache the rows of the first chunk are requested before anything else, so that their way from HBM
+    // overlaps the Q prologue.  In the workgroup that stores the new position that row is not in the cache yet (and
+    // rows past the end repeat it): it is patched in from LDS below, with the very values the cache receives.
+    constexpr bool EARLY = !QC;
+    const uint32_t pos_chunk = pos / OXB_ATTN_CHUNK;
+    uint32_t na = 0, nb = 0;  // pages of the chunk whose rows are requested next
+    auto request_first = [&]() {
+        if (first < n_chunks) {
+            uint32_t pa, pb;
+            pages_of(first, pa, pb);
+            load_k(first, pa, pb);
+            load_v(first, pa, pb);
+            const uint32_t second = next_needed(first + p.n_splits);
+            if (second < n_chunks) pages_of(second, na, nb);
+        }
+    };
+    // Inputs of the prologue, requested before the cache rows: loads return in issue order, so whatever the prologue
+    // waits for must not queue behind the rows from HBM.  Lane d holds elements d and d + hd/2 of a head (the RoPE pair).
+    constexpr int KI = (HD / 2 + 63) / 64;
+    struct HeadIn { float lo[KI], hi[KI]; };
+    auto load_head = [&](const float* in, HeadIn& r) {
+#pragma unroll
+        for (int it = 0; it < KI; it++) {
+            const uint32_t d = lane + 64 * it;
+            r.lo[it] = d < half ? in[d] : 0.f;
+            r.hi[it] = d < half ? in[d + half] : 0.f;
+        }
+    };
+    // sum of squares in the order of a strided walk over the head (all low halves, then all high halves)
+    auto head_inv_rms = [&](const HeadIn& r) {
         float ss = 0.f;
-        for (uint32_t d = lane; d < HD; d += 64) ss = fmaf(in[d], in[d], ss);
+#pragma unroll
+        for (int it = 0; it < KI; it++) ss = fmaf(r.lo[it], r.lo[it], ss);
+#pragma unroll
+        for (int it = 0; it < KI; it++) ss = fmaf(r.hi[it], r.hi[it], ss);
 #pragma unroll
         for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-        const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
-        for (uint32_t d = lane; d < half; d += 64) {
-            const float lo_ = p.q_norm[d] * in[d] * inv, hi_ = p.q_norm[d + half] * in[d + half] * inv;
-            qs[h * HD + d] = (lo_ * cs[d] - hi_ * sn[d]) * p.scale;
-            qs[h * HD + d + half] = (lo_ * sn[d] + hi_ * cs[d]) * p.scale;
+        return 1.0f / sqrtf(ss / (float)HD + p.eps);
+    };
+    HeadIn q_in, cs_sn, qn, kv_in, kn;  // cs_sn: lo = cos, hi = sin; kv_in: the new K row (wave 0) or V row (wave 1) of the owner
+    {
+#pragma unroll
+        for (int it = 0; it < KI; it++) {
+            const uint32_t d = lane + 64 * it;
+            cs_sn.lo[it] = d < half ? cs[d] : 0.f;
+            cs_sn.hi[it] = d < half ? sn[d] : 0.f;
+        }
+        load_head(p.q_norm, qn);
+        if (wave < G) load_head(qkv + (size_t)(h0 + wave) * HD, q_in);
+        if (owner && wave == 0) {
+            load_head(qkv + (size_t)(p.nq + kvh) * HD, kv_in);
+            load_head(p.k_norm, kn);
+        } else if (owner && wave == 1) {
+            load_head(qkv + (size_t)(p.nq + p.nkv + kvh) * HD, kv_in);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    if (EARLY) request_first();
+    __builtin_amdgcn_sched_barrier(0);
+    // --- Q of the group's heads: RMSNorm over the head, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd) ---
+    for (uint32_t h = wave; h < G; h += 4) {
+        if (h != wave) load_head(qkv + (size_t)(h0 + h) * HD, q_in);
+        const float inv = head_inv_rms(q_in);
+#pragma unroll
+        for (int it = 0; it < KI; it++) {
+            const uint32_t d = lane + 64 * it;
+            if (d < half) {
+                const float lo_ = qn.lo[it] * q_in.lo[it] * inv, hi_ = qn.hi[it] * q_in.hi[it] * inv;
+                qs[h * HD + d] = (lo_ * cs_sn.lo[it] - hi_ * cs_sn.hi[it]) * p.scale;
+                qs[h * HD + d + half] = (lo_ * cs_sn.hi[it] + hi_ * cs_sn.lo[it]) * p.scale;
+            }
         }
     }
     // --- K and V of the new position, by the workgroup whose slot walks its chunk (wave 0 and wave 1) ---
     const size_t new_row = kv_row(p.kv, b, p.layer, kvh, pos);
     if (owner) {
         if (wave == 0) {
-            const float* in = qkv + (size_t)(p.nq + kvh) * HD;
-            float ss = 0.f;
-            for (uint32_t d = lane; d < HD; d += 64) ss = fmaf(in[d], in[d], ss);
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
-            const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
-            constexpr int KI = (HD / 2 + 63) / 64;
+            const float inv = head_inv_rms(kv_in);
             float klo[KI], khi[KI], mx = 0.f;
 #pragma unroll
             for (int it = 0; it < KI; it++) {
                 const uint32_t d = lane + 64 * it;
                 klo[it] = khi[it] = 0.f;
                 if (d < half) {
-                    const float lo_ = p.k_norm[d] * in[d] * inv, hi_ = p.k_norm[d + half] * in[d + half] * inv;
-                    klo[it] = lo_ * cs[d] - hi_ * sn[d];
-                    khi[it] = lo_ * sn[d] + hi_ * cs[d];
+                    const float lo_ = kn.lo[it] * kv_in.lo[it] * inv, hi_ = kn.hi[it] * kv_in.hi[it] * inv;
+                    klo[it] = lo_ * cs_sn.lo[it] - hi_ * cs_sn.hi[it];
+                    khi[it] = lo_ * cs_sn.hi[it] + hi_ * cs_sn.lo[it];
                     mx = fmaxf(mx, fmaxf(fabsf(klo[it]), fabsf(khi[it])));
                 }
             }
@@ -356,21 +439,15 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
                         Kc[new_row * HD + d] = (uint8_t)kv_encode<KVM>(klo[it], scale);
                         Kc[new_row * HD + d + half] = (uint8_t)kv_encode<KVM>(khi[it], scale);
                     } else {
-                        Kc[new_row * HD + d] = (_Float16)klo[it];
-                        Kc[new_row * HD + d + half] = (_Float16)khi[it];
+                        Kc[new_row * HD + d] = kv_new[0][d] = (_Float16)klo[it];
+                        Kc[new_row * HD + d + half] = kv_new[0][d + half] = (_Float16)khi[it];
                     }
                 }
             }
         } else if (wave == 1) {
-            const float* in = qkv + (size_t)(p.nq + p.nkv + kvh) * HD;
-            constexpr int VI = (HD + 63) / 64;
-            float vv[VI], mx = 0.f;
+            float mx = 0.f;
 #pragma unroll
-            for (int it = 0; it < VI; it++) {
-                const uint32_t d = lane + 64 * it;
-                vv[it] = d < HD ? in[d] : 0.f;
-                mx = fmaxf(mx, fabsf(vv[it]));
-            }
+            for (int it = 0; it < KI; it++) mx = fmaxf(mx, fmaxf(fabsf(kv_in.lo[it]), fabsf(kv_in.hi[it])));
             float scale = 1.f;
             if constexpr (QC) {
 #pragma unroll
@@ -379,25 +456,26 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
                 if (lane == 0) Vsc[new_row] = scale;
             }
 #pragma unroll
-            for (int it = 0; it < VI; it++) {
+            for (int it = 0; it < KI; it++) {
                 const uint32_t d = lane + 64 * it;
-                if (d < HD) {
-                    if constexpr (QC) Vc[new_row * HD + d] = (uint8_t)kv_encode<KVM>(vv[it], scale);
-                    else Vc[new_row * HD + d] = (_Float16)vv[it];
+                if (d < half) {
+                    if constexpr (QC) {
+                        Vc[new_row * HD + d] = (uint8_t)kv_encode<KVM>(kv_in.lo[it], scale);
+                        Vc[new_row * HD + d + half] = (uint8_t)kv_encode<KVM>(kv_in.hi[it], scale);
+                    } else {
+                        Vc[new_row * HD + d] = kv_new[1][d] = (_Float16)kv_in.lo[it];
+                        Vc[new_row * HD + d + half] = kv_new[1][d + half] = (_Float16)kv_in.hi[it];
+                    }
                 }
             }
         }
     }
-    __syncthreads();  // publishes qs and, within this workgroup, the new cache rows
-    uint32_t na = 0, nb = 0;  // pages of the chunk whose rows are requested next
-    if (first < n_chunks) {
-        uint32_t pa, pb;
-        pages_of(first, pa, pb);
-        load_k(first, pa, pb);
-        load_v(first, pa, pb);
-        const uint32_t second = next_needed(first + p.n_splits);
-        if (second < n_chunks) pages_of(second, na, nb);
-    }
+    // publishes qs and the LDS copy of the new rows.  The requested cache rows stay in flight across it, unless this
+    // workgroup will read the new position's rows back from the cache (requests after the prologue, or a walk of
+    // several chunks that ends in the new position's): then the stores must have landed first.
+    if (owner && !(EARLY && pos_chunk == first)) __syncthreads();
+    else lds_barrier();
+    if (!EARLY) request_first();
 
     // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo
     v8h_t qh[KS], ql[KS];
@@ -411,7 +489,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             qh[s][e] = hi;
             ql[s][e] = (_Float16)(x - (float)hi);
         }
-    __syncthreads();  // Q is in registers everywhere: its LDS copy may be overwritten
+    lds_barrier();  // Q is in registers everywhere: its LDS copy may be overwritten
     v4f O[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
@@ -422,6 +500,8 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         const uint32_t key0 = chunk * OXB_ATTN_CHUNK + 32 * wave;
         const uint32_t nxt = next_needed(chunk + p.n_splits);
         const bool more = nxt < n_chunks;
+        // rows of the new position (and the repeats of it past the end) come from LDS where they were requested early
+        const bool patch = EARLY && owner && chunk == pos_chunk && chunk == first;
         chunk = nxt;
         // stage the V block in the wave's LDS slice (the previous block's gathers were issued before: LDS runs in
         // order) and request the next chunk's
@@ -438,7 +518,9 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
                 *reinterpret_cast<v4i*>(dst) = (v4i){(int)d[0], (int)d[1], (int)d[2], (int)d[3]};
                 *reinterpret_cast<v4i*>(dst + 8) = (v4i){(int)d[4], (int)d[5], (int)d[6], (int)d[7]};
             } else {
-                *reinterpret_cast<v4i*>(vs + (id / VPR) * VSTR + (id % VPR) * 8) = vr[i];
+                v4i piece = vr[i];
+                if (patch && key0 + id / VPR >= pos) piece = *reinterpret_cast<const v4i*>(&kv_new[1][(id % VPR) * 8]);
+                *reinterpret_cast<v4i*>(vs + (id / VPR) * VSTR + (id % VPR) * 8) = piece;
             }
         }
         const float4 vc0 = vsc0, vc1 = vsc1;
@@ -453,6 +535,10 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             } else {
                 a0 = k0r[s];
                 a1 = k1r[s];
+                if (patch) {
+                    if (key0 + qi >= pos) a0 = *reinterpret_cast<const v8h_t*>(&kv_new[0][32 * s + 8 * g]);
+                    if (key0 + 16 + qi >= pos) a1 = *reinterpret_cast<const v8h_t*>(&kv_new[0][32 * s + 8 * g]);
+                }
             }
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, qh[s], s0, 0, 0, 0);
             s0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(a0, ql[s], s0, 0, 0, 0);
@@ -546,10 +632,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     float* mo = reinterpret_cast<float*>(&vs_all[0][0]);  // [wave][head 16][HD], then [wave][head 16] m, [wave][head 16] l
     float* mm = mo + 4 * 16 * HD;
     float* ml = mm + 4 * 16;
+    if (qi < G) {
 #pragma unroll
-    for (int sl = 0; sl < NS; sl++)
-        *reinterpret_cast<float4*>(&mo[(wave * 16 + qi) * HD + 16 * sl + 4 * g]) =
-            make_float4(O[sl][0] * u_run, O[sl][1] * u_run, O[sl][2] * u_run, O[sl][3] * u_run);
+        for (int sl = 0; sl < NS; sl++)
+            *reinterpret_cast<float4*>(&mo[(wave * 16 + qi) * HD + 16 * sl + 4 * g]) =
+                make_float4(O[sl][0] * u_run, O[sl][1] * u_run, O[sl][2] * u_run, O[sl][3] * u_run);
+    }
     if (g == 0) {
         mm[wave * 16 + qi] = m_run;
         ml[wave * 16 + qi] = l_run;
@@ -569,31 +657,38 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             p.out_single[((size_t)b * p.nq + h0 + h) * HD + d] = o * (l > 0.f ? 1.0f / l : 0.f);
             continue;
         }
-        part[h * part_head + d] = o;
+        put(h * part_head + d, o);
         if (d == 0) {
-            part[h * part_head + HD] = M;
-            part[h * part_head + HD + 1] = l;
+            put(h * part_head + HD, M);
+            put(h * part_head + HD + 1, l);
         }
     }
+    if (p.out_single) return;
+    if (attn_last_arrival(p, b, kvh, min(n_chunks, p.n_splits), &last_flag))  // (the barrier inside also retires mo / mm / ml)
+        attn_merge_heads(p, b, h0, G, G, reinterpret_cast<float*>(&vs_all[0][0]), p.out_merged);
 }
 
-// Merge the slot results of the q heads into the attention output [batch][nq * hd] (fp32), the input of the O
-// projection.  Grid (sequences, parts), 256 threads: a workgroup takes a run of whole heads; per head one wave works out
-// the softmax weights of the slots (one slot per lane), then every thread adds the weighted slot outputs of four
-// dimensions in ascending slot order.
-__global__ __launch_bounds__(256) void attn_combine_kernel(OxbAttnParams p, uint32_t heads_per, float* __restrict__ out) {
-    extern __shared__ float sm[];  // [heads here][64] slot weights | [heads here] 1 / sum
-    const uint32_t b = blockIdx.x, tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
-    const uint32_t h_first = blockIdx.y * heads_per;
-    if (h_first >= p.nq) return;
-    const uint32_t nh = (h_first + heads_per <= p.nq ? heads_per : p.nq - h_first);
-    const uint32_t e0 = h_first * hd, e1 = e0 + nh * hd;
+// Merge the slot results of heads h_first .. h_first + nh - 1 of sequence b into the attention output
+// [batch][nq * hd] (fp32), the input of the O projection, by the 256 threads of a workgroup: per head one wave works
+// out the softmax weights of the slots (one slot per lane), then every thread adds the weighted slot outputs of four
+// dimensions in ascending slot order.  sm: (heads_per * 65) floats of LDS: [head][64] slot weights | [head] 1 / sum.
+// The slot results were written by other workgroups of this same launch: agent-coherent loads.
+__device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_t b, uint32_t h_first, uint32_t nh, uint32_t heads_per,
+                                                 float* sm, float* __restrict__ out) {
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, hd = p.hd, qd = p.nq * hd;
     const uint32_t stride = hd + OXB_ATTN_PART_PAD;
     float* wts = sm;
     float* inv_l = wts + heads_per * 64;
+    const uint32_t e0 = h_first * hd, e1 = e0 + nh * hd;
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
     const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
+    const __amdgpu_buffer_rsrc_t r_part = make_rsrc(part, p.nq * p.n_splits * stride * 4u);
+    auto ld4 = [&](const float* q) -> float4 {
+        const v4f v = buf_load_f128_coherent(r_part, (uint32_t)(q - part) * 4u);
+        return make_float4(v.x, v.y, v.z, v.w);
+    };
+    auto ld1 = [&](const float* q) -> float { return buf_load_f32_coherent(r_part, (uint32_t)(q - part) * 4u); };
     // The first slots' partial outputs of this thread's first four elements do not depend on the slot weights:
     // request them before the weights are worked out, so that both round trips to memory overlap.
     constexpr int PRE = 8;
@@ -603,11 +698,11 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(OxbAttnParams p, uint
         const float* ph = part + (size_t)(e / hd) * p.n_splits * stride + e % hd;
 #pragma unroll
         for (int u = 0; u < PRE; u++)
-            pre[u] = (e < e1 && (uint32_t)u < used) ? *reinterpret_cast<const float4*>(ph + (size_t)u * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+            pre[u] = (e < e1 && (uint32_t)u < used) ? ld4(ph + (size_t)u * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
     }
     for (uint32_t hh = tid >> 6; hh < nh; hh += 4) {
         const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
-        const float mv = lane < used ? ph[0] : -INFINITY, lv = lane < used ? ph[1] : 0.f;
+        const float mv = lane < used ? ld1(ph) : -INFINITY, lv = lane < used ? ld1(ph + 1) : 0.f;
         float M = mv;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
@@ -639,11 +734,11 @@ __global__ __launch_bounds__(256) void attn_combine_kernel(OxbAttnParams p, uint
         for (; s + PRE <= used; s += PRE) {
             float4 v[PRE];
 #pragma unroll
-            for (int u = 0; u < PRE; u++) v[u] = *reinterpret_cast<const float4*>(ph + (size_t)(s + u) * stride);
+            for (int u = 0; u < PRE; u++) v[u] = ld4(ph + (size_t)(s + u) * stride);
             fold(v, s);
         }
         for (; s < used; s++) {
-            const float4 v = *reinterpret_cast<const float4*>(ph + (size_t)s * stride);
+            const float4 v = ld4(ph + (size_t)s * stride);
             const float w = wts[hh * 64 + s];
             acc.x = fmaf(v.x, w, acc.x), acc.y = fmaf(v.y, w, acc.y), acc.z = fmaf(v.z, w, acc.z), acc.w = fmaf(v.w, w, acc.w);
         }
@@ -710,7 +805,7 @@ hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, h
 
 hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStream_t st) {
     if (p.chunk != OXB_ATTN_CHUNK || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS || p.nq % p.nkv || p.nq / p.nkv > 16 ||
-        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 || (p.out_single && p.n_splits != 1) ||
+        !p.qkv || !p.q_norm || !p.k_norm || !p.cos_t || !p.sin_t || p.kv_mode > OXB_KV_FP8_E4M3 || (p.out_single && p.n_splits != 1) || (!p.out_single && (!p.done || !p.out_merged)) ||
         (p.kv_mode != OXB_KV_F16 && (!p.k_scale || !p.v_scale)) ||
         (p.kv.page_table ? (p.kv.page_shift < 4 || p.kv.page_shift > 7) : (p.kv.row_stride % OXB_ATTN_CHUNK != 0 || p.kv.row_stride < p.max_seq)))
         return hipErrorInvalidValue;
@@ -738,15 +833,6 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
 #undef OXB_ATTN_CASE
         default: return hipErrorInvalidValue;
     }
-    return hipGetLastError();
-}
-
-hipError_t oxb_launch_attn_combine(const OxbAttnParams& p, uint32_t batch, float* d_out, hipStream_t st) {
-    if (batch == 0 || !d_out || (p.hd & 3u) || p.n_splits == 0 || p.n_splits > OXB_ATTN_MAX_SPLITS) return hipErrorInvalidValue;
-    // about 16 workgroups per sequence, whole heads each
-    const uint32_t heads_per = (p.nq + 15u) / 16u, parts = (p.nq + heads_per - 1) / heads_per;
-    const size_t shm = (size_t)heads_per * 65 * sizeof(float);
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(batch, parts), dim3(256), shm, st, p, heads_per, d_out);
     return hipGetLastError();
 }
 

@@ -38,6 +38,7 @@ struct Model {
     float *hidden = nullptr, *qkv = nullptr, *attn_part = nullptr, *attn_out = nullptr,
           *gu = nullptr, *act = nullptr, *logits = nullptr;  // gu: [batch][2 inter] gate || up sums, act: [batch][inter] SwiGLU output
     uint32_t *tokens = nullptr, *pos = nullptr;
+    uint32_t* attn_done = nullptr;  // [batch][nkv] arrival counters of the attention workgroups, 0 between launches
     void* argmax_ws = nullptr;
     // KV cache: rows of hd fp16 values or one-byte codes, a quantised cache also one f32 scale per row.  Contiguous:
     // [batch][n_layers][nkv][row_stride] rows; paged: a pool [n_pages][n_layers][nkv][2^page_shift] rows and, per
@@ -303,8 +304,9 @@ static int kv_sync_table(Model& m) {
 
 // QK-norm + RoPE + KV store + split-KV attention of one layer for the whole decode batch, one launch; leaves the
 // slot results in m.attn_part and the parameters the merge needs in *ap.
-static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, OxbAttnParams* out,
-                                   float* out_single = nullptr) {
+// One launch: QK-norm, RoPE, the store of the new rows, attention over the cache and the merge of the KV slots into
+// m.attn_out (with a single slot per sequence the kernel writes its output directly).
+static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm) {
     const oxb_model_desc& d = m.d;
     OxbAttnParams ap;
     ap.qkv = m.qkv;
@@ -323,7 +325,9 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.window = m.window;
     ap.sinks = m.sinks;
     ap.part = m.attn_part;
-    ap.out_single = out_single;
+    ap.out_single = m.n_splits == 1 ? m.attn_out : nullptr;
+    ap.out_merged = m.attn_out;
+    ap.done = m.attn_done;
     ap.pos = m.pos;
     ap.nq = d.nq;
     ap.nkv = d.nkv;
@@ -334,7 +338,6 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.chunk = m.chunk;
     ap.n_splits = m.n_splits;
     ap.scale = 1.0f / sqrtf((float)d.hd);
-    *out = ap;
     OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, g_rt.stream), "kernel launch failed: attention");
     return OXB_HIP_OK;
 }
@@ -357,13 +360,7 @@ static int encode_decode_step_gemm(Model& m) {
         const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
         if (rc) return rc;
         OXB_TRY(gemm_device(*wqkv, m.hidden, d.h, m.qkv, B, qkv_rows, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, attn_norm, d.eps, &m.gws));
-        OxbAttnParams ap;
-        if (m.n_splits == 1) {  // one slot per sequence: the attention kernel finishes its output itself
-            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap, m.attn_out));
-        } else {
-            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
-            OXB_TRY_HIP(oxb_launch_attn_combine(ap, B, m.attn_out, st), "kernel launch failed: attn_combine");
-        }
+        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm));
         OXB_TRY(gemm_device(*wo, m.attn_out, qd, m.hidden, B, d.h, OXB_GEMM_RESIDUAL, m.hidden, OXB_PACK_IDENT, nullptr, 0.f, &m.gws));
         // SwiGLU in the epilogue of the gate || up product
         OXB_TRY(gemm_device(*wgu, m.hidden, d.h, m.gu, B, d.inter, OXB_GEMM_SWIGLU, nullptr, OXB_PACK_RMSNORM, ffn_norm, d.eps, &m.gws));
@@ -401,13 +398,7 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
             OXB_TRY(gemv_launch(*wqkv, m.hidden + (size_t)b0 * d.h, d.h, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows,
                                 OXB_GEMV_PRO_RMSNORM, attn_norm, d.eps, OXB_GEMV_STORE, nullptr));
         }
-        OxbAttnParams ap;
-        if (m.n_splits == 1) {  // one slot per sequence: the attention kernel finishes its output itself
-            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap, m.attn_out));
-        } else {
-            OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, &ap));
-            OXB_TRY_HIP(oxb_launch_attn_combine(ap, d.batch, m.attn_out, st), "kernel launch failed: attn_combine");
-        }
+        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm));
         for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
             const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
             OXB_TRY(encode_ffn(m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo, *wgu, *wdn,
@@ -687,11 +678,18 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         (rc = dev_alloc(m, (void**)&m.attn_out, B * qd * 4)) || (rc = dev_alloc(m, (void**)&m.gu, B * 2 * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.act, B * d.inter * 4)) ||
         (rc = dev_alloc(m, (void**)&m.logits, B * (d.lm_head ? d.vocab : 1) * 4)) || (rc = dev_alloc(m, (void**)&m.tokens, B * 4)) ||
-        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
+        (rc = dev_alloc(m, (void**)&m.pos, B * 4)) || (rc = dev_alloc(m, (void**)&m.attn_done, B * d.nkv * 4)) || (rc = dev_alloc(m, &m.argmax_ws, B * OXB_ARGMAX_MAX_PARTS * 8)) || (rc = alloc_kv_cache(m, OXB_KV_F16, 0, 0)) ||
         (rc = dev_alloc(m, (void**)&m.cos_t, (size_t)d.max_seq * (d.hd / 2) * 4)) ||
         (rc = dev_alloc(m, (void**)&m.sin_t, (size_t)d.max_seq * (d.hd / 2) * 4))) {
         free_model(m);
         return rc;
+    }
+    {
+        hipError_t e = hipMemset(m.attn_done, 0, B * d.nkv * 4);
+        if (e != hipSuccess) {
+            free_model(m);
+            return hip_fail(e, "counter clear");
+        }
     }
     // RoPE table, computed as RopeTable::new does (crates/oxibonsai-model/src/layers/rope.rs:27-48): all in f32.
     {
