@@ -688,7 +688,7 @@ static hipError_t launch_gemm_case(const OxbGemmParams& p, uint32_t grid, hipStr
     return hipGetLastError();
 }
 
-struct GemmPlan { uint32_t rt, tpw, ksplit, sb_per_split; };
+struct GemmPlan { uint32_t rt, tpw, ksplit, sb_per_split, ct; };
 
 // Row tiles per workgroup and K slices: minimise (rounds of workgroups over the CUs) x (time of one workgroup),
 // where a workgroup costs, per superblock of its K slice, its row tiles per wave plus about one more for staging,
@@ -698,8 +698,8 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
     constexpr uint32_t BM = 128;
     const uint32_t n_mt = (p.M + BM - 1) / BM;
     static const uint32_t rts[] = {5, 4, 3, 2, 1};
-    GemmPlan best = {1, 4, 1, p.n_sb};
-    if (p.mode == OXB_GEMM_SWIGLU) best = {2, 8, 1, p.n_sb};
+    GemmPlan best = {1, 4, 1, p.n_sb, 8};
+    if (p.mode == OXB_GEMM_SWIGLU) best = {2, 8, 1, p.n_sb, 8};
     uint64_t best_cost = ~0ull;
     const bool sw = p.mode == OXB_GEMM_SWIGLU;  // even tile counts per wave, no K split (the epilogue is not linear)
     const bool can_split = (p.ldy & 3u) == 0 && !sw;
@@ -717,9 +717,17 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
                 const uint64_t wgs = (uint64_t)groups * n_mt * ks;
                 uint64_t cost = ((wgs + n_cus - 1) / n_cus) * ((uint64_t)spk * (rt + 1) + 2 * rt + 2);
                 if (ks > 1) cost += (uint64_t)ks * 2 + 4;  // the reduction pass
-                if (cost < best_cost) best_cost = cost, best = {rt, tpw, ks, spk};
+                if (cost < best_cost) best_cost = cost, best = {rt, tpw, ks, spk, 8};
             }
         }
+    }
+    // Small matrices leave the 128-token tile short of workgroups (one or two row tiles per wave and still fewer
+    // workgroups than CUs): there a 64-token tile with one row tile per wave doubles their number.  Measured at 512
+    // tokens: 4096 x 4096 26.2 -> 23.0 us, 6144 x 4096 37.0 -> 33.2, 5120 x 2560 (TQ2) 26.6 -> 24.6, 4096 x 2048 17.5 ->
+    // 15.8, 2048 x 2048 14.9 -> 11.4; with more workgroups to begin with the wider tile wins.
+    if (!sw && best.ksplit == 1 && best.rt <= 2) {
+        const uint64_t wgs = (uint64_t)((p.n_tiles + best.tpw - 1) / best.tpw) * n_mt;
+        if (best.rt == 1 || wgs < n_cus) best = {1, 4, 1, p.n_sb, 4};
     }
     return best;
 }
@@ -764,9 +772,9 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     p.M_pad = (p.M + 15u) / 16u * 16u;
     if (p.M <= OXB_GEMM_NARROW_MAX_M) return launch_gemm_narrow(fmt, p, n_cus, st);
     if (p.mode == OXB_GEMM_SWIGLU && (p.n_rows & 31u) != 0) return hipErrorInvalidValue;  // whole gate and up row tiles
-    constexpr uint32_t CT = 8, BM = 16 * CT;
-    p.n_mt = (p.M + BM - 1) / BM;
     const GemmPlan plan = plan_gemm(p, n_cus);
+    const uint32_t BM = 16 * plan.ct;  // tokens per workgroup tile
+    p.n_mt = (p.M + BM - 1) / BM;
     const uint32_t best_rt = plan.rt, best_tpw = plan.tpw;
     p.ksplit = plan.ksplit;
     p.sb_per_split = plan.sb_per_split;
@@ -776,7 +784,7 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     const uint32_t grid = p.n_ng * p.n_mt * p.ksplit;
     hipError_t err = hipErrorInvalidValue;
 #define OXB_GEMM_CASE(F, R) \
-    if (fmt == F && best_rt == R) err = launch_gemm_case<F, R, CT>(p, grid, st);
+    if (fmt == F && best_rt == R && plan.ct == 8) err = launch_gemm_case<F, R, 8>(p, grid, st);
     OXB_GEMM_CASE(OXB_FMT_Q1, 1)
     OXB_GEMM_CASE(OXB_FMT_Q1, 2)
     OXB_GEMM_CASE(OXB_FMT_Q1, 3)
@@ -788,6 +796,7 @@ hipError_t oxb_launch_gemm(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t
     OXB_GEMM_CASE(OXB_FMT_TQ2, 4)
     OXB_GEMM_CASE(OXB_FMT_TQ2, 5)
 #undef OXB_GEMM_CASE
+    if (plan.ct == 4 && best_rt == 1) err = fmt == OXB_FMT_Q1 ? launch_gemm_case<OXB_FMT_Q1, 1, 4>(p, grid, st) : launch_gemm_case<OXB_FMT_TQ2, 1, 4>(p, grid, st);
     if (err != hipSuccess || p.ksplit == 1) return err;
     const size_t plane = (size_t)p.M * p.ldy, n4 = plane / 4;
     hipLaunchKernelGGL(gemm_splitk_reduce_kernel, dim3((uint32_t)((n4 + 255) / 256)), dim3(256), 0, st, p.part, p.ksplit, plane,
