@@ -75,9 +75,17 @@ def _compare_cache(gpu, cpu, cfg, mode, n_pos):
     for L in range(cfg["n_layers"]):
         for hh in range(cfg["nkv"]):
             gk, gv, gks, gvs = gpu.read_kv(L, hh, 0, n_pos)
-            if mode == KV_F16:     # rows of O(1) values; layer 1's carry the 1e-4 of noise of the layer below
-                assert np.allclose(gk.astype(np.float32), k[L, hh, :n_pos], rtol=2e-3, atol=1e-3)
-                assert np.allclose(gv.astype(np.float32), v[L, hh, :n_pos], rtol=2e-3, atol=1e-3)
+            if mode == KV_F16:
+                # Both sides round an fp32 value to fp16.  In layer 0 the two fp32 values differ only by the summation
+                # order of the QKV projection (1e-6 of the row scale): the stored rows are equal or one fp16 step apart.
+                # From layer 1 on the inputs themselves differ: every one-step flip in the cache of the layer below moves
+                # that layer's attention output, hence this layer's K and V, by up to 1e-3 (rows of O(1) values).
+                for got, want in ((gk.astype(np.float32), k[L, hh, :n_pos]), (gv.astype(np.float32), v[L, hh, :n_pos])):
+                    step = np.ldexp(1.0, np.floor(np.log2(np.maximum(np.abs(want), 2.0 ** -14))).astype(int) - 10)
+                    if L == 0:
+                        assert np.all(np.abs(got - want) <= step + 2e-5), float(np.max(np.abs(got - want) - step))
+                    else:
+                        assert np.allclose(got, want, rtol=2e-3, atol=1e-3)
                 assert np.all(gks == 1.0) and np.all(gvs == 1.0)
                 continue
             for got_c, got_s, want_c, want_s in ((gk, gks, kc[L, hh, :n_pos], ks[L, hh, :n_pos]),
