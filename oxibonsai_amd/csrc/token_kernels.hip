@@ -3,7 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 #include <stdint.h>
-#include <hipcub/hipcub.hpp>
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
 
 #include "device_utils.h"
 #include "token_kernels.h"
@@ -645,8 +646,8 @@ static size_t align256(size_t v) { return (v + 255u) & ~(size_t)255u; }
 struct FullWs { size_t e, ps, is, iota, pmax, sum, tmp, tmp_bytes, total; };
 static hipError_t full_ws_layout(uint32_t n, uint32_t batch, FullWs* w) {
     size_t tmp = 0;
-    hipError_t err = hipcub::DeviceRadixSort::SortPairsDescending(nullptr, tmp, (const float*)nullptr, (float*)nullptr,
-                                                                 (const uint32_t*)nullptr, (uint32_t*)nullptr, (int)n);
+    hipError_t err = rocprim::radix_sort_pairs_desc(nullptr, tmp, (const float*)nullptr, (float*)nullptr, (const uint32_t*)nullptr,
+                                                    (uint32_t*)nullptr, (unsigned int)n);
     if (err != hipSuccess) return err;
     const size_t rows = align256((size_t)n * 4 * batch), parts = (n + OXB_FULL_SPAN - 1) / OXB_FULL_SPAN;
     w->e = 0;
@@ -686,8 +687,8 @@ static hipError_t launch_sample_full(const float* d_logits, uint32_t n, uint32_t
     auto sort_rows = [&]() -> hipError_t {  // e -> ps (descending, stable), iota -> is
         for (uint32_t b = 0; b < batch; b++) {
             size_t tmp = w.tmp_bytes;
-            hipError_t r = hipcub::DeviceRadixSort::SortPairsDescending(base + w.tmp, tmp, e + (size_t)b * n, ps + (size_t)b * n, iota,
-                                                                        is + (size_t)b * n, (int)n, 0, 32, st);
+            hipError_t r = rocprim::radix_sort_pairs_desc(base + w.tmp, tmp, e + (size_t)b * n, ps + (size_t)b * n, iota,
+                                                          is + (size_t)b * n, (unsigned int)n, 0, 32, st);
             if (r != hipSuccess) return r;
         }
         return hipSuccess;
