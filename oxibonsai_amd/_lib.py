@@ -8,7 +8,8 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "lib", "liboxb_hip.so")
+# OXB_HIP_LIBRARY names another build of the same library (comparing two builds on one GPU)
+LIB_PATH = os.environ.get("OXB_HIP_LIBRARY") or os.path.join(_HERE, "lib", "liboxb_hip.so")
 _lib = None
 
 u8p = C.POINTER(C.c_uint8)
