@@ -516,6 +516,33 @@ def main() -> int:
     batch8 = {"batch": B8, "ms_per_step": round(ms8, 6), "algorithmic_bytes_per_step": set_bytes8,
               "GB/s": round(set_bytes8 / (ms8 * 1e-3) / 1e9, 1), "weight_passes_per_gemv": 2,
               "note": "exact GEMV route, four vectors share a pass over the weights; weights counted once"}
+    if not args.no_batch8:
+        # the same eight vectors through the route the decode pipeline takes from five sequences on: activations packed
+        # to fp16, one pass over the weights on the fp16 matrix cores (prefill tolerance instead of fp32-exact products)
+        def step8g(i: int) -> None:
+            c = i % args.copies
+            for name, n_rows, k in SHAPES:
+                rc = L.oxb_hip_gemm_dev(ids[name][c], d_x8[name].data_ptr(), d_y8[name].data_ptr(), B8, n_rows, k)
+                if rc:
+                    raise RuntimeError(_lib.last_error())
+
+        for i in range(3):
+            step8g(i)
+        torch.cuda.synchronize()
+        g8g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g8g, stream=stream):
+            for i in range(args.copies):
+                step8g(i)
+        assert L.oxb_hip_set_stream(C.c_void_p(stream.cuda_stream)) == 0
+        g8g.replay()
+        e0.record(stream)
+        for _ in range(8):
+            g8g.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms8g = e0.elapsed_time(e1) / (8 * args.copies)
+        batch8["fp16_matrix_core_route"] = {"ms_per_step": round(ms8g, 6), "GB/s": round(set_bytes8 / (ms8g * 1e-3) / 1e9, 1),
+                                            "note": "packer + narrow GEMM per matrix, one pass over the weights, fp16 activations (1e-2 gate)"}
 
     # --- roofline of the dominant kernel: the gate||up GEMV alone, HIP events on its stream --------
     name, n_rows, k = SHAPES[1]
