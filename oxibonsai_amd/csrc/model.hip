@@ -38,6 +38,10 @@ struct Model {
     float *hidden = nullptr, *qkv = nullptr, *attn_part = nullptr, *attn_out = nullptr,
           *gu = nullptr, *act = nullptr, *logits = nullptr;  // gu: [batch][2 inter] gate || up sums, act: [batch][inter] SwiGLU output
     uint32_t *tokens = nullptr, *pos = nullptr;
+    // pinned host staging of a decode call's small transfers (embedding rows and positions in, tokens out): copies from
+    // and to pageable memory go through the runtime's own staging and cost about 10 us per call more
+    float* h_hidden = nullptr;
+    uint32_t *h_pos = nullptr, *h_tokens = nullptr;
     uint32_t* attn_done = nullptr;  // [batch][nkv] arrival counters of the attention workgroups, 0 between launches
     void* argmax_ws = nullptr;
     // KV cache: rows of hd fp16 values or one-byte codes, a quantised cache also one f32 scale per row.  Contiguous:
@@ -109,6 +113,10 @@ static void free_kv_cache(Model& m) {
 static void free_model(Model& m) {
     if (m.graph_exec) (void)hipGraphExecDestroy(m.graph_exec);
     m.graph_exec = nullptr;
+    if (m.h_hidden) (void)hipHostFree(m.h_hidden);
+    if (m.h_pos) (void)hipHostFree(m.h_pos);
+    m.h_hidden = nullptr;
+    m.h_pos = m.h_tokens = nullptr;
     for (void* p : m.allocs) (void)hipFree(p);
     m.allocs.clear();
     for (void* p : m.pf_allocs) (void)hipFree(p);
@@ -685,7 +693,14 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         return rc;
     }
     {
-        hipError_t e = hipMemset(m.attn_done, 0, B * d.nkv * 4);
+        hipError_t e = hipHostMalloc((void**)&m.h_hidden, B * d.h * 4, hipHostMallocDefault);
+        if (e == hipSuccess) e = hipHostMalloc((void**)&m.h_pos, B * 2 * 4, hipHostMallocDefault);
+        if (e != hipSuccess) {
+            free_model(m);
+            return fail(OXB_HIP_OUT_OF_MEMORY, "out of host memory: pinned staging of %zu bytes", B * d.h * 4);
+        }
+        m.h_tokens = m.h_pos + B;
+        e = hipMemset(m.attn_done, 0, B * d.nkv * 4);
         if (e != hipSuccess) {
             free_model(m);
             return hip_fail(e, "counter clear");
@@ -971,14 +986,18 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + 1));
     OXB_TRY(kv_sync_table(m));
     hipStream_t st = g_rt.stream;
-    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
-    OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    // (the previous call ended with a stream synchronisation, so the staging buffers are free)
+    memcpy(m.h_hidden, hidden, (size_t)d.batch * d.h * 4);
+    memcpy(m.h_pos, pos, (size_t)d.batch * 4);
+    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, m.h_hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
+    OXB_TRY_HIP(hipMemcpyAsync(m.pos, m.h_pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
     OXB_TRY(run_decode_step(m));
-    if (token_out) OXB_TRY_HIP(hipMemcpyAsync(token_out, m.tokens, (size_t)d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
+    if (token_out) OXB_TRY_HIP(hipMemcpyAsync(m.h_tokens, m.tokens, (size_t)d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
     if (logits_or_null)
         OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits, (size_t)d.batch * d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: decode: %s", hipGetErrorString(e));
+    if (token_out) memcpy(token_out, m.h_tokens, (size_t)d.batch * 4);
     return OXB_HIP_OK;
     OXB_API_END
 }
