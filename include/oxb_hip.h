@@ -49,7 +49,8 @@ int  oxb_hip_device_count(void);
 int  oxb_hip_device_info(char* name, size_t name_cap, size_t* free_bytes, size_t* total_bytes);
 /* GpuBackendTrait::synchronize (KG/mod.rs:403) */
 int  oxb_hip_synchronize(void);
-/* Run on the caller's HIP stream (hipStream_t passed as void*); NULL restores the library's own stream. */
+/* Run on the caller's HIP stream (hipStream_t passed as void*); NULL restores the library's own stream.
+ * The decode step's graph is recorded on the library's own stream and replayed on the stream in use. */
 int  oxb_hip_set_stream(void* hip_stream);
 const char* oxb_hip_last_error(void);
 

@@ -931,6 +931,16 @@ int oxb_hip_model_reset(uint64_t model) {
     OXB_API_END
 }
 
+static bool stream_is_capturing(hipStream_t st) {
+    if (st == g_rt.own_stream) return false;
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(st, &cs) != hipSuccess) {
+        (void)hipGetLastError();
+        return true;  // unknown: launch plainly
+    }
+    return cs != hipStreamCaptureStatusNone;
+}
+
 // One decode step on m.hidden / m.pos (device): replayed from the captured graph, captured on first use, or launched
 // kernel by kernel when capture is off or failed.
 static int run_decode_step(Model& m) {
@@ -944,19 +954,24 @@ static int run_decode_step(Model& m) {
     }
     if (m.graph_exec) {
         OXB_TRY_HIP(hipGraphLaunch(m.graph_exec, st), "graph launch");
-    } else if (!m.graph_failed && st == g_rt.own_stream) {
-        // capture the whole token once; on any capture problem fall back to plain launches for good
+    } else if (!m.graph_failed && !stream_is_capturing(st)) {
+        // Capture the whole token once; on any capture problem fall back to plain launches for good.  The capture
+        // records on the library's own stream (nothing runs there); the graph is replayed on the stream in use, so a
+        // caller that set its own stream gets the replay too.  A caller's stream that is itself being captured takes
+        // the plain launches into the caller's graph.
         hipGraph_t graph = nullptr;
         m.graph_gen = g_rt.weights_gen;
-        hipError_t e = hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal);
+        g_rt.stream = g_rt.own_stream;
+        hipError_t e = hipStreamBeginCapture(g_rt.own_stream, hipStreamCaptureModeThreadLocal);
         int rc = OXB_HIP_OK;
         if (e == hipSuccess) {
             rc = encode_decode_step(m, true);
-            hipError_t e2 = hipStreamEndCapture(st, &graph);
+            hipError_t e2 = hipStreamEndCapture(g_rt.own_stream, &graph);
             if (rc == OXB_HIP_OK && e2 == hipSuccess && graph) e = hipGraphInstantiate(&m.graph_exec, graph, nullptr, nullptr, 0);
             else e = e2 == hipSuccess ? hipErrorUnknown : e2;
             if (graph) (void)hipGraphDestroy(graph);
         }
+        g_rt.stream = st;
         if (rc) return rc;
         if (e != hipSuccess || !m.graph_exec) {
             (void)hipGetLastError();

@@ -134,3 +134,37 @@ def test_replacing_or_freeing_a_weight_of_a_live_model(backend):
         assert np.all(np.isfinite(got))
     finally:
         gpu.close()
+
+
+def test_graph_replay_on_a_stream_the_caller_set(backend):
+    """The token's graph is recorded on the library's own stream and replayed on whichever stream is in use: a caller
+    that hands in its own stream gets the replay, and the same logits as on the library's stream."""
+    import ctypes as C
+
+    from oxibonsai_amd import _lib
+    cfg = dict(fmt=Q1, n_layers=2, h=256, inter=512, nq=4, nkv=2, hd=64, vocab=96, max_seq=32, eps=1e-6, rope_theta=1e6)
+    w = synth.make_model(cfg, 910)
+    rows = [synth.embedding_rows(911, [i], cfg["h"])[0] * 50.0 for i in range(5)]
+    ref = HipModel(backend, cfg, w, batch=1)
+    try:
+        want = [ref.forward(r, i)[0][0].copy() for i, r in enumerate(rows)]
+        assert ref.uses_graph()
+    finally:
+        ref.close()
+    L = _lib.lib()
+    hip = C.CDLL("libamdhip64.so.7")      # the runtime the library is linked against, already loaded
+    stream = C.c_void_p()
+    assert hip.hipStreamCreateWithFlags(C.byref(stream), C.c_uint(1)) == 0 and stream.value    # hipStreamNonBlocking
+    assert L.oxb_hip_set_stream(stream) == 0
+    try:
+        gpu = HipModel(backend, cfg, w, batch=1)
+        try:
+            for i, r in enumerate(rows):
+                got = gpu.forward(r, i)[0][0]
+                assert np.array_equal(got, want[i]), i
+            assert gpu.uses_graph()
+        finally:
+            gpu.close()
+    finally:
+        assert L.oxb_hip_set_stream(None) == 0
+        assert hip.hipStreamDestroy(stream) == 0
