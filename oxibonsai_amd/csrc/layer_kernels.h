@@ -57,4 +57,9 @@ hipError_t oxb_launch_attn_decode(const OxbAttnParams& p, uint32_t batch, hipStr
 hipError_t oxb_launch_rmsnorm(const float* d_x, const float* d_w, uint32_t n, uint32_t nvec, float eps, float* d_out, hipStream_t st);
 // d_ws: batch * OXB_ARGMAX_MAX_PARTS * 8 bytes of scratch for the per-span maxima.
 #define OXB_ARGMAX_MAX_PARTS 256u
-hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st);
+// host_copy_or_null: pinned host memory that receives the token ids too (readable after the stream is synchronised)
+hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st,
+                             uint32_t* host_copy_or_null = nullptr);
+// hidden rows (n_floats, a multiple of 4) and positions from pinned host memory to their device buffers, one launch
+hipError_t oxb_launch_stage_in(const float* h_hidden, uint32_t n_floats, const uint32_t* h_pos, uint32_t n_pos, float* d_hidden,
+                               uint32_t* d_pos, hipStream_t st);

@@ -183,6 +183,13 @@ hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n
 // stores them to the cache and, after a barrier, reads them back like any other row.
 // ---------------------------------------------------------------------------
 typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
+typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
+// ds_read_b64_tr_b16: each lane gives the LDS address of four consecutive halves; within every block of 16 lanes these
+// are the rows of a 4 x 16 tile (lane i: row i / 4, columns 4 (i % 4) .. + 3), and lane j gets column j of the tile.
+__device__ __forceinline__ v4h_t lds_read_tr16(const _Float16* q) {
+    typedef short v4s_t __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(v4h_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)q));
+}
 
 // Options of the kernel (template KVM, fields window / sinks):
 //  * quantised cache rows (kv_quant_device.h): one byte per value plus an f32 scale per row.  The codes enter the
@@ -193,6 +200,7 @@ typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
 //  * sliding window with attention sinks (is_in_window, crates/oxibonsai-model/src/layers/sliding_window.rs:173-189):
 //    the first `sinks` keys stay visible, the others while pos - key < window - sinks; chunks without a visible key
 //    are not walked.  window == 0: every key up to pos is visible.
+#define OXB_ATTN_MERGE_LDS_BYTES(heads_per) ((heads_per) * 65 * 4 + 12 + 256 * 16)  // LDS attn_merge_heads needs
 __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_t b, uint32_t h_first, uint32_t nh, uint32_t heads_per,
                                                  float* sm, float* __restrict__ out);
 
@@ -226,7 +234,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     __shared__ uint32_t last_flag;
     __shared__ __attribute__((aligned(16))) _Float16 kv_new[2][HD];  // the new position's K and V rows as stored (fp16 cache)
     static_assert(sizeof(vs_all) >= 16 * HD * sizeof(float), "Q must fit in the V slices");
-    static_assert(sizeof(vs_all) >= 16 * 65 * sizeof(float), "the merge's slot weights must fit in the V slices");
+    static_assert(sizeof(vs_all) >= OXB_ATTN_MERGE_LDS_BYTES(16), "the merge's slot weights and partial sums must fit in the V slices");
     float* qs = reinterpret_cast<float*>(&vs_all[0][0]);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -617,9 +625,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         // O^T += V^T P^T; A operand gathered from the staged block
 #pragma unroll
         for (int sl = 0; sl < NS; sl++) {
-            v8h_t a;
-#pragma unroll
-            for (int e = 0; e < 8; e++) a[e] = vs[(e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) * VSTR + 16 * sl + qi];
+            // a[e] = V[4 g + e][16 sl + qi], a[4 + e] = V[16 + 4 g + e][16 sl + qi]: two transposing LDS reads.  The 16 lanes
+            // of a block hand in the addresses of a 4 x 16 tile (lane i: row i / 4, columns 4 (i % 4) .. + 3) and lane j
+            // receives column j.
+            const _Float16* tile = vs + (4 * g + (qi >> 2)) * VSTR + 16 * sl + 4 * (qi & 3u);
+            const v4h_t t0 = lds_read_tr16(tile), t1 = lds_read_tr16(tile + 16 * VSTR);
+            const v8h_t a = {t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
 #pragma unroll
             for (int v = 0; v < 4; v++) O[sl][v] *= alpha;
             O[sl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, ph, O[sl], 0, 0, 0);
@@ -670,8 +681,12 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
 
 // Merge the slot results of heads h_first .. h_first + nh - 1 of sequence b into the attention output
 // [batch][nq * hd] (fp32), the input of the O projection, by the 256 threads of a workgroup: per head one wave works
-// out the softmax weights of the slots (one slot per lane), then every thread adds the weighted slot outputs of four
-// dimensions in ascending slot order.  sm: (heads_per * 65) floats of LDS: [head][64] slot weights | [head] 1 / sum.
+// out the softmax weights of the slots (one slot per lane); the weighted slot outputs of a group of four dimensions
+// are added by NPAR threads, thread j taking slots j, j + NPAR, ... in ascending order, and the NPAR sums meet in LDS
+// in thread order.  Every thread requests its first 16 slot outputs before the weights are worked out; NPAR is the
+// smallest of 1, 2, 4 that covers the slots in use with those requests (one round trip to memory for the whole merge),
+// as far as 256 threads allow for the heads' nh * hd / 4 groups.
+// sm: heads_per * 65 floats of LDS ([head][64] slot weights | [head] 1 / sum), then 256 float4 for the partial sums.
 // The slot results were written by other workgroups of this same launch: agent-coherent loads.
 __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_t b, uint32_t h_first, uint32_t nh, uint32_t heads_per,
                                                  float* sm, float* __restrict__ out) {
@@ -679,7 +694,8 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
     const uint32_t stride = hd + OXB_ATTN_PART_PAD;
     float* wts = sm;
     float* inv_l = wts + heads_per * 64;
-    const uint32_t e0 = h_first * hd, e1 = e0 + nh * hd;
+    float4* sums = reinterpret_cast<float4*>(sm + ((heads_per * 65 + 3) & ~3u));
+    const uint32_t e0 = h_first * hd;
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
     const float* part = p.part + (size_t)b * p.nq * p.n_splits * stride;
@@ -689,16 +705,21 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
         return make_float4(v.x, v.y, v.z, v.w);
     };
     auto ld1 = [&](const float* q) -> float { return buf_load_f32_coherent(r_part, (uint32_t)(q - part) * 4u); };
-    // The first slots' partial outputs of this thread's first four elements do not depend on the slot weights:
-    // request them before the weights are worked out, so that both round trips to memory overlap.
-    constexpr int PRE = 8;
+    const uint32_t groups = nh * hd / 4;
+    // as few threads per group as keep all slots within the first 16 requests (more would only add the LDS step)
+    const uint32_t npar_max = groups <= 64 ? 4u : groups <= 128 ? 2u : 1u;
+    const uint32_t npar = used <= 16u || npar_max == 1u ? 1u : (used <= 32u || npar_max == 2u ? 2u : 4u);
+    const uint32_t tg = 256u / npar, sh = tid / tg, egl = tid % tg;  // this thread: group egl (+ tg, ...), slots sh + npar u
+    constexpr int PRE = 16;
     float4 pre[PRE];
     {
-        const uint32_t e = e0 + tid * 4;
+        const uint32_t e = e0 + egl * 4;
         const float* ph = part + (size_t)(e / hd) * p.n_splits * stride + e % hd;
 #pragma unroll
-        for (int u = 0; u < PRE; u++)
-            pre[u] = (e < e1 && (uint32_t)u < used) ? ld4(ph + (size_t)u * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int u = 0; u < PRE; u++) {
+            const uint32_t sl = sh + npar * u;
+            pre[u] = (egl < groups && sl < used) ? ld4(ph + (size_t)sl * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
     for (uint32_t hh = tid >> 6; hh < nh; hh += 4) {
         const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
@@ -714,37 +735,49 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
         if (lane == 0) inv_l[hh] = L > 0.f ? 1.0f / L : 0.f;
     }
     __syncthreads();
-    for (uint32_t e = e0 + tid * 4; e < e1; e += 1024) {
-        const uint32_t h = e / hd, d = e % hd, hh = h - h_first;
+    for (uint32_t eg0 = 0; eg0 < groups; eg0 += tg) {  // uniform trip count: the barrier below is reached by every thread
+        const uint32_t eg = eg0 + egl, e = e0 + eg * 4;
+        const bool live = eg < groups;
+        const uint32_t h = live ? e / hd : h_first, d = e % hd, hh = h - h_first;
         const float* ph = part + (size_t)h * p.n_splits * stride + d;
         float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
-        // slots are added in ascending order, PRE requests in flight at a time
-        auto fold = [&](const float4 (&v)[PRE], uint32_t s0) {
+        // PRE requests in flight at a time; slots past `used` count as zeros with weight 0
+        auto fold = [&](const float4 (&v)[PRE], uint32_t u0) {
 #pragma unroll
             for (int u = 0; u < PRE; u++) {
-                const float w = s0 + u < used ? wts[hh * 64 + s0 + u] : 0.f;  // (slots past `used` were loaded as zeros)
+                const uint32_t sl = sh + npar * (u0 + u);
+                const float w = sl < used ? wts[hh * 64 + sl] : 0.f;
                 acc.x = fmaf(v[u].x, w, acc.x), acc.y = fmaf(v[u].y, w, acc.y), acc.z = fmaf(v[u].z, w, acc.z), acc.w = fmaf(v[u].w, w, acc.w);
             }
         };
-        uint32_t s = 0;
-        if (e == e0 + tid * 4) {  // the element group whose first slots are already here
+        uint32_t u0 = 0;
+        if (eg0 == 0) {  // the group whose first slots are already here
             fold(pre, 0);
-            s = PRE;
+            u0 = PRE;
         }
-        for (; s + PRE <= used; s += PRE) {
+        for (; live && sh + npar * u0 < used; u0 += PRE) {
             float4 v[PRE];
 #pragma unroll
-            for (int u = 0; u < PRE; u++) v[u] = ld4(ph + (size_t)(s + u) * stride);
-            fold(v, s);
+            for (int u = 0; u < PRE; u++) {
+                const uint32_t sl = sh + npar * (u0 + u);
+                v[u] = sl < used ? ld4(ph + (size_t)sl * stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+            fold(v, u0);
         }
-        for (; s < used; s++) {
-            const float4 v = ld4(ph + (size_t)s * stride);
-            const float w = wts[hh * 64 + s];
-            acc.x = fmaf(v.x, w, acc.x), acc.y = fmaf(v.y, w, acc.y), acc.z = fmaf(v.z, w, acc.z), acc.w = fmaf(v.w, w, acc.w);
+        if (npar > 1) {  // (then all groups fit one pass)
+            if (sh) sums[tid] = acc;
+            __syncthreads();
+            if (!sh)
+                for (uint32_t j = 1; j < npar; j++) {
+                    const float4 o = sums[j * tg + egl];
+                    acc.x += o.x, acc.y += o.y, acc.z += o.z, acc.w += o.w;
+                }
         }
-        const float il = inv_l[hh];
-        acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
-        *reinterpret_cast<float4*>(out + (size_t)b * qd + e) = acc;
+        if (live && !sh) {
+            const float il = inv_l[hh];
+            acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
+            *reinterpret_cast<float4*>(out + (size_t)b * qd + e) = acc;
+        }
     }
 }
 
@@ -781,13 +814,37 @@ __global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __rest
 }
 
 __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pv, const uint32_t* __restrict__ pi,
-                                                           uint32_t parts, uint32_t* __restrict__ out) {
+                                                           uint32_t parts, uint32_t* __restrict__ out, uint32_t* __restrict__ host_copy) {
     float best = -INFINITY;
     uint32_t idx = 0xFFFFFFFFu;
     for (uint32_t i = threadIdx.x; i < parts; i += 64) argmax_merge(best, idx, pv[blockIdx.x * parts + i], pi[blockIdx.x * parts + i]);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) argmax_merge(best, idx, __shfl_xor(best, o, 64), __shfl_xor(idx, o, 64));
-    if (threadIdx.x == 0) out[blockIdx.x] = idx == 0xFFFFFFFFu ? 0u : idx;
+    if (threadIdx.x == 0) {
+        out[blockIdx.x] = idx == 0xFFFFFFFFu ? 0u : idx;
+        if (host_copy) {  // pinned host memory: the caller reads it after synchronising, without a copy of its own
+            host_copy[blockIdx.x] = idx == 0xFFFFFFFFu ? 0u : idx;
+            __threadfence_system();
+        }
+    }
+}
+
+// Pinned host staging -> device: the hidden rows and positions of a decode call, in one launch ahead of the step's
+// graph (two small asynchronous copies cost more than the step's first kernel).
+__global__ __launch_bounds__(256) void stage_in_kernel(const float4* __restrict__ h_hidden, uint32_t n4, const uint32_t* __restrict__ h_pos,
+                                                        uint32_t n_pos, float4* __restrict__ hidden, uint32_t* __restrict__ pos) {
+    const uint32_t i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) hidden[i] = h_hidden[i];
+    if (i < n_pos) pos[i] = h_pos[i];
+}
+
+hipError_t oxb_launch_stage_in(const float* h_hidden, uint32_t n_floats, const uint32_t* h_pos, uint32_t n_pos, float* d_hidden,
+                               uint32_t* d_pos, hipStream_t st) {
+    if ((n_floats & 3u) || n_floats == 0) return hipErrorInvalidValue;
+    const uint32_t n4 = n_floats / 4, n = n4 > n_pos ? n4 : n_pos;
+    hipLaunchKernelGGL(stage_in_kernel, dim3((n + 255) / 256), dim3(256), 0, st, reinterpret_cast<const float4*>(h_hidden), n4, h_pos, n_pos,
+                       reinterpret_cast<float4*>(d_hidden), d_pos);
+    return hipGetLastError();
 }
 
 // ---------------------------------------------------------------------------
@@ -870,12 +927,13 @@ uint32_t oxb_argmax_parts(uint32_t n) {
     return p < 1 ? 1 : (p > OXB_ARGMAX_MAX_PARTS ? OXB_ARGMAX_MAX_PARTS : p);
 }
 
-hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st) {
+hipError_t oxb_launch_argmax(const float* d_logits, uint32_t n, uint32_t batch, uint32_t* d_out, void* d_ws, hipStream_t st,
+                             uint32_t* host_copy_or_null) {
     if (n == 0 || batch == 0 || !d_ws) return hipErrorInvalidValue;
     const uint32_t parts = oxb_argmax_parts(n), span = (n + parts - 1) / parts;
     float* pv = reinterpret_cast<float*>(d_ws);
     uint32_t* pi = reinterpret_cast<uint32_t*>(d_ws) + (size_t)batch * parts;
     hipLaunchKernelGGL(argmax_partial_kernel, dim3(parts, batch), dim3(256), 0, st, d_logits, n, span, pv, pi);
-    hipLaunchKernelGGL(argmax_final_kernel, dim3(batch), dim3(64), 0, st, pv, pi, parts, d_out);
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(batch), dim3(64), 0, st, pv, pi, parts, d_out, host_copy_or_null);
     return hipGetLastError();
 }

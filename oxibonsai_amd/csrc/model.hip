@@ -378,7 +378,7 @@ static int encode_decode_step_gemm(Model& m) {
     const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
     if (rc) return rc;
     OXB_TRY(gemm_device(*lm, m.hidden, d.h, m.logits, B, d.vocab, OXB_GEMM_STORE, nullptr, OXB_PACK_RMSNORM, final_norm, d.eps, &m.gws));
-    OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, B, m.tokens, m.argmax_ws, st), "kernel launch failed: argmax");
+    OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, B, m.tokens, m.argmax_ws, st, m.h_tokens), "kernel launch failed: argmax");
     return OXB_HIP_OK;
 }
 
@@ -422,7 +422,7 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
             OXB_TRY(gemv_launch(*lm, m.hidden + (size_t)b0 * d.h, d.h, nb, m.logits + (size_t)b0 * d.vocab, d.vocab,
                                 OXB_GEMV_PRO_RMSNORM, final_norm, d.eps, OXB_GEMV_STORE, nullptr));
         }
-        OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, m.argmax_ws, st), "kernel launch failed: argmax");
+        OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, m.argmax_ws, st, m.h_tokens), "kernel launch failed: argmax");
     }
     return OXB_HIP_OK;
 }
@@ -693,8 +693,8 @@ int oxb_hip_model_create(const oxb_model_desc* desc, uint64_t* model) {
         return rc;
     }
     {
-        hipError_t e = hipHostMalloc((void**)&m.h_hidden, B * d.h * 4, hipHostMallocDefault);
-        if (e == hipSuccess) e = hipHostMalloc((void**)&m.h_pos, B * 2 * 4, hipHostMallocDefault);
+        hipError_t e = hipHostMalloc((void**)&m.h_hidden, B * d.h * 4, hipHostMallocCoherent);
+        if (e == hipSuccess) e = hipHostMalloc((void**)&m.h_pos, B * 2 * 4, hipHostMallocCoherent);
         if (e != hipSuccess) {
             free_model(m);
             return fail(OXB_HIP_OUT_OF_MEMORY, "out of host memory: pinned staging of %zu bytes", B * d.h * 4);
@@ -1004,10 +1004,9 @@ int oxb_hip_decode(uint64_t model, const float* hidden, const uint32_t* pos, flo
     // (the previous call ended with a stream synchronisation, so the staging buffers are free)
     memcpy(m.h_hidden, hidden, (size_t)d.batch * d.h * 4);
     memcpy(m.h_pos, pos, (size_t)d.batch * 4);
-    OXB_TRY_HIP(hipMemcpyAsync(m.hidden, m.h_hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
-    OXB_TRY_HIP(hipMemcpyAsync(m.pos, m.h_pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
+    // one kernel reads the pinned rows and positions; the step's last kernel leaves the token ids in pinned memory too
+    OXB_TRY_HIP(oxb_launch_stage_in(m.h_hidden, d.batch * d.h, m.h_pos, d.batch, m.hidden, m.pos, st), "kernel launch failed: stage_in");
     OXB_TRY(run_decode_step(m));
-    if (token_out) OXB_TRY_HIP(hipMemcpyAsync(m.h_tokens, m.tokens, (size_t)d.batch * 4, hipMemcpyDeviceToHost, st), "token download");
     if (logits_or_null)
         OXB_TRY_HIP(hipMemcpyAsync(logits_or_null, m.logits, (size_t)d.batch * d.vocab * 4, hipMemcpyDeviceToHost, st), "logits download");
     hipError_t e = hipStreamSynchronize(st);

@@ -208,14 +208,20 @@ class HipModel:
 
     def forward(self, hidden, pos, want_logits: bool = True):
         """hidden: [batch, h] embedding rows; pos: [batch] positions -> (logits [batch, vocab] or None, tokens [batch])."""
-        hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(self.batch, self.cfg["h"])
-        pv = np.ascontiguousarray(np.broadcast_to(np.asarray(pos, dtype=np.uint32), (self.batch,)))
+        n = self.batch * self.cfg["h"]
+        if type(hidden) is np.ndarray and hidden.dtype == np.float32 and hidden.size == n and hidden.flags.c_contiguous:
+            hv = hidden             # (the per-token call of a decode loop: nothing to convert)
+        else:
+            hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(self.batch, self.cfg["h"])
+        io = self.__dict__.get("_io")
+        if io is None:      # position and token arrays of the calls, with their pointers
+            pb, tb = np.zeros(self.batch, dtype=np.uint32), np.zeros(self.batch, dtype=np.uint32)
+            io = self._io = (pb, tb, pb.ctypes.data_as(_lib.u32p), tb.ctypes.data_as(_lib.u32p))
+        io[0][:] = pos      # a scalar, or one position per sequence
         logits = np.empty((self.batch, self.cfg["vocab"]), dtype=np.float32) if want_logits else None
-        tokens = np.empty(self.batch, dtype=np.uint32)
-        _check(self._lib.oxb_hip_decode(self.id, hv.ctypes.data_as(_lib.f32p), pv.ctypes.data_as(_lib.u32p),
-                                        logits.ctypes.data_as(_lib.f32p) if want_logits else None,
-                                        tokens.ctypes.data_as(_lib.u32p)))
-        return logits, tokens
+        _check(self._lib.oxb_hip_decode(self.id, hv.ctypes.data_as(_lib.f32p), io[2],
+                                        logits.ctypes.data_as(_lib.f32p) if want_logits else None, io[3]))
+        return logits, io[1].copy()
 
     def forward_hidden(self, hidden, pos) -> np.ndarray:
         """All layers and the final norm, no LM head (try_cuda_full_forward, gpu_backend/cuda_full_layer/encode_q1.rs:813):
