@@ -43,6 +43,16 @@ __device__ __forceinline__ uint32_t buf_load_b32(__amdgpu_buffer_rsrc_t r, uint3
 // prefetched weight tiles) stay in flight across it.
 __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
+// ds_read_b64_tr_b16, the transposing LDS read of gfx950: each lane gives the address of four consecutive halves;
+// within every block of 16 lanes these are the rows of a 4 x 16 tile (lane i: row i / 4, columns 4 (i % 4) .. + 3),
+// and lane j receives column j of the tile (rows 0 .. 3).  It turns a row-major [key][d] block into the matrix cores'
+// operand layout (k = key contiguous per lane) without 2-byte gathers.
+typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ v4h_t lds_read_tr16(const _Float16* q) {
+    typedef short v4s_t __attribute__((ext_vector_type(4)));
+    return __builtin_bit_cast(v4h_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)q));
+}
+
 
 // Agent-coherent accesses (the sc1 cache-policy bit): the store is written through to memory, the load is served from
 // memory and not from this CU's L1 or this XCD's L2.  Data that other workgroups of the same launch produce and

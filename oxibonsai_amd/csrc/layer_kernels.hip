@@ -183,13 +183,6 @@ hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n
 // stores them to the cache and, after a barrier, reads them back like any other row.
 // ---------------------------------------------------------------------------
 typedef _Float16 v8h_t __attribute__((ext_vector_type(8)));
-typedef _Float16 v4h_t __attribute__((ext_vector_type(4)));
-// ds_read_b64_tr_b16: each lane gives the LDS address of four consecutive halves; within every block of 16 lanes these
-// are the rows of a 4 x 16 tile (lane i: row i / 4, columns 4 (i % 4) .. + 3), and lane j gets column j of the tile.
-__device__ __forceinline__ v4h_t lds_read_tr16(const _Float16* q) {
-    typedef short v4s_t __attribute__((ext_vector_type(4)));
-    return __builtin_bit_cast(v4h_t, __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) v4s_t*)q));
-}
 
 // Options of the kernel (template KVM, fields window / sinks):
 //  * quantised cache rows (kv_quant_device.h): one byte per value plus an f32 scale per row.  The codes enter the

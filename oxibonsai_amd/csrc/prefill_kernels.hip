@@ -258,9 +258,10 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
         m_run = m_new;
 #pragma unroll
         for (int sl = 0; sl < NS; sl++) {
-            v8h a;
-#pragma unroll
-            for (int e = 0; e < 8; e++) a[e] = vb[(e < 4 ? 4 * g + e : 16 + 4 * g + e - 4) * STR + 16 * sl + qi];
+            // a[e] = V[4 g + e][16 sl + qi], a[4 + e] = V[16 + 4 g + e][16 sl + qi]: two transposing reads
+            const _Float16* tile = vb + (4 * g + (qi >> 2)) * STR + 16 * sl + 4 * (qi & 3u);
+            const v4h_t t0 = lds_read_tr16(tile), t1 = lds_read_tr16(tile + 16 * STR);
+            const v8h a = {t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
 #pragma unroll
             for (int v = 0; v < 4; v++) O[sl][v] *= alpha;
             O[sl] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, pb, O[sl], 0, 0, 0);
