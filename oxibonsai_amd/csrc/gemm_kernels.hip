@@ -320,7 +320,7 @@ __device__ __forceinline__ void block_steps(const v8h* __restrict__ xsb, v8h (&A
 }
 
 template <int FMT, int RT, int CT>
-__global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGemmParams p) {
+__global__ __launch_bounds__(OXB_GEMM_THREADS, RT == 3 ? 2 : 1) void gemm_mfma_kernel(const OxbGemmParams p) {
     constexpr int BM = 16 * CT;
     // two stages of the token tile: [chunk 4g+s][token] x 16 bytes.  Separate arrays, so that loads in flight
     // into one stage do not make reads of the other wait.
@@ -334,15 +334,27 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     const uint32_t sb0 = ks * p.sb_per_split, sb1 = min(sb0 + p.sb_per_split, p.n_sb);
     // row tiles: the workgroup's [wg_t0, wg_t1), split evenly over the four waves
     const uint32_t wg_t0 = n_g * p.tpw, wg_t1 = min(wg_t0 + p.tpw, p.n_tiles);
-    const uint32_t per = (p.tpw + 3u) / 4u;  // <= RT
-    const uint32_t t0 = wg_t0 + wave * per;
-    const uint32_t t1 = min(t0 + per, wg_t1);
-    const uint32_t n_valid = t1 > t0 ? t1 - t0 : 0u;
-    // SWIGLU mode (the matrix is gate || up): the tile sequence interleaves gate tile j and up tile j, and every
-    // wave starts on a gate tile (the launcher gives it an even count), so accumulators 2q and 2q+1 hold both
-    // factors of 16 output rows.
+    // SWIGLU mode (the matrix is gate || up).  Even RT: the tile sequence interleaves gate tile j and up tile j, and
+    // every wave starts on a gate tile (the launcher gives it an even count), so accumulators 2q and 2q+1 hold both
+    // factors of 16 output rows.  Odd RT (three tiles per wave, the count that still runs two workgroups per CU): waves 0
+    // and 1 take RT gate tiles each, waves 2 and 3 the up tiles of the same rows; the up factors cross over through the
+    // LDS stages once the K loop is done.
     const bool sw = p.mode == OXB_GEMM_SWIGLU;
+    constexpr bool SPLIT = RT == 3;  // (of the SWIGLU mode; other odd counts are never launched in it)
     auto tile_of = [&](uint32_t u) -> uint32_t { return sw ? ((u & 1u) ? p.n_tiles / 2 + (u >> 1) : (u >> 1)) : u; };
+    uint32_t t0 = 0, n_valid = 0, up_base = 0;  // first tile index of this wave (an index into tile_of, or with SPLIT a gate tile)
+    if (sw && SPLIT) {
+        const uint32_t half_tiles = p.n_tiles / 2, g_first = n_g * (2 * RT) + (wave & 1u) * RT;
+        t0 = g_first;
+        n_valid = g_first < half_tiles ? min((uint32_t)RT, half_tiles - g_first) : 0u;
+        up_base = (wave >> 1) ? half_tiles : 0u;
+    } else {
+        const uint32_t per = (p.tpw + 3u) / 4u;  // <= RT
+        t0 = wg_t0 + wave * per;
+        const uint32_t t1 = min(t0 + per, wg_t1);
+        n_valid = t1 > t0 ? t1 - t0 : 0u;
+    }
+    auto tile_at = [&](uint32_t rt) -> uint32_t { return (sw && SPLIT) ? up_base + t0 + rt : tile_of(t0 + rt); };
 
     const __amdgpu_buffer_rsrc_t rc = make_rsrc(p.codes, p.codes_bytes), rs = make_rsrc(p.scales, p.scales_bytes);
     const __amdgpu_buffer_rsrc_t rx = make_rsrc(p.xh, p.xh_bytes);
@@ -388,8 +400,8 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
     stage_x(sb0 * 4, xs0);
 #pragma unroll
     for (int rt = 0; rt < RT; rt++) {
-        load_half<FMT>(H[rt][0], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
-        load_half<FMT>(H[rt][1], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
+        load_half<FMT>(H[rt][0], rc, rs, tile_at(rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 0, lane);
+        load_half<FMT>(H[rt][1], rc, rs, tile_at(rt), (uint32_t)rt < n_valid, p.n_sb, sb0, 1, lane);
     }
     publish();
     BlockDec bd[RT], bdn[RT];
@@ -417,7 +429,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             bdn[rt] = prepare_block<FMT>(H[rt][1], 0);
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][0], rc, rs, tile_at(rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 0, lane);
         if (KEEP_W) __builtin_amdgcn_sched_barrier(0);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
         publish_keep_weights();
@@ -439,7 +451,7 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
             bdn[rt] = prepare_block<FMT>(H[rt][0], 0);
         }
 #pragma unroll
-        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, tile_of(t0 + rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
+        for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][1], rc, rs, tile_at(rt), (uint32_t)rt < n_valid, p.n_sb, sb + 1, 1, lane);
         if (KEEP_W) __builtin_amdgcn_sched_barrier(0);
         block_steps<FMT, RT, CT>(x1, A, bd, bdn, acc, boff);
         publish_keep_weights();
@@ -449,6 +461,55 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS) void gemm_mfma_kernel(const OxbGe
 
     // epilogue: lane holds rows 4g..4g+3 of the row tile for token 16ct + r
     const bool vec_ok = (p.ldy & 3u) == 0;
+    if (sw && SPLIT) {
+        // The K loop ended behind a barrier with no stage load in flight: both stages are free.  Up waves leave their
+        // factors (already scaled back by the row's power of two) in the stage of their half, tile by tile as
+        // [rt][ct][lane] float4; the gate waves of the same half pick them up.
+        float4* ex = reinterpret_cast<float4*>((wave & 1u) ? xs1 : xs0);
+        static_assert(!SPLIT || (size_t)RT * CT * 64 * 16 <= sizeof(xs0), "the up factors of a wave fit a stage");
+        if (wave >> 1) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ct++) {
+                const uint32_t m = m0 + ct * 16 + r;
+                const int e = m < p.M ? p.xsh[m] : 0;
+#pragma unroll
+                for (int rt = 0; rt < RT; rt++) {
+                    float u[4];
+#pragma unroll
+                    for (int v = 0; v < 4; v++) u[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(acc[rt][ct][v], e);
+                    ex[(rt * CT + ct) * 64 + lane] = make_float4(u[0], u[1], u[2], u[3]);
+                }
+            }
+        }
+        __syncthreads();
+        if (wave >> 1) return;
+#pragma unroll
+        for (int ct = 0; ct < CT; ct++) {
+            const uint32_t m = m0 + ct * 16 + r;
+            if (m >= p.M) continue;
+            const int e = p.xsh[m];
+            float* yr = p.y + (size_t)m * p.ldy;
+#pragma unroll
+            for (int rt = 0; rt < RT; rt++) {
+                if ((uint32_t)rt >= n_valid) continue;
+                const uint32_t n = (t0 + rt) * 16 + 4 * g, n_lim = p.n_rows / 2;
+                const float4 u = ex[(rt * CT + ct) * 64 + lane];
+                const float uu[4] = {u.x, u.y, u.z, u.w};
+                float o[4];
+#pragma unroll
+                for (int v = 0; v < 4; v++)
+                    o[v] = silu_mul(e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(acc[rt][ct][v], e), uu[v]);
+                if (vec_ok && n + 3 < n_lim) {
+                    *reinterpret_cast<float4*>(yr + n) = make_float4(o[0], o[1], o[2], o[3]);
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 4; v++)
+                        if (n + v < n_lim) yr[n + v] = o[v];
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int ct = 0; ct < CT; ct++) {
         const uint32_t m = m0 + ct * 16 + r;
@@ -711,7 +772,7 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
             // CU, whose starts and epilogues overlap) measured faster than two pairs (308 registers, one workgroup per
             // CU) on both quoted gate || up shapes at 2048 tokens: 24576 x 4096 357 against 368 us, 12288 x 2048 109
             // against 121 us.
-            if (sw && rt != 2) continue;
+            if (sw && rt != 2) continue;  // (three tiles per wave are considered below)
             for (uint32_t tpw = 4 * rt; tpw > (sw ? 4 * rt - 1 : 4 * rt - 4); tpw--) {
                 const uint32_t groups = (p.n_tiles + tpw - 1) / tpw;
                 const uint64_t wgs = (uint64_t)groups * n_mt * ks;
@@ -729,6 +790,10 @@ static GemmPlan plan_gemm(const OxbGemmParams& p, uint32_t n_cus) {
         const uint64_t wgs = (uint64_t)((p.n_tiles + best.tpw - 1) / best.tpw) * n_mt;
         if (best.rt == 1 || wgs < n_cus) best = {1, 4, 1, p.n_sb, 4};
     }
+    // gate || up with three tiles per wave (two gate waves, two up waves; still two workgroups per CU): fewer LDS reads
+    // per MFMA than with two.  Measured at 2048 tokens (plain stores): 24576 x 4096 310 against 343 us, 19456 x 2560
+    // (TQ2) 181 against 193, 12288 x 2048 (TQ2) 92 against 101; taken where its workgroups still cover the CUs.
+    if (sw && (uint64_t)((p.n_tiles / 2 + 5) / 6) * n_mt >= n_cus) best = {3, 12, 1, p.n_sb, 8};
     return best;
 }
 

@@ -26,6 +26,9 @@ WIDE = dict(n_layers=1, h=256, inter=512, nq=2, nkv=2, hd=256, vocab=64, max_seq
 G4_HD32 = dict(n_layers=2, h=128, inter=256, nq=4, nkv=1, hd=32, vocab=64, max_seq=200, eps=1e-6, rope_theta=1e4)
 G4_HD256 = dict(n_layers=1, h=1024, inter=512, nq=4, nkv=1, hd=256, vocab=64, max_seq=96, eps=1e-6, rope_theta=1e6)
 G8_HD128 = dict(n_layers=1, h=1024, inter=512, nq=8, nkv=1, hd=128, vocab=64, max_seq=160, eps=1e-6, rope_theta=1e6)
+# an FFN wide enough (392 gate tiles x 4 token tiles of 128) for the gate || up GEMM to take three row tiles per wave, gate
+# and up tiles in different waves; 392 = 65 x 6 + 2 and 500 = 3 x 128 + 116: the last workgroups are partly empty
+LONG_FFN = dict(n_layers=1, h=256, inter=6272, nq=4, nkv=2, hd=64, vocab=64, max_seq=520, eps=1e-6, rope_theta=1e6)
 
 
 def _rows(seed, n, h):
@@ -50,7 +53,8 @@ def _check(got, want, tok):
 
 @pytest.mark.parametrize("fmt", [TQ2, Q1])
 @pytest.mark.parametrize("cfg,n", [(TINY, 8), (TINY, 17), (TINY, 33), (SMALL, 130), (MID, 70), (WIDE, 40),
-                                   (G4_HD32, 97), (G4_HD32, 32), (G4_HD256, 50), (G8_HD128, 100), (SMALL, 1), (SMALL, 65)])
+                                   (G4_HD32, 97), (G4_HD32, 32), (G4_HD256, 50), (G8_HD128, 100), (SMALL, 1), (SMALL, 65),
+                                   (LONG_FFN, 500)])
 def test_prefill_matches_sequential_oracle(backend, fmt, cfg, n):
     cfg = dict(cfg, fmt=fmt)
     w = synth.make_model(cfg, 100 + n)
