@@ -366,6 +366,263 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
     }
 }
 
+// ---------------------------------------------------------------------------
+// One activation vector, Q1 weights: the fp4 matrix-core route.
+//
+// v_mfma_scale_f32_16x16x128_f8f6f4 with both operands in fp4 (E2M1) multiplies a whole 128-weight block of 16 rows
+// in one instruction that takes as long as one of the two int8 instructions above, and an fp4 operand is a nibble:
+// the code dword of a lane ANDed with 0x11111111 << m is already four operands' worth - bit m of nibble i is weight
+// 4 i + m of the lane's 32, and the nibbles 0001 / 0010 / 0100 read 0.5 / 1 / 2 as E2M1 numbers (m = 0, 1, 2), while
+// (w & 0x88888888) | 0x22222222 reads -1 / +1 (m = 3).  So a block costs 3 ANDs and one AND-OR instead of 8 ANDs and a
+// shift.  The activation meets them as sixteen base-4 digits of a 32-bit magnitude with the sign in every digit: digit j
+// of all 128 activations is row j of the A operand, an E2M1 number d / 2 with d in 0..3.  |x| is scaled by a power of
+// two - one per K slice of a wave, as above - so that x = 2^(E - 30) X with |X| < 2^30, and the integer that is cut into
+// digits is X 2^(1 - s) for a weight whose set bit reads 2^s (the sum of b 2^s times it is twice the sum over the set
+// bits; the accumulator starts at minus the sum over all of them, which one extra MFMA per block against constant
+// operands computes in the prologue) and X with the opposite sign for m = 3.  Products and their sums over a block are
+// small multiples of 1/8: every matrix-core result is exact.  A lane then holds the block sums of digits 4 g .. 4 g + 3
+// for weight row c: four FMAs with the block's fp16 scale keep one fp32 accumulator per digit, four more per tile join
+// them with the digits' powers of four, and two lane exchanges add the four lane groups before the wave leaves its
+// sixteen row sums in LDS, where one wave per tile group (they take turns) adds the waves' sums and stores the rows.
+// A block costs 8 vector instructions and one MFMA where the int8 route needs 15 and two.
+// ---------------------------------------------------------------------------
+typedef int v8i __attribute__((ext_vector_type(8)));
+#define OXB_F4_P 30          // |x| < 2^E  ->  |X| < 2^30
+#define OXB_F4_CELL 68       // dwords per (block, 32-weight group) cell of the staging area: 16 digits x 4 dwords + 4 of padding
+#define OXB_F4_STAGE (16 * OXB_F4_CELL)
+
+// Dynamic LDS of a launch: [S][OXB_F4_STAGE] staging dwords | part [4][TG][S][16] floats | red [16] | flags [4]
+__host__ __device__ inline size_t oxb_gemv_f4_lds_bytes(uint32_t S, uint32_t tg) {
+    return ((size_t)S * OXB_F4_STAGE + (size_t)4 * tg * S * 16 + 16 + 4) * 4;
+}
+
+// Sum over the four 16-lane rows of a wave, in every lane: (r0 + r1) + (r2 + r3).  v_permlane16_swap exchanges the odd
+// rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the
+// lower half of the second; on two copies of one value each leaves the two addends of a pair side by side.
+__device__ __forceinline__ float sum_rows4(float v) {
+    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
+__device__ __forceinline__ uint32_t bfi_u32(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
+
+__device__ __forceinline__ v4f mfma_f4(const v4i a, const v4i b, const v4f c) {
+    const v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0}, b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+    // formats 4 = fp4 for both operands; block scales 2^0 (E8M0 127)
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
+}
+
+template <int NSBW, int TG, int PRO>
+__global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
+    constexpr int FMT = OXB_FMT_Q1;
+    extern __shared__ uint32_t smem[];
+    const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
+    const uint32_t c = lane & 15u, g = lane >> 4;  // D: weight row c of the tile, digits 4 g .. 4 g + 3
+    const bool swiglu = p.epi == OXB_GEMV_SWIGLU;
+    uint32_t* stage = smem + (size_t)s * OXB_F4_STAGE;
+    float* part = (float*)(smem + (size_t)S * OXB_F4_STAGE);
+    float* red = part + (size_t)4 * TG * S * 16;
+    int* flags = (int*)(red + 16);
+
+    const uint32_t lane_c = lane * 16u, lane_s = c * 8u;
+    const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
+    const int sb_lim = (int)(p.sb_begin + p.sb_count) - (int)sb0;
+    const __amdgpu_buffer_rsrc_t r_codes = make_rsrc(p.codes, p.codes_bytes);
+    const __amdgpu_buffer_rsrc_t r_scales = make_rsrc(p.scales, p.scales_bytes);
+
+    const uint32_t half_tiles = p.n_tiles >> 1;
+    const uint32_t n_units = swiglu ? half_tiles : p.n_tiles;
+    const uint32_t upw = swiglu ? (p.tpw >> 1) : p.tpw, u_begin = blockIdx.x * upw;
+    const uint32_t groups = p.tpw / TG;
+    auto unit_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return u_begin + (swiglu ? (grp >> 1) : grp) * TG + t; };
+    auto tile_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return unit_of(grp, t) + ((swiglu && (grp & 1u)) ? half_tiles : 0u); };
+    auto slot_ok = [&](uint32_t grp, uint32_t t) -> bool { return grp < groups && unit_of(grp, t) < n_units && unit_of(grp, t) < u_begin + upw; };
+
+    // ---- prologue ----
+    // lane -> (block q of the superblock, 32-weight group gq, bit position m); its eight activations per superblock
+    // are the weights 4 i + m of that group, i = 0 .. 7: nibble i of operand register m.
+    const uint32_t pq = lane >> 4, pg = (lane >> 2) & 3u, pm = lane & 3u;
+    const uint32_t koff = (128u * pq + 32u * pg + pm) * 4u;
+    const __amdgpu_buffer_rsrc_t r_x = make_rsrc(p.x, p.k * 4u);
+    const __amdgpu_buffer_rsrc_t r_w = make_rsrc(p.norm_w, PRO == OXB_GEMV_PRO_RMSNORM ? p.k * 4u : 0u);
+    float xe[NSBW][8], we[NSBW][8];
+#pragma unroll
+    for (int i = 0; i < NSBW; i++) {
+        const uint32_t off = i < sb_lim ? (sb0 + i) * 2048u + koff : OXB_OOB;  // beyond k the buffer returns 0
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            xe[i][e] = __uint_as_float(buf_load_b32(r_x, off + 16u * e));
+            if (PRO == OXB_GEMV_PRO_RMSNORM) we[i][e] = __uint_as_float(buf_load_b32(r_w, off + 16u * e));
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    TileRegs<FMT, NSBW> ring[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++) {
+        load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    if (threadIdx.x == 0) flags[0] = 0;
+
+    uint32_t bad = 0;
+    if (PRO == OXB_GEMV_PRO_RMSNORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < NSBW; i++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                ss = fmaf(xe[i][e], xe[i][e], ss);
+                xe[i][e] *= we[i][e];
+            }
+        const uint32_t c0 = p.sb_begin * 512u, c1 = (p.sb_begin + S * NSBW) * 512u;
+        if (c0 > 0 || c1 < p.k) {  // what the waves of this launch do not cover between them
+            for (uint32_t i = threadIdx.x; i < p.k; i += blockDim.x)
+                if (i < c0 || i >= c1) ss = fmaf(p.x[i], p.x[i], ss);
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        if (lane == 0) red[s] = ss;
+        __syncthreads();
+        float rp[8], tot = 0.f;  // S <= 8 sums, requested together and added in wave order
+#pragma unroll
+        for (uint32_t w = 0; w < 8; w++) rp[w] = red[w < S ? w : 0u];
+#pragma unroll
+        for (uint32_t w = 0; w < 8; w++) tot += w < S ? rp[w] : 0.f;
+        const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+        bad |= !(fabsf(inv_rms) <= 3.402823466e38f);
+#pragma unroll
+        for (int i = 0; i < NSBW; i++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) xe[i][e] *= inv_rms;
+    } else {
+        __syncthreads();  // flag cleared
+    }
+    uint32_t mxb = 0;
+#pragma unroll
+    for (int i = 0; i < NSBW; i++)
+#pragma unroll
+        for (int e = 0; e < 8; e++) mxb = max(mxb, __float_as_uint(xe[i][e]) & 0x7FFFFFFFu);
+    mxb = half_umax(mxb);
+    mxb = max((uint32_t)__builtin_amdgcn_readlane((int)mxb, 0), (uint32_t)__builtin_amdgcn_readlane((int)mxb, 32));
+    bad |= mxb >= 0x7F800000u;
+    if (__builtin_amdgcn_ballot_w64(bad != 0) != 0 && lane == 0) atomicOr(&flags[0], 1);
+    const uint32_t be = mxb >> 23;
+    const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x|
+    const int sh = OXB_F4_P - E + (pm == 0 ? 2 : (pm == 1 ? 1 : 0));
+    const uint32_t flip = pm == 3 ? 0x80000000u : 0u;  // the m = 3 operand reads -1 for a set bit
+
+    v4i A[NSBW][4];   // [superblock][block]: digit c of the block's activations, group g
+    v4f C4[NSBW][4];  // accumulator start values of digits 4 g .. 4 g + 3
+#pragma unroll
+    for (int i = 0; i < NSBW; i++) {
+        uint32_t r[8], sg = 0;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            r[e] = (uint32_t)rintf(ldexpf(fabsf(xe[i][e]), sh));
+            sg = (((__float_as_uint(xe[i][e]) ^ flip) >> 31) << (4 * e + 3)) | sg;
+        }
+        // 8 x 8 nibble transpose: tr[n] nibble e = r[e] nibble n = digits 2 n and 2 n + 1 of activation e
+        uint32_t lo[4], hi[4], tl[4], th[4];
+#pragma unroll
+        for (int a = 0; a < 4; a++) {
+            lo[a] = bfi_u32(0x0F0F0F0Fu, r[2 * a], r[2 * a + 1] << 4);
+            hi[a] = bfi_u32(0x0F0F0F0Fu, r[2 * a] >> 4, r[2 * a + 1]);
+        }
+        transpose_bytes4(lo, tl);
+        transpose_bytes4(hi, th);
+        uint32_t* cell = stage + (pq * 4 + pg) * OXB_F4_CELL + pm;
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            cell[(4 * b + 0) * 4] = (tl[b] & 0x33333333u) | sg;          // digit 4 b
+            cell[(4 * b + 1) * 4] = ((tl[b] >> 2) & 0x33333333u) | sg;   // digit 4 b + 1
+            cell[(4 * b + 2) * 4] = (th[b] & 0x33333333u) | sg;          // digit 4 b + 2
+            cell[(4 * b + 3) * 4] = ((th[b] >> 2) & 0x33333333u) | sg;   // digit 4 b + 3
+        }
+        // the staging area is this wave's own: LDS operations of a wave execute in order
+        __builtin_amdgcn_wave_barrier();
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int q = 0; q < 4; q++) A[i][q] = *reinterpret_cast<const v4i*>(&stage[(q * 4 + g) * OXB_F4_CELL + c * 4]);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            // minus the sum over the block of 2^(s - 1) a for m < 3: operands -0.5, -1, -2 and one halving
+            const v4f h = mfma_f4(A[i][q], (v4i){(int)0x99999999u, (int)0xAAAAAAAAu, (int)0xCCCCCCCCu, 0}, (v4f){0.f, 0.f, 0.f, 0.f});
+            C4[i][q] = (v4f){0.5f * h[0], 0.5f * h[1], 0.5f * h[2], 0.5f * h[3]};
+        }
+    }
+    // digit j of X is worth 2 * 4^j; the tile sums leave the wave as 2^-32 of that, and 2^(E - 30 + 32) follows
+    float MQ[4];
+#pragma unroll
+    for (int jj = 0; jj < 4; jj++) MQ[jj] = ldexpf(1.0f, 2 * (int)(4 * g + jj) - 31);
+    const int EX = mxb ? E - OXB_F4_P + 32 : 0;
+
+    // ---- main loop ----
+    for (uint32_t grp = 0; grp < groups; grp++) {
+        float* buf = part + (size_t)(grp & 3u) * TG * S * 16;
+#pragma unroll
+        for (int t = 0; t < TG; t++) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            const TileRegs<FMT, NSBW>& r = ring[t];
+#pragma unroll
+            for (int i = 0; i < NSBW; i++) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const uint32_t w = (uint32_t)r.w[i][0][q];
+                    const v4i b = {(int)(w & 0x11111111u), (int)(w & 0x22222222u), (int)(w & 0x44444444u),
+                                   (int)((w & 0x88888888u) | 0x22222222u)};
+                    const v4f d = mfma_f4(A[i][q], b, C4[i][q]);
+                    const uint32_t scw = (q < 2) ? r.sc[i].x : r.sc[i].y;
+                    const float sc = f16_bits_to_f32((q & 1) ? scw >> 16 : scw & 0xFFFFu);
+#pragma unroll
+                    for (int jj = 0; jj < 4; jj++) acc[jj] = fmaf(d[jj], sc, acc[jj]);
+                }
+            }
+            load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(grp + 1, t), slot_ok(grp + 1, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
+            __builtin_amdgcn_sched_barrier(0);
+            float v = acc[0] * MQ[0];
+            v = fmaf(acc[1], MQ[1], v);
+            v = fmaf(acc[2], MQ[2], v);
+            v = fmaf(acc[3], MQ[3], v);
+            v = ldexpf(sum_rows4(v), EX);
+            if (lane < 16) buf[((size_t)t * S + s) * 16 + lane] = v;
+        }
+        lds_barrier();
+        if (swiglu && !(grp & 1u)) continue;  // the gate sums wait for the up sums of the same rows
+        // One wave (they take turns) finishes the group: lane -> (tile t of the group, row c), the S sums of the
+        // waves requested together and added in wave order, then the epilogue.  No second barrier: the next groups
+        // write other quarters of `part`, and a quarter is reused only after two more barriers.
+        if (s != (swiglu ? grp >> 1 : grp) % S) continue;
+        const float* gbuf = part + (size_t)((grp - 1) & 3u) * TG * S * 16;
+        const uint32_t t = lane >> 4;
+        if (t >= (uint32_t)TG || !slot_ok(grp, t)) continue;
+        float pv[8], pg[8];
+#pragma unroll
+        for (uint32_t w = 0; w < 8; w++) {
+            const uint32_t wc = w < S ? w : S - 1;
+            pv[w] = buf[((size_t)t * S + wc) * 16 + c];
+            if (swiglu) pg[w] = gbuf[((size_t)t * S + wc) * 16 + c];
+        }
+        const int bad_in = flags[0];
+        float v0 = 0.f, v1 = 0.f;
+#pragma unroll
+        for (uint32_t w = 0; w < 8; w++) {
+            v0 += w < S ? pv[w] : 0.f;  // a wave that does not exist adds +0
+            if (swiglu) v1 += w < S ? pg[w] : 0.f;
+        }
+        if (bad_in) v0 = __int_as_float(0x7FC00000);
+        const uint32_t row = unit_of(grp, t) * 16 + c;
+        if (row >= (swiglu ? (p.n_rows >> 1) : p.n_rows)) continue;
+        if (swiglu) v0 = (v1 / (1.0f + expf(-v1))) * v0;  // v1 = gate, v0 = up
+        else if (p.epi == OXB_GEMV_ACCUM) v0 += p.y[row];
+        else if (p.epi == OXB_GEMV_RESIDUAL) v0 += p.residual[row];
+        p.y[row] = v0;
+    }
+}
+
 // The same grid, waves, ring and addresses as gemv_kernel, and no arithmetic beyond an OR.
 template <int FMT, int NSBW, int TG>
 __global__ __launch_bounds__(512) void stream_floor_kernel(const OxbGemvParams p) {
@@ -520,6 +777,16 @@ static hipError_t launch_gemv_t(const OxbGemvParams& p, const GemvPlan& pl, hipS
     return hipGetLastError();
 }
 
+template <int NSBW, int TG>
+static hipError_t launch_gemv_f4_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    const size_t shm = oxb_gemv_f4_lds_bytes(pl.S, TG);
+    if (p.pro == OXB_GEMV_PRO_RMSNORM)
+        hipLaunchKernelGGL((gemv_f4_kernel<NSBW, TG, OXB_GEMV_PRO_RMSNORM>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+    else
+        hipLaunchKernelGGL((gemv_f4_kernel<NSBW, TG, OXB_GEMV_PRO_F32>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+    return hipGetLastError();
+}
+
 template <int FMT, int NSBW, int TG>
 static hipError_t launch_floor_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
     hipLaunchKernelGGL((stream_floor_kernel<FMT, NSBW, TG>), dim3(pl.grid), dim3(pl.S * 64), 0, st, p);
@@ -547,8 +814,18 @@ static bool check_gemv_args(const OxbGemvParams& p) {
 hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {
     if (p.n_tiles == 0) return hipSuccess;
     GemvPlan pl;
+    // The fp4 kernel's registers let two workgroups share a CU; that pays where a workgroup has many tiles to
+    // spread its prologue over (the LM head: 18 -> 16.8 us), and costs where it has few (the second prologue).
+    const bool f4 = fmt == OXB_FMT_Q1 && p.nvec == 1;
+    if (f4 && p.epi != OXB_GEMV_SWIGLU && p.n_tiles >= 32u * n_cus) n_cus *= 2;
     if (!check_gemv_args(p) || !plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
+    if (f4) {  // one vector of Q1 weights: the fp4 route
+#define OXB_F4_CASE(N, T) \
+    if (pl.nsbw == N && pl.tg == T) return launch_gemv_f4_t<N, T>(p, pl, st);
+        OXB_F4_CASE(1, 1) OXB_F4_CASE(1, 2) OXB_F4_CASE(1, 3) OXB_F4_CASE(1, 4) OXB_F4_CASE(2, 1) OXB_F4_CASE(2, 2) OXB_F4_CASE(3, 1)
+#undef OXB_F4_CASE
+    }
     OXB_GEMV_CASES(launch_gemv_t)
     return hipErrorInvalidValue;
 }
@@ -557,6 +834,7 @@ hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus
     if (p.n_tiles == 0) return hipSuccess;
     GemvPlan pl;
     p.epi = OXB_GEMV_STORE;
+    if (fmt == OXB_FMT_Q1 && p.n_tiles >= 32u * n_cus) n_cus *= 2;  // as the single-vector route plans it
     if (!plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
     OXB_GEMV_CASES(launch_floor_t)

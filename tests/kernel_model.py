@@ -78,7 +78,86 @@ def _weight_bytes(fmt: int, codes, tile: int, sb: int, q: int) -> np.ndarray:
     return out
 
 
-def gemv(fmt: int, codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
+F4_P = 30                    # fp4 route: x = 2^(E - 30) X with |X| < 2^30
+_F4_OPERAND = np.array([0.5, 1.0, 2.0])     # what a set bit reads at position m = 0, 1, 2 of its nibble
+
+
+def quantise_block_f4(xb: np.ndarray, E: int):
+    """fp4 route, one 128-activation block at the slice exponent E -> (digit values [128][16] as the E2M1 numbers
+    the A operand holds, sign included; start values [16] of the sixteen digit rows)."""
+    k = np.arange(128)
+    m = k & 3                                       # k = 32 g + 4 i + m: bit m of nibble i of the lane's code dword
+    sh = (F4_P - E + np.array([2, 1, 0, 0])[m]).astype(np.int32)
+    mag = np.rint(np.ldexp(np.abs(xb.astype(np.float32)), sh).astype(np.float32)).astype(np.float64)
+    mag = np.nan_to_num(mag, nan=0.0).astype(np.uint64)
+    neg = np.signbit(xb) ^ (m == 3)                 # the m = 3 operand reads -1 for a set bit
+    dig = np.stack([((mag >> np.uint64(2 * j)) & np.uint64(3)).astype(np.float64) * 0.5 for j in range(16)], axis=-1)
+    dig = np.where(neg[:, None], -dig, dig)
+    bc = np.where(m < 3, -np.array([0.5, 1.0, 2.0, 0.0])[m], 0.0)
+    start = 0.5 * (bc[:, None] * dig).sum(axis=0)
+    return dig, start
+
+
+def _weight_operands_f4(codes, tile: int, sb: int, q: int) -> np.ndarray:
+    """E2M1 operand values [16 rows][128 k] of block q of unit (tile, sb), as the AND masks produce them."""
+    out = np.zeros((16, 128), dtype=np.float64)
+    for g in range(4):
+        lanes = g * 16 + np.arange(16)
+        w = codes[tile, sb, lanes * 4 + q].astype(np.int64)
+        for i in range(32):
+            b = (w >> i) & 1
+            out[:, 32 * g + i] = np.where(b == 1, -1.0, 1.0) if (i & 3) == 3 else b * _F4_OPERAND[i & 3]
+    return out
+
+
+def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
+    """gemv_f4_kernel step by step (Q1 weights, one activation vector)."""
+    n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512
+    x = np.asarray(x, dtype=np.float32)
+    xp = np.zeros(n_sb * 512, dtype=np.float32)
+    xp[:k] = x
+    codes = codes_u8.view(np.uint32).reshape(n_tiles, n_sb, 256)
+    scales = scales_u8.view(np.float16).reshape(n_tiles, n_sb, 16, 4).astype(np.float32)  # [row][q]
+    mq = np.ldexp(np.float32(1.0), 2 * np.arange(16) - 31).astype(np.float32)
+    y = np.zeros(n_rows, dtype=np.float32)
+    for tile in range(n_tiles):
+        total = None
+        for sb_begin in range(0, n_sb, MAX_SB):                 # launches
+            sb_count = min(MAX_SB, n_sb - sb_begin)
+            nsbw = (sb_count + 7) // 8
+            S = (sb_count + nsbw - 1) // nsbw
+            launch = np.zeros(16, dtype=np.float32)             # waves added in order
+            for s in range(S):
+                acc = np.zeros((16, 16), dtype=np.float32)      # [row][digit]
+                sb_lo, sb_hi = sb_begin + s * nsbw, min(sb_begin + (s + 1) * nsbw, sb_begin + sb_count)
+                E, zero = slice_exponent(xp[sb_lo * 512:sb_hi * 512])
+                if E is None:
+                    return np.full(n_rows, np.nan, dtype=np.float32)
+                for sb in range(sb_lo, sb_hi):
+                    for q in range(4):
+                        dig, start = quantise_block_f4(xp[(sb * 4 + q) * 128:(sb * 4 + q + 1) * 128], E)
+                        r = _f32(start[None, :] + _weight_operands_f4(codes, tile, sb, q) @ dig)   # exact
+                        acc = _fma32(r, np.repeat(scales[tile, sb, :, q][:, None], 16, axis=1), acc)
+                vg = []
+                for g in range(4):                              # the four digits of a lane group, joined by FMAs
+                    v = (acc[:, 4 * g] * mq[4 * g]).astype(np.float32)
+                    for jj in range(1, 4):
+                        v = _fma32(acc[:, 4 * g + jj], np.full(16, mq[4 * g + jj], np.float32), v)
+                    vg.append(v)
+                v = ((vg[0] + vg[1]).astype(np.float32) + (vg[2] + vg[3]).astype(np.float32)).astype(np.float32)
+                launch = (launch + np.ldexp(v, 0 if zero else E - F4_P + 32).astype(np.float32)).astype(np.float32)
+            total = launch if total is None else (total + launch).astype(np.float32)
+        rows = tile * 16 + np.arange(16)
+        ok = rows < n_rows
+        y[rows[ok]] = total[ok]
+    return y
+
+
+def gemv(fmt: int, codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray, route: str | None = None) -> np.ndarray:
+    """The route a single activation vector takes on the device: fp4 for Q1 weights, int8 for TQ2 (`route="i8"`
+    forces the int8 route, which Q1 weights take from two vectors on)."""
+    if fmt == 0 and route != "i8":
+        return gemv_f4(codes_u8, scales_u8, n_rows, k, x)
     n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512
     x = np.asarray(x, dtype=np.float32)
     xp = np.zeros(n_sb * 512, dtype=np.float32)

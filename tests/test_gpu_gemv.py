@@ -167,7 +167,12 @@ def test_gemv_properties(backend, fmt):
         xo[100] = 5000.0                                                            # one massive outlier
         want = dense_f64(fmt, a, n, k) @ xo.astype(np.float64)
         assert np.max(np.abs(_gemv(backend, fmt, h, xo, n, k) - want)) < 1e-6 * np.max(np.abs(want))
-        assert np.array_equal(backend.gemv_cached_batch(h, np.stack([x1, x2]), n, k)[1], y2)  # gemm row = gemv
+        yb = backend.gemv_cached_batch(h, np.stack([x1, x2]), n, k)[1]
+        if fmt == TQ2:
+            assert np.array_equal(yb, y2)                                                # a batch row = the single vector
+        else:
+            # Q1: one vector takes the fp4 route, two and more the int8 route; both are exact up to their fp32 joins
+            assert np.max(np.abs(yb - y2)) < 2e-6 * np.max(np.abs(y2))
     finally:
         backend.free_weights(h)
     zero = a.copy().reshape(-1, 18 if fmt == Q1 else 34)
