@@ -172,6 +172,9 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
             }
     };
     load_x(0);
+    // every wave's activation requests enter the CU's memory pipeline before any wave's weight requests
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     TileRegs<FMT, NSBW> ring[TG];
 #pragma unroll
@@ -457,6 +460,11 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
             if (PRO == OXB_GEMV_PRO_RMSNORM) we[i][e] = __uint_as_float(buf_load_b32(r_w, off + 16u * e));
         }
     }
+    // Every wave's activation requests enter the CU's memory pipeline before any wave's weight requests: without
+    // the barrier the activations of the waves that start last wait behind the weight tiles of the first ones, and
+    // their whole prologue with them (gate||up 24576 x 4096: 6.5 -> 5.7 us).
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     TileRegs<FMT, NSBW> ring[TG];
 #pragma unroll
