@@ -33,7 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 # (x 1.000) of the kernel named beside it, from the profile named beside it.  The algorithmic figure is 14 270 464.
 GATE_UP_HBM_TRAFFIC_BYTES = 14_498_816
 GATE_UP_HBM_TRAFFIC_SOURCE = "profiles/gemv_q1_qwen3_8b_set_hbm_traffic.txt"
-GATE_UP_KERNEL = "gemv_kernel<0, 1, 3, 0> (Q1, one superblock of K per wave, three row tiles in flight, fp32 input) gate||up 24576x4096"
+GATE_UP_KERNEL = "gemv_f4_kernel<1, 3, 0> (Q1 weights, one activation vector, one superblock of K per wave, three row tiles in flight, fp32 input) gate||up 24576x4096"
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
 FMT_TQ2 = 1
@@ -611,7 +611,7 @@ def main() -> int:
         "metric": "quant GEMV HBM GB/s", "value": round(value, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 MFMA on four exact base-256 digits of 30-bit fixed-point activations (exact block sums), fp32 scales and accumulation",
+        "dtype": "fp4 (E2M1) MFMA on sixteen base-4 digits of 32-bit fixed-point activations (exact block sums), fp32 scales and accumulation; int8 MFMA on four base-256 digits for ternary weights and for two to four vectors",
         "data": "synthetic",
         "config": {"workload": "Q1_0_g128 GEMV set, Qwen3-8B shapes (6144x4096, 24576x4096, 4096x12288), batch 1",
                    "algorithmic_bytes_per_step": set_bytes, "weight_copies": args.copies,
