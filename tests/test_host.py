@@ -103,6 +103,38 @@ def test_device_arithmetic_model_matches_oracle(fmt, shape):
     assert np.max(np.abs(y - yo)) < 1e-5
 
 
+@pytest.mark.parametrize("shape", [(16, 128), (40, 640), (33, 1024)])
+def test_int8_route_model_of_q1_weights_matches_oracle(shape):
+    """Q1 weights take the int8 route from two activation vectors on; its model stays held to the oracle too."""
+    n, k = shape
+    a = synth.make_blocks(Q1, 11, n, k)
+    x = synth.normal_f32(5, k)
+    y = kernel_model.gemv(Q1, *ox.repack(Q1, a, n, k), n, k, x, route="i8")
+    want = dense_f64(Q1, a, n, k) @ x.astype(np.float64)
+    yo = oracle.gemv(Q1, a, x, n, k)
+    assert np.max(np.abs(y - want)) <= max(np.max(np.abs(yo - want)) * 2, 1e-6)
+    assert np.max(np.abs(y - yo)) < 1e-5
+    y4 = kernel_model.gemv(Q1, *ox.repack(Q1, a, n, k), n, k, x)                  # the fp4 route of one vector
+    assert np.max(np.abs(y - y4)) < 2e-6 * max(1.0, float(np.max(np.abs(y4))))
+
+
+def test_fp4_route_model_special_inputs():
+    """Zero vectors, a NaN, an outlier and exact power-of-two scaling through the model of the fp4 route."""
+    a = cross_tier_q1(32, 512)
+    rep = ox.repack(Q1, a, 32, 512)
+    x = synth.normal_f32(3, 512)
+    y = kernel_model.gemv(Q1, *rep, 32, 512, x)
+    assert np.all(kernel_model.gemv(Q1, *rep, 32, 512, np.zeros(512, np.float32)) == 0)
+    for s in (-100, 66):
+        assert np.array_equal(kernel_model.gemv(Q1, *rep, 32, 512, np.ldexp(x, s).astype(np.float32)), np.ldexp(y, s).astype(np.float32))
+    xo = x.copy()
+    xo[17] = 3000.0
+    want = dense_f64(Q1, a, 32, 512) @ xo.astype(np.float64)
+    assert np.max(np.abs(kernel_model.gemv(Q1, *rep, 32, 512, xo) - want)) < 1e-6 * np.max(np.abs(want)) + 1e-4
+    xo[3] = np.nan
+    assert np.all(np.isnan(kernel_model.gemv(Q1, *rep, 32, 512, xo)))
+
+
 def test_device_arithmetic_model_reference_kats():
     for fmt, pat, x, want in [
         (Q1, 0xFF, np.arange(128, dtype=np.float32), 8128.0),
