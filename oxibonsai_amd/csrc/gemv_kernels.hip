@@ -217,8 +217,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
                 for (uint32_t i = threadIdx.x; i < p.k; i += blockDim.x)
                     if (i < c0 || i >= c1) ss = fmaf(xv[i], xv[i], ss);
             }
-#pragma unroll
-            for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+            ss = wave_sum_f32(ss);
             if (lane == 0) red[s] = ss;
             __syncthreads();
             float tot = 0.f;
@@ -399,16 +398,6 @@ __host__ __device__ inline size_t oxb_gemv_f4_lds_bytes(uint32_t S, uint32_t tg)
     return ((size_t)S * OXB_F4_STAGE + (size_t)4 * tg * S * 16 + 16 + 4) * 4;
 }
 
-// Sum over the four 16-lane rows of a wave, in every lane: (r0 + r1) + (r2 + r3).  v_permlane16_swap exchanges the odd
-// rows of its first operand with the even rows of its second, v_permlane32_swap the upper half of the first with the
-// lower half of the second; on two copies of one value each leaves the two addends of a pair side by side.
-__device__ __forceinline__ float sum_rows4(float v) {
-    const auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
-    const auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
-    return __uint_as_float(b[0]) + __uint_as_float(b[1]);
-}
-
 __device__ __forceinline__ uint32_t bfi_u32(uint32_t mask, uint32_t a, uint32_t b) { return (a & mask) | (b & ~mask); }
 
 __device__ __forceinline__ v4f mfma_f4(const v4i a, const v4i b, const v4f c) {
@@ -489,8 +478,7 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
             for (uint32_t i = threadIdx.x; i < p.k; i += blockDim.x)
                 if (i < c0 || i >= c1) ss = fmaf(p.x[i], p.x[i], ss);
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        ss = wave_sum_f32(ss);
         if (lane == 0) red[s] = ss;
         __syncthreads();
         float rp[8], tot = 0.f;  // S <= 8 sums, requested together and added in wave order

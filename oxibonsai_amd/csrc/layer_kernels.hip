@@ -61,8 +61,7 @@ __global__ __launch_bounds__(256) void qk_norm_rope_store_kernel(OxbQkParams p) 
             hi[it] = d < half ? in[d + half] : 0.f;
             ss = fmaf(lo[it], lo[it], fmaf(hi[it], hi[it], ss));
         }
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        ss = wave_sum_f32(ss);
         const float inv_rms = 1.0f / sqrtf(ss / (float)hd + p.eps);
         float o_lo[KI], o_hi[KI], kmax = 0.f;
 #pragma unroll
@@ -145,8 +144,7 @@ __global__ __launch_bounds__(64) void kv_quantize_rows_kernel(const float* __res
     const float* row = x + (size_t)blockIdx.x * n;
     float mx = 0.f;
     for (uint32_t d = threadIdx.x; d < n; d += 64) mx = fmaxf(mx, fabsf(row[d]));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+    mx = wave_max_f32(mx);
     const float scale = kv_row_scale<KVM>(mx);
     for (uint32_t d = threadIdx.x; d < n; d += 64) codes[(size_t)blockIdx.x * n + d] = (uint8_t)kv_encode<KVM>(row[d], scale);
     if (threadIdx.x == 0) scales[blockIdx.x] = scale;
@@ -370,8 +368,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         for (int it = 0; it < KI; it++) ss = fmaf(r.lo[it], r.lo[it], ss);
 #pragma unroll
         for (int it = 0; it < KI; it++) ss = fmaf(r.hi[it], r.hi[it], ss);
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+        ss = wave_sum_f32(ss);
         return 1.0f / sqrtf(ss / (float)HD + p.eps);
     };
     HeadIn q_in, cs_sn, qn, kv_in, kn;  // cs_sn: lo = cos, hi = sin; kv_in: the new K row (wave 0) or V row (wave 1) of the owner
@@ -427,8 +424,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             }
             float scale = 1.f;
             if constexpr (QC) {
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                mx = wave_max_f32(mx);
                 scale = kv_row_scale<KVM>(mx);
                 if (lane == 0) Ksc[new_row] = scale;
             }
@@ -451,8 +447,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             for (int it = 0; it < KI; it++) mx = fmaxf(mx, fmaxf(fabsf(kv_in.lo[it]), fabsf(kv_in.hi[it])));
             float scale = 1.f;
             if constexpr (QC) {
-#pragma unroll
-                for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, 64));
+                mx = wave_max_f32(mx);
                 scale = kv_row_scale<KVM>(mx);
                 if (lane == 0) Vsc[new_row] = scale;
             }
@@ -578,8 +573,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             sv[4 + v] = vis[4 + v] ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = max_rows4(mx);
         const float m_new = fmaxf(m_run, mx);      // finite: the block holds a visible key
         float alpha = expf(m_run - m_new);         // 0 for the wave's first block
         float vw[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // V row scales of the lane's keys in units of u_run
@@ -588,8 +582,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             float vmx = 0.f;
 #pragma unroll
             for (int e = 0; e < 8; e++) vmx = fmaxf(vmx, vis[e] ? va[e] : 0.f);
-            vmx = fmaxf(vmx, __shfl_xor(vmx, 16, 64));
-            vmx = fmaxf(vmx, __shfl_xor(vmx, 32, 64));
+            vmx = max_rows4(vmx);
             const float u_new = fmaxf(u_run, vmx);  // > 0: a visible row's scale is at least f32::EPSILON
             const float inv_u = 1.0f / u_new;
 #pragma unroll
@@ -611,8 +604,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             ph[e] = hi;
             pl[e] = (_Float16)(pv - (float)hi);
         }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
+        sum = sum_rows4(sum);
         l_run += sum;
         m_run = m_new;
         // O^T += V^T P^T; A operand gathered from the staged block
@@ -718,12 +710,10 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
         const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
         const float mv = lane < used ? ld1(ph) : -INFINITY, lv = lane < used ? ld1(ph + 1) : 0.f;
         float M = mv;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+        M = wave_max_f32(M);
         const float w = lane < used ? expf(mv - M) : 0.f;
         float L = w * lv;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+        L = wave_sum_f32(L);
         wts[hh * 64 + lane] = w;
         if (lane == 0) inv_l[hh] = L > 0.f ? 1.0f / L : 0.f;
     }
@@ -901,8 +891,7 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const float* __restrict__ 
     }
     float ss = 0.f;
     for (uint32_t i = tid; i < n; i += 256) ss += xv[i] * xv[i];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+    ss = wave_sum_f32(ss);
     if ((tid & 63u) == 0) part[tid >> 6] = ss;
     __syncthreads();
     const float inv_rms = 1.0f / sqrtf((part[0] + part[1] + part[2] + part[3]) / (float)n + eps);

@@ -103,8 +103,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
                 ss = fmaf(f[e], f[e], ss);
             }
         }
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
+        ss = sum_rows4(ss);
         const float inv = 1.0f / sqrtf(ss / (float)HD + p.eps);
 #pragma unroll
         for (int s = 0; s < KS; s++)
@@ -237,8 +236,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
             sv[4 + v] = vb_ ? s1[v] : -INFINITY;
             mx = fmaxf(mx, fmaxf(sv[v], sv[4 + v]));
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        mx = max_rows4(mx);
         // without a window key 0 is visible to every query, so the maximum is finite from the first block on; with
         // one, a query may see nothing yet: it keeps its empty state (all probabilities 0)
         const float m_new = fmaxf(m_run, mx);
@@ -252,8 +250,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(OxbPrefillAttnParams 
             sum += pe;
             pb[e] = (_Float16)pe;
         }
-        sum += __shfl_xor(sum, 16, 64);
-        sum += __shfl_xor(sum, 32, 64);
+        sum = sum_rows4(sum);
         l_run = l_run * alpha + sum;
         m_run = m_new;
 #pragma unroll
