@@ -80,14 +80,18 @@ __device__ __forceinline__ void transpose_bytes4(const uint32_t t[4], uint32_t o
     o[3] = __builtin_amdgcn_perm(p23h, p01h, 0x07060302u);
 }
 
-// Unsigned maximum / integer sum over the 32 lanes of a half wave (lanes 0-31, 32-63), result in every lane.  Zero is
-// the identity of both, so the DPP moves (which hand 0 to a lane without a source) fold into the arithmetic.
-__device__ __forceinline__ uint32_t half_umax(uint32_t v) {
+// Unsigned maximum over the 64 lanes of a wave (in every lane) and integer sum over the 32 lanes of a half wave
+// (lanes 0-31, 32-63).  Zero is the identity of both, so the DPP moves (which hand 0 to a lane without a source) fold
+// into the arithmetic; the rows of the maximum meet through the lane-swap instructions, not through LDS.
+__device__ __forceinline__ uint32_t wave_umax(uint32_t v) {
     v = max(v, dpp_u32<0xB1>(v));    // quad_perm [1,0,3,2]
     v = max(v, dpp_u32<0x4E>(v));    // quad_perm [2,3,0,1]
     v = max(v, dpp_u32<0x141>(v));   // row_half_mirror
     v = max(v, dpp_u32<0x140>(v));   // row_mirror
-    return max(v, (uint32_t)__builtin_amdgcn_ds_swizzle((int)v, 0x401F));  // lane ^ 16
+    const auto a = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+    v = max(a[0], a[1]);
+    const auto b = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+    return max(b[0], b[1]);
 }
 __device__ __forceinline__ int half_isum(int v) {
     v += dpp_i32<0xB1>(v);
@@ -239,8 +243,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
                     if (PRO == OXB_GEMV_PRO_RMSNORM) xe[i][pass][bb] *= inv_rms;
                     mxb = max(mxb, __float_as_uint(xe[i][pass][bb]) & 0x7FFFFFFFu);
                 }
-        mxb = half_umax(mxb);
-        mxb = max((uint32_t)__builtin_amdgcn_readlane((int)mxb, 0), (uint32_t)__builtin_amdgcn_readlane((int)mxb, 32));
+        mxb = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_umax(mxb));
         bad |= mxb >= 0x7F800000u;
         const uint32_t be = mxb >> 23;
         const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x| (subnormal maxima share the smallest E)
@@ -500,8 +503,7 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     for (int i = 0; i < NSBW; i++)
 #pragma unroll
         for (int e = 0; e < 8; e++) mxb = max(mxb, __float_as_uint(xe[i][e]) & 0x7FFFFFFFu);
-    mxb = half_umax(mxb);
-    mxb = max((uint32_t)__builtin_amdgcn_readlane((int)mxb, 0), (uint32_t)__builtin_amdgcn_readlane((int)mxb, 32));
+    mxb = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_umax(mxb));
     bad |= mxb >= 0x7F800000u;
     if (__builtin_amdgcn_ballot_w64(bad != 0) != 0 && lane == 0) atomicOr(&flags[0], 1);
     const uint32_t be = mxb >> 23;
