@@ -455,8 +455,9 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     // Every wave's activation requests enter the CU's memory pipeline before any wave's weight requests: without
     // the barrier the activations of the waves that start last wait behind the weight tiles of the first ones, and
     // their whole prologue with them (gate||up 24576 x 4096: 6.5 -> 5.7 us).
+    if (threadIdx.x == 0) flags[0] = 0;  // cleared for every wave once the barrier is passed
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
+    lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
     TileRegs<FMT, NSBW> ring[TG];
 #pragma unroll
@@ -464,8 +465,10 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
         load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (threadIdx.x == 0) flags[0] = 0;
 
+    // RMSNorm: the weights are multiplied in here; the scalar 1 / rms is positive and the same for the whole vector, so
+    // it does not change which power of two the slices get and is applied to the row sums at the end (the waves
+    // leave their sums of squares in LDS and go on: no barrier, no wait for the other slices in the prologue).
     uint32_t bad = 0;
     if (PRO == OXB_GEMV_PRO_RMSNORM) {
         float ss = 0.f;
@@ -483,20 +486,6 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
         }
         ss = wave_sum_f32(ss);
         if (lane == 0) red[s] = ss;
-        __syncthreads();
-        float rp[8], tot = 0.f;  // S <= 8 sums, requested together and added in wave order
-#pragma unroll
-        for (uint32_t w = 0; w < 8; w++) rp[w] = red[w < S ? w : 0u];
-#pragma unroll
-        for (uint32_t w = 0; w < 8; w++) tot += w < S ? rp[w] : 0.f;
-        const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
-        bad |= !(fabsf(inv_rms) <= 3.402823466e38f);
-#pragma unroll
-        for (int i = 0; i < NSBW; i++)
-#pragma unroll
-            for (int e = 0; e < 8; e++) xe[i][e] *= inv_rms;
-    } else {
-        __syncthreads();  // flag cleared
     }
     uint32_t mxb = 0;
 #pragma unroll
@@ -604,12 +593,26 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
             pv[w] = buf[((size_t)t * S + wc) * 16 + c];
             if (swiglu) pg[w] = gbuf[((size_t)t * S + wc) * 16 + c];
         }
-        const int bad_in = flags[0];
+        float rp[8];
+        if (PRO == OXB_GEMV_PRO_RMSNORM) {
+#pragma unroll
+            for (uint32_t w = 0; w < 8; w++) rp[w] = red[w < S ? w : 0u];
+        }
+        int bad_in = flags[0];
         float v0 = 0.f, v1 = 0.f;
 #pragma unroll
         for (uint32_t w = 0; w < 8; w++) {
             v0 += w < S ? pv[w] : 0.f;  // a wave that does not exist adds +0
             if (swiglu) v1 += w < S ? pg[w] : 0.f;
+        }
+        if (PRO == OXB_GEMV_PRO_RMSNORM) {  // the waves' sums of squares in wave order, then 1 / rms on the row sums
+            float tot = 0.f;
+#pragma unroll
+            for (uint32_t w = 0; w < 8; w++) tot += w < S ? rp[w] : 0.f;
+            const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+            bad_in |= !(fabsf(inv_rms) <= 3.402823466e38f);
+            v0 *= inv_rms;
+            v1 *= inv_rms;
         }
         if (bad_in) v0 = __int_as_float(0x7FC00000);
         const uint32_t row = unit_of(grp, t) * 16 + c;
