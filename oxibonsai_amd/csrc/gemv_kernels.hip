@@ -113,9 +113,9 @@ struct Fix {
 
 #define OXB_GEMV_META 4  // ints of per-block metadata a wave leaves in LDS: the four accumulator start values
 
-// Dynamic LDS of a launch: [S][NSBW * 512] staging dwords | [S][NSBW * 4][META] | part [4][TG][S][64] floats | red [16] | flags [4]
+// Dynamic LDS of a launch: [S][NSBW * 512] staging dwords | [S][NSBW * 4][META] | part [4][TG][S][64] floats | red [4][8] | flags [4]
 __host__ __device__ inline size_t oxb_gemv_lds_bytes(uint32_t S, uint32_t nsbw, uint32_t tg) {
-    return ((size_t)S * nsbw * 512 + (size_t)S * nsbw * 4 * OXB_GEMV_META + (size_t)4 * tg * S * 64 + 16 + 4) * 4;
+    return ((size_t)S * nsbw * 512 + (size_t)S * nsbw * 4 * OXB_GEMV_META + (size_t)4 * tg * S * 64 + 32 + 4) * 4;
 }
 
 // Workgroup wg handles tile slots [wg * tpw, +tpw) in groups of TG (TG tiles are in flight per wave).  For the SwiGLU
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
     int* meta = (int*)(smem + (size_t)S * NSBW * 512) + (size_t)s * NSBW * 4 * OXB_GEMV_META;
     float* part = (float*)(smem + (size_t)S * NSBW * 512 + (size_t)S * NSBW * 4 * OXB_GEMV_META);
     float* red = part + (size_t)4 * TG * S * 64;
-    int* flags = (int*)(red + 16);
+    int* flags = (int*)(red + 32);
 
     const uint32_t lane_c = lane * 16u, lane_s = c * 8u;
     const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
@@ -176,9 +176,10 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
             }
     };
     load_x(0);
+    if (threadIdx.x < 4) flags[threadIdx.x] = 0;  // cleared for every wave once the barrier is passed
     // every wave's activation requests enter the CU's memory pipeline before any wave's weight requests
     __builtin_amdgcn_sched_barrier(0);
-    __builtin_amdgcn_s_barrier();
+    lds_barrier();
     __builtin_amdgcn_sched_barrier(0);
     TileRegs<FMT, NSBW> ring[TG];
 #pragma unroll
@@ -186,7 +187,6 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
         load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
         __builtin_amdgcn_sched_barrier(0);
     }
-    if (threadIdx.x < 4) flags[threadIdx.x] = 0;
 
     v4i A[NSBW][4][2];  // [superblock][block][MFMA]: digit d of vector v in lanes with c = 4 v + d
     v4i C4[NSBW][4];    // accumulator start values (they cancel the bias of the unsigned code encodings), lanes with g = v
@@ -201,10 +201,11 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
         }
     auto quantise_vector = [&](const uint32_t v) {
         uint32_t bad = 0;
-        float inv_rms = 1.f;
         if (PRO == OXB_GEMV_PRO_RMSNORM) {
             // Sum of squares over the whole vector: every wave adds its own slice (in registers already); what the
-            // waves of this launch do not cover between them is added by a strided loop.
+            // waves of this launch do not cover between them is added by a strided loop.  The sums meet in LDS and
+            // 1 / rms - a positive scalar, which does not change the slices' powers of two - is applied to the row
+            // sums at the end, so the prologue neither waits for the other waves nor for a square root.
             float ss = 0.f;
 #pragma unroll
             for (int i = 0; i < NSBW; i++)
@@ -222,15 +223,7 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
                     if (i < c0 || i >= c1) ss = fmaf(xv[i], xv[i], ss);
             }
             ss = wave_sum_f32(ss);
-            if (lane == 0) red[s] = ss;
-            __syncthreads();
-            float tot = 0.f;
-            for (uint32_t w = 0; w < S; w++) tot += red[w];
-            inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
-            bad |= !(fabsf(inv_rms) <= 3.402823466e38f);
-            __syncthreads();
-        } else if (v == 0) {
-            __syncthreads();  // flags cleared
+            if (lane == 0) red[v * 8 + s] = ss;
         }
         // exponent of the slice: |x| as integers are ordered like the floats, NaN and infinity on top
         uint32_t mxb = 0;
@@ -240,7 +233,6 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
             for (int pass = 0; pass < 2; pass++)
 #pragma unroll
                 for (int bb = 0; bb < 4; bb++) {
-                    if (PRO == OXB_GEMV_PRO_RMSNORM) xe[i][pass][bb] *= inv_rms;
                     mxb = max(mxb, __float_as_uint(xe[i][pass][bb]) & 0x7FFFFFFFu);
                 }
         mxb = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_umax(mxb));
@@ -359,6 +351,14 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
             for (uint32_t w = 0; w < S; w++) v0 += buf[((size_t)t * S + w) * 64 + ln];
             if (swiglu)
                 for (uint32_t w = 0; w < S; w++) v1 += gbuf[((size_t)t * S + w) * 64 + ln];
+            if (PRO == OXB_GEMV_PRO_RMSNORM) {
+                float tot = 0.f;
+                for (uint32_t w = 0; w < S; w++) tot += red[vv * 8 + w];
+                const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+                if (!(fabsf(inv_rms) <= 3.402823466e38f)) v0 = __int_as_float(0x7FC00000);
+                v0 *= inv_rms;
+                v1 *= inv_rms;
+            }
             if (flags[vv]) v0 = __int_as_float(0x7FC00000);
             const uint32_t row = unit_of(grp, t) * 16 + cc;
             if (row >= (swiglu ? (p.n_rows >> 1) : p.n_rows)) continue;
