@@ -220,13 +220,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     constexpr int KS = HD / 32, NS = HD / 16, VSTR = HD + 8;
     constexpr int VPR = QC ? HD / 16 : HD / 8;  // 16-byte pieces per V row
     constexpr int VL = 32 * VPR / 64;           // pieces of the wave's 32-row V block per lane
-    // V block per wave; before the loop its start holds Q * scale of the group's heads, after it the merge buffers
+    // V block per wave; after the loop the merge buffers.  Q * scale of the group's heads has an area of its own, so
+    // that a wave whose Q operands are in registers starts staging V without waiting for the others.
     __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];
+    __shared__ __attribute__((aligned(16))) float qs[16 * HD];
     __shared__ uint32_t last_flag;
     __shared__ __attribute__((aligned(16))) _Float16 kv_new[2][HD];  // the new position's K and V rows as stored (fp16 cache)
-    static_assert(sizeof(vs_all) >= 16 * HD * sizeof(float), "Q must fit in the V slices");
     static_assert(sizeof(vs_all) >= OXB_ATTN_MERGE_LDS_BYTES(16), "the merge's slot weights and partial sums must fit in the V slices");
-    float* qs = reinterpret_cast<float*>(&vs_all[0][0]);
     const uint32_t tid = threadIdx.x, lane = tid & 63u, qi = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t slot = blockIdx.x, kvh = blockIdx.y, b = blockIdx.z;
@@ -485,7 +485,6 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             qh[s][e] = hi;
             ql[s][e] = (_Float16)(x - (float)hi);
         }
-    lds_barrier();  // Q is in registers everywhere: its LDS copy may be overwritten
     v4f O[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
