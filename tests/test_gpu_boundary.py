@@ -234,10 +234,12 @@ def test_lm_head_joins_a_live_model(backend, fmt):
 
 
 @pytest.mark.parametrize("fmt", [Q1, TQ2])
-def test_batch_attn_phase(backend, fmt):
-    """RMSNorm + fused QKV product in one launch, against the oracle's RMSNorm and GEMV."""
+@pytest.mark.parametrize("h", [1024, 640, 13312, 16384])
+def test_batch_attn_phase(backend, fmt, h):
+    """RMSNorm + fused QKV product in one launch, against the oracle's RMSNorm and GEMV.  Rows longer than 12288 take
+    a second, accumulating launch: each applies 1 / rms of the whole row to its own part of the sum."""
     from oxibonsai_amd.model import batch_attn_phase
-    h, qr, kr = 1024, 512, 256
+    qr, kr = 512, 256
     a = synth.make_blocks(fmt, 0xA77 + fmt, qr + 2 * kr, h)
     x = synth.normal_f32(0xA78, h)
     nw = (1.0 + synth.normal_f32(0xA79, h, 0.02)).astype(np.float32)
