@@ -408,6 +408,11 @@ __device__ __forceinline__ v4f mfma_f4(const v4i a, const v4i b, const v4f c) {
     // formats 4 = fp4 for both operands; block scales 2^0 (E8M0 127)
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7F7F7F7F);
 }
+// the same with the B operand's block scale at 2^-1 (E8M0 126)
+__device__ __forceinline__ v4f mfma_f4_half_b(const v4i a, const v4i b, const v4f c) {
+    const v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0}, b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7E7E7E7E);
+}
 
 template <int NSBW, int TG, int PRO>
 __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
@@ -498,7 +503,7 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     const uint32_t be = mxb >> 23;
     const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x|
     const int sh = OXB_F4_P - E + (pm == 0 ? 2 : (pm == 1 ? 1 : 0));
-    const uint32_t flip = pm == 3 ? 0x80000000u : 0u;  // the m = 3 operand reads -1 for a set bit
+    const uint32_t flip = pm == 3 ? 0x88888888u : 0u;  // the m = 3 operand reads -1 for a set bit: all eight signs turn
 
     v4i A[NSBW][4];   // [superblock][block]: digit c of the block's activations, group g
     v4f C4[NSBW][4];  // accumulator start values of digits 4 g .. 4 g + 3
@@ -508,8 +513,9 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
 #pragma unroll
         for (int e = 0; e < 8; e++) {
             r[e] = (uint32_t)rintf(ldexpf(fabsf(xe[i][e]), sh));
-            sg = (((__float_as_uint(xe[i][e]) ^ flip) >> 31) << (4 * e + 3)) | sg;
+            sg |= (uint32_t)(__float_as_int(xe[i][e]) >> 31) & (8u << (4 * e));  // the sign into bit 3 of nibble e
         }
+        sg ^= flip;
         // 8 x 8 nibble transpose: tr[n] nibble e = r[e] nibble n = digits 2 n and 2 n + 1 of activation e
         uint32_t lo[4], hi[4], tl[4], th[4];
 #pragma unroll
@@ -536,9 +542,8 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            // minus the sum over the block of 2^(s - 1) a for m < 3: operands -0.5, -1, -2 and one halving
-            const v4f h = mfma_f4(A[i][q], (v4i){(int)0x99999999u, (int)0xAAAAAAAAu, (int)0xCCCCCCCCu, 0}, (v4f){0.f, 0.f, 0.f, 0.f});
-            C4[i][q] = (v4f){0.5f * h[0], 0.5f * h[1], 0.5f * h[2], 0.5f * h[3]};
+            // minus the sum over the block of 2^(s - 1) a for m < 3: operands -0.5, -1, -2 at a block scale of 1/2
+            C4[i][q] = mfma_f4_half_b(A[i][q], (v4i){(int)0x99999999u, (int)0xAAAAAAAAu, (int)0xCCCCCCCCu, 0}, (v4f){0.f, 0.f, 0.f, 0.f});
         }
     }
     // digit j of X is worth 2 * 4^j; the tile sums leave the wave as 2^-32 of that, and 2^(E - 30 + 32) follows
