@@ -574,7 +574,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
         mx = max_rows4(mx);
         const float m_new = fmaxf(m_run, mx);      // finite: the block holds a visible key
-        float alpha = expf(m_run - m_new);         // 0 for the wave's first block
+        float alpha = __expf(m_run - m_new);         // 0 for the wave's first block
         float vw[8] = {1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f, 1.f};  // V row scales of the lane's keys in units of u_run
         if constexpr (QC) {
             const float va[8] = {vc0.x, vc0.y, vc0.z, vc0.w, vc1.x, vc1.y, vc1.z, vc1.w};
@@ -596,7 +596,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         v8h_t ph, pl;
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            const float pe = expf(sv[e] - m_new);
+            const float pe = __expf(sv[e] - m_new);
             sum += pe;
             const float pv = QC ? pe * vw[e] : pe;
             const _Float16 hi = (_Float16)pv;
@@ -644,7 +644,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         float o = 0.f, l = 0.f;
 #pragma unroll
         for (int w = 0; w < 4; w++) {
-            const float wgt = mm[w * 16 + h] == -INFINITY ? 0.f : expf(mm[w * 16 + h] - M);  // a wave that saw no key
+            const float wgt = mm[w * 16 + h] == -INFINITY ? 0.f : __expf(mm[w * 16 + h] - M);  // a wave that saw no key
             o = fmaf(mo[(w * 16 + h) * HD + d], wgt, o);
             l = fmaf(ml[w * 16 + h], wgt, l);
         }
@@ -710,7 +710,7 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
         const float mv = lane < used ? ld1(ph) : -INFINITY, lv = lane < used ? ld1(ph + 1) : 0.f;
         float M = mv;
         M = wave_max_f32(M);
-        const float w = lane < used ? expf(mv - M) : 0.f;
+        const float w = lane < used ? __expf(mv - M) : 0.f;
         float L = w * lv;
         L = wave_sum_f32(L);
         wts[hh * 64 + lane] = w;
