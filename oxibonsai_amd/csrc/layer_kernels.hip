@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     // V block per wave; after the loop the merge buffers.  Q * scale of the group's heads has an area of its own, so
     // that a wave whose Q operands are in registers starts staging V without waiting for the others.
     __shared__ __attribute__((aligned(16))) _Float16 vs_all[4][32 * VSTR];
-    __shared__ __attribute__((aligned(16))) float qs[16 * HD];
+    __shared__ __attribute__((aligned(16))) _Float16 qs[2][16 * HD];  // fp16 hi and lo parts, as the B operands take them
     __shared__ uint32_t last_flag;
     __shared__ __attribute__((aligned(16))) _Float16 kv_new[2][HD];  // the new position's K and V rows as stored (fp16 cache)
     static_assert(sizeof(vs_all) >= OXB_ATTN_MERGE_LDS_BYTES(16), "the merge's slot weights and partial sums must fit in the V slices");
@@ -400,8 +400,13 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
             const uint32_t d = lane + 64 * it;
             if (d < half) {
                 const float lo_ = qn.lo[it] * q_in.lo[it] * inv, hi_ = qn.hi[it] * q_in.hi[it] * inv;
-                qs[h * HD + d] = (lo_ * cs_sn.lo[it] - hi_ * cs_sn.hi[it]) * p.scale;
-                qs[h * HD + d + half] = (lo_ * cs_sn.hi[it] + hi_ * cs_sn.lo[it]) * p.scale;
+                // split into fp16 hi + lo here, once per value (not once per lane that reads it)
+                const float qa = (lo_ * cs_sn.lo[it] - hi_ * cs_sn.hi[it]) * p.scale, qb = (lo_ * cs_sn.hi[it] + hi_ * cs_sn.lo[it]) * p.scale;
+                const _Float16 ha = (_Float16)qa, hb = (_Float16)qb;
+                qs[0][h * HD + d] = ha;
+                qs[1][h * HD + d] = (_Float16)(qa - (float)ha);
+                qs[0][h * HD + d + half] = hb;
+                qs[1][h * HD + d + half] = (_Float16)(qb - (float)hb);
             }
         }
     }
@@ -473,18 +478,16 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     else lds_barrier();
     if (!EARLY) request_first();
 
-    // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo
+    // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo: one
+    // 16-byte LDS read each.  Columns past the group's heads repeat head 0; nothing of them is ever stored.
     v8h_t qh[KS], ql[KS];
+    const uint32_t hq = qi < G ? qi : 0u;
 #pragma unroll
-    for (int s = 0; s < KS; s++)
-#pragma unroll
-        for (int e = 0; e < 8; e++) {
-            const uint32_t d = QC ? (HD / 4) * g + 8 * s + e : 32 * s + 8 * g + e;
-            const float x = qi < G ? qs[qi * HD + d] : 0.f;
-            const _Float16 hi = (_Float16)x;
-            qh[s][e] = hi;
-            ql[s][e] = (_Float16)(x - (float)hi);
-        }
+    for (int s = 0; s < KS; s++) {
+        const uint32_t d = QC ? (HD / 4) * g + 8 * s : 32 * s + 8 * g;
+        qh[s] = *reinterpret_cast<const v8h_t*>(&qs[0][hq * HD + d]);
+        ql[s] = *reinterpret_cast<const v8h_t*>(&qs[1][hq * HD + d]);
+    }
     v4f O[NS];
 #pragma unroll
     for (int i = 0; i < NS; i++) O[i] = (v4f){0.f, 0.f, 0.f, 0.f};
