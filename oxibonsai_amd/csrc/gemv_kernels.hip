@@ -29,7 +29,9 @@
 // planes in memory.  Every workgroup repeats that work; it hides behind the first HBM round trip.
 //
 // Kernels:
-//   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y
+//   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y: ternary weights, and Q1
+//                        weights against two to four vectors (int8 matrix cores, described above)
+//   gemv_f4_kernel       the same for one vector of Q1 weights on the fp4 matrix-core instruction (described there)
 //   stream_floor_kernel  the same loads and nothing else (measurement aid)
 //   dequant_kernel       resident layout -> fp32 weights (bit-exactness check)
 //   repack_kernel        the reference's block bytes (array of structs) -> resident layout, at upload

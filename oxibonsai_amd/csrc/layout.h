@@ -15,6 +15,8 @@
 //  Q1_0_g128 codes : unit (tile, sb) = 64 lanes x 16 B.
 //     lane (r,g), dword q (0..3) = sign bits 32g..32g+31 of block 4*sb+q, row 16*tile+r
 //     (bit i of the dword = weight 128*(4sb+q) + 32g + i; 1 -> +d, 0 -> -d).
+//     The fp4 route of the GEMV (v_mfma_scale_f32_16x16x128_f8f6f4) reads the same dword as eight E2M1 nibbles:
+//     bit m of nibble n is weight 4n + m, and the lane is again (row r, k-group g) of the B operand.
 //
 //  TQ2_0_g128 codes: unit (tile, sb, half) = 64 lanes x 16 B, half = 0,1.
 //     lane (r,g), dword 2*e+m (e,m in 0..1) = the 16 two-bit fields of weights
