@@ -699,6 +699,13 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
     const uint32_t tg = 256u / npar, sh = tid / tg, egl = tid % tg;  // this thread: group egl (+ tg, ...), slots sh + npar u
     constexpr int PRE = 16;
     float4 pre[PRE];
+    // the maxima and sums of the wave's first head are requested ahead of the slot outputs: loads return in issue
+    // order, and the weights are worked out while the outputs are still on their way
+    float mv0 = -INFINITY, lv0 = 0.f;
+    if ((tid >> 6) < nh) {
+        const float* ph = part + ((size_t)(h_first + (tid >> 6)) * p.n_splits + lane) * stride + hd;
+        if (lane < used) mv0 = ld1(ph), lv0 = ld1(ph + 1);
+    }
     {
         const uint32_t e = e0 + egl * 4;
         const float* ph = part + (size_t)(e / hd) * p.n_splits * stride + e % hd;
@@ -710,7 +717,8 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
     }
     for (uint32_t hh = tid >> 6; hh < nh; hh += 4) {
         const float* ph = part + ((size_t)(h_first + hh) * p.n_splits + lane) * stride + hd;
-        const float mv = lane < used ? ld1(ph) : -INFINITY, lv = lane < used ? ld1(ph + 1) : 0.f;
+        const bool first_head = hh == (tid >> 6);
+        const float mv = first_head ? mv0 : (lane < used ? ld1(ph) : -INFINITY), lv = first_head ? lv0 : (lane < used ? ld1(ph + 1) : 0.f);
         float M = mv;
         M = wave_max_f32(M);
         const float w = lane < used ? __expf(mv - M) : 0.f;
