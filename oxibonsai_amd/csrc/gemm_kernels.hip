@@ -67,12 +67,9 @@ __device__ __forceinline__ void row_stats(const float* __restrict__ xr, const fl
                !(fabsf(a.w) <= 3.402823466e38f);
         mx = fmaxf(fmaxf(mx, fmaxf(fabsf(a.x), fabsf(a.y))), fmaxf(fabsf(a.z), fabsf(a.w)));
     }
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-        ss += __shfl_xor(ss, o, 64);
-        mx = fmaxf(mx, __shfl_xor(mx, o, 64));
-        bad |= __shfl_xor(bad, o, 64);
-    }
+    ss = wave_sum_f32(ss);  // DPP and lane swaps: no trips through the LDS pipeline
+    mx = wave_max_f32(mx);
+    bad = __builtin_amdgcn_ballot_w64(bad != 0) != 0;
     if ((tid & 63u) == 0) red_s[tid >> 6] = ss, red_m[tid >> 6] = mx, red_b[tid >> 6] = bad;
     __syncthreads();
     if (tid == 0) {
