@@ -87,7 +87,7 @@ DECODE_CFG = dict(fmt=FMT_Q1, n_layers=36, h=4096, inter=12288, nq=32, nkv=8, hd
 
 
 def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 32), with_gguf: bool = True,
-               long_context: int = 0, long_only: str = "") -> dict:
+               long_context: int = 0, long_only: str = "", long_batches=(8,)) -> dict:
     """Greedy batch-1 decode of the random-init 8B-shape Q1 model: one batched prefill of `prompt_len` random
     token ids fills the context (timed on its own), then `n_tokens` greedy steps are timed.  The per-token time
     is what the caller of the fused entry point sees: embedding row H2D, the replayed HIP graph (36 layers,
@@ -244,6 +244,30 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
                                         "ms_per_token": round(spent / steps_l * 1e3, 4), "tok_per_s": round(steps_l / spent, 1),
                                         "kv_bytes_read_per_token": 2 * cfg["n_layers"] * cfg["nkv"] * kv_row * seen})
         ml.close()
+        # several sequences at once, each deep in its own context: the cache reads dominate the step
+        res["long_context_batched"] = []
+        for B in (() if long_only else long_batches):
+            mlb = HipModel(be, dict(cfg, max_seq=long_context + 64), w, batch=B)
+            t0 = time.perf_counter()
+            for sq in range(B):
+                for c in range(reps):
+                    n = min(prompt_len, long_context - c * prompt_len)
+                    mlb.prefill(rows[:n], pos_start=c * prompt_len, seq=sq, want_logits=False)
+            t_fill = time.perf_counter() - t0
+            toks, spent, steps_l = [int(ids[sq]) for sq in range(B)], 0.0, 16
+            for i in range(steps_l + 2):
+                hidden = np.stack([emb(t) for t in toks])
+                t0 = time.perf_counter()
+                _, out = mlb.forward(hidden, np.full(B, long_context + i, dtype=np.uint32), want_logits=False)
+                if i >= 2:
+                    spent += time.perf_counter() - t0
+                toks = [int(t) for t in out]
+            kv_bytes = B * 2 * cfg["n_layers"] * cfg["nkv"] * cfg["hd"] * 2 * long_context
+            res["long_context_batched"].append({"batch": B, "cache": "fp16 cache", "context_before": long_context,
+                                                "fill_s": round(t_fill, 2), "ms_per_step": round(spent / steps_l * 1e3, 4),
+                                                "tok_per_s": round(B * steps_l / spent, 1), "kv_bytes_read_per_step": kv_bytes,
+                                                "kv_read_GBps": round(kv_bytes / (spent / steps_l) / 1e9, 1)})
+            mlb.close()
     if with_cpu:
         # CPU SIMD tier on the same matrices: linear layers only (one layer x 36 + LM head), an upper bound on its tok/s
         from oracle import oracle
@@ -395,6 +419,8 @@ def main() -> int:
     ap.add_argument("--long-context", type=int, default=32000,
                     help="context of the long-context decode runs (fp16 / int8 / fp8 cache, sliding window); 0 = skip")
     ap.add_argument("--long-context-only", type=str, default="", help="run only the long-context option of this name")
+    ap.add_argument("--long-context-batches", type=str, default="8",
+                    help="batch sizes decoded with every sequence at the long context (fp16 cache; 32 sequences hold 151 GB of cache)")
     ap.add_argument("--no-ternary", action="store_true", help="skip the ternary 1.7B-shape decode leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -642,7 +668,8 @@ def main() -> int:
     if not args.no_decode:
         out["decode"] = decode_leg(be, args.decode_context, args.decode_tokens, not args.no_cpu,
                                    tuple(int(b) for b in args.decode_batches.split(",") if b), not args.no_gguf,
-                                   args.long_context, args.long_context_only)
+                                   args.long_context, args.long_context_only,
+                                   tuple(int(b) for b in args.long_context_batches.split(",") if b))
         if not args.no_ternary:
             out["decode_ternary_1p7b"] = decode_ternary_leg(be, args.decode_context, args.decode_tokens)
     print(json.dumps(out), flush=True)
