@@ -48,7 +48,13 @@ __device__ __forceinline__ uint32_t pack_h2(float a, float b) {
 }
 __device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
 
-// Multiplier and exponent of one token row; all 256 threads of the workgroup call it, thread 0 gets the result.
+// Multiplier and exponent of one token row from the threads' partial results (sum of squares of x, largest |a|,
+// non-finite seen); all 256 threads of the workgroup call it, thread 0 gets the result.
+template <int OP>
+__device__ __forceinline__ void row_finish(float ss, float mx, int bad, uint32_t k, float eps, float* red_s, float* red_m,
+                                           int* red_b, float* mul_out, int32_t* xsh_out);
+
+// The same with the pass over the row in front: a float4 per thread and step, in row order.
 template <int OP>
 __device__ __forceinline__ void row_stats(const float* __restrict__ xr, const float* __restrict__ w, uint32_t k, float eps,
                                           float* red_s, float* red_m, int* red_b, float* mul_out, int32_t* xsh_out) {
@@ -67,6 +73,13 @@ __device__ __forceinline__ void row_stats(const float* __restrict__ xr, const fl
                !(fabsf(a.w) <= 3.402823466e38f);
         mx = fmaxf(fmaxf(mx, fmaxf(fabsf(a.x), fabsf(a.y))), fmaxf(fabsf(a.z), fabsf(a.w)));
     }
+    row_finish<OP>(ss, mx, bad, k, eps, red_s, red_m, red_b, mul_out, xsh_out);
+}
+
+template <int OP>
+__device__ __forceinline__ void row_finish(float ss, float mx, int bad, uint32_t k, float eps, float* red_s, float* red_m,
+                                           int* red_b, float* mul_out, int32_t* xsh_out) {
+    const uint32_t tid = threadIdx.x;
     ss = wave_sum_f32(ss);  // DPP and lane swaps: no trips through the LDS pipeline
     mx = wave_max_f32(mx);
     bad = __builtin_amdgcn_ballot_w64(bad != 0) != 0;
@@ -122,30 +135,81 @@ __device__ __forceinline__ uint4 pack_item(const float* __restrict__ xr, const f
                       pack_h2(a.w * mul, b.w * mul));
 }
 
-// Both steps in one launch for a few token rows (decode batches): one workgroup per token row finds the row's
-// multiplier and then packs the row; rows M .. M_pad - 1 are zero-filled.  Same arithmetic as the two-kernel route.
-template <int FMT, int OP>
+// The two 16-byte pieces of token row xr behind chunk c = 4g + s of block blk (pack_item's loads).
+template <int FMT>
+__device__ __forceinline__ void item_offsets(uint32_t blk, uint32_t c, uint32_t* o0, uint32_t* o1) {
+    const uint32_t g = c >> 2, s = c & 3u;
+    const uint32_t k0 = FMT == OXB_FMT_Q1 ? 32 * g + 4 * s : 32 * g + 16 * (s >> 1) + 4 * (s & 1u);
+    *o0 = blk * 128 + k0;
+    *o1 = *o0 + (FMT == OXB_FMT_Q1 ? 16 : 8);
+}
+
+// Both steps in one launch for a few token rows (decode batches): one workgroup per token row, one pass over the row.
+// A thread requests all of its items - the pieces it will pack, NI of them for rows of up to 2048 NI values - before
+// it uses any, keeps them in registers while the workgroup finds the row's multiplier, and packs them from there;
+// rows M .. M_pad - 1 are zero-filled.  With eight to thirty-two workgroups on the whole GPU the launch is as long
+// as its chain of memory round trips: this way it is one for the row and one for the store.  (The sum of squares adds
+// the row's values in another order than row_stats does: the multiplier may differ from the two-kernel route's in the
+// last bit, within what fp16 activations already cost.)
+template <int FMT, int OP, int NI>
 __global__ __launch_bounds__(256) void xh_pack_rows_kernel(const float* __restrict__ x, const float* __restrict__ w, uint32_t ldx,
                                                             uint32_t k, float eps, uint32_t M, uint32_t M_pad, uint32_t nblk_pad,
                                                             int32_t* __restrict__ xsh, uint4* __restrict__ xh) {
     __shared__ float red_s[4], red_m[4];
     __shared__ int red_b[4];
     __shared__ float mul_s;
-    const uint32_t m = blockIdx.x, tid = threadIdx.x;
-    const float* xr = x + (size_t)m * ldx;
-    float mul = 0.f;
-    if (m < M) {  // uniform over the workgroup
-        int32_t e = 0;
-        row_stats<OP>(xr, w, k, eps, red_s, red_m, red_b, &mul, &e);
-        if (tid == 0) mul_s = mul, xsh[m] = e;
-        __syncthreads();
-        mul = mul_s;
+    const uint32_t m = blockIdx.x, tid = threadIdx.x, n_items = nblk_pad * 16;
+    if (m >= M) {  // uniform over the workgroup
+        for (uint32_t id = tid; id < n_items; id += 256) xh[(size_t)id * M_pad + m] = make_uint4(0, 0, 0, 0);
+        return;
     }
-    for (uint32_t id = tid; id < nblk_pad * 16; id += 256) {
-        const uint32_t blk = id >> 4, c = id & 15u;
-        uint4 o = make_uint4(0, 0, 0, 0);
-        if (m < M && blk * 128 < k) o = pack_item<FMT, OP>(xr, w, k, blk, c, mul);
-        xh[(size_t)id * M_pad + m] = o;
+    const float* xr = x + (size_t)m * ldx;
+    float4 a[NI], b[NI], wa[NI], wb[NI];
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+        const uint32_t id = it * 256 + tid;
+        uint32_t o0, o1;
+        item_offsets<FMT>(id >> 4, id & 15u, &o0, &o1);
+        const bool ok = id < n_items && (id >> 4) * 128 < k;  // blocks past k are padding
+        a[it] = ok ? *reinterpret_cast<const float4*>(xr + o0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        b[it] = ok ? *reinterpret_cast<const float4*>(xr + o1) : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (OP == OXB_PACK_RMSNORM) {
+            wa[it] = ok ? *reinterpret_cast<const float4*>(w + o0) : make_float4(0.f, 0.f, 0.f, 0.f);
+            wb[it] = ok ? *reinterpret_cast<const float4*>(w + o1) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    float ss = 0.f, mx = 0.f;
+    int bad = 0;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+        float4& p = a[it];
+        float4& q = b[it];
+        if (OP == OXB_PACK_RMSNORM) {
+            ss = fmaf(p.x, p.x, fmaf(p.y, p.y, fmaf(p.z, p.z, fmaf(p.w, p.w, ss))));
+            ss = fmaf(q.x, q.x, fmaf(q.y, q.y, fmaf(q.z, q.z, fmaf(q.w, q.w, ss))));
+            p = make_float4(wa[it].x * p.x, wa[it].y * p.y, wa[it].z * p.z, wa[it].w * p.w);
+            q = make_float4(wb[it].x * q.x, wb[it].y * q.y, wb[it].z * q.z, wb[it].w * q.w);
+        }
+        const float v[8] = {p.x, p.y, p.z, p.w, q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            bad |= !(fabsf(v[e]) <= 3.402823466e38f);
+            mx = fmaxf(mx, fabsf(v[e]));
+        }
+    }
+    float mul = 0.f;
+    int32_t e = 0;
+    row_finish<OP>(ss, mx, bad, k, eps, red_s, red_m, red_b, &mul, &e);
+    if (tid == 0) mul_s = mul, xsh[m] = e;
+    __syncthreads();
+    mul = mul_s;
+#pragma unroll
+    for (int it = 0; it < NI; it++) {
+        const uint32_t id = it * 256 + tid;
+        if (id >= n_items) continue;
+        const float4 p = a[it], q = b[it];
+        xh[(size_t)id * M_pad + m] = make_uint4(pack_h2(p.x * mul, q.x * mul), pack_h2(p.y * mul, q.y * mul),
+                                                pack_h2(p.z * mul, q.z * mul), pack_h2(p.w * mul, q.w * mul));
     }
 }
 
@@ -702,19 +766,25 @@ size_t oxb_xh_bytes(uint32_t k, uint32_t M) {
     return nblk_pad * 16 * M_pad * 16;
 }
 
-#define OXB_PACK_ROWS_MAX 64  // up to this many token rows the one-launch packer is used
+#define OXB_PACK_ROWS_MAX 64  // up to this many token rows (of at most 16384 values) the one-launch packer is used
 
 template <int OP>
 static void launch_pack_op(int fmt, const float* d_x, const float* d_w, uint32_t ldx, uint32_t k, uint32_t M, uint32_t M_pad,
                            uint32_t nblk_pad, float eps, float* d_rowmul, uint32_t* d_xh, int32_t* d_xsh, hipStream_t st) {
-    if (M <= OXB_PACK_ROWS_MAX) {
-        if (fmt == OXB_FMT_Q1)
-            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_Q1, OP>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, M_pad,
-                               nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));
-        else
-            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_TQ2, OP>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, M_pad,
-                               nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));
-        return;
+    const uint32_t per_thread = (nblk_pad * 16 + 255) / 256;  // items of a row per thread of the one-launch packer
+    if (M <= OXB_PACK_ROWS_MAX && per_thread <= 8) {
+#define OXB_ROWS_CASE(NI)                                                                                                      \
+    if (per_thread <= NI) {                                                                                                    \
+        if (fmt == OXB_FMT_Q1)                                                                                                 \
+            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_Q1, OP, NI>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, \
+                               M_pad, nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));                                        \
+        else                                                                                                                   \
+            hipLaunchKernelGGL((xh_pack_rows_kernel<OXB_FMT_TQ2, OP, NI>), dim3(M_pad), dim3(256), 0, st, d_x, d_w, ldx, k, eps, M, \
+                               M_pad, nblk_pad, d_xsh, reinterpret_cast<uint4*>(d_xh));                                        \
+        return;                                                                                                                \
+    }
+        OXB_ROWS_CASE(1) OXB_ROWS_CASE(2) OXB_ROWS_CASE(4) OXB_ROWS_CASE(6) OXB_ROWS_CASE(8)
+#undef OXB_ROWS_CASE
     }
     hipLaunchKernelGGL(row_stats_kernel<OP>, dim3(M), dim3(256), 0, st, d_x, d_w, ldx, k, eps, d_rowmul, d_xsh);
     const dim3 grid(M_pad / 16, nblk_pad < 16 ? nblk_pad : 16);
