@@ -44,7 +44,10 @@ def _check_against_truth(got, w64, x, extra=0.0):
                                    (300, 70, 2048), (16, 1, 512), (15, 17, 384), (129, 333, 128),
                                    # few token rows (decode batches): 1, 2 and 4 row tiles per workgroup, K runs
                                    # that do not divide by the eight waves, one and two token tiles
-                                   (8, 8200, 256), (32, 16400, 128), (9, 16400, 256), (20, 4100, 1152), (5, 48, 12288), (31, 9000, 1536)])
+                                   (8, 8200, 256), (32, 16400, 128), (9, 16400, 256), (20, 4100, 1152), (5, 48, 12288), (31, 9000, 1536),
+                                   # the one-launch packer of up to 64 rows: its longest row (eight items per thread), one
+                                   # block more (two-kernel route), item counts between its instantiations, 64 rows
+                                   (5, 100, 16384), (8, 48, 16512), (31, 50, 8576), (64, 33, 6144), (3, 16, 2176)])
 def test_gemm_matches_oracle(backend, fmt, shape):
     m, n, k = shape
     a = synth.make_blocks(fmt, 900 + m + n, n, k)
