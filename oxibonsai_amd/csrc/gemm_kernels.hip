@@ -871,17 +871,25 @@ static hipError_t launch_narrow_case(const OxbGemmParams& p, hipStream_t st) {
     return hipGetLastError();
 }
 
-// Row tiles per workgroup: as many as still leave about one workgroup per CU (every workgroup reads all of the
-// packed activations, so fewer, fatter workgroups mean less traffic out of L2).
+// Row tiles per workgroup (1, 2 or 4): the count that minimises (rounds of workgroups over the CUs) x (row tiles + 2 - a
+// workgroup's time grows with its tiles on top of a fixed part: its start, the K-split sum and the epilogue).  What
+// counts is the last round: 384 workgroups of one tile leave half the CUs with two and the launch as long as those
+// (QKV 6144 x 4096, 8 rows: 5.5 us against 4.7 us as 192 workgroups of two tiles; 32 rows: 8.2 against 6.1).  A tie
+// goes to the larger workgroups (every workgroup reads all of the packed activations); 8B-shape decode with this rule
+// against "as many tiles as leave a workgroup per CU": +2 % at 8 and at 32 sequences.
 static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
     p.ksplit = 1;
     p.sb_per_split = p.n_sb;
-    uint32_t rt = p.n_tiles >= 4 * n_cus ? 4 : (p.n_tiles >= 2 * n_cus ? 2 : 1);
-    if (p.mode == OXB_GEMM_SWIGLU) {
-        if ((p.n_rows & 31u) != 0) return hipErrorInvalidValue;  // gate and up halves of whole row tiles
-        if (rt < 2) rt = 2;
-    }
+    const bool sw = p.mode == OXB_GEMM_SWIGLU;
+    if (sw && (p.n_rows & 31u) != 0) return hipErrorInvalidValue;  // gate and up halves of whole row tiles
     const uint32_t ct = p.M_pad / 16;
+    uint32_t rt = sw ? 2 : 1;
+    uint64_t best_cost = ~0ull;
+    for (uint32_t r = sw ? 2 : 1; r <= 4; r *= 2) {
+        const uint32_t wgs = sw ? (p.n_tiles / 2 + r / 2 - 1) / (r / 2) : (p.n_tiles + r - 1) / r;
+        const uint64_t cost = (uint64_t)((wgs + n_cus - 1) / n_cus) * (r + 2);
+        if (cost <= best_cost) best_cost = cost, rt = r;
+    }
 #define OXB_NARROW_CASE(F, R, C) \
     if (fmt == F && rt == R && ct == C) return launch_narrow_case<F, R, C>(p, st);
     OXB_NARROW_CASE(OXB_FMT_Q1, 1, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 2, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 4, 1)
