@@ -31,7 +31,8 @@
 // Kernels:
 //   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y: ternary weights, and Q1
 //                        weights against two to four vectors (int8 matrix cores, described above)
-//   gemv_f4_kernel       the same for one vector of Q1 weights on the fp4 matrix-core instruction (described there)
+//   gemv_f4_kernel       the same for one vector on the fp4 matrix-core instruction (described there): Q1 weights
+//                        always, TQ2 weights where a workgroup has many row tiles (the LM head)
 //   stream_floor_kernel  the same loads and nothing else (measurement aid)
 //   dequant_kernel       resident layout -> fp32 weights (bit-exactness check)
 //   repack_kernel        the reference's block bytes (array of structs) -> resident layout, at upload
@@ -416,9 +417,22 @@ __device__ __forceinline__ v4f mfma_f4_half_b(const v4i a, const v4i b, const v4
     return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x7E7E7E7E);
 }
 
-template <int NSBW, int TG, int PRO>
+// the same with the B operand's block scale at 2^1 (E8M0 128)
+__device__ __forceinline__ v4f mfma_f4_double_b(const v4i a, const v4i b, const v4f c) {
+    const v8i a8 = {a[0], a[1], a[2], a[3], 0, 0, 0, 0}, b8 = {b[0], b[1], b[2], b[3], 0, 0, 0, 0};
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a8, b8, c, 4, 4, 0, 0x7F7F7F7F, 0, 0x80808080);
+}
+
+// TQ2 weights on the same route.  A stored field is value + 1 (0, 1, 2) and reads (value + 1) / 2 as an E2M1 nibble:
+// the even fields of a code dword are in place after one AND with 0x33333333, the odd ones after a shift by two - and
+// an add of 0x10101010 before the AND, which turns the two's-complement fields at in-byte position 3 into value + 1 like
+// the others (the carry runs into bits that the AND drops).  The two dwords of a lane's 32 weights give the four operand
+// registers: register j, nibble n is weight 2 n + (j & 1) + 16 (j >> 1) of the group, and the prologue's lane m = j
+// quantises exactly those eight activations.  At a block scale of 2 the MFMA sums (value + 1) * digit / 2; the start
+// value - the same digits against a constant -1 - takes the digit sums off again.  No shifts by bit position and no
+// sign turns: every weight reads the same.  A block costs 8 + 4 vector instructions and one MFMA.
+template <int FMT, int NSBW, int TG, int PRO>
 __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
-    constexpr int FMT = OXB_FMT_Q1;
     extern __shared__ uint32_t smem[];
     const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
     const uint32_t c = lane & 15u, g = lane >> 4;  // D: weight row c of the tile, digits 4 g .. 4 g + 3
@@ -443,10 +457,12 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     auto slot_ok = [&](uint32_t grp, uint32_t t) -> bool { return grp < groups && unit_of(grp, t) < n_units && unit_of(grp, t) < u_begin + upw; };
 
     // ---- prologue ----
-    // lane -> (block q of the superblock, 32-weight group gq, bit position m); its eight activations per superblock
-    // are the weights 4 i + m of that group, i = 0 .. 7: nibble i of operand register m.
+    // lane -> (block q of the superblock, 32-weight group gq, operand register m); its eight activations per superblock
+    // are nibble i = 0 .. 7 of that register: Q1 the weights 4 i + m of the group (bit position m), TQ2 the weights
+    // 2 i + (m & 1) + 16 (m >> 1).
     const uint32_t pq = lane >> 4, pg = (lane >> 2) & 3u, pm = lane & 3u;
-    const uint32_t koff = (128u * pq + 32u * pg + pm) * 4u;
+    constexpr uint32_t XS = FMT == OXB_FMT_Q1 ? 16u : 8u;  // bytes between the lane's consecutive activations
+    const uint32_t koff = (128u * pq + 32u * pg + (FMT == OXB_FMT_Q1 ? pm : (pm & 1u) + 16u * (pm >> 1))) * 4u;
     const __amdgpu_buffer_rsrc_t r_x = make_rsrc(p.x, p.k * 4u);
     const __amdgpu_buffer_rsrc_t r_w = make_rsrc(p.norm_w, PRO == OXB_GEMV_PRO_RMSNORM ? p.k * 4u : 0u);
     float xe[NSBW][8], we[NSBW][8];
@@ -455,8 +471,8 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
         const uint32_t off = i < sb_lim ? (sb0 + i) * 2048u + koff : OXB_OOB;  // beyond k the buffer returns 0
 #pragma unroll
         for (int e = 0; e < 8; e++) {
-            xe[i][e] = __uint_as_float(buf_load_b32(r_x, off + 16u * e));
-            if (PRO == OXB_GEMV_PRO_RMSNORM) we[i][e] = __uint_as_float(buf_load_b32(r_w, off + 16u * e));
+            xe[i][e] = __uint_as_float(buf_load_b32(r_x, off + XS * e));
+            if (PRO == OXB_GEMV_PRO_RMSNORM) we[i][e] = __uint_as_float(buf_load_b32(r_w, off + XS * e));
         }
     }
     // Every wave's activation requests enter the CU's memory pipeline before any wave's weight requests: without
@@ -504,8 +520,8 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     if (__builtin_amdgcn_ballot_w64(bad != 0) != 0 && lane == 0) atomicOr(&flags[0], 1);
     const uint32_t be = mxb >> 23;
     const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x|
-    const int sh = OXB_F4_P - E + (pm == 0 ? 2 : (pm == 1 ? 1 : 0));
-    const uint32_t flip = pm == 3 ? 0x88888888u : 0u;  // the m = 3 operand reads -1 for a set bit: all eight signs turn
+    const int sh = OXB_F4_P - E + (FMT == OXB_FMT_Q1 ? (pm == 0 ? 2 : (pm == 1 ? 1 : 0)) : 0);
+    const uint32_t flip = (FMT == OXB_FMT_Q1 && pm == 3) ? 0x88888888u : 0u;  // Q1, m = 3: the operand reads -1 for a set bit, all eight signs turn
 
     v4i A[NSBW][4];   // [superblock][block]: digit c of the block's activations, group g
     v4f C4[NSBW][4];  // accumulator start values of digits 4 g .. 4 g + 3
@@ -544,8 +560,12 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
         __builtin_amdgcn_wave_barrier();
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            // minus the sum over the block of 2^(s - 1) a for m < 3: operands -0.5, -1, -2 at a block scale of 1/2
-            C4[i][q] = mfma_f4_half_b(A[i][q], (v4i){(int)0x99999999u, (int)0xAAAAAAAAu, (int)0xCCCCCCCCu, 0}, (v4f){0.f, 0.f, 0.f, 0.f});
+            // Q1: minus the sum over the block of 2^(s - 1) a for m < 3: operands -0.5, -1, -2 at a block scale of 1/2;
+            // TQ2: minus the sum of all digits
+            if (FMT == OXB_FMT_Q1)
+                C4[i][q] = mfma_f4_half_b(A[i][q], (v4i){(int)0x99999999u, (int)0xAAAAAAAAu, (int)0xCCCCCCCCu, 0}, (v4f){0.f, 0.f, 0.f, 0.f});
+            else
+                C4[i][q] = mfma_f4(A[i][q], (v4i){(int)0xAAAAAAAAu, (int)0xAAAAAAAAu, (int)0xAAAAAAAAu, (int)0xAAAAAAAAu}, (v4f){0.f, 0.f, 0.f, 0.f});
         }
     }
     // digit j of X is worth 2 * 4^j; the tile sums leave the wave as 2^-32 of that, and 2^(E - 30 + 32) follows
@@ -565,10 +585,19 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
             for (int i = 0; i < NSBW; i++) {
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const uint32_t w = (uint32_t)r.w[i][0][q];
-                    const v4i b = {(int)(w & 0x11111111u), (int)(w & 0x22222222u), (int)(w & 0x44444444u),
-                                   (int)((w & 0x88888888u) | 0x22222222u)};
-                    const v4f d = mfma_f4(A[i][q], b, C4[i][q]);
+                    v4f d;
+                    if (FMT == OXB_FMT_Q1) {
+                        const uint32_t w = (uint32_t)r.w[i][0][q];
+                        const v4i b = {(int)(w & 0x11111111u), (int)(w & 0x22222222u), (int)(w & 0x44444444u),
+                                       (int)((w & 0x88888888u) | 0x22222222u)};
+                        d = mfma_f4(A[i][q], b, C4[i][q]);
+                    } else {
+                        const uint32_t lo = (uint32_t)r.w[i][FMT == OXB_FMT_Q1 ? 0 : q >> 1][2 * (q & 1)];
+                        const uint32_t hi = (uint32_t)r.w[i][FMT == OXB_FMT_Q1 ? 0 : q >> 1][2 * (q & 1) + 1];
+                        const v4i b = {(int)(lo & 0x33333333u), (int)(((lo >> 2) + 0x10101010u) & 0x33333333u),
+                                       (int)(hi & 0x33333333u), (int)(((hi >> 2) + 0x10101010u) & 0x33333333u)};
+                        d = mfma_f4_double_b(A[i][q], b, C4[i][q]);
+                    }
                     const uint32_t scw = (q < 2) ? r.sc[i].x : r.sc[i].y;
                     const float sc = f16_bits_to_f32((q & 1) ? scw >> 16 : scw & 0xFFFFu);
 #pragma unroll
@@ -785,13 +814,13 @@ static hipError_t launch_gemv_t(const OxbGemvParams& p, const GemvPlan& pl, hipS
     return hipGetLastError();
 }
 
-template <int NSBW, int TG>
+template <int FMT, int NSBW, int TG>
 static hipError_t launch_gemv_f4_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
     const size_t shm = oxb_gemv_f4_lds_bytes(pl.S, TG);
     if (p.pro == OXB_GEMV_PRO_RMSNORM)
-        hipLaunchKernelGGL((gemv_f4_kernel<NSBW, TG, OXB_GEMV_PRO_RMSNORM>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+        hipLaunchKernelGGL((gemv_f4_kernel<FMT, NSBW, TG, OXB_GEMV_PRO_RMSNORM>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
     else
-        hipLaunchKernelGGL((gemv_f4_kernel<NSBW, TG, OXB_GEMV_PRO_F32>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+        hipLaunchKernelGGL((gemv_f4_kernel<FMT, NSBW, TG, OXB_GEMV_PRO_F32>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
     return hipGetLastError();
 }
 
@@ -824,15 +853,17 @@ hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t
     GemvPlan pl;
     // The fp4 kernel's registers let two workgroups share a CU; that pays where a workgroup has many tiles to
     // spread its prologue over (the LM head: 18 -> 16.8 us), and costs where it has few (the second prologue).
-    const bool f4 = fmt == OXB_FMT_Q1 && p.nvec == 1;
-    if (f4 && p.epi != OXB_GEMV_SWIGLU && p.n_tiles >= 32u * n_cus) n_cus *= 2;
+    // TQ2 weights take it only where a workgroup has many tiles: its block costs 12 instructions and one MFMA against
+    // 15 and two on the int8 route, but its prologue (sixteen digits instead of four) is the longer one - measured,
+    // 1.7B shapes: 3.65 / 3.56 / 4.13 / 5.99 us against 3.19 / 3.11 / 3.88 / 4.80 on the int8 route (QKV, O,
+    // gate || up, down), the LM head 151936 x 2048 15.5 against 17.6 us.
+    const bool many = p.epi != OXB_GEMV_SWIGLU && p.n_tiles >= 32u * n_cus;
+    const bool f4 = p.nvec == 1 && (fmt == OXB_FMT_Q1 || many);
+    if (f4 && many) n_cus *= 2;
     if (!check_gemv_args(p) || !plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
-    if (f4) {  // one vector of Q1 weights: the fp4 route
-#define OXB_F4_CASE(N, T) \
-    if (pl.nsbw == N && pl.tg == T) return launch_gemv_f4_t<N, T>(p, pl, st);
-        OXB_F4_CASE(1, 1) OXB_F4_CASE(1, 2) OXB_F4_CASE(1, 3) OXB_F4_CASE(1, 4) OXB_F4_CASE(2, 1) OXB_F4_CASE(2, 2) OXB_F4_CASE(3, 1)
-#undef OXB_F4_CASE
+    if (f4) {  // one vector: the fp4 route
+        OXB_GEMV_CASES(launch_gemv_f4_t)
     }
     OXB_GEMV_CASES(launch_gemv_t)
     return hipErrorInvalidValue;
@@ -842,7 +873,7 @@ hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus
     if (p.n_tiles == 0) return hipSuccess;
     GemvPlan pl;
     p.epi = OXB_GEMV_STORE;
-    if (fmt == OXB_FMT_Q1 && p.n_tiles >= 32u * n_cus) n_cus *= 2;  // as the single-vector route plans it
+    if (p.n_tiles >= 32u * n_cus) n_cus *= 2;  // as the single-vector route plans it (fp4 for both formats at this size)
     if (!plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
     OXB_GEMV_CASES(launch_floor_t)

@@ -79,44 +79,59 @@ def _weight_bytes(fmt: int, codes, tile: int, sb: int, q: int) -> np.ndarray:
 
 
 F4_P = 30                    # fp4 route: x = 2^(E - 30) X with |X| < 2^30
+F4_TQ2_MIN_TILES = 32 * 256  # row tiles from which one vector of TQ2 weights takes the fp4 route on a 256-CU GPU
 _F4_OPERAND = np.array([0.5, 1.0, 2.0])     # what a set bit reads at position m = 0, 1, 2 of its nibble
 
 
-def quantise_block_f4(xb: np.ndarray, E: int):
+def quantise_block_f4(xb: np.ndarray, E: int, fmt: int = 0):
     """fp4 route, one 128-activation block at the slice exponent E -> (digit values [128][16] as the E2M1 numbers
-    the A operand holds, sign included; start values [16] of the sixteen digit rows)."""
+    the A operand holds, sign included; start values [16] of the sixteen digit rows).  Q1: the shift and the sign
+    follow the bit position m of the weight in its nibble; TQ2: every weight reads the same."""
     k = np.arange(128)
-    m = k & 3                                       # k = 32 g + 4 i + m: bit m of nibble i of the lane's code dword
-    sh = (F4_P - E + np.array([2, 1, 0, 0])[m]).astype(np.int32)
+    m = k & 3                                       # Q1: k = 32 g + 4 i + m: bit m of nibble i of the lane's code dword
+    sh = (F4_P - E + (np.array([2, 1, 0, 0])[m] if fmt == 0 else 0 * m)).astype(np.int32)
     mag = np.rint(np.ldexp(np.abs(xb.astype(np.float32)), sh).astype(np.float32)).astype(np.float64)
     mag = np.nan_to_num(mag, nan=0.0).astype(np.uint64)
-    neg = np.signbit(xb) ^ (m == 3)                 # the m = 3 operand reads -1 for a set bit
+    neg = np.signbit(xb) ^ ((m == 3) if fmt == 0 else False)    # Q1: the m = 3 operand reads -1 for a set bit
     dig = np.stack([((mag >> np.uint64(2 * j)) & np.uint64(3)).astype(np.float64) * 0.5 for j in range(16)], axis=-1)
     dig = np.where(neg[:, None], -dig, dig)
-    bc = np.where(m < 3, -np.array([0.5, 1.0, 2.0, 0.0])[m], 0.0)
-    start = 0.5 * (bc[:, None] * dig).sum(axis=0)
+    if fmt == 0:
+        bc = np.where(m < 3, -np.array([0.5, 1.0, 2.0, 0.0])[m], 0.0)
+        start = 0.5 * (bc[:, None] * dig).sum(axis=0)
+    else:
+        start = -dig.sum(axis=0)                    # the digits against a constant -1
     return dig, start
 
 
-def _weight_operands_f4(codes, tile: int, sb: int, q: int) -> np.ndarray:
-    """E2M1 operand values [16 rows][128 k] of block q of unit (tile, sb), as the AND masks produce them."""
+def _weight_operands_f4(codes, tile: int, sb: int, q: int, fmt: int = 0) -> np.ndarray:
+    """E2M1 operand values [16 rows][128 k] of block q of unit (tile, sb), as the AND masks produce them (TQ2: times
+    the block scale of 2 the instruction applies to that operand: field + 1 -> 0, 1, 2)."""
     out = np.zeros((16, 128), dtype=np.float64)
     for g in range(4):
         lanes = g * 16 + np.arange(16)
-        w = codes[tile, sb, lanes * 4 + q].astype(np.int64)
-        for i in range(32):
-            b = (w >> i) & 1
-            out[:, 32 * g + i] = np.where(b == 1, -1.0, 1.0) if (i & 3) == 3 else b * _F4_OPERAND[i & 3]
+        if fmt == 0:
+            w = codes[tile, sb, lanes * 4 + q].astype(np.int64)
+            for i in range(32):
+                b = (w >> i) & 1
+                out[:, 32 * g + i] = np.where(b == 1, -1.0, 1.0) if (i & 3) == 3 else b * _F4_OPERAND[i & 3]
+        else:
+            for m in range(2):
+                w = codes[tile, sb, (q >> 1) * 256 + lanes * 4 + (q & 1) * 2 + m].astype(np.int64)
+                even = w & 0x33333333
+                odd = ((w >> 2) + 0x10101010) & 0x33333333
+                for n in range(8):
+                    out[:, 32 * g + 16 * m + 2 * n] = (even >> (4 * n)) & 15
+                    out[:, 32 * g + 16 * m + 2 * n + 1] = (odd >> (4 * n)) & 15
     return out
 
 
-def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray) -> np.ndarray:
-    """gemv_f4_kernel step by step (Q1 weights, one activation vector)."""
+def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray, fmt: int = 0) -> np.ndarray:
+    """gemv_f4_kernel step by step (one activation vector)."""
     n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512
     x = np.asarray(x, dtype=np.float32)
     xp = np.zeros(n_sb * 512, dtype=np.float32)
     xp[:k] = x
-    codes = codes_u8.view(np.uint32).reshape(n_tiles, n_sb, 256)
+    codes = codes_u8.view(np.uint32).reshape(n_tiles, n_sb, 256 if fmt == 0 else 512)
     scales = scales_u8.view(np.float16).reshape(n_tiles, n_sb, 16, 4).astype(np.float32)  # [row][q]
     mq = np.ldexp(np.float32(1.0), 2 * np.arange(16) - 31).astype(np.float32)
     y = np.zeros(n_rows, dtype=np.float32)
@@ -135,8 +150,8 @@ def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x:
                     return np.full(n_rows, np.nan, dtype=np.float32)
                 for sb in range(sb_lo, sb_hi):
                     for q in range(4):
-                        dig, start = quantise_block_f4(xp[(sb * 4 + q) * 128:(sb * 4 + q + 1) * 128], E)
-                        r = _f32(start[None, :] + _weight_operands_f4(codes, tile, sb, q) @ dig)   # exact
+                        dig, start = quantise_block_f4(xp[(sb * 4 + q) * 128:(sb * 4 + q + 1) * 128], E, fmt)
+                        r = _f32(start[None, :] + _weight_operands_f4(codes, tile, sb, q, fmt) @ dig)   # exact
                         acc = _fma32(r, np.repeat(scales[tile, sb, :, q][:, None], 16, axis=1), acc)
                 vg = []
                 for g in range(4):                              # the four digits of a lane group, joined by FMAs
@@ -154,10 +169,12 @@ def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x:
 
 
 def gemv(fmt: int, codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray, route: str | None = None) -> np.ndarray:
-    """The route a single activation vector takes on the device: fp4 for Q1 weights, int8 for TQ2 (`route="i8"`
-    forces the int8 route, which Q1 weights take from two vectors on)."""
-    if fmt == 0 and route != "i8":
-        return gemv_f4(codes_u8, scales_u8, n_rows, k, x)
+    """The route a single activation vector takes on the device: fp4 for Q1 weights and, from 32 row tiles per CU on
+    (256 CUs: the LM head), for TQ2 weights; int8 otherwise and for two to four vectors (`route="i8"` / `"f4"` force one)."""
+    if route is None:
+        route = "f4" if fmt == 0 or (n_rows + 15) // 16 >= F4_TQ2_MIN_TILES else "i8"
+    if route == "f4":
+        return gemv_f4(codes_u8, scales_u8, n_rows, k, x, fmt)
     n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512
     x = np.asarray(x, dtype=np.float32)
     xp = np.zeros(n_sb * 512, dtype=np.float32)

@@ -9,6 +9,7 @@ import pytest
 import oxibonsai_amd as ox
 from helpers import (Q1, TQ2, block, cross_tier_q1, dense_f64, metal_tq2, parity_violations, q1_block, rel_err,
                      simd_parity_tq2, tq2_block)
+from kernel_model import F4_TQ2_MIN_TILES, gemv_f4 as model_gemv_f4
 from oracle import oracle
 from oxibonsai_amd import synth
 
@@ -168,11 +169,10 @@ def test_gemv_properties(backend, fmt):
         want = dense_f64(fmt, a, n, k) @ xo.astype(np.float64)
         assert np.max(np.abs(_gemv(backend, fmt, h, xo, n, k) - want)) < 1e-6 * np.max(np.abs(want))
         yb = backend.gemv_cached_batch(h, np.stack([x1, x2]), n, k)[1]
-        if fmt == TQ2:
-            assert np.array_equal(yb, y2)                                                # a batch row = the single vector
-        else:
-            # Q1: one vector takes the fp4 route, two and more the int8 route; both are exact up to their fp32 joins
-            assert np.max(np.abs(yb - y2)) < 2e-6 * np.max(np.abs(y2))
+        # one vector takes the fp4 route, two and more the int8 route; both are exact up to their fp32 joins
+        assert np.max(np.abs(yb - y2)) < 2e-6 * np.max(np.abs(y2))
+        yb3 = backend.gemv_cached_batch(h, np.stack([x2, x1, x2]), n, k)
+        assert np.array_equal(yb3[0], yb) and np.array_equal(yb3[2], yb)            # a batch row does not depend on its place
     finally:
         backend.free_weights(h)
     zero = a.copy().reshape(-1, 18 if fmt == Q1 else 34)
@@ -218,3 +218,31 @@ def test_caller_chosen_handle_ids_and_replacement(backend):
     assert np.max(np.abs(y1 - oracle.gemv(Q1, a1, x, 32, 256))) < 1e-5
     assert np.max(np.abs(y2 - oracle.gemv(Q1, a2, x, 32, 256))) < 1e-5
     backend.free_weights(h)
+
+
+def test_tq2_single_vector_takes_the_fp4_route_on_lm_head_sized_matrices(backend):
+    """From 32 row tiles per CU on, one vector of TQ2 weights goes through the fp4 kernel (two workgroups per CU):
+    bit-equal to the numpy model of that route on the tiles compared (the model walks every block in Python), every
+    row within 1e-5 of the scalar oracle; power-of-two scaling stays exact; ragged last tile, K of two superblocks
+    with the second one partial."""
+    n, k = 16 * F4_TQ2_MIN_TILES + 5, 640
+    a = synth.make_blocks(TQ2, 77, n, k)
+    x = synth.normal_f32(78, k)
+    h = backend.upload_weights_ternary(a, n, k)
+    try:
+        y = backend.gemv_tq2_g128_cached(h, x, n, k)
+        y2 = backend.gemv_tq2_g128_cached(h, np.ldexp(x, 9).astype(np.float32), n, k)
+    finally:
+        backend.free_weights(h)
+    want = oracle.gemv(TQ2, a, x, n, k)
+    assert parity_violations(y, want, GEMV_REL_TOL) == 0
+    assert np.max(np.abs(y - want)) < 1e-5                      # outputs are O(1): the scalar oracle's own order effects
+    assert np.array_equal(y2, np.ldexp(y, 9).astype(np.float32))
+    # the model on the first 40, some middle and the last rows: same blocks, row tiles are independent
+    nblk = k // 128
+    blocks = a.reshape(n, nblk * 34)
+    for r0, r1 in ((0, 40), (65536, 65536 + 48), (n - 21, n)):
+        sub = np.ascontiguousarray(blocks[r0:r1]).reshape(-1)
+        codes, scales = ox.repack(TQ2, sub, r1 - r0, k)
+        m = model_gemv_f4(codes, scales, r1 - r0, k, x, TQ2)
+        assert np.array_equal(y[r0:r1].view(np.uint32), m.view(np.uint32)), (r0, r1)

@@ -103,18 +103,19 @@ def test_device_arithmetic_model_matches_oracle(fmt, shape):
     assert np.max(np.abs(y - yo)) < 1e-5
 
 
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
 @pytest.mark.parametrize("shape", [(16, 128), (40, 640), (33, 1024)])
-def test_int8_route_model_of_q1_weights_matches_oracle(shape):
-    """Q1 weights take the int8 route from two activation vectors on; its model stays held to the oracle too."""
+def test_int8_route_model_matches_oracle(fmt, shape):
+    """From two activation vectors on the weights take the int8 route; its model stays held to the oracle too."""
     n, k = shape
-    a = synth.make_blocks(Q1, 11, n, k)
+    a = synth.make_blocks(fmt, 11, n, k)
     x = synth.normal_f32(5, k)
-    y = kernel_model.gemv(Q1, *ox.repack(Q1, a, n, k), n, k, x, route="i8")
-    want = dense_f64(Q1, a, n, k) @ x.astype(np.float64)
-    yo = oracle.gemv(Q1, a, x, n, k)
+    y = kernel_model.gemv(fmt, *ox.repack(fmt, a, n, k), n, k, x, route="i8")
+    want = dense_f64(fmt, a, n, k) @ x.astype(np.float64)
+    yo = oracle.gemv(fmt, a, x, n, k)
     assert np.max(np.abs(y - want)) <= max(np.max(np.abs(yo - want)) * 2, 1e-6)
     assert np.max(np.abs(y - yo)) < 1e-5
-    y4 = kernel_model.gemv(Q1, *ox.repack(Q1, a, n, k), n, k, x)                  # the fp4 route of one vector
+    y4 = kernel_model.gemv(fmt, *ox.repack(fmt, a, n, k), n, k, x, route="f4")     # the fp4 route of one vector
     assert np.max(np.abs(y - y4)) < 2e-6 * max(1.0, float(np.max(np.abs(y4))))
 
 
@@ -133,6 +134,29 @@ def test_fp4_route_model_special_inputs():
     assert np.max(np.abs(kernel_model.gemv(Q1, *rep, 32, 512, xo) - want)) < 1e-6 * np.max(np.abs(want)) + 1e-4
     xo[3] = np.nan
     assert np.all(np.isnan(kernel_model.gemv(Q1, *rep, 32, 512, xo)))
+
+
+def test_fp4_route_model_tq2_kats_and_special_inputs():
+    """The TQ2 variant of the fp4 route (taken by LM-head-sized launches): the reference's closed forms, every field
+    position incl. the two's-complement ones, zero and NaN inputs, exact power-of-two scaling."""
+    for pat, x, want in [(0xAA, np.ones(128, np.float32), 128.0), (0x00, np.ones(128, np.float32), -128.0),
+                         (0x46, np.ones(128, np.float32), 0.0), (0xFF, np.ones(128, np.float32), 0.0),
+                         (0x02, np.arange(128, dtype=np.float32), float(sum(range(0, 128, 4)) - sum(k for k in range(128) if k % 4))),
+                         (0x80, np.arange(128, dtype=np.float32), float(sum(range(3, 128, 4)) - sum(k for k in range(128) if k % 4 != 3)))]:
+        a = block(TQ2, 1.0, pat)
+        y = kernel_model.gemv(TQ2, *ox.repack(TQ2, a, 1, 128), 1, 128, x, route="f4")
+        assert y[0] == want, (hex(pat), y[0], want)
+    a = synth.make_blocks(TQ2, 5, 20, 640)
+    rep = ox.repack(TQ2, a, 20, 640)
+    x = synth.normal_f32(3, 640)
+    y = kernel_model.gemv(TQ2, *rep, 20, 640, x, route="f4")
+    want = dense_f64(TQ2, a, 20, 640) @ x.astype(np.float64)
+    assert np.max(np.abs(y - want)) < 1e-5
+    assert np.all(kernel_model.gemv(TQ2, *rep, 20, 640, np.zeros(640, np.float32), route="f4") == 0)
+    for s in (-100, 66):
+        assert np.array_equal(kernel_model.gemv(TQ2, *rep, 20, 640, np.ldexp(x, s).astype(np.float32), route="f4"), np.ldexp(y, s).astype(np.float32))
+    x[7] = np.nan
+    assert np.all(np.isnan(kernel_model.gemv(TQ2, *rep, 20, 640, x, route="f4")))
 
 
 def test_device_arithmetic_model_reference_kats():
