@@ -641,7 +641,7 @@ def main() -> int:
         "metric": "quant GEMV HBM GB/s", "value": round(value, 2), "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp4 (E2M1) MFMA on sixteen base-4 digits of 32-bit fixed-point activations (exact block sums), fp32 scales and accumulation; int8 MFMA on four base-256 digits for ternary weights of layer size and for two to four vectors",
+        "dtype": "fp4 (E2M1) MFMA on sixteen base-4 digits of 32-bit fixed-point activations (exact block sums), fp32 scales and accumulation; int8 MFMA on four base-256 digits for two to four vectors",
         "data": "synthetic",
         "config": {"workload": "Q1_0_g128 GEMV set, Qwen3-8B shapes (6144x4096, 24576x4096, 4096x12288), batch 1",
                    "algorithmic_bytes_per_step": set_bytes, "weight_copies": args.copies,

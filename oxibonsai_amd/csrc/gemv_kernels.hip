@@ -29,10 +29,9 @@
 // planes in memory.  Every workgroup repeats that work; it hides behind the first HBM round trip.
 //
 // Kernels:
-//   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y: ternary weights, and Q1
-//                        weights against two to four vectors (int8 matrix cores, described above)
-//   gemv_f4_kernel       the same for one vector on the fp4 matrix-core instruction (described there): Q1 weights
-//                        always, TQ2 weights where a workgroup has many row tiles (the LM head)
+//   gemv_kernel          codes/scales (tiled SoA, see layout.h) x fp32 activations -> y for two to four vectors
+//                        (int8 matrix cores, described above)
+//   gemv_f4_kernel       the same for one vector on the fp4 matrix-core instruction (described there)
 //   stream_floor_kernel  the same loads and nothing else (measurement aid)
 //   dequant_kernel       resident layout -> fp32 weights (bit-exactness check)
 //   repack_kernel        the reference's block bytes (array of structs) -> resident layout, at upload
@@ -430,7 +429,8 @@ __device__ __forceinline__ v4f mfma_f4_double_b(const v4i a, const v4i b, const 
 // registers: register j, nibble n is weight 2 n + (j & 1) + 16 (j >> 1) of the group, and the prologue's lane m = j
 // quantises exactly those eight activations.  At a block scale of 2 the MFMA sums (value + 1) * digit / 2; the start
 // value - the same digits against a constant -1 - takes the digit sums off again.  No shifts by bit position and no
-// sign turns: every weight reads the same.  A block costs 8 + 4 vector instructions and one MFMA.
+// sign turns: every weight reads the same.  A block costs 8 + 4 vector instructions and one MFMA (the int8 route: 15
+// and two).
 template <int FMT, int NSBW, int TG, int PRO>
 __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     extern __shared__ uint32_t smem[];
@@ -459,10 +459,12 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     // ---- prologue ----
     // lane -> (block q of the superblock, 32-weight group gq, operand register m); its eight activations per superblock
     // are nibble i = 0 .. 7 of that register: Q1 the weights 4 i + m of the group (bit position m), TQ2 the weights
-    // 2 i + (m & 1) + 16 (m >> 1).
+    // 2 i + (m & 1) + 16 (m >> 1).  Both load the Q1 set - the four lanes of a group take 16 consecutive bytes per
+    // request - and TQ2 exchanges within the quad afterwards (requests of two 8-byte pieces per quad instead had the
+    // activations arrive 0.5 us later: QKV 4096 x 2048 3.78 against 3.22 us).
     const uint32_t pq = lane >> 4, pg = (lane >> 2) & 3u, pm = lane & 3u;
-    constexpr uint32_t XS = FMT == OXB_FMT_Q1 ? 16u : 8u;  // bytes between the lane's consecutive activations
-    const uint32_t koff = (128u * pq + 32u * pg + (FMT == OXB_FMT_Q1 ? pm : (pm & 1u) + 16u * (pm >> 1))) * 4u;
+    constexpr uint32_t XS = 16u;  // bytes between the lane's consecutive activations
+    const uint32_t koff = (128u * pq + 32u * pg + pm) * 4u;
     const __amdgpu_buffer_rsrc_t r_x = make_rsrc(p.x, p.k * 4u);
     const __amdgpu_buffer_rsrc_t r_w = make_rsrc(p.norm_w, PRO == OXB_GEMV_PRO_RMSNORM ? p.k * 4u : 0u);
     float xe[NSBW][8], we[NSBW][8];
@@ -523,6 +525,22 @@ __global__ __launch_bounds__(512) void gemv_f4_kernel(const OxbGemvParams p) {
     const int sh = OXB_F4_P - E + (FMT == OXB_FMT_Q1 ? (pm == 0 ? 2 : (pm == 1 ? 1 : 0)) : 0);
     const uint32_t flip = (FMT == OXB_FMT_Q1 && pm == 3) ? 0x88888888u : 0u;  // Q1, m = 3: the operand reads -1 for a set bit, all eight signs turn
 
+    if (FMT == OXB_FMT_TQ2) {
+        // lane m holds the activations 4 e + m (what precedes does not depend on which lane holds which); it needs
+        // 2 n + (m & 1) + 16 (m >> 1) = element (n >> 1) + 4 (m >> 1) of lane 2 (n & 1) + (m & 1) of its quad
+#pragma unroll
+        for (int i = 0; i < NSBW; i++) {
+            float t[8];
+#pragma unroll
+            for (int n = 0; n < 8; n++) {
+                const float lo = (n & 1) ? dpp_f32<0xEE>(xe[i][n >> 1]) : dpp_f32<0x44>(xe[i][n >> 1]);          // quad_perm [2,3,2,3] / [0,1,0,1]
+                const float hi = (n & 1) ? dpp_f32<0xEE>(xe[i][4 + (n >> 1)]) : dpp_f32<0x44>(xe[i][4 + (n >> 1)]);
+                t[n] = (pm >> 1) ? hi : lo;
+            }
+#pragma unroll
+            for (int n = 0; n < 8; n++) xe[i][n] = t[n];
+        }
+    }
     v4i A[NSBW][4];   // [superblock][block]: digit c of the block's activations, group g
     v4f C4[NSBW][4];  // accumulator start values of digits 4 g .. 4 g + 3
 #pragma unroll
@@ -853,16 +871,12 @@ hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t
     GemvPlan pl;
     // The fp4 kernel's registers let two workgroups share a CU; that pays where a workgroup has many tiles to
     // spread its prologue over (the LM head: 18 -> 16.8 us), and costs where it has few (the second prologue).
-    // TQ2 weights take it only where a workgroup has many tiles: its block costs 12 instructions and one MFMA against
-    // 15 and two on the int8 route, but its prologue (sixteen digits instead of four) is the longer one - measured,
-    // 1.7B shapes: 3.65 / 3.56 / 4.13 / 5.99 us against 3.19 / 3.11 / 3.88 / 4.80 on the int8 route (QKV, O,
-    // gate || up, down), the LM head 151936 x 2048 15.5 against 17.6 us.
     const bool many = p.epi != OXB_GEMV_SWIGLU && p.n_tiles >= 32u * n_cus;
-    const bool f4 = p.nvec == 1 && (fmt == OXB_FMT_Q1 || many);
+    const bool f4 = p.nvec == 1;
     if (f4 && many) n_cus *= 2;
     if (!check_gemv_args(p) || !plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
-    if (f4) {  // one vector: the fp4 route
+    if (f4) {  // one vector, either format: the fp4 route
         OXB_GEMV_CASES(launch_gemv_f4_t)
     }
     OXB_GEMV_CASES(launch_gemv_t)
@@ -873,7 +887,7 @@ hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus
     if (p.n_tiles == 0) return hipSuccess;
     GemvPlan pl;
     p.epi = OXB_GEMV_STORE;
-    if (p.n_tiles >= 32u * n_cus) n_cus *= 2;  // as the single-vector route plans it (fp4 for both formats at this size)
+    if (p.n_tiles >= 32u * n_cus) n_cus *= 2;  // as the single-vector route plans it 
     if (!plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
     OXB_GEMV_CASES(launch_floor_t)

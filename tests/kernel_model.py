@@ -79,7 +79,6 @@ def _weight_bytes(fmt: int, codes, tile: int, sb: int, q: int) -> np.ndarray:
 
 
 F4_P = 30                    # fp4 route: x = 2^(E - 30) X with |X| < 2^30
-F4_TQ2_MIN_TILES = 32 * 256  # row tiles from which one vector of TQ2 weights takes the fp4 route on a 256-CU GPU
 _F4_OPERAND = np.array([0.5, 1.0, 2.0])     # what a set bit reads at position m = 0, 1, 2 of its nibble
 
 
@@ -169,10 +168,10 @@ def gemv_f4(codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x:
 
 
 def gemv(fmt: int, codes_u8: np.ndarray, scales_u8: np.ndarray, n_rows: int, k: int, x: np.ndarray, route: str | None = None) -> np.ndarray:
-    """The route a single activation vector takes on the device: fp4 for Q1 weights and, from 32 row tiles per CU on
-    (256 CUs: the LM head), for TQ2 weights; int8 otherwise and for two to four vectors (`route="i8"` / `"f4"` force one)."""
+    """The route a single activation vector takes on the device: fp4 (`route="i8"` forces the int8 route, which the
+    weights take from two vectors on)."""
     if route is None:
-        route = "f4" if fmt == 0 or (n_rows + 15) // 16 >= F4_TQ2_MIN_TILES else "i8"
+        route = "f4"
     if route == "f4":
         return gemv_f4(codes_u8, scales_u8, n_rows, k, x, fmt)
     n_tiles, n_sb = (n_rows + 15) // 16, (k + 511) // 512

@@ -9,7 +9,7 @@ import pytest
 import oxibonsai_amd as ox
 from helpers import (Q1, TQ2, block, cross_tier_q1, dense_f64, metal_tq2, parity_violations, q1_block, rel_err,
                      simd_parity_tq2, tq2_block)
-from kernel_model import F4_TQ2_MIN_TILES, gemv_f4 as model_gemv_f4
+from kernel_model import gemv_f4 as model_gemv_f4
 from oracle import oracle
 from oxibonsai_amd import synth
 
@@ -220,12 +220,12 @@ def test_caller_chosen_handle_ids_and_replacement(backend):
     backend.free_weights(h)
 
 
-def test_tq2_single_vector_takes_the_fp4_route_on_lm_head_sized_matrices(backend):
-    """From 32 row tiles per CU on, one vector of TQ2 weights goes through the fp4 kernel (two workgroups per CU):
+def test_tq2_single_vector_on_an_lm_head_sized_matrix(backend):
+    """From 32 row tiles per CU on the single-vector kernel runs two workgroups per CU; ternary weights at that size:
     bit-equal to the numpy model of that route on the tiles compared (the model walks every block in Python), every
     row within 1e-5 of the scalar oracle; power-of-two scaling stays exact; ragged last tile, K of two superblocks
     with the second one partial."""
-    n, k = 16 * F4_TQ2_MIN_TILES + 5, 640
+    n, k = 16 * 32 * 256 + 5, 640
     a = synth.make_blocks(TQ2, 77, n, k)
     x = synth.normal_f32(78, k)
     h = backend.upload_weights_ternary(a, n, k)
