@@ -31,9 +31,9 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 # HBM bytes one gate||up GEMV launch moves: rocprofv3 FETCH_SIZE (x 2.000, calibrated on a 256 MiB copy) + WRITE_SIZE
 # (x 1.000) of the kernel named beside it, from the profile named beside it.  The algorithmic figure is 14 270 464.
-GATE_UP_HBM_TRAFFIC_BYTES = 14_489_600
+GATE_UP_HBM_TRAFFIC_BYTES = 14_486_528
 GATE_UP_HBM_TRAFFIC_SOURCE = "profiles/gemv_q1_qwen3_8b_set_hbm_traffic.txt"
-GATE_UP_KERNEL = "gemv_f4_kernel<1, 3, 0> (Q1 weights, one activation vector, one superblock of K per wave, three row tiles in flight, fp32 input) gate||up 24576x4096"
+GATE_UP_KERNEL = "gemv_f4_kernel<0, 1, 3, 0> (Q1 weights, one activation vector, one superblock of K per wave, three row tiles in flight, fp32 input) gate||up 24576x4096"
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
 FMT_TQ2 = 1
