@@ -279,3 +279,13 @@ def test_rust_overlay_mirrors_the_reference_signatures():
                                      "gate_up_handle_id", "gate_bytes", "up_bytes", "down_handle_id", "down_bytes", "hidden_size",
                                      "intermediate_size"]
     assert params("try_hip_qkv") == ["input", "output", "weight_handle_id", "q_bytes", "k_bytes", "v_bytes", "n_rows", "k"]
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """bench.py measures one GPU: --gpus above 1 ends with a message and a non-zero status before anything is loaded."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "one GPU" in r.stderr and r.stdout.strip() == ""
