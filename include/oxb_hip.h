@@ -77,21 +77,16 @@ int  oxb_hip_weight_info(uint64_t id, int* fmt, uint32_t* n_rows, uint32_t* k, s
 int  oxb_hip_dequant(uint64_t id, float* out, size_t out_len);
 
 /* ---- GEMV / GEMM on resident weights: gemv_q1_g128_cached (KG/mod.rs:457), gemv_tq2_g128_cached (:484).
- * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (weights are streamed once per four vectors). */
+ * x: [batch][k], y: [batch][n_rows], both row-major fp32; batch >= 1 (one pass over the weights serves up to eight
+ * vectors).
+ * Non-finite activations, a deliberate difference: the kernels turn each activation vector into fixed point, which
+ * has no infinity, so a vector that holds an infinity or a NaN anywhere gives a quiet NaN in EVERY output row of that
+ * vector.  The reference's fp32 sums (crates/oxibonsai-kernels/src/gemv.rs:60-84) give +-infinity in the rows a lone
+ * infinity reaches with one sign and NaN where +inf meets -inf or a NaN; none of its tests fixes the case.  The same
+ * holds for the fused model entry points, whose projections are these kernels. */
 int  oxb_hip_gemv(uint64_t id, const float* x, float* y, uint32_t n_rows, uint32_t k, uint32_t batch);
 /* Same with device-resident x / y, asynchronous on the current stream. */
 int  oxb_hip_gemv_dev(uint64_t id, const float* d_x, float* d_y, uint32_t n_rows, uint32_t k, uint32_t batch);
-
-/* Measurement aid (the reference's counterpart is its CUDA_PROFILE / OXIBONSAI_PROFILE_GPU instrumentation,
- * KG/cuda_full_layer/mod.rs:339-344, KG/metal_full_layer/functions.rs:17-35): launch the GEMV kernel (which quantises
- * d_x in its prologue) `iters` times, launch i on weight ids[i % n_ids] (same shape and format), bracketed by HIP
- * events on the stream the kernel runs on.  *avg_us = mean time per launch in microseconds.
- * _floor launches, in place of the GEMV, a kernel that only reads the same codes and scales with the same grid, waves and
- * load ring: the time below which no kernel that streams these bytes can finish on this GPU. */
-int  oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y,
-                          uint32_t n_rows, uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us);
-int  oxb_hip_profile_gemv_floor(const uint64_t* ids, uint32_t n_ids, uint32_t n_rows, uint32_t k, uint32_t warmup,
-                                uint32_t iters, float* avg_us);
 
 /* ---- uncached one-shot calls: gemv_q1_g128 (KG/mod.rs:412), gemm_q1_g128 (:425) and their ternary twins.
  * Validation follows the scalar kernels (crates/oxibonsai-kernels/src/gemv.rs:32-58): k % 128, buffer lengths. */
@@ -105,11 +100,9 @@ int  oxb_hip_gemv_tq2_g128(const uint8_t* aos, size_t n_bytes, const float* x, s
  * y[m][n_rows] = x[m][k] * W^T on the fp16 matrix cores with fp32 accumulation: weights and products are exact,
  * activations are rounded to fp16 after a per-row power-of-two scaling (relative 2^-11 per element).  Use
  * oxb_hip_gemv with batch = m where fp32-exact products are required.  _dev takes device pointers and does not
- * synchronize; profile_gemm packs x once, then times `iters` GEMM launches with events on the library's stream. */
+ * synchronize. */
 int  oxb_hip_gemm(uint64_t id, const float* x, float* y, uint32_t m, uint32_t n_rows, uint32_t k);
 int  oxb_hip_gemm_dev(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k);
-int  oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
-                          uint32_t warmup, uint32_t iters, float* avg_us);
 /* oxb_hip_gemm_dev for callers that cannot allocate (no counterpart in the reference): code under HIP graph capture,
  * serving loops and harnesses that forbid hipMalloc.  Same kernels and results, but the call's scratch - packed fp16
  * activations, per-row exponents, the partial sums of a K split - lies in a 32 MiB array inside the library's code
@@ -295,10 +288,6 @@ int  oxb_hip_decode_tokens(uint64_t model, uint64_t embedding, const uint32_t* t
 typedef struct { float temperature; uint32_t top_k; float top_p; } oxb_sampling;
 int  oxb_hip_decode_tokens_sampled(uint64_t model, uint64_t embedding, const uint32_t* tokens, const uint32_t* pos,
                                    uint32_t n_steps, const oxb_sampling* params, uint64_t* rng_state, uint32_t* tokens_out);
-/* The f32 sum of x[0..n) taken element by element from 0, as the loop `sum += *v` of the reference's softmax does
- * (sampling.rs:126-130); all x >= 0.  The filter-off sampler depends on this order bit for bit; exposed so that it can
- * be checked on its own. */
-int  oxb_hip_sum_in_order(const float* x, uint32_t n, float* sum_out);
 /* The sampler alone on host logits [batch][vocab] (vocab <= 524288). */
 int  oxb_hip_sample_logits(const float* logits, uint32_t vocab, uint32_t batch, const oxb_sampling* params,
                            uint64_t* rng_state, uint32_t* tokens_out);

@@ -100,6 +100,8 @@ def lib() -> C.CDLL:
         L.oxb_simd_set_threads.restype = None
         L.oxb_simd_gemv.argtypes = [C.c_int, u8p, sz, f32p, sz, f32p, sz, sz, sz]
         L.oxb_simd_gemm.argtypes = [C.c_int, u8p, sz, f32p, sz, f32p, sz, sz, sz, sz]
+        L.oxb_simd_gemm_x4.argtypes = [C.c_int, u8p, sz, f32p, sz, f32p, sz, sz, sz, sz]
+        L.oxb_forward_batch.argtypes = [C.c_void_p, C.c_void_p, f32p, sz, sz, f32p, f32p]
         _lib = L
     return _lib
 
@@ -171,11 +173,13 @@ def simd_gemv(fmt: int, blocks, x, n_rows: int, k: int, out: np.ndarray | None =
     return y
 
 
-def simd_gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int) -> np.ndarray:
+def simd_gemm(fmt: int, blocks, x, m: int, n_rows: int, k: int, x4: bool = False) -> np.ndarray:
+    """x4: the route for long prompts (four token rows share each decoded weight chunk; the same bits)."""
     b, xv = _bytes(blocks), _vec(x).reshape(-1)
     bb = Q1_BYTES if fmt == 0 else TQ2_BYTES
     y = np.zeros(m * n_rows, dtype=np.float32)
-    _check(lib().oxb_simd_gemm(fmt, _u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, m, n_rows, k))
+    fn = lib().oxb_simd_gemm_x4 if x4 else lib().oxb_simd_gemm
+    _check(fn(fmt, _u8(b), b.size // bb, _f32(xv), xv.size, _f32(y), y.size, m, n_rows, k))
     return y.reshape(m, n_rows)
 
 
@@ -345,16 +349,19 @@ class OracleModel:
     """
 
     def __init__(self, cfg: dict, weights: dict, kv_f16: bool = False, dot_f64: bool = False, kv_mode: int = None,
-                 window: int = 0, sinks: int = 0):
+                 window: int = 0, sinks: int = 0, simd: bool = False):
         """dot_f64: every linear layer sums in double (not the reference's arithmetic; a yardstick for how far the
-        fp32 summation order moves the result at a given model size).  kv_mode: one of KV_* (default f32, or f16 with
+        fp32 summation order moves the result at a given model size).  simd: the linear layers run on the CPU SIMD
+        tier (the reference's AVX-512 / AVX2 kernels as restated in oxb_simd.cpp, which the tests hold to the scalar
+        kernels) - what makes prompts of thousands of tokens at the 8B shape affordable.  kv_mode: one of KV_* (default f32, or f16 with
         kv_f16); window / sinks: sliding-window attention (window 0 = every earlier position is visible)."""
         if kv_mode is None:
             kv_mode = KV_F16 if kv_f16 else KV_F32
         self.kv_mode = kv_mode
         self.cfg = cfg
         self._keep = []
-        fmt = cfg["fmt"] + (2 if dot_f64 else 0)
+        assert not (dot_f64 and simd)
+        fmt = cfg["fmt"] + (2 if dot_f64 else 0) + (4 if simd else 0)
         h, inter, nq, nkv, hd = cfg["h"], cfg["inter"], cfg["nq"], cfg["nkv"], cfg["hd"]
 
         def lin(arr, n_rows, k):
@@ -387,6 +394,15 @@ class OracleModel:
                                     _f32(logits) if want_logits else None, _f32(normed)))
         return (logits, normed) if want_normed else logits
 
+    def forward_batch(self, hidden, pos_start: int, want_logits: bool = True):
+        """n consecutive positions of the sequence at once (hidden [n][h]), layer by layer: the values of n forward
+        calls in a row.  Returns the last position's logits (or None)."""
+        hv = np.ascontiguousarray(hidden, dtype=np.float32).reshape(-1, self.cfg["h"])
+        logits = np.empty(self.cfg["vocab"], dtype=np.float32) if want_logits else None
+        _check(lib().oxb_forward_batch(C.byref(self._model), self._state, _f32(hv), pos_start, hv.shape[0],
+                                       _f32(logits) if want_logits else None, None))
+        return logits
+
     def cache(self):
         """K and V as attention reads them, [layer][kv_head][max_seq][hd] f32; for a quantised cache also the codes
         (uint8, same shape) and the scales [layer][kv_head][max_seq]: (k, v, k_codes, v_codes, k_scale, v_scale)."""
@@ -402,6 +418,19 @@ class OracleModel:
         return (view(0, C.c_float, n, np.float32, shape), view(1, C.c_float, n, np.float32, shape),
                 view(2, C.c_uint8, n, np.uint8, shape), view(3, C.c_uint8, n, np.uint8, shape),
                 view(4, C.c_float, n // c["hd"], np.float32, shape[:3]), view(5, C.c_float, n // c["hd"], np.float32, shape[:3]))
+
+    def cache_rows(self, layer: int, kv_head: int, pos0: int, n: int):
+        """Rows pos0 .. pos0 + n - 1 of one (layer, kv head) as attention reads them -> (k, v), f32 [n][hd] copies
+        (cache() copies the whole cache, which at a context of 32 768 is gigabytes)."""
+        c = self.cfg
+        assert pos0 + n <= c["max_seq"]
+        off = ((layer * c["nkv"] + kv_head) * c["max_seq"] + pos0) * c["hd"]
+        out = []
+        for which in (0, 1):
+            base = lib().oxb_state_cache(self._state, which)
+            ptr = C.cast(base + off * 4, C.POINTER(C.c_float))
+            out.append(np.ctypeslib.as_array(ptr, shape=(n * c["hd"],)).reshape(n, c["hd"]).copy())
+        return out[0], out[1]
 
     def load_rows(self, layer: int, kv_head: int, pos0: int, k_rows, v_rows):
         """Cache rows as attention shall read them (f32 [n][hd]), e.g. the rows another implementation stored."""

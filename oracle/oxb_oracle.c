@@ -574,6 +574,8 @@ static void linear_fwd_f64(int fmt, const oxb_linear* l, const float* x, float* 
 }
 
 static int linear_fwd(int fmt, const oxb_linear* l, const float* x, float* y) {
+    if (fmt >= 4) /* the SIMD tier, itself held to the scalar kernels by the tests */
+        return oxb_simd_gemv(fmt - 4, l->blocks, l->n_rows * (l->k / OXB_QK), x, l->k, y, l->n_rows, l->n_rows, l->k);
     if (fmt >= 2) {
         linear_fwd_f64(fmt - 2, l, x, y);
         return OXB_OK;
@@ -685,6 +687,109 @@ int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, siz
     if (normed_out) memcpy(normed_out, s->normed, h * 4);
     if (logits) return linear_fwd(m->fmt, &m->lm_head, s->normed, logits);       /* mod.rs:874-880 */
     return OXB_OK;
+}
+
+/* n tokens through one linear layer: x [n][k] -> y [n][n_rows]. */
+static int linear_batch(int fmt, const oxb_linear* l, const float* x, float* y, size_t n) {
+    if (fmt >= 4)
+        return oxb_simd_gemm_x4(fmt - 4, l->blocks, l->n_rows * (l->k / OXB_QK), x, n * l->k, y, n * l->n_rows, n, l->n_rows, l->k);
+    for (size_t t = 0; t < n; t++) {
+        int rc = linear_fwd(fmt, l, x + t * l->k, y + t * l->n_rows);
+        if (rc) return rc;
+    }
+    return OXB_OK;
+}
+
+/* The reference's batched prefill has no arithmetic of its own: its parity test holds it to the token-by-token
+ * forward (model/tests/metal_prefill_ternary_parity_tests.rs:226-366), and so does this - the operations of
+ * oxb_forward_ex, applied to all n tokens one layer at a time. */
+int oxb_forward_batch(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos_start, size_t n,
+                      float* logits, float* normed_out) {
+    if (n == 0 || pos_start + n > m->max_seq || s->frozen || m->hd > 512) return OXB_ERR_DIMENSION_MISMATCH;
+    const size_t h = m->h, hd = m->hd, half = hd / 2, nq = m->nq, nkv = m->nkv, inter = m->inter;
+    const size_t group = nq / nkv, qd = nq * hd, kd = nkv * hd;
+    float* hid = (float*)malloc(n * h * 4);
+    float* nrm = (float*)malloc(n * h * 4);
+    float* q = (float*)malloc(n * qd * 4);
+    float* k = (float*)malloc(n * kd * 4);
+    float* v = (float*)malloc(n * kd * 4);
+    float* att = (float*)malloc(n * qd * 4);
+    float* gate = (float*)malloc(n * inter * 4);
+    float* up = (float*)malloc(n * inter * 4);
+    int rc = OXB_OK;
+    if (!hid || !nrm || !q || !k || !v || !att || !gate || !up) { rc = OXB_ERR_BUFFER_TOO_SMALL; goto out; }
+    memcpy(hid, hidden_in, n * h * 4);
+    for (size_t L = 0; L < m->n_layers && !rc; L++) {
+        const oxb_layer* ly = &m->layers[L];
+#pragma omp parallel for schedule(static)
+        for (size_t t = 0; t < n; t++) oxb_rms_norm(hid + t * h, ly->attn_norm, nrm + t * h, h, m->eps);
+        if ((rc = linear_batch(m->fmt, &ly->q, nrm, q, n))) break;
+        if ((rc = linear_batch(m->fmt, &ly->k, nrm, k, n))) break;
+        if ((rc = linear_batch(m->fmt, &ly->v, nrm, v, n))) break;
+#pragma omp parallel for schedule(static)
+        for (size_t t = 0; t < n; t++) {
+            const size_t pos = pos_start + t;
+            const float* c = s->cos_t + pos * half;
+            const float* sn = s->sin_t + pos * half;
+            float tmp[512];
+            for (size_t hh = 0; hh < nq; hh++) {
+                oxb_rms_norm(q + t * qd + hh * hd, ly->q_norm, tmp, hd, m->eps);
+                oxb_rope_apply(tmp, q + t * qd + hh * hd, c, sn, half);
+            }
+            for (size_t hh = 0; hh < nkv; hh++) {
+                float kr[512];
+                oxb_rms_norm(k + t * kd + hh * hd, ly->k_norm, tmp, hd, m->eps);
+                oxb_rope_apply(tmp, kr, c, sn, half);
+                const size_t row = (L * nkv + hh) * m->max_seq + pos, off = row * hd;
+                if (m->kv_mode >= OXB_KV_I8) {
+                    oxb_kv_quantize_row(m->kv_mode, kr, hd, s->k_codes + off, &s->k_scale[row]);
+                    oxb_kv_quantize_row(m->kv_mode, v + t * kd + hh * hd, hd, s->v_codes + off, &s->v_scale[row]);
+                    oxb_kv_dequantize_row(m->kv_mode, s->k_codes + off, hd, s->k_scale[row], s->k_cache + off);
+                    oxb_kv_dequantize_row(m->kv_mode, s->v_codes + off, hd, s->v_scale[row], s->v_cache + off);
+                    continue;
+                }
+                for (size_t d = 0; d < hd; d++) {
+                    float kv = kr[d], vv = v[t * kd + hh * hd + d];
+                    if (m->kv_mode == OXB_KV_F16) {
+                        kv = oxb_f16_to_f32(oxb_f32_to_f16(kv));
+                        vv = oxb_f16_to_f32(oxb_f32_to_f16(vv));
+                    }
+                    s->k_cache[off + d] = kv;
+                    s->v_cache[off + d] = vv;
+                }
+            }
+        }
+        /* every row of the run is in the cache now; token t reads positions 0 .. pos_start + t only */
+#pragma omp parallel for schedule(dynamic, 1) collapse(2)
+        for (size_t t = 0; t < n; t++)
+            for (size_t qh = 0; qh < nq; qh++) {
+                const size_t base = (L * nkv + qh / group) * m->max_seq * hd;
+                oxb_attention_head_windowed(q + t * qd + qh * hd, s->k_cache + base, s->v_cache + base,
+                                            att + t * qd + qh * hd, pos_start + t + 1, hd, m->window, m->sinks);
+            }
+        if ((rc = linear_batch(m->fmt, &ly->o, att, nrm, n))) break;
+#pragma omp parallel for schedule(static)
+        for (size_t t = 0; t < n; t++) {
+            for (size_t i = 0; i < h; i++) hid[t * h + i] += nrm[t * h + i];
+            oxb_rms_norm(hid + t * h, ly->ffn_norm, nrm + t * h, h, m->eps);
+        }
+        if ((rc = linear_batch(m->fmt, &ly->gate, nrm, gate, n))) break;
+        if ((rc = linear_batch(m->fmt, &ly->up, nrm, up, n))) break;
+#pragma omp parallel for schedule(static)
+        for (size_t t = 0; t < n; t++) oxb_swiglu(gate + t * inter, up + t * inter, gate + t * inter, inter);
+        if ((rc = linear_batch(m->fmt, &ly->down, gate, nrm, n))) break;
+#pragma omp parallel for schedule(static)
+        for (size_t t = 0; t < n; t++)
+            for (size_t i = 0; i < h; i++) hid[t * h + i] += nrm[t * h + i];
+    }
+    if (!rc) {
+        oxb_rms_norm(hid + (n - 1) * h, m->final_norm, s->normed, h, m->eps);
+        if (normed_out) memcpy(normed_out, s->normed, h * 4);
+        if (logits) rc = linear_fwd(m->fmt, &m->lm_head, s->normed, logits);
+    }
+out:
+    free(hid); free(nrm); free(q); free(k); free(v); free(att); free(gate); free(up);
+    return rc;
 }
 
 /* Test aid: rows pos0 .. pos0 + n - 1 of one (layer, kv head) as attention shall read them, e.g. the rows another

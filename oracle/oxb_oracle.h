@@ -117,7 +117,8 @@ typedef struct {
 } oxb_layer;
 
 typedef struct {
-    int fmt;                  /* 0 / 1 as above; 2 / 3: the same formats with every linear layer summed in double */
+    int fmt;                  /* 0 / 1 as above; 2 / 3: the same formats with every linear layer summed in double;
+                                 4 / 5: the same formats with the linear layers on the CPU SIMD tier (oxb_simd.cpp) */
     size_t n_layers, h, inter, nq, nkv, hd, vocab, max_seq;
     float eps, rope_theta;
     const oxb_layer* layers;
@@ -144,6 +145,18 @@ int oxb_forward(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t
 /* Same but also returns the hidden state after the final norm (may be NULL). */
 int oxb_forward_ex(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos,
                    float* logits, float* normed_out);
+
+/* A run of n consecutive positions pos_start .. pos_start + n - 1 of one sequence, layer by layer (every operation
+ * is per token, so the values are those of n calls of oxb_forward_ex in a row; the linear layers go through the
+ * batched products).  hidden_in [n][h]; logits / normed_out (either may be NULL) receive the last position's. */
+int oxb_forward_batch(const oxb_model* m, oxb_state* s, const float* hidden_in, size_t pos_start, size_t n,
+                      float* logits, float* normed_out);
+
+/* CPU SIMD tier (oxb_simd.cpp): the model forward uses it for its linear layers when oxb_model.fmt is 4 / 5. */
+int oxb_simd_gemv(int fmt, const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                  float* y, size_t y_len, size_t n_rows, size_t k);
+int oxb_simd_gemm_x4(int fmt, const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                     float* y, size_t y_len, size_t m, size_t n_rows, size_t k);
 
 #ifdef __cplusplus
 }

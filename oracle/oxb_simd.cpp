@@ -107,6 +107,75 @@ void tq2_rows_avx512(const uint8_t* blocks, const float* x, float* y, size_t row
     }
 }
 
+/* Four token rows at a time over the same weight rows: every (token, weight row) sum is formed by exactly the
+ * operations of the single-token kernels above, in the same order, so the results are the same bits; what is
+ * shared is the decoded sign / code vector of a chunk, and four independent accumulator chains keep the FMA units
+ * busy.  A test aid for prompts of thousands of tokens (oxb_simd_gemm_x4), not one of the reference's tiers. */
+__attribute__((target("avx512f,avx512bw,avx512vl")))
+void q1_rows_avx512_x4(const uint8_t* blocks, const float* x, size_t ldx, float* y, size_t ldy, size_t row0, size_t row1,
+                       size_t bpr) {
+    /* two weight rows per pass, so that each activation chunk is loaded once for both */
+    for (size_t r = row0; r < row1; r += 2) {
+        const bool two = r + 1 < row1;
+        const uint8_t* rb0 = blocks + r * bpr * OXB_Q1_BYTES;
+        const uint8_t* rb1 = two ? rb0 + bpr * OXB_Q1_BYTES : rb0;
+        __m512 a0[4], a1[4], b0[4], b1[4];   /* a: row r, b: row r + 1; 0 / 1: even / odd chunks */
+        for (int t = 0; t < 4; t++) a0[t] = a1[t] = b0[t] = b1[t] = _mm512_setzero_ps();
+        for (size_t bi = 0; bi < bpr; bi++) {
+            const uint8_t* pa = rb0 + bi * OXB_Q1_BYTES;
+            const uint8_t* pb = rb1 + bi * OXB_Q1_BYTES;
+            const float da = f16_bits_to_f32(pa), db = f16_bits_to_f32(pb);
+            const __m512 sa = _mm512_set1_ps(da), na = _mm512_set1_ps(-da), sb = _mm512_set1_ps(db), nb = _mm512_set1_ps(-db);
+            const float* xb = x + bi * OXB_QK;
+            for (int c = 0; c < 8; c++) {
+                uint16_t ua, ub;   /* little-endian host: the two mask bytes as they lie */
+                std::memcpy(&ua, pa + 2 + 2 * c, 2);
+                std::memcpy(&ub, pb + 2 + 2 * c, 2);
+                const __mmask16 ma = (__mmask16)ua, mb = (__mmask16)ub;
+                /* fma(d, +-x, acc) and fma(+-d, x, acc) round the same exact value: the sign goes to the scale once */
+                const __m512 wa = _mm512_mask_blend_ps(ma, na, sa), wb = _mm512_mask_blend_ps(mb, nb, sb);
+                for (int t = 0; t < 4; t++) {
+                    const __m512 xv = _mm512_loadu_ps(xb + t * ldx + 16 * c);
+                    if (c & 1) { a1[t] = _mm512_fmadd_ps(wa, xv, a1[t]); b1[t] = _mm512_fmadd_ps(wb, xv, b1[t]); }
+                    else       { a0[t] = _mm512_fmadd_ps(wa, xv, a0[t]); b0[t] = _mm512_fmadd_ps(wb, xv, b0[t]); }
+                }
+            }
+        }
+        for (int t = 0; t < 4; t++) {
+            y[t * ldy + r] = _mm512_reduce_add_ps(_mm512_add_ps(a0[t], a1[t]));
+            if (two) y[t * ldy + r + 1] = _mm512_reduce_add_ps(_mm512_add_ps(b0[t], b1[t]));
+        }
+    }
+}
+
+__attribute__((target("avx512f,avx512bw,avx512vl")))
+void tq2_rows_avx512_x4(const uint8_t* blocks, const float* x, size_t ldx, float* y, size_t ldy, size_t row0, size_t row1,
+                        size_t bpr) {
+    for (size_t r = row0; r < row1; r++) {
+        const uint8_t* rb = blocks + r * bpr * OXB_TQ2_BYTES;
+        float row_sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (size_t bi = 0; bi < bpr; bi++) {
+            const uint8_t* b = rb + bi * OXB_TQ2_BYTES;
+            const float* xb = x + bi * OXB_QK;
+            __m512 acc0[4], acc1[4];
+            for (int t = 0; t < 4; t++) acc0[t] = acc1[t] = _mm512_setzero_ps();
+            for (int g = 0; g < 4; g++) {
+                uint32_t p0, p1;
+                std::memcpy(&p0, b + 8 * g, 4);
+                std::memcpy(&p1, b + 8 * g + 4, 4);
+                const __m512 w0 = tq2_decode16_avx512(p0), w1 = tq2_decode16_avx512(p1);
+                for (int t = 0; t < 4; t++) {
+                    acc0[t] = _mm512_fmadd_ps(w0, _mm512_loadu_ps(xb + t * ldx + 32 * g), acc0[t]);
+                    acc1[t] = _mm512_fmadd_ps(w1, _mm512_loadu_ps(xb + t * ldx + 32 * g + 16), acc1[t]);
+                }
+            }
+            const float d = f16_bits_to_f32(b + 32);
+            for (int t = 0; t < 4; t++) row_sum[t] += d * _mm512_reduce_add_ps(_mm512_add_ps(acc0[t], acc1[t]));
+        }
+        for (int t = 0; t < 4; t++) y[t * ldy + r] = row_sum[t];
+    }
+}
+
 /* -------------------------------- AVX2 ---------------------------------- */
 __attribute__((target("avx2,fma")))
 inline float hsum256(__m256 v) {
@@ -341,5 +410,33 @@ int oxb_simd_gemm(int fmt, const uint8_t* blocks, size_t n_blocks, const float* 
     });
     return OXB_OK;
 }
+
+/* The same product as oxb_simd_gemm, bit for bit, for long prompts: on the AVX-512 tier four token rows share each
+ * decoded weight chunk (above); tasks are (group of four tokens) x (run of 1024 weight rows).  Other tiers and the
+ * last m % 4 token rows take oxb_simd_gemm's route.  Not a restatement of a reference tier: a test aid. */
+int oxb_simd_gemm_x4(int fmt, const uint8_t* blocks, size_t n_blocks, const float* x, size_t x_len,
+                     float* y, size_t y_len, size_t m, size_t n_rows, size_t k) {
+    if (k % OXB_QK) return OXB_ERR_NOT_BLOCK_ALIGNED;
+    if (x_len < m * k) return OXB_ERR_DIMENSION_MISMATCH;
+    if (y_len < m * n_rows) return OXB_ERR_BUFFER_TOO_SMALL;
+    size_t bpr = k / OXB_QK;
+    if (n_blocks < n_rows * bpr) return OXB_ERR_BUFFER_TOO_SMALL;
+    ensure_init();
+    const size_t m4 = g_tier == TIER_AVX512 ? m / 4 : 0;
+    if (m4) {
+        const size_t chunk = 1024, rc = (n_rows + chunk - 1) / chunk;
+        g_pool->parallel_for(m4 * rc, [&](size_t task) {
+            const size_t g = task / rc, r0 = (task % rc) * chunk, r1 = std::min(n_rows, r0 + chunk);
+            if (fmt == 0) q1_rows_avx512_x4(blocks, x + 4 * g * k, k, y + 4 * g * n_rows, n_rows, r0, r1, bpr);
+            else          tq2_rows_avx512_x4(blocks, x + 4 * g * k, k, y + 4 * g * n_rows, n_rows, r0, r1, bpr);
+        });
+    }
+    const size_t done = 4 * m4;
+    if (done < m)
+        return oxb_simd_gemm(fmt, blocks, n_blocks, x + done * k, x_len - done * k, y + done * n_rows, y_len - done * n_rows,
+                             m - done, n_rows, k);
+    return OXB_OK;
+}
+
 
 }  // extern "C"

@@ -20,6 +20,7 @@
 #include <vector>
 
 #include "../../include/oxb_hip.h"
+#include "../../include/oxb_hip_measure.h"
 #include "gemm_kernels.h"
 #include "gguf.h"
 #include "gemv_kernels.h"
@@ -1040,11 +1041,16 @@ int oxb_hip_model_set_lm_head(uint64_t model, uint64_t final_norm, uint64_t lm_h
         m.logits = p;
         m.logits_cap = need;
     }
+    // The new head is committed only if everything that depends on it succeeds: on an error the model keeps the
+    // head it had (its graph was dropped above and is captured again by the next step; workspaces only ever grow).
+    const oxb_model_desc before = m.d;
     m.d.final_norm = final_norm;
     m.d.lm_head = lm_head;
     m.d.vocab = lm_head ? vocab : 0;
-    OXB_TRY(size_gemm_workspaces(m));
-    return check_model_handles(m);
+    rc = size_gemm_workspaces(m);
+    if (!rc) rc = check_model_handles(m);
+    if (rc) m.d = before;
+    return rc;
     OXB_API_END
 }
 
@@ -1059,19 +1065,20 @@ int oxb_hip_decode_hidden(uint64_t model, const float* hidden, const uint32_t* p
     for (uint32_t b = 0; b < d.batch; b++)
         if (pos[b] >= d.max_seq)
             return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: position %u exceeds the context of %u", pos[b], d.max_seq);
+    // the normed rows go through the gate || up buffer (free once the last layer is done): 2 * inter values per
+    // sequence.  Checked, like every argument, before the step touches the cache.
+    if ((size_t)2 * d.inter < d.h) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden %u exceeds 2 x intermediate %u", d.h, d.inter);
     if (m.checked_gen != g_rt.weights_gen) OXB_TRY(check_model_handles(m));
+    int rc = OXB_HIP_OK;
+    const float* final_norm = d.final_norm ? vec_ptr(d.final_norm, d.h, "final_norm", &rc) : nullptr;
+    if (rc) return rc;
     for (uint32_t b = 0; b < d.batch; b++) OXB_TRY(kv_reserve(m, b, (uint64_t)pos[b] + 1));
     OXB_TRY(kv_sync_table(m));
     hipStream_t st = g_rt.stream;
     OXB_TRY_HIP(hipMemcpyAsync(m.hidden, hidden, (size_t)d.batch * d.h * 4, hipMemcpyHostToDevice, st), "hidden upload");
     OXB_TRY_HIP(hipMemcpyAsync(m.pos, pos, (size_t)d.batch * 4, hipMemcpyHostToDevice, st), "position upload");
     OXB_TRY(encode_decode_step(m, false));
-    // the normed rows go through the gate || up buffer: free once the last layer is done, 2 * inter values per sequence
-    int rc = OXB_HIP_OK;
-    const float* final_norm = d.final_norm ? vec_ptr(d.final_norm, d.h, "final_norm", &rc) : nullptr;
-    if (rc) return rc;
     float* dst = m.gu;
-    if ((size_t)2 * d.inter < d.h) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: hidden %u exceeds 2 x intermediate %u", d.h, d.inter);
     OXB_TRY_HIP(oxb_launch_rmsnorm(m.hidden, final_norm, d.h, d.batch, d.eps, dst, st), "kernel launch failed: rmsnorm");
     for (uint32_t b = 0; b < d.batch; b++)
         OXB_TRY_HIP(hipMemcpyAsync(normed_out + (size_t)b * d.h, dst + (size_t)b * d.h, (size_t)d.h * 4, hipMemcpyDeviceToHost, st),

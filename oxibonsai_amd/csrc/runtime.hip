@@ -16,6 +16,7 @@
 #include <vector>
 
 #include "../../include/oxb_hip.h"
+#include "../../include/oxb_hip_measure.h"
 #include "gemm_kernels.h"
 #include "gemv_kernels.h"
 #include "layout.h"
@@ -96,9 +97,8 @@ static void free_weight_mem(Weight& w) {
     w.d_raw = nullptr;
 }
 
-// Block bytes -> device, shape still open.
-static int upload_weight_bytes(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes) {
-    if (!id) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: id pointer is null");
+// Block bytes -> a device copy, shape still open.  Nothing in the handle table changes here.
+static int make_weight_bytes(int fmt, const uint8_t* aos, size_t n_bytes, Weight* out) {
     const size_t bb = fmt == OXB_FMT_Q1 ? OXB_Q1_AOS_BYTES : OXB_TQ2_AOS_BYTES;
     if (!aos || n_bytes == 0 || n_bytes % bb != 0)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer of %zu bytes is not a whole number of %zu-byte blocks",
@@ -116,6 +116,13 @@ static int upload_weight_bytes(uint64_t* id, int fmt, const uint8_t* aos, size_t
         (void)hipFree(w.d_raw);
         return hip_fail(e, "weight upload");
     }
+    *out = w;
+    return OXB_HIP_OK;
+}
+
+// A finished weight takes its place in the handle table; the one it replaces (a caller-chosen id may name one) is
+// freed only now, when the new copy is complete, so a failed upload leaves the old weight in use.
+static void store_weight(uint64_t* id, const Weight& w) {
     if (*id == 0) *id = g_rt.next_id++;
     if (Weight* old = find_weight(*id)) {
         (void)hipStreamSynchronize(g_rt.stream);  // a launch in flight may still read the old copy
@@ -123,6 +130,14 @@ static int upload_weight_bytes(uint64_t* id, int fmt, const uint8_t* aos, size_t
         g_rt.weights_gen++;
     }
     g_rt.weights[*id] = w;
+}
+
+static int upload_weight_bytes(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes) {
+    if (!id) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: id pointer is null");
+    Weight w;
+    int rc = make_weight_bytes(fmt, aos, n_bytes, &w);
+    if (rc) return rc;
+    store_weight(id, w);
     return OXB_HIP_OK;
 }
 
@@ -174,16 +189,16 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
     const size_t need = (size_t)n_rows * (k / OXB_QK) * bb;
     if (!aos || n_bytes < need)
         return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: weight buffer holds %zu bytes, %zu needed", n_bytes, need);
-    const uint64_t asked = *id;
-    int rc = upload_weight_bytes(id, fmt, aos, need);
+    Weight w;  // raw copy, then the repack; the handle table is touched only when both have succeeded
+    int rc = make_weight_bytes(fmt, aos, need, &w);
     if (rc) return rc;
-    rc = bind_shape(*find_weight(*id), n_rows, k);
+    rc = bind_shape(w, n_rows, k);
     if (rc) {
-        free_weight_mem(*find_weight(*id));
-        g_rt.weights.erase(*id);
-        *id = asked;
+        free_weight_mem(w);
+        return rc;
     }
-    return rc;
+    store_weight(id, w);
+    return OXB_HIP_OK;
 }
 
 // One GEMV over resident weights, any K: launches of at most OXB_GEMV_MAX_SB superblocks, the first with the wanted

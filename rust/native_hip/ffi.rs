@@ -127,18 +127,12 @@ extern "C" {
     // GEMV / GEMM
     pub fn oxb_hip_gemv(id: u64, x: *const f32, y: *mut f32, n_rows: u32, k: u32, batch: u32) -> c_int;
     pub fn oxb_hip_gemv_dev(id: u64, d_x: *const f32, d_y: *mut f32, n_rows: u32, k: u32, batch: u32) -> c_int;
-    pub fn oxb_hip_profile_gemv(ids: *const u64, n_ids: u32, d_x: *const f32, d_y: *mut f32, n_rows: u32, k: u32,
-                                warmup: u32, iters: u32, avg_us: *mut f32) -> c_int;
-    pub fn oxb_hip_profile_gemv_floor(ids: *const u64, n_ids: u32, n_rows: u32, k: u32, warmup: u32, iters: u32,
-                                      avg_us: *mut f32) -> c_int;
     pub fn oxb_hip_gemv_q1_g128(aos: *const u8, n_bytes: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize,
                                 n_rows: u32, k: u32) -> c_int;
     pub fn oxb_hip_gemv_tq2_g128(aos: *const u8, n_bytes: usize, x: *const f32, x_len: usize, y: *mut f32, y_len: usize,
                                  n_rows: u32, k: u32) -> c_int;
     pub fn oxb_hip_gemm(id: u64, x: *const f32, y: *mut f32, m: u32, n_rows: u32, k: u32) -> c_int;
     pub fn oxb_hip_gemm_dev(id: u64, d_x: *const f32, d_y: *mut f32, m: u32, n_rows: u32, k: u32) -> c_int;
-    pub fn oxb_hip_profile_gemm(id: u64, d_x: *const f32, d_y: *mut f32, m: u32, n_rows: u32, k: u32, warmup: u32,
-                                iters: u32, avg_us: *mut f32) -> c_int;
     /// No allocation inside the call (for callers under graph capture or in loops that must not call hipMalloc):
     /// scratch is a 32 MiB array inside the library, larger shapes are `InvalidArgument`, overlapping calls race.
     pub fn oxb_hip_gemm_dev_static(id: u64, d_x: *const f32, d_y: *mut f32, m: u32, n_rows: u32, k: u32) -> c_int;
@@ -183,7 +177,6 @@ extern "C" {
     pub fn oxb_hip_decode_tokens(model: u64, embedding: u64, tokens: *const u32, pos: *const u32, n_steps: u32, tokens_out: *mut u32) -> c_int;
     pub fn oxb_hip_decode_tokens_sampled(model: u64, embedding: u64, tokens: *const u32, pos: *const u32, n_steps: u32,
                                          params: *const OxbSampling, rng_state: *mut u64, tokens_out: *mut u32) -> c_int;
-    pub fn oxb_hip_sum_in_order(x: *const f32, n: u32, sum_out: *mut f32) -> c_int;
     pub fn oxb_hip_sample_logits(logits: *const f32, vocab: u32, batch: u32, params: *const OxbSampling, rng_state: *mut u64,
                                  tokens_out: *mut u32) -> c_int;
     pub fn oxb_hip_prefill_tokens(model: u64, embedding: u64, seq: u32, ids: *const u32, n_tokens: u32, pos_start: u32,

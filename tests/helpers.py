@@ -126,6 +126,7 @@ class DeviceBuffer:
             h.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
             h.hipMemset.argtypes = [C.c_void_p, C.c_int, C.c_size_t]
             h.hipDeviceSynchronize.argtypes = []
+            h.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
             cls._hip = h
         return cls._hip
 

@@ -2,11 +2,16 @@
 
   configs[1]  Q1_0_g128 GEMV at the Qwen3-8B shapes, batch 8 (batch 1 is in test_gpu_gemv.py)
   configs[3]  random-init ternary Qwen3-1.7B, KV context 4096: a seeded prompt, then 128 free-running greedy steps
-  configs[4]  random-init Qwen3-8B-shape Q1 model: decode at batch 8 and 32, and one step at a context of ~32 000
+  configs[4]  random-init Qwen3-8B-shape Q1 model: the 2048-token prefill followed by greedy steps, decode at batch 8
+              and 32, one step at a context of ~32 000, and batch 8 with a KV context of 32 768 whose last sequence is
+              filled to ~32 000 positions (cache offsets beyond 2^32 elements)
 
 Greedy tokens follow the reference's parity test (crates/oxibonsai-model/tests/metal_prefill_ternary_parity_tests.rs:
 317-366): the token must equal the oracle's wherever the oracle's own top-2 margin exceeds the logit tolerance; the
 margin of every step is reported.  Tolerances at these sizes are those of test_gpu_model.test_full_size_shapes_match_oracle."""
+import sys
+import time
+
 import numpy as np
 import pytest
 
@@ -88,6 +93,12 @@ def c4_model():
     yield w
 
 
+@pytest.fixture(scope="module")
+def c4_table():
+    """Embedding rows of 5000 token ids, O(1) activations."""
+    return synth.embedding_rows(0xC4E, range(5000), C4["h"]) * 50.0
+
+
 N_DISTINCT = 4
 
 
@@ -129,7 +140,7 @@ def test_config4_q1_8b_batched_decode(backend, c4_model, c4_oracle_steps, B):
         gpu.close()
 
 
-def test_config4_q1_8b_decode_at_context_32000(backend, c4_model):
+def test_config4_q1_8b_decode_at_context_32000(backend, c4_model, c4_table):
     """KV context 32 768 at the 8B shape: a prompt of 31 990 positions goes in through the batched prefill, then decode
     steps follow.  The oracle cannot walk 32 000 positions of a 36-layer model in test time, so it reads the device's
     own cache rows (every layer and kv head) and is held frozen over them: its forward of the new position then shows
@@ -139,7 +150,7 @@ def test_config4_q1_8b_decode_at_context_32000(backend, c4_model):
     gpu = HipModel(backend, cfg, c4_model, batch=1)
     try:
         ids = synth.token_ids(0xB0A5A1C4, n, 5000)
-        table = synth.embedding_rows(0xC4E, range(5000), cfg["h"]) * 50.0
+        table = c4_table
         for p0 in range(0, n, 4096):                                  # chunked prefill, 4096 positions per call
             gpu.prefill(table[ids[p0:p0 + 4096]], pos_start=p0, want_logits=False)
         steps = []
@@ -161,6 +172,141 @@ def test_config4_q1_8b_decode_at_context_32000(backend, c4_model):
             top2 = np.sort(want)[-2:]
             if top2[1] - top2[0] > 2 * tol:
                 assert tok == oracle.argmax_first(want), step
+        assert gpu.uses_graph()
+    finally:
+        gpu.close()
+
+
+def _say(capsys, msg):
+    """A progress line past pytest's capture: the long tests below must not look hung to whoever watches the output."""
+    with capsys.disabled():
+        print(msg, file=sys.stderr, flush=True)
+
+
+N_PROMPT = 2048
+
+
+@pytest.mark.timeout(900)
+def test_config4_q1_8b_prefill_2048_then_greedy(backend, c4_model, c4_table, capsys):
+    """configs[4] as quoted: 2048 random token ids through the batched prefill (try_cuda_prefill,
+    gpu_backend/cuda_prefill/try_apis.rs:42 -> the LM head of encode_q1.rs:881), then greedy decode on the cache it
+    wrote, at the 8B shape with a KV context of 32 768.  The oracle runs the same 2048 positions layer by layer with
+    its linear layers on the CPU SIMD tier (bit-equal to its token-by-token forward, tests/test_oracle_batch.py; the
+    tier is held to the scalar kernels in tests/test_oracle.py).  Every GEMM tile of the prefill is full here (16
+    token tiles of 128 at the real N and K), which the 8-token prefill of test_full_size_shapes_match_oracle never
+    reaches.  Tolerance: the prefill's (fp16 activations), 5e-3 of the largest logit; the rows of the first layer
+    within one fp16 step plus 2^-11 of the row's scale of the oracle's, those of the last layer within 2e-2 of the row's scale."""
+    cfg = C4
+    ids = synth.token_ids(0xB0A5A1C5, N_PROMPT, 5000)
+    rows = c4_table[ids]
+    gpu = HipModel(backend, cfg, c4_model, batch=1)
+    try:
+        got, tok = gpu.prefill(rows, pos_start=0)
+        _say(capsys, f"config 4: device prefill of {N_PROMPT} tokens done, oracle running")
+        cpu = oracle.OracleModel(cfg, c4_model, kv_f16=True, simd=True)
+        t0 = time.time()
+        want = cpu.forward_batch(rows[:N_PROMPT // 2], 0, want_logits=False)
+        _say(capsys, f"config 4: oracle at position {N_PROMPT // 2} after {time.time() - t0:.0f} s")
+        want = cpu.forward_batch(rows[N_PROMPT // 2:], N_PROMPT // 2)
+        _say(capsys, f"config 4: oracle prefill done after {time.time() - t0:.0f} s")
+        tol = 5e-3 * float(np.max(np.abs(want)))
+        err = float(np.max(np.abs(got - want)))
+        assert err < tol, ("prefill logits", err, tol)
+        top2 = np.sort(want)[-2:]
+        if top2[1] - top2[0] > 2 * tol:
+            assert tok == oracle.argmax_first(want)
+        assert tok == int(np.argmax(got))
+        # what the prefill left in the cache
+        for L, bar in ((0, None), (cfg["n_layers"] - 1, 2e-2)):
+            for hh in (0, cfg["nkv"] - 1):
+                k, v, _, _ = gpu.read_kv(L, hh, 0, N_PROMPT)
+                wk, wv = cpu.cache_rows(L, hh, 0, N_PROMPT)
+                for a, b, name in ((k, wk, "K"), (v, wv, "V")):
+                    a = a.astype(np.float32)
+                    if bar is None:        # one fp16 step of the value plus the GEMM's fp16 activations (2^-11 of the row's scale)
+                        step = (np.spacing(np.maximum(np.abs(a), np.abs(b)).astype(np.float16)).astype(np.float32)
+                                + 2.0 ** -11 * np.max(np.abs(b), axis=1, keepdims=True))
+                        assert np.all(np.abs(a - b) <= step), (L, hh, name, float(np.max(np.abs(a - b) / step)))
+                    else:
+                        scale = np.max(np.abs(b), axis=1, keepdims=True)
+                        assert np.all(np.abs(a - b) <= bar * scale), (L, hh, name, float(np.max(np.abs(a - b) / scale)))
+        # greedy decode on that cache; the device's token feeds both sides
+        worst, undecided = err / tol, 0
+        for step in range(4):
+            r = _row(0xC4D, tok, cfg["h"])
+            want = cpu.forward(r, N_PROMPT + step)
+            g, t = gpu.forward(r, N_PROMPT + step)
+            tol = 5e-3 * float(np.max(np.abs(want)))
+            err = float(np.max(np.abs(g[0] - want)))
+            worst = max(worst, err / tol)
+            assert err < tol, (step, err, tol)
+            top2 = np.sort(want)[-2:]
+            if top2[1] - top2[0] > 2 * tol:
+                assert int(t[0]) == oracle.argmax_first(want), step
+            else:
+                undecided += 1
+            assert int(t[0]) == int(np.argmax(g[0]))
+            tok = int(t[0])
+        _say(capsys, f"config 4: prefill {N_PROMPT} + 4 greedy steps, worst logit error {worst:.2f} of the tolerance, "
+                     f"{undecided} steps inside the tolerance of a tie, oracle {time.time() - t0:.0f} s")
+        assert gpu.uses_graph()
+    finally:
+        gpu.close()
+
+
+@pytest.mark.timeout(600)
+def test_config4_q1_8b_batch8_at_kv_context_32768(backend, c4_model, c4_oracle_steps, c4_table, capsys):
+    """Batch 8 with a KV context of 32 768, as configs[4] quotes it: the last of the eight sequences is filled to
+    31 990 positions, so its cache rows lie beyond 2^32 elements from the start of the allocation (the reference
+    indexes its cache with u32 element counts, gpu_backend/cuda_full_layer/mod.rs:128-130: the case a 64-bit offset
+    exists for).  Sequences 0-6 decode from position 0 with the inputs of c4_oracle_steps; sequence 7 is held to the
+    oracle frozen over the device's own cache rows, as in the batch-1 test above.  Batches of five and more run
+    their projections as fp16 matrix-core GEMMs: prefill tolerance."""
+    cfg, B, n = C4, 8, 31990
+    assert (B - 1) * cfg["n_layers"] * cfg["nkv"] * cfg["max_seq"] * cfg["hd"] > 2 ** 32
+    gpu = HipModel(backend, cfg, c4_model, batch=B)
+    try:
+        ids = synth.token_ids(0xB0A5A1C6, n, 5000)
+        table = c4_table
+        for p0 in range(0, n, 4096):
+            gpu.prefill(table[ids[p0:p0 + 4096]], pos_start=p0, seq=B - 1, want_logits=False)
+        _say(capsys, "config 4, batch 8: sequence 7 filled")
+        steps = []
+        for step in range(2):
+            deep = _row(0xC4F, 7 + step, cfg["h"])
+            hidden = np.stack([_row(0xC40 + b % N_DISTINCT, 1000 * (b % N_DISTINCT) + step, cfg["h"]) for b in range(B - 1)] + [deep])
+            pos = np.array([step] * (B - 1) + [n + step], dtype=np.uint32)
+            got, toks = gpu.forward(hidden, pos)
+            steps.append((deep, got.copy(), toks.copy()))
+            for b in range(B - 1):
+                want = c4_oracle_steps[b % N_DISTINCT][step]
+                tol = 5e-3 * float(np.max(np.abs(want)))
+                err = float(np.max(np.abs(got[b] - want)))
+                assert err < tol, (step, b, err, tol)
+                top2 = np.sort(want)[-2:]
+                if top2[1] - top2[0] > 2 * tol:
+                    assert int(toks[b]) == oracle.argmax_first(want), (step, b)
+                if b >= N_DISTINCT:
+                    assert np.allclose(got[b], got[b - N_DISTINCT], rtol=0, atol=1e-4), (step, b)
+        # no other sequence's rows were touched by the deep one's (and the other way round)
+        k0, v0, _, _ = gpu.read_kv(0, 0, 0, 4, seq=0)
+        k4, v4, _, _ = gpu.read_kv(0, 0, 0, 4, seq=N_DISTINCT)
+        assert np.array_equal(k0[:2], k4[:2]) and np.array_equal(v0[:2], v4[:2]) and not np.any(k0[2:]) and not np.any(v0[2:])
+        cpu = oracle.OracleModel(cfg, c4_model, kv_f16=True, simd=True)
+        for L in range(cfg["n_layers"]):
+            for hh in range(cfg["nkv"]):
+                k, v, _, _ = gpu.read_kv(L, hh, 0, n + 2, seq=B - 1)
+                cpu.load_rows(L, hh, 0, k.astype(np.float32), v.astype(np.float32))
+        cpu.freeze()
+        _say(capsys, "config 4, batch 8: oracle holds the deep sequence's rows")
+        for step, (deep, got, toks) in enumerate(steps):
+            want = cpu.forward(deep, n + step)
+            tol = 5e-3 * float(np.max(np.abs(want)))
+            err = float(np.max(np.abs(got[B - 1] - want)))
+            assert err < tol, (step, err, tol)
+            top2 = np.sort(want)[-2:]
+            if top2[1] - top2[0] > 2 * tol:
+                assert int(toks[B - 1]) == oracle.argmax_first(want), step
         assert gpu.uses_graph()
     finally:
         gpu.close()

@@ -54,6 +54,7 @@ def test_static_scratch_gemm_rejects_what_does_not_fit(backend):
     n, k, m = 256, 4096, 4096                           # packed activations alone: 32 * 16 * 4096 * 16 B = 32 MiB + the rest
     a = synth.make_blocks(Q1, 9, n, k)
     h = backend.upload_weights_raw(a, n, k)
+    d_x = d_y = None
     try:
         d_x, d_y = DeviceBuffer(m * k * 4), DeviceBuffer(m * n * 4)
         d_x.fill(0)
@@ -63,7 +64,46 @@ def test_static_scratch_gemm_rejects_what_does_not_fit(backend):
         assert L.oxb_hip_synchronize() == 0
         assert L.oxb_hip_gemm_dev_static(int(h), d_x.ptr, d_y.ptr, 16, n, k) == 0   # and small shapes still run
         assert L.oxb_hip_synchronize() == 0
+    finally:
+        for b in (d_x, d_y):
+            if b is not None:
+                b.free()
+        backend.free_weights(h)
+
+
+def _free_bytes() -> int:
+    hip = DeviceBuffer.hip()
+    free, total = C.c_size_t(0), C.c_size_t(0)
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
+def test_static_scratch_gemm_allocates_nothing(backend):
+    """What the entry point exists for: the device's free memory is the same before and after a call, also for a
+    shape larger than any the entry point has seen in this process (a fallback to the library's growing workspace
+    would show here: the probe is first shown to see an allocation of the size in question)."""
+    L = _lib.lib()
+    n, k, m = 1040, 8192, 900                           # packed activations: 8192 x 1024 halves = 16 MiB of the 32
+    a = synth.make_blocks(TQ2, 77, n, k)
+    x = synth.normal_f32(78, m * k).reshape(m, k)
+    h = backend.upload_weights_ternary(a, n, k)
+    d_x, d_y = DeviceBuffer.from_numpy(x), DeviceBuffer(m * n * 4)
+    try:
+        assert L.oxb_hip_synchronize() == 0
+        before = _free_bytes()
+        probe = DeviceBuffer(16 << 20)
+        assert _free_bytes() < before                   # hipMemGetInfo notices 16 MiB
+        probe.free()
+        assert _free_bytes() == before
+        d_y.fill(0xFF)
+        assert L.oxb_hip_gemm_dev_static(int(h), d_x.ptr, d_y.ptr, m, n, k) == 0, _lib.last_error()
+        assert L.oxb_hip_synchronize() == 0
+        assert _free_bytes() == before
+        got = d_y.to_numpy(np.float32, (m, n))
+        d_y.fill(0xFF)
+        assert L.oxb_hip_gemm_dev(int(h), d_x.ptr, d_y.ptr, m, n, k) == 0, _lib.last_error()
+        assert np.array_equal(got.view(np.uint32), d_y.to_numpy(np.float32, (m, n)).view(np.uint32))
+    finally:
         d_x.free()
         d_y.free()
-    finally:
         backend.free_weights(h)
