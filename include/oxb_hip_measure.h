@@ -24,6 +24,12 @@ int  oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x,
                           uint32_t n_rows, uint32_t k, uint32_t warmup, uint32_t iters, float* avg_us);
 int  oxb_hip_profile_gemv_floor(const uint64_t* ids, uint32_t n_ids, uint32_t n_rows, uint32_t k, uint32_t warmup,
                                 uint32_t iters, float* avg_us);
+/* Route selection of oxb_hip_gemv / oxb_hip_gemv_dev, for A/B measurements and tests.  On one route the activations
+ * are quantised by a launch of their own and up to eight vectors share one pass over the weights; on the other every
+ * workgroup quantises them in its prologue (four vectors per pass).  n = 1 (the default): by shape - the first route
+ * from five vectors on, and from two where K exceeds 4096; n = 0: never the first route; n >= 2: the first route from
+ * n vectors on. */
+int  oxb_hip_set_gemv_packed_min_batch(uint32_t n);
 /* Packs x once, then times `iters` prefill GEMM launches with events on the library's stream. */
 int  oxb_hip_profile_gemm(uint64_t id, const float* d_x, float* d_y, uint32_t m, uint32_t n_rows, uint32_t k,
                           uint32_t warmup, uint32_t iters, float* avg_us);

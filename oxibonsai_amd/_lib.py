@@ -79,6 +79,7 @@ _SIGNATURES = {
     "oxb_hip_decode_tokens_sampled": ([C.c_uint64, C.c_uint64, u32p, u32p, C.c_uint32, C.c_void_p, u64p, u32p], C.c_int),
     "oxb_hip_sample_logits": ([f32p, C.c_uint32, C.c_uint32, C.c_void_p, u64p, u32p], C.c_int),
     "oxb_hip_sum_in_order": ([f32p, C.c_uint32, f32p], C.c_int),
+    "oxb_hip_set_gemv_packed_min_batch": ([C.c_uint32], C.c_int),
     "oxb_hip_prefill_tokens": ([C.c_uint64, C.c_uint64, C.c_uint32, u32p, C.c_uint32, C.c_uint32, f32p, u32p], C.c_int),
     "oxb_hip_repack_sizes": ([C.c_int, C.c_uint32, C.c_uint32, szp, szp], C.c_int),
     "oxb_hip_repack": ([C.c_int, u8p, C.c_size_t, C.c_uint32, C.c_uint32, u8p, C.c_size_t, u8p, C.c_size_t], C.c_int),

@@ -444,15 +444,17 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS, RT == 3 ? 2 : 1) void gemm_mfma_k
                                                      (int)xoff[it], (int)soff, 0, 0);
     };
     auto publish = [&]() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory"); };
-    // In the blocks that also request the next superblock's weights, those 3 RT loads are issued after the stage's
-    // loads (memory reads return in order) and stay in flight across the barrier: they come from HBM and have until
-    // the end of the following block, instead of stalling the whole workgroup at the end of this one.
+    // In the blocks that also request the next superblock's weights, those 2 RT loads (codes and scales of each row
+    // tile, load_half) are issued after the stage's loads (memory reads return in order) and stay in flight across
+    // the barrier: they come from HBM and have until the end of the following block, instead of stalling the whole
+    // workgroup at the end of this one.  The count must be exactly the weight loads: one more, and a piece of the
+    // token-tile stage may still be on its way when the next block reads it.
     // Measured: three row tiles per wave gain 19 % from it (QKV 6144 x 4096 at 2048 tokens: 105 -> 85 us); with two, four
     // or five tiles the time does not change or gets 3 % worse, so those keep the plain wait.
     constexpr bool KEEP_W = RT == 3;
     auto publish_keep_weights = [&]() {
         if (KEEP_W)
-            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(3 * RT) : "memory");
+            asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(2 * RT) : "memory");
         else
             publish();
     };

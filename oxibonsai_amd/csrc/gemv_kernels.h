@@ -5,7 +5,8 @@
 
 #include "layout.h"
 
-#define OXB_GEMV_MAX_BATCH 4  // activation vectors per pass over the weights
+#define OXB_GEMV_MAX_BATCH 4         // activation vectors per pass over the weights when the kernel quantises them itself
+#define OXB_GEMV_PACKED_MAX_BATCH 8  // ... when oxb_launch_gemv_pack has quantised them (OxbGemvParams::xq)
 #define OXB_GEMV_MAX_SB 24    // superblocks (512 weights of K) one launch covers: 8 waves x 3
 
 // What the kernel's prologue does with x before quantising it, and what its epilogue does with the row sums.
@@ -19,14 +20,17 @@ enum { OXB_GEMV_STORE = 0,          // y = W a
 struct OxbGemvParams {
     const uint32_t* codes;   // resident codes section
     const uint16_t* scales;  // resident scales section
-    const float* x;          // [nvec][ldx] fp32 activations (device)
+    const float* x;          // [nvec][ldx] fp32 activations (device); unused when xq is set
+    const uint32_t* xq;      // the same vectors as oxb_launch_gemv_pack left them (pro applied there), or nullptr
+    uint32_t xq_bytes;       // extent of xq
+    uint32_t nvg;            // groups of four vectors in xq: (nvec + 3) / 4
     const float* norm_w;     // [k], OXB_GEMV_PRO_RMSNORM only
     float eps;
     float* y;                // [nvec][ldy]
     const float* residual;   // [nvec][ldy], OXB_GEMV_RESIDUAL only
     uint32_t n_rows, n_tiles, n_sb, k;
     uint32_t sb_begin, sb_count;  // K range handled by this launch, in superblocks
-    uint32_t nvec;                // 1 .. OXB_GEMV_MAX_BATCH
+    uint32_t nvec;                // 1 .. OXB_GEMV_MAX_BATCH (OXB_GEMV_PACKED_MAX_BATCH with xq)
     uint32_t ldx, ldy;
     uint32_t tpw;                 // filled by the launcher: tile slots per workgroup
     uint32_t codes_bytes, scales_bytes;  // buffer extents (loads beyond them read 0)
@@ -36,6 +40,13 @@ struct OxbGemvParams {
 // One launch covers at most OXB_GEMV_MAX_SB superblocks of K; the caller splits longer rows (first launch with the
 // wanted epilogue, the following ones with OXB_GEMV_ACCUM).  OXB_GEMV_SWIGLU needs the whole K in one launch.
 hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st);
+// Quantises nvec <= OXB_GEMV_PACKED_MAX_BATCH activation vectors of length k once for oxb_launch_gemv (pro as there:
+// with OXB_GEMV_PRO_RMSNORM the norm weights are multiplied in and the sums of squares are left for the GEMV's
+// epilogue); d_out needs oxb_gemv_pack_bytes(k, nvec) bytes.  The GEMV launch then takes xq = d_out, the same nvec
+// and pro, and any sb_begin / sb_count range.
+size_t oxb_gemv_pack_bytes(uint32_t k, uint32_t nvec);
+hipError_t oxb_launch_gemv_pack(int fmt, int pro, const float* d_x, uint32_t ldx, uint32_t nvec, uint32_t k, const float* d_norm_w,
+                                uint32_t* d_out, hipStream_t st);
 // Measurement aid: reads the same codes and scales with the same grid, waves and load ring as oxb_launch_gemv would
 // use, and does nothing else - the time below which no kernel that streams these bytes can finish.
 hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st);

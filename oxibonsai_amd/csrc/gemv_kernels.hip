@@ -374,6 +374,342 @@ __global__ __launch_bounds__(512) void gemv_kernel(const OxbGemvParams p) {
 }
 
 // ---------------------------------------------------------------------------
+// Five to eight activation vectors (and any count above one, where it is faster): quantised once, multiplied in one
+// pass over the weights.
+//
+// gemv_kernel quantises every vector in every workgroup, which at eight vectors is three quarters of its instructions,
+// and its sixteen A rows hold four vectors, so eight take two passes over the weights.  Here gemv_pack_kernel does the
+// quantising once per GEMV - one wave per (superblock of K, vector), each superblock with a power of two of its own -
+// and leaves, per group of four vectors and superblock, exactly what a wave of the GEMV holds in registers: the A
+// operands of the eight MFMAs (lane l's 16 bytes at l * 16), the accumulator start values, the exponents and, for the
+// RMSNorm prologue, the sums of squares.  gemv_packed_kernel loads them (L2 hits: 8.3 KB per superblock and group)
+// instead of computing them, expands each code dword once and feeds it to the MFMAs of both vector groups.  Where a
+// wave's K slice is too long for two groups' operands to stay in registers (more than one superblock per wave), the
+// groups take turns on the tiles that wait in the ring, and the operands of one follow those of the other through the
+// same registers.
+// Packed layout, dwords, for n_sb superblocks and nvg groups, unit = vg * n_sb + sb:
+//   A   [unit][q * 2 + m][lane][4]      C4 [unit][q][v][4]      EX [unit][v]      SS [unit][v]      CL [unit][q][v][2]
+// (CL = the start values folded as the kernel joins the digit sums, d0 + 256 d1 and d2 + 256 d3: two registers per
+// block instead of four, for the kernels whose K slice leaves no room for C4)
+// ---------------------------------------------------------------------------
+#define OXB_GEMV_EX_BAD 0x7FFFFFFF  // exponent entry of a (superblock, vector) that holds an infinity or a NaN
+
+__host__ __device__ inline size_t oxb_gemv_pack_dwords(uint32_t n_sb, uint32_t nvg) {
+    return (size_t)nvg * n_sb * (2048 + 64 + 4 + 4 + 32);
+}
+
+template <int FMT, int PRO>
+__global__ __launch_bounds__(64) void gemv_pack_kernel(const float* __restrict__ x, uint32_t ldx, uint32_t nvec, uint32_t k,
+                                                       const float* __restrict__ norm_w, uint32_t n_sb, uint32_t nvg,
+                                                       uint32_t* __restrict__ out) {
+    const uint32_t lane = threadIdx.x, sb = blockIdx.x, vec = blockIdx.y, vg = vec >> 2, v = vec & 3u;
+    const uint32_t unit = vg * n_sb + sb, units = nvg * n_sb;
+    uint32_t* A = out + (size_t)unit * 2048;
+    int* C4 = (int*)(out + (size_t)units * 2048 + (size_t)unit * 64);
+    int* EXo = (int*)(out + (size_t)units * (2048 + 64) + (size_t)unit * 4);
+    float* SSo = (float*)(out + (size_t)units * (2048 + 64 + 4) + (size_t)unit * 4);
+    int* CL = (int*)(out + (size_t)units * (2048 + 64 + 4 + 4) + (size_t)unit * 32);
+    constexpr uint32_t KS = FMT == OXB_FMT_Q1 ? 8 : 4;
+    const uint32_t j = lane & 7u, gg = (lane >> 3) & 3u, blh = lane >> 5;
+    const uint32_t koff = (FMT == OXB_FMT_Q1 ? 32 * gg + j : 32 * gg + 16 * (j >> 2) + (j & 3u)) * 4u;
+    const int js = Fix<FMT>::shift_of(j);
+    // a vector beyond nvec reads as zeros: its operands are written all the same, so the GEMV needs no special case
+    const __amdgpu_buffer_rsrc_t r_x = make_rsrc(x + (size_t)(vec < nvec ? vec : 0) * ldx, vec < nvec ? k * 4u : 0u);
+    const __amdgpu_buffer_rsrc_t r_w = make_rsrc(norm_w, PRO == OXB_GEMV_PRO_RMSNORM ? k * 4u : 0u);
+    float xe[2][4], we[2][4];
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        const uint32_t off = (sb * 4 + pass * 2 + blh) * 512u + koff;  // beyond k the buffer returns 0
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) {
+            xe[pass][bb] = __uint_as_float(buf_load_b32(r_x, off + KS * 4u * bb));
+            if (PRO == OXB_GEMV_PRO_RMSNORM) we[pass][bb] = __uint_as_float(buf_load_b32(r_w, off + KS * 4u * bb));
+        }
+    }
+    float ss = 0.f;
+    if (PRO == OXB_GEMV_PRO_RMSNORM) {
+#pragma unroll
+        for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++) {
+                ss = fmaf(xe[pass][bb], xe[pass][bb], ss);
+                xe[pass][bb] *= we[pass][bb];
+            }
+        ss = wave_sum_f32(ss);
+    }
+    uint32_t mxb = 0;
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) mxb = max(mxb, __float_as_uint(xe[pass][bb]) & 0x7FFFFFFFu);
+    mxb = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave_umax(mxb));
+    const bool bad = mxb >= 0x7F800000u;
+    const uint32_t be = mxb >> 23;
+    const int E = (int)(be ? be : 1u) - 126;  // 2^E > max |x| (subnormal maxima share the smallest E)
+    const int sh = Fix<FMT>::P - E - js;
+#pragma unroll
+    for (int pass = 0; pass < 2; pass++) {
+        const uint32_t bl = pass * 2 + blh;
+        int r[4];
+#pragma unroll
+        for (int bb = 0; bb < 4; bb++) r[bb] = bad ? 0 : (int)rintf(ldexpf(xe[pass][bb], sh));
+        uint32_t tb[4];
+        int cl = (r[0] & 0x7FFF) + (r[1] & 0x7FFF) + (r[2] & 0x7FFF) + (r[3] & 0x7FFF);
+        int ch = (r[0] >> 15) + (r[1] >> 15) + (r[2] >> 15) + (r[3] >> 15);
+        if (FMT == OXB_FMT_Q1) {
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++) tb[bb] = (((uint32_t)r[bb] << 1) + 0x00808080u) ^ 0x00808080u;
+        } else {
+#pragma unroll
+            for (int bb = 0; bb < 4; bb++) tb[bb] = ((uint32_t)r[bb] + 0x00808080u) ^ 0x00808080u;
+            if ((j & 3u) == 3u) cl = 0, ch = 0;  // field 3 is two's complement: no bias
+        }
+        cl = half_isum(cl << js), ch = half_isum(ch << js);
+        uint32_t D[4];
+        transpose_bytes4(tb, D);
+        const uint32_t m = j >> 2, jj = j & 3u;
+#pragma unroll
+        for (int d = 0; d < 4; d++) A[(((bl * 2 + m) * 64 + gg * 16 + 4 * v + d) << 2) + jj] = D[d];
+        if ((lane & 31u) == 0) {
+            const long long nc = -(((long long)ch << 15) + cl);  // as three balanced digits and a remainder
+            const unsigned long long t = ((unsigned long long)nc + 0x808080ull) ^ 0x808080ull;
+            const v4i c4 = {(int)(signed char)(t & 0xFF), (int)(signed char)((t >> 8) & 0xFF), (int)(signed char)((t >> 16) & 0xFF),
+                            (int)((long long)t >> 24)};
+            *reinterpret_cast<v4i*>(C4 + (bl * 4 + v) * 4) = c4;
+            CL[(bl * 4 + v) * 2] = c4[0] + (int)((uint32_t)c4[1] << 8);
+            CL[(bl * 4 + v) * 2 + 1] = c4[2] + (int)((uint32_t)c4[3] << 8);
+        }
+    }
+    if (lane == 0) {
+        EXo[v] = bad ? OXB_GEMV_EX_BAD : (mxb ? E - Fix<FMT>::P : 0);
+        SSo[v] = ss;
+    }
+}
+
+// Dynamic LDS of a launch: part [4][NVG][TG][S][64] floats | flags [8]
+__host__ __device__ inline size_t oxb_gemv_packed_lds_bytes(uint32_t S, uint32_t tg, uint32_t nvg) {
+    return ((size_t)4 * nvg * tg * S * 64 + 8) * 4;
+}
+
+// One 128-weight block of a waiting tile -> the two int8 B operands.  The code dword passes through an empty asm
+// statement so that two expansions of the same dword (one per vector group) stay two: kept alive between the groups
+// they would cost eight registers per block.
+template <int FMT, int NSBW>
+__device__ __forceinline__ void expand_block(const TileRegs<FMT, NSBW>& r, int i, int q, v4i& b0, v4i& b1) {
+    if (FMT == OXB_FMT_Q1) {  // 32 sign bits: low nibbles of the four bytes, then the high nibbles
+        uint32_t d0 = (uint32_t)r.w[i][0][q];
+        asm volatile("" : "+v"(d0));
+        const uint32_t d1 = d0 >> 4;
+        b0 = (v4i){(int)(d0 & 0x01010101u), (int)(d0 & 0x02020202u), (int)(d0 & 0x04040404u), (int)(d0 & 0x08080808u)};
+        b1 = (v4i){(int)(d1 & 0x01010101u), (int)(d1 & 0x02020202u), (int)(d1 & 0x04040404u), (int)(d1 & 0x08080808u)};
+    } else {  // 16 two-bit fields each
+        uint32_t d0 = (uint32_t)r.w[i][q >> 1][(q & 1) * 2], d1 = (uint32_t)r.w[i][q >> 1][(q & 1) * 2 + 1];
+        asm volatile("" : "+v"(d0), "+v"(d1));
+        b0 = (v4i){(int)(d0 & 0x03030303u), (int)(d0 & 0x0C0C0C0Cu), (int)(d0 & 0x30303030u), (int)(d0 & 0xC0C0C0C0u)};
+        b1 = (v4i){(int)(d1 & 0x03030303u), (int)(d1 & 0x0C0C0C0Cu), (int)(d1 & 0x30303030u), (int)(d1 & 0xC0C0C0C0u)};
+    }
+}
+template <int FMT, int NSBW>
+__device__ __forceinline__ float block_scale(const TileRegs<FMT, NSBW>& r, int i, int q) {
+    const uint32_t scw = (q < 2) ? r.sc[i].x : r.sc[i].y;
+    return f16_bits_to_f32((q & 1) ? scw >> 16 : scw & 0xFFFFu);
+}
+
+// What the packer left for one (vector group, superblock): MFMA A operands, accumulator start values, exponent.
+template <bool FOLDED>
+struct PackedOps {
+    v4i A[4][2];
+    v4i C4[FOLDED ? 1 : 4];
+    int CL[FOLDED ? 4 : 1][2];
+    int EX;
+};
+
+// NVG = vector groups of the launch (1 or 2: up to eight vectors).  A wave's operands are NVG * NSBW (group,
+// superblock) pairs; NSBW of them are in registers at a time: with a one-superblock slice and two groups both are
+// resident and every expanded block feeds both groups' MFMAs; with longer slices the pairs of group 0 are replaced,
+// as they are used up, by those of group 1 (and back, for the next tile group), so that the requests run NSBW - 1
+// pairs ahead of their use.
+// ONE: every workgroup has a single tile group (the launcher knows): no loop around the tile groups, nothing carried
+// from one to the next - with long K slices that is what keeps the operands of two vector groups out of scratch memory.
+template <int FMT, int NSBW, int TG, int NVG, bool ONE>
+__global__ __launch_bounds__(512) void gemv_packed_kernel(const OxbGemvParams p) {
+    extern __shared__ uint32_t smem[];
+    constexpr bool SIDE = NSBW == 1 && NVG == 2;  // both groups resident, side by side
+    constexpr int NOPS = SIDE ? 2 : NSBW, P = NVG * NSBW;
+    constexpr bool FOLDED = NSBW >= 3;  // start values as two registers per block, added behind the MFMAs
+    typedef PackedOps<FOLDED> Ops;
+    const uint32_t lane = threadIdx.x & 63u, s = threadIdx.x >> 6, S = blockDim.x >> 6;
+    const uint32_t c = lane & 15u, g = lane >> 4;  // D: weight row c of the tile, activation vector g of the group
+    const bool swiglu = p.epi == OXB_GEMV_SWIGLU;
+    float* part = (float*)smem;
+    int* flags = (int*)(part + (size_t)4 * NVG * TG * S * 64);
+
+    const uint32_t lane_c = lane * 16u, lane_s = c * 8u;
+    const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
+    const int sb_lim = (int)(p.sb_begin + p.sb_count) - (int)sb0;  // superblocks of this wave's slice that exist
+    const __amdgpu_buffer_rsrc_t r_codes = make_rsrc(p.codes, p.codes_bytes);
+    const __amdgpu_buffer_rsrc_t r_scales = make_rsrc(p.scales, p.scales_bytes);
+    const __amdgpu_buffer_rsrc_t r_q = make_rsrc(p.xq, p.xq_bytes);
+
+    const uint32_t half_tiles = p.n_tiles >> 1;
+    const uint32_t n_units = swiglu ? half_tiles : p.n_tiles;
+    const uint32_t upw = swiglu ? (p.tpw >> 1) : p.tpw, u_begin = blockIdx.x * upw;
+    const uint32_t groups = ONE ? 1u : p.tpw / TG;
+    auto unit_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return u_begin + (swiglu ? (grp >> 1) : grp) * TG + t; };
+    auto tile_of = [&](uint32_t grp, uint32_t t) -> uint32_t { return unit_of(grp, t) + ((swiglu && (grp & 1u)) ? half_tiles : 0u); };
+    auto slot_ok = [&](uint32_t grp, uint32_t t) -> bool { return grp < groups && unit_of(grp, t) < n_units && unit_of(grp, t) < u_begin + upw; };
+
+    // ---- prologue: requests for the first operands, then (behind a barrier) the weight ring ----
+    const uint32_t q_units = NVG * p.n_sb;
+    const uint32_t c4_base = q_units * 2048u * 4u, ex_base = q_units * (2048u + 64u) * 4u;
+    Ops ops[NOPS];
+    const uint32_t cl_base = q_units * (2048u + 64u + 8u) * 4u;
+    auto load_ops = [&](Ops& o, int vgi, int i, bool wanted) {  // !wanted: zeros, and no data moves
+        const bool ok = wanted && i < sb_lim;
+        const uint32_t unit = __builtin_amdgcn_readfirstlane((uint32_t)vgi * p.n_sb + sb0 + (uint32_t)i);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+#pragma unroll
+            for (int m = 0; m < 2; m++) o.A[q][m] = buf_load_b128(r_q, ok ? lane_c : OXB_OOB, unit * 8192u + (q * 2 + m) * 1024u);
+            if (FOLDED) {
+                const v2u cl = __builtin_amdgcn_raw_buffer_load_b64(r_q, (int)(ok ? g * 8u : OXB_OOB), (int)(cl_base + unit * 128u + q * 32u), 0);
+                o.CL[q][0] = (int)cl.x;
+                o.CL[q][1] = (int)cl.y;
+            } else {
+                o.C4[q] = buf_load_b128(r_q, ok ? g * 16u : OXB_OOB, c4_base + unit * 256u + q * 64u);
+            }
+        }
+        o.EX = (int)buf_load_b32(r_q, ok ? g * 4u : OXB_OOB, ex_base + unit * 16u);
+    };
+    // pair n = (group n / NSBW, superblock n % NSBW) of the wave's slice lives in ops[n % NOPS]
+#pragma unroll
+    for (int n = 0; n < NOPS; n++) load_ops(ops[n], n / NSBW, n % NSBW, true);
+    if (threadIdx.x < 8) flags[threadIdx.x] = 0;  // cleared for every wave once the barrier is passed
+    // every wave's operand requests enter the CU's memory pipeline before any wave's weight requests
+    __builtin_amdgcn_sched_barrier(0);
+    lds_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    TileRegs<FMT, NSBW> ring[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++) {
+        load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+    // a slice with an infinity or a NaN in it: every output of that vector becomes NaN
+    auto take_ex = [&](Ops& o, int vgi) -> int {
+        if (o.EX == OXB_GEMV_EX_BAD) {
+            flags[vgi * 4 + g] = 1;
+            return 0;
+        }
+        return o.EX;
+    };
+
+    // ---- main loop ----
+    for (uint32_t grp = 0; grp < groups; grp++) {
+        float* buf = part + (size_t)(grp & 3u) * NVG * TG * S * 64;
+        float accf[NVG][TG];
+#pragma unroll
+        for (int vgi = 0; vgi < NVG; vgi++)
+#pragma unroll
+            for (int t = 0; t < TG; t++) accf[vgi][t] = 0.f;
+        if (SIDE) {
+            const int ex0 = take_ex(ops[0], 0), ex1 = take_ex(ops[NOPS - 1], 1);
+#pragma unroll
+            for (int t = 0; t < TG; t++) {
+                float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    v4i b0, b1;
+                    expand_block<FMT, NSBW>(ring[t], 0, q, b0, b1);
+                    const float sc = block_scale<FMT, NSBW>(ring[t], 0, q);
+                    v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ops[0].A[q][0], b0, ops[0].C4[q], 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ops[0].A[q][1], b1, acc, 0, 0, 0);
+                    v4i bcc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ops[NOPS - 1].A[q][0], b0, ops[NOPS - 1].C4[q], 0, 0, 0);
+                    bcc = __builtin_amdgcn_mfma_i32_16x16x64_i8(ops[NOPS - 1].A[q][1], b1, bcc, 0, 0, 0);
+                    a0 = fmaf(fmaf((float)(acc[2] + (acc[3] << 8)), 65536.0f, (float)(acc[0] + (acc[1] << 8))), sc, a0);
+                    a1 = fmaf(fmaf((float)(bcc[2] + (bcc[3] << 8)), 65536.0f, (float)(bcc[0] + (bcc[1] << 8))), sc, a1);
+                }
+                load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(grp + 1, t), slot_ok(grp + 1, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
+                __builtin_amdgcn_sched_barrier(0);
+                accf[0][t] = ldexpf(a0, ex0);  // the superblock's 2^(E - P)
+                accf[NVG - 1][t] = ldexpf(a1, ex1);
+            }
+        } else {
+#pragma unroll
+            for (int n = 0; n < P; n++) {
+                const int vgi = n / NSBW, i = n % NSBW;
+                Ops& o = ops[n % NOPS];
+                const int ex = take_ex(o, vgi);
+#pragma unroll
+                for (int t = 0; t < TG; t++) {
+                    float a0 = 0.f;
+#pragma unroll
+                    for (int q = 0; q < 4; q++) {
+                        v4i b0, b1;
+                        expand_block<FMT, NSBW>(ring[t], i, q, b0, b1);
+                        v4i acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.A[q][0], b0, FOLDED ? (v4i){0, 0, 0, 0} : o.C4[FOLDED ? 0 : q], 0, 0, 0);
+                        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(o.A[q][1], b1, acc, 0, 0, 0);
+                        int lo = acc[0] + (acc[1] << 8), hi = acc[2] + (acc[3] << 8);
+                        if (FOLDED) lo += o.CL[FOLDED ? q : 0][0], hi += o.CL[FOLDED ? q : 0][1];
+                        a0 = fmaf(fmaf((float)hi, 65536.0f, (float)lo), block_scale<FMT, NSBW>(ring[t], i, q), a0);
+                    }
+                    accf[vgi][t] += ldexpf(a0, ex);
+                }
+                // this pair's registers take the pair NSBW further on (of the next tile group, past the end)
+                if (P > NOPS && !(ONE && n + NOPS >= P)) {  // unconditional requests (out of range when nothing follows): no second copy to select from
+                    __builtin_amdgcn_sched_barrier(0);  // not above the pair's last use: the requests reuse its registers
+                    load_ops(o, ((n + NOPS) % P) / NSBW, i, n + NOPS < P || grp + 1 < groups);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            if (!ONE) {
+#pragma unroll
+                for (int t = 0; t < TG; t++) {
+                    load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(grp + 1, t), slot_ok(grp + 1, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+        }
+#pragma unroll
+        for (int vgi = 0; vgi < NVG; vgi++)
+#pragma unroll
+            for (int t = 0; t < TG; t++) buf[(((size_t)vgi * TG + t) * S + s) * 64 + lane] = accf[vgi][t];
+        lds_barrier();
+        if (swiglu && !(grp & 1u)) continue;  // the gate sums wait for the up sums of the same rows
+        // thread -> (vector group, slot, vector, row): add the S partial sums in wave order, then the epilogue.  No
+        // second barrier: the next groups write other quarters of `part`, and a quarter is reused only after two more.
+        const float* gbuf = part + (size_t)((grp - 1) & 3u) * NVG * TG * S * 64;
+        for (uint32_t idx = threadIdx.x; idx < (uint32_t)NVG * TG * 64; idx += blockDim.x) {
+            const uint32_t vgt = idx / ((uint32_t)TG * 64), rem = idx % ((uint32_t)TG * 64);
+            const uint32_t t = rem >> 6, ln = rem & 63u, cc = ln & 15u, vv = vgt * 4 + (ln >> 4);
+            if (vv >= p.nvec || !slot_ok(grp, t)) continue;
+            const size_t o0 = (((size_t)vgt * TG + t) * S) * 64 + ln;
+            float v0 = 0.f, v1 = 0.f;
+            for (uint32_t w = 0; w < S; w++) v0 += buf[o0 + (size_t)w * 64];
+            if (swiglu)
+                for (uint32_t w = 0; w < S; w++) v1 += gbuf[o0 + (size_t)w * 64];
+            if (p.pro == OXB_GEMV_PRO_RMSNORM) {  // the superblocks' sums of squares in order, then 1 / rms on the row sums
+                const float* ssq = (const float*)p.xq + (size_t)q_units * (2048 + 64 + 4) + (size_t)vgt * p.n_sb * 4 + (ln >> 4);
+                float tot = 0.f;
+                for (uint32_t sb = 0; sb < p.n_sb; sb++) tot += ssq[(size_t)sb * 4];
+                const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+                if (!(fabsf(inv_rms) <= 3.402823466e38f)) v0 = __int_as_float(0x7FC00000);
+                v0 *= inv_rms;
+                v1 *= inv_rms;
+            }
+            if (flags[vv]) v0 = __int_as_float(0x7FC00000);
+            const uint32_t row = unit_of(grp, t) * 16 + cc;
+            if (row >= (swiglu ? (p.n_rows >> 1) : p.n_rows)) continue;
+            const size_t o = (size_t)vv * p.ldy + row;
+            if (swiglu) v0 = (v1 / (1.0f + expf(-v1))) * v0;  // v1 = gate, v0 = up
+            else if (p.epi == OXB_GEMV_ACCUM) v0 += p.y[o];
+            else if (p.epi == OXB_GEMV_RESIDUAL) v0 += p.residual[o];
+            p.y[o] = v0;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 // One activation vector, Q1 weights: the fp4 matrix-core route.
 //
 // v_mfma_scale_f32_16x16x128_f8f6f4 with both operands in fp4 (E2M1) multiplies a whole 128-weight block of 16 rows
@@ -808,7 +1144,7 @@ static bool plan_gemv(int fmt, const OxbGemvParams& p, uint32_t n_cus, GemvPlan*
     if (swiglu && ((p.n_tiles & 1u) || (p.n_rows & 31u))) return false;  // whole gate and up tiles
     const uint32_t units = swiglu ? p.n_tiles / 2 : p.n_tiles;
     uint32_t tg_max = 1;
-    if (pl->nsbw == 1) tg_max = fmt == OXB_FMT_Q1 ? 4u : 3u;
+    if (pl->nsbw == 1) tg_max = (fmt == OXB_FMT_Q1 && !(p.xq && p.nvg == 2)) ? 4u : 3u;  // (eight vectors x four tiles: 64 KB of partial sums)
     else if (pl->nsbw == 2) tg_max = fmt == OXB_FMT_Q1 ? 2u : 1u;
     const uint32_t per = (units + n_cus - 1) / n_cus;
     static const uint32_t ring_weight[5] = {0, 130, 108, 103, 100};
@@ -848,6 +1184,24 @@ static hipError_t launch_floor_t(const OxbGemvParams& p, const GemvPlan& pl, hip
     return hipGetLastError();
 }
 
+template <int FMT, int NSBW, int TG, int NVG>
+static hipError_t launch_gemv_packed_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    const size_t shm = oxb_gemv_packed_lds_bytes(pl.S, TG, NVG);
+    if (NSBW >= 2 && p.epi != OXB_GEMV_SWIGLU && pl.tpw == (uint32_t)TG)
+        hipLaunchKernelGGL((gemv_packed_kernel<FMT, NSBW, TG, NVG, NSBW >= 2>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+    else
+        hipLaunchKernelGGL((gemv_packed_kernel<FMT, NSBW, TG, NVG, false>), dim3(pl.grid), dim3(pl.S * 64), shm, st, p);
+    return hipGetLastError();
+}
+template <int FMT, int NSBW, int TG>
+static hipError_t launch_gemv_packed1_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    return launch_gemv_packed_t<FMT, NSBW, TG, 1>(p, pl, st);
+}
+template <int FMT, int NSBW, int TG>
+static hipError_t launch_gemv_packed2_t(const OxbGemvParams& p, const GemvPlan& pl, hipStream_t st) {
+    return launch_gemv_packed_t<FMT, NSBW, TG, 2>(p, pl, st);
+}
+
 #define OXB_GEMV_CASES(LAUNCH)                                                                                        \
     OXB_CASE(OXB_FMT_Q1, 1, 1, LAUNCH) OXB_CASE(OXB_FMT_Q1, 1, 2, LAUNCH) OXB_CASE(OXB_FMT_Q1, 1, 3, LAUNCH)         \
     OXB_CASE(OXB_FMT_Q1, 1, 4, LAUNCH) OXB_CASE(OXB_FMT_Q1, 2, 1, LAUNCH) OXB_CASE(OXB_FMT_Q1, 2, 2, LAUNCH)         \
@@ -857,7 +1211,8 @@ static hipError_t launch_floor_t(const OxbGemvParams& p, const GemvPlan& pl, hip
     if (fmt == F && pl.nsbw == N && pl.tg == T) return LAUNCH<F, N, T>(p, pl, st);
 
 static bool check_gemv_args(const OxbGemvParams& p) {
-    if (p.nvec == 0 || p.nvec > OXB_GEMV_MAX_BATCH) return false;
+    if (p.nvec == 0 || p.nvec > (p.xq ? OXB_GEMV_PACKED_MAX_BATCH : OXB_GEMV_MAX_BATCH)) return false;
+    if (p.xq && (p.nvg != (p.nvec + 3) / 4 || p.xq_bytes < oxb_gemv_pack_dwords(p.n_sb, p.nvg) * 4)) return false;
     if (p.codes_bytes >= 0x7FFFFFFFull || (uint64_t)p.k * 4 >= 0x7FFFFFFFull) return false;
     if (p.pro != OXB_GEMV_PRO_F32 && p.pro != OXB_GEMV_PRO_RMSNORM) return false;
     if (p.pro == OXB_GEMV_PRO_RMSNORM && !p.norm_w) return false;
@@ -872,15 +1227,43 @@ hipError_t oxb_launch_gemv(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t
     // The fp4 kernel's registers let two workgroups share a CU; that pays where a workgroup has many tiles to
     // spread its prologue over (the LM head: 18 -> 16.8 us), and costs where it has few (the second prologue).
     const bool many = p.epi != OXB_GEMV_SWIGLU && p.n_tiles >= 32u * n_cus;
-    const bool f4 = p.nvec == 1;
+    const bool f4 = p.nvec == 1 && !p.xq;
     if (f4 && many) n_cus *= 2;
     if (!check_gemv_args(p) || !plan_gemv(fmt, p, n_cus, &pl)) return hipErrorInvalidValue;
     p.tpw = pl.tpw;
+    if (p.xq) {  // operands from the packer: one pass over the weights for up to eight vectors
+        if (p.nvg == 1) {
+            OXB_GEMV_CASES(launch_gemv_packed1_t)
+        } else {
+            OXB_GEMV_CASES(launch_gemv_packed2_t)
+        }
+        return hipErrorInvalidValue;
+    }
     if (f4) {  // one vector, either format: the fp4 route
         OXB_GEMV_CASES(launch_gemv_f4_t)
     }
     OXB_GEMV_CASES(launch_gemv_t)
     return hipErrorInvalidValue;
+}
+
+size_t oxb_gemv_pack_bytes(uint32_t k, uint32_t nvec) {
+    return oxb_gemv_pack_dwords((k / OXB_QK + 3) / 4, (nvec + 3) / 4) * 4;
+}
+
+hipError_t oxb_launch_gemv_pack(int fmt, int pro, const float* d_x, uint32_t ldx, uint32_t nvec, uint32_t k, const float* d_norm_w,
+                                uint32_t* d_out, hipStream_t st) {
+    const uint32_t n_sb = (k / OXB_QK + 3) / 4, nvg = (nvec + 3) / 4;
+    if (nvec == 0 || nvg > OXB_GEMV_PACKED_MAX_BATCH / 4 || n_sb == 0 || (pro == OXB_GEMV_PRO_RMSNORM && !d_norm_w)) return hipErrorInvalidValue;
+    const dim3 grid(n_sb, nvg * 4);
+    if (fmt == OXB_FMT_Q1 && pro == OXB_GEMV_PRO_RMSNORM)
+        hipLaunchKernelGGL((gemv_pack_kernel<OXB_FMT_Q1, OXB_GEMV_PRO_RMSNORM>), grid, dim3(64), 0, st, d_x, ldx, nvec, k, d_norm_w, n_sb, nvg, d_out);
+    else if (fmt == OXB_FMT_Q1)
+        hipLaunchKernelGGL((gemv_pack_kernel<OXB_FMT_Q1, OXB_GEMV_PRO_F32>), grid, dim3(64), 0, st, d_x, ldx, nvec, k, d_norm_w, n_sb, nvg, d_out);
+    else if (pro == OXB_GEMV_PRO_RMSNORM)
+        hipLaunchKernelGGL((gemv_pack_kernel<OXB_FMT_TQ2, OXB_GEMV_PRO_RMSNORM>), grid, dim3(64), 0, st, d_x, ldx, nvec, k, d_norm_w, n_sb, nvg, d_out);
+    else
+        hipLaunchKernelGGL((gemv_pack_kernel<OXB_FMT_TQ2, OXB_GEMV_PRO_F32>), grid, dim3(64), 0, st, d_x, ldx, nvec, k, d_norm_w, n_sb, nvg, d_out);
+    return hipGetLastError();
 }
 
 hipError_t oxb_launch_gemv_stream_floor(int fmt, OxbGemvParams p, uint32_t n_cus, hipStream_t st) {

@@ -204,9 +204,19 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
 // One GEMV over resident weights, any K: launches of at most OXB_GEMV_MAX_SB superblocks, the first with the wanted
 // epilogue, the rest accumulating.  nvec <= OXB_GEMV_MAX_BATCH vectors share each pass over the weights.
 int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, float* d_y, uint32_t ldy, int pro,
-                const float* d_norm_w, float eps, int epi, const float* d_residual) {
+                const float* d_norm_w, float eps, int epi, const float* d_residual, DevBuf* pack_ws) {
     OxbGemvParams p;
     memset(&p, 0, sizeof p);
+    if (pack_ws) {  // quantise the vectors once, in a launch of its own; the GEMV then loads its operands
+        const size_t need = oxb_gemv_pack_bytes(w.L.k, nvec);
+        int rc = pack_ws->ensure(need);
+        if (rc) return rc;
+        hipError_t e = oxb_launch_gemv_pack((int)w.L.fmt, pro, d_x, ldx, nvec, w.L.k, d_norm_w, (uint32_t*)pack_ws->ptr, g_rt.stream);
+        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv_pack");
+        p.xq = (const uint32_t*)pack_ws->ptr;
+        p.xq_bytes = (uint32_t)need;
+        p.nvg = (nvec + 3) / 4;
+    }
     p.codes = w.d_codes;
     p.scales = w.d_scales;
     p.x = d_x;
@@ -234,15 +244,31 @@ int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, 
     return OXB_HIP_OK;
 }
 
-// x (device, [batch][k]) -> y (device, [batch][ldy]), OXB_GEMV_MAX_BATCH vectors per pass over the weights.
+// Vectors from which a GEMV quantises its activations in a launch of its own (then up to eight share one pass over
+// the weights) instead of in every workgroup's prologue (four per pass).
+// 1 = by shape (the default), 0 = never, n >= 2 = from n vectors on.  By shape: five vectors and more always; two to
+// four where a wave's K slice is longer than one superblock (K above 4096), because there the prologue that every
+// workgroup repeats costs more than the extra launch (measured at K = 6144 and 12288 against 2048 and 4096).
+static uint32_t g_packed_min_batch = 1;
+uint32_t gemv_packed_min_batch(uint32_t k) {
+    if (g_packed_min_batch == 0) return 0xFFFFFFFFu;
+    if (g_packed_min_batch >= 2) return g_packed_min_batch;
+    return k > 4096 ? 2u : 5u;
+}
+
+// x (device, [batch][k]) -> y (device, [batch][ldy]): up to eight vectors per pass over the weights (four, and the
+// quantisation in the kernel itself, for what is left below gemv_packed_min_batch(k)).
 int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, uint32_t ldy, int mode,
                 const float* d_residual) {
     const uint32_t k = w.L.k;
-    for (uint32_t b0 = 0; b0 < batch; b0 += OXB_GEMV_MAX_BATCH) {
-        const uint32_t nb = (batch - b0) < OXB_GEMV_MAX_BATCH ? (batch - b0) : OXB_GEMV_MAX_BATCH;
+    for (uint32_t b0 = 0; b0 < batch;) {
+        const uint32_t left = batch - b0;
+        const bool packed = left >= gemv_packed_min_batch(k);
+        const uint32_t cap = packed ? OXB_GEMV_PACKED_MAX_BATCH : OXB_GEMV_MAX_BATCH, nb = left < cap ? left : cap;
         int rc = gemv_launch(w, d_x + (size_t)b0 * k, k, nb, d_y + (size_t)b0 * ldy, ldy, OXB_GEMV_PRO_F32, nullptr, 0.f, mode,
-                             d_residual ? d_residual + (size_t)b0 * ldy : nullptr);
+                             d_residual ? d_residual + (size_t)b0 * ldy : nullptr, packed ? &g_rt.gemv_pack : nullptr);
         if (rc) return rc;
+        b0 += nb;
     }
     return OXB_HIP_OK;
 }
@@ -368,6 +394,7 @@ void oxb_hip_shutdown(void) {
     g_rt.ws_x.release();
     g_rt.ws_y.release();
     g_rt.ws_aux.release();
+    g_rt.gemv_pack.release();
     g_rt.gemm_ws.release();
     (void)hipStreamDestroy(g_rt.own_stream);
     g_rt.static_scratch = nullptr;
@@ -558,6 +585,12 @@ static int profile_gemv_impl(bool floor_only, const uint64_t* ids, uint32_t n_id
     (void)hipEventDestroy(ev0);
     (void)hipEventDestroy(ev1);
     return rc;
+}
+
+int oxb_hip_set_gemv_packed_min_batch(uint32_t n) {
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    g_packed_min_batch = n;
+    return OXB_HIP_OK;
 }
 
 int oxb_hip_profile_gemv(const uint64_t* ids, uint32_t n_ids, const float* d_x, float* d_y, uint32_t n_rows,

@@ -146,6 +146,88 @@ def test_gemv_batched_matches_oracle(backend, fmt, n, k, batch):
         assert np.max(np.abs(got[b] - want[b])) < 1e-5 * scale + 1e-6, b
 
 
+@pytest.fixture
+def packed_from_two():
+    """Every batch above one through the route that quantises the vectors in a launch of their own (by default it
+    starts at five vectors); the default comes back afterwards."""
+    from oxibonsai_amd import _lib
+    assert _lib.lib().oxb_hip_set_gemv_packed_min_batch(2) == 0
+    yield
+    assert _lib.lib().oxb_hip_set_gemv_packed_min_batch(1) == 0
+
+
+PACKED_SHAPES = [
+    (Q1, 24576, 4096), (Q1, 4096, 12288), (Q1, 6144, 4096), (TQ2, 12288, 2048), (TQ2, 2048, 6144),   # the model shapes
+    (Q1, 1, 128), (TQ2, 17, 128), (Q1, 37, 640), (TQ2, 250, 1152), (Q1, 1000, 2560), (TQ2, 333, 9728),
+    (Q1, 5000, 8192),                      # two superblocks per wave and several tile groups per workgroup
+    (TQ2, 4100, 10240),                    # three superblocks per wave, two tiles per workgroup
+    (Q1, 48, 12800), (TQ2, 24, 17408),     # K beyond one launch: the following launches accumulate
+]
+
+
+@pytest.mark.parametrize("fmt,n,k", PACKED_SHAPES)
+def test_gemv_packed_route_matches_oracle(backend, packed_from_two, fmt, n, k):
+    """Two to eight vectors (and nineteen: 8 + 8 + 3) quantised once per GEMV and multiplied in one pass over the
+    weights; vectors of very different magnitude share a launch, one vector is all zeros, one ends in a run of
+    zeros (a whole superblock without a non-zero value)."""
+    a = synth.make_blocks(fmt, 2100 + n, n, k)
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        for batch in (2, 3, 4, 5, 7, 8, 19):
+            xs = synth.normal_f32(50 + batch, batch * k).reshape(batch, k)
+            xs[1] *= 1e-3
+            xs[batch - 1] *= 250.0
+            if batch > 2:
+                xs[2] = 0.0
+            if k >= 1024:
+                xs[0, -600:] = 0.0
+            got = backend.gemv_cached_batch(h, xs, n, k)
+            want = oracle.gemm(fmt, a, xs, batch, n, k)
+            for b in range(batch):
+                scale = max(np.max(np.abs(want[b])), 1e-30)
+                assert np.max(np.abs(got[b] - want[b])) < 1e-5 * scale + 1e-6, (batch, b)
+            if batch > 2:
+                assert not np.any(got[2])
+    finally:
+        backend.free_weights(h)
+
+
+@pytest.mark.parametrize("fmt", [Q1, TQ2])
+def test_gemv_packed_route_properties(backend, packed_from_two, fmt):
+    n, k = 777, 3072
+    a = synth.make_blocks(fmt, 31, n, k)
+    h = _upload(backend, fmt, a, n, k)
+    try:
+        x = np.stack([synth.normal_f32(10 + i, k) for i in range(8)])
+        y = backend.gemv_cached_batch(h, x, n, k)
+        truth = x.astype(np.float64) @ dense_f64(fmt, a, n, k).T
+        assert np.max(np.abs(y - truth)) < 1e-6 * np.max(np.abs(truth))
+        assert np.array_equal(backend.gemv_cached_batch(h, x, n, k), y)                       # deterministic
+        # a vector's result depends neither on its place in the batch nor on its companions
+        perm = [5, 2, 7, 0, 3, 6, 1, 4]
+        assert np.array_equal(backend.gemv_cached_batch(h, x[perm], n, k), y[perm])
+        assert np.array_equal(backend.gemv_cached_batch(h, x[:3], n, k), y[:3])
+        for s in (-100, 66):                                                                  # power-of-two scaling is exact
+            xs = x.copy()
+            xs[6] = np.ldexp(x[6], s)
+            ys = backend.gemv_cached_batch(h, xs, n, k)
+            assert np.array_equal(ys[6], np.ldexp(y[6], s).astype(np.float32)), s
+            assert np.array_equal(np.delete(ys, 6, 0), np.delete(y, 6, 0))
+        # an infinity or a NaN makes every output of its own vector NaN and leaves the other vectors alone
+        xb = x.copy()
+        xb[1, 5], xb[6, 3000] = np.nan, np.inf
+        yb = backend.gemv_cached_batch(h, xb, n, k)
+        assert np.all(np.isnan(yb[1])) and np.all(np.isnan(yb[6]))
+        assert np.array_equal(np.delete(yb, [1, 6], 0), np.delete(y, [1, 6], 0))
+        # both routes are exact up to their fp32 joins: the four-vector route must agree to the last few bits
+        from oxibonsai_amd import _lib
+        assert _lib.lib().oxb_hip_set_gemv_packed_min_batch(0) == 0
+        y4 = backend.gemv_cached_batch(h, x, n, k)
+        assert np.max(np.abs(y4 - y)) < 2e-6 * np.max(np.abs(y))
+    finally:
+        backend.free_weights(h)
+
+
 @pytest.mark.parametrize("fmt", [Q1, TQ2])
 def test_gemv_properties(backend, fmt):
     n, k = 777, 3072
