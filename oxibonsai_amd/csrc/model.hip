@@ -72,6 +72,7 @@ struct Model {
     float *pf_hidden = nullptr, *pf_qkv = nullptr, *pf_attn = nullptr, *pf_gu = nullptr;
     std::vector<void*> pf_allocs;
     GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
+    DevBuf gpack;       // quantised activation vectors of the captured GEMV-based step (batches of two to eight): likewise
     // a model loaded from a file owns the weights it uploaded
     std::vector<uint64_t> owned_mats, owned_vecs;
     DevBuf tok_hist, tok_ids;  // token history of the on-device generation loop; prompt ids of a token prefill
@@ -124,6 +125,7 @@ static void free_model(Model& m) {
     m.pf_allocs.clear();
     m.pf_cap = 0;
     m.gws.release();
+    m.gpack.release();
     free_kv_cache(m);
     m.tok_hist.release();
     m.tok_ids.release();
@@ -179,32 +181,43 @@ static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, 
         if (rc_) return rc_;     \
     } while (0)
 
+// nb activation vectors through one projection.  From gemv_packed_min_batch(K) vectors on they are quantised by a launch
+// of their own into `pack` (sized by the caller: this runs inside stream captures) and up to eight share the pass.
+static int proj(const Weight& w, const float* x, uint32_t ldx, uint32_t nb, float* y, uint32_t ldy, int pro, const float* norm_w,
+                float eps, int epi, const float* residual, DevBuf* pack) {
+    const bool packed = pack && nb >= gemv_packed_min_batch(w.L.k);
+    return gemv_launch(w, x, ldx, nb, y, ldy, pro, norm_w, eps, epi, residual, packed ? pack : nullptr);
+}
+
 // gate || up with SwiGLU behind it: one launch when K fits one GEMV launch (the epilogue needs whole row sums),
 // else the plain product into gu and a separate SwiGLU.
 static int gate_up_swiglu(const Weight& gate_up, const float* x, uint32_t ldx, uint32_t nb, const float* norm_w, float eps,
-                          float* gu, float* act, uint32_t inter) {
+                          float* gu, float* act, uint32_t inter, DevBuf* pack) {
     if (gate_up.L.n_sb <= OXB_GEMV_MAX_SB)
-        return gemv_launch(gate_up, x, ldx, nb, act, inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_SWIGLU, nullptr);
-    OXB_TRY(gemv_launch(gate_up, x, ldx, nb, gu, 2 * inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_STORE, nullptr));
+        return proj(gate_up, x, ldx, nb, act, inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_SWIGLU, nullptr, pack);
+    OXB_TRY(proj(gate_up, x, ldx, nb, gu, 2 * inter, OXB_GEMV_PRO_RMSNORM, norm_w, eps, OXB_GEMV_STORE, nullptr, pack));
     OXB_TRY_HIP(oxb_launch_swiglu(gu, inter, nb, act, inter, g_rt.stream), "kernel launch failed: swiglu");
     return OXB_HIP_OK;
 }
 
-// The FFN half of a layer on nb <= OXB_GEMV_MAX_BATCH vectors: O-proj + residual, RMSNorm -> gate || up -> SwiGLU,
-// down + residual: three launches (RMSNorm rides in the gate || up kernel's prologue, SwiGLU in its epilogue).
+// The FFN half of a layer on nb <= OXB_GEMV_PACKED_MAX_BATCH vectors: O-proj + residual, RMSNorm -> gate || up -> SwiGLU,
+// down + residual: three launches (RMSNorm rides in the gate || up kernel's prologue, SwiGLU in its epilogue), plus
+// one pack launch in front of each where the vectors are quantised ahead.
 static int encode_ffn(float* hidden, const float* attn_out, const float* ffn_norm, float eps, const Weight& o,
                       const Weight& gate_up, const Weight& down, float* gu, float* act, uint32_t h, uint32_t inter,
-                      uint32_t attn_k, uint32_t nb) {
-    OXB_TRY(gemv_launch(o, attn_out, attn_k, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden));
-    OXB_TRY(gate_up_swiglu(gate_up, hidden, h, nb, ffn_norm, eps, gu, act, inter));
-    OXB_TRY(gemv_launch(down, act, inter, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden));
+                      uint32_t attn_k, uint32_t nb, DevBuf* pack) {
+    OXB_TRY(proj(o, attn_out, attn_k, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden, pack));
+    OXB_TRY(gate_up_swiglu(gate_up, hidden, h, nb, ffn_norm, eps, gu, act, inter, pack));
+    OXB_TRY(proj(down, act, inter, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden, pack));
     return OXB_HIP_OK;
 }
 
 // Decode batches from this size on run their projections through the prefill GEMM (fp16 activations on the
 // matrix cores, one pass over the weights for the whole batch) instead of the fp32-exact GEMV, which streams
-// the weights once per four sequences.
-#define OXB_DECODE_GEMM_MIN_BATCH (OXB_GEMV_MAX_BATCH + 1)
+// the weights once per eight sequences.
+#define OXB_DECODE_GEMM_MIN_BATCH (OXB_GEMV_PACKED_MAX_BATCH + 1)
+// Sequences per pass of the GEMV-based step: all of them up to eight.
+static uint32_t decode_chunk(uint32_t batch) { return batch <= OXB_GEMV_PACKED_MAX_BATCH ? batch : OXB_GEMV_PACKED_MAX_BATCH; }
 
 // Looks every handle of the model up with the shape the model needs (which also binds a weight that was uploaded
 // without one).  Run at creation and again whenever a weight or vector was replaced or freed since, before a decode
@@ -234,6 +247,12 @@ static int check_model_handles(Model& m) {
 // capture, for every projection shape of the model (the LM head included when there is one).
 static int size_gemm_workspaces(Model& m) {
     const oxb_model_desc& d = m.d;
+    if (d.batch >= 2) {  // the pack buffer of the GEMV-based step (also what a larger batch's decode_hidden runs)
+        uint32_t kmax = d.h > d.inter ? d.h : d.inter;
+        if (d.nq * d.hd > kmax) kmax = d.nq * d.hd;
+        int rc = m.gpack.ensure(oxb_gemv_pack_bytes(kmax, decode_chunk(d.batch)));
+        if (rc) return rc;
+    }
     if (d.batch < OXB_DECODE_GEMM_MIN_BATCH) return OXB_HIP_OK;
     const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
     uint32_t kx = d.h > d.inter ? d.h : d.inter;
@@ -389,6 +408,8 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
     const oxb_model_desc& d = m.d;
     hipStream_t st = g_rt.stream;
     const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
+    const uint32_t chunk = decode_chunk(d.batch);
+    DevBuf* pack = m.gpack.ptr ? &m.gpack : nullptr;
     int rc = OXB_HIP_OK;
     for (uint32_t L = 0; L < d.n_layers; L++) {
         const oxb_layer_ids& ly = m.layers[L];
@@ -401,27 +422,27 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
         const Weight* wgu = mat_ptr(ly.gate_up, d.fmt, 2 * d.inter, d.h, "gate_up", &rc);
         const Weight* wdn = mat_ptr(ly.down, d.fmt, d.h, d.inter, "down", &rc);
         if (rc) return rc;
-        // attention input: RMSNorm -> QKV in one launch per pass of OXB_GEMV_MAX_BATCH sequences
-        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
-            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY(gemv_launch(*wqkv, m.hidden + (size_t)b0 * d.h, d.h, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows,
-                                OXB_GEMV_PRO_RMSNORM, attn_norm, d.eps, OXB_GEMV_STORE, nullptr));
+        // attention input: RMSNorm -> QKV in one launch per pass of `chunk` sequences
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += chunk) {
+            const uint32_t nb = (d.batch - b0) < chunk ? (d.batch - b0) : chunk;
+            OXB_TRY(proj(*wqkv, m.hidden + (size_t)b0 * d.h, d.h, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows,
+                         OXB_GEMV_PRO_RMSNORM, attn_norm, d.eps, OXB_GEMV_STORE, nullptr, pack));
         }
         OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm));
-        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
-            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += chunk) {
+            const uint32_t nb = (d.batch - b0) < chunk ? (d.batch - b0) : chunk;
             OXB_TRY(encode_ffn(m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo, *wgu, *wdn,
-                               m.gu + (size_t)b0 * 2 * d.inter, m.act + (size_t)b0 * d.inter, d.h, d.inter, qd, nb));
+                               m.gu + (size_t)b0 * 2 * d.inter, m.act + (size_t)b0 * d.inter, d.h, d.inter, qd, nb, pack));
         }
     }
     if (with_lm_head) {
         const float* final_norm = vec_ptr(d.final_norm, d.h, "final_norm", &rc);
         const Weight* lm = mat_ptr(d.lm_head, d.fmt, d.vocab, d.h, "lm_head", &rc);
         if (rc) return rc;
-        for (uint32_t b0 = 0; b0 < d.batch; b0 += OXB_GEMV_MAX_BATCH) {
-            const uint32_t nb = (d.batch - b0) < OXB_GEMV_MAX_BATCH ? (d.batch - b0) : OXB_GEMV_MAX_BATCH;
-            OXB_TRY(gemv_launch(*lm, m.hidden + (size_t)b0 * d.h, d.h, nb, m.logits + (size_t)b0 * d.vocab, d.vocab,
-                                OXB_GEMV_PRO_RMSNORM, final_norm, d.eps, OXB_GEMV_STORE, nullptr));
+        for (uint32_t b0 = 0; b0 < d.batch; b0 += chunk) {
+            const uint32_t nb = (d.batch - b0) < chunk ? (d.batch - b0) : chunk;
+            OXB_TRY(proj(*lm, m.hidden + (size_t)b0 * d.h, d.h, nb, m.logits + (size_t)b0 * d.vocab, d.vocab,
+                         OXB_GEMV_PRO_RMSNORM, final_norm, d.eps, OXB_GEMV_STORE, nullptr, pack));
         }
         OXB_TRY_HIP(oxb_launch_argmax(m.logits, d.vocab, d.batch, m.tokens, m.argmax_ws, st, m.h_tokens), "kernel launch failed: argmax");
     }
@@ -1199,7 +1220,7 @@ int oxb_hip_ffn_phase(int fmt, float* hidden, const float* attn_out, const float
     OXB_TRY_HIP(hipMemcpyAsync(d_hidden, hidden, (size_t)h * 4, hipMemcpyHostToDevice, st), "hidden upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_norm, norm_w, (size_t)h * 4, hipMemcpyHostToDevice, st), "norm upload");
     OXB_TRY_HIP(hipMemcpyAsync(d_attn, attn_out, (size_t)attn_k * 4, hipMemcpyHostToDevice, st), "attn_out upload");
-    OXB_TRY(encode_ffn(d_hidden, d_attn, d_norm, eps, *wo, *wgu, *wdn, d_gu, d_act, h, inter, attn_k, 1));
+    OXB_TRY(encode_ffn(d_hidden, d_attn, d_norm, eps, *wo, *wgu, *wdn, d_gu, d_act, h, inter, attn_k, 1, nullptr));
     OXB_TRY_HIP(hipMemcpyAsync(hidden, d_hidden, (size_t)h * 4, hipMemcpyDeviceToHost, st), "hidden download");
     hipError_t e = hipStreamSynchronize(st);
     if (e != hipSuccess) return fail(OXB_HIP_SYNC_FAILED, "device synchronization failed: ffn_phase: %s", hipGetErrorString(e));
