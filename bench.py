@@ -29,14 +29,34 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
-# HBM bytes one gate||up GEMV launch moves: rocprofv3 FETCH_SIZE (x 2.000, calibrated on a 256 MiB copy) + WRITE_SIZE
-# (x 1.000) of the kernel named beside it, from the profile named beside it.  The algorithmic figure is 14 270 464.
-GATE_UP_HBM_TRAFFIC_BYTES = 14_486_528
+# HBM bytes one gate||up GEMV launch moves come from the committed counter profile named here: rocprofv3 FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch) of the kernel row named beside it, each times the factor the same file derives from a
+# 256 MiB copy.  The algorithmic figure is 14 270 464.
 GATE_UP_HBM_TRAFFIC_SOURCE = "profiles/gemv_q1_qwen3_8b_set_hbm_traffic.txt"
+GATE_UP_KERNEL_ROW = "gemv_f4_kernel<0, 1, 3, 0>"
 GATE_UP_KERNEL = "gemv_f4_kernel<0, 1, 3, 0> (Q1 weights, one activation vector, one superblock of K per wave, three row tiles in flight, fp32 input) gate||up 24576x4096"
 SHAPES = [("qkv", 6144, 4096), ("gate_up", 24576, 4096), ("down", 4096, 12288)]
 FMT_Q1 = 0
 FMT_TQ2 = 1
+
+
+def traffic_from_profile(path: str, kernel_row: str):
+    """HBM bytes per launch of `kernel_row` from a counter summary under profiles/: the per-dispatch averages of its
+    FETCH_SIZE and WRITE_SIZE rows (KiB), each scaled by the 'factor' the summary states for that counter.  None when
+    the file or a row is missing (the figure is then left out rather than guessed)."""
+    import re
+    try:
+        text = open(os.path.join(ROOT, path)).read()
+    except OSError:
+        return None
+    total = 0.0
+    for counter in ("FETCH_SIZE", "WRITE_SIZE"):
+        row = re.search(r"^.*%s\(OxbGemvParams\)\s+%s\s+\d+\s+\d+\s+([0-9.]+)" % (re.escape(kernel_row), counter), text, flags=re.M)
+        fac = re.search(r"^\s*%s reads .*factor ([0-9.]+)" % counter, text, flags=re.M)
+        if not row or not fac:
+            return None
+        total += float(row.group(1)) * float(fac.group(1)) * 1024.0
+    return int(round(total))
 
 
 def algorithmic_bytes(n_rows: int, k: int, batch: int = 1, block_bytes: int = 18) -> int:
@@ -135,6 +155,14 @@ def decode_leg(be, prompt_len: int, n_tokens: int, with_cpu: bool, batches=(8, 3
            "kv_bytes_per_token_at_end": 2 * cfg["n_layers"] * cfg["nkv"] * cfg["hd"] * 2 * (prompt_len + n_tokens),
            "weight_stream_GBps": round(weight_bytes / (spent / n_tokens) / 1e9, 1),
            "distinct_tokens": len(set(tokens))}
+    # HBM bound of a token: every weight block once, plus the K and V rows of the context (fp16) at the mean position
+    # of the timed tokens; norms, activations and the embedding row are below 1 MB and left out
+    kv_mean = 2 * cfg["n_layers"] * cfg["nkv"] * cfg["hd"] * 2 * (prompt_len + (n_tokens + 1) // 2)
+    bound_us = (weight_bytes + kv_mean) / (HBM_PEAK_GBPS * 1e9) * 1e6
+    res["roofline"] = {"bound": "hbm", "bytes_per_token": weight_bytes + kv_mean, "weight_bytes": weight_bytes,
+                       "kv_bytes_at_mean_context": kv_mean, "bound_us": round(bound_us, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                       "achieved": round((weight_bytes + kv_mean) / (spent / n_tokens) / 1e9, 1),
+                       "frac": round(bound_us / (spent / n_tokens * 1e6), 4)}
     # the same loop without a host round trip per token: embedding lookup (a Q1_0_g128 table here), forward and
     # argmax stay on the device, the host gets all ids at the end (oxb_hip_decode_tokens)
     from oxibonsai_amd.model import Embedding
@@ -553,8 +581,31 @@ def main() -> int:
         ms8 = e0.elapsed_time(e1) / (8 * args.copies)
     set_bytes8 = sum(algorithmic_bytes(r, k, B8) for _, r, k in SHAPES)
     batch8 = {"batch": B8, "ms_per_step": round(ms8, 6), "algorithmic_bytes_per_step": set_bytes8,
-              "GB/s": round(set_bytes8 / (ms8 * 1e-3) / 1e9, 1), "weight_passes_per_gemv": 2,
-              "note": "exact GEMV route, four vectors share a pass over the weights; weights counted once"}
+              "GB/s": round(set_bytes8 / (ms8 * 1e-3) / 1e9, 1), "frac_of_hbm_peak": round(set_bytes8 / (ms8 * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+              "weight_passes_per_gemv": 1, "launches_per_gemv": 2,
+              "note": "exact GEMV route: a pack launch quantises the eight vectors once, the GEMV loads its int8 MFMA operands "
+                      "and streams the weights once for all eight"}
+    if not args.no_batch8:
+        # the same step with every workgroup quantising the vectors in its prologue, four vectors per pass over the weights
+        L.oxb_hip_set_gemv_packed_min_batch(0)
+        for i in range(3):
+            step8(i)
+        torch.cuda.synchronize()
+        g8k = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g8k, stream=stream):
+            for i in range(args.copies):
+                step8(i)
+        L.oxb_hip_set_gemv_packed_min_batch(1)
+        assert L.oxb_hip_set_stream(C.c_void_p(stream.cuda_stream)) == 0
+        g8k.replay()
+        e0.record(stream)
+        for _ in range(8):
+            g8k.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+        ms8k = e0.elapsed_time(e1) / (8 * args.copies)
+        batch8["quantised_in_every_workgroup_route"] = {"ms_per_step": round(ms8k, 6), "GB/s": round(set_bytes8 / (ms8k * 1e-3) / 1e9, 1),
+                                                        "note": "two passes of four vectors, no pack launch (the route batches of two to four take at K <= 4096)"}
     if not args.no_batch8:
         # the same eight vectors through the route the decode pipeline takes from five sequences on: activations packed
         # to fp16, one pass over the weights on the fp16 matrix cores (prefill tolerance instead of fp32-exact products)
@@ -640,6 +691,20 @@ def main() -> int:
                                     "bytes_per_launch": c0_bytes}
     for h in c0_ids:
         be.free_weights(h)
+    # the ternary LM head 151936 x 2048 (configs[3]'s last GEMV; 3 rotating copies, 242 MB)
+    tl_rows, tl_k = 151936, 2048
+    tl_blocks = synth.make_tq2_blocks(0xB0A5A103F0, tl_rows * (tl_k // 128))
+    tl_ids = [be.upload_weights_ternary(tl_blocks, tl_rows, tl_k) for _ in range(3)]
+    arr = (C.c_uint64 * 3)(*[int(h) for h in tl_ids])
+    L.oxb_hip_profile_gemv(arr, 3, c0_x.data_ptr(), lm_y.data_ptr(), tl_rows, tl_k, 6, 60, C.byref(us))
+    tl_bytes = algorithmic_bytes(tl_rows, tl_k, 1, 34)
+    per_kernel["tq2_lm_head_151936x2048"] = {"us": round(us.value, 3), "GB/s": round(tl_bytes / (us.value * 1e-6) / 1e9, 1),
+                                             "bytes_per_launch": tl_bytes}
+    for h in tl_ids:
+        be.free_weights(h)
+    for v in per_kernel.values():
+        v["frac"] = round(v["GB/s"] / HBM_PEAK_GBPS, 4)
+    slowest = max((nm for nm, _, _ in SHAPES), key=lambda nm: per_kernel[nm]["us"])
 
     launch_context = measure_launch_context(torch, stream, kbytes, args.copies)
     launch_context["streaming_read_floor"] = floors
@@ -659,9 +724,10 @@ def main() -> int:
                    "steps_per_replayed_graph": per_graph * args.steps,
                    "batch8": batch8},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_HBM_TRAFFIC_BYTES,
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic_from_profile(GATE_UP_HBM_TRAFFIC_SOURCE, GATE_UP_KERNEL_ROW),
                      "traffic_source": GATE_UP_HBM_TRAFFIC_SOURCE, "kernel": GATE_UP_KERNEL, "bytes_per_launch": kbytes,
                      "avg_launch_us": round(avg_us.value, 3), "launch_context": launch_context, "per_kernel": per_kernel,
+                     "slowest_kernel_of_the_step": {"name": slowest, **per_kernel[slowest]},
                      "per_kernel_cache_resident": cache_resident},
     }
     if not args.no_cpu:

@@ -36,7 +36,11 @@
 //!
 //! Every function here has the name, argument list and return type of its `cuda` counterpart, so the model crate's
 //! call sites (`crates/oxibonsai-model/src/model/types/forward_cuda/q1.rs`, `ternary.rs`) switch tiers by a `cfg`
-//! on the function name alone.
+//! on the function name alone.  The one type that differs is the error of the prefill entry points
+//! (`try_cuda_prefill` returns `Result<(), CudaGraphError>`, `cuda_prefill/try_apis.rs:318-342`): the model crate only
+//! formats it (`forward_cuda/q1.rs` logs `{e}` and falls back), and for code that does name the type this module
+//! converts (`From<HipGraphError> for CudaGraphError`, when both tiers are compiled in) or, in a build without the
+//! CUDA tier, offers the HIP error under the CUDA name (`pub use native_hip::CudaGraphError`).
 
 pub mod backend;
 pub mod ffi;
@@ -66,6 +70,26 @@ pub enum HipGraphError {
     /// A mutex was poisoned.
     LockPoisoned,
 }
+
+/// Both tiers compiled in: a `?` in code written against the CUDA tier's error type takes a HIP error as it is.
+/// Every variant has its namesake in `CudaGraphError` (`gpu_backend/cuda_graph/types.rs:25-39`).
+#[cfg(all(feature = "native-cuda", any(target_os = "linux", target_os = "windows")))]
+impl From<HipGraphError> for super::cuda_graph::CudaGraphError {
+    fn from(e: HipGraphError) -> Self {
+        use super::cuda_graph::CudaGraphError as C;
+        match e {
+            HipGraphError::DeviceNotFound(s) => C::DeviceNotFound(s),
+            HipGraphError::DriverError(s) => C::DriverError(s),
+            HipGraphError::WeightNotFound(id) => C::WeightNotFound(id),
+            HipGraphError::WeightLayoutError(s) => C::WeightLayoutError(s),
+            HipGraphError::LockPoisoned => C::LockPoisoned,
+        }
+    }
+}
+
+/// Without the CUDA tier the name `CudaGraphError` is free: call sites that spell it keep compiling.
+#[cfg(not(all(feature = "native-cuda", any(target_os = "linux", target_os = "windows"))))]
+pub type CudaGraphError = HipGraphError;
 
 impl std::fmt::Display for HipGraphError {
     fn fmt(&self, f: &mut std::fmt::Formatter<'_>) -> std::fmt::Result {

@@ -283,6 +283,23 @@ def test_rust_overlay_mirrors_the_reference_signatures():
     assert params("try_hip_qkv") == ["input", "output", "weight_handle_id", "q_bytes", "k_bytes", "v_bytes", "n_rows", "k"]
 
 
+def test_rust_overlay_error_type_fits_the_cuda_call_sites():
+    """try_hip_prefill returns HipGraphError where try_cuda_prefill returns CudaGraphError
+    (gpu_backend/cuda_prefill/try_apis.rs:318-342): every HIP variant must have its namesake in the reference's enum
+    (gpu_backend/cuda_graph/types.rs:25-39, restated here), a conversion must exist for builds with both tiers and
+    an alias for builds without the CUDA tier."""
+    src = open(os.path.join(ROOT, "rust", "native_hip", "mod.rs")).read()
+    body = re.search(r"pub enum HipGraphError \{(.*?)\n\}", src, flags=re.S).group(1)
+    variants = set(re.findall(r"^\s{4}([A-Z][A-Za-z]+)", body, flags=re.M))
+    cuda = {"DeviceNotFound", "CompilationFailed", "DriverError", "WeightNotFound", "WeightLayoutError", "LockPoisoned"}
+    assert variants and variants <= cuda
+    conv = re.search(r"impl From<HipGraphError> for super::cuda_graph::CudaGraphError \{(.*?)\n\}", src, flags=re.S).group(1)
+    for v in variants:
+        assert f"HipGraphError::{v}" in conv and f"C::{v}" in conv, v
+    assert "pub type CudaGraphError = HipGraphError;" in src
+    assert src.count("impl std::error::Error for HipGraphError") == 1
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU: --gpus above 1 ends with a message and a non-zero status before anything is loaded."""
     import subprocess
