@@ -626,6 +626,10 @@ static uint32_t attn_slots(const Model& m, uint32_t kv_mode) {
     const uint32_t per_cu = kv_mode == OXB_KV_F16 ? 1u : 2u;
     const uint32_t want = (per_cu * g_rt.n_cus + d.nkv * d.batch - 1) / (d.nkv * d.batch);
     if (n > want) n = want;
+    if (const char* e = getenv("OXB_HIP_ATTN_SLOTS")) {  // measurement aid: a fixed slot count
+        const long v = strtol(e, nullptr, 10);
+        if (v > 0) n = (uint32_t)v < n ? (uint32_t)v : n;
+    }
     if (n > OXB_ATTN_MAX_SPLITS) n = OXB_ATTN_MAX_SPLITS;
     return n;
 }
