@@ -486,9 +486,9 @@ __global__ __launch_bounds__(64) void gemv_pack_kernel(const float* __restrict__
     }
 }
 
-// Dynamic LDS of a launch: part [4][NVG][TG][S][64] floats | flags [8]
+// Dynamic LDS of a launch: part [4][NVG][TG][S][64] floats | flags [8] | inv_rms [8]
 __host__ __device__ inline size_t oxb_gemv_packed_lds_bytes(uint32_t S, uint32_t tg, uint32_t nvg) {
-    return ((size_t)4 * nvg * tg * S * 64 + 8) * 4;
+    return ((size_t)4 * nvg * tg * S * 64 + 8 + 8) * 4;
 }
 
 // One 128-weight block of a waiting tile -> the two int8 B operands.  The code dword passes through an empty asm
@@ -543,6 +543,7 @@ __global__ __launch_bounds__(512) void gemv_packed_kernel(const OxbGemvParams p)
     const bool swiglu = p.epi == OXB_GEMV_SWIGLU;
     float* part = (float*)smem;
     int* flags = (int*)(part + (size_t)4 * NVG * TG * S * 64);
+    float* inv_rms_v = (float*)(flags + 8);  // 1 / rms of each vector (RMSNorm prologue)
 
     const uint32_t lane_c = lane * 16u, lane_s = c * 8u;
     const uint32_t sb0 = __builtin_amdgcn_readfirstlane(p.sb_begin + s * NSBW);
@@ -585,6 +586,21 @@ __global__ __launch_bounds__(512) void gemv_packed_kernel(const OxbGemvParams p)
 #pragma unroll
     for (int n = 0; n < NOPS; n++) load_ops(ops[n], n / NSBW, n % NSBW, true);
     if (threadIdx.x < 8) flags[threadIdx.x] = 0;  // cleared for every wave once the barrier is passed
+    // RMSNorm: the superblocks' sums of squares in order -> 1 / rms per vector, once per workgroup (the merge below
+    // applies it to the row sums; it is first read behind the barrier that ends the first tile group)
+    // (thread 4 g + v adds for vector v of group g; eight superblocks per round of requests, the first round issued
+    // here with the operands, so that it is back long before the first weight tile)
+    const bool norm_thread = p.pro == OXB_GEMV_PRO_RMSNORM && threadIdx.x < NVG * 4;
+    const __amdgpu_buffer_rsrc_t r_ss = make_rsrc((const float*)p.xq + (size_t)NVG * p.n_sb * (2048 + 64 + 4), NVG * p.n_sb * 16u);
+    auto ss_round = [&](uint32_t sb_first, float (&v)[8]) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) {
+            const uint32_t sb = sb_first + i;
+            v[i] = __uint_as_float(buf_load_b32(r_ss, norm_thread && sb < p.n_sb ? (((threadIdx.x >> 2) * p.n_sb + sb) * 4 + (threadIdx.x & 3u)) * 4u : OXB_OOB));
+        }
+    };
+    float ss_first[8];
+    ss_round(0, ss_first);
     // every wave's operand requests enter the CU's memory pipeline before any wave's weight requests
     __builtin_amdgcn_sched_barrier(0);
     lds_barrier();
@@ -594,6 +610,18 @@ __global__ __launch_bounds__(512) void gemv_packed_kernel(const OxbGemvParams p)
     for (int t = 0; t < TG; t++) {
         load_tile<FMT, NSBW>(ring[t], r_codes, r_scales, tile_of(0, t), slot_ok(0, t), p.n_sb, sb0, sb_lim, lane_c, lane_s);
         __builtin_amdgcn_sched_barrier(0);
+    }
+    if (p.pro == OXB_GEMV_PRO_RMSNORM && s == 0) {  // wave-uniform: only the first wave has such threads
+        float tot = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; i++) tot += ss_first[i];  // entries past the last superblock read as +0
+        for (uint32_t sb = 8; sb < p.n_sb; sb += 8) {
+            float more[8];
+            ss_round(sb, more);
+#pragma unroll
+            for (int i = 0; i < 8; i++) tot += more[i];
+        }
+        if (norm_thread) inv_rms_v[threadIdx.x] = 1.0f / sqrtf(tot / (float)p.k + p.eps);
     }
     // a slice with an infinity or a NaN in it: every output of that vector becomes NaN
     auto take_ex = [&](Ops& o, int vgi) -> int {
@@ -688,11 +716,8 @@ __global__ __launch_bounds__(512) void gemv_packed_kernel(const OxbGemvParams p)
             for (uint32_t w = 0; w < S; w++) v0 += buf[o0 + (size_t)w * 64];
             if (swiglu)
                 for (uint32_t w = 0; w < S; w++) v1 += gbuf[o0 + (size_t)w * 64];
-            if (p.pro == OXB_GEMV_PRO_RMSNORM) {  // the superblocks' sums of squares in order, then 1 / rms on the row sums
-                const float* ssq = (const float*)p.xq + (size_t)q_units * (2048 + 64 + 4) + (size_t)vgt * p.n_sb * 4 + (ln >> 4);
-                float tot = 0.f;
-                for (uint32_t sb = 0; sb < p.n_sb; sb++) tot += ssq[(size_t)sb * 4];
-                const float inv_rms = 1.0f / sqrtf(tot / (float)p.k + p.eps);
+            if (p.pro == OXB_GEMV_PRO_RMSNORM) {  // 1 / rms on the row sums
+                const float inv_rms = inv_rms_v[vv];
                 if (!(fabsf(inv_rms) <= 3.402823466e38f)) v0 = __int_as_float(0x7FC00000);
                 v0 *= inv_rms;
                 v1 *= inv_rms;

@@ -377,6 +377,14 @@ int oxb_hip_init(int device_ordinal) {
     g_rt.device = device_ordinal;
     g_rt.n_cus = (uint32_t)prop.multiProcessorCount;
     snprintf(g_rt.name, sizeof g_rt.name, "%s (%s)", prop.name, prop.gcnArchName);
+    // The pack buffer of the batched GEMV exists from the start (eight vectors of K = 32768 fit: 1.1 MB), so that a
+    // caller who captures oxb_hip_gemv_dev into a graph of its own needs no warm-up call for it to grow.
+    const int rc_pack = g_rt.gemv_pack.ensure(oxb_gemv_pack_bytes(32768, OXB_GEMV_PACKED_MAX_BATCH));
+    if (rc_pack) {
+        (void)hipStreamDestroy(g_rt.own_stream);
+        g_rt.own_stream = g_rt.stream = nullptr;
+        return rc_pack;
+    }
     g_rt.ready = true;
     return OXB_HIP_OK;
     OXB_API_END

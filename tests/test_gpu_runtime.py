@@ -168,3 +168,57 @@ def test_graph_replay_on_a_stream_the_caller_set(backend):
     finally:
         assert L.oxb_hip_set_stream(None) == 0
         assert hip.hipStreamDestroy(stream) == 0
+
+
+def test_batched_gemv_captured_cold_into_a_callers_graph(backend):
+    """oxb_hip_gemv_dev with eight vectors, captured into the caller's own HIP graph as the first call of its shape
+    (no warm-up that could grow a workspace: the pack buffer of the batched route exists from oxb_hip_init on), then
+    replayed three times with the inputs changed in between; every replay is held to the eager result."""
+    import ctypes as C
+
+    from helpers import DeviceBuffer
+    from oxibonsai_amd import _lib
+    L, hip = _lib.lib(), DeviceBuffer.hip()
+    for f, args in (("hipStreamCreate", [C.POINTER(C.c_void_p)]), ("hipStreamDestroy", [C.c_void_p]),
+                    ("hipStreamBeginCapture", [C.c_void_p, C.c_int]), ("hipStreamEndCapture", [C.c_void_p, C.POINTER(C.c_void_p)]),
+                    ("hipGraphInstantiate", [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t]),
+                    ("hipGraphLaunch", [C.c_void_p, C.c_void_p]), ("hipStreamSynchronize", [C.c_void_p]),
+                    ("hipGraphExecDestroy", [C.c_void_p]), ("hipGraphDestroy", [C.c_void_p])):
+        getattr(hip, f).argtypes = args
+    n, k, B = 1040, 7168, 8                      # a K no other test uses: nothing of this shape has run before
+    a = synth.make_blocks(TQ2, 611, n, k)
+    h = backend.upload_weights_ternary(a, n, k)
+    xs = [synth.normal_f32(620 + i, B * k).reshape(B, k) for i in range(3)]
+    d_x, d_y = DeviceBuffer.from_numpy(xs[0]), DeviceBuffer(B * n * 4)
+    stream, graph, gexec = C.c_void_p(0), C.c_void_p(0), C.c_void_p(0)
+    assert hip.hipStreamCreate(C.byref(stream)) == 0
+    try:
+        assert L.oxb_hip_set_stream(stream) == 0
+        assert hip.hipStreamBeginCapture(stream, 0) == 0                       # hipStreamCaptureModeGlobal
+        rc = L.oxb_hip_gemv_dev(int(h), d_x.ptr, d_y.ptr, n, k, B)
+        err = _lib.last_error() if rc else ""
+        assert hip.hipStreamEndCapture(stream, C.byref(graph)) == 0
+        assert rc == 0, err
+        assert hip.hipGraphInstantiate(C.byref(gexec), graph, None, None, 0) == 0
+        for x in xs:
+            assert hip.hipMemcpy(d_x.ptr, np.ascontiguousarray(x).ctypes.data, x.nbytes, 1) == 0
+            d_y.fill(0xFF)
+            assert hip.hipGraphLaunch(gexec, stream) == 0
+            assert hip.hipStreamSynchronize(stream) == 0
+            got = d_y.to_numpy(np.float32, (B, n))
+            assert L.oxb_hip_set_stream(None) == 0
+            want = backend.gemv_cached_batch(h, x, n, k)                         # eager, on the library's own stream
+            assert L.oxb_hip_set_stream(stream) == 0
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            ref = oracle.gemm(TQ2, a, x, B, n, k)
+            assert np.max(np.abs(got - ref)) < 1e-5 * np.max(np.abs(ref))
+    finally:
+        L.oxb_hip_set_stream(None)
+        if gexec:
+            hip.hipGraphExecDestroy(gexec)
+        if graph:
+            hip.hipGraphDestroy(graph)
+        hip.hipStreamDestroy(stream)
+        d_x.free()
+        d_y.free()
+        backend.free_weights(h)
