@@ -229,6 +229,9 @@ int  oxb_hip_model_kv_capacity(uint64_t model, uint32_t seq, uint32_t* n_tokens)
 /* quantize_row_i8 / quantize_row_fp8 on the device for n_rows rows of n values each (host buffers): the same
  * routine the attention kernels store new rows with. */
 int  oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, uint32_t n, uint8_t* codes, float* scales);
+/* The way back, code * scale (dequantize_row, crates/oxibonsai-model/src/kv_cache_quant.rs:69-71, 545-556; fp8_e4m3_decode,
+ * crates/oxibonsai-core/src/quant_fp8.rs), with the widening of the codes that the attention kernels use; n % 4 == 0. */
+int  oxb_hip_kv_dequantize_rows(int kv_dtype, const uint8_t* codes, const float* scales, uint32_t n_rows, uint32_t n, float* rows);
 
 /* ---- the steps either side of the fused forward: checkpoint file -> device, token ids in, token ids out.
  * oxb_hip_gguf_info (no GPU needed) and oxb_hip_load_gguf read a GGUF file the way GgufFile::parse does

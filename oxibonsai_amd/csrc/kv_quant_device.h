@@ -88,13 +88,10 @@ __device__ __forceinline__ void kv_dec4(uint32_t w, uint32_t& lo, uint32_t& hi) 
         lo = __builtin_bit_cast(uint32_t, a);
         hi = __builtin_bit_cast(uint32_t, b);
     } else {
-        // byte s eeee mmm -> fp16 bits s 0eeee mmm0000000 = value * 2^-8 (subnormal codes become fp16 subnormals);
-        // the multiplication by 256 is exact and leaves normal numbers only
-        const kvh2_t k = {(_Float16)256.0f, (_Float16)256.0f};
-        const uint32_t a = __builtin_amdgcn_perm(0u, w, 0x010c000cu), b = __builtin_amdgcn_perm(0u, w, 0x030c020cu);
-        const uint32_t ta = ((a >> 1) & 0x3F803F80u) | (a & 0x80008000u), tb = ((b >> 1) & 0x3F803F80u) | (b & 0x80008000u);
-        lo = __builtin_bit_cast(uint32_t, __builtin_bit_cast(kvh2_t, ta) * k);
-        hi = __builtin_bit_cast(uint32_t, __builtin_bit_cast(kvh2_t, tb) * k);
+        // the conversion instruction of gfx950 (OCP E4M3: the format of fp8_e4m3_encode) widens two codes at a time,
+        // exactly: every E4M3 value, subnormal codes included, is an fp16 number
+        lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, false));  // bytes 0, 1
+        hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(w, 1.0f, true));   // bytes 2, 3
     }
 }
 

@@ -44,6 +44,8 @@ struct OxbAttnParams {
 };
 
 // n_rows rows of n values -> one-byte codes [n_rows][n] and a scale per row (kv_mode: OXB_KV_I8 or OXB_KV_FP8_E4M3).
+hipError_t oxb_launch_kv_dequantize_rows(int kv_mode, const uint8_t* d_codes, const float* d_scales, uint32_t n_rows, uint32_t n,
+                                         float* d_out, hipStream_t st);
 hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n_rows, uint32_t n, uint8_t* d_codes, float* d_scales,
                                        hipStream_t st);
 hipError_t oxb_launch_qk_norm_rope_store(const OxbQkParams& p, uint32_t batch, hipStream_t st);

@@ -150,6 +150,36 @@ __global__ __launch_bounds__(64) void kv_quantize_rows_kernel(const float* __res
     if (threadIdx.x == 0) scales[blockIdx.x] = scale;
 }
 
+// Quantised rows back to f32 as attention reads them, code * scale (dequantize_row, kv_cache_quant.rs:69-71, 545-556):
+// the codes are widened four at a time by the routine the attention kernels use (kv_dec4), which is what this is for.
+template <int KVM>
+__global__ __launch_bounds__(256) void kv_dequantize_rows_kernel(const uint32_t* __restrict__ codes4, const float* __restrict__ scales,
+                                                                 uint32_t n, uint64_t total4, float* __restrict__ out) {
+    const uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;  // one dword of four codes; n % 4 == 0
+    if (i >= total4) return;
+    uint32_t lo, hi;
+    kv_dec4<KVM>(codes4[i], lo, hi);
+    const kvh2_t a = __builtin_bit_cast(kvh2_t, lo), b = __builtin_bit_cast(kvh2_t, hi);
+    const float sc = scales[(i * 4) / n];
+    out[i * 4 + 0] = (float)a[0] * sc;
+    out[i * 4 + 1] = (float)a[1] * sc;
+    out[i * 4 + 2] = (float)b[0] * sc;
+    out[i * 4 + 3] = (float)b[1] * sc;
+}
+
+hipError_t oxb_launch_kv_dequantize_rows(int kv_mode, const uint8_t* d_codes, const float* d_scales, uint32_t n_rows, uint32_t n,
+                                         float* d_out, hipStream_t st) {
+    if (n_rows == 0 || n == 0 || (n & 3u)) return hipErrorInvalidValue;
+    const uint64_t total4 = (uint64_t)n_rows * n / 4;
+    const dim3 grid((uint32_t)((total4 + 255) / 256));
+    if (kv_mode == OXB_KV_I8)
+        hipLaunchKernelGGL(kv_dequantize_rows_kernel<OXB_KV_I8>, grid, dim3(256), 0, st, (const uint32_t*)d_codes, d_scales, n, total4, d_out);
+    else if (kv_mode == OXB_KV_FP8_E4M3)
+        hipLaunchKernelGGL(kv_dequantize_rows_kernel<OXB_KV_FP8_E4M3>, grid, dim3(256), 0, st, (const uint32_t*)d_codes, d_scales, n, total4, d_out);
+    else return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 hipError_t oxb_launch_kv_quantize_rows(int kv_mode, const float* d_x, uint32_t n_rows, uint32_t n, uint8_t* d_codes, float* d_scales,
                                        hipStream_t st) {
     if (n_rows == 0 || n == 0) return hipErrorInvalidValue;

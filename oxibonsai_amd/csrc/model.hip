@@ -944,6 +944,33 @@ int oxb_hip_kv_quantize_rows(int kv_dtype, const float* rows, uint32_t n_rows, u
     OXB_API_END
 }
 
+int oxb_hip_kv_dequantize_rows(int kv_dtype, const uint8_t* codes, const float* scales, uint32_t n_rows, uint32_t n, float* rows) {
+    OXB_API_BEGIN
+    std::lock_guard<std::recursive_mutex> lk(g_mu);
+    if (!rows || !codes || !scales) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: null buffer");
+    if (kv_dtype != OXB_KV_DTYPE_I8 && kv_dtype != OXB_KV_DTYPE_FP8_E4M3)
+        return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: KV cache type %d has no quantised rows", kv_dtype);
+    if (n & 3u) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: rows of %u values (a multiple of 4 is needed)", n);
+    if (n_rows == 0 || n == 0) return OXB_HIP_OK;
+    OXB_TRY(ensure_init());
+    DevBuf x, c, sc;
+    int rc = OXB_HIP_OK;
+    const size_t cnt = (size_t)n_rows * n;
+    if (!(rc = x.ensure(cnt * 4)) && !(rc = c.ensure(cnt)) && !(rc = sc.ensure((size_t)n_rows * 4))) {
+        hipError_t e = hipMemcpyAsync(c.ptr, codes, cnt, hipMemcpyHostToDevice, g_rt.stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(sc.ptr, scales, (size_t)n_rows * 4, hipMemcpyHostToDevice, g_rt.stream);
+        if (e == hipSuccess) e = oxb_launch_kv_dequantize_rows(kv_dtype, (const uint8_t*)c.ptr, (const float*)sc.ptr, n_rows, n, (float*)x.ptr, g_rt.stream);
+        if (e == hipSuccess) e = hipMemcpyAsync(rows, x.ptr, cnt * 4, hipMemcpyDeviceToHost, g_rt.stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(g_rt.stream);
+        if (e != hipSuccess) rc = hip_fail(e, "kv row dequantisation");
+    }
+    x.release();
+    c.release();
+    sc.release();
+    return rc;
+    OXB_API_END
+}
+
 int oxb_hip_model_reset(uint64_t model) {
     OXB_API_BEGIN
     std::lock_guard<std::recursive_mutex> lk(g_mu);

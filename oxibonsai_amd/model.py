@@ -119,6 +119,20 @@ def kv_quantize_rows(kv_dtype: int, rows):
     return codes, scales
 
 
+def kv_dequantize_rows(kv_dtype: int, codes, scales) -> np.ndarray:
+    """dequantize_row (crates/oxibonsai-model/src/kv_cache_quant.rs:69-71, 545-556) on the device, through the
+    widening the attention kernels use: codes uint8 [n_rows][n], scales f32 [n_rows] -> f32 [n_rows][n]."""
+    lib = _lib.lib()
+    c = np.ascontiguousarray(codes, dtype=np.uint8)
+    s = np.ascontiguousarray(scales, dtype=np.float32).reshape(-1)
+    if c.ndim != 2 or s.size != c.shape[0]:
+        raise ValueError("codes must be 2-D with one scale per row")
+    out = np.empty(c.shape, dtype=np.float32)
+    _check(lib.oxb_hip_kv_dequantize_rows(kv_dtype, c.ctypes.data_as(_lib.u8p), s.ctypes.data_as(_lib.f32p), c.shape[0], c.shape[1],
+                                          out.ctypes.data_as(_lib.f32p)))
+    return out
+
+
 class Embedding:
     """Token embedding table resident on the device in its stored form (F32, F16, Q1_0_g128 or TQ2_0_g128)."""
 

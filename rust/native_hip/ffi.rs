@@ -164,6 +164,7 @@ extern "C" {
     pub fn oxb_hip_model_kv_pool(model: u64, info: *mut OxbKvPoolInfo) -> c_int;
     pub fn oxb_hip_model_kv_capacity(model: u64, seq: u32, n_tokens: *mut u32) -> c_int;
     pub fn oxb_hip_kv_quantize_rows(kv_dtype: c_int, rows: *const f32, n_rows: u32, n: u32, codes: *mut u8, scales: *mut f32) -> c_int;
+    pub fn oxb_hip_kv_dequantize_rows(kv_dtype: c_int, codes: *const u8, scales: *const f32, n_rows: u32, n: u32, rows: *mut f32) -> c_int;
     // checkpoint file, token ids
     pub fn oxb_hip_gguf_info(path: *const c_char, info: *mut OxbGgufInfo) -> c_int;
     pub fn oxb_hip_gguf_metadata(path: *const c_char, key: *const c_char, out: *mut c_char, out_cap: usize) -> c_int;

@@ -58,6 +58,26 @@ def test_row_quantiser_equals_oracle_bit_for_bit(backend, mode, n):
         assert np.array_equal(codes[r], wc), (r, np.nonzero(codes[r] != wc)[0][:5])
 
 
+@pytest.mark.parametrize("mode", [KV_I8, KV_FP8_E4M3])
+def test_every_code_widens_to_the_oracles_value(backend, mode):
+    """All 256 code bytes, in each of the four byte positions of a dword and under several row scales, through the
+    widening the attention kernels use (oxb_hip_kv_dequantize_rows): code * scale must be the oracle's
+    dequantize_row bit for bit (E4M3: subnormal codes, both zeros, +-448; the two NaN codes must come out NaN)."""
+    from oxibonsai_amd.model import kv_dequantize_rows
+    base = np.arange(256, dtype=np.uint8)
+    codes = np.stack([np.roll(base, r) for r in range(4)] + [base[::-1].copy()])          # every byte in every position
+    scales = np.array([1.0, 0.37, 2.0 ** -20, 117.5, 1.1920929e-07], dtype=np.float32)
+    got = kv_dequantize_rows(mode, codes, scales)
+    for r in range(codes.shape[0]):
+        want = oracle.kv_dequantize_row(ORACLE_MODE[mode], codes[r], scales[r])
+        nan = np.isnan(want)
+        assert np.array_equal(np.isnan(got[r]), nan), r
+        assert np.array_equal(got[r][~nan].view(np.uint32), want[~nan].view(np.uint32)), (r, np.nonzero(got[r][~nan] != want[~nan])[0][:5])
+    assert mode == KV_I8 or np.count_nonzero(np.isnan(got[0])) == 2
+    with pytest.raises(GpuError):
+        kv_dequantize_rows(mode, np.zeros((1, 30), dtype=np.uint8), np.ones(1, dtype=np.float32))     # rows of whole dwords
+
+
 def test_row_quantiser_rejects_bad_arguments(backend):
     with pytest.raises(GpuError):
         kv_quantize_rows(KV_F16, np.zeros((2, 32), dtype=np.float32))     # fp16 rows have no codes
