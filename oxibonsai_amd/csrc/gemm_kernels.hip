@@ -624,7 +624,11 @@ __global__ __launch_bounds__(OXB_GEMM_THREADS, RT == 3 ? 2 : 1) void gemm_mfma_k
 
 template <int FMT, int RT, int CT>
 __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(const OxbGemmParams p) {
-    __shared__ float red[8][RT * CT * 4][64];
+    // The partial sums meet in LDS in passes of PT row tiles (all of them up to four; pairs beyond, so that the
+    // array stays within 64 KB): in SWIGLU mode a pass holds gate tiles and the up tiles of the same rows.
+    constexpr int PT = RT <= 4 ? RT : 2, NPASS = RT / PT;
+    static_assert(RT % PT == 0, "row tiles per pass");
+    __shared__ float red[8][PT * CT * 4][64];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, g = lane >> 4;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     // Row tiles of this workgroup.  Plain modes: RT consecutive tiles.  SWIGLU mode (the matrix is gate || up,
@@ -659,7 +663,10 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
                     dst[s][ct] = __builtin_bit_cast(v8h, buf_load_b128(rx, blk < blk_end ? off : OXB_OOB, blk * blk_stride));
                 }
         };
-        HalfRegs<FMT> H[RT][2], Hn[RT][2];
+        // RING: the next superblock's weights wait in a second register set; with more than four row tiles there
+        // is no room for one, and a half is requested again in place once its second block has been prepared.
+        constexpr bool RING = RT <= 4;
+        HalfRegs<FMT> H[RT][2], Hn[RING ? RT : 1][2];
 #pragma unroll
         for (int rt = 0; rt < RT; rt++) {
             load_half<FMT>(H[rt][0], rc, rs, tile_of(rt), valid(rt), p.n_sb, sb0, 0, lane);
@@ -668,10 +675,12 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
         load_b(sb0 * 4u, B[0]);
         for (uint32_t sb = sb0; sb < sb1; sb++) {
             // next superblock's weights (all zero past the slice: never used)
+            if (RING) {
 #pragma unroll
-            for (int rt = 0; rt < RT; rt++) {
-                load_half<FMT>(Hn[rt][0], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 0, lane);
-                load_half<FMT>(Hn[rt][1], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 1, lane);
+                for (int rt = 0; rt < RT; rt++) {
+                    load_half<FMT>(Hn[RING ? rt : 0][0], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 0, lane);
+                    load_half<FMT>(Hn[RING ? rt : 0][1], rc, rs, tile_of(rt), valid(rt) && sb + 1 < sb1, p.n_sb, sb + 1, 1, lane);
+                }
             }
 #pragma unroll
             for (int bi = 0; bi < 4; bi++) {
@@ -679,6 +688,10 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
                 BlockDec bd[RT];
 #pragma unroll
                 for (int rt = 0; rt < RT; rt++) bd[rt] = prepare_block<FMT>(H[rt][bi >> 1], bi & 1);
+                if (!RING && (bi & 1) && sb + 1 < sb1) {  // (wave-uniform) both blocks of the half are in bd now
+#pragma unroll
+                    for (int rt = 0; rt < RT; rt++) load_half<FMT>(H[rt][bi >> 1], rc, rs, tile_of(rt), valid(rt), p.n_sb, sb + 1, bi >> 1, lane);
+                }
 #pragma unroll
                 for (int s = 0; s < 4; s++) {
                     v8h A[RT];
@@ -690,16 +703,28 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
                             acc[rt][ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A[rt], B[bi & 1][s][ct], acc[rt][ct], 0, 0, 0);
                 }
             }
+            if (RING) {
 #pragma unroll
-            for (int rt = 0; rt < RT; rt++) H[rt][0] = Hn[rt][0], H[rt][1] = Hn[rt][1];
+                for (int rt = 0; rt < RT; rt++) H[rt][0] = Hn[RING ? rt : 0][0], H[rt][1] = Hn[RING ? rt : 0][1];
+            }
         }
     }
+    // row tile behind slot q of pass ps: all tiles in order with a single pass; with pairs, SWIGLU mode takes a gate
+    // tile and the up tile of the same rows, the plain modes two neighbours
+    auto pass_rt = [&](int ps, int q) -> int { return NPASS == 1 ? q : (sw ? ps + q * (int)HP : ps * PT + q); };
 #pragma unroll
-    for (int rt = 0; rt < RT; rt++)
+    for (int ps = 0; ps < NPASS; ps++) {
+    if (ps) __syncthreads();  // the last pass has been read
+#pragma unroll
+    for (int q = 0; q < PT; q++)
 #pragma unroll
         for (int ct = 0; ct < CT; ct++)
 #pragma unroll
-            for (int v = 0; v < 4; v++) red[wave][(rt * CT + ct) * 4 + v][lane] = acc[rt][ct][v];
+            for (int v = 0; v < 4; v++) {
+                // (constant register indices in both arms: the choice is a select, not an indexed array)
+                const int rt_sw = NPASS == 1 ? q : ps + q * (int)HP, rt_pl = NPASS == 1 ? q : ps * PT + q;
+                red[wave][(q * CT + ct) * 4 + v][lane] = sw ? acc[rt_sw < RT ? rt_sw : 0][ct][v] : acc[rt_pl][ct][v];
+            }
     __syncthreads();
     // wave w finishes the accumulator tiles w, w + 8, ...: lane holds rows 4g..4g+3 of row tile rt for token 16ct + r
     const bool vec_ok = (p.ldy & 3u) == 0;
@@ -712,16 +737,18 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
             o[v] = e == INT32_MIN ? __int_as_float(0x7FC00000) : ldexpf(a, e);
         }
     };
-    const uint32_t n_out = sw ? HP * CT : RT * CT;
-    for (uint32_t idx = wave; idx < n_out; idx += 8) {
-        const uint32_t rt = idx / CT, ct = idx % CT, m = ct * 16 + r;
+    // slots of a pass that hold output rows: all of them; in SWIGLU mode the gate slots (half of a single pass, slot 0 of a pair)
+    const uint32_t q_out = sw ? (NPASS == 1 ? HP : 1u) : (uint32_t)PT, q_up = NPASS == 1 ? HP : 1u;
+    for (uint32_t idx = wave; idx < q_out * CT; idx += 8) {
+        const uint32_t q = idx / CT, ct = idx % CT, m = ct * 16 + r;
+        const uint32_t rt = (uint32_t)pass_rt(ps, (int)q);
         if (!valid((int)rt) || m >= p.M) continue;
         const int e = p.xsh[m];
         float o[4];
         total(idx, o, e);
         if (sw) {  // y[m][row] = silu(gate) * up, rows counted within the gate half
             float u[4];
-            total((rt + HP) * CT + ct, u, e);
+            total((q + q_up) * CT + ct, u, e);
 #pragma unroll
             for (int v = 0; v < 4; v++) o[v] = silu_mul(o[v], u[v]);
         }
@@ -739,6 +766,7 @@ __global__ __launch_bounds__(OXB_GEMM_NARROW_THREADS) void gemm_narrow_kernel(co
             for (int v = 0; v < 4; v++)
                 if (n + v < n_lim) yr[n + v] = rr ? rr[n + v] + o[v] : o[v];
         }
+    }
     }
 }
 
@@ -873,12 +901,14 @@ static hipError_t launch_narrow_case(const OxbGemmParams& p, hipStream_t st) {
     return hipGetLastError();
 }
 
-// Row tiles per workgroup (1, 2 or 4): the count that minimises (rounds of workgroups over the CUs) x (row tiles + 2 - a
+// Row tiles per workgroup (1, 2, 4 or - Q1 - 6): the count that minimises (rounds of workgroups over the CUs) x (row tiles + 2 - a
 // workgroup's time grows with its tiles on top of a fixed part: its start, the K-split sum and the epilogue).  What
 // counts is the last round: 384 workgroups of one tile leave half the CUs with two and the launch as long as those
 // (QKV 6144 x 4096, 8 rows: 5.5 us against 4.7 us as 192 workgroups of two tiles; 32 rows: 8.2 against 6.1).  A tie
 // goes to the larger workgroups (every workgroup reads all of the packed activations); 8B-shape decode with this rule
-// against "as many tiles as leave a workgroup per CU": +2 % at 8 and at 32 sequences.
+// against "as many tiles as leave a workgroup per CU": +2 % at 8 and at 32 sequences.  Six tiles (three gate and three up
+// tiles in SWIGLU mode) make gate || up 24576 x 4096 one workgroup per CU: at four, the 384 workgroups - one resident per
+// CU at their register count - ran in two rounds (32 rows: 17.4 -> 13.0 us per launch, the LM head 78 -> 74 us).
 static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, hipStream_t st) {
     p.ksplit = 1;
     p.sb_per_split = p.n_sb;
@@ -887,7 +917,9 @@ static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, h
     const uint32_t ct = p.M_pad / 16;
     uint32_t rt = sw ? 2 : 1;
     uint64_t best_cost = ~0ull;
-    for (uint32_t r = sw ? 2 : 1; r <= 4; r *= 2) {
+    static const uint32_t choices[4] = {1, 2, 4, 6};
+    for (uint32_t ci = sw ? 1 : 0; ci < (fmt == OXB_FMT_Q1 ? 4u : 3u); ci++) {  // (six tiles: Q1 only - the ternary decoder's registers do not fit)
+        const uint32_t r = choices[ci];
         const uint32_t wgs = sw ? (p.n_tiles / 2 + r / 2 - 1) / (r / 2) : (p.n_tiles + r - 1) / r;
         const uint64_t cost = (uint64_t)((wgs + n_cus - 1) / n_cus) * (r + 2);
         if (cost <= best_cost) best_cost = cost, rt = r;
@@ -896,6 +928,7 @@ static hipError_t launch_gemm_narrow(int fmt, OxbGemmParams p, uint32_t n_cus, h
     if (fmt == F && rt == R && ct == C) return launch_narrow_case<F, R, C>(p, st);
     OXB_NARROW_CASE(OXB_FMT_Q1, 1, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 2, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 4, 1)
     OXB_NARROW_CASE(OXB_FMT_Q1, 1, 2) OXB_NARROW_CASE(OXB_FMT_Q1, 2, 2) OXB_NARROW_CASE(OXB_FMT_Q1, 4, 2)
+    OXB_NARROW_CASE(OXB_FMT_Q1, 6, 1) OXB_NARROW_CASE(OXB_FMT_Q1, 6, 2)
     OXB_NARROW_CASE(OXB_FMT_TQ2, 1, 1) OXB_NARROW_CASE(OXB_FMT_TQ2, 2, 1) OXB_NARROW_CASE(OXB_FMT_TQ2, 4, 1)
     OXB_NARROW_CASE(OXB_FMT_TQ2, 1, 2) OXB_NARROW_CASE(OXB_FMT_TQ2, 2, 2) OXB_NARROW_CASE(OXB_FMT_TQ2, 4, 2)
 #undef OXB_NARROW_CASE

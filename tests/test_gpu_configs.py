@@ -113,11 +113,13 @@ def c4_oracle_steps(c4_model):
     return out
 
 
-@pytest.mark.parametrize("B", [8, 32])
+@pytest.mark.parametrize("B", [8, 12, 32])
 def test_config4_q1_8b_batched_decode(backend, c4_model, c4_oracle_steps, B):
-    """Batch 8 and 32 at the 8B shape: sequence b carries the inputs of sequence b % 4, each of the four is held to its
-    own oracle, and sequences with equal inputs must agree with each other.  These batches run their projections as
-    fp16 matrix-core GEMMs: prefill tolerance."""
+    """Batch 8 and 32 at the 8B shape (and 12: one token tile on the matrix-core route): sequence b carries the inputs
+    of sequence b % 4, each of the four is held to its own oracle, and sequences with equal inputs must agree with each
+    other.  Batches of nine and more run their projections as fp16 matrix-core GEMMs - gate || up and the LM head with
+    six row tiles per workgroup, which only shapes of this size select: prefill tolerance.  Batch 8 takes the fp32-exact
+    packed GEMV and is held to the same bar."""
     cfg = dict(C4, max_seq=64)
     gpu = HipModel(backend, cfg, c4_model, batch=B)
     try:
