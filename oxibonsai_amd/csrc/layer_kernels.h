@@ -41,6 +41,12 @@ struct OxbAttnParams {
     const uint32_t* pos;                 // [batch], device; seq_len = pos + 1
     uint32_t nq, nkv, hd, max_seq, n_layers, layer, chunk, n_splits;
     float scale;                         // 1 / sqrt(hd)
+    // Optional: the workgroup that merges the slots of (sequence b, kv head) also leaves its 512 outputs quantised for
+    // the O projection's packed GEMV (gemv_pack_device.h) as superblock `kv head` of vector b - instead of a pack launch
+    // between the two kernels.  Only where a kv head's q heads are exactly one superblock (nq / nkv * hd == 512) and the
+    // slots are merged in the kernel (n_splits > 1); pack_fmt = the O weight's format.
+    uint32_t* pack_out;                  // nullptr = off
+    uint32_t pack_fmt, pack_n_sb, pack_nvg;
 };
 
 // n_rows rows of n values -> one-byte codes [n_rows][n] and a scale per row (kv_mode: OXB_KV_I8 or OXB_KV_FP8_E4M3).

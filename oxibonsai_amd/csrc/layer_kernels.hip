@@ -15,6 +15,7 @@
 #include "device_utils.h"
 #include "kv_quant_device.h"
 #include "layer_kernels.h"
+#include "gemv_pack_device.h"
 
 // ---------------------------------------------------------------------------
 // Per-head QK-RMSNorm + half-split RoPE + KV store (fp16, or quantised rows: kv_quant_device.h)
@@ -712,6 +713,10 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
     float* wts = sm;
     float* inv_l = wts + heads_per * 64;
     float4* sums = reinterpret_cast<float4*>(sm + ((heads_per * 65 + 3) & ~3u));
+    // The merged outputs once more, for the quantiser at the end: 128 groups of four, in the entries of `sums` that the
+    // partial sums never use (those are written by threads tg and up, and with 128 groups tg >= 128).
+    float4* keep = sums;
+    const bool pack = p.pack_out != nullptr && nh * hd == 512u;
     const uint32_t e0 = h_first * hd;
     const uint32_t n_chunks = (p.pos[b] + p.chunk) / p.chunk;  // chunks that hold positions 0..pos
     const uint32_t used = n_chunks < p.n_splits ? n_chunks : p.n_splits;
@@ -800,6 +805,27 @@ __device__ __forceinline__ void attn_merge_heads(const OxbAttnParams& p, uint32_
             const float il = inv_l[hh];
             acc.x *= il, acc.y *= il, acc.z *= il, acc.w *= il;
             *reinterpret_cast<float4*>(out + (size_t)b * qd + e) = acc;
+            if (pack) keep[eg] = acc;
+        }
+    }
+    if (pack) {  // (uniform) one wave quantises the 512 outputs for the O projection: superblock e0 / 512 of vector b
+        __syncthreads();
+        if (tid < 64) {
+            const float* kf = reinterpret_cast<const float*>(keep);
+            float xe[2][4];
+            if (p.pack_fmt == OXB_FMT_Q1) {
+#pragma unroll
+                for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+                    for (int bb = 0; bb < 4; bb++) xe[pass][bb] = kf[gemv_pack_elem<OXB_FMT_Q1>(tid, pass, bb)];
+                gemv_pack_write<OXB_FMT_Q1>(xe, 0.f, tid, e0 / 512u, b, p.pack_n_sb, p.pack_nvg, p.pack_out);
+            } else {
+#pragma unroll
+                for (int pass = 0; pass < 2; pass++)
+#pragma unroll
+                    for (int bb = 0; bb < 4; bb++) xe[pass][bb] = kf[gemv_pack_elem<OXB_FMT_TQ2>(tid, pass, bb)];
+                gemv_pack_write<OXB_FMT_TQ2>(xe, 0.f, tid, e0 / 512u, b, p.pack_n_sb, p.pack_nvg, p.pack_out);
+            }
         }
     }
 }

@@ -73,6 +73,8 @@ struct Model {
     std::vector<void*> pf_allocs;
     GemmWorkspace gws;  // GEMM scratch of the captured large-batch decode step: sized at creation, never moved
     DevBuf gpack;       // quantised activation vectors of the captured GEMV-based step (batches of two to eight): likewise
+    DevBuf gpack_o;     // the O projection's quantised input where the attention kernel writes it itself; starts as zeros (= zero vectors) and
+                        // nothing else writes it, so the slots of a last vector group's absent vectors stay zero vectors
     // a model loaded from a file owns the weights it uploaded
     std::vector<uint64_t> owned_mats, owned_vecs;
     DevBuf tok_hist, tok_ids;  // token history of the on-device generation loop; prompt ids of a token prefill
@@ -126,6 +128,7 @@ static void free_model(Model& m) {
     m.pf_cap = 0;
     m.gws.release();
     m.gpack.release();
+    m.gpack_o.release();
     free_kv_cache(m);
     m.tok_hist.release();
     m.tok_ids.release();
@@ -184,9 +187,9 @@ static const Weight* mat_ptr(uint64_t id, int fmt, uint32_t n_rows, uint32_t k, 
 // nb activation vectors through one projection.  From gemv_packed_min_batch(K) vectors on they are quantised by a launch
 // of their own into `pack` (sized by the caller: this runs inside stream captures) and up to eight share the pass.
 static int proj(const Weight& w, const float* x, uint32_t ldx, uint32_t nb, float* y, uint32_t ldy, int pro, const float* norm_w,
-                float eps, int epi, const float* residual, DevBuf* pack) {
+                float eps, int epi, const float* residual, DevBuf* pack, bool prepacked = false) {
     const bool packed = pack && nb >= gemv_packed_min_batch(w.L.k);
-    return gemv_launch(w, x, ldx, nb, y, ldy, pro, norm_w, eps, epi, residual, packed ? pack : nullptr);
+    return gemv_launch(w, x, ldx, nb, y, ldy, pro, norm_w, eps, epi, residual, packed ? pack : nullptr, packed && prepacked);
 }
 
 // gate || up with SwiGLU behind it: one launch when K fits one GEMV launch (the epilogue needs whole row sums),
@@ -205,8 +208,10 @@ static int gate_up_swiglu(const Weight& gate_up, const float* x, uint32_t ldx, u
 // one pack launch in front of each where the vectors are quantised ahead.
 static int encode_ffn(float* hidden, const float* attn_out, const float* ffn_norm, float eps, const Weight& o,
                       const Weight& gate_up, const Weight& down, float* gu, float* act, uint32_t h, uint32_t inter,
-                      uint32_t attn_k, uint32_t nb, DevBuf* pack) {
-    OXB_TRY(proj(o, attn_out, attn_k, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden, pack));
+                      uint32_t attn_k, uint32_t nb, DevBuf* pack, DevBuf* o_prepacked = nullptr) {
+    // (o_prepacked: the attention kernel has left attn_out quantised there)
+    OXB_TRY(proj(o, attn_out, attn_k, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden, o_prepacked ? o_prepacked : pack,
+                 o_prepacked != nullptr));
     OXB_TRY(gate_up_swiglu(gate_up, hidden, h, nb, ffn_norm, eps, gu, act, inter, pack));
     OXB_TRY(proj(down, act, inter, nb, hidden, h, OXB_GEMV_PRO_F32, nullptr, 0.f, OXB_GEMV_RESIDUAL, hidden, pack));
     return OXB_HIP_OK;
@@ -252,6 +257,12 @@ static int size_gemm_workspaces(Model& m) {
         if (d.nq * d.hd > kmax) kmax = d.nq * d.hd;
         int rc = m.gpack.ensure(oxb_gemv_pack_bytes(kmax, decode_chunk(d.batch)));
         if (rc) return rc;
+        if (d.batch <= OXB_GEMV_PACKED_MAX_BATCH && !m.gpack_o.ptr) {
+            const size_t n = oxb_gemv_pack_bytes(d.nq * d.hd, d.batch);
+            if ((rc = m.gpack_o.ensure(n))) return rc;
+            OXB_TRY_HIP(hipMemsetAsync(m.gpack_o.ptr, 0, n, g_rt.stream), "pack buffer clear");  // (never inside a capture: sized at creation)
+            OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "pack buffer clear");
+        }
     }
     if (d.batch < OXB_DECODE_GEMM_MIN_BATCH) return OXB_HIP_OK;
     const uint32_t qd = d.nq * d.hd, kd = d.nkv * d.hd, qkv_rows = qd + 2 * kd;
@@ -334,7 +345,7 @@ static int kv_sync_table(Model& m) {
 // slot results in m.attn_part and the parameters the merge needs in *ap.
 // One launch: QK-norm, RoPE, the store of the new rows, attention over the cache and the merge of the KV slots into
 // m.attn_out (with a single slot per sequence the kernel writes its output directly).
-static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm) {
+static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, const float* k_norm, const Weight* pack_for = nullptr) {
     const oxb_model_desc& d = m.d;
     OxbAttnParams ap;
     ap.qkv = m.qkv;
@@ -366,6 +377,10 @@ static int encode_decode_attention(Model& m, uint32_t L, const float* q_norm, co
     ap.chunk = m.chunk;
     ap.n_splits = m.n_splits;
     ap.scale = 1.0f / sqrtf((float)d.hd);
+    ap.pack_out = pack_for ? (uint32_t*)m.gpack_o.ptr : nullptr;  // the O projection's operands, written by the merging workgroups
+    ap.pack_fmt = pack_for ? (uint32_t)pack_for->L.fmt : 0;
+    ap.pack_n_sb = pack_for ? pack_for->L.n_sb : 0;
+    ap.pack_nvg = (d.batch + 3) / 4;
     OXB_TRY_HIP(oxb_launch_attn_decode(ap, d.batch, g_rt.stream), "kernel launch failed: attention");
     return OXB_HIP_OK;
 }
@@ -428,11 +443,16 @@ static int encode_decode_step(Model& m, bool with_lm_head) {
             OXB_TRY(proj(*wqkv, m.hidden + (size_t)b0 * d.h, d.h, nb, m.qkv + (size_t)b0 * qkv_rows, qkv_rows,
                          OXB_GEMV_PRO_RMSNORM, attn_norm, d.eps, OXB_GEMV_STORE, nullptr, pack));
         }
-        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm));
+        // Where the q heads of a kv head are one superblock of the O projection's input and the batch's vectors are
+        // quantised ahead of that GEMV, the attention kernel's merging workgroups do the quantising: no pack launch.
+        const bool fuse_o = m.gpack_o.ptr && d.batch <= OXB_GEMV_PACKED_MAX_BATCH && d.batch >= gemv_packed_min_batch(qd) &&
+                            m.n_splits > 1 && (d.nq / d.nkv) * d.hd == 512u && m.gpack_o.cap >= oxb_gemv_pack_bytes(qd, d.batch);
+        OXB_TRY(encode_decode_attention(m, L, q_norm, k_norm, fuse_o ? wo : nullptr));
         for (uint32_t b0 = 0; b0 < d.batch; b0 += chunk) {
             const uint32_t nb = (d.batch - b0) < chunk ? (d.batch - b0) : chunk;
             OXB_TRY(encode_ffn(m.hidden + (size_t)b0 * d.h, m.attn_out + (size_t)b0 * qd, ffn_norm, d.eps, *wo, *wgu, *wdn,
-                               m.gu + (size_t)b0 * 2 * d.inter, m.act + (size_t)b0 * d.inter, d.h, d.inter, qd, nb, pack));
+                               m.gu + (size_t)b0 * 2 * d.inter, m.act + (size_t)b0 * d.inter, d.h, d.inter, qd, nb, pack,
+                               fuse_o ? &m.gpack_o : nullptr));
         }
     }
     if (with_lm_head) {

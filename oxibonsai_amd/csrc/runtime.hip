@@ -204,15 +204,19 @@ int upload_weight(uint64_t* id, int fmt, const uint8_t* aos, size_t n_bytes, uin
 // One GEMV over resident weights, any K: launches of at most OXB_GEMV_MAX_SB superblocks, the first with the wanted
 // epilogue, the rest accumulating.  nvec <= OXB_GEMV_MAX_BATCH vectors share each pass over the weights.
 int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, float* d_y, uint32_t ldy, int pro,
-                const float* d_norm_w, float eps, int epi, const float* d_residual, DevBuf* pack_ws) {
+                const float* d_norm_w, float eps, int epi, const float* d_residual, DevBuf* pack_ws, bool prepacked) {
     OxbGemvParams p;
     memset(&p, 0, sizeof p);
     if (pack_ws) {  // quantise the vectors once, in a launch of its own; the GEMV then loads its operands
         const size_t need = oxb_gemv_pack_bytes(w.L.k, nvec);
-        int rc = pack_ws->ensure(need);
-        if (rc) return rc;
-        hipError_t e = oxb_launch_gemv_pack((int)w.L.fmt, pro, d_x, ldx, nvec, w.L.k, d_norm_w, (uint32_t*)pack_ws->ptr, g_rt.stream);
-        if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv_pack");
+        if (prepacked) {  // (the kernel that produced the vectors has left them quantised in pack_ws)
+            if (pack_ws->cap < need || pro != OXB_GEMV_PRO_F32) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: packed operands of %zu bytes, %zu needed", pack_ws->cap, need);
+        } else {
+            int rc = pack_ws->ensure(need);
+            if (rc) return rc;
+            hipError_t e = oxb_launch_gemv_pack((int)w.L.fmt, pro, d_x, ldx, nvec, w.L.k, d_norm_w, (uint32_t*)pack_ws->ptr, g_rt.stream);
+            if (e != hipSuccess) return hip_fail(e, "kernel launch failed: gemv_pack");
+        }
         p.xq = (const uint32_t*)pack_ws->ptr;
         p.xq_bytes = (uint32_t)need;
         p.nvg = (nvec + 3) / 4;

@@ -80,9 +80,10 @@ int gemv_device(const Weight& w, const float* d_x, float* d_y, uint32_t batch, u
 // nvec <= OXB_GEMV_MAX_BATCH vectors x [nvec][ldx] through one pass over the weights: pro / epi are OXB_GEMV_PRO_* /
 // OXB_GEMV_* (RMSNorm with d_norm_w and eps in front; store, residual add or SwiGLU behind).
 // With pack_ws the vectors (up to OXB_GEMV_PACKED_MAX_BATCH) are quantised by a launch of their own into that buffer
-// (grown on demand: never inside a stream capture) and the GEMV loads its operands from there.
+// (grown on demand: never inside a stream capture) and the GEMV loads its operands from there; with `prepacked` the
+// buffer already holds them (left there by the kernel that produced the vectors) and no pack launch is made.
 int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, float* d_y, uint32_t ldy, int pro,
-                const float* d_norm_w, float eps, int epi, const float* d_residual, DevBuf* pack_ws = nullptr);
+                const float* d_norm_w, float eps, int epi, const float* d_residual, DevBuf* pack_ws = nullptr, bool prepacked = false);
 uint32_t gemv_packed_min_batch(uint32_t k);
 // x (device, [m][ldx]) -> y (device, [m][ldy]) through the fp16 packer + MFMA GEMM.  pack_op (OXB_PACK_*) names the
 // row-wise producer fused into the packer: RMSNorm with weights d_pack_w and eps, or SwiGLU of x = [gate | up].

@@ -311,3 +311,65 @@ def test_wide_ffn_takes_four_row_tiles_per_workgroup(backend, fmt):
         assert parity_violations(got, want, 1e-2) == 0
     finally:
         gpu.close()
+
+
+FUSED_O = dict(n_layers=2, h=1024, inter=1536, nq=8, nkv=2, hd=128, vocab=256, max_seq=384, eps=1e-6, rope_theta=1e6)
+
+
+@pytest.mark.parametrize("fmt", [TQ2, Q1])
+@pytest.mark.parametrize("B", [5, 8])
+def test_attention_leaves_the_o_projection_its_operands(backend, fmt, B):
+    """Four q heads of 128 per kv head are one 512-value superblock of the O projection's input: with five to eight
+    sequences the attention kernel's merging workgroups quantise their outputs for that GEMV themselves and no pack
+    launch runs in between (five sequences leave three slots of the second vector group without a vector).  All
+    sequences decode from position 0 past the first chunk boundary - one, then two attention slots in use - under the
+    fp32-exact gate; then a NaN in one sequence's input must stay in that sequence."""
+    cfg = dict(FUSED_O, fmt=fmt)
+    w = synth.make_model(cfg, 131 + fmt)
+    gpu = HipModel(backend, cfg, w, batch=B)
+    cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
+    try:
+        for pos in range(132):
+            hidden = np.stack([synth.embedding_rows(400 + b, [(7 * pos + b) % 199], cfg["h"])[0] * 50.0 for b in range(B)])
+            check = pos < 3 or pos >= 127
+            got, toks = gpu.forward(hidden, np.full(B, pos, dtype=np.uint32), want_logits=check)
+            for b in range(B):
+                want = cpus[b].forward(hidden[b], pos, want_logits=check)
+                if check:
+                    assert parity_violations(got[b], want) == 0, (pos, b, float(np.max(np.abs(got[b] - want))))
+                    assert toks[b] == int(np.argmax(got[b]))
+        assert gpu.uses_graph()
+        hidden = np.stack([synth.embedding_rows(500 + b, [b], cfg["h"])[0] * 50.0 for b in range(B)])
+        hidden[1, 17] = np.nan
+        got, _ = gpu.forward(hidden, np.full(B, 132, dtype=np.uint32))
+        assert np.all(np.isnan(got[1]))
+        for b in (0, 2, B - 1):
+            assert parity_violations(got[b], cpus[b].forward(hidden[b], 132)) == 0, b
+    finally:
+        gpu.close()
+
+
+@pytest.mark.parametrize("B", [6, 7])
+def test_attention_packs_for_sequences_of_different_lengths(backend, B):
+    """The same route with prompts of 5 to 300 positions per sequence (one to three slots in use per sequence); the prompts
+    went in through the batched prefill, so the prefill tolerance applies."""
+    cfg = dict(FUSED_O, fmt=Q1)
+    w = synth.make_model(cfg, 141)
+    lens = [5, 127, 128, 200, 257, 300, 129][:B]
+    gpu = HipModel(backend, cfg, w, batch=B)
+    cpus = [oracle.OracleModel(cfg, w, kv_f16=True) for _ in range(B)]
+    try:
+        for b, n in enumerate(lens):
+            ctx = synth.embedding_rows(600 + b, [(7 * i + b) % 199 for i in range(n)], cfg["h"]) * 50.0
+            gpu.prefill(ctx, seq=b, want_logits=False)
+            for i, r in enumerate(ctx):
+                cpus[b].forward(r, i, want_logits=False)
+        for step in range(3):
+            hidden = np.stack([synth.embedding_rows(700 + b, [step], cfg["h"])[0] * 50.0 for b in range(B)])
+            got, toks = gpu.forward(hidden, np.array([n + step for n in lens], dtype=np.uint32))
+            for b in range(B):
+                want = cpus[b].forward(hidden[b], lens[b] + step)
+                assert parity_violations(got[b], want, 1e-2) == 0, (step, b, float(np.max(np.abs(got[b] - want))))
+                assert toks[b] == int(np.argmax(got[b]))
+    finally:
+        gpu.close()
