@@ -128,7 +128,8 @@ def test_config4_q1_8b_batched_decode(backend, c4_model, c4_oracle_steps, B):
             got, toks = gpu.forward(np.stack([rows[b % N_DISTINCT] for b in range(B)]), np.full(B, step, dtype=np.uint32))
             for s in range(N_DISTINCT):
                 want = c4_oracle_steps[s][step]
-                tol = 5e-3 * float(np.max(np.abs(want)))
+                # eight sequences take the fp32-exact route: the batch-1 decode bar; more run on fp16 activations
+                tol = (5e-4 if B <= 8 else 5e-3) * float(np.max(np.abs(want)))
                 err = float(np.max(np.abs(got[s] - want)))
                 assert err < tol, (B, step, s, err, tol)
                 top2 = np.sort(want)[-2:]

@@ -60,21 +60,25 @@ def test_small_model_128_greedy_steps(backend, fmt):
 
 
 def test_mid_model_long_context_crosses_attention_chunks(backend):
-    # head_dim 128 and a context past two 1024-position attention chunks
+    # head_dim 128 and a context past two 1024-position attention chunks.  The oracle's linear layers run on its SIMD
+    # tier here (2100 positions; held to the scalar tier in test_oracle.py, 2e-5 of the logit scale apart at position 300)
     cfg = dict(MID, fmt=Q1)
     w = synth.make_model(cfg, 5)
-    cpu = oracle.OracleModel(cfg, w, kv_f16=True)
+    cpu = oracle.OracleModel(cfg, w, kv_f16=True, simd=True)
     gpu = HipModel(backend, cfg, w, batch=1)
+    rows = synth.embedding_rows(9, [pos % 97 for pos in range(2100)], cfg["h"]) * 50.0
     try:
+        run = 0                                     # first position the oracle has not seen yet
         for pos in range(2100):
-            hidden = synth.embedding_rows(9, [pos % 97], cfg["h"])[0] * 50.0
             if pos % 300 == 0 or pos in (1023, 1024, 1025, 2047, 2048, 2099):
-                want = cpu.forward(hidden, pos)
-                got, _ = gpu.forward(hidden, pos)
+                if pos > run:                       # the oracle takes the positions in between layer by layer (bit-equal
+                    cpu.forward_batch(rows[run:pos], run, want_logits=False)   # to its token-by-token forward, all cores)
+                want = cpu.forward(rows[pos], pos)
+                run = pos + 1
+                got, _ = gpu.forward(rows[pos], pos)
                 assert parity_violations(got[0], want) == 0, pos
-            else:                                   # keep both KV caches in step without the LM head compare
-                cpu.forward(hidden, pos, want_logits=False)
-                gpu.forward(hidden, pos, want_logits=False)
+            else:                                   # the device decodes every position, without the LM head compare
+                gpu.forward(rows[pos], pos, want_logits=False)
     finally:
         gpu.close()
 
