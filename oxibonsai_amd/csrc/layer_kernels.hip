@@ -367,8 +367,11 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     // With an fp16 cache the rows of the first chunk are requested before anything else, so that their way from HBM
     // overlaps the Q prologue.  In the workgroup that stores the new position that row is not in the cache yet (and
     // rows past the end repeat it): it is patched in from LDS below, with the very values the cache receives.
+    // With a quantised cache there is no such patch: every workgroup requests early except the one whose first chunk
+    // holds the new position, which waits until its own stores of that row have landed.
     constexpr bool EARLY = !QC;
     const uint32_t pos_chunk = pos / OXB_ATTN_CHUNK;
+    const bool early = EARLY || !(owner && pos_chunk == first);  // (the same for the whole workgroup)
     uint32_t na = 0, nb = 0;  // pages of the chunk whose rows are requested next
     auto request_first = [&]() {
         if (first < n_chunks) {
@@ -420,7 +423,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
         }
     }
     __builtin_amdgcn_sched_barrier(0);
-    if (EARLY) request_first();
+    if (early) request_first();
     __builtin_amdgcn_sched_barrier(0);
     // --- Q of the group's heads: RMSNorm over the head, RoPE on the pairs (d, d + hd/2), times 1/sqrt(hd) ---
     for (uint32_t h = wave; h < G; h += 4) {
@@ -507,7 +510,7 @@ __global__ __launch_bounds__(256) void attn_decode_fused_kernel(OxbAttnParams p)
     // several chunks that ends in the new position's): then the stores must have landed first.
     if (owner && !(EARLY && pos_chunk == first)) __syncthreads();
     else lds_barrier();
-    if (!EARLY) request_first();
+    if (!early) request_first();
 
     // B operands: lane (head = qi, g) holds the eight Q values that meet its K values in step s, as hi + lo: one
     // 16-byte LDS read each.  Columns past the group's heads repeat head 0; nothing of them is ever stored.
