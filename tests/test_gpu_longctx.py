@@ -147,7 +147,8 @@ def _decode_parity(backend, cfg, fmt, mode, window, sinks, steps, seed, batch=1,
     cfg = dict(cfg, fmt=fmt)
     w = synth.make_model(cfg, seed)
     tol = tol or {KV_F16: 1e-3, KV_I8: 2e-3, KV_FP8_E4M3: 5e-3}[mode]
-    gemm_path = batch >= 3          # the projections of such a batch run as fp16 GEMMs
+    gemm_path = batch >= 3          # held like a batch on the fp16 GEMM route (nine sequences and more): with several
+                                    # sequences some quantised code always lands on the other side of a rounding boundary
     if gemm_path:
         tol = 1e-2
     cpus = [oracle.OracleModel(cfg, w, kv_mode=ORACLE_MODE[mode], window=window, sinks=sinks) for _ in range(batch)]
@@ -198,6 +199,18 @@ def test_decode_with_window_and_quantised_cache(backend, mode):
 @pytest.mark.parametrize("batch", [2, 4])
 def test_batched_decode_with_options(backend, batch):
     _decode_parity(backend, SMALL, Q1, KV_I8, 40, 2, 150, seed=61, batch=batch, check_every=9)
+
+
+# four q heads of 128 per kv head: with five to eight sequences the attention kernel's merging workgroups also quantise
+# their output for the O projection (one 512-value superblock each)
+PACKS_FOR_O = dict(n_layers=2, h=256, inter=384, nq=8, nkv=2, hd=128, vocab=128, max_seq=256, eps=1e-6, rope_theta=1e6)
+
+
+@pytest.mark.parametrize("mode,window,sinks", [(KV_I8, 0, 0), (KV_F16, 40, 2), (KV_FP8_E4M3, 100, 3)])
+def test_batched_decode_with_options_where_attention_packs_for_o(backend, mode, window, sinks):
+    """Six sequences past the first chunk boundary with a quantised cache and / or a window: the option variants of the
+    attention kernel share the merge that leaves the O projection its operands."""
+    assert _decode_parity(backend, PACKS_FOR_O, Q1, mode, window, sinks, 140, seed=91, batch=6, check_every=9)
 
 
 def test_sequences_at_different_positions_with_a_window(backend):
