@@ -9,9 +9,10 @@ where the oracle's own pre-rounding value sits on such a boundary, and logits un
 2e-3 (INT8: one code step is 1/127 of the row maximum) or 5e-3 (E4M3: one code step is 1/8 of the value itself, and a
 few dozen of the ~3e5 cached values of a run land on the other side of a boundary).
 
-Where the projections run as fp16 GEMMs (prefill, decode batches of 3 and more) K and V carry 2^-11 of relative noise
+Where the projections run as fp16 GEMMs (prefill, decode batches of nine and more) K and V carry 2^-11 of relative noise
 before they are quantised, so a few percent of the codes differ from the free-running oracle's and the logits agree only
-to within the quantisation noise itself (held to 2e-2 of the largest logit).  The tight check there runs the oracle over
+to within the quantisation noise itself (held to 2e-2 of the largest logit); batches of three to eight, on the fp32-exact
+GEMVs, are held the same way: among several sequences some code always lands on the other side of a boundary.  The tight check there runs the oracle over
 the device's own cache rows (OracleModel.load_rows + freeze): same rows, so the attention arithmetic is compared at the
 ordinary tolerance."""
 import numpy as np
