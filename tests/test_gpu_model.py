@@ -83,10 +83,10 @@ def test_mid_model_long_context_crosses_attention_chunks(backend):
         gpu.close()
 
 
-@pytest.mark.parametrize("B,tol", [(2, 1e-3), (3, 1e-2)])
+@pytest.mark.parametrize("B,tol", [(2, 1e-3), (3, 1e-3), (6, 1e-3)])
 def test_batched_sequences_are_independent(backend, B, tol):
-    # two sequences share one pass of the fp32-exact GEMV; from three on the projections take the fp16 matrix-core
-    # route and are held to its tolerance
+    # up to eight sequences share one pass of the fp32-exact GEMVs (four with the kernel quantising them itself, more
+    # through the pack launch): the batch-1 gate
     cfg = dict(SMALL, fmt=TQ2)
     w = synth.make_model(cfg, 31)
     gpu = HipModel(backend, cfg, w, batch=B)
@@ -185,7 +185,7 @@ def test_gqa_group_shapes(backend, nq, nkv, hd):
 @pytest.mark.parametrize("fmt", [TQ2, Q1])
 @pytest.mark.parametrize("B", [9, 20, 40])   # one and two token tiles of the narrow GEMM, then the wide one
 def test_large_batch_decode_runs_on_the_matrix_cores(backend, fmt, B):
-    """From 3 sequences on, a decode step sends its projections through the matrix-core GEMM (fp16 activations):
+    """From 9 sequences on, a decode step sends its projections through the matrix-core GEMM (fp16 activations):
     logits are held to the prefill tolerance 1e-2 under the reference's gate form; the step is still replayed
     from a captured graph and sequences stay independent."""
     cfg = dict(SMALL, fmt=fmt)
