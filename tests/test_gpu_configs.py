@@ -265,15 +265,15 @@ def test_config4_q1_8b_prefill_2048_then_greedy(backend, c4_model, c4_table, cap
         gpu.close()
 
 
-def test_config4_q1_8b_prefill_and_decode_repeat_bit_for_bit(backend, c4_model, c4_table):
-    """The 2048-token prefill and the eight-sequence decode steps behind it, twice from a cleared cache: every logit
+@pytest.mark.parametrize("B", [8, 32])
+def test_config4_q1_8b_prefill_and_decode_repeat_bit_for_bit(backend, c4_model, c4_table, B):
+    """The 2048-token prefill and decode steps of eight (fp32-exact GEMVs) and 32 sequences (fp16 GEMMs) behind it, twice from a cleared cache: every logit
     and every cache row of the first and the last layer must come out bit for bit the same (the reference holds its
     fused path to the same property on a small model, cuda_full_layer/encode_ternary.rs:966-1149).  No oracle is
     involved: this is the check that an unordered sum or a read that overtakes a write would fail some of the time."""
     cfg = dict(C4, max_seq=2304)
     ids = synth.token_ids(0xB0A5A1C6, N_PROMPT, 5000)
     rows = c4_table[ids]
-    B = 8
     gpu = HipModel(backend, cfg, c4_model, batch=B)
     try:
         runs = []
@@ -282,7 +282,7 @@ def test_config4_q1_8b_prefill_and_decode_repeat_bit_for_bit(backend, c4_model, 
             logits, tok = gpu.prefill(rows, pos_start=0, seq=B - 1)
             kv = [gpu.read_kv(L, hh, 0, N_PROMPT, seq=B - 1)[:2] for L in (0, cfg["n_layers"] - 1) for hh in (0, cfg["nkv"] - 1)]
             steps = []
-            for step in range(3):                    # sequence 7 continues behind its prompt, the others start at 0
+            for step in range(3):                    # the last sequence continues behind its prompt, the others start at 0
                 hidden = np.stack([_row(0xC4E + b, step, cfg["h"]) for b in range(B)])
                 pos = np.array([step] * (B - 1) + [N_PROMPT + step], dtype=np.uint32)
                 g, t = gpu.forward(hidden, pos)
