@@ -210,7 +210,8 @@ int gemv_launch(const Weight& w, const float* d_x, uint32_t ldx, uint32_t nvec, 
     if (pack_ws) {  // quantise the vectors once, in a launch of its own; the GEMV then loads its operands
         const size_t need = oxb_gemv_pack_bytes(w.L.k, nvec);
         if (prepacked) {  // (the kernel that produced the vectors has left them quantised in pack_ws)
-            if (pack_ws->cap < need || pro != OXB_GEMV_PRO_F32) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: packed operands of %zu bytes, %zu needed", pack_ws->cap, need);
+            if (pro != OXB_GEMV_PRO_F32) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: operands packed ahead carry no RMSNorm");
+            if (pack_ws->cap < need) return fail(OXB_HIP_INVALID_ARGUMENT, "invalid argument: packed operands of %zu bytes, %zu needed", pack_ws->cap, need);
         } else {
             int rc = pack_ws->ensure(need);
             if (rc) return rc;
