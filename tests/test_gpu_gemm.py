@@ -157,6 +157,20 @@ def test_gemm_prefill_shapes_qwen3_4b_ternary(backend, name, n, k):
     assert np.all(np.isfinite(got))
 
 
+@pytest.mark.parametrize("m,n,k", [(32, 24576, 8192), (9, 24556, 6656), (17, 24576, 512)])
+def test_gemm_few_rows_six_row_tiles_per_workgroup(backend, m, n, k):
+    """Q1 matrices of 1536 row tiles and more at up to 32 token rows take six row tiles per workgroup.  K of 8192 and
+    6656: a wave's K slice is two superblocks, so the weights of the next one are requested in place of the one just
+    prepared (no second register set), the second with a last slice that is shorter than the others and a last
+    workgroup that is not full; K of 512: seven of the eight waves have no slice at all."""
+    a = synth.make_blocks(Q1, 8200 + m, n, k)
+    x = synth.normal_f32(8201 + m, m * k).reshape(m, k)
+    got = _gemm(backend, Q1, a, x, m, n, k)
+    want = oracle.simd_gemm(Q1, a, x, m, n, k, x4=True)
+    assert parity_violations(got, want, GEMM_REL_TOL) == 0
+    assert np.max(np.abs(got - want)) < 3e-3 * np.sqrt(np.mean(want.astype(np.float64) ** 2))
+
+
 def test_gemm_prefill_shape_q1_8b_gate_up(backend):
     m, n, k = 256, 24576, 4096
     a = synth.make_blocks(Q1, 8000, n, k)
