@@ -260,8 +260,7 @@ static int size_gemm_workspaces(Model& m) {
         if (d.batch <= OXB_GEMV_PACKED_MAX_BATCH && !m.gpack_o.ptr) {
             const size_t n = oxb_gemv_pack_bytes(d.nq * d.hd, d.batch);
             if ((rc = m.gpack_o.ensure(n))) return rc;
-            OXB_TRY_HIP(hipMemsetAsync(m.gpack_o.ptr, 0, n, g_rt.stream), "pack buffer clear");  // (never inside a capture: sized at creation)
-            OXB_TRY_HIP(hipStreamSynchronize(g_rt.stream), "pack buffer clear");
+            OXB_TRY_HIP(hipMemset(m.gpack_o.ptr, 0, n), "pack buffer clear");  // (at creation, like the cache's scales: never inside a capture)
         }
     }
     if (d.batch < OXB_DECODE_GEMM_MIN_BATCH) return OXB_HIP_OK;
